@@ -1,0 +1,118 @@
+/*
+ * C ABI of libtorch_int_hip.so: hand-written gfx950 (MI355X) kernels for the
+ * INT8 W8A8 operator set of torch-int.  Each entry point replaces one function
+ * bound by the upstream pybind11 module `torch_int._CUDA`
+ * (torch_int/kernels/bindings.cpp:5-20) and is what a binding for that module
+ * calls after it has validated and allocated tensors.
+ *
+ * Conventions shared by every entry point
+ *   - all pointers are DEVICE pointers on the current HIP device; operands are
+ *     packed row-major with the innermost dimension contiguous;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); the
+ *     call only enqueues work, it never synchronises, allocates or frees;
+ *   - the return value is 0 on success, otherwise a TI_ERR_* code, and
+ *     ti_last_error() gives a human-readable reason for the calling thread;
+ *     on error nothing has been launched;
+ *   - zero-sized problems (M, N or batch == 0) succeed without a launch;
+ *     K == 0 yields the epilogue of an all-zero accumulator.
+ *
+ * Arithmetic (identical in all kernels)
+ *   acc = sum_k int32(x[m,k]) * int32(w[n,k])      exact int32
+ *   t   = fmaf(alpha, float(acc), beta * float(bias[n]))
+ *   s8 outputs  = (int8) rint(clamp(t, -128, 127))      round-half-to-even
+ *   s32 scaled  = saturating (int32) rint(t)
+ */
+#ifndef TORCH_INT_HIP_H
+#define TORCH_INT_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TI_OK 0
+#define TI_ERR_INVALID_ARG 1   /* null pointer, negative size, size beyond int32 tiling limits */
+#define TI_ERR_ALIGNMENT 2     /* pointer not aligned to its element size */
+#define TI_ERR_LAUNCH 3        /* hipLaunchKernel reported an error */
+#define TI_ERR_NO_DEVICE 4     /* no usable gfx950 device */
+
+/* Library version (major*10000 + minor*100 + patch). */
+int ti_version(void);
+
+/* Reason for the last non-zero return on this thread ("" if none). */
+const char* ti_last_error(void);
+
+/* Verifies that a HIP device is present and is gfx950; returns TI_OK or
+ * TI_ERR_NO_DEVICE.  Optional: every entry point works without it. */
+int ti_init(void);
+
+/* Bytes of scratch the linear entry points can use for (M,N,K) to split the K
+ * loop over workgroups when M is small (decode).  Passing a smaller or NULL
+ * workspace is always legal and only selects a non-split kernel. */
+int64_t ti_linear_workspace_bytes(int64_t M, int64_t N, int64_t K);
+
+/* ---- W8A8 linear: out[M,N] = epilogue(x[M,K] . w[N,K]^T, bias[N]) ---- */
+
+/* replaces linear_a8_w8_b32_o32 (torch_int/kernels/linear.cu:13-136;
+ * declared torch_int/kernels/include/linear.h:6-9): out = acc + bias, int32. */
+int ti_linear_a8_w8_b32_o32(const int8_t* x, const int8_t* w, const int32_t* bias, int32_t* out,
+                            int64_t M, int64_t N, int64_t K,
+                            void* workspace, int64_t workspace_bytes, void* stream);
+
+/* replaces linear_a8_w8_b32_o32_with_scaling (linear.cu:139-243; linear.h:12-17):
+ * out = sat_s32(rint(alpha*acc + beta*bias)). */
+int ti_linear_a8_w8_b32_o32_with_scaling(const int8_t* x, const int8_t* w, const int32_t* bias,
+                                         int32_t* out, int64_t M, int64_t N, int64_t K,
+                                         float alpha, float beta,
+                                         void* workspace, int64_t workspace_bytes, void* stream);
+
+/* replaces linear_a8_w8_bfp32_ofp32 (linear.cu:246-365; linear.h:20-25):
+ * out = alpha*acc + beta*bias, fp32 bias and output. */
+int ti_linear_a8_w8_bfp32_ofp32(const int8_t* x, const int8_t* w, const float* bias, float* out,
+                                int64_t M, int64_t N, int64_t K, float alpha, float beta,
+                                void* workspace, int64_t workspace_bytes, void* stream);
+
+/* replaces linear_a8_w8_b8_o8 (linear.cu:369-473; linear.h:36-41):
+ * out = s8(rint(clamp(alpha*acc + beta*bias, -128, 127))). */
+int ti_linear_a8_w8_b8_o8(const int8_t* x, const int8_t* w, const int8_t* bias, int8_t* out,
+                          int64_t M, int64_t N, int64_t K, float alpha, float beta,
+                          void* workspace, int64_t workspace_bytes, void* stream);
+
+/* replaces linear_relu_a8_w8_b8_o8 (linear.cu:476-625; linear.h:28-33):
+ * out = s8(rint(min(max(alpha*acc + beta*bias, 0), 127))). */
+int ti_linear_relu_a8_w8_b8_o8(const int8_t* x, const int8_t* w, const int8_t* bias, int8_t* out,
+                               int64_t M, int64_t N, int64_t K, float alpha, float beta,
+                               void* workspace, int64_t workspace_bytes, void* stream);
+
+/* ---- batched A . B^T: c[b,M,N] = epilogue(a[b,M,K] . b[b,N,K]^T) ---- */
+
+/* replaces bmm_s8t_s8n_f32t (torch_int/kernels/bmm.cu:10-108; include/bmm.h:4):
+ * c = alpha * float(acc). */
+int ti_bmm_s8t_s8n_f32t(const int8_t* a, const int8_t* b, float* c,
+                        int64_t batch, int64_t M, int64_t N, int64_t K, float alpha, void* stream);
+
+/* replaces bmm_s8t_s8n_s8t (bmm.cu:110-208; bmm.h:6):
+ * c = s8(rint(clamp(alpha * float(acc), -128, 127))). */
+int ti_bmm_s8t_s8n_s8t(const int8_t* a, const int8_t* b, int8_t* c,
+                       int64_t batch, int64_t M, int64_t N, int64_t K, float alpha, void* stream);
+
+/* replaces bmm_s8t_s8n_s32t (bmm.cu:210-295; bmm.h:8): c = acc. */
+int ti_bmm_s8t_s8n_s32t(const int8_t* a, const int8_t* b, int32_t* c,
+                        int64_t batch, int64_t M, int64_t N, int64_t K, void* stream);
+
+/* ---- fused dequantise + residual add + LayerNorm + quantise ---- */
+
+/* replaces dq_add_layernorm_q (torch_int/kernels/fused.cu:5-25; include/fused.h:6-14):
+ *   r_out[row,i] = fmaf(input_scale, float(input[row,i]), residual[row,i])
+ *   q_out[row,i] = s8(rint(clamp(LN(r_out[row,:])[i] * gamma[i] + beta[i], -128, 127)))
+ * over `rows` rows of H elements; biased variance, eps added before the sqrt.
+ * r_out may alias residual (in-place residual stream). */
+int ti_dq_add_layernorm_q(const int32_t* input, float input_scale, const float* residual,
+                          const float* gamma, const float* beta, float eps,
+                          float* r_out, int8_t* q_out, int64_t rows, int64_t H, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TORCH_INT_HIP_H */

@@ -1,0 +1,200 @@
+"""TEST INFRASTRUCTURE ONLY: Python face of the CPU oracle (``ti_oracle.c``).
+
+Only tests, ``__graft_entry__.smoke()`` and the CPU-baseline leg of ``bench.py``
+may import this module.  The shipped package never does.
+
+Every function takes CPU tensors and returns new CPU tensors with the same
+positional signature as the ``torch_int._CUDA`` entry point of the same name
+(upstream ``torch_int/kernels/bindings.cpp:5-20``).
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libti_oracle.so")
+_lib = None
+
+
+def build(force=False):
+    """Compile ``ti_oracle.c`` with gcc (see the Makefile beside it)."""
+    if force and os.path.exists(_LIB_PATH):
+        os.remove(_LIB_PATH)
+    subprocess.check_call(["make", "-s", "-C", _HERE, "libti_oracle.so"])
+
+
+def _load():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        _lib = ctypes.CDLL(_LIB_PATH)
+        _lib.orc_num_threads.restype = ctypes.c_int
+    return _lib
+
+
+def num_threads():
+    return int(_load().orc_num_threads())
+
+
+def _p(t):
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def _i64(v):
+    return ctypes.c_int64(int(v))
+
+
+def _f32(v):
+    # pybind11 narrows a Python float to C float at the call boundary
+    # (upstream bindings.cpp); np.float32() is the same round-to-nearest.
+    return ctypes.c_float(float(np.float32(v)))
+
+
+def _chk(t, dtype, name):
+    assert t.device.type == "cpu", f"{name}: oracle takes CPU tensors"
+    assert t.dtype == dtype, f"{name}: expected {dtype}, got {t.dtype}"
+    return t.contiguous()
+
+
+def gemm_acc(a, b):
+    """int32 accumulators of A . B^T.  a: [M,K] or [B,M,K]; b: [N,K] or [B,N,K]."""
+    a = _chk(a, torch.int8, "a")
+    b = _chk(b, torch.int8, "b")
+    if a.dim() == 2:
+        batch, (M, K), N = 1, a.shape, b.shape[0]
+        out = torch.empty((M, N), dtype=torch.int32)
+    else:
+        batch, M, K = a.shape
+        N = b.shape[1]
+        out = torch.empty((batch, M, N), dtype=torch.int32)
+    assert b.shape[-1] == K
+    _load().orc_gemm_s8_acc(_p(a), _p(b), _p(out), _i64(batch), _i64(M), _i64(N), _i64(K))
+    return out
+
+
+def gemm_acc_naive64(a, b):
+    a = _chk(a, torch.int8, "a")
+    b = _chk(b, torch.int8, "b")
+    if a.dim() == 2:
+        a3, b3 = a[None], b[None]
+    else:
+        a3, b3 = a, b
+    batch, M, K = a3.shape
+    N = b3.shape[1]
+    out = torch.empty((batch, M, N), dtype=torch.int64)
+    _load().orc_gemm_s8_acc_naive64(_p(a3.contiguous()), _p(b3.contiguous()), _p(out),
+                                    _i64(batch), _i64(M), _i64(N), _i64(K))
+    return out if a.dim() == 3 else out[0]
+
+
+def gemm_acc_torch(a, b):
+    """The reference's CPU integer emulation: torch int32 matmul."""
+    return torch.matmul(a.to(torch.int32), b.to(torch.int32).transpose(-1, -2))
+
+
+# ---- epilogues on a ready accumulator (used with either accumulation route) ----
+
+def epi_b32_o32(acc, bias):
+    acc = _chk(acc, torch.int32, "acc")
+    bias = _chk(bias.reshape(-1), torch.int32, "bias")
+    out = torch.empty_like(acc)
+    N = acc.shape[-1]
+    _load().orc_epi_b32_o32(_p(acc), _p(bias), _p(out), _i64(acc.numel() // N), _i64(N))
+    return out
+
+
+def epi_b32_o32_scaled(acc, bias, alpha, beta):
+    acc = _chk(acc, torch.int32, "acc")
+    bias = _chk(bias.reshape(-1), torch.int32, "bias")
+    out = torch.empty_like(acc)
+    N = acc.shape[-1]
+    _load().orc_epi_b32_o32_scaled(_p(acc), _p(bias), _p(out), _i64(acc.numel() // N), _i64(N),
+                                   _f32(alpha), _f32(beta))
+    return out
+
+
+def epi_bfp32_ofp32(acc, bias, alpha, beta):
+    acc = _chk(acc, torch.int32, "acc")
+    bias = _chk(bias.reshape(-1), torch.float32, "bias")
+    out = torch.empty(acc.shape, dtype=torch.float32)
+    N = acc.shape[-1]
+    _load().orc_epi_bfp32_ofp32(_p(acc), _p(bias), _p(out), _i64(acc.numel() // N), _i64(N),
+                                _f32(alpha), _f32(beta))
+    return out
+
+
+def epi_b8_o8(acc, bias, alpha, beta, relu=False):
+    acc = _chk(acc, torch.int32, "acc")
+    bias = _chk(bias.reshape(-1), torch.int8, "bias")
+    out = torch.empty(acc.shape, dtype=torch.int8)
+    N = acc.shape[-1]
+    fn = _load().orc_epi_relu_b8_o8 if relu else _load().orc_epi_b8_o8
+    fn(_p(acc), _p(bias), _p(out), _i64(acc.numel() // N), _i64(N), _f32(alpha), _f32(beta))
+    return out
+
+
+def epi_f32t(acc, alpha):
+    acc = _chk(acc, torch.int32, "acc")
+    out = torch.empty(acc.shape, dtype=torch.float32)
+    _load().orc_epi_f32t(_p(acc), _p(out), _i64(acc.numel()), _f32(alpha))
+    return out
+
+
+def epi_s8t(acc, alpha):
+    acc = _chk(acc, torch.int32, "acc")
+    out = torch.empty(acc.shape, dtype=torch.int8)
+    _load().orc_epi_s8t(_p(acc), _p(out), _i64(acc.numel()), _f32(alpha))
+    return out
+
+
+# ---- the nine entry points ----
+
+def linear_a8_w8_b32_o32(x, w, bias, acc_fn=gemm_acc):
+    return epi_b32_o32(acc_fn(x, w), bias)
+
+
+def linear_a8_w8_b32_o32_with_scaling(x, w, bias, alpha, beta, acc_fn=gemm_acc):
+    return epi_b32_o32_scaled(acc_fn(x, w), bias, alpha, beta)
+
+
+def linear_a8_w8_bfp32_ofp32(x, w, bias, alpha, beta, acc_fn=gemm_acc):
+    return epi_bfp32_ofp32(acc_fn(x, w), bias, alpha, beta)
+
+
+def linear_a8_w8_b8_o8(x, w, bias, alpha, beta, acc_fn=gemm_acc):
+    return epi_b8_o8(acc_fn(x, w), bias, alpha, beta)
+
+
+def linear_relu_a8_w8_b8_o8(x, w, bias, alpha, beta, acc_fn=gemm_acc):
+    return epi_b8_o8(acc_fn(x, w), bias, alpha, beta, relu=True)
+
+
+def bmm_s8t_s8n_f32t(a, b, alpha, acc_fn=gemm_acc):
+    return epi_f32t(acc_fn(a, b), alpha)
+
+
+def bmm_s8t_s8n_s8t(a, b, alpha, acc_fn=gemm_acc):
+    return epi_s8t(acc_fn(a, b), alpha)
+
+
+def bmm_s8t_s8n_s32t(a, b, acc_fn=gemm_acc):
+    return acc_fn(a, b)
+
+
+def dq_add_layernorm_q(inp, input_scale, residual, gamma, beta, eps):
+    inp = _chk(inp, torch.int32, "input")
+    residual = _chk(residual, torch.float32, "residual")
+    gamma = _chk(gamma, torch.float32, "gamma")
+    beta = _chk(beta, torch.float32, "beta")
+    H = inp.shape[-1]
+    assert residual.shape == inp.shape and gamma.numel() == H and beta.numel() == H
+    r = torch.empty(inp.shape, dtype=torch.float32)
+    q = torch.empty(inp.shape, dtype=torch.int8)
+    rows = inp.numel() // H if H else 0
+    _load().orc_dq_add_layernorm_q(_p(inp), _f32(input_scale), _p(residual), _p(gamma), _p(beta),
+                                   _f32(eps), _p(r), _p(q), _i64(rows), _i64(H))
+    return r, q

@@ -1,0 +1,258 @@
+/*
+ * TEST INFRASTRUCTURE ONLY.  CPU restatement of the arithmetic of torch-int's
+ * INT8 W8A8 operators.  Nothing in the shipped package may link, load or call
+ * this file; it exists so tests, the smoke check and the bench's CPU-baseline
+ * leg have an independent answer to compare the HIP kernels with.
+ *
+ * Each function cites the reference file it follows (paths relative to the
+ * upstream torch-int tree).
+ *
+ * Canonical arithmetic (shared with the kernels):
+ *   acc[m,n] = sum_k int32(A[m,k]) * int32(W[n,k])          exact, wrapping int32
+ *   f32(i)   = int32 -> fp32, round-to-nearest-even
+ *   t        = fmaf(alpha, f32(acc), beta (*) f32(bias))    (*) = separately rounded fp32 multiply
+ *   rne      = rintf under the default rounding mode (ties to even)
+ *   sat_s8   = clamp to [-128, 127]
+ *
+ * Parity status of the restatement:
+ *   - integer accumulation, s32 outputs: pinned (closed form; cross-checked in
+ *     tests against numpy int64 matmul, torch CPU int32 matmul and an fp64
+ *     route, and against the 16x16x16 literal matrices held by the
+ *     reference's tests/test_bmm.py:36-106).
+ *   - fp32 epilogues (fma form, rounding, saturation): pinned by special cases
+ *     the mathematics fixes (alpha=1/beta=0 identity, alpha=0, exact .5 ties,
+ *     saturation edges, ReLU) and by the orderings the reference tests state
+ *     (tests/test_linear_kernels.py:64,81; tests/test_bmm.py:15).  The
+ *     sub-LSB choice "fma vs mul+add" is what CUTLASS' LinearCombination
+ *     compiles to; CUTLASS is an un-vendored submodule of the reference
+ *     (.gitmodules:1-4, no pinned commit), so that one choice is
+ *     "parity unpinned" against the original binary and is fixed here by
+ *     definition.
+ *   - dq_add_layernorm_q: r is pinned to torch.add(res, in, alpha=s) (<=1 ulp);
+ *     q is pinned to torch layer_norm within +-1 LSB (summation order differs),
+ *     and bit-exactly to the fixed reduction tree defined below.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stddef.h>
+#include <string.h>
+
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+/* ---------------------------------------------------------------- helpers */
+
+static inline float f32_of_i32(int32_t v) { return (float)v; } /* RNE per C11 Annex F */
+
+static inline int8_t sat_rne_s8(float t) {
+  /* clamp first, then round half-to-even: reference tests/test_linear_kernels.py:64
+     (`.clamp(-128, 127).round()`); NaN -> 0 like a saturating float->int convert */
+  if (t != t) return 0;
+  if (t < -128.0f) t = -128.0f;
+  if (t > 127.0f) t = 127.0f;
+  return (int8_t)rintf(t);
+}
+
+static inline int32_t sat_rne_s32(float t) {
+  if (t != t) return 0;
+  if (t >= 2147483648.0f) return INT32_MAX;
+  if (t <= -2147483648.0f) return INT32_MIN;
+  return (int32_t)rintf(t);
+}
+
+int orc_num_threads(void) {
+#ifdef _OPENMP
+  return omp_get_max_threads();
+#else
+  return 1;
+#endif
+}
+
+/* -------------------------------------------------- integer accumulation */
+
+/* acc[b,m,n] = sum_k A[b,m,k] * B[b,n,k].
+ * Follows torch_int/kernels/linear.cu:17-19,30-32 (A row-major [M,K], weight
+ * row-major [N,K] used as column-major [K,N]) and torch_int/kernels/bmm.cu:11-20,
+ * 71-73 (batch strides M*K, N*K, M*N). */
+void orc_gemm_s8_acc(const int8_t* A, const int8_t* B, int32_t* acc,
+                     int64_t batch, int64_t M, int64_t N, int64_t K) {
+  int64_t rows = batch * M;
+#pragma omp parallel for schedule(static)
+  for (int64_t bm = 0; bm < rows; ++bm) {
+    int64_t b = bm / M;
+    const int8_t* a = A + bm * K;
+    const int8_t* Bb = B + b * N * K;
+    int32_t* out = acc + bm * N;
+    for (int64_t n = 0; n < N; ++n) {
+      const int8_t* w = Bb + n * K;
+      int32_t s = 0;
+      for (int64_t k = 0; k < K; ++k) s += (int32_t)a[k] * (int32_t)w[k];
+      out[n] = s;
+    }
+  }
+}
+
+/* Plain triple loop with 64-bit accumulation and no vectorisable structure:
+ * used only by tests as a second, differently-written route. */
+void orc_gemm_s8_acc_naive64(const int8_t* A, const int8_t* B, int64_t* acc,
+                             int64_t batch, int64_t M, int64_t N, int64_t K) {
+  for (int64_t b = 0; b < batch; ++b)
+    for (int64_t n = 0; n < N; ++n)
+      for (int64_t m = 0; m < M; ++m) {
+        volatile int64_t s = 0;
+        for (int64_t k = K - 1; k >= 0; --k)
+          s = s + (int64_t)A[(b * M + m) * K + k] * (int64_t)B[(b * N + n) * K + k];
+        acc[(b * M + m) * N + n] = s;
+      }
+}
+
+/* ------------------------------------------------------------- epilogues */
+/* All take acc [rows, N] (rows = batch*M) and a per-column bias [N]. */
+
+/* torch_int/kernels/linear.cu:13-136: out = acc + bias, int32 (alpha = 1,
+ * NoBetaScaling, :41-44,100); wrapping two's-complement add. */
+void orc_epi_b32_o32(const int32_t* acc, const int32_t* bias, int32_t* out,
+                     int64_t rows, int64_t N) {
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < rows; ++r)
+    for (int64_t n = 0; n < N; ++n)
+      out[r * N + n] = (int32_t)((uint32_t)acc[r * N + n] + (uint32_t)bias[n]);
+}
+
+/* torch_int/kernels/linear.cu:139-243: LinearCombination<int32,4,int32,float>
+ * (:169-171): fp32 combine, round to nearest, saturate to int32. */
+void orc_epi_b32_o32_scaled(const int32_t* acc, const int32_t* bias, int32_t* out,
+                            int64_t rows, int64_t N, float alpha, float beta) {
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < rows; ++r)
+    for (int64_t n = 0; n < N; ++n) {
+      float bb = beta * f32_of_i32(bias[n]);
+      out[r * N + n] = sat_rne_s32(fmaf(alpha, f32_of_i32(acc[r * N + n]), bb));
+    }
+}
+
+/* torch_int/kernels/linear.cu:246-365: LinearCombination<float,4,int32,float>
+ * (:276-278): out = alpha*acc + beta*bias in fp32. */
+void orc_epi_bfp32_ofp32(const int32_t* acc, const float* bias, float* out,
+                         int64_t rows, int64_t N, float alpha, float beta) {
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < rows; ++r)
+    for (int64_t n = 0; n < N; ++n) {
+      float bb = beta * bias[n];
+      out[r * N + n] = fmaf(alpha, f32_of_i32(acc[r * N + n]), bb);
+    }
+}
+
+/* torch_int/kernels/linear.cu:369-473 (clamp epilogue, :399-400):
+ * out = s8(rne(clamp(alpha*acc + beta*bias, -128, 127))). */
+void orc_epi_b8_o8(const int32_t* acc, const int8_t* bias, int8_t* out,
+                   int64_t rows, int64_t N, float alpha, float beta) {
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < rows; ++r)
+    for (int64_t n = 0; n < N; ++n) {
+      float bb = beta * f32_of_i32((int32_t)bias[n]);
+      out[r * N + n] = sat_rne_s8(fmaf(alpha, f32_of_i32(acc[r * N + n]), bb));
+    }
+}
+
+/* torch_int/kernels/linear.cu:476-625 (LinearCombinationRelu, :500-511):
+ * out = sat_s8(rne(max(alpha*acc + beta*bias, 0))), values in [0,127]
+ * (reference tests/test_linear_kernels.py:81 `.clamp(0, 127).round()`). */
+void orc_epi_relu_b8_o8(const int32_t* acc, const int8_t* bias, int8_t* out,
+                        int64_t rows, int64_t N, float alpha, float beta) {
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < rows; ++r)
+    for (int64_t n = 0; n < N; ++n) {
+      float bb = beta * f32_of_i32((int32_t)bias[n]);
+      float t = fmaf(alpha, f32_of_i32(acc[r * N + n]), bb);
+      if (!(t > 0.0f)) t = 0.0f; /* NaN -> 0 as well */
+      out[r * N + n] = sat_rne_s8(t);
+    }
+}
+
+/* torch_int/kernels/bmm.cu:10-108: beta = 0, so the source operand is never
+ * read (:33-35,81): out = alpha * f32(acc), one fp32 multiply. */
+void orc_epi_f32t(const int32_t* acc, float* out, int64_t count, float alpha) {
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < count; ++i) out[i] = alpha * f32_of_i32(acc[i]);
+}
+
+/* torch_int/kernels/bmm.cu:110-208 (LinearCombinationClamp, :133-135,181):
+ * out = sat_s8(rne(alpha * f32(acc))); reference tests/test_bmm.py:14-15. */
+void orc_epi_s8t(const int32_t* acc, int8_t* out, int64_t count, float alpha) {
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < count; ++i) out[i] = sat_rne_s8(alpha * f32_of_i32(acc[i]));
+}
+
+/* torch_int/kernels/bmm.cu:210-295: out = acc (the s32 BMM needs no epilogue). */
+
+/* ------------------------------------------------- dq_add_layernorm_q */
+
+/* Fixed reduction tree over one row of H values, written so a 256-lane
+ * workgroup (4 wavefronts of 64) can reproduce it bit for bit:
+ *   - the row is cut into chunks of 4 consecutive elements; chunk c belongs to
+ *     lane (c mod 256) and is that lane's (c div 256)-th chunk;
+ *   - a lane adds its elements to a running fp32 sum in ascending index order;
+ *   - the 64 lanes of a wavefront are combined by a xor-butterfly with
+ *     offsets 32,16,8,4,2,1 (fp32 add is commutative, so every lane ends with
+ *     the same bits);
+ *   - the 4 wavefront sums are added left to right.
+ * `term(i)` is v[i] for the mean and (v[i]-mu)^2 (one rounding for the
+ * subtraction, one for the product) for the variance. */
+static float tree_sum(const float* v, int64_t H, int use_sq, float mu) {
+  float lane[256];
+  for (int t = 0; t < 256; ++t) lane[t] = 0.0f;
+  int64_t nchunks = (H + 3) / 4;
+  for (int64_t c = 0; c < nchunks; ++c) {
+    int t = (int)(c % 256);
+    for (int j = 0; j < 4; ++j) {
+      int64_t i = c * 4 + j;
+      if (i >= H) break;
+      float x = v[i];
+      if (use_sq) {
+        float d = x - mu;
+        x = d * d;
+      }
+      lane[t] = lane[t] + x;
+    }
+  }
+  float wsum[4];
+  for (int w = 0; w < 4; ++w) {
+    float cur[64], nxt[64];
+    for (int l = 0; l < 64; ++l) cur[l] = lane[w * 64 + l];
+    for (int off = 32; off >= 1; off >>= 1) {
+      for (int l = 0; l < 64; ++l) nxt[l] = cur[l] + cur[l ^ off];
+      memcpy(cur, nxt, sizeof(cur));
+    }
+    wsum[w] = cur[0];
+  }
+  return ((wsum[0] + wsum[1]) + wsum[2]) + wsum[3];
+}
+
+/* torch_int/kernels/fused.cu:5-25 and torch_int/functional/fused.py:5-12:
+ *   r = res + s * f32(in)            (torch.add with alpha: one fused multiply-add)
+ *   y = layer_norm(r; gamma, beta, eps) over the last dim, biased variance
+ *   q = s8(rne(clamp(y, -128, 127)))
+ * returns (r, q).  mean = sum/H, var = sum((r-mean)^2)/H, rstd = 1/sqrtf(var+eps),
+ * y = fmaf((r-mean)*rstd, gamma, beta). */
+void orc_dq_add_layernorm_q(const int32_t* in, float scale, const float* res,
+                            const float* gamma, const float* beta, float eps,
+                            float* r_out, int8_t* q_out, int64_t rows, int64_t H) {
+#pragma omp parallel for schedule(static)
+  for (int64_t row = 0; row < rows; ++row) {
+    const int32_t* x = in + row * H;
+    const float* rs = res + row * H;
+    float* r = r_out + row * H;
+    int8_t* q = q_out + row * H;
+    for (int64_t i = 0; i < H; ++i) r[i] = fmaf(scale, f32_of_i32(x[i]), rs[i]);
+    float fH = (float)H;
+    float mu = tree_sum(r, H, 0, 0.0f) / fH;
+    float var = tree_sum(r, H, 1, mu) / fH;
+    float rstd = 1.0f / sqrtf(var + eps);
+    for (int64_t i = 0; i < H; ++i) {
+      float y = fmaf((r[i] - mu) * rstd, gamma[i], beta[i]);
+      q[i] = sat_rne_s8(y);
+    }
+  }
+}

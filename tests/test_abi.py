@@ -1,0 +1,85 @@
+"""CPU-side checks of the C-ABI library and the host validation in torch_int._CUDA
+(no kernel is launched here)."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "torch_int_hip.h")
+
+
+def _declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ti_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    import torch_int._CUDA as C
+    lib = ctypes.CDLL(C.LIB_PATH)
+    names = _declared_symbols()
+    assert len(names) >= 13
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/torch_int_hip.h but not exported"
+    assert C._lib.ti_version() >= 100
+    assert C._lib.ti_last_error() == b""
+
+
+def test_python_module_mirrors_upstream_bindings():
+    import torch_int._CUDA as C
+    import torch_int.kernels as K
+    expected = {"linear_relu_a8_w8_b8_o8", "linear_a8_w8_b32_o32", "linear_a8_w8_bfp32_ofp32",
+                "linear_a8_w8_b32_o32_with_scaling", "linear_a8_w8_b8_o8", "dq_add_layernorm_q",
+                "bmm_s8t_s8n_s8t", "bmm_s8t_s8n_f32t", "bmm_s8t_s8n_s32t"}  # upstream bindings.cpp:5-20
+    assert set(C.__all__) == expected
+    for n in expected:
+        assert callable(getattr(C, n)) and getattr(K, n) is getattr(C, n)
+    # the reference's own import lines work unchanged
+    from torch_int._CUDA import bmm_s8t_s8n_s8t, linear_a8_w8_b8_o8  # noqa: F401
+    from torch_int.functional.bmm import bmm_i8_o8, bmm_i8_o32  # noqa: F401
+    from torch_int.functional.fused import dq_add_layernorm_q_cpp, dq_add_layernorm_q_py  # noqa: F401
+    from torch_int.nn.linear import W8A8B8O8Linear, W8A8BFP32OFP32Linear  # noqa: F401
+
+
+def test_c_abi_rejects_bad_arguments_without_a_device():
+    import torch_int._CUDA as C
+    lib = C._lib
+    buf = ctypes.create_string_buffer(64)
+    p = ctypes.addressof(buf)
+    # negative size
+    rc = lib.ti_bmm_s8t_s8n_s32t(p, p, p, 1, -1, 4, 16, None)
+    assert rc == 1 and b"negative" in lib.ti_last_error()
+    # NULL operand with a non-empty problem
+    rc = lib.ti_linear_a8_w8_b8_o8(None, p, p, p, 4, 4, 16, 1.0, 1.0, None, 0, None)
+    assert rc == 1 and b"NULL" in lib.ti_last_error()
+    # misaligned int32 output
+    rc = lib.ti_bmm_s8t_s8n_s32t(p, p, p + 1, 1, 1, 4, 16, None)
+    assert rc == 2 and b"aligned" in lib.ti_last_error()
+    # beyond the 32-bit tiling limits
+    rc = lib.ti_linear_a8_w8_b32_o32(p, p, p, p, 1 << 20, 4, 1 << 20, None, 0, None)
+    assert rc == 1 and b"limits" in lib.ti_last_error()
+    # empty problems succeed without touching pointers or a device
+    assert lib.ti_linear_a8_w8_b8_o8(None, None, None, None, 0, 16, 16, 1.0, 1.0, None, 0, None) == 0
+    assert lib.ti_dq_add_layernorm_q(None, 1.0, None, None, None, 1e-5, None, None, 0, 128, None) == 0
+    assert lib.ti_last_error() == b""
+
+
+def test_host_validation_raises_and_never_computes_on_cpu():
+    import torch_int._CUDA as C
+    x = torch.zeros(4, 16, dtype=torch.int8)
+    w = torch.zeros(8, 16, dtype=torch.int8)
+    b = torch.zeros(8, dtype=torch.int8)
+    with pytest.raises(RuntimeError, match="only run on a HIP"):
+        C.linear_a8_w8_b8_o8(x, w, b, 1.0, 1.0)
+    with pytest.raises(RuntimeError, match="must be torch.int8"):
+        C.linear_a8_w8_b8_o8(x.float(), w, b, 1.0, 1.0)
+    with pytest.raises(RuntimeError, match="2-D"):
+        C.linear_a8_w8_b8_o8(x[None], w, b, 1.0, 1.0)
+    with pytest.raises(RuntimeError, match="only run on a HIP"):
+        C.bmm_s8t_s8n_s32t(x[None], w[None])
+    with pytest.raises(RuntimeError, match="only run on a HIP"):
+        C.dq_add_layernorm_q(torch.zeros(2, 8, dtype=torch.int32), 1.0, torch.zeros(2, 8), torch.ones(8),
+                             torch.zeros(8), 1e-5)

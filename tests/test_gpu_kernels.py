@@ -1,0 +1,311 @@
+"""Parity of the HIP kernels with the CPU oracle, through torch_int._CUDA -> C ABI.
+
+Bars: bit-exact for int32 and int8 outputs; fp32 outputs within 1 ulp (in practice 0:
+the kernels and the oracle spell the same fma).  Inputs are generated on the CPU from a
+seeded generator and copied to the GPU, so both sides see identical bytes.
+"""
+import json
+import os
+import sys
+
+import pytest
+import torch
+
+from oracle import oracle as orc
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+DEV = "cuda:0"
+
+
+def _say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def _s8(g, *shape, lo=-127, hi=128):
+    return torch.randint(lo, hi, shape, dtype=torch.int8, generator=g)
+
+
+def _scal(g, lo, hi):
+    return float(torch.empty(1).uniform_(lo, hi, generator=g).item())
+
+
+def _ulp_diff(a, b):
+    """max distance in units of the last place between two fp32 tensors."""
+    ai = a.contiguous().view(torch.int32).long()
+    bi = b.contiguous().view(torch.int32).long()
+    ai = torch.where(ai < 0, -(ai & 0x7fffffff), ai)
+    bi = torch.where(bi < 0, -(bi & 0x7fffffff), bi)
+    return (ai - bi).abs().max().item() if a.numel() else 0
+
+
+def _linear_case(C, variant, M, N, K, seed, alpha=None, beta=None):
+    g = torch.Generator().manual_seed(seed)
+    x, w = _s8(g, M, K), _s8(g, N, K)
+    alpha = _scal(g, 1e-4, 1e-2) if alpha is None else alpha
+    beta = _scal(g, 1e-4, 1e-2) if beta is None else beta
+    if variant == "b32_o32":
+        bias = torch.randint(-65535, 65535, (N,), dtype=torch.int32, generator=g)
+        ref = orc.linear_a8_w8_b32_o32(x, w, bias)
+        out = C.linear_a8_w8_b32_o32(x.to(DEV), w.to(DEV), bias.to(DEV))
+    elif variant == "b32_o32_scaled":
+        bias = torch.randint(-2 ** 31, 2 ** 31 - 1, (N,), dtype=torch.int64, generator=g).to(torch.int32)
+        ref = orc.linear_a8_w8_b32_o32_with_scaling(x, w, bias, alpha, beta)
+        out = C.linear_a8_w8_b32_o32_with_scaling(x.to(DEV), w.to(DEV), bias.to(DEV), alpha, beta)
+    elif variant == "bfp32_ofp32":
+        bias = torch.randn(N, generator=g)
+        ref = orc.linear_a8_w8_bfp32_ofp32(x, w, bias, alpha, beta)
+        out = C.linear_a8_w8_bfp32_ofp32(x.to(DEV), w.to(DEV), bias.to(DEV), alpha, beta)
+    elif variant == "b8_o8":
+        bias = _s8(g, N)
+        ref = orc.linear_a8_w8_b8_o8(x, w, bias, alpha, beta)
+        out = C.linear_a8_w8_b8_o8(x.to(DEV), w.to(DEV), bias.to(DEV), alpha, beta)
+    elif variant == "relu_b8_o8":
+        bias = _s8(g, N)
+        ref = orc.linear_relu_a8_w8_b8_o8(x, w, bias, alpha, beta)
+        out = C.linear_relu_a8_w8_b8_o8(x.to(DEV), w.to(DEV), bias.to(DEV), alpha, beta)
+    else:
+        raise AssertionError(variant)
+    out = out.cpu()
+    assert out.shape == ref.shape and out.dtype == ref.dtype
+    if out.dtype == torch.float32:
+        assert _ulp_diff(out, ref) <= 1, f"{variant} {M}x{N}x{K}: {_ulp_diff(out, ref)} ulp"
+    else:
+        nbad = (out != ref).sum().item()
+        assert nbad == 0, f"{variant} {M}x{N}x{K}: {nbad} mismatches"
+    return out
+
+
+VARIANTS = ["b32_o32", "b32_o32_scaled", "bfp32_ofp32", "b8_o8", "relu_b8_o8"]
+
+# (M, N, K): upstream minimum shapes (tests/test_linear_shape.py:9,26), upstream kernel
+# test shape (tests/test_linear_kernels.py:8), ragged edges, every tile family.
+LINEAR_SHAPES = [
+    (1, 4, 16), (1, 16, 16), (128, 1024, 512), (3, 20, 48), (65, 100, 272), (64, 64, 128),
+    (130, 260, 400), (257, 513, 1040), (300, 768, 768), (512, 1024, 256),
+]
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+def test_linear_shapes(variant):
+    import torch_int._CUDA as C
+    for i, (M, N, K) in enumerate(LINEAR_SHAPES):
+        _say(f"linear {variant} M={M} N={N} K={K}")
+        _linear_case(C, variant, M, N, K, seed=100 + i)
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+def test_linear_large_tiles(variant):
+    # enough 256x256 tiles to select the large-tile kernel, with ragged M and N
+    import torch_int._CUDA as C
+    for (M, N, K) in [(2048, 5120, 256), (2100, 5000, 272), (4096, 2560, 128)]:
+        _say(f"linear-large {variant} M={M} N={N} K={K}")
+        _linear_case(C, variant, M, N, K, seed=7)
+
+
+def test_linear_opt125m_config():
+    # BASELINE config 1: x [4,512,768], W [768,768], bias [768], alpha 1e-3, beta 1e-2, seed 0
+    import torch_int._CUDA as C
+    _say("linear C1")
+    out = _linear_case(C, "b8_o8", 2048, 768, 768, seed=0, alpha=0.001, beta=0.01)
+    assert (out == 127).any() and (out == -128).any()  # saturates by design
+
+
+def test_linear_odd_k_and_bias_shapes():
+    import torch_int._CUDA as C
+    for (M, N, K) in [(5, 7, 13), (33, 17, 100), (1, 128, 513)]:
+        for v in VARIANTS:
+            _say(f"linear-odd {v} M={M} N={N} K={K}")
+            _linear_case(C, v, M, N, K, seed=11)
+    g = torch.Generator().manual_seed(5)
+    x, w, b = _s8(g, 8, 32), _s8(g, 16, 32), _s8(g, 16)
+    ref = orc.linear_a8_w8_b8_o8(x, w, b, 0.01, 0.5)
+    out = C.linear_a8_w8_b8_o8(x.to(DEV), w.to(DEV), b.view(1, 16).to(DEV), 0.01, 0.5)  # [1,N] bias as modules hold it
+    assert torch.equal(out.cpu(), ref)
+    out = C.linear_a8_w8_b8_o8(x.to(DEV), w.to(DEV), b, 0.01, 0.5)  # CPU bias is moved like upstream does
+    assert torch.equal(out.cpu(), ref)
+    assert C.linear_a8_w8_b8_o8(x[:0].to(DEV), w.to(DEV), b.to(DEV), 1.0, 1.0).shape == (0, 16)
+
+
+def test_linear_ties_and_saturation_on_device():
+    import torch_int._CUDA as C
+    # K = 16 ones against small integers: acc = sum of a row, alpha = 0.5 produces exact .5 ties
+    x = torch.zeros(64, 16, dtype=torch.int8)
+    x[:, 0] = torch.arange(-32, 32, dtype=torch.int8)
+    x[:, 1] = 127
+    x[:, 2] = torch.arange(0, 64, dtype=torch.int8)
+    w = torch.zeros(16, 16, dtype=torch.int8)
+    w[:, 0] = 1
+    w[8:, 1] = 2
+    w[4:12, 2] = -3
+    bias = torch.arange(-8, 8, dtype=torch.int8)
+    for alpha, beta in [(0.5, 0.5), (0.5, 0.0), (1.0, 0.0), (0.25, 1.0), (0.0, 0.5)]:
+        for fn_name in ["linear_a8_w8_b8_o8", "linear_relu_a8_w8_b8_o8"]:
+            _say(f"ties {fn_name} alpha={alpha} beta={beta}")
+            ref = getattr(orc, fn_name)(x, w, bias, alpha, beta)
+            out = getattr(C, fn_name)(x.to(DEV), w.to(DEV), bias.to(DEV), alpha, beta).cpu()
+            assert torch.equal(out, ref)
+    ib = bias.to(torch.int32) * 1000
+    ref = orc.linear_a8_w8_b32_o32_with_scaling(x, w, ib, 0.5, 0.0005)
+    out = C.linear_a8_w8_b32_o32_with_scaling(x.to(DEV), w.to(DEV), ib.to(DEV), 0.5, 0.0005).cpu()
+    assert torch.equal(out, ref)
+    ref = orc.linear_a8_w8_b32_o32_with_scaling(x, w, ib, 3e7, 1.0)  # saturates int32
+    out = C.linear_a8_w8_b32_o32_with_scaling(x.to(DEV), w.to(DEV), ib.to(DEV), 3e7, 1.0).cpu()
+    assert torch.equal(out, ref) and (out == 2 ** 31 - 1).any() and (out == -2 ** 31).any()
+
+
+def test_linear_large_accumulators_round_like_the_oracle():
+    # |acc| > 2^24: the int32 -> fp32 conversion is inexact and must round to nearest even
+    import torch_int._CUDA as C
+    M, N, K = 32, 32, 4096
+    x = torch.full((M, K), 127, dtype=torch.int8)
+    w = torch.full((N, K), 127, dtype=torch.int8)
+    g = torch.Generator().manual_seed(2)
+    x[:, :64] = _s8(g, M, 64)
+    w[:, 64:128] = _s8(g, N, 64)
+    bias = torch.randn(N, generator=g)
+    ref = orc.linear_a8_w8_bfp32_ofp32(x, w, bias, 1.0, 1.0)
+    assert ref.abs().max() > 2 ** 25
+    out = C.linear_a8_w8_bfp32_ofp32(x.to(DEV), w.to(DEV), bias.to(DEV), 1.0, 1.0).cpu()
+    assert _ulp_diff(out, ref) == 0
+    ib = torch.zeros(N, dtype=torch.int32)
+    assert torch.equal(C.linear_a8_w8_b32_o32(x.to(DEV), w.to(DEV), ib.to(DEV)).cpu(),
+                       orc.linear_a8_w8_b32_o32(x, w, ib))
+
+
+# ------------------------------------------------------------------ batched products
+
+def _bmm_case(C, B, M, N, K, seed, prob_lhs=False):
+    g = torch.Generator().manual_seed(seed)
+    a = _s8(g, B, M, K, lo=0 if prob_lhs else -127)
+    b = _s8(g, B, N, K)
+    alpha = _scal(g, 1e-3 if prob_lhs else 1e-4, 1e-2)
+    ad, bd = a.to(DEV), b.to(DEV)
+    ref32 = orc.bmm_s8t_s8n_s32t(a, b)
+    assert torch.equal(C.bmm_s8t_s8n_s32t(ad, bd).cpu(), ref32), f"s32t {B}x{M}x{N}x{K}"
+    out8 = C.bmm_s8t_s8n_s8t(ad, bd, alpha).cpu()
+    assert torch.equal(out8, orc.epi_s8t(ref32, alpha)), f"s8t {B}x{M}x{N}x{K}"
+    outf = C.bmm_s8t_s8n_f32t(ad, bd, alpha).cpu()
+    assert _ulp_diff(outf, orc.epi_f32t(ref32, alpha)) == 0, f"f32t {B}x{M}x{N}x{K}"
+
+
+def test_bmm_shapes():
+    import torch_int._CUDA as C
+    # upstream minimum shapes (tests/test_bmm_shape.py:8,19), kernel test shapes
+    # (tests/test_bmm.py:8,114), ragged, decode-like (M=1, src_len not a multiple of 16)
+    shapes = [(1, 1, 4, 16), (1, 1, 16, 16), (1, 512, 32, 512), (1, 512, 12288, 512), (3, 70, 50, 96),
+              (5, 33, 129, 128), (8, 1, 513, 128), (8, 1, 128, 513), (2, 130, 130, 528), (16, 128, 128, 128)]
+    for i, (B, M, N, K) in enumerate(shapes):
+        _say(f"bmm B={B} M={M} N={N} K={K}")
+        _bmm_case(C, B, M, N, K, seed=200 + i)
+
+
+def test_bmm_literal_fixture_from_upstream_tests():
+    import torch_int._CUDA as C
+    with open(os.path.join(GOLDEN, "bmm_literal_16x16.json")) as f:
+        fx = json.load(f)
+    a = torch.tensor(fx["a"], dtype=torch.int8)[None].to(DEV)
+    b_nk = torch.tensor(fx["b_kn"], dtype=torch.int8).t().contiguous()[None].to(DEV)
+    assert C.bmm_s8t_s8n_s32t(a, b_nk)[0].cpu().tolist() == fx["acc"]
+    assert C.bmm_s8t_s8n_s8t(a, b_nk, fx["scale"])[0].cpu().tolist() == fx["expected_s8"]
+
+
+@pytest.mark.parametrize("S", [128, 512])
+def test_bmm_attention_config(S):
+    # BASELINE config 3 at a reduced batch*heads (the full 160 is covered by properties below)
+    import torch_int._CUDA as C
+    BH, d = 8, 128
+    _say(f"attention bmm S={S}")
+    _bmm_case(C, BH, S, S, d, seed=31)                  # Q.K^T
+    _bmm_case(C, BH, S, d, S, seed=32, prob_lhs=True)   # P.V^T^T
+
+
+def test_bmm_full_size_properties():
+    # B*H = 160, S = 512, d = 128 (BASELINE config 3): size-independent checks
+    import torch_int._CUDA as C
+    g = torch.Generator().manual_seed(9)
+    BH, S, d = 160, 512, 128
+    q, k = _s8(g, BH, S, d).to(DEV), _s8(g, BH, S, d).to(DEV)
+    _say("bmm full-size properties")
+    s32 = C.bmm_s8t_s8n_s32t(q, k)
+    # (Q K^T)^T = K Q^T
+    assert torch.equal(s32.transpose(1, 2), C.bmm_s8t_s8n_s32t(k, q))
+    # a checksum of checksums: sum over n of acc[b,m,n] = q[b,m,:] . sum_n k[b,n,:]
+    ksum = k.long().sum(1)
+    assert torch.equal(s32.long().sum(2), torch.einsum("bmk,bk->bm", q.long(), ksum))
+    # batches are independent: the first 3 batches alone give the same slices
+    assert torch.equal(C.bmm_s8t_s8n_s32t(q[:3].contiguous(), k[:3].contiguous()), s32[:3])
+    # the fp32 and int8 epilogues are pure functions of the accumulator
+    alpha = 0.00123
+    f = C.bmm_s8t_s8n_f32t(q, k, alpha)
+    assert torch.equal(f, s32.float() * alpha)
+    o8 = C.bmm_s8t_s8n_s8t(q, k, alpha)
+    assert torch.equal(o8, (s32.float() * alpha).clamp(-128, 127).round().to(torch.int8))
+    # three full batches against the oracle
+    ref = orc.bmm_s8t_s8n_s32t(q[157:].cpu(), k[157:].cpu())
+    assert torch.equal(s32[157:].cpu(), ref)
+
+
+# ------------------------------------------------------------------ dq_add_layernorm_q
+
+def _ln_case(C, shape, seed, spread=20.0):
+    g = torch.Generator().manual_seed(seed)
+    H = shape[-1]
+    inp = torch.randint(-65536, 65536, shape, dtype=torch.int32, generator=g)
+    res = torch.randn(shape, generator=g)
+    gamma = (1 + 0.02 * torch.randn(H, generator=g)) * spread
+    beta = 0.02 * torch.randn(H, generator=g) * spread
+    s = _scal(g, 1e-4, 1e-2)
+    r_ref, q_ref = orc.dq_add_layernorm_q(inp, s, res, gamma, beta, 1e-5)
+    r, q = C.dq_add_layernorm_q(inp.to(DEV), s, res.to(DEV), gamma.to(DEV), beta.to(DEV), 1e-5)
+    assert r.dtype == torch.float32 and q.dtype == torch.int8 and r.shape == shape and q.shape == shape
+    assert _ulp_diff(r.cpu(), r_ref) == 0, f"r {shape}"
+    nbad = (q.cpu() != q_ref).sum().item()
+    assert nbad == 0, f"q {shape}: {nbad} mismatches"
+    # and the upstream composition of torch ops, on the GPU, within +-1 LSB
+    from torch_int.functional.fused import dq_add_layernorm_q_py
+    r_t, q_t = dq_add_layernorm_q_py(inp.to(DEV), s, res.to(DEV), gamma.to(DEV), beta.to(DEV), 1e-5)
+    assert _ulp_diff(r, r_t) <= 1
+    assert (q.int() - q_t.int()).abs().max().item() <= 1
+    assert (q != q_t).float().mean().item() <= 0.01 + 1.0 / q.numel()
+
+
+def test_ln_q_shapes():
+    import torch_int._CUDA as C
+    # upstream test shape (tests/test_dq_add_ln_q.py:8), OPT widths, odd H, H beyond the register path
+    for i, shape in enumerate([(2, 3, 4), (7, 768), (4, 5, 5120), (3, 9216), (2, 12288), (5, 1023), (3, 1),
+                               (2, 16384), (2, 20000), (1, 17)]):
+        _say(f"ln_q shape={shape}")
+        _ln_case(C, shape, seed=300 + i)
+
+
+def test_ln_q_full_size_and_in_place():
+    import torch_int._CUDA as C
+    _say("ln_q C4 [4,512,5120]")
+    _ln_case(C, (4, 512, 5120), seed=0)
+    # r_out may alias the residual (C ABI contract): call the library directly
+    g = torch.Generator().manual_seed(1)
+    inp = torch.randint(-65536, 65536, (64, 5120), dtype=torch.int32, generator=g)
+    res = torch.randn(64, 5120, generator=g)
+    gamma, beta = torch.ones(5120) * 30, torch.zeros(5120)
+    r_ref, q_ref = orc.dq_add_layernorm_q(inp, 0.003, res, gamma, beta, 1e-5)
+    d_in, d_res, d_g, d_b = inp.to(DEV), res.to(DEV), gamma.to(DEV), beta.to(DEV)
+    q = torch.empty((64, 5120), dtype=torch.int8, device=DEV)
+    rc = C._lib.ti_dq_add_layernorm_q(d_in.data_ptr(), 0.003, d_res.data_ptr(), d_g.data_ptr(), d_b.data_ptr(),
+                                      1e-5, d_res.data_ptr(), q.data_ptr(), 64, 5120,
+                                      torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    assert torch.equal(d_res.cpu(), r_ref) and torch.equal(q.cpu(), q_ref)
+
+
+def test_runs_are_deterministic():
+    # identical bytes on repeated launches (an LDS race would show up here)
+    import torch_int._CUDA as C
+    g = torch.Generator().manual_seed(77)
+    x, w, b = _s8(g, 1024, 1024).to(DEV), _s8(g, 2048, 1024).to(DEV), _s8(g, 2048).to(DEV)
+    first = C.linear_a8_w8_b8_o8(x, w, b, 0.002, 0.01)
+    first32 = C.linear_a8_w8_b32_o32(x, w, b.to(torch.int32))
+    for _ in range(5):
+        assert torch.equal(C.linear_a8_w8_b8_o8(x, w, b, 0.002, 0.01), first)
+        assert torch.equal(C.linear_a8_w8_b32_o32(x, w, b.to(torch.int32)), first32)

@@ -1,0 +1,37 @@
+"""Builds libtorch_int_hip.so (gfx950) in-tree with hipcc.
+
+Run as a script (``python torch-int_amd/build.py``) or call ``build()``.
+The library lands in ``torch-int_amd/torch_int/lib/`` next to the Python
+package that loads it with ctypes.
+"""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB_DIR = os.path.join(HERE, "torch_int", "lib")
+LIB_PATH = os.path.join(LIB_DIR, "libtorch_int_hip.so")
+SOURCES = ["api.hip", "gemm_s8.hip", "ln_q.hip"]
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "-ffp-contract=off",              # the epilogues spell out every fma themselves
+    "-fno-fast-math",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-function",
+]
+
+
+def build(verbose=True, extra_flags=()):
+    os.makedirs(LIB_DIR, exist_ok=True)
+    cmd = [HIPCC, *FLAGS, *extra_flags, "-o", LIB_PATH] + [os.path.join(CSRC, s) for s in SOURCES]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    build(extra_flags=sys.argv[1:])

@@ -1,0 +1,167 @@
+// extern "C" surface of libtorch_int_hip.so: argument validation and dispatch.
+// Declarations and the contract of each entry point live in
+// include/torch_int_hip.h.
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include "ti_common.h"
+
+namespace ti {
+
+static thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+static int check_dims(const char* op, int64_t batch, int64_t M, int64_t N, int64_t K) {
+  if (batch < 0 || M < 0 || N < 0 || K < 0)
+    return fail(TI_ERR_INVALID_ARG, "%s: negative dimension (batch=%lld M=%lld N=%lld K=%lld)", op,
+                (long long)batch, (long long)M, (long long)N, (long long)K);
+  const int64_t lim = 0x7fffffffLL;
+  if (M > lim || N > lim || K > lim || batch > 65535 || M * K > lim || N * K > lim)
+    return fail(TI_ERR_INVALID_ARG,
+                "%s: size beyond kernel limits (batch<=65535, M*K and N*K < 2^31 per batch; got batch=%lld "
+                "M=%lld N=%lld K=%lld)",
+                op, (long long)batch, (long long)M, (long long)N, (long long)K);
+  return TI_OK;
+}
+
+static int check_ptr(const char* op, const char* name, const void* p, size_t align, bool needed) {
+  if (!needed) return TI_OK;
+  if (p == nullptr) return fail(TI_ERR_INVALID_ARG, "%s: %s is NULL", op, name);
+  if (reinterpret_cast<uintptr_t>(p) % align)
+    return fail(TI_ERR_ALIGNMENT, "%s: %s is not aligned to %zu bytes", op, name, align);
+  return TI_OK;
+}
+
+static int run_gemm(const char* op, int kind, const void* a, const void* b, const void* bias, size_t bias_elt,
+                    void* c, size_t out_elt, int64_t batch, int64_t M, int64_t N, int64_t K, float alpha,
+                    float beta, void* ws, int64_t ws_bytes, void* stream) {
+  g_err[0] = 0;
+  if (int rc = check_dims(op, batch, M, N, K)) return rc;
+  const bool nonempty = batch > 0 && M > 0 && N > 0;
+  if (int rc = check_ptr(op, "input", a, 1, nonempty && K > 0)) return rc;
+  if (int rc = check_ptr(op, "weight", b, 1, nonempty && K > 0)) return rc;
+  if (int rc = check_ptr(op, "bias", bias, bias_elt ? bias_elt : 1, nonempty && bias_elt > 0)) return rc;
+  if (int rc = check_ptr(op, "output", c, out_elt, nonempty)) return rc;
+  if (ws_bytes < 0) return fail(TI_ERR_INVALID_ARG, "%s: negative workspace size", op);
+  GemmParams p;
+  p.A = static_cast<const int8_t*>(a);
+  p.B = static_cast<const int8_t*>(b);
+  p.bias = bias;
+  p.C = c;
+  p.M = (int)M;
+  p.N = (int)N;
+  p.K = (int)K;
+  p.batch = (int)batch;
+  p.strideA = M * K;
+  p.strideB = N * K;
+  p.strideC = M * N;
+  p.alpha = alpha;
+  p.beta = beta;
+  return launch_gemm(kind, p, ws, ws_bytes, static_cast<hipStream_t>(stream));
+}
+
+}  // namespace ti
+
+using namespace ti;
+
+extern "C" {
+
+int ti_version(void) { return 100; }
+
+const char* ti_last_error(void) { return g_err; }
+
+int ti_init(void) {
+  g_err[0] = 0;
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(TI_ERR_NO_DEVICE, "hipGetDevice: %s", hipGetErrorString(e));
+  hipDeviceProp_t prop;
+  e = hipGetDeviceProperties(&prop, dev);
+  if (e != hipSuccess) return fail(TI_ERR_NO_DEVICE, "hipGetDeviceProperties: %s", hipGetErrorString(e));
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return fail(TI_ERR_NO_DEVICE, "device %d is %s; this library holds gfx950 code only", dev, prop.gcnArchName);
+  return TI_OK;
+}
+
+int64_t ti_linear_workspace_bytes(int64_t M, int64_t N, int64_t K) { return gemm_workspace_bytes(M, N, K); }
+
+int ti_linear_a8_w8_b32_o32(const int8_t* x, const int8_t* w, const int32_t* bias, int32_t* out, int64_t M,
+                            int64_t N, int64_t K, void* ws, int64_t ws_bytes, void* stream) {
+  return run_gemm("linear_a8_w8_b32_o32", EPI_S32_BIAS, x, w, bias, 4, out, 4, 1, M, N, K, 1.0f, 1.0f, ws,
+                  ws_bytes, stream);
+}
+
+int ti_linear_a8_w8_b32_o32_with_scaling(const int8_t* x, const int8_t* w, const int32_t* bias, int32_t* out,
+                                         int64_t M, int64_t N, int64_t K, float alpha, float beta, void* ws,
+                                         int64_t ws_bytes, void* stream) {
+  return run_gemm("linear_a8_w8_b32_o32_with_scaling", EPI_S32_SCALED, x, w, bias, 4, out, 4, 1, M, N, K, alpha,
+                  beta, ws, ws_bytes, stream);
+}
+
+int ti_linear_a8_w8_bfp32_ofp32(const int8_t* x, const int8_t* w, const float* bias, float* out, int64_t M,
+                                int64_t N, int64_t K, float alpha, float beta, void* ws, int64_t ws_bytes,
+                                void* stream) {
+  return run_gemm("linear_a8_w8_bfp32_ofp32", EPI_F32_BIAS, x, w, bias, 4, out, 4, 1, M, N, K, alpha, beta, ws,
+                  ws_bytes, stream);
+}
+
+int ti_linear_a8_w8_b8_o8(const int8_t* x, const int8_t* w, const int8_t* bias, int8_t* out, int64_t M,
+                          int64_t N, int64_t K, float alpha, float beta, void* ws, int64_t ws_bytes,
+                          void* stream) {
+  return run_gemm("linear_a8_w8_b8_o8", EPI_S8_BIAS, x, w, bias, 1, out, 1, 1, M, N, K, alpha, beta, ws,
+                  ws_bytes, stream);
+}
+
+int ti_linear_relu_a8_w8_b8_o8(const int8_t* x, const int8_t* w, const int8_t* bias, int8_t* out, int64_t M,
+                               int64_t N, int64_t K, float alpha, float beta, void* ws, int64_t ws_bytes,
+                               void* stream) {
+  return run_gemm("linear_relu_a8_w8_b8_o8", EPI_S8_RELU, x, w, bias, 1, out, 1, 1, M, N, K, alpha, beta, ws,
+                  ws_bytes, stream);
+}
+
+int ti_bmm_s8t_s8n_f32t(const int8_t* a, const int8_t* b, float* c, int64_t batch, int64_t M, int64_t N,
+                        int64_t K, float alpha, void* stream) {
+  return run_gemm("bmm_s8t_s8n_f32t", EPI_F32_SCALE, a, b, nullptr, 0, c, 4, batch, M, N, K, alpha, 0.0f,
+                  nullptr, 0, stream);
+}
+
+int ti_bmm_s8t_s8n_s8t(const int8_t* a, const int8_t* b, int8_t* c, int64_t batch, int64_t M, int64_t N,
+                       int64_t K, float alpha, void* stream) {
+  return run_gemm("bmm_s8t_s8n_s8t", EPI_S8_SCALE, a, b, nullptr, 0, c, 1, batch, M, N, K, alpha, 0.0f, nullptr,
+                  0, stream);
+}
+
+int ti_bmm_s8t_s8n_s32t(const int8_t* a, const int8_t* b, int32_t* c, int64_t batch, int64_t M, int64_t N,
+                        int64_t K, void* stream) {
+  return run_gemm("bmm_s8t_s8n_s32t", EPI_S32_RAW, a, b, nullptr, 0, c, 4, batch, M, N, K, 1.0f, 0.0f, nullptr,
+                  0, stream);
+}
+
+int ti_dq_add_layernorm_q(const int32_t* input, float input_scale, const float* residual, const float* gamma,
+                          const float* beta, float eps, float* r_out, int8_t* q_out, int64_t rows, int64_t H,
+                          void* stream) {
+  g_err[0] = 0;
+  const char* op = "dq_add_layernorm_q";
+  if (rows < 0 || H < 0) return fail(TI_ERR_INVALID_ARG, "%s: negative size (rows=%lld H=%lld)", op,
+                                     (long long)rows, (long long)H);
+  if (rows > 0x7fffffffLL || H > 0x7fffffffLL)
+    return fail(TI_ERR_INVALID_ARG, "%s: rows and H must be below 2^31", op);
+  const bool nonempty = rows > 0 && H > 0;
+  if (int rc = check_ptr(op, "input", input, 4, nonempty)) return rc;
+  if (int rc = check_ptr(op, "residual", residual, 4, nonempty)) return rc;
+  if (int rc = check_ptr(op, "gamma", gamma, 4, nonempty)) return rc;
+  if (int rc = check_ptr(op, "beta", beta, 4, nonempty)) return rc;
+  if (int rc = check_ptr(op, "residual_out", r_out, 4, nonempty)) return rc;
+  if (int rc = check_ptr(op, "q_out", q_out, 1, nonempty)) return rc;
+  return launch_dq_add_layernorm_q(input, input_scale, residual, gamma, beta, eps, r_out, q_out, rows, H,
+                                   static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,346 @@
+// INT8 x INT8 -> INT32 "NT" GEMM (C = A . B^T) for gfx950 with fused fp32
+// epilogues.  One mainloop serves the W8A8 linears and the batched attention
+// products; the epilogue kind is a template parameter.
+//
+// Mainloop (gemm_tile_kernel):
+//   - a workgroup owns a BM x BN output tile and walks K in steps of 128 bytes;
+//   - A (BM x 128) and B (BN x 128) panels are staged in LDS, two stages deep;
+//     rows are 128 bytes = eight 16-byte chunks, and chunk c of row r is stored
+//     at chunk position c ^ ((r >> 1) & 7) so that both the 16-byte row-wise
+//     stores and the column-wise 16-byte fragment reads spread over all banks;
+//   - each wavefront computes a (BM/WAVES_M) x (BN/WAVES_N) sub-tile out of
+//     32x32 blocks with v_mfma_i32_32x32x32_i8 (K = 32 per instruction, 16
+//     bytes of each operand per lane);
+//   - SWAP selects which matrix feeds the "row" operand of the MFMA.  With
+//     SWAP the weight rows do, their order inside each 32-row block is
+//     permuted when the panel is written to LDS, and a lane ends up holding 16
+//     consecutive output columns of one output row (16-byte s8 stores).
+//     Without SWAP a lane holds one output column of 16 rows and the 32 lanes
+//     of a half-wave store 128 contiguous bytes of 32-bit results.
+#include "ti_common.h"
+
+namespace ti {
+
+static constexpr int BK = 128;        // bytes of K per mainloop step
+static constexpr int CHUNKS = BK / 16;  // 16-byte chunks per LDS row
+
+// position of a logical tile row inside the LDS panel
+template <bool PERMUTE>
+__device__ __forceinline__ int phys_row(int r) {
+  if (!PERMUTE) return r;
+  // inside each block of 32 rows: logical 16h + 4q + j  ->  MFMA row 8q + 4h + j
+  return (r & ~31) | ((r & 12) << 1) | ((r & 16) >> 2) | (r & 3);
+}
+
+__device__ __forceinline__ int lds_off(int prow, int chunk) {
+  return prow * BK + (((chunk ^ (prow >> 1)) & 7) << 4);
+}
+
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int KIND_, bool SWAP_>
+struct TileCfg {
+  static constexpr int BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, KIND = KIND_;
+  static constexpr bool SWAP = SWAP_;
+  static constexpr int NT = WAVES_M * WAVES_N * 64;
+  static constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
+  static constexpr int TM = WTM / 32, TN = WTN / 32;
+  static constexpr int A_SLOTS = BM * CHUNKS / NT, B_SLOTS = BN * CHUNKS / NT;
+  static constexpr int STAGE_BYTES = (BM + BN) * BK;
+  static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
+  static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be made of 32x32 blocks");
+  static_assert((BM * CHUNKS) % NT == 0 && (BN * CHUNKS) % NT == 0, "panel must split evenly over threads");
+};
+
+// Maps the linear workgroup id to an output tile so that (i) the workgroups
+// that share an XCD (ids congruent mod 8 are dispatched to the same XCD, each
+// with a private L2) own a contiguous run of tiles and (ii) consecutive tiles
+// walk down GROUP rows of tiles before moving to the next column, which keeps
+// the A rows and B rows a run touches small enough to stay in that L2.
+__device__ __forceinline__ void tile_of_workgroup(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
+  const int total = tiles_m * tiles_n;
+  const int NXCD = 8;
+  int per = (total + NXCD - 1) / NXCD;
+  int tall = total % NXCD;
+  if (tall == 0) tall = NXCD;
+  int xcd = pid % NXCD, local = pid / NXCD;
+  int id = (xcd < tall) ? xcd * per + local : tall * per + (xcd - tall) * (per - 1) + local;
+  const int GROUP = 8;
+  int width = GROUP * tiles_n;
+  int g = id / width;
+  int first = g * GROUP;
+  int gsz = tiles_m - first < GROUP ? tiles_m - first : GROUP;
+  int in = id - g * width;
+  tm = first + in % gsz;
+  tn = in / gsz;
+}
+
+template <class Cfg>
+__global__ __launch_bounds__(Cfg::NT) void gemm_tile_kernel(GemmParams p, int tiles_m, int tiles_n) {
+  using E = Epi<Cfg::KIND>;
+  using Out = typename E::Out;
+  using BiasT = typename E::Bias;
+  constexpr int BM = Cfg::BM, BN = Cfg::BN, NT = Cfg::NT, TM = Cfg::TM, TN = Cfg::TN;
+  constexpr bool SWAP = Cfg::SWAP;
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wave_m = wave / Cfg::WAVES_N, wave_n = wave % Cfg::WAVES_N;
+  int tile_m, tile_n;
+  tile_of_workgroup(blockIdx.x, tiles_m, tiles_n, tile_m, tile_n);
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int M = p.M, N = p.N, K = p.K;
+  const int8_t* __restrict__ A = p.A + (long long)blockIdx.z * p.strideA;
+  const int8_t* __restrict__ B = p.B + (long long)blockIdx.z * p.strideB;
+
+  // ---- global -> LDS assignment: slot i of thread t moves chunk (t & 7) of row i*NT/8 + t/8
+  const int ld_chunk = tid & 7;
+  const int ld_row = tid >> 3;
+  constexpr int ROWS_PER_SLOT = NT / CHUNKS;
+  int a_goff[Cfg::A_SLOTS], b_goff[Cfg::B_SLOTS];
+  int a_soff[Cfg::A_SLOTS], b_soff[Cfg::B_SLOTS];
+#pragma unroll
+  for (int i = 0; i < Cfg::A_SLOTS; ++i) {
+    int r = i * ROWS_PER_SLOT + ld_row;
+    int gr = m0 + r < M ? m0 + r : M - 1;  // rows past the edge re-read the last row; never stored
+    a_goff[i] = gr * K + ld_chunk * 16;
+    a_soff[i] = lds_off(phys_row<false>(r), ld_chunk);
+  }
+#pragma unroll
+  for (int i = 0; i < Cfg::B_SLOTS; ++i) {
+    int r = i * ROWS_PER_SLOT + ld_row;
+    int gr = n0 + r < N ? n0 + r : N - 1;
+    b_goff[i] = gr * K + ld_chunk * 16;
+    b_soff[i] = BM * BK + lds_off(phys_row<SWAP>(r), ld_chunk);
+  }
+
+  v4i a_reg[Cfg::A_SLOTS], b_reg[Cfg::B_SLOTS];
+  auto load_global = [&](int kt) {
+    const int kbase = kt * BK;
+    const bool ok = kbase + ld_chunk * 16 < K;  // K % 16 == 0: a chunk is all in or all out
+#pragma unroll
+    for (int i = 0; i < Cfg::A_SLOTS; ++i) {
+      v4i z = {0, 0, 0, 0};
+      a_reg[i] = ok ? *reinterpret_cast<const v4i*>(A + (size_t)(unsigned)a_goff[i] + kbase) : z;
+    }
+#pragma unroll
+    for (int i = 0; i < Cfg::B_SLOTS; ++i) {
+      v4i z = {0, 0, 0, 0};
+      b_reg[i] = ok ? *reinterpret_cast<const v4i*>(B + (size_t)(unsigned)b_goff[i] + kbase) : z;
+    }
+  };
+  auto store_lds = [&](int stage) {
+    char* s = smem + stage * Cfg::STAGE_BYTES;
+#pragma unroll
+    for (int i = 0; i < Cfg::A_SLOTS; ++i) *reinterpret_cast<v4i*>(s + a_soff[i]) = a_reg[i];
+#pragma unroll
+    for (int i = 0; i < Cfg::B_SLOTS; ++i) *reinterpret_cast<v4i*>(s + b_soff[i]) = b_reg[i];
+  };
+
+  // ---- fragment addressing: lane reads row (lane & 31), chunk 2*ks + (lane >> 5)
+  const int frow = lane & 31;
+  const int fkey = ((lane >> 5) ^ (frow >> 1)) & 7;  // chunk position for ks = 0
+  const int a_frag = (wave_m * Cfg::WTM + frow) * BK + (fkey << 4);
+  const int b_frag = BM * BK + (wave_n * Cfg::WTN + frow) * BK + (fkey << 4);
+
+  v16i acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+
+  auto compute = [&](int stage) {
+    const char* s = smem + stage * Cfg::STAGE_BYTES;
+#pragma unroll
+    for (int ks = 0; ks < BK / 32; ++ks) {
+      v4i fa[TM], fb[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        fa[i] = *reinterpret_cast<const v4i*>(s + ((a_frag ^ (ks << 5)) + i * 32 * BK));
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        fb[j] = *reinterpret_cast<const v4i*>(s + ((b_frag ^ (ks << 5)) + j * 32 * BK));
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = SWAP ? __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[j], fa[i], acc[i][j], 0, 0, 0)
+                           : __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    }
+  };
+
+  const int KT = (K + BK - 1) / BK;
+  if (KT > 0) {
+    load_global(0);
+    store_lds(0);
+  }
+  __syncthreads();
+  for (int kt = 0; kt < KT; ++kt) {
+    const bool more = kt + 1 < KT;
+    if (more) load_global(kt + 1);
+    compute(kt & 1);
+    if (more) store_lds((kt + 1) & 1);
+    __syncthreads();
+  }
+
+  // ---- epilogue
+  Out* __restrict__ C = reinterpret_cast<Out*>(p.C) + (long long)blockIdx.z * p.strideC;
+  const BiasT* __restrict__ bias = reinterpret_cast<const BiasT*>(p.bias);
+  const float alpha = p.alpha, beta = p.beta;
+  const int half = lane >> 5;
+  if (SWAP) {
+    // lane owns row m = .. + (lane & 31) and 16 consecutive columns per block
+    constexpr int VEC = 16 / sizeof(Out);  // outputs per 16-byte store
+    const bool vec_ok = (N % VEC) == 0;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int nb = n0 + wave_n * Cfg::WTN + j * 32 + half * 16;
+      float bt[16];
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        BiasT bv = BiasT(0);
+        if (E::kHasBias && nb + v < N) bv = bias[nb + v];
+        bt[v] = E::bias_term(bv, beta);
+      }
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const int m = m0 + wave_m * Cfg::WTM + i * 32 + frow;
+        if (m >= M) continue;
+        Out* dst = C + (long long)m * N + nb;
+        if (vec_ok && nb + 16 <= N) {
+          if constexpr (sizeof(Out) == 1) {
+            v4i w;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              unsigned b0 = (unsigned char)E::apply(acc[i][j][4 * q + 0], bt[4 * q + 0], alpha);
+              unsigned b1 = (unsigned char)E::apply(acc[i][j][4 * q + 1], bt[4 * q + 1], alpha);
+              unsigned b2 = (unsigned char)E::apply(acc[i][j][4 * q + 2], bt[4 * q + 2], alpha);
+              unsigned b3 = (unsigned char)E::apply(acc[i][j][4 * q + 3], bt[4 * q + 3], alpha);
+              w[q] = (int)(b0 | (b1 << 8) | (b2 << 16) | (b3 << 24));
+            }
+            *reinterpret_cast<v4i*>(dst) = w;
+          } else {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              Out o0 = E::apply(acc[i][j][4 * q + 0], bt[4 * q + 0], alpha);
+              Out o1 = E::apply(acc[i][j][4 * q + 1], bt[4 * q + 1], alpha);
+              Out o2 = E::apply(acc[i][j][4 * q + 2], bt[4 * q + 2], alpha);
+              Out o3 = E::apply(acc[i][j][4 * q + 3], bt[4 * q + 3], alpha);
+              v4i w = {__builtin_bit_cast(int, o0), __builtin_bit_cast(int, o1),
+                       __builtin_bit_cast(int, o2), __builtin_bit_cast(int, o3)};
+              *reinterpret_cast<v4i*>(dst + 4 * q) = w;
+            }
+          }
+        } else {
+#pragma unroll
+          for (int v = 0; v < 16; ++v)
+            if (nb + v < N) dst[v] = E::apply(acc[i][j][v], bt[v], alpha);
+        }
+      }
+    }
+  } else {
+    // lane owns column n = .. + (lane & 31) and rows 8*(v/4) + 4*half + v%4 of each block
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int n = n0 + wave_n * Cfg::WTN + j * 32 + frow;
+      BiasT bv = BiasT(0);
+      if (E::kHasBias && n < N) bv = bias[n];
+      const float bt = E::bias_term(bv, beta);
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int m = m0 + wave_m * Cfg::WTM + i * 32 + 8 * (v >> 2) + 4 * half + (v & 3);
+          if (m < M && n < N) C[(long long)m * N + n] = E::apply(acc[i][j][v], bt, alpha);
+        }
+      }
+    }
+  }
+}
+
+// Any-shape fallback (K not a multiple of 16 or operands not 16-byte aligned):
+// one thread per output element, scalar loop over K.
+template <int KIND>
+__global__ __launch_bounds__(256) void gemm_scalar_kernel(GemmParams p) {
+  using E = Epi<KIND>;
+  using Out = typename E::Out;
+  using BiasT = typename E::Bias;
+  const long long total = (long long)p.M * p.N;
+  const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  const int m = (int)(idx / p.N), n = (int)(idx % p.N);
+  const int8_t* a = p.A + (long long)blockIdx.z * p.strideA + (long long)m * p.K;
+  const int8_t* b = p.B + (long long)blockIdx.z * p.strideB + (long long)n * p.K;
+  int acc = 0;
+  for (int k = 0; k < p.K; ++k) acc += (int)a[k] * (int)b[k];
+  BiasT bv = BiasT(0);
+  if (E::kHasBias) bv = reinterpret_cast<const BiasT*>(p.bias)[n];
+  Out* C = reinterpret_cast<Out*>(p.C) + (long long)blockIdx.z * p.strideC;
+  C[idx] = E::apply(acc, E::bias_term(bv, p.beta), p.alpha);
+}
+
+// ------------------------------------------------------------------ host side
+
+template <class Cfg>
+static int launch_tile(const GemmParams& p, hipStream_t stream) {
+  static bool attr_set = false;  // benign race: setting the attribute twice is harmless
+  auto kern = gemm_tile_kernel<Cfg>;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
+    if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    attr_set = true;
+  }
+  const int tiles_m = (p.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (p.N + Cfg::BN - 1) / Cfg::BN;
+  dim3 grid(tiles_m * tiles_n, 1, p.batch);
+  hipLaunchKernelGGL(kern, grid, dim3(Cfg::NT), Cfg::LDS_BYTES, stream, p, tiles_m, tiles_n);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "gemm launch: %s", hipGetErrorString(e));
+  return TI_OK;
+}
+
+template <int KIND>
+static int launch_kind(const GemmParams& p, hipStream_t stream) {
+  using Out = typename Epi<KIND>::Out;
+  const bool aligned = (p.K % 16 == 0) && ((reinterpret_cast<uintptr_t>(p.A) & 15) == 0) &&
+                       ((reinterpret_cast<uintptr_t>(p.B) & 15) == 0) &&
+                       (p.strideA % 16 == 0) && (p.strideB % 16 == 0) &&
+                       ((reinterpret_cast<uintptr_t>(p.C) & 15) == 0) &&
+                       ((p.strideC * (long long)sizeof(Out)) % 16 == 0);
+  if (!aligned) {
+    const long long total = (long long)p.M * p.N;
+    dim3 grid((unsigned)((total + 255) / 256), 1, p.batch);
+    hipLaunchKernelGGL(gemm_scalar_kernel<KIND>, grid, dim3(256), 0, stream, p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "gemm launch: %s", hipGetErrorString(e));
+    return TI_OK;
+  }
+  // 8-bit outputs take the orientation whose lanes own 16 consecutive columns.
+  constexpr bool SWAP = sizeof(Out) == 1;
+  const long long t256 = (long long)((p.M + 255) / 256) * ((p.N + 255) / 256) * p.batch;
+  const long long t128 = (long long)((p.M + 127) / 128) * ((p.N + 127) / 128) * p.batch;
+  if (t256 >= 160) return launch_tile<TileCfg<256, 256, 2, 4, KIND, SWAP>>(p, stream);
+  if (t128 >= 128) return launch_tile<TileCfg<128, 128, 2, 2, KIND, SWAP>>(p, stream);
+  return launch_tile<TileCfg<64, 64, 2, 2, KIND, SWAP>>(p, stream);
+}
+
+long long gemm_workspace_bytes(long long, long long, long long) { return 0; }
+
+int launch_gemm(int kind, const GemmParams& p, void*, long long, hipStream_t stream) {
+  if (p.M == 0 || p.N == 0 || p.batch == 0) return TI_OK;
+  switch (kind) {
+    case EPI_S32_BIAS: return launch_kind<EPI_S32_BIAS>(p, stream);
+    case EPI_S32_SCALED: return launch_kind<EPI_S32_SCALED>(p, stream);
+    case EPI_F32_BIAS: return launch_kind<EPI_F32_BIAS>(p, stream);
+    case EPI_S8_BIAS: return launch_kind<EPI_S8_BIAS>(p, stream);
+    case EPI_S8_RELU: return launch_kind<EPI_S8_RELU>(p, stream);
+    case EPI_F32_SCALE: return launch_kind<EPI_F32_SCALE>(p, stream);
+    case EPI_S8_SCALE: return launch_kind<EPI_S8_SCALE>(p, stream);
+    case EPI_S32_RAW: return launch_kind<EPI_S32_RAW>(p, stream);
+  }
+  return fail(TI_ERR_INVALID_ARG, "unknown epilogue kind %d", kind);
+}
+
+}  // namespace ti

@@ -1,0 +1,188 @@
+// dq_add_layernorm_q for gfx950: dequantise an int32 tensor, add it to the fp32
+// residual stream, LayerNorm over the last dimension and quantise to int8, in
+// one pass over HBM (13 bytes per element: 4 in + 4 residual in + 4 residual
+// out + 1 int8 out).
+//
+// One 256-lane workgroup per row.  The row lives in registers between the
+// three phases (sum, sum of squared deviations, normalise), so each input
+// byte is read once.  The fp32 reduction order is fixed:
+//   chunk c (elements 4c..4c+3) belongs to lane c % 256; a lane adds its
+//   elements in ascending order; wavefronts combine with a xor butterfly
+//   (offsets 32..1); the four wavefront sums are added left to right.
+#include "ti_common.h"
+
+namespace ti {
+
+__device__ __forceinline__ float wave_butterfly_sum(float s) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) s = s + __shfl_xor(s, off, 64);
+  return s;
+}
+
+__device__ __forceinline__ float block_sum_256(float s, float* red) {
+  s = wave_butterfly_sum(s);
+  const int wave = threadIdx.x >> 6;
+  __syncthreads();  // previous use of red[] is over
+  if ((threadIdx.x & 63) == 0) red[wave] = s;
+  __syncthreads();
+  return ((red[0] + red[1]) + red[2]) + red[3];
+}
+
+__device__ __forceinline__ int pack_s8x4(float y0, float y1, float y2, float y3) {
+  unsigned b0 = (unsigned char)(int8_t)rne_s8(y0);
+  unsigned b1 = (unsigned char)(int8_t)rne_s8(y1);
+  unsigned b2 = (unsigned char)(int8_t)rne_s8(y2);
+  unsigned b3 = (unsigned char)(int8_t)rne_s8(y3);
+  return (int)(b0 | (b1 << 8) | (b2 << 16) | (b3 << 24));
+}
+
+// H % 4 == 0, H <= NC * 1024, all row starts 16-byte aligned.
+template <int NC>
+__global__ __launch_bounds__(256) void ln_q_rows_kernel(const int32_t* __restrict__ in, float scale,
+                                                        const float* res,  // may alias r_out
+                                                        const float* __restrict__ gamma,
+                                                        const float* __restrict__ beta, float eps,
+                                                        float* r_out, int8_t* __restrict__ q_out, int H) {
+  __shared__ float red[4];
+  const long long row = blockIdx.x;
+  const int t = threadIdx.x;
+  const int nchunks = H >> 2;
+  const v4i* in4 = reinterpret_cast<const v4i*>(in + row * H);
+  const v4f* res4 = reinterpret_cast<const v4f*>(res + row * H);
+  v4f* rout4 = reinterpret_cast<v4f*>(r_out + row * H);
+  int* q4 = reinterpret_cast<int*>(q_out + row * H);
+
+  v4f r[NC];
+  float s = 0.0f;
+#pragma unroll
+  for (int i = 0; i < NC; ++i) {
+    const int c = t + i * 256;
+    if (c < nchunks) {
+      v4i x = in4[c];
+      v4f a = res4[c];
+      v4f v;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) v[j] = __builtin_fmaf(scale, (float)x[j], a[j]);
+      r[i] = v;
+      rout4[c] = v;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) s = s + v[j];
+    }
+  }
+  const float fH = (float)H;
+  const float mu = block_sum_256(s, red) / fH;
+  float s2 = 0.0f;
+#pragma unroll
+  for (int i = 0; i < NC; ++i) {
+    const int c = t + i * 256;
+    if (c < nchunks) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float d = r[i][j] - mu;
+        float sq = d * d;
+        s2 = s2 + sq;
+      }
+    }
+  }
+  const float var = block_sum_256(s2, red) / fH;
+  const float rstd = 1.0f / __builtin_sqrtf(var + eps);
+  const v4f* g4 = reinterpret_cast<const v4f*>(gamma);
+  const v4f* b4 = reinterpret_cast<const v4f*>(beta);
+#pragma unroll
+  for (int i = 0; i < NC; ++i) {
+    const int c = t + i * 256;
+    if (c < nchunks) {
+      v4f g = g4[c], b = b4[c];
+      float y[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) y[j] = __builtin_fmaf((r[i][j] - mu) * rstd, g[j], b[j]);
+      q4[c] = pack_s8x4(y[0], y[1], y[2], y[3]);
+    }
+  }
+}
+
+// Any H and alignment: same reduction tree, scalar accesses, the row is
+// recomputed from the inputs in each phase instead of being kept in registers.
+__global__ __launch_bounds__(256) void ln_q_rows_generic_kernel(const int32_t* __restrict__ in, float scale,
+                                                                const float* res, const float* __restrict__ gamma,
+                                                                const float* __restrict__ beta, float eps,
+                                                                float* r_out, int8_t* __restrict__ q_out, int H) {
+  __shared__ float red[4];
+  const long long row = blockIdx.x;
+  const int t = threadIdx.x;
+  const int32_t* x = in + row * H;
+  const float* a = res + row * H;
+  float* ro = r_out + row * H;
+  int8_t* q = q_out + row * H;
+  const int nchunks = (H + 3) >> 2;
+  float s = 0.0f;
+  for (int c = t; c < nchunks; c += 256)
+    for (int j = 0; j < 4; ++j) {
+      const int i = c * 4 + j;
+      if (i < H) s = s + __builtin_fmaf(scale, (float)x[i], a[i]);
+    }
+  const float fH = (float)H;
+  const float mu = block_sum_256(s, red) / fH;
+  float s2 = 0.0f;
+  for (int c = t; c < nchunks; c += 256)
+    for (int j = 0; j < 4; ++j) {
+      const int i = c * 4 + j;
+      if (i < H) {
+        float d = __builtin_fmaf(scale, (float)x[i], a[i]) - mu;
+        float sq = d * d;
+        s2 = s2 + sq;
+      }
+    }
+  const float var = block_sum_256(s2, red) / fH;
+  const float rstd = 1.0f / __builtin_sqrtf(var + eps);
+  // r_out may alias res: each element is read (above and here) only by the
+  // lane that writes it, and the write comes last.
+  for (int c = t; c < nchunks; c += 256)
+    for (int j = 0; j < 4; ++j) {
+      const int i = c * 4 + j;
+      if (i < H) {
+        float v = __builtin_fmaf(scale, (float)x[i], a[i]);
+        float y = __builtin_fmaf((v - mu) * rstd, gamma[i], beta[i]);
+        ro[i] = v;
+        q[i] = (int8_t)rne_s8(y);
+      }
+    }
+}
+
+template <int NC>
+static void launch_rows(const int32_t* in, float scale, const float* res, const float* gamma, const float* beta,
+                        float eps, float* r_out, int8_t* q_out, long long rows, int H, hipStream_t stream) {
+  hipLaunchKernelGGL(ln_q_rows_kernel<NC>, dim3((unsigned)rows), dim3(256), 0, stream, in, scale, res, gamma,
+                     beta, eps, r_out, q_out, H);
+}
+
+int launch_dq_add_layernorm_q(const int32_t* in, float scale, const float* res, const float* gamma,
+                              const float* beta, float eps, float* r_out, int8_t* q_out, long long rows,
+                              long long H, hipStream_t stream) {
+  if (rows == 0 || H == 0) return TI_OK;
+  auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+  const bool fast = (H % 4 == 0) && H <= 16 * 1024 && al16(in) && al16(res) && al16(gamma) && al16(beta) &&
+                    al16(r_out) && ((reinterpret_cast<uintptr_t>(q_out) & 3) == 0);
+  const int h = (int)H;
+  if (fast) {
+    const int nc = (int)((H + 1023) / 1024);
+#define TI_LN_CASE(n)                                                                     \
+  case n:                                                                                 \
+    launch_rows<n>(in, scale, res, gamma, beta, eps, r_out, q_out, rows, h, stream);      \
+    break;
+    switch (nc) {
+      TI_LN_CASE(1) TI_LN_CASE(2) TI_LN_CASE(3) TI_LN_CASE(4) TI_LN_CASE(5) TI_LN_CASE(6) TI_LN_CASE(7)
+      TI_LN_CASE(8) TI_LN_CASE(9) TI_LN_CASE(10) TI_LN_CASE(11) TI_LN_CASE(12) TI_LN_CASE(13)
+      TI_LN_CASE(14) TI_LN_CASE(15) TI_LN_CASE(16)
+    }
+#undef TI_LN_CASE
+  } else {
+    hipLaunchKernelGGL(ln_q_rows_generic_kernel, dim3((unsigned)rows), dim3(256), 0, stream, in, scale, res,
+                       gamma, beta, eps, r_out, q_out, h);
+  }
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "dq_add_layernorm_q launch: %s", hipGetErrorString(e));
+  return TI_OK;
+}
+
+}  // namespace ti

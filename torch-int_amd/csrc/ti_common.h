@@ -1,0 +1,154 @@
+// Shared declarations for the gfx950 INT8 kernels: error reporting, vector
+// types and the fp32 epilogues every GEMM/BMM kernel applies to its int32
+// accumulators.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "../../include/torch_int_hip.h"
+
+namespace ti {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+// Records a formatted reason for the calling thread and returns `code`.
+int fail(int code, const char* fmt, ...);
+
+// ---------------------------------------------------------------- epilogues
+// Kinds of output transform.  The *_BIAS kinds read a per-column bias.
+enum EpiKind : int {
+  EPI_S32_BIAS = 0,    // out = acc + bias                      (int32, wrapping)
+  EPI_S32_SCALED = 1,  // out = sat_s32(rint(fma(a, acc, b*bias)))
+  EPI_F32_BIAS = 2,    // out = fma(a, acc, b*bias)             (fp32 bias)
+  EPI_S8_BIAS = 3,     // out = s8(rint(clamp(fma(a, acc, b*bias))))
+  EPI_S8_RELU = 4,     // out = s8(rint(min(max(fma(..), 0), 127)))
+  EPI_F32_SCALE = 5,   // out = a * acc
+  EPI_S8_SCALE = 6,    // out = s8(rint(clamp(a * acc)))
+  EPI_S32_RAW = 7,     // out = acc
+};
+
+__device__ __forceinline__ float clamp_s8f(float t) {
+  // NaN -> 0, like a saturating convert.  fminf/fmaxf would return the
+  // non-NaN operand, so test explicitly.
+  t = (t != t) ? 0.0f : t;
+  t = t < -128.0f ? -128.0f : t;
+  t = t > 127.0f ? 127.0f : t;
+  return t;
+}
+
+__device__ __forceinline__ int rne_s8(float t) { return (int)__builtin_rintf(clamp_s8f(t)); }
+
+__device__ __forceinline__ int rne_sat_s32(float t) {
+  if (t != t) return 0;
+  if (t >= 2147483648.0f) return 2147483647;
+  if (t <= -2147483648.0f) return (-2147483647 - 1);
+  return (int)__builtin_rintf(t);
+}
+
+template <int KIND>
+struct Epi;
+
+template <>
+struct Epi<EPI_S32_BIAS> {
+  using Out = int32_t;
+  using Bias = int32_t;
+  static constexpr bool kHasBias = true;
+  // the "bias term" is carried as raw bits so one code path serves all kinds
+  static __device__ __forceinline__ float bias_term(Bias b, float) { return __int_as_float(b); }
+  static __device__ __forceinline__ Out apply(int acc, float bt, float) {
+    return (int32_t)((uint32_t)acc + (uint32_t)__float_as_int(bt));
+  }
+};
+template <>
+struct Epi<EPI_S32_SCALED> {
+  using Out = int32_t;
+  using Bias = int32_t;
+  static constexpr bool kHasBias = true;
+  static __device__ __forceinline__ float bias_term(Bias b, float beta) { return beta * (float)b; }
+  static __device__ __forceinline__ Out apply(int acc, float bt, float alpha) {
+    return rne_sat_s32(__builtin_fmaf(alpha, (float)acc, bt));
+  }
+};
+template <>
+struct Epi<EPI_F32_BIAS> {
+  using Out = float;
+  using Bias = float;
+  static constexpr bool kHasBias = true;
+  static __device__ __forceinline__ float bias_term(Bias b, float beta) { return beta * b; }
+  static __device__ __forceinline__ Out apply(int acc, float bt, float alpha) {
+    return __builtin_fmaf(alpha, (float)acc, bt);
+  }
+};
+template <>
+struct Epi<EPI_S8_BIAS> {
+  using Out = int8_t;
+  using Bias = int8_t;
+  static constexpr bool kHasBias = true;
+  static __device__ __forceinline__ float bias_term(Bias b, float beta) { return beta * (float)(int)b; }
+  static __device__ __forceinline__ Out apply(int acc, float bt, float alpha) {
+    return (int8_t)rne_s8(__builtin_fmaf(alpha, (float)acc, bt));
+  }
+};
+template <>
+struct Epi<EPI_S8_RELU> {
+  using Out = int8_t;
+  using Bias = int8_t;
+  static constexpr bool kHasBias = true;
+  static __device__ __forceinline__ float bias_term(Bias b, float beta) { return beta * (float)(int)b; }
+  static __device__ __forceinline__ Out apply(int acc, float bt, float alpha) {
+    float t = __builtin_fmaf(alpha, (float)acc, bt);
+    t = (t > 0.0f) ? t : 0.0f;  // also maps NaN to 0
+    return (int8_t)rne_s8(t);
+  }
+};
+template <>
+struct Epi<EPI_F32_SCALE> {
+  using Out = float;
+  using Bias = float;
+  static constexpr bool kHasBias = false;
+  static __device__ __forceinline__ float bias_term(Bias, float) { return 0.0f; }
+  static __device__ __forceinline__ Out apply(int acc, float, float alpha) { return alpha * (float)acc; }
+};
+template <>
+struct Epi<EPI_S8_SCALE> {
+  using Out = int8_t;
+  using Bias = int8_t;
+  static constexpr bool kHasBias = false;
+  static __device__ __forceinline__ float bias_term(Bias, float) { return 0.0f; }
+  static __device__ __forceinline__ Out apply(int acc, float, float alpha) {
+    return (int8_t)rne_s8(alpha * (float)acc);
+  }
+};
+template <>
+struct Epi<EPI_S32_RAW> {
+  using Out = int32_t;
+  using Bias = int32_t;
+  static constexpr bool kHasBias = false;
+  static __device__ __forceinline__ float bias_term(Bias, float) { return 0.0f; }
+  static __device__ __forceinline__ Out apply(int acc, float, float) { return acc; }
+};
+
+// Problem description handed to every GEMM kernel.  A is [batch, M, K], B is
+// [batch, N, K], C is [batch, M, N], all packed; bias is [N] (shared by batches).
+struct GemmParams {
+  const int8_t* A;
+  const int8_t* B;
+  const void* bias;
+  void* C;
+  int M, N, K, batch;
+  long long strideA, strideB, strideC;  // elements between consecutive batches
+  float alpha, beta;
+};
+
+// Launchers (gemm_s8.hip).  `kind` is an EpiKind.  Returns a TI_* status.
+int launch_gemm(int kind, const GemmParams& p, void* workspace, long long workspace_bytes,
+                hipStream_t stream);
+long long gemm_workspace_bytes(long long M, long long N, long long K);
+
+// ln_q.hip
+int launch_dq_add_layernorm_q(const int32_t* in, float scale, const float* res, const float* gamma,
+                              const float* beta, float eps, float* r_out, int8_t* q_out,
+                              long long rows, long long H, hipStream_t stream);
+
+}  // namespace ti

@@ -1,0 +1,433 @@
+"""INT8 OPT blocks on the MI355X kernels (upstream ``torch_int/models/opt.py``).
+
+``Int8OPTAttention`` and ``Int8OPTDecoderLayer`` keep upstream's constructor
+signatures, sub-module names, scale algebra and forward semantics.  The
+decoder / model / causal-LM wrappers carry their own small OPT scaffolding
+(token + learned position embeddings with the +2 offset, additive causal
+mask, final LayerNorm, fp ``lm_head``) instead of borrowing methods from a
+particular ``transformers`` release; any object with OPTConfig's field names
+works as ``config``.
+"""
+from dataclasses import dataclass
+from typing import List, Optional, Tuple
+
+import torch
+from torch import nn
+
+from ..nn.bmm import BMM_S8T_S8N_F32T, BMM_S8T_S8N_S8T
+from ..nn.fused import LayerNormQ
+from ..nn.linear import W8A8B8O8Linear, W8A8B8O8LinearReLU, W8A8BFP32OFP32Linear
+
+
+class Int8OPTAttention(nn.Module):
+    """Multi-head self-attention with int8 projections and int8 Q.K^T / P.V products.
+
+    upstream: ``torch_int/models/opt.py:22-199``.
+    """
+
+    def __init__(self, embed_dim: int, num_heads: int):
+        super().__init__()
+        self.embed_dim = embed_dim
+        self.num_heads = num_heads
+        self.head_dim = embed_dim // num_heads
+        if self.head_dim * num_heads != embed_dim:
+            raise ValueError(f"embed_dim must be divisible by num_heads (got `embed_dim`: {embed_dim}"
+                             f" and `num_heads`: {num_heads}).")
+        self.attention_weight_scale = 1.0
+        self.qk_bmm = BMM_S8T_S8N_F32T(1.0)
+        self.pv_bmm = BMM_S8T_S8N_S8T(1.0)
+        self.k_proj = W8A8B8O8Linear(embed_dim, embed_dim)
+        self.v_proj = W8A8B8O8Linear(embed_dim, embed_dim)
+        self.q_proj = W8A8B8O8Linear(embed_dim, embed_dim)
+        self.out_proj = W8A8BFP32OFP32Linear(embed_dim, embed_dim)
+
+    @staticmethod
+    @torch.no_grad()
+    def from_float(module, input_scale: float, q_output_scale: float, k_output_scale: float,
+                   v_output_scale: float, out_input_scale: float):
+        """``module`` is an fp OPT attention (attributes embed_dim, num_heads, scaling,
+        q/k/v/out_proj).  The 1/sqrt(d) factor is folded into q_proj, in place on ``module``."""
+        q = Int8OPTAttention(module.embed_dim, module.num_heads)
+        q_output_scale = q_output_scale * module.scaling
+        module.q_proj.weight *= module.scaling
+        module.q_proj.bias *= module.scaling
+        q.q_proj = W8A8B8O8Linear.from_float(module.q_proj, input_scale, q_output_scale)
+        q.k_proj = W8A8B8O8Linear.from_float(module.k_proj, input_scale, k_output_scale)
+        q.v_proj = W8A8B8O8Linear.from_float(module.v_proj, input_scale, v_output_scale)
+        q.out_proj = W8A8BFP32OFP32Linear.from_float(module.out_proj, out_input_scale)
+        q.qk_bmm = BMM_S8T_S8N_F32T.from_scale(q_output_scale, k_output_scale)
+        # probabilities are quantised with scale 1/127
+        q.pv_bmm = BMM_S8T_S8N_S8T.from_scale(1.0 / 127, v_output_scale, out_input_scale)
+        return q
+
+    def _shape(self, tensor: torch.Tensor, seq_len: int, bsz: int):
+        return tensor.view(bsz, seq_len, self.num_heads, self.head_dim).transpose(1, 2).contiguous()
+
+    @torch.no_grad()
+    def forward(self, hidden_states: torch.Tensor, key_value_states: Optional[torch.Tensor] = None,
+                past_key_value: Optional[Tuple[torch.Tensor]] = None,
+                attention_mask: Optional[torch.Tensor] = None,
+                layer_head_mask: Optional[torch.Tensor] = None, output_attentions: bool = False,
+                ) -> Tuple[torch.Tensor, Optional[torch.Tensor], Optional[Tuple[torch.Tensor]]]:
+        """hidden_states: int8 [batch, time, channel] -> (fp32 output, probs or None, (k, v) int8 cache)."""
+        cross = key_value_states is not None
+        bsz, tgt_len, _ = hidden_states.size()
+        H, d = self.num_heads, self.head_dim
+
+        query = self.q_proj(hidden_states)
+        if cross and past_key_value is not None:
+            key, value = past_key_value
+        else:
+            kv_src = key_value_states if cross else hidden_states
+            key = self._shape(self.k_proj(kv_src), -1, bsz)
+            value = self._shape(self.v_proj(kv_src), -1, bsz)
+            if not cross and past_key_value is not None:
+                key = torch.cat([past_key_value[0], key], dim=2)
+                value = torch.cat([past_key_value[1], value], dim=2)
+        present = (key, value)
+
+        query = self._shape(query, tgt_len, bsz).view(bsz * H, -1, d)
+        key = key.view(bsz * H, -1, d)
+        value = value.view(bsz * H, -1, d)
+        src_len = key.size(1)
+
+        scores = self.qk_bmm(query, key)  # fp32 [bsz*H, tgt, src]
+        if scores.size() != (bsz * H, tgt_len, src_len):
+            raise ValueError(f"Attention weights should be of size {(bsz * H, tgt_len, src_len)}, but is"
+                             f" {scores.size()}")
+        if attention_mask is not None:
+            if attention_mask.size() != (bsz, 1, tgt_len, src_len):
+                raise ValueError(f"Attention mask should be of size {(bsz, 1, tgt_len, src_len)}, but is"
+                                 f" {attention_mask.size()}")
+            scores = scores.view(bsz, H, tgt_len, src_len) + attention_mask
+            scores = torch.clamp_min(scores, torch.finfo(scores.dtype).min)
+            scores = scores.view(bsz * H, tgt_len, src_len)
+        probs = nn.functional.softmax(scores, dim=-1)
+
+        if layer_head_mask is not None:
+            if layer_head_mask.size() != (H,):
+                raise ValueError(f"Head mask for a single layer should be of size {(H,)}, but is"
+                                 f" {layer_head_mask.size()}")
+            probs = (layer_head_mask.view(1, -1, 1, 1) * probs.view(bsz, H, tgt_len, src_len)
+                     ).view(bsz * H, tgt_len, src_len)
+        probs_out = probs.view(bsz, H, tgt_len, src_len) if output_attentions else None
+
+        # P.V with V transposed to [bsz*H, d, src]: (P V) = P . (V^T)^T.  The probabilities are
+        # scaled and rounded in place, so with output_attentions the returned view holds
+        # round(127 p), which is what upstream returns too (models/opt.py:166-178).
+        probs_q = probs.mul_(127).round_().to(torch.int8)
+        value_t = value.transpose(1, 2).contiguous()
+        ctx = self.pv_bmm(probs_q, value_t)  # int8 [bsz*H, tgt, d]
+        if ctx.size() != (bsz * H, tgt_len, d):
+            raise ValueError(f"`attn_output` should be of size {(bsz, H, tgt_len, d)}, but is {ctx.size()}")
+        ctx = ctx.view(bsz, H, tgt_len, d).transpose(1, 2).reshape(bsz, tgt_len, self.embed_dim).contiguous()
+        return self.out_proj(ctx), probs_out, present
+
+
+class Int8OPTDecoderLayer(nn.Module):
+    """Pre-LN OPT block on an fp residual stream: LayerNormQ -> int8 attention -> add ->
+    LayerNormQ -> fc1 (ReLU, int8) -> fc2 (fp32) -> add.  The input tensor is updated in
+    place, as upstream does (``torch_int/models/opt.py:202-299``)."""
+
+    def __init__(self, embed_dim, num_attention_heads, ffn_dim):
+        super().__init__()
+        self.embed_dim = embed_dim
+        self.self_attn = Int8OPTAttention(embed_dim=embed_dim, num_heads=num_attention_heads)
+        self.self_attn_layer_norm = LayerNormQ(embed_dim)
+        self.fc1 = W8A8B8O8LinearReLU(embed_dim, ffn_dim)
+        self.fc2 = W8A8BFP32OFP32Linear(ffn_dim, embed_dim)
+        self.final_layer_norm = LayerNormQ(embed_dim)
+
+    @staticmethod
+    def from_float(module, attn_input_scale: float, q_output_scale: float, k_output_scale: float,
+                   v_output_scale: float, out_input_scale: float, fc1_input_scale: float,
+                   fc2_input_scale: float):
+        q = Int8OPTDecoderLayer(module.embed_dim, module.self_attn.num_heads, module.fc1.out_features)
+        q.self_attn_layer_norm = LayerNormQ.from_float(module.self_attn_layer_norm, attn_input_scale)
+        q.self_attn = Int8OPTAttention.from_float(module.self_attn, attn_input_scale, q_output_scale,
+                                                  k_output_scale, v_output_scale, out_input_scale)
+        q.final_layer_norm = LayerNormQ.from_float(module.final_layer_norm, fc1_input_scale)
+        q.fc1 = W8A8B8O8LinearReLU.from_float(module.fc1, fc1_input_scale, fc2_input_scale)
+        q.fc2 = W8A8BFP32OFP32Linear.from_float(module.fc2, fc2_input_scale)
+        return q
+
+    def forward(self, hidden_states: torch.Tensor, attention_mask: Optional[torch.Tensor] = None,
+                layer_head_mask: Optional[torch.Tensor] = None, output_attentions: Optional[bool] = False,
+                use_cache: Optional[bool] = False, past_key_value: Optional[Tuple[torch.Tensor]] = None):
+        """hidden_states: fp [batch, time, embed_dim] residual stream -> tuple starting with it."""
+        residual = hidden_states
+        x = self.self_attn_layer_norm(hidden_states)
+        x, attn_weights, present = self.self_attn(
+            hidden_states=x, past_key_value=past_key_value, attention_mask=attention_mask,
+            layer_head_mask=layer_head_mask, output_attentions=output_attentions)
+        residual.add_(x.to(residual.dtype))
+        x = self.final_layer_norm(residual)
+        x = self.fc2(self.fc1(x))
+        residual.add_(x.to(residual.dtype))
+        outputs = (residual,)
+        if output_attentions:
+            outputs += (attn_weights,)
+        if use_cache:
+            outputs += (present,)
+        return outputs
+
+
+# --------------------------------------------------------------------------------------
+# OPT scaffolding around the int8 blocks
+# --------------------------------------------------------------------------------------
+
+@dataclass
+class OPTConfigLite:
+    """The OPTConfig fields the int8 model reads, with OPT-125m defaults."""
+    vocab_size: int = 50272
+    hidden_size: int = 768
+    num_hidden_layers: int = 12
+    ffn_dim: int = 3072
+    num_attention_heads: int = 12
+    max_position_embeddings: int = 2048
+    word_embed_proj_dim: Optional[int] = None
+    pad_token_id: int = 1
+    do_layer_norm_before: bool = True
+    _remove_final_layer_norm: bool = False
+    use_cache: bool = True
+
+    def __post_init__(self):
+        if self.word_embed_proj_dim is None:
+            self.word_embed_proj_dim = self.hidden_size
+
+
+@dataclass
+class BaseModelOutputWithPast:
+    last_hidden_state: torch.Tensor = None
+    past_key_values: Optional[tuple] = None
+    hidden_states: Optional[tuple] = None
+    attentions: Optional[tuple] = None
+
+
+@dataclass
+class CausalLMOutputWithPast:
+    loss: Optional[torch.Tensor] = None
+    logits: torch.Tensor = None
+    past_key_values: Optional[tuple] = None
+    hidden_states: Optional[tuple] = None
+    attentions: Optional[tuple] = None
+
+
+class OPTLearnedPositionalEmbedding(nn.Embedding):
+    """Learned absolute positions; OPT reserves the first two rows, so indices are offset by 2."""
+    offset = 2
+
+    def __init__(self, num_embeddings: int, embedding_dim: int):
+        super().__init__(num_embeddings + self.offset, embedding_dim)
+
+    def forward(self, attention_mask: torch.Tensor, past_key_values_length: int = 0):
+        mask = attention_mask.long()
+        positions = torch.cumsum(mask, dim=1) * mask - 1  # padded slots get -1
+        return super().forward(positions[:, past_key_values_length:] + self.offset)
+
+
+def _additive_decoder_mask(attention_mask, tgt_len, past_len, dtype, device):
+    """[bsz, 1, tgt, past+tgt] mask: 0 where attention is allowed, finfo.min where the
+    key is in the future or is padding (both conditions add up)."""
+    bsz, src_len = attention_mask.shape
+    neg = torch.finfo(dtype).min
+    keep = attention_mask[:, None, None, :].to(dtype)
+    pad = (1.0 - keep).masked_fill((1.0 - keep).bool(), neg).expand(bsz, 1, tgt_len, src_len)
+    if tgt_len <= 1:
+        return pad.contiguous()
+    q_pos = torch.arange(past_len, past_len + tgt_len, device=device)[:, None]
+    k_pos = torch.arange(src_len, device=device)[None, :]
+    causal = torch.zeros((tgt_len, src_len), dtype=dtype, device=device).masked_fill(k_pos > q_pos, neg)
+    return pad + causal[None, None]
+
+
+class Int8OPTDecoder(nn.Module):
+    """Stack of ``Int8OPTDecoderLayer`` with fp embeddings and final LayerNorm
+    (upstream ``torch_int/models/opt.py:302-398``).  Without a KV cache the token dimension
+    is padded to a multiple of 16 with <pad> (id 1, masked out) and the result sliced back,
+    exactly as upstream; with a cache the new tokens are used as they are."""
+
+    def __init__(self, config):
+        super().__init__()
+        self.config = config
+        self.padding_idx = config.pad_token_id
+        self.max_target_positions = config.max_position_embeddings
+        self.vocab_size = config.vocab_size
+        D, E = config.hidden_size, config.word_embed_proj_dim
+        self.embed_tokens = nn.Embedding(config.vocab_size, E, self.padding_idx)
+        self.embed_positions = OPTLearnedPositionalEmbedding(config.max_position_embeddings, D)
+        self.project_out = nn.Linear(D, E, bias=False) if E != D else None
+        self.project_in = nn.Linear(E, D, bias=False) if E != D else None
+        if config.do_layer_norm_before and not getattr(config, "_remove_final_layer_norm", False):
+            self.final_layer_norm = nn.LayerNorm(D)
+        else:
+            self.final_layer_norm = None
+        self.layers = nn.ModuleList(
+            [Int8OPTDecoderLayer(D, config.num_attention_heads, config.ffn_dim)
+             for _ in range(config.num_hidden_layers)])
+
+    def get_input_embeddings(self):
+        return self.embed_tokens
+
+    def set_input_embeddings(self, value):
+        self.embed_tokens = value
+
+    @staticmethod
+    def from_float(module, decoder_layer_scales):
+        q = Int8OPTDecoder(module.config)
+        q.embed_tokens = module.embed_tokens
+        q.embed_positions = module.embed_positions
+        q.project_out = module.project_out
+        q.project_in = getattr(module, "project_in", None)
+        q.final_layer_norm = module.final_layer_norm
+        for i, layer in enumerate(module.layers):
+            q.layers[i] = Int8OPTDecoderLayer.from_float(layer, **decoder_layer_scales[i])
+        return q
+
+    @torch.no_grad()
+    def forward(self, input_ids: torch.LongTensor = None, attention_mask: Optional[torch.Tensor] = None,
+                head_mask: Optional[torch.Tensor] = None,
+                past_key_values: Optional[List[Tuple[torch.Tensor]]] = None,
+                inputs_embeds: Optional[torch.Tensor] = None, use_cache: Optional[bool] = None,
+                output_attentions: Optional[bool] = None, output_hidden_states: Optional[bool] = None,
+                return_dict: Optional[bool] = None):
+        use_cache = bool(use_cache) if use_cache is not None else False
+        if inputs_embeds is None:
+            input_ids = input_ids.view(-1, input_ids.shape[-1])
+        input_len = (input_ids if input_ids is not None else inputs_embeds).shape[1]
+        past_len = past_key_values[0][0].shape[2] if past_key_values else 0
+
+        pad_len = (-input_len) % 16 if (past_len == 0 and inputs_embeds is None) else 0
+        if pad_len:
+            input_ids = nn.functional.pad(input_ids, (0, pad_len), value=1)
+            if attention_mask is not None:
+                attention_mask = nn.functional.pad(attention_mask, (0, pad_len), value=0)
+        if inputs_embeds is None:
+            inputs_embeds = self.embed_tokens(input_ids)
+        bsz, tgt_len = inputs_embeds.shape[:2]
+        if attention_mask is None:
+            attention_mask = torch.ones((bsz, past_len + tgt_len), dtype=torch.bool, device=inputs_embeds.device)
+        pos = self.embed_positions(attention_mask, past_len)
+        mask = _additive_decoder_mask(attention_mask, tgt_len, past_len, inputs_embeds.dtype,
+                                      inputs_embeds.device)
+        if self.project_in is not None:
+            inputs_embeds = self.project_in(inputs_embeds)
+        hidden = inputs_embeds + pos  # a fresh tensor: the layers update it in place
+
+        all_hidden = () if output_hidden_states else None
+        all_attn = () if output_attentions else None
+        cache = () if use_cache else None
+        for i, layer in enumerate(self.layers):
+            if output_hidden_states:
+                all_hidden += (hidden.clone(),)
+            out = layer(hidden, attention_mask=mask,
+                        layer_head_mask=head_mask[i] if head_mask is not None else None,
+                        output_attentions=bool(output_attentions), use_cache=use_cache,
+                        past_key_value=past_key_values[i] if past_key_values else None)
+            hidden = out[0]
+            if output_attentions:
+                all_attn += (out[1],)
+            if use_cache:
+                cache += (out[-1],)
+        if self.final_layer_norm is not None:
+            hidden = self.final_layer_norm(hidden)
+        if self.project_out is not None:
+            hidden = self.project_out(hidden)
+        if output_hidden_states:
+            all_hidden += (hidden,)
+        if pad_len:
+            hidden = hidden[:, :input_len, :]
+        return BaseModelOutputWithPast(last_hidden_state=hidden, past_key_values=cache,
+                                       hidden_states=all_hidden, attentions=all_attn)
+
+
+class Int8OPTModel(nn.Module):
+    """upstream ``torch_int/models/opt.py:401-417``."""
+
+    def __init__(self, config):
+        super().__init__()
+        self.config = config
+        self.decoder = Int8OPTDecoder(config)
+
+    def get_input_embeddings(self):
+        return self.decoder.embed_tokens
+
+    def set_input_embeddings(self, value):
+        self.decoder.embed_tokens = value
+
+    def get_decoder(self):
+        return self.decoder
+
+    @staticmethod
+    def from_float(module, decoder_layer_scales):
+        q = Int8OPTModel(module.config)
+        q.decoder = Int8OPTDecoder.from_float(module.decoder, decoder_layer_scales)
+        return q
+
+    def forward(self, *args, **kwargs):
+        return self.decoder(*args, **kwargs)
+
+
+class Int8OPTForCausalLM(nn.Module):
+    """Int8 decoder + fp ``lm_head`` (not quantised; upstream ``torch_int/models/opt.py:420-450``)."""
+    _keys_to_ignore_on_load_missing = [r"lm_head.weight"]
+
+    def __init__(self, config):
+        super().__init__()
+        self.config = config
+        self.model = Int8OPTModel(config)
+        self.lm_head = nn.Linear(config.word_embed_proj_dim, config.vocab_size, bias=False)
+
+    @staticmethod
+    def from_float(module, decoder_layer_scales):
+        q = Int8OPTForCausalLM(module.config)
+        q.model = Int8OPTModel.from_float(module.model, decoder_layer_scales)
+        q.lm_head = module.lm_head
+        return q
+
+    def get_input_embeddings(self):
+        return self.model.decoder.embed_tokens
+
+    def set_input_embeddings(self, value):
+        self.model.decoder.embed_tokens = value
+
+    def get_output_embeddings(self):
+        return self.lm_head
+
+    def set_output_embeddings(self, new_embeddings):
+        self.lm_head = new_embeddings
+
+    def set_decoder(self, decoder):
+        self.model.decoder = decoder
+
+    def get_decoder(self):
+        return self.model.decoder
+
+    @torch.no_grad()
+    def forward(self, input_ids: torch.LongTensor = None, attention_mask: Optional[torch.Tensor] = None,
+                head_mask: Optional[torch.Tensor] = None, past_key_values=None,
+                inputs_embeds: Optional[torch.Tensor] = None, labels: Optional[torch.LongTensor] = None,
+                use_cache: Optional[bool] = None, output_attentions: Optional[bool] = None,
+                output_hidden_states: Optional[bool] = None, return_dict: Optional[bool] = None):
+        out = self.model.decoder(input_ids=input_ids, attention_mask=attention_mask, head_mask=head_mask,
+                                 past_key_values=past_key_values, inputs_embeds=inputs_embeds,
+                                 use_cache=use_cache, output_attentions=output_attentions,
+                                 output_hidden_states=output_hidden_states)
+        logits = self.lm_head(out.last_hidden_state.to(self.lm_head.weight.dtype)).contiguous()
+        loss = None
+        if labels is not None:
+            shift = logits[..., :-1, :].contiguous()
+            loss = nn.functional.cross_entropy(shift.view(-1, shift.size(-1)),
+                                               labels[..., 1:].contiguous().view(-1).to(logits.device))
+        return CausalLMOutputWithPast(loss=loss, logits=logits, past_key_values=out.past_key_values,
+                                      hidden_states=out.hidden_states, attentions=out.attentions)
+
+    def prepare_inputs_for_generation(self, input_ids, past_key_values=None, attention_mask=None, **kwargs):
+        if past_key_values:
+            input_ids = input_ids[:, -1:]
+        return {"input_ids": input_ids, "attention_mask": attention_mask,
+                "past_key_values": past_key_values, "use_cache": kwargs.get("use_cache")}
+
+    @staticmethod
+    def _reorder_cache(past, beam_idx):
+        return tuple(tuple(s.index_select(0, beam_idx) for s in layer) for layer in past)

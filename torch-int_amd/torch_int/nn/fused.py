@@ -1,0 +1,41 @@
+"""LayerNorm layers that emit int8 (upstream ``torch_int/nn/fused.py:5-43``)."""
+import torch
+import torch.nn.functional as F
+
+from ..functional.fused import dq_add_layernorm_q_cpp
+
+
+class _QuantLayerNormBase(torch.nn.Module):
+    def __init__(self, dim, eps=1e-5):
+        super().__init__()
+        self.input_scale = 1.0
+        self.eps = eps
+        self.register_buffer("weight", torch.ones(dim, dtype=torch.float32))
+        self.register_buffer("bias", torch.zeros(dim, dtype=torch.float32))
+
+
+class LayerNormQ(_QuantLayerNormBase):
+    """fp -> int8: LayerNorm in fp32, round half-even, clamp to [-128, 127].
+    ``from_float`` folds the output scale into weight and bias."""
+
+    def forward(self, x):
+        y = F.layer_norm(x.to(self.weight.dtype), x.shape[-1:], self.weight, self.bias, self.eps)
+        return y.round().clamp(-128, 127).to(torch.int8)
+
+    @staticmethod
+    def from_float(module: torch.nn.LayerNorm, output_scale: float):
+        dim = module.normalized_shape[0]
+        assert dim == module.weight.numel() == module.bias.numel()
+        q = LayerNormQ(dim, module.eps)
+        q.weight = module.weight / output_scale
+        q.bias = module.bias / output_scale
+        return q
+
+
+class DQ_Add_LayerNorm_Q(_QuantLayerNormBase):
+    """(fp residual, int32 branch output) -> (new fp residual, int8 LayerNorm of it),
+    one fused kernel.  Note the argument order: residual first."""
+
+    def forward(self, residual_input_fp, input_int32):
+        return dq_add_layernorm_q_cpp(input_int32, self.input_scale, residual_input_fp,
+                                      self.weight, self.bias, self.eps)

@@ -1,0 +1,146 @@
+"""W8A8 linear layers (upstream ``torch_int/nn/linear.py:16-229``).
+
+Every class keeps upstream's constructor signature, buffer names/shapes/dtypes
+(``weight`` int8 [out, in], ``bias`` [1, out], 0-dim fp32 ``a``/``b``) and
+``from_float`` algebra; ``forward`` flattens the leading dimensions, calls one
+``torch_int._CUDA`` entry point and restores the shape.
+"""
+import torch
+
+from .. import _CUDA
+from ..functional.quantization import quantize_per_tensor_absmax
+from ._scalars import ScalarCacheMixin
+
+
+class _W8A8Base(ScalarCacheMixin, torch.nn.Module):
+    _bias_dtype = torch.int8
+
+    def __init__(self, in_features, out_features):
+        super().__init__()
+        self.in_features = in_features
+        self.out_features = out_features
+        weight = torch.randint(-127, 127, (out_features, in_features), dtype=torch.int8)
+        self.register_buffer("weight", weight)
+        self.register_buffer("bias", torch.zeros((1, out_features), dtype=self._bias_dtype))
+
+    def _register_scales(self, alpha, beta=None):
+        self.register_buffer("a", torch.tensor(alpha))
+        if beta is not None:
+            self.register_buffer("b", torch.tensor(beta))
+
+    def to(self, *args, **kwargs):
+        # integer buffers must follow device moves but never a floating dtype cast
+        super().to(*args, **kwargs)
+        device = torch._C._nn._parse_to(*args, **kwargs)[0]
+        if device is not None:
+            self.weight = self.weight.to(device)
+            self.bias = self.bias.to(device)
+        return self
+
+    def _run(self, x):
+        raise NotImplementedError
+
+    @torch.no_grad()
+    def forward(self, x):
+        lead = x.shape[:-1]
+        y = self._run(x.reshape(-1, x.shape[-1]))
+        return y.view(*lead, -1)
+
+    @staticmethod
+    def _quantize_weight(module):
+        return quantize_per_tensor_absmax(module.weight)
+
+
+class W8A8B8O8Linear(_W8A8Base):
+    """int8 in, int8 bias, int8 out (q/k/v projections)."""
+
+    def __init__(self, in_features, out_features, alpha=1.0, beta=1.0):
+        super().__init__(in_features, out_features)
+        self._register_scales(alpha, beta)
+
+    def _run(self, x):
+        return _CUDA.linear_a8_w8_b8_o8(x, self.weight, self.bias, self._scalar("a"), self._scalar("b"))
+
+    @classmethod
+    def from_float(cls, module, input_scale, output_scale):
+        q = cls(module.in_features, module.out_features)
+        q.weight, w_scale = cls._quantize_weight(module)
+        q.bias, b_scale = quantize_per_tensor_absmax(module.bias)
+        q.a = input_scale * w_scale / output_scale
+        q.b = b_scale / output_scale
+        return q
+
+
+class W8A8B8O8LinearReLU(W8A8B8O8Linear):
+    """As W8A8B8O8Linear with a fused ReLU: outputs in [0, 127] (fc1)."""
+
+    def _run(self, x):
+        return _CUDA.linear_relu_a8_w8_b8_o8(x, self.weight, self.bias, self._scalar("a"), self._scalar("b"))
+
+
+class W8A8B32O32LinearWithoutScaling(_W8A8Base):
+    """int8 in, int32 bias, raw int32 accumulators out."""
+    _bias_dtype = torch.int32
+
+    def _run(self, x):
+        return _CUDA.linear_a8_w8_b32_o32(x, self.weight, self.bias)
+
+
+class W8A8B32O32Linear(_W8A8Base):
+    """int8 in, int32 bias, int32 out = round(a*acc + b*bias)."""
+    _bias_dtype = torch.int32
+
+    def __init__(self, in_features, out_features, alpha=1.0, beta=1.0):
+        super().__init__(in_features, out_features)
+        self._register_scales(alpha, beta)
+
+    def _run(self, x):
+        return _CUDA.linear_a8_w8_b32_o32_with_scaling(x, self.weight, self.bias, self._scalar("a"),
+                                                       self._scalar("b"))
+
+    @classmethod
+    def from_float(cls, module, input_scale, output_scale):
+        q = cls(module.in_features, module.out_features)
+        q.weight, w_scale = cls._quantize_weight(module)
+        module.bias = module.bias.float()
+        b_scale = module.bias.abs().max() / (2 ** 31 - 1)
+        q.bias = (module.bias / b_scale).round().to(torch.int32)
+        q.a = input_scale * w_scale / output_scale
+        q.b = b_scale / output_scale
+        q.input_scale, q.output_scale = input_scale, output_scale
+        q.weight_scale, q.bias_scale = w_scale, b_scale
+        return q
+
+
+class W8A8BFP32OFP32Linear(_W8A8Base):
+    """int8 in, fp32 bias, fp32 out = a*acc + bias (out_proj, fc2).  The bias
+    stays fp32 through ``.half()`` / ``.to(dtype)``."""
+    _bias_dtype = torch.float32
+
+    def __init__(self, in_features, out_features, alpha=1.0, beta=1.0):
+        super().__init__(in_features, out_features)
+        self._register_scales(alpha)
+
+    def _apply(self, fn, *args, **kwargs):
+        super()._apply(fn, *args, **kwargs)
+        self.bias = self.bias.to(torch.float32)
+        return self
+
+    def to(self, *args, **kwargs):
+        super().to(*args, **kwargs)
+        self.bias = self.bias.to(torch.float32)
+        return self
+
+    def _run(self, x):
+        if self.bias.dtype != torch.float32:
+            self.bias = self.bias.to(torch.float32)
+        return _CUDA.linear_a8_w8_bfp32_ofp32(x, self.weight, self.bias, self._scalar("a"), 1)
+
+    @classmethod
+    def from_float(cls, module, input_scale):
+        q = cls(module.in_features, module.out_features)
+        q.weight, w_scale = cls._quantize_weight(module)
+        q.bias = module.bias.to(torch.float32)
+        q.a = input_scale * w_scale
+        q.input_scale, q.weight_scale = input_scale, w_scale
+        return q
