@@ -232,8 +232,8 @@ def test_bmm_full_size_properties():
     # (Q K^T)^T = K Q^T
     assert torch.equal(s32.transpose(1, 2), C.bmm_s8t_s8n_s32t(k, q))
     # a checksum of checksums: sum over n of acc[b,m,n] = q[b,m,:] . sum_n k[b,n,:]
-    ksum = k.long().sum(1)
-    assert torch.equal(s32.long().sum(2), torch.einsum("bmk,bk->bm", q.long(), ksum))
+    ksum = k.long().sum(1)  # every value below stays far under 2^53, so fp64 is exact
+    assert torch.equal(s32.long().sum(2), torch.einsum("bmk,bk->bm", q.double(), ksum.double()).long())
     # batches are independent: the first 3 batches alone give the same slices
     assert torch.equal(C.bmm_s8t_s8n_s32t(q[:3].contiguous(), k[:3].contiguous()), s32[:3])
     # the fp32 and int8 epilogues are pure functions of the accumulator
