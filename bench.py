@@ -1,0 +1,240 @@
+#!/usr/bin/env python3
+"""Headline benchmark: the W8A8 linear-kernel sweep at OPT-13B shapes on one MI355X.
+
+One "step" is one pass over BASELINE config 2: (N,K) in {(5120,5120), (20480,5120),
+(5120,20480)} x M in {1,16,128,512,2048,8192} x the four variants (s32 bias/out, fp32
+bias/out, s8 bias/out, fused-ReLU s8 out) = 72 GEMM launches on synthetic int8 data that
+is resident in HBM before the clock starts.  `value` = 2*M*N*K summed over the sweep,
+divided by the wall time of a step, in TOPS.
+
+Also reported on the same JSON line:
+  roofline      the MFMA-bound part of the sweep (M >= 2048): ops per launch / mean launch
+                duration measured with HIP events on the launch stream, against 5.0 POP/s;
+  cpu_baseline  the reference's CPU integer emulation (torch int32 matmul + the fp32
+                epilogue) timed on this box's host cores on a bounded sample;
+  cases         per-case microseconds, TOPS, GB/s and the binding roofline;
+  hbm_kernels   attention BMMs and dq_add_layernorm_q against the 8 TB/s HBM roofline;
+  decoder_layer_ms   Int8OPTDecoderLayer at OPT-13B shape (batch 4, seq 512).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (os.path.join(ROOT, "torch-int_amd"), ROOT):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+PEAK_INT8_TOPS = 5000.0   # MI355X dense INT8 MFMA, TOP/s
+PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
+SHAPES = [(5120, 5120), (20480, 5120), (5120, 20480)]   # (N, K): qkv/out_proj, fc1, fc2
+MS = [1, 16, 128, 512, 2048, 8192]
+VARIANTS = ["b32_o32", "bfp32_ofp32", "b8_o8", "relu_b8_o8"]
+BIAS_BYTES = {"b32_o32": 4, "bfp32_ofp32": 4, "b8_o8": 1, "relu_b8_o8": 1}
+OUT_BYTES = {"b32_o32": 4, "bfp32_ofp32": 4, "b8_o8": 1, "relu_b8_o8": 1}
+
+
+def gemm_bytes(M, N, K, variant):
+    return M * K + N * K + N * BIAS_BYTES[variant] + M * N * OUT_BYTES[variant]
+
+
+def build_sweep(torch, C, dev):
+    g = torch.Generator().manual_seed(0)
+
+    def s8(*shape):
+        return torch.randint(-127, 128, shape, dtype=torch.int8, generator=g).to(dev)
+
+    cases = []
+    for (N, K) in SHAPES:
+        w = s8(N, K)
+        bias = {
+            "b32_o32": torch.randint(-65535, 65535, (N,), dtype=torch.int32, generator=g).to(dev),
+            "bfp32_ofp32": torch.randn(N, generator=g).to(dev),
+            "b8_o8": s8(N),
+        }
+        bias["relu_b8_o8"] = bias["b8_o8"]
+        for M in MS:
+            x = s8(M, K)
+            for v in VARIANTS:
+                alpha = float(torch.empty(1).uniform_(1e-4, 1e-2, generator=g))
+                beta = float(torch.empty(1).uniform_(1e-4, 1e-2, generator=g))
+                if v == "b32_o32":
+                    fn = (lambda x=x, w=w, b=bias[v]: C.linear_a8_w8_b32_o32(x, w, b))
+                elif v == "bfp32_ofp32":
+                    fn = (lambda x=x, w=w, b=bias[v], a=alpha, be=beta: C.linear_a8_w8_bfp32_ofp32(x, w, b, a, be))
+                elif v == "b8_o8":
+                    fn = (lambda x=x, w=w, b=bias[v], a=alpha, be=beta: C.linear_a8_w8_b8_o8(x, w, b, a, be))
+                else:
+                    fn = (lambda x=x, w=w, b=bias[v], a=alpha, be=beta: C.linear_relu_a8_w8_b8_o8(x, w, b, a, be))
+                cases.append({"variant": v, "M": M, "N": N, "K": K, "fn": fn,
+                              "ops": 2.0 * M * N * K, "bytes": float(gemm_bytes(M, N, K, v))})
+    return cases
+
+
+def event_time_ms(torch, fn, iters, warm=2):
+    """Mean duration of fn() in ms, HIP events on the current (launch) stream."""
+    for _ in range(warm):
+        fn()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(iters):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / iters
+
+
+def cpu_baseline(torch):
+    """torch CPU int32 matmul + the oracle's fp32 epilogue (the reference's integer emulation),
+    on an M=256 slice of the q/k/v/out_proj shape, all four variants."""
+    from oracle import oracle as orc
+    g = torch.Generator().manual_seed(0)
+    M, N, K = 256, 5120, 5120
+    x = torch.randint(-127, 128, (M, K), dtype=torch.int8, generator=g)
+    w = torch.randint(-127, 128, (N, K), dtype=torch.int8, generator=g)
+    b8 = torch.randint(-127, 128, (N,), dtype=torch.int8, generator=g)
+    b32 = torch.randint(-65535, 65535, (N,), dtype=torch.int32, generator=g)
+    bf = torch.randn(N, generator=g)
+    t0 = time.perf_counter()
+    orc.linear_a8_w8_b32_o32(x, w, b32, acc_fn=orc.gemm_acc_torch)
+    orc.linear_a8_w8_bfp32_ofp32(x, w, bf, 0.001, 1.0, acc_fn=orc.gemm_acc_torch)
+    orc.linear_a8_w8_b8_o8(x, w, b8, 0.001, 0.01, acc_fn=orc.gemm_acc_torch)
+    orc.linear_relu_a8_w8_b8_o8(x, w, b8, 0.001, 0.01, acc_fn=orc.gemm_acc_torch)
+    dt = time.perf_counter() - t0
+    ops = 4 * 2.0 * M * N * K
+    return {"value": ops / dt / 1e12, "unit": "TOPS", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"4 variants x (M={M}, N={N}, K={K}) torch int32 matmul + fp32 epilogue, "
+                      f"{dt:.1f} s, host cpu_count={os.cpu_count()}"}
+
+
+def hbm_kernels(torch, C, dev):
+    out = []
+    g = torch.Generator().manual_seed(1)
+    for S in (512,):
+        q = torch.randint(-127, 128, (160, S, 128), dtype=torch.int8, generator=g).to(dev)
+        k = torch.randint(-127, 128, (160, S, 128), dtype=torch.int8, generator=g).to(dev)
+        p = torch.randint(0, 128, (160, S, S), dtype=torch.int8, generator=g).to(dev)
+        vt = torch.randint(-127, 128, (160, 128, S), dtype=torch.int8, generator=g).to(dev)
+        ms = event_time_ms(torch, lambda: C.bmm_s8t_s8n_f32t(q, k, 0.002), 50)
+        by = 160.0 * (2 * S * 128 + 4 * S * S)
+        out.append({"kernel": "bmm_s8t_s8n_f32t", "shape": [160, S, S, 128], "us": ms * 1e3,
+                    "GBps": by / ms / 1e6, "frac": by / ms / 1e6 / PEAK_HBM_GBS})
+        ms = event_time_ms(torch, lambda: C.bmm_s8t_s8n_s8t(p, vt, 0.002), 50)
+        by = 160.0 * (S * S + 128 * S + S * 128)
+        out.append({"kernel": "bmm_s8t_s8n_s8t", "shape": [160, S, 128, S], "us": ms * 1e3,
+                    "GBps": by / ms / 1e6, "frac": by / ms / 1e6 / PEAK_HBM_GBS})
+    rows, H = 2048, 5120
+    inp = torch.randint(-65536, 65536, (rows, H), dtype=torch.int32, generator=g).to(dev)
+    res = torch.randn(rows, H, generator=g).to(dev)
+    gamma, beta = torch.ones(H, device=dev), torch.zeros(H, device=dev)
+    ms = event_time_ms(torch, lambda: C.dq_add_layernorm_q(inp, 0.01, res, gamma, beta, 1e-5), 100)
+    by = 13.0 * rows * H + 8 * H
+    out.append({"kernel": "dq_add_layernorm_q", "shape": [rows, H], "us": ms * 1e3,
+                "GBps": by / ms / 1e6, "frac": by / ms / 1e6 / PEAK_HBM_GBS})
+    return out
+
+
+def decoder_layer_ms(torch, dev):
+    from torch_int.models.opt import Int8OPTDecoderLayer
+    torch.manual_seed(0)
+    D, H, F, B, T = 5120, 40, 20480, 4, 512
+    layer = Int8OPTDecoderLayer(D, H, F)
+    for lin in (layer.self_attn.q_proj, layer.self_attn.k_proj, layer.self_attn.v_proj, layer.fc1):
+        lin.bias = torch.randint(-127, 128, (1, lin.out_features), dtype=torch.int8)
+        lin.a.fill_(float(torch.empty(1).uniform_(1e-4, 1e-2)))
+        lin.b.fill_(float(torch.empty(1).uniform_(1e-4, 1e-2)))
+    for lin in (layer.self_attn.out_proj, layer.fc2):
+        lin.bias = torch.randn(1, lin.out_features)
+        lin.a.fill_(float(torch.empty(1).uniform_(1e-4, 1e-2)))
+    layer.self_attn.qk_bmm.a.fill_(0.003)
+    layer.self_attn.pv_bmm.a.fill_(0.004)
+    layer = layer.to(dev)
+    hidden = torch.randn(B, T, D, device=dev)
+    mask = torch.zeros(T, T, device=dev).masked_fill(
+        torch.triu(torch.ones(T, T, dtype=torch.bool, device=dev), 1), torch.finfo(torch.float32).min)
+    mask = mask[None, None].expand(B, 1, T, T).contiguous()
+    return event_time_ms(torch, lambda: layer(hidden.clone(), attention_mask=mask), 10)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--sweep-only", action="store_true", help="skip the per-case, HBM-kernel and layer sections")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (the path has no collectives); use --gpus 1")
+
+    import torch
+    import torch_int._CUDA as C
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no HIP device; the INT8 kernels have no CPU fallback")
+    dev = torch.device("cuda:0")
+    assert C._lib.ti_init() == 0, C._lib.ti_last_error().decode()
+
+    cases = build_sweep(torch, C, dev)
+    sweep_ops = sum(c["ops"] for c in cases)
+
+    def step():
+        for c in cases:
+            c["fn"]()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    value = sweep_ops / (ms_per_step * 1e-3) / 1e12
+
+    result = {
+        "metric": "INT8 GEMM TOPS at OPT-13B shapes (W8A8 linear sweep)", "value": value, "unit": "TOPS",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8",
+        "data": "synthetic",
+        "config": {"workload": "OPT-13B W8A8 linear sweep: (N,K) in {5120x5120, 20480x5120, 5120x20480} x "
+                               "M in {1,16,128,512,2048,8192} x {b32_o32, bfp32_ofp32, b8_o8, relu_b8_o8}",
+                   "launches_per_step": len(cases), "ops_per_step": sweep_ops},
+    }
+
+    if not args.sweep_only:
+        # per-case launch durations (HIP events on the launch stream)
+        table = []
+        mfma_ops = mfma_ms = 0.0
+        n_mfma = 0
+        for c in cases:
+            iters = 20 if c["M"] >= 2048 else 50
+            ms = event_time_ms(torch, c["fn"], iters)
+            tops = c["ops"] / ms / 1e9
+            gbs = c["bytes"] / ms / 1e6
+            bound = "mfma" if c["M"] >= 2048 else "hbm"
+            frac = tops / PEAK_INT8_TOPS if bound == "mfma" else gbs / PEAK_HBM_GBS
+            table.append({"variant": c["variant"], "M": c["M"], "N": c["N"], "K": c["K"], "us": round(ms * 1e3, 2),
+                          "TOPS": round(tops, 1), "GBps": round(gbs, 1), "bound": bound, "frac": round(frac, 4)})
+            if bound == "mfma":
+                mfma_ops += c["ops"]
+                mfma_ms += ms
+                n_mfma += 1
+        achieved = mfma_ops / mfma_ms / 1e9
+        result["roofline"] = {
+            "bound": "mfma", "achieved": achieved, "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
+            "frac": achieved / PEAK_INT8_TOPS, "traffic": None,
+            "kernel": "gemm_tile_kernel<256x256x128> (all M>=2048 cases of the sweep)",
+            "ops_per_launch": mfma_ops / n_mfma, "avg_launch_ms": mfma_ms / n_mfma, "launches": n_mfma}
+        result["cases"] = table
+        result["hbm_kernels"] = hbm_kernels(torch, C, dev)
+        result["decoder_layer_ms"] = decoder_layer_ms(torch, dev)
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(torch)
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -73,6 +73,105 @@ __device__ __forceinline__ void tile_of_workgroup(int pid, int tiles_m, int tile
   tn = in / gsz;
 }
 
+// Applies the epilogue to a wavefront's accumulators and stores them.
+template <class Cfg>
+__device__ __forceinline__ void store_tile(v16i (&acc)[Cfg::TM][Cfg::TN], const GemmParams& p, int m0, int n0,
+                                           int wave_m, int wave_n, int lane) {
+  using E = Epi<Cfg::KIND>;
+  using Out = typename E::Out;
+  using BiasT = typename E::Bias;
+  constexpr int TM = Cfg::TM, TN = Cfg::TN;
+  constexpr bool SWAP = Cfg::SWAP;
+  const int M = p.M, N = p.N;
+  const int frow = lane & 31;
+  Out* __restrict__ C = reinterpret_cast<Out*>(p.C) + (long long)blockIdx.z * p.strideC;
+  const BiasT* __restrict__ bias = reinterpret_cast<const BiasT*>(p.bias);
+  const float alpha = p.alpha, beta = p.beta;
+  const int half = lane >> 5;
+  if (SWAP) {
+    // lane owns row m = .. + (lane & 31) and 16 consecutive columns per block
+    constexpr int VEC = 16 / sizeof(Out);  // outputs per 16-byte store
+    const bool vec_ok = (N % VEC) == 0;
+    const bool bias_al = (reinterpret_cast<uintptr_t>(bias) & 15) == 0;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int nb = n0 + wave_n * Cfg::WTN + j * 32 + half * 16;
+      float bt[16];
+      if (E::kHasBias && vec_ok && bias_al && nb + 16 <= N) {
+        // 16 consecutive bias values in one (int8) or four (32-bit) 16-byte loads
+        BiasT bv[16];
+        constexpr int BV = 16 / sizeof(BiasT);
+#pragma unroll
+        for (int q = 0; q < 16 / BV; ++q) {
+          v4i w = *reinterpret_cast<const v4i*>(bias + nb + q * BV);
+          __builtin_memcpy(&bv[q * BV], &w, 16);
+        }
+#pragma unroll
+        for (int v = 0; v < 16; ++v) bt[v] = E::bias_term(bv[v], beta);
+      } else {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          BiasT bv = BiasT(0);
+          if (E::kHasBias && nb + v < N) bv = bias[nb + v];
+          bt[v] = E::bias_term(bv, beta);
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const int m = m0 + wave_m * Cfg::WTM + i * 32 + frow;
+        if (m >= M) continue;
+        Out* dst = C + (long long)m * N + nb;
+        if (vec_ok && nb + 16 <= N) {
+          if constexpr (sizeof(Out) == 1) {
+            v4i w;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              unsigned b0 = (unsigned char)E::apply(acc[i][j][4 * q + 0], bt[4 * q + 0], alpha);
+              unsigned b1 = (unsigned char)E::apply(acc[i][j][4 * q + 1], bt[4 * q + 1], alpha);
+              unsigned b2 = (unsigned char)E::apply(acc[i][j][4 * q + 2], bt[4 * q + 2], alpha);
+              unsigned b3 = (unsigned char)E::apply(acc[i][j][4 * q + 3], bt[4 * q + 3], alpha);
+              w[q] = (int)(b0 | (b1 << 8) | (b2 << 16) | (b3 << 24));
+            }
+            *reinterpret_cast<v4i*>(dst) = w;
+          } else {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              Out o0 = E::apply(acc[i][j][4 * q + 0], bt[4 * q + 0], alpha);
+              Out o1 = E::apply(acc[i][j][4 * q + 1], bt[4 * q + 1], alpha);
+              Out o2 = E::apply(acc[i][j][4 * q + 2], bt[4 * q + 2], alpha);
+              Out o3 = E::apply(acc[i][j][4 * q + 3], bt[4 * q + 3], alpha);
+              v4i w = {__builtin_bit_cast(int, o0), __builtin_bit_cast(int, o1),
+                       __builtin_bit_cast(int, o2), __builtin_bit_cast(int, o3)};
+              *reinterpret_cast<v4i*>(dst + 4 * q) = w;
+            }
+          }
+        } else {
+#pragma unroll
+          for (int v = 0; v < 16; ++v)
+            if (nb + v < N) dst[v] = E::apply(acc[i][j][v], bt[v], alpha);
+        }
+      }
+    }
+  } else {
+    // lane owns column n = .. + (lane & 31) and rows 8*(v/4) + 4*half + v%4 of each block
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int n = n0 + wave_n * Cfg::WTN + j * 32 + frow;
+      BiasT bv = BiasT(0);
+      if (E::kHasBias && n < N) bv = bias[n];
+      const float bt = E::bias_term(bv, beta);
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int m = m0 + wave_m * Cfg::WTM + i * 32 + 8 * (v >> 2) + 4 * half + (v & 3);
+          if (m < M && n < N) C[(long long)m * N + n] = E::apply(acc[i][j][v], bt, alpha);
+        }
+      }
+    }
+  }
+}
+
 template <class Cfg>
 __global__ __launch_bounds__(Cfg::NT) void gemm_tile_kernel(GemmParams p, int tiles_m, int tiles_n) {
   using E = Epi<Cfg::KIND>;
@@ -185,79 +284,145 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_tile_kernel(GemmParams p, int ti
     __syncthreads();
   }
 
-  // ---- epilogue
-  Out* __restrict__ C = reinterpret_cast<Out*>(p.C) + (long long)blockIdx.z * p.strideC;
-  const BiasT* __restrict__ bias = reinterpret_cast<const BiasT*>(p.bias);
-  const float alpha = p.alpha, beta = p.beta;
-  const int half = lane >> 5;
-  if (SWAP) {
-    // lane owns row m = .. + (lane & 31) and 16 consecutive columns per block
-    constexpr int VEC = 16 / sizeof(Out);  // outputs per 16-byte store
-    const bool vec_ok = (N % VEC) == 0;
+  store_tile<Cfg>(acc, p, m0, n0, wave_m, wave_n, lane);
+}
+
+// ---------------------------------------------------------------------------
+// Pipelined mainloop for K % 64 == 0: global -> LDS copies bypass registers
+// (global_load_lds_dwordx4), K advances 64 bytes per step and PSTAGES LDS
+// stages keep PSTAGES-1 steps of loads in flight.
+//
+// LDS stage = [A panel BM x 64][B panel BN x 64].  A row is four 16-byte
+// chunks; chunk c of panel row r sits at chunk position c ^ ((r >> 2) & 3).
+// One wavefront copy instruction fills 1 KiB of LDS = 16 consecutive panel
+// rows, lane l landing at row l/4, position l%4; the swizzle (and, with SWAP,
+// the row permutation of the B panel) is applied by choosing which global
+// chunk each lane fetches.
+//
+// Synchronisation per step: every wave waits until its own copies for this
+// step have landed (s_waitcnt vmcnt), then one workgroup barrier makes all
+// copies visible and proves that every wave is done reading the stage that is
+// refilled next.
+#define TI_GLOBAL_AS __attribute__((address_space(1)))
+#define TI_LDS_AS __attribute__((address_space(3)))
+
+static constexpr int PBK = 64;
+static constexpr int PSTAGES = 4;
+
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int KIND_, bool SWAP_>
+struct PipeCfg {
+  static constexpr int BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, KIND = KIND_;
+  static constexpr bool SWAP = SWAP_;
+  static constexpr int NWAVES = WAVES_M * WAVES_N;
+  static constexpr int NT = NWAVES * 64;
+  static constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
+  static constexpr int TM = WTM / 32, TN = WTN / 32;
+  static constexpr int STAGE_BYTES = (BM + BN) * PBK;
+  static constexpr int LDS_BYTES = PSTAGES * STAGE_BYTES;
+  static constexpr int COPIES = (BM + BN) / 16 / NWAVES;  // copy instructions per wave per step
+  static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be made of 32x32 blocks");
+  static_assert((BM + BN) % (16 * NWAVES) == 0 && BM % 16 == 0, "panels must split into 1 KiB copies per wave");
+  static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
+};
+
+template <int N>
+__device__ __forceinline__ void wait_copies_then_barrier() {
+  // "memory": no LDS access may be moved across this point by the compiler
+  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N) : "memory");
+}
+
+template <class Cfg>
+__global__ __launch_bounds__(Cfg::NT) void gemm_pipe_kernel(GemmParams p, int tiles_m, int tiles_n) {
+  constexpr int BM = Cfg::BM, BN = Cfg::BN, TM = Cfg::TM, TN = Cfg::TN, COPIES = Cfg::COPIES;
+  constexpr bool SWAP = Cfg::SWAP;
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave_m = wave / Cfg::WAVES_N, wave_n = wave % Cfg::WAVES_N;
+  int tile_m, tile_n;
+  tile_of_workgroup(blockIdx.x, tiles_m, tiles_n, tile_m, tile_n);
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int M = p.M, N = p.N, K = p.K;
+  const int8_t* __restrict__ A = p.A + (long long)blockIdx.z * p.strideA;
+  const int8_t* __restrict__ B = p.B + (long long)blockIdx.z * p.strideB;
+
+  // ---- copy assignment: copy j of this wave fills stage bytes [(wave*COPIES + j) * 1024, +1024)
+  const TI_GLOBAL_AS int8_t* src[COPIES];
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int nb = n0 + wave_n * Cfg::WTN + j * 32 + half * 16;
-      float bt[16];
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        BiasT bv = BiasT(0);
-        if (E::kHasBias && nb + v < N) bv = bias[nb + v];
-        bt[v] = E::bias_term(bv, beta);
-      }
-#pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        const int m = m0 + wave_m * Cfg::WTM + i * 32 + frow;
-        if (m >= M) continue;
-        Out* dst = C + (long long)m * N + nb;
-        if (vec_ok && nb + 16 <= N) {
-          if constexpr (sizeof(Out) == 1) {
-            v4i w;
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-              unsigned b0 = (unsigned char)E::apply(acc[i][j][4 * q + 0], bt[4 * q + 0], alpha);
-              unsigned b1 = (unsigned char)E::apply(acc[i][j][4 * q + 1], bt[4 * q + 1], alpha);
-              unsigned b2 = (unsigned char)E::apply(acc[i][j][4 * q + 2], bt[4 * q + 2], alpha);
-              unsigned b3 = (unsigned char)E::apply(acc[i][j][4 * q + 3], bt[4 * q + 3], alpha);
-              w[q] = (int)(b0 | (b1 << 8) | (b2 << 16) | (b3 << 24));
-            }
-            *reinterpret_cast<v4i*>(dst) = w;
-          } else {
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-              Out o0 = E::apply(acc[i][j][4 * q + 0], bt[4 * q + 0], alpha);
-              Out o1 = E::apply(acc[i][j][4 * q + 1], bt[4 * q + 1], alpha);
-              Out o2 = E::apply(acc[i][j][4 * q + 2], bt[4 * q + 2], alpha);
-              Out o3 = E::apply(acc[i][j][4 * q + 3], bt[4 * q + 3], alpha);
-              v4i w = {__builtin_bit_cast(int, o0), __builtin_bit_cast(int, o1),
-                       __builtin_bit_cast(int, o2), __builtin_bit_cast(int, o3)};
-              *reinterpret_cast<v4i*>(dst + 4 * q) = w;
-            }
-          }
-        } else {
-#pragma unroll
-          for (int v = 0; v < 16; ++v)
-            if (nb + v < N) dst[v] = E::apply(acc[i][j][v], bt[v], alpha);
-        }
-      }
-    }
-  } else {
-    // lane owns column n = .. + (lane & 31) and rows 8*(v/4) + 4*half + v%4 of each block
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int n = n0 + wave_n * Cfg::WTN + j * 32 + frow;
-      BiasT bv = BiasT(0);
-      if (E::kHasBias && n < N) bv = bias[n];
-      const float bt = E::bias_term(bv, beta);
-#pragma unroll
-      for (int i = 0; i < TM; ++i) {
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const int m = m0 + wave_m * Cfg::WTM + i * 32 + 8 * (v >> 2) + 4 * half + (v & 3);
-          if (m < M && n < N) C[(long long)m * N + n] = E::apply(acc[i][j][v], bt, alpha);
-        }
-      }
+  for (int j = 0; j < COPIES; ++j) {
+    const int slab = wave * COPIES + j;          // 16-row slab inside [A panel | B panel]
+    const int prow = slab * 16 + (lane >> 2);    // panel row this lane fills (A rows first)
+    const int pos = lane & 3;
+    if (slab * 16 < BM) {
+      const int chunk = pos ^ ((prow >> 2) & 3);
+      const int gr = m0 + prow < M ? m0 + prow : M - 1;  // edge rows re-read the last row; never stored
+      src[j] = (const TI_GLOBAL_AS int8_t*)(A + (size_t)gr * K + chunk * 16);
+    } else {
+      const int br = prow - BM;
+      const int chunk = pos ^ ((br >> 2) & 3);
+      int lr = br;
+      if (SWAP) lr = (br & ~31) | ((br & 4) << 2) | ((br & 24) >> 1) | (br & 3);  // MFMA row 8q+4h+j -> 16h+4q+j
+      const int gr = n0 + lr < N ? n0 + lr : N - 1;
+      src[j] = (const TI_GLOBAL_AS int8_t*)(B + (size_t)gr * K + chunk * 16);
     }
   }
+  auto issue_copies = [&](int kt) {
+    TI_LDS_AS char* dst = (TI_LDS_AS char*)smem + (kt % PSTAGES) * Cfg::STAGE_BYTES + wave * COPIES * 1024;
+#pragma unroll
+    for (int j = 0; j < COPIES; ++j)
+      __builtin_amdgcn_global_load_lds((const TI_GLOBAL_AS void*)(src[j] + kt * PBK), (TI_LDS_AS void*)(dst + j * 1024),
+                                       16, 0, 0);
+  };
+
+  // ---- fragment addressing: lane reads panel row (lane & 31), chunk 2*ks + (lane >> 5)
+  const int frow = lane & 31;
+  const int fpos = ((lane >> 5) ^ (frow >> 2)) & 3;  // chunk position for ks = 0
+  const int a_frag = (wave_m * Cfg::WTM + frow) * PBK + (fpos << 4);
+  const int b_frag = BM * PBK + (wave_n * Cfg::WTN + frow) * PBK + (fpos << 4);
+
+  v16i acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+
+  const int KT = K / PBK;
+#pragma unroll
+  for (int s = 0; s < PSTAGES - 1; ++s)
+    if (s < KT) issue_copies(s);
+
+  for (int kt = 0; kt < KT; ++kt) {
+    // copies for steps kt+1 .. kt+PSTAGES-2 may stay in flight
+    const int ahead = KT - 1 - kt;
+    if (ahead >= 2) wait_copies_then_barrier<2 * COPIES>();
+    else if (ahead == 1) wait_copies_then_barrier<COPIES>();
+    else wait_copies_then_barrier<0>();
+    if (kt + PSTAGES - 1 < KT) issue_copies(kt + PSTAGES - 1);
+
+    const char* s = smem + (kt % PSTAGES) * Cfg::STAGE_BYTES;
+#pragma unroll
+    for (int ks = 0; ks < PBK / 32; ++ks) {
+      v4i fa[TM], fb[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        fa[i] = *reinterpret_cast<const v4i*>(s + ((a_frag ^ (ks << 5)) + i * 32 * PBK));
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        fb[j] = *reinterpret_cast<const v4i*>(s + ((b_frag ^ (ks << 5)) + j * 32 * PBK));
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = SWAP ? __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[j], fa[i], acc[i][j], 0, 0, 0)
+                           : __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    }
+  }
+
+  store_tile<Cfg>(acc, p, m0, n0, wave_m, wave_n, lane);
 }
 
 // Any-shape fallback (K not a multiple of 16 or operands not 16-byte aligned):
@@ -301,6 +466,24 @@ static int launch_tile(const GemmParams& p, hipStream_t stream) {
   return TI_OK;
 }
 
+template <class Cfg>
+static int launch_pipe(const GemmParams& p, hipStream_t stream) {
+  static bool attr_set = false;
+  auto kern = gemm_pipe_kernel<Cfg>;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
+    if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    attr_set = true;
+  }
+  const int tiles_m = (p.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (p.N + Cfg::BN - 1) / Cfg::BN;
+  dim3 grid(tiles_m * tiles_n, 1, p.batch);
+  hipLaunchKernelGGL(kern, grid, dim3(Cfg::NT), Cfg::LDS_BYTES, stream, p, tiles_m, tiles_n);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "gemm launch: %s", hipGetErrorString(e));
+  return TI_OK;
+}
+
 template <int KIND>
 static int launch_kind(const GemmParams& p, hipStream_t stream) {
   using Out = typename Epi<KIND>::Out;
@@ -321,6 +504,10 @@ static int launch_kind(const GemmParams& p, hipStream_t stream) {
   constexpr bool SWAP = sizeof(Out) == 1;
   const long long t256 = (long long)((p.M + 255) / 256) * ((p.N + 255) / 256) * p.batch;
   const long long t128 = (long long)((p.M + 127) / 128) * ((p.N + 127) / 128) * p.batch;
+  if (p.K % PBK == 0 && p.K >= PBK) {
+    if (t256 >= 160) return launch_pipe<PipeCfg<256, 256, 2, 4, KIND, SWAP>>(p, stream);
+    if (t128 >= 128) return launch_pipe<PipeCfg<128, 128, 2, 2, KIND, SWAP>>(p, stream);
+  }
   if (t256 >= 160) return launch_tile<TileCfg<256, 256, 2, 4, KIND, SWAP>>(p, stream);
   if (t128 >= 128) return launch_tile<TileCfg<128, 128, 2, 2, KIND, SWAP>>(p, stream);
   return launch_tile<TileCfg<64, 64, 2, 2, KIND, SWAP>>(p, stream);
