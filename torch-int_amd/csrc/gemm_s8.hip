@@ -17,6 +17,8 @@
 //     consecutive output columns of one output row (16-byte s8 stores).
 //     Without SWAP a lane holds one output column of 16 rows and the 32 lanes
 //     of a half-wave store 128 contiguous bytes of 32-bit results.
+#include <cstdlib>
+#include <type_traits>
 #include "ti_common.h"
 
 namespace ti {
@@ -75,8 +77,8 @@ __device__ __forceinline__ void tile_of_workgroup(int pid, int tiles_m, int tile
 
 // Applies the epilogue to a wavefront's accumulators and stores them.
 template <class Cfg>
-__device__ __forceinline__ void store_tile(v16i (&acc)[Cfg::TM][Cfg::TN], const GemmParams& p, int m0, int n0,
-                                           int wave_m, int wave_n, int lane) {
+__device__ __forceinline__ void store_tile(v16i (&acc)[Cfg::TM][Cfg::TN], const GemmParams& p, int batch, int m0,
+                                           int n0, int wave_m, int wave_n, int lane) {
   using E = Epi<Cfg::KIND>;
   using Out = typename E::Out;
   using BiasT = typename E::Bias;
@@ -84,7 +86,7 @@ __device__ __forceinline__ void store_tile(v16i (&acc)[Cfg::TM][Cfg::TN], const 
   constexpr bool SWAP = Cfg::SWAP;
   const int M = p.M, N = p.N;
   const int frow = lane & 31;
-  Out* __restrict__ C = reinterpret_cast<Out*>(p.C) + (long long)blockIdx.z * p.strideC;
+  Out* __restrict__ C = reinterpret_cast<Out*>(p.C) + (long long)batch * p.strideC;
   const BiasT* __restrict__ bias = reinterpret_cast<const BiasT*>(p.bias);
   const float alpha = p.alpha, beta = p.beta;
   const int half = lane >> 5;
@@ -284,13 +286,18 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_tile_kernel(GemmParams p, int ti
     __syncthreads();
   }
 
-  store_tile<Cfg>(acc, p, m0, n0, wave_m, wave_n, lane);
+  store_tile<Cfg>(acc, p, blockIdx.z, m0, n0, wave_m, wave_n, lane);
 }
 
 // ---------------------------------------------------------------------------
-// Pipelined mainloop for K % 64 == 0: global -> LDS copies bypass registers
-// (global_load_lds_dwordx4), K advances 64 bytes per step and PSTAGES LDS
-// stages keep PSTAGES-1 steps of loads in flight.
+// Pipelined, persistent mainloop for K % 64 == 0.
+//
+// Global -> LDS copies bypass registers (global_load_lds_dwordx4), K advances
+// 64 bytes per step and STAGES LDS stages keep STAGES-1 steps of copies in
+// flight.  A workgroup walks a list of output tiles (blockIdx.x, +gridDim.x,
+// ...); the copy stream runs STAGES-1 steps ahead of the multiply stream and
+// crosses tile boundaries, so the epilogue of one tile overlaps the first
+// copies of the next.
 //
 // LDS stage = [A panel BM x 64][B panel BN x 64].  A row is four 16-byte
 // chunks; chunk c of panel row r sits at chunk position c ^ ((r >> 2) & 3).
@@ -299,30 +306,32 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_tile_kernel(GemmParams p, int ti
 // the row permutation of the B panel) is applied by choosing which global
 // chunk each lane fetches.
 //
-// Synchronisation per step: every wave waits until its own copies for this
-// step have landed (s_waitcnt vmcnt), then one workgroup barrier makes all
-// copies visible and proves that every wave is done reading the stage that is
-// refilled next.
+// One K step of a wavefront: read the second half (k 32..63) of the step's
+// fragments while the first half multiplies; then wait until this wave's own
+// copies for the next step have landed (s_waitcnt vmcnt), pass one workgroup
+// barrier (all copies visible; every wave done with the stage that is about
+// to be refilled), issue the copies STAGES-1 steps ahead, read the first half
+// of the next step's fragments and multiply the second half of this one.
 #define TI_GLOBAL_AS __attribute__((address_space(1)))
 #define TI_LDS_AS __attribute__((address_space(3)))
 
 static constexpr int PBK = 64;
-static constexpr int PSTAGES = 4;
 
-template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int KIND_, bool SWAP_>
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int STAGES_, int KIND_, bool SWAP_>
 struct PipeCfg {
   static constexpr int BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, KIND = KIND_;
+  static constexpr int STAGES = STAGES_;
   static constexpr bool SWAP = SWAP_;
   static constexpr int NWAVES = WAVES_M * WAVES_N;
   static constexpr int NT = NWAVES * 64;
   static constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
   static constexpr int TM = WTM / 32, TN = WTN / 32;
   static constexpr int STAGE_BYTES = (BM + BN) * PBK;
-  static constexpr int LDS_BYTES = PSTAGES * STAGE_BYTES;
+  static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
   static constexpr int COPIES = (BM + BN) / 16 / NWAVES;  // copy instructions per wave per step
   static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be made of 32x32 blocks");
   static_assert((BM + BN) % (16 * NWAVES) == 0 && BM % 16 == 0, "panels must split into 1 KiB copies per wave");
-  static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
+  static_assert(LDS_BYTES <= 160 * 1024 && STAGES >= 3, "LDS budget");
 };
 
 template <int N>
@@ -331,9 +340,11 @@ __device__ __forceinline__ void wait_copies_then_barrier() {
   asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N) : "memory");
 }
 
+// items = tiles_m * tiles_n * batch work items; item -> (batch, tile) with the tile index minor.
 template <class Cfg>
-__global__ __launch_bounds__(Cfg::NT) void gemm_pipe_kernel(GemmParams p, int tiles_m, int tiles_n) {
+__global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe_kernel(GemmParams p, int tiles_m, int tiles_n, int items) {
   constexpr int BM = Cfg::BM, BN = Cfg::BN, TM = Cfg::TM, TN = Cfg::TN, COPIES = Cfg::COPIES;
+  constexpr int S = Cfg::STAGES;
   constexpr bool SWAP = Cfg::SWAP;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
@@ -341,39 +352,64 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_pipe_kernel(GemmParams p, int ti
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wave_m = wave / Cfg::WAVES_N, wave_n = wave % Cfg::WAVES_N;
-  int tile_m, tile_n;
-  tile_of_workgroup(blockIdx.x, tiles_m, tiles_n, tile_m, tile_n);
-  const int m0 = tile_m * BM, n0 = tile_n * BN;
   const int M = p.M, N = p.N, K = p.K;
-  const int8_t* __restrict__ A = p.A + (long long)blockIdx.z * p.strideA;
-  const int8_t* __restrict__ B = p.B + (long long)blockIdx.z * p.strideB;
+  const int KT = K / PBK;
+  const int tiles = tiles_m * tiles_n;
+  const int first = blockIdx.x, stride = gridDim.x;
+  const int my_items = (items - first + stride - 1) / stride;  // >= 1 (grid <= items)
+  const int G = my_items * KT;                                  // K steps this workgroup multiplies
 
-  // ---- copy assignment: copy j of this wave fills stage bytes [(wave*COPIES + j) * 1024, +1024)
+  // ---- copy stream: copy j of this wave fills stage bytes [(wave*COPIES + j) * 1024, +1024)
   const TI_GLOBAL_AS int8_t* src[COPIES];
+  auto set_copy_item = [&](int item) {
+    const int b = item / tiles;
+    int tile_m, tile_n;
+    tile_of_workgroup(item - b * tiles, tiles_m, tiles_n, tile_m, tile_n);
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int8_t* A = p.A + (long long)b * p.strideA;
+    const int8_t* B = p.B + (long long)b * p.strideB;
 #pragma unroll
-  for (int j = 0; j < COPIES; ++j) {
-    const int slab = wave * COPIES + j;          // 16-row slab inside [A panel | B panel]
-    const int prow = slab * 16 + (lane >> 2);    // panel row this lane fills (A rows first)
-    const int pos = lane & 3;
-    if (slab * 16 < BM) {
-      const int chunk = pos ^ ((prow >> 2) & 3);
-      const int gr = m0 + prow < M ? m0 + prow : M - 1;  // edge rows re-read the last row; never stored
-      src[j] = (const TI_GLOBAL_AS int8_t*)(A + (size_t)gr * K + chunk * 16);
-    } else {
-      const int br = prow - BM;
-      const int chunk = pos ^ ((br >> 2) & 3);
-      int lr = br;
-      if (SWAP) lr = (br & ~31) | ((br & 4) << 2) | ((br & 24) >> 1) | (br & 3);  // MFMA row 8q+4h+j -> 16h+4q+j
-      const int gr = n0 + lr < N ? n0 + lr : N - 1;
-      src[j] = (const TI_GLOBAL_AS int8_t*)(B + (size_t)gr * K + chunk * 16);
+    for (int j = 0; j < COPIES; ++j) {
+      const int slab = wave * COPIES + j;        // 16-row slab inside [A panel | B panel]
+      const int prow = slab * 16 + (lane >> 2);  // panel row this lane fills (A rows first)
+      const int pos = lane & 3;
+      if (slab * 16 < BM) {
+        const int chunk = pos ^ ((prow >> 2) & 3);
+        const int gr = m0 + prow < M ? m0 + prow : M - 1;  // edge rows re-read the last row; never stored
+        src[j] = (const TI_GLOBAL_AS int8_t*)(A + (size_t)gr * K + chunk * 16);
+      } else {
+        const int br = prow - BM;
+        const int chunk = pos ^ ((br >> 2) & 3);
+        int lr = br;
+        if (SWAP) lr = (br & ~31) | ((br & 4) << 2) | ((br & 24) >> 1) | (br & 3);  // MFMA row 8q+4h+j -> 16h+4q+j
+        const int gr = n0 + lr < N ? n0 + lr : N - 1;
+        src[j] = (const TI_GLOBAL_AS int8_t*)(B + (size_t)gr * K + chunk * 16);
+      }
     }
-  }
-  auto issue_copies = [&](int kt) {
-    TI_LDS_AS char* dst = (TI_LDS_AS char*)smem + (kt % PSTAGES) * Cfg::STAGE_BYTES + wave * COPIES * 1024;
+  };
+  // Copy cursor: work item, K step inside it, global step.  When it runs past the last
+  // item it keeps re-copying the final K step into the stage that is free anyway, so
+  // that exactly S-1 steps of copies are in flight at every step and the wait counts
+  // below never change.
+  int c_item = first, c_kt = 0, c_g = 0, c_live = 1;
+  auto issue_copies = [&]() {
+    TI_LDS_AS char* dst = (TI_LDS_AS char*)smem + (c_g % S) * Cfg::STAGE_BYTES + wave * COPIES * 1024;
 #pragma unroll
     for (int j = 0; j < COPIES; ++j)
-      __builtin_amdgcn_global_load_lds((const TI_GLOBAL_AS void*)(src[j] + kt * PBK), (TI_LDS_AS void*)(dst + j * 1024),
+      __builtin_amdgcn_global_load_lds((const TI_GLOBAL_AS void*)(src[j] + c_kt * PBK), (TI_LDS_AS void*)(dst + j * 1024),
                                        16, 0, 0);
+    c_kt += c_live;
+    ++c_g;
+  };
+  auto advance_copy_item = [&]() {  // call when c_live && c_kt == KT
+    if (c_g < G) {
+      c_kt = 0;
+      c_item += stride;
+      set_copy_item(c_item);
+    } else {
+      c_live = 0;
+      c_kt = KT - 1;
+    }
   };
 
   // ---- fragment addressing: lane reads panel row (lane & 31), chunk 2*ks + (lane >> 5)
@@ -383,46 +419,104 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_pipe_kernel(GemmParams p, int ti
   const int b_frag = BM * PBK + (wave_n * Cfg::WTN + frow) * PBK + (fpos << 4);
 
   v16i acc[TM][TN];
+  auto zero_acc = [&]() {
 #pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < TN; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
-
-  const int KT = K / PBK;
-#pragma unroll
-  for (int s = 0; s < PSTAGES - 1; ++s)
-    if (s < KT) issue_copies(s);
-
-  for (int kt = 0; kt < KT; ++kt) {
-    // copies for steps kt+1 .. kt+PSTAGES-2 may stay in flight
-    const int ahead = KT - 1 - kt;
-    if (ahead >= 2) wait_copies_then_barrier<2 * COPIES>();
-    else if (ahead == 1) wait_copies_then_barrier<COPIES>();
-    else wait_copies_then_barrier<0>();
-    if (kt + PSTAGES - 1 < KT) issue_copies(kt + PSTAGES - 1);
-
-    const char* s = smem + (kt % PSTAGES) * Cfg::STAGE_BYTES;
-#pragma unroll
-    for (int ks = 0; ks < PBK / 32; ++ks) {
-      v4i fa[TM], fb[TN];
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-        fa[i] = *reinterpret_cast<const v4i*>(s + ((a_frag ^ (ks << 5)) + i * 32 * PBK));
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
       for (int j = 0; j < TN; ++j)
-        fb[j] = *reinterpret_cast<const v4i*>(s + ((b_frag ^ (ks << 5)) + j * 32 * PBK));
 #pragma unroll
-      for (int i = 0; i < TM; ++i)
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+  };
+  auto read_frags = [&](int g, int ks, v4i (&fa)[TM], v4i (&fb)[TN]) {
+    const char* s = smem + (g % S) * Cfg::STAGE_BYTES;
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
-          acc[i][j] = SWAP ? __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[j], fa[i], acc[i][j], 0, 0, 0)
-                           : __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    for (int i = 0; i < TM; ++i)
+      fa[i] = *reinterpret_cast<const v4i*>(s + ((a_frag ^ (ks << 5)) + i * 32 * PBK));
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+      fb[j] = *reinterpret_cast<const v4i*>(s + ((b_frag ^ (ks << 5)) + j * 32 * PBK));
+  };
+  auto mma = [&](v4i (&fa)[TM], v4i (&fb)[TN]) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        acc[i][j] = SWAP ? __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[j], fa[i], acc[i][j], 0, 0, 0)
+                         : __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+  };
+  // scheduling hint: one LDS read after each of the first TM+TN MFMAs of a group
+  auto interleave = [&]() {
+#pragma unroll
+    for (int i = 0; i < TM + TN; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 DS read
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - (TM + TN), 0);
+  };
+
+  // ---- prologue: S-1 steps of copies, wait for the first
+  set_copy_item(c_item);
+#pragma unroll
+  for (int s = 0; s < S - 1; ++s) {
+    issue_copies();
+    if (c_live && c_kt == KT) advance_copy_item();
+  }
+  wait_copies_then_barrier<(S - 2) * COPIES>();
+
+  v4i fa0[TM], fb0[TN], fa1[TM], fb1[TN];
+  read_frags(0, 0, fa0, fb0);
+  zero_acc();
+
+  int item = first, kt = 0, g = 0;  // multiply cursor
+  // One K step.  LAST = last K step of a work item: the next item's first fragments are
+  // read after the epilogue instead, so they do not occupy registers during it.
+  auto step = [&](auto last) {
+    constexpr bool LAST = decltype(last)::value;
+    read_frags(g, 1, fa1, fb1);
+    mma(fa0, fb0);
+    interleave();
+    wait_copies_then_barrier<(S - 3) * COPIES>();  // step g+1 landed; g+2 .. g+S-2 may be in flight
+    issue_copies();                                // step g+S-1 into the stage step g-1 used
+    if (!LAST) read_frags(g + 1, 0, fa0, fb0);
+    mma(fa1, fb1);
+    if (!LAST) interleave();
+  };
+  auto finish_item = [&]() {
+    const int b = item / tiles;
+    int tile_m, tile_n;
+    tile_of_workgroup(item - b * tiles, tiles_m, tiles_n, tile_m, tile_n);
+    // opaque copy of the lane id: keeps the epilogue's address arithmetic inside the loop
+    // (hoisted, it would occupy registers during the whole mainloop)
+    int lane_here = lane;
+    asm volatile("" : "+v"(lane_here));
+    store_tile<Cfg>(acc, p, b, tile_m * BM, tile_n * BN, wave_m, wave_n, lane_here);
+    item += stride;
+    kt = 0;
+    zero_acc();
+  };
+
+  while (g < G) {
+    // steps until the multiply or the copy cursor reaches the end of its work item
+    int n = KT - kt;
+    if (c_live && KT - c_kt < n) n = KT - c_kt;
+    const bool item_done = kt + n == KT;
+    const int plain = item_done ? n - 1 : n;
+    for (int i = 0; i < plain; ++i) {
+      step(std::false_type{});
+      ++g;
+    }
+    if (item_done) {
+      step(std::true_type{});
+      ++g;
+    }
+    kt += n;
+    if (c_live && c_kt == KT) advance_copy_item();
+    if (item_done) {
+      finish_item();
+      if (g < G) read_frags(g, 0, fa0, fb0);
     }
   }
-
-  store_tile<Cfg>(acc, p, m0, n0, wave_m, wave_n, lane);
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // the trailing filler copies must land before the LDS is released
 }
 
 // Any-shape fallback (K not a multiple of 16 or operands not 16-byte aligned):
@@ -466,6 +560,18 @@ static int launch_tile(const GemmParams& p, hipStream_t stream) {
   return TI_OK;
 }
 
+static int num_cus() {
+  static int n = 0;
+  if (n == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+      n = prop.multiProcessorCount;
+    if (n <= 0) n = 256;
+  }
+  return n;
+}
+
 template <class Cfg>
 static int launch_pipe(const GemmParams& p, hipStream_t stream) {
   static bool attr_set = false;
@@ -477,8 +583,12 @@ static int launch_pipe(const GemmParams& p, hipStream_t stream) {
     attr_set = true;
   }
   const int tiles_m = (p.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (p.N + Cfg::BN - 1) / Cfg::BN;
-  dim3 grid(tiles_m * tiles_n, 1, p.batch);
-  hipLaunchKernelGGL(kern, grid, dim3(Cfg::NT), Cfg::LDS_BYTES, stream, p, tiles_m, tiles_n);
+  const long long items = (long long)tiles_m * tiles_n * p.batch;
+  if (items > 0x7fffffffLL) return fail(TI_ERR_INVALID_ARG, "too many output tiles (%lld)", items);
+  // one resident workgroup per LDS-sized slot; a multiple of 8 keeps the XCD mapping of tile ids
+  const long long slots = (long long)num_cus() * ((160 * 1024) / Cfg::LDS_BYTES);
+  const int grid = (int)(items < slots ? items : slots);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, p, tiles_m, tiles_n, (int)items);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "gemm launch: %s", hipGetErrorString(e));
   return TI_OK;
@@ -505,8 +615,11 @@ static int launch_kind(const GemmParams& p, hipStream_t stream) {
   const long long t256 = (long long)((p.M + 255) / 256) * ((p.N + 255) / 256) * p.batch;
   const long long t128 = (long long)((p.M + 127) / 128) * ((p.N + 127) / 128) * p.batch;
   if (p.K % PBK == 0 && p.K >= PBK) {
-    if (t256 >= 160) return launch_pipe<PipeCfg<256, 256, 2, 4, KIND, SWAP>>(p, stream);
-    if (t128 >= 128) return launch_pipe<PipeCfg<128, 128, 2, 2, KIND, SWAP>>(p, stream);
+    static const int variant = getenv("TI_TILE") ? atoi(getenv("TI_TILE")) : 0;
+    if (t256 >= 160 && variant == 1) return launch_pipe<PipeCfg<256, 128, 2, 2, 3, KIND, SWAP>>(p, stream);
+    if (t256 >= 160 && variant == 2) return launch_pipe<PipeCfg<128, 256, 2, 2, 3, KIND, SWAP>>(p, stream);
+    if (t256 >= 160) return launch_pipe<PipeCfg<256, 256, 2, 4, 4, KIND, SWAP>>(p, stream);
+    if (t128 >= 128) return launch_pipe<PipeCfg<128, 128, 2, 2, 4, KIND, SWAP>>(p, stream);
   }
   if (t256 >= 160) return launch_tile<TileCfg<256, 256, 2, 4, KIND, SWAP>>(p, stream);
   if (t128 >= 128) return launch_tile<TileCfg<128, 128, 2, 2, KIND, SWAP>>(p, stream);

@@ -28,23 +28,24 @@ enum EpiKind : int {
   EPI_S32_RAW = 7,     // out = acc
 };
 
-__device__ __forceinline__ float clamp_s8f(float t) {
-  // NaN -> 0, like a saturating convert.  fminf/fmaxf would return the
-  // non-NaN operand, so test explicitly.
-  t = (t != t) ? 0.0f : t;
-  t = t < -128.0f ? -128.0f : t;
-  t = t > 127.0f ? 127.0f : t;
-  return t;
-}
-
-__device__ __forceinline__ int rne_s8(float t) { return (int)__builtin_rintf(clamp_s8f(t)); }
-
+// round-half-even then v_cvt_i32_f32, which saturates to int32 and maps NaN to 0
 __device__ __forceinline__ int rne_sat_s32(float t) {
-  if (t != t) return 0;
-  if (t >= 2147483648.0f) return 2147483647;
-  if (t <= -2147483648.0f) return (-2147483647 - 1);
-  return (int)__builtin_rintf(t);
+  const float r = __builtin_rintf(t);
+  int o;
+  asm("v_cvt_i32_f32 %0, %1" : "=v"(o) : "v"(r));
+  return o;
 }
+
+// s8(rint(clamp(t, lo, 127))): rounding first and clamping the integer gives the same
+// value for every finite t (the bounds are integers), one VALU op cheaper.
+template <int LO>
+__device__ __forceinline__ int rne_clamp(float t) {
+  int i = rne_sat_s32(t);
+  i = i < LO ? LO : i;
+  i = i > 127 ? 127 : i;
+  return i;
+}
+__device__ __forceinline__ int rne_s8(float t) { return rne_clamp<-128>(t); }
 
 template <int KIND>
 struct Epi;
@@ -97,9 +98,8 @@ struct Epi<EPI_S8_RELU> {
   static constexpr bool kHasBias = true;
   static __device__ __forceinline__ float bias_term(Bias b, float beta) { return beta * (float)(int)b; }
   static __device__ __forceinline__ Out apply(int acc, float bt, float alpha) {
-    float t = __builtin_fmaf(alpha, (float)acc, bt);
-    t = (t > 0.0f) ? t : 0.0f;  // also maps NaN to 0
-    return (int8_t)rne_s8(t);
+    // relu then clamp == integer clamp to [0, 127] after rounding (NaN -> 0 either way)
+    return (int8_t)rne_clamp<0>(__builtin_fmaf(alpha, (float)acc, bt));
   }
 };
 template <>

@@ -26,7 +26,9 @@ __all__ = [
     "dq_add_layernorm_q",
 ]
 
-LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libtorch_int_hip.so")
+# TORCH_INT_HIP_LIB points at another build of the same library (e.g. an experiment)
+LIB_PATH = os.environ.get("TORCH_INT_HIP_LIB") or os.path.join(
+    os.path.dirname(os.path.abspath(__file__)), "lib", "libtorch_int_hip.so")
 
 _vp, _i64, _f32, _int = ctypes.c_void_p, ctypes.c_int64, ctypes.c_float, ctypes.c_int
 
