@@ -91,12 +91,82 @@ def test_decoder_layer_small():
     assert err <= 1e-3, err
 
 
+def _capture(layer):
+    """Forward hooks that keep (inputs, output) of every kernel-backed or fp32 sub-module."""
+    rec, handles = {}, []
+    a = layer.self_attn
+    mods = {"ln1": layer.self_attn_layer_norm, "q": a.q_proj, "k": a.k_proj, "v": a.v_proj, "qk": a.qk_bmm,
+            "pv": a.pv_bmm, "out": a.out_proj, "ln2": layer.final_layer_norm, "fc1": layer.fc1, "fc2": layer.fc2}
+    for name, m in mods.items():
+        def hook(mod, inp, out, name=name):
+            rec[name] = (tuple(t.detach().clone() for t in inp), out.detach().clone())
+        handles.append(m.register_forward_hook(hook))
+    return rec, handles
+
+
 @torch.no_grad()
 def test_decoder_layer_opt13b_shape():
-    # BASELINE config 4: hidden 5120, 40 heads, FFN 20480, batch 4, seq 512, causal mask
-    _say("decoder layer OPT-13B shape (CPU emulation takes a while)")
-    err = _compare_layer(5120, 40, 20480, 4, 512, seed=2, fast=True)
-    assert err <= 1e-3, err
+    """BASELINE config 4: hidden 5120, 40 heads, FFN 20480, batch 4, seq 512, causal mask.
+
+    With per-tensor scales drawn from U(1e-4, 1e-2) nearly every int8 activation saturates,
+    so the layer as a whole amplifies a one-LSB difference after the fp32 softmax/LayerNorm
+    into O(1%) output changes; end-to-end comparison is meaningless at this config.  Instead
+    every operator of the GPU forward pass is checked on the inputs it actually received:
+    kernel-backed operators bit for bit against the oracle (on a sample of rows / heads, all
+    columns), fp32 library operators within 1e-3 relative error of their CPU versions."""
+    from oracle import oracle as orc
+    D, H, F, B, T = 5120, 40, 20480, 4, 512
+    g = torch.Generator().manual_seed(2)
+    layer = randomize_int8_layer(Int8OPTDecoderLayer(D, H, F), g)
+    hidden = torch.randn(B, T, D, generator=g)
+    mask = causal_mask(B, T, T)
+    gl = copy.deepcopy(layer).to(DEV)
+    rec, handles = _capture(gl)
+    _say("decoder layer OPT-13B shape: GPU forward")
+    h_gpu = hidden.to(DEV)
+    out = gl(h_gpu, attention_mask=mask.to(DEV), use_cache=True)
+    assert out[0] is h_gpu and out[0].shape == (B, T, D) and torch.isfinite(out[0]).all()
+    for h in handles:
+        h.remove()
+    rows = torch.cat([torch.arange(0, 64), torch.arange(1000, 1064), torch.arange(B * T - 64, B * T)])
+
+    def check_linear(name, ref_fn, lin, scalars):
+        _say("  check", name)
+        x, y = rec[name][0][0].cpu().view(B * T, -1)[rows], rec[name][1].cpu().view(B * T, -1)[rows]
+        ref = ref_fn(x.contiguous(), lin.weight, lin.bias, *scalars, acc_fn=orc.gemm_acc_torch)
+        if ref.dtype == torch.float32:
+            assert torch.equal(y, ref), name
+        else:
+            assert (y != ref).sum().item() == 0, name
+
+    a = layer.self_attn
+    for name, lin in (("q", a.q_proj), ("k", a.k_proj), ("v", a.v_proj)):
+        check_linear(name, orc.linear_a8_w8_b8_o8, lin, (lin.a.item(), lin.b.item()))
+    check_linear("out", orc.linear_a8_w8_bfp32_ofp32, a.out_proj, (a.out_proj.a.item(), 1))
+    check_linear("fc1", orc.linear_relu_a8_w8_b8_o8, layer.fc1, (layer.fc1.a.item(), layer.fc1.b.item()))
+    check_linear("fc2", orc.linear_a8_w8_bfp32_ofp32, layer.fc2, (layer.fc2.a.item(), 1))
+    heads = torch.tensor([0, 39, 77, 159])
+    _say("  check qk / pv")
+    (q_in, k_in), s_out = rec["qk"]
+    assert s_out.shape == (B * H, T, T)
+    assert torch.equal(s_out[heads].cpu(), orc.bmm_s8t_s8n_f32t(q_in[heads].cpu(), k_in[heads].cpu(), a.qk_bmm.a.item()))
+    (p_in, v_in), c_out = rec["pv"]
+    assert c_out.shape == (B * H, T, D // H) and int(p_in.min()) >= 0
+    assert torch.equal(c_out[heads].cpu(), orc.bmm_s8t_s8n_s8t(p_in[heads].cpu(), v_in[heads].cpu(), a.pv_bmm.a.item()))
+    # fp32 library pieces: LayerNormQ (int8 within one LSB) and softmax -> int8 probabilities
+    _say("  check layer norms and softmax")
+    for name, ln in (("ln1", layer.self_attn_layer_norm), ("ln2", layer.final_layer_norm)):
+        x, y = rec[name][0][0].cpu(), rec[name][1].cpu()
+        ref = ln(x)
+        assert (y.int() - ref.int()).abs().max() <= 1 and (y != ref).float().mean() < 1e-3, name
+    probs_gpu = p_in[heads].float() / 127
+    scores = s_out[heads].cpu().view(4, T, T) + mask[0, 0]
+    probs_cpu = torch.softmax(torch.clamp_min(scores, torch.finfo(torch.float32).min), -1)
+    assert (probs_gpu.cpu() - probs_cpu).abs().max() <= 0.5 / 127 + 1e-3
+    # residual algebra: out = hidden + attn_out + fc2_out, in that order, in fp32
+    r1 = hidden.to(DEV) + rec["out"][1]
+    assert torch.equal(rec["ln2"][0][0], r1)
+    assert torch.equal(out[0], r1 + rec["fc2"][1])
 
 
 @torch.no_grad()
