@@ -29,6 +29,10 @@ for _p in (os.path.join(ROOT, "torch-int_amd"), ROOT):
 
 PEAK_INT8_TOPS = 5000.0   # MI355X dense INT8 MFMA, TOP/s
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
+# HBM bytes per launch of the dominant kernel need rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE), which
+# cannot be taken from inside this process; the measured figure is kept in profiles/ (1.44 GB for the
+# 8192x20480x5120 s8 case against 0.31 GB algorithmic).
+TRAFFIC_NOTE = None
 SHAPES = [(5120, 5120), (20480, 5120), (5120, 20480)]   # (N, K): qkv/out_proj, fc1, fc2
 MS = [1, 16, 128, 512, 2048, 8192]
 VARIANTS = ["b32_o32", "bfp32_ofp32", "b8_o8", "relu_b8_o8"]
@@ -225,8 +229,8 @@ def main():
         achieved = mfma_ops / mfma_ms / 1e9
         result["roofline"] = {
             "bound": "mfma", "achieved": achieved, "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
-            "frac": achieved / PEAK_INT8_TOPS, "traffic": None,
-            "kernel": "gemm_tile_kernel<256x256x128> (all M>=2048 cases of the sweep)",
+            "frac": achieved / PEAK_INT8_TOPS, "traffic": TRAFFIC_NOTE,
+            "kernel": "gemm_pipe_kernel<256x256x64, 4 stages> (all M>=2048 cases of the sweep)",
             "ops_per_launch": mfma_ops / n_mfma, "avg_launch_ms": mfma_ms / n_mfma, "launches": n_mfma}
         result["cases"] = table
         result["hbm_kernels"] = hbm_kernels(torch, C, dev)
