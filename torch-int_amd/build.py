@@ -24,12 +24,25 @@ FLAGS = [
 ]
 
 
+def build_fastcall(verbose=True):
+    """The optional CPython forwarder (plain C, gcc): cuts per-call overhead of the Python wrappers."""
+    import sysconfig
+    out = os.path.join(LIB_DIR, "_ti_fastcall" + sysconfig.get_config_var("EXT_SUFFIX"))
+    cmd = ["gcc", "-O2", "-fPIC", "-shared", "-Wall", "-I" + sysconfig.get_paths()["include"],
+           os.path.join(CSRC, "fastcall.c"), "-o", out, "-L" + LIB_DIR, "-ltorch_int_hip", "-Wl,-rpath,$ORIGIN"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return out
+
+
 def build(verbose=True, extra_flags=()):
     os.makedirs(LIB_DIR, exist_ok=True)
     cmd = [HIPCC, *FLAGS, *extra_flags, "-o", LIB_PATH] + [os.path.join(CSRC, s) for s in SOURCES]
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)
+    build_fastcall(verbose)
     return LIB_PATH
 
 

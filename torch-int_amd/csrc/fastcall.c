@@ -1,0 +1,103 @@
+/* _ti_fastcall: a minimal CPython module that forwards already-validated raw
+ * pointers and sizes to the C ABI of libtorch_int_hip.so.  It exists only to
+ * cut the per-call cost of ctypes argument conversion (several microseconds,
+ * which is more than a decode-sized kernel takes); it has no logic of its own
+ * and no dependency on torch. */
+#define PY_SSIZE_T_CLEAN
+#include <Python.h>
+#include <stdint.h>
+#include "../../include/torch_int_hip.h"
+
+static inline void* as_ptr(PyObject* o) { return (void*)(uintptr_t)PyLong_AsUnsignedLongLong(o); }
+static inline int64_t as_i64(PyObject* o) { return (int64_t)PyLong_AsLongLong(o); }
+static inline float as_f32(PyObject* o) { return (float)PyFloat_AsDouble(o); }
+
+/* linear(kind, x, w, bias, out, M, N, K, alpha, beta, ws, ws_bytes, stream) -> status */
+static PyObject* fc_linear(PyObject* self, PyObject* const* a, Py_ssize_t n) {
+  (void)self;
+  if (n != 13) {
+    PyErr_SetString(PyExc_TypeError, "linear expects 13 arguments");
+    return NULL;
+  }
+  long kind = PyLong_AsLong(a[0]);
+  void *x = as_ptr(a[1]), *w = as_ptr(a[2]), *b = as_ptr(a[3]), *o = as_ptr(a[4]);
+  int64_t M = as_i64(a[5]), N = as_i64(a[6]), K = as_i64(a[7]);
+  float alpha = as_f32(a[8]), beta = as_f32(a[9]);
+  void* ws = as_ptr(a[10]);
+  int64_t wsb = as_i64(a[11]);
+  void* st = as_ptr(a[12]);
+  if (PyErr_Occurred()) return NULL;
+  int rc;
+  switch (kind) {
+    case 0: rc = ti_linear_a8_w8_b32_o32(x, w, b, o, M, N, K, ws, wsb, st); break;
+    case 1: rc = ti_linear_a8_w8_b32_o32_with_scaling(x, w, b, o, M, N, K, alpha, beta, ws, wsb, st); break;
+    case 2: rc = ti_linear_a8_w8_bfp32_ofp32(x, w, b, o, M, N, K, alpha, beta, ws, wsb, st); break;
+    case 3: rc = ti_linear_a8_w8_b8_o8(x, w, b, o, M, N, K, alpha, beta, ws, wsb, st); break;
+    case 4: rc = ti_linear_relu_a8_w8_b8_o8(x, w, b, o, M, N, K, alpha, beta, ws, wsb, st); break;
+    default:
+      PyErr_SetString(PyExc_ValueError, "unknown linear kind");
+      return NULL;
+  }
+  return PyLong_FromLong(rc);
+}
+
+/* bmm(kind, a, b, c, batch, M, N, K, alpha, stream) -> status */
+static PyObject* fc_bmm(PyObject* self, PyObject* const* a, Py_ssize_t n) {
+  (void)self;
+  if (n != 10) {
+    PyErr_SetString(PyExc_TypeError, "bmm expects 10 arguments");
+    return NULL;
+  }
+  long kind = PyLong_AsLong(a[0]);
+  void *pa = as_ptr(a[1]), *pb = as_ptr(a[2]), *pc = as_ptr(a[3]);
+  int64_t B = as_i64(a[4]), M = as_i64(a[5]), N = as_i64(a[6]), K = as_i64(a[7]);
+  float alpha = as_f32(a[8]);
+  void* st = as_ptr(a[9]);
+  if (PyErr_Occurred()) return NULL;
+  int rc;
+  switch (kind) {
+    case 5: rc = ti_bmm_s8t_s8n_f32t(pa, pb, pc, B, M, N, K, alpha, st); break;
+    case 6: rc = ti_bmm_s8t_s8n_s8t(pa, pb, pc, B, M, N, K, alpha, st); break;
+    case 7: rc = ti_bmm_s8t_s8n_s32t(pa, pb, pc, B, M, N, K, st); break;
+    default:
+      PyErr_SetString(PyExc_ValueError, "unknown bmm kind");
+      return NULL;
+  }
+  return PyLong_FromLong(rc);
+}
+
+/* ln_q(input, scale, residual, gamma, beta, eps, r_out, q_out, rows, H, stream) -> status */
+static PyObject* fc_ln_q(PyObject* self, PyObject* const* a, Py_ssize_t n) {
+  (void)self;
+  if (n != 11) {
+    PyErr_SetString(PyExc_TypeError, "ln_q expects 11 arguments");
+    return NULL;
+  }
+  void* in = as_ptr(a[0]);
+  float scale = as_f32(a[1]);
+  void *res = as_ptr(a[2]), *g = as_ptr(a[3]), *b = as_ptr(a[4]);
+  float eps = as_f32(a[5]);
+  void *ro = as_ptr(a[6]), *qo = as_ptr(a[7]);
+  int64_t rows = as_i64(a[8]), H = as_i64(a[9]);
+  void* st = as_ptr(a[10]);
+  if (PyErr_Occurred()) return NULL;
+  return PyLong_FromLong(ti_dq_add_layernorm_q(in, scale, res, g, b, eps, ro, qo, rows, H, st));
+}
+
+static PyObject* fc_last_error(PyObject* self, PyObject* noargs) {
+  (void)self;
+  (void)noargs;
+  return PyUnicode_FromString(ti_last_error());
+}
+
+static PyMethodDef methods[] = {
+    {"linear", (PyCFunction)(void (*)(void))fc_linear, METH_FASTCALL, "forward to ti_linear_*"},
+    {"bmm", (PyCFunction)(void (*)(void))fc_bmm, METH_FASTCALL, "forward to ti_bmm_*"},
+    {"ln_q", (PyCFunction)(void (*)(void))fc_ln_q, METH_FASTCALL, "forward to ti_dq_add_layernorm_q"},
+    {"last_error", fc_last_error, METH_NOARGS, "ti_last_error()"},
+    {NULL, NULL, 0, NULL}};
+
+static struct PyModuleDef moddef = {PyModuleDef_HEAD_INIT, "_ti_fastcall", "raw-pointer forwarder to libtorch_int_hip.so",
+                                    -1, methods, NULL, NULL, NULL, NULL};
+
+PyMODINIT_FUNC PyInit__ti_fastcall(void) { return PyModule_Create(&moddef); }

@@ -519,6 +519,265 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe_kernel(GemmParams p, int
   __builtin_amdgcn_s_waitcnt(0x0F70);  // the trailing filler copies must land before the LDS is released
 }
 
+// Epilogue of the M <= 16 kernels: the lane holds row m and columns nb .. nb+3.
+template <int KIND>
+__device__ __forceinline__ void store_skinny_tile(v4i acc, const GemmParams& p, int batch, int m, int nb) {
+  using E = Epi<KIND>;
+  using Out = typename E::Out;
+  using BiasT = typename E::Bias;
+  const int N = p.N;
+  Out* C = reinterpret_cast<Out*>(p.C) + (long long)batch * p.strideC;
+  const BiasT* bias = reinterpret_cast<const BiasT*>(p.bias);
+  Out o[4];
+#pragma unroll
+  for (int v = 0; v < 4; ++v) {
+    BiasT bv = BiasT(0);
+    if (E::kHasBias && nb + v < N) bv = bias[nb + v];
+    o[v] = E::apply(acc[v], E::bias_term(bv, p.beta), p.alpha);
+  }
+  Out* dst = C + (long long)m * N + nb;
+  const bool whole = (N % 4 == 0) && nb + 4 <= N;
+  if (whole && sizeof(Out) == 4) {
+    using W = typename std::conditional<sizeof(Out) == 4, Out, int>::type;
+    v4i w4 = {__builtin_bit_cast(int, (W)o[0]), __builtin_bit_cast(int, (W)o[1]), __builtin_bit_cast(int, (W)o[2]),
+              __builtin_bit_cast(int, (W)o[3])};
+    *reinterpret_cast<v4i*>(dst) = w4;
+  } else if (whole) {
+    *reinterpret_cast<unsigned*>(dst) = (unsigned)(unsigned char)o[0] | ((unsigned)(unsigned char)o[1] << 8) |
+                                        ((unsigned)(unsigned char)o[2] << 16) | ((unsigned)(unsigned char)o[3] << 24);
+  } else {
+#pragma unroll
+    for (int v = 0; v < 4; ++v)
+      if (nb + v < N) dst[v] = o[v];
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Skinny GEMM for M <= 16 (decode): HBM-bound, every weight byte is used once.
+//
+// A workgroup of NW waves owns 16 weight rows (output columns); the waves
+// split K evenly and add their partial 16x16 tiles through LDS at the end.
+// Weight fragments go straight from global memory into MFMA operand registers
+// (no LDS): for the j-th v_mfma_i32_16x16x64_i8 of a 256-byte K block, lane
+// (r = lane & 15, g = lane >> 4) loads 16-byte chunk 4j + g of row r, so one
+// load instruction reads 64 contiguous bytes of each of 16 rows.
+// All loads of NBLK blocks are issued before the first MFMA so that each wave
+// keeps NBLK KiB of weights in flight.
+template <int NBLK, int KIND>
+__global__ __launch_bounds__(1024) void gemm_skinny_kernel(GemmParams p) {
+  using E = Epi<KIND>;
+  using Out = typename E::Out;
+  using BiasT = typename E::Bias;
+  extern __shared__ int red[];  // [NW - 1][256]
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int nw = blockDim.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int M = p.M, N = p.N, K = p.K;
+  const int n0 = blockIdx.x * 16;
+  const int8_t* A = p.A + (long long)blockIdx.z * p.strideA;
+  const int8_t* B = p.B + (long long)blockIdx.z * p.strideB;
+  const int nrow = n0 + r < N ? n0 + r : N - 1;
+  const int mrow = r < M ? r : M - 1;
+  const v4i* wp = reinterpret_cast<const v4i*>(B + (size_t)nrow * K) + g;
+  const v4i* xp = reinterpret_cast<const v4i*>(A + (size_t)mrow * K) + g;
+  // this wave's range of 16-byte chunks, a whole number of 256-byte blocks (16 chunks) long
+  const int chunks = K >> 4;
+  const int per_wave = (((chunks + nw - 1) / nw) + 15) & ~15;
+  const int c_begin = wave * per_wave;
+  const int c_end = c_begin + per_wave < chunks ? c_begin + per_wave : chunks;
+
+  v4i acc = {0, 0, 0, 0};
+  int c = c_begin;
+  for (; c + 16 * NBLK <= c_end; c += 16 * NBLK) {
+    v4i w[NBLK][4], x[NBLK][4];
+#pragma unroll
+    for (int b = 0; b < NBLK; ++b)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) w[b][j] = __builtin_nontemporal_load(wp + c + b * 16 + j * 4);
+#pragma unroll
+    for (int b = 0; b < NBLK; ++b)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) x[b][j] = xp[c + b * 16 + j * 4];
+#pragma unroll
+    for (int b = 0; b < NBLK; ++b)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[b][j], x[b][j], acc, 0, 0, 0);
+  }
+  for (; c < c_end; c += 16) {  // remaining blocks; chunks past the end count as zeros
+    const v4i z = {0, 0, 0, 0};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const bool ok = c + j * 4 + g < c_end;
+      v4i w = ok ? wp[c + j * 4] : z;
+      v4i x = ok ? xp[c + j * 4] : z;
+      acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(w, x, acc, 0, 0, 0);
+    }
+  }
+
+  // ---- add the K slices (integer adds: any order gives the same bits)
+  if (wave > 0) {
+#pragma unroll
+    for (int v = 0; v < 4; ++v) red[(wave - 1) * 256 + v * 64 + lane] = acc[v];
+  }
+  __syncthreads();
+  if (wave > 0) return;
+  for (int w = 0; w < nw - 1; ++w)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) acc[v] += red[w * 256 + v * 64 + lane];
+
+  if (r >= M) return;
+  store_skinny_tile<KIND>(acc, p, blockIdx.z, r, n0 + 4 * g);
+}
+
+// ---------------------------------------------------------------------------
+// Streaming GEMM for M <= 16 with many output columns (decode projections):
+// the weight matrix is read once, in 1 KiB contiguous runs.
+//
+// A workgroup of four waves owns 16 weight rows at a time (a "strip") and
+// walks K in blocks of 1024 bytes; it is persistent and takes strips
+// blockIdx.x, +gridDim.x, ...  One global->LDS copy instruction moves the
+// whole 1 KiB block of one row (64 lanes x 16 bytes, contiguous in HBM); lane
+// l fetches chunk l ^ row, so that the later 16-byte fragment reads of 16
+// different rows at the same logical chunk hit 16 different bank groups.  The
+// 16 activation rows of the block (rows >= M repeat row M-1; L2-resident) are
+// staged the same way.  S stages of 32 KiB keep S-1 blocks of copies in flight
+// and the copy stream runs across strip boundaries.  Wave w multiplies the
+// w-th 256-byte quarter of a block with four v_mfma_i32_16x16x64_i8; at the
+// end of a strip the four partial tiles are added through LDS and wave 0
+// applies the epilogue.  Requires K % 1024 == 0.
+static constexpr int SBK = 1024;
+static constexpr int S_RED = 3 * 256 * 4;  // partial tiles of waves 1..3
+
+// MX = activation rows staged per block (1, 4 or 16 >= M); S = LDS stages.
+template <int KIND, int MX, int S>
+__global__ __launch_bounds__(256) void gemm_stream_kernel(GemmParams p, int strips_per_batch, int strips) {
+  constexpr int ROWS = 16 + MX;              // row copies per block
+  constexpr int COPIES = (ROWS + 3) / 4;     // per wave; indices past ROWS repeat the last row copy
+  constexpr int STAGE = ROWS * SBK;
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  int* red = reinterpret_cast<int*>(smem + S * STAGE);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 15, g = lane >> 4;
+  const int M = p.M, N = p.N, K = p.K;
+  const int KB = K / SBK;
+  const int first = blockIdx.x, stride = gridDim.x;
+  const int my_strips = (strips - first + stride - 1) / stride;
+  const int G = my_strips * KB;
+
+  // copy q of a block: q < 16 weight row q, else activation row q - 16; wave w does q = w, w+4, ...
+  const TI_GLOBAL_AS int8_t* src[COPIES];
+  auto set_copy_strip = [&](int strip) {
+    const int b = strip / strips_per_batch;
+    const int n0 = (strip - b * strips_per_batch) * 16;
+    const int8_t* A = p.A + (long long)b * p.strideA;
+    const int8_t* B = p.B + (long long)b * p.strideB;
+#pragma unroll
+    for (int i = 0; i < COPIES; ++i) {
+      int q = wave + 4 * i;
+      q = q < ROWS ? q : ROWS - 1;
+      if (q < 16) {
+        const int nrow = n0 + q < N ? n0 + q : N - 1;
+        src[i] = (const TI_GLOBAL_AS int8_t*)(B + (size_t)nrow * K + ((lane ^ q) << 4));
+      } else {
+        const int xr = q - 16;
+        const int mrow = xr < M ? xr : M - 1;
+        src[i] = (const TI_GLOBAL_AS int8_t*)(A + (size_t)mrow * K + ((lane ^ xr) << 4));
+      }
+    }
+  };
+  // Copy cursor; past the last strip it keeps re-copying the final block into the free
+  // stage so that the number of copies in flight (and the wait count) never changes.
+  int c_strip = first, c_kb = 0, c_g = 0, c_live = 1;
+  auto issue = [&]() {
+    TI_LDS_AS char* dst = (TI_LDS_AS char*)smem + (c_g % S) * STAGE;
+    const size_t off = (size_t)c_kb * SBK;
+#pragma unroll
+    for (int i = 0; i < COPIES; ++i) {
+      int q = wave + 4 * i;
+      q = q < ROWS ? q : ROWS - 1;
+      __builtin_amdgcn_global_load_lds((const TI_GLOBAL_AS void*)(src[i] + off), (TI_LDS_AS void*)(dst + q * SBK), 16,
+                                       0, 0);
+    }
+    c_kb += c_live;
+    ++c_g;
+    if (c_live && c_kb == KB) {
+      if (c_g < G) {
+        c_kb = 0;
+        c_strip += stride;
+        set_copy_strip(c_strip);
+      } else {
+        c_live = 0;
+        c_kb = KB - 1;
+      }
+    }
+  };
+  // fragment j of this wave's quarter: logical chunk wave*16 + 4j + g, stored at chunk ^ row
+  const int xr = r < MX ? r : MX - 1;
+  int woff[4], xoff[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int c = wave * 16 + 4 * j + g;
+    woff[j] = r * SBK + ((c ^ r) << 4);
+    xoff[j] = (16 + xr) * SBK + ((c ^ xr) << 4);
+  }
+
+  set_copy_strip(c_strip);
+#pragma unroll
+  for (int i = 0; i < S - 1; ++i) issue();
+
+  v4i acc = {0, 0, 0, 0};
+  int strip = first, kb = 0;
+  for (int gs = 0; gs < G; ++gs) {
+    // block gs has landed (S-2 younger blocks may be in flight); all waves are done with block gs-1
+    wait_copies_then_barrier<(S - 2) * COPIES>();
+    issue();  // block gs+S-1 into the stage block gs-1 used
+    const char* st = smem + (gs % S) * STAGE;
+    v4i wf[4], xf[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      wf[j] = *reinterpret_cast<const v4i*>(st + woff[j]);
+      xf[j] = *reinterpret_cast<const v4i*>(st + xoff[j]);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[j], xf[j], acc, 0, 0, 0);
+    if (++kb == KB) {
+      // ---- strip finished: add the four quarters (integer adds: any order gives the same bits)
+      if (wave > 0) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) red[(wave - 1) * 256 + v * 64 + lane] = acc[v];
+      }
+      __syncthreads();
+      if (wave == 0) {
+#pragma unroll
+        for (int w = 0; w < 3; ++w)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) acc[v] += red[w * 256 + v * 64 + lane];
+        const int b = strip / strips_per_batch;
+        if (r < M) store_skinny_tile<KIND>(acc, p, b, r, (strip - b * strips_per_batch) * 16 + 4 * g);
+      }
+      // the next write to red[] is at least one workgroup barrier (top of the next block) away
+      acc = v4i{0, 0, 0, 0};
+      kb = 0;
+      strip += stride;
+    }
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // trailing filler copies must land before the LDS is released
+}
+
+// waves per workgroup for the skinny kernel: enough waves to cover HBM latency, at
+// least one 256-byte block of K per wave
+static int skinny_waves(const GemmParams& p) {
+  const long long strips = (long long)((p.N + 15) / 16) * p.batch;
+  long long nw = (4096 + strips - 1) / strips;
+  const long long kmax = p.K / 256 > 0 ? p.K / 256 : 1;
+  if (nw > kmax) nw = kmax;
+  if (nw > 16) nw = 16;
+  if (nw < 1) nw = 1;
+  return (int)nw;
+}
+
 // Any-shape fallback (K not a multiple of 16 or operands not 16-byte aligned):
 // one thread per output element, scalar loop over K.
 template <int KIND>
@@ -610,14 +869,50 @@ static int launch_kind(const GemmParams& p, hipStream_t stream) {
     if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "gemm launch: %s", hipGetErrorString(e));
     return TI_OK;
   }
+  if (p.M <= 16 && p.K % SBK == 0 && (long long)((p.N + 15) / 16) * p.batch >= 256) {
+    const int spb = (p.N + 15) / 16;
+    const long long strips = (long long)spb * p.batch;
+    if (strips > 0x7fffffffLL) return fail(TI_ERR_INVALID_ARG, "too many output strips (%lld)", strips);
+    const int cus = num_cus();
+    // Stage depth beyond two did not raise the measured bandwidth (5.2-5.4 TB/s at N=20480), so two
+    // stages and as many resident workgroups as the LDS allows.
+    auto launch = [&](auto kern, int rows, int per_cu) -> int {
+      const int lds = 2 * rows * SBK + S_RED;
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+      if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+      const long long slots = (long long)cus * per_cu;
+      hipLaunchKernelGGL(kern, dim3((unsigned)(strips < slots ? strips : slots)), dim3(256), lds, stream, p, spb,
+                         (int)strips);
+      e = hipGetLastError();
+      if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "gemm launch: %s", hipGetErrorString(e));
+      return TI_OK;
+    };
+    if (p.M == 1) return launch(gemm_stream_kernel<KIND, 1, 2>, 17, 4);
+    if (p.M <= 4) return launch(gemm_stream_kernel<KIND, 4, 2>, 20, 3);
+    return launch(gemm_stream_kernel<KIND, 16, 2>, 32, 2);
+  }
+  if (p.M <= 16) {
+    const int nw = skinny_waves(p);
+    dim3 grid((p.N + 15) / 16, 1, p.batch);
+    const size_t lds = (size_t)(nw - 1) * 256 * sizeof(int);
+    // blocks of K per wave decide how many loads are worth batching
+    const int blocks_per_wave = p.K / 256 / nw;
+    if (blocks_per_wave >= 4)
+      hipLaunchKernelGGL((gemm_skinny_kernel<4, KIND>), grid, dim3(64 * nw), lds, stream, p);
+    else if (blocks_per_wave >= 2)
+      hipLaunchKernelGGL((gemm_skinny_kernel<2, KIND>), grid, dim3(64 * nw), lds, stream, p);
+    else
+      hipLaunchKernelGGL((gemm_skinny_kernel<1, KIND>), grid, dim3(64 * nw), lds, stream, p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "gemm launch: %s", hipGetErrorString(e));
+    return TI_OK;
+  }
   // 8-bit outputs take the orientation whose lanes own 16 consecutive columns.
   constexpr bool SWAP = sizeof(Out) == 1;
   const long long t256 = (long long)((p.M + 255) / 256) * ((p.N + 255) / 256) * p.batch;
   const long long t128 = (long long)((p.M + 127) / 128) * ((p.N + 127) / 128) * p.batch;
   if (p.K % PBK == 0 && p.K >= PBK) {
-    static const int variant = getenv("TI_TILE") ? atoi(getenv("TI_TILE")) : 0;
-    if (t256 >= 160 && variant == 1) return launch_pipe<PipeCfg<256, 128, 2, 2, 3, KIND, SWAP>>(p, stream);
-    if (t256 >= 160 && variant == 2) return launch_pipe<PipeCfg<128, 256, 2, 2, 3, KIND, SWAP>>(p, stream);
     if (t256 >= 160) return launch_pipe<PipeCfg<256, 256, 2, 4, 4, KIND, SWAP>>(p, stream);
     if (t128 >= 128) return launch_pipe<PipeCfg<128, 128, 2, 2, 4, KIND, SWAP>>(p, stream);
   }

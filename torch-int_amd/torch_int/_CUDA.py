@@ -65,7 +65,41 @@ def _load_library():
 
 
 _lib = _load_library()
-_workspaces = {}  # device index -> uint8 tensor used as split-K scratch
+
+
+def _load_fastcall():
+    """The optional CPython forwarder built next to the library (csrc/fastcall.c).  It calls the
+    same C ABI; without it the calls go through ctypes, a few microseconds slower each."""
+    if os.environ.get("TORCH_INT_HIP_LIB"):
+        return None  # the forwarder is linked against the default library
+    import glob
+    import importlib.util
+    hits = glob.glob(os.path.join(os.path.dirname(LIB_PATH), "_ti_fastcall*.so"))
+    if not hits:
+        return None
+    try:
+        spec = importlib.util.spec_from_file_location("_ti_fastcall", hits[0])
+        mod = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(mod)
+        return mod
+    except Exception:  # pragma: no cover - e.g. built for another interpreter
+        return None
+
+
+_fast = _load_fastcall()
+_workspaces = {}  # (device index, stream) -> zero-initialised uint8 tensor used as split-K scratch
+_raw_stream = torch._C._cuda_getCurrentRawStream
+_current_device = torch.cuda.current_device
+_empty = torch.empty
+_I8, _I32, _F32 = torch.int8, torch.int32, torch.float32
+
+# kind codes shared with csrc/ti_common.h (EpiKind) and csrc/fastcall.c
+_K_B32, _K_B32S, _K_F32, _K_S8, _K_RELU, _K_BMM_F32, _K_BMM_S8, _K_BMM_S32 = range(8)
+_LINEAR_CTYPES = {_K_B32: _lib.ti_linear_a8_w8_b32_o32, _K_B32S: _lib.ti_linear_a8_w8_b32_o32_with_scaling,
+                  _K_F32: _lib.ti_linear_a8_w8_bfp32_ofp32, _K_S8: _lib.ti_linear_a8_w8_b8_o8,
+                  _K_RELU: _lib.ti_linear_relu_a8_w8_b8_o8}
+_BMM_CTYPES = {_K_BMM_F32: _lib.ti_bmm_s8t_s8n_f32t, _K_BMM_S8: _lib.ti_bmm_s8t_s8n_s8t,
+               _K_BMM_S32: _lib.ti_bmm_s8t_s8n_s32t}
 
 
 def _fail(op, msg):
@@ -87,34 +121,33 @@ def _check(op, name, t, dtype, ndim, device=None):
         _fail(op, f"{name} must be contiguous (packed row-major), got strides {t.stride()}")
 
 
-def _stream(device):
-    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
-
-
-def _call(op, fn, device, *args):
-    if device.index != torch.cuda.current_device():
-        with torch.cuda.device(device):
-            rc = fn(*args)
-    else:
-        rc = fn(*args)
+def _status(op, rc):
     if rc != 0:
-        _fail(op, f"{_lib.ti_last_error().decode()} (status {rc})")
+        msg = _fast.last_error() if _fast is not None else _lib.ti_last_error().decode()
+        _fail(op, f"{msg} (status {rc})")
 
 
-def _workspace(device, nbytes):
+def _workspace(dev_index, stream, nbytes):
+    """Split-K scratch: zero-filled once; the kernels leave it zeroed.  One per (device, stream) so
+    that calls on different streams never share it."""
     if nbytes <= 0:
-        return None, 0
-    ws = _workspaces.get(device.index)
+        return 0, 0
+    key = (dev_index, stream)
+    ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
-        ws = torch.empty(int(nbytes), dtype=torch.uint8, device=device)
-        _workspaces[device.index] = ws
-    return ws, ws.numel()
+        ws = torch.zeros(int(nbytes), dtype=torch.uint8, device=torch.device("cuda", dev_index))
+        _workspaces[key] = ws
+    return ws.data_ptr(), ws.numel()
 
 
-def _linear(op, fn, x, w, bias, bias_dtype, out_dtype, scalars):
-    _check(op, "input", x, torch.int8, 2)
+def _linear(op, kind, x, w, bias, bias_dtype, out_dtype, alpha, beta):
+    # fast accept path first; the slow path below names what is wrong
+    if not (type(x) is torch.Tensor and type(w) is torch.Tensor and x.dtype is _I8 and w.dtype is _I8
+            and x.dim() == 2 and w.dim() == 2 and x.is_cuda and w.device == x.device
+            and x.is_contiguous() and w.is_contiguous()):
+        _check(op, "input", x, _I8, 2)
+        _check(op, "weight", w, _I8, 2, x.device)
     dev = x.device
-    _check(op, "weight", w, torch.int8, 2, dev)
     if not isinstance(bias, torch.Tensor):
         _fail(op, f"bias must be a torch.Tensor, got {type(bias).__name__}")
     if bias.device != dev:
@@ -125,75 +158,106 @@ def _linear(op, fn, x, w, bias, bias_dtype, out_dtype, scalars):
         _fail(op, f"input is [{M},{K}] but weight is {tuple(w.shape)}: inner dimensions differ")
     if bias.numel() != N:
         _fail(op, f"bias has {bias.numel()} elements, weight has {N} output rows")
-    bias = bias.reshape(-1)
-    _check(op, "bias", bias, bias_dtype, 1, dev)
-    out = torch.empty((M, N), dtype=out_dtype, device=dev)
+    if bias.dtype is not bias_dtype:
+        _fail(op, f"bias must be {bias_dtype}, got {bias.dtype}")
+    if not bias.is_contiguous():
+        bias = bias.contiguous()
+    out = _empty((M, N), dtype=out_dtype, device=dev)
     if M == 0 or N == 0:
         return out
-    ws, ws_bytes = _workspace(dev, _lib.ti_linear_workspace_bytes(M, N, K))
-    _call(op, fn, dev, x.data_ptr(), w.data_ptr(), bias.data_ptr(), out.data_ptr(), M, N, K, *scalars,
-          ws.data_ptr() if ws is not None else None, ws_bytes, _stream(dev))
+    idx = dev.index
+    switch = idx != _current_device()
+    if switch:
+        prev = _current_device()
+        torch.cuda.set_device(idx)
+    try:
+        stream = _raw_stream(idx)
+        ws_ptr, ws_bytes = 0, 0  # no kernel uses split-K scratch yet (ti_linear_workspace_bytes() == 0)
+        if _fast is not None:
+            rc = _fast.linear(kind, x.data_ptr(), w.data_ptr(), bias.data_ptr(), out.data_ptr(), M, N, K,
+                              alpha, beta, ws_ptr, ws_bytes, stream)
+        else:
+            scal = () if kind == _K_B32 else (alpha, beta)
+            rc = _LINEAR_CTYPES[kind](x.data_ptr(), w.data_ptr(), bias.data_ptr(), out.data_ptr(), M, N, K, *scal,
+                                      ws_ptr or None, ws_bytes, stream or None)
+    finally:
+        if switch:
+            torch.cuda.set_device(prev)
+    if rc:
+        _status(op, rc)
     return out
 
 
 def linear_a8_w8_b32_o32(input, weight, bias):
     """int32 [M,N] = input[M,K] . weight[N,K]^T + bias[N]  (upstream linear.cu:13-136)."""
-    return _linear("linear_a8_w8_b32_o32", _lib.ti_linear_a8_w8_b32_o32, input, weight, bias,
-                   torch.int32, torch.int32, ())
+    return _linear("linear_a8_w8_b32_o32", _K_B32, input, weight, bias, _I32, _I32, 1.0, 1.0)
 
 
 def linear_a8_w8_b32_o32_with_scaling(input, weight, bias, alpha, beta):
     """int32 [M,N] = sat(round(alpha*acc + beta*bias))  (upstream linear.cu:139-243)."""
-    return _linear("linear_a8_w8_b32_o32_with_scaling", _lib.ti_linear_a8_w8_b32_o32_with_scaling,
-                   input, weight, bias, torch.int32, torch.int32, (float(alpha), float(beta)))
+    return _linear("linear_a8_w8_b32_o32_with_scaling", _K_B32S, input, weight, bias, _I32, _I32,
+                   float(alpha), float(beta))
 
 
 def linear_a8_w8_bfp32_ofp32(input, weight, bias, alpha, beta):
     """fp32 [M,N] = alpha*acc + beta*bias, fp32 bias  (upstream linear.cu:246-365)."""
-    return _linear("linear_a8_w8_bfp32_ofp32", _lib.ti_linear_a8_w8_bfp32_ofp32, input, weight, bias,
-                   torch.float32, torch.float32, (float(alpha), float(beta)))
+    return _linear("linear_a8_w8_bfp32_ofp32", _K_F32, input, weight, bias, _F32, _F32, float(alpha), float(beta))
 
 
 def linear_a8_w8_b8_o8(input, weight, bias, alpha, beta):
     """int8 [M,N] = sat_s8(round(alpha*acc + beta*bias)), int8 bias  (upstream linear.cu:369-473)."""
-    return _linear("linear_a8_w8_b8_o8", _lib.ti_linear_a8_w8_b8_o8, input, weight, bias,
-                   torch.int8, torch.int8, (float(alpha), float(beta)))
+    return _linear("linear_a8_w8_b8_o8", _K_S8, input, weight, bias, _I8, _I8, float(alpha), float(beta))
 
 
 def linear_relu_a8_w8_b8_o8(input, weight, bias, alpha, beta):
     """int8 [M,N] in [0,127] = sat_s8(round(relu(alpha*acc + beta*bias)))  (upstream linear.cu:476-625)."""
-    return _linear("linear_relu_a8_w8_b8_o8", _lib.ti_linear_relu_a8_w8_b8_o8, input, weight, bias,
-                   torch.int8, torch.int8, (float(alpha), float(beta)))
+    return _linear("linear_relu_a8_w8_b8_o8", _K_RELU, input, weight, bias, _I8, _I8, float(alpha), float(beta))
 
 
-def _bmm(op, fn, a, b, out_dtype, scalars):
-    _check(op, "A", a, torch.int8, 3)
+def _bmm(op, kind, a, b, out_dtype, alpha):
+    _check(op, "A", a, _I8, 3)
     dev = a.device
-    _check(op, "B", b, torch.int8, 3, dev)
+    _check(op, "B", b, _I8, 3, dev)
     batch, M, K = a.shape
     if b.shape[0] != batch or b.shape[2] != K:
         _fail(op, f"A is {tuple(a.shape)} and B is {tuple(b.shape)}: batch and inner dimensions must match")
     N = b.shape[1]
-    out = torch.empty((batch, M, N), dtype=out_dtype, device=dev)
+    out = _empty((batch, M, N), dtype=out_dtype, device=dev)
     if out.numel() == 0:
         return out
-    _call(op, fn, dev, a.data_ptr(), b.data_ptr(), out.data_ptr(), batch, M, N, K, *scalars, _stream(dev))
+    idx = dev.index
+    switch = idx != _current_device()
+    if switch:
+        prev = _current_device()
+        torch.cuda.set_device(idx)
+    try:
+        stream = _raw_stream(idx)
+        if _fast is not None:
+            rc = _fast.bmm(kind, a.data_ptr(), b.data_ptr(), out.data_ptr(), batch, M, N, K, alpha, stream)
+        else:
+            scal = () if kind == _K_BMM_S32 else (alpha,)
+            rc = _BMM_CTYPES[kind](a.data_ptr(), b.data_ptr(), out.data_ptr(), batch, M, N, K, *scal, stream or None)
+    finally:
+        if switch:
+            torch.cuda.set_device(prev)
+    if rc:
+        _status(op, rc)
     return out
 
 
 def bmm_s8t_s8n_f32t(A, B, alpha):
     """fp32 [B,M,N] = alpha * (A[B,M,K] . B[B,N,K]^T)  (upstream bmm.cu:10-108)."""
-    return _bmm("bmm_s8t_s8n_f32t", _lib.ti_bmm_s8t_s8n_f32t, A, B, torch.float32, (float(alpha),))
+    return _bmm("bmm_s8t_s8n_f32t", _K_BMM_F32, A, B, _F32, float(alpha))
 
 
 def bmm_s8t_s8n_s8t(A, B, alpha):
     """int8 [B,M,N] = sat_s8(round(alpha * (A . B^T)))  (upstream bmm.cu:110-208)."""
-    return _bmm("bmm_s8t_s8n_s8t", _lib.ti_bmm_s8t_s8n_s8t, A, B, torch.int8, (float(alpha),))
+    return _bmm("bmm_s8t_s8n_s8t", _K_BMM_S8, A, B, _I8, float(alpha))
 
 
 def bmm_s8t_s8n_s32t(A, B):
     """int32 [B,M,N] = A . B^T  (upstream bmm.cu:210-295)."""
-    return _bmm("bmm_s8t_s8n_s32t", _lib.ti_bmm_s8t_s8n_s32t, A, B, torch.int32, ())
+    return _bmm("bmm_s8t_s8n_s32t", _K_BMM_S32, A, B, _I32, 1.0)
 
 
 def dq_add_layernorm_q(input, input_scale, residual_input, gamma, beta, epsilon):
@@ -203,25 +267,37 @@ def dq_add_layernorm_q(input, input_scale, residual_input, gamma, beta, epsilon)
     ln_output = int8(round(clamp(layer_norm(residual_output) * gamma + beta, -128, 127))).
     """
     op = "dq_add_layernorm_q"
-    _check(op, "input", input, torch.int32, None)
+    _check(op, "input", input, _I32, None)
     dev = input.device
     if input.dim() < 1:
         _fail(op, "input must have at least one dimension")
-    _check(op, "residual_input", residual_input, torch.float32, None, dev)
+    _check(op, "residual_input", residual_input, _F32, None, dev)
     if residual_input.shape != input.shape:
         _fail(op, f"input is {tuple(input.shape)} but residual_input is {tuple(residual_input.shape)}")
     H = input.shape[-1]
     gamma = gamma.detach() if isinstance(gamma, torch.Tensor) else gamma
     beta = beta.detach() if isinstance(beta, torch.Tensor) else beta
-    _check(op, "gamma", gamma, torch.float32, 1, dev)
-    _check(op, "beta", beta, torch.float32, 1, dev)
+    _check(op, "gamma", gamma, _F32, 1, dev)
+    _check(op, "beta", beta, _F32, 1, dev)
     if gamma.numel() != H or beta.numel() != H:
         _fail(op, f"gamma/beta must have {H} elements, got {gamma.numel()} and {beta.numel()}")
     r_out = torch.empty_like(residual_input)
-    q_out = torch.empty(input.shape, dtype=torch.int8, device=dev)
+    q_out = _empty(input.shape, dtype=_I8, device=dev)
     if input.numel() == 0:
         return r_out, q_out
-    _call(op, _lib.ti_dq_add_layernorm_q, dev, input.data_ptr(), float(input_scale), residual_input.data_ptr(),
-          gamma.data_ptr(), beta.data_ptr(), float(epsilon), r_out.data_ptr(), q_out.data_ptr(),
-          input.numel() // H, H, _stream(dev))
+    idx = dev.index
+    switch = idx != _current_device()
+    if switch:
+        prev = _current_device()
+        torch.cuda.set_device(idx)
+    try:
+        stream = _raw_stream(idx)
+        args = (input.data_ptr(), float(input_scale), residual_input.data_ptr(), gamma.data_ptr(), beta.data_ptr(),
+                float(epsilon), r_out.data_ptr(), q_out.data_ptr(), input.numel() // H, H)
+        rc = _fast.ln_q(*args, stream) if _fast is not None else _lib.ti_dq_add_layernorm_q(*args, stream or None)
+    finally:
+        if switch:
+            torch.cuda.set_device(prev)
+    if rc:
+        _status(op, rc)
     return r_out, q_out
