@@ -112,6 +112,24 @@ int ti_dq_add_layernorm_q(const int32_t* input, float input_scale, const float* 
                           const float* gamma, const float* beta, float eps,
                           float* r_out, int8_t* q_out, int64_t rows, int64_t H, void* stream);
 
+/* ---- fused element-wise chains of the OPT blocks (no counterpart in the reference's native
+ * module: upstream runs these as sequences of torch ops) ---- */
+
+/* x != NULL: residual[row,i] += x[row,i] (in place), then
+ *            q_out = s8(clamp(rint(LN(residual[row,:])[i] * gamma[i] + beta[i]), -128, 127));
+ * x == NULL: the same without the add (residual is only read).
+ * Replaces `residual.add_(h); LayerNormQ(residual)` (torch_int/models/opt.py:281-283) and
+ * LayerNormQ.forward on fp32 input (torch_int/nn/fused.py:13-18). */
+int ti_add_layernorm_q(const float* x, float* residual, const float* gamma, const float* beta, float eps,
+                       int8_t* q_out, int64_t rows, int64_t H, void* stream);
+
+/* probs[b*heads+h, t, s] = s8(rint(127 * softmax_s(max(scores[b*heads+h,t,s] + mask[b,0,t,s], -FLT_MAX))));
+ * scores [batch*heads, T, S] fp32, mask [batch, 1, T, S] fp32 or NULL.
+ * Replaces the mask add, clamp, softmax, *127, round and int8 cast between the two
+ * attention products (torch_int/models/opt.py:144-178). */
+int ti_attn_softmax_q(const float* scores, const float* mask, int8_t* probs, int64_t batch, int64_t heads,
+                      int64_t T, int64_t S, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -198,3 +198,40 @@ def dq_add_layernorm_q(inp, input_scale, residual, gamma, beta, eps):
     _load().orc_dq_add_layernorm_q(_p(inp), _f32(input_scale), _p(residual), _p(gamma), _p(beta),
                                    _f32(eps), _p(r), _p(q), _i64(rows), _i64(H))
     return r, q
+
+
+# ---- fused chains of the OPT blocks (ti_add_layernorm_q / ti_attn_softmax_q) ----
+
+def add_layernorm_q(x, residual, gamma, beta, eps):
+    """(updated residual, int8 LayerNorm of it); x may be None (no add; residual returned as is)."""
+    residual = _chk(residual, torch.float32, "residual")
+    gamma = _chk(gamma, torch.float32, "gamma")
+    beta = _chk(beta, torch.float32, "beta")
+    H = residual.shape[-1]
+    rows = residual.numel() // H if H else 0
+    q = torch.empty(residual.shape, dtype=torch.int8)
+    if x is None:
+        _load().orc_add_layernorm_q(None, _p(residual), _p(gamma), _p(beta), _f32(eps), None, _p(q),
+                                    _i64(rows), _i64(H))
+        return residual, q
+    x = _chk(x, torch.float32, "x")
+    assert x.shape == residual.shape
+    r = torch.empty_like(residual)
+    _load().orc_add_layernorm_q(_p(x), _p(residual), _p(gamma), _p(beta), _f32(eps), _p(r), _p(q), _i64(rows), _i64(H))
+    return r, q
+
+
+def attn_softmax_q(scores, mask, heads):
+    """int8 round(127 softmax(max(scores + mask, finfo.min))); scores [batch*heads, T, S], mask [batch,1,T,S] or None."""
+    scores = _chk(scores, torch.float32, "scores")
+    BH, T, S = scores.shape
+    batch = BH // heads
+    assert batch * heads == BH
+    out = torch.empty(scores.shape, dtype=torch.int8)
+    mp = None
+    if mask is not None:
+        mask = _chk(mask, torch.float32, "mask")
+        assert mask.shape == (batch, 1, T, S)
+        mp = _p(mask)
+    _load().orc_attn_softmax_q(_p(scores), mp, _p(out), _i64(batch), _i64(heads), _i64(T), _i64(S))
+    return out

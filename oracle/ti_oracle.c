@@ -35,6 +35,7 @@
 #include <math.h>
 #include <stdint.h>
 #include <stddef.h>
+#include <stdlib.h>
 #include <string.h>
 
 #ifdef _OPENMP
@@ -254,5 +255,101 @@ void orc_dq_add_layernorm_q(const int32_t* in, float scale, const float* res,
       float y = fmaf((r[i] - mu) * rstd, gamma[i], beta[i]);
       q[i] = sat_rne_s8(y);
     }
+  }
+}
+
+/* ------------------------------------------- fused chains of the OPT blocks */
+
+/* residual.add_(x) followed by LayerNormQ (torch_int/models/opt.py:281-283 and
+ * torch_int/nn/fused.py:13-18): r = res + x (x may be NULL: r = res), the same
+ * fixed-tree LayerNorm as above, q = clamp(rint(y), -128, 127).  `r_out` may be
+ * NULL when x is NULL. */
+void orc_add_layernorm_q(const float* x, const float* res, const float* gamma, const float* beta, float eps,
+                         float* r_out, int8_t* q_out, int64_t rows, int64_t H) {
+#pragma omp parallel for schedule(static)
+  for (int64_t row = 0; row < rows; ++row) {
+    float* r = (float*)malloc(sizeof(float) * (size_t)(H > 0 ? H : 1));
+    int8_t* q = q_out + row * H;
+    for (int64_t i = 0; i < H; ++i) r[i] = x ? res[row * H + i] + x[row * H + i] : res[row * H + i];
+    float fH = (float)H;
+    float mu = tree_sum(r, H, 0, 0.0f) / fH;
+    float var = tree_sum(r, H, 1, mu) / fH;
+    float rstd = 1.0f / sqrtf(var + eps);
+    for (int64_t i = 0; i < H; ++i) q[i] = sat_rne_s8(fmaf((r[i] - mu) * rstd, gamma[i], beta[i]));
+    if (r_out)
+      for (int64_t i = 0; i < H; ++i) r_out[row * H + i] = r[i];
+    free(r);
+  }
+}
+
+/* e^x for x <= 0 as a fixed sequence of fp32 operations (Cody-Waite reduction, degree-6
+ * Taylor polynomial in Horner form with fma, exponent-field scaling); ~1 ulp. */
+static float exp_nonpos(float x) {
+  if (!(x > -87.0f)) return 0.0f;
+  float n = rintf(x * 1.44269504088896341f);
+  float r = fmaf(n, -0.693145751953125f, x);
+  r = fmaf(n, -1.42860682030941723e-6f, r);
+  float p = 1.0f / 720.0f;
+  p = fmaf(p, r, 1.0f / 120.0f);
+  p = fmaf(p, r, 1.0f / 24.0f);
+  p = fmaf(p, r, 1.0f / 6.0f);
+  p = fmaf(p, r, 0.5f);
+  p = fmaf(p, r, 1.0f);
+  p = fmaf(p, r, 1.0f);
+  union { int32_t i; float f; } u;
+  u.i = ((int32_t)n + 127) << 23;
+  return p * u.f;
+}
+
+/* The chain between the two attention products (torch_int/models/opt.py:144-178):
+ * s = max(scores + mask, -FLT_MAX); p = softmax(s) over the last dim; probs = int8(rint(127 p)).
+ * scores [batch*heads, T, S], mask [batch, 1, T, S] or NULL.  Reduction order: chunk c
+ * (elements 4c..4c+3) belongs to lane c mod 64, a lane visits its elements in ascending order,
+ * lanes combine with a xor butterfly (offsets 32..1). */
+void orc_attn_softmax_q(const float* scores, const float* mask, int8_t* probs, int64_t batch, int64_t heads,
+                        int64_t T, int64_t S) {
+  const float lowest = -3.402823466e+38f;
+  int64_t rows = batch * heads * T;
+#pragma omp parallel for schedule(static)
+  for (int64_t row = 0; row < rows; ++row) {
+    const float* src = scores + row * S;
+    const float* msk = NULL;
+    if (mask) {
+      int64_t bh = row / T, t = row % T;
+      msk = mask + ((bh / heads) * T + t) * S;
+    }
+    float* v = (float*)malloc(sizeof(float) * (size_t)(S > 0 ? S : 1));
+    float lane_m[64], lane_s[64];
+    for (int l = 0; l < 64; ++l) { lane_m[l] = lowest; lane_s[l] = 0.0f; }
+    int64_t nchunks = (S + 3) / 4;
+    for (int64_t c = 0; c < nchunks; ++c)
+      for (int j = 0; j < 4; ++j) {
+        int64_t i = c * 4 + j;
+        if (i >= S) break;
+        float x = src[i];
+        if (msk) x = x + msk[i];
+        x = x > lowest ? x : lowest;
+        v[i] = x;
+        int l = (int)(c % 64);
+        lane_m[l] = lane_m[l] > x ? lane_m[l] : x;
+      }
+    float m = lowest;
+    for (int l = 0; l < 64; ++l) m = m > lane_m[l] ? m : lane_m[l];  /* max is order-independent */
+    for (int64_t c = 0; c < nchunks; ++c)
+      for (int j = 0; j < 4; ++j) {
+        int64_t i = c * 4 + j;
+        if (i >= S) break;
+        v[i] = exp_nonpos(v[i] - m);
+        lane_s[c % 64] = lane_s[c % 64] + v[i];
+      }
+    float cur[64], nxt[64];
+    memcpy(cur, lane_s, sizeof(cur));
+    for (int off = 32; off >= 1; off >>= 1) {
+      for (int l = 0; l < 64; ++l) nxt[l] = cur[l] + cur[l ^ off];
+      memcpy(cur, nxt, sizeof(cur));
+    }
+    float s = cur[0];
+    for (int64_t i = 0; i < S; ++i) probs[row * S + i] = (int8_t)(int)rintf((v[i] / s) * 127.0f);
+    free(v);
   }
 }

@@ -104,6 +104,38 @@ def test_linear_large_tiles(variant):
         _linear_case(C, variant, M, N, K, seed=7)
 
 
+@pytest.mark.parametrize("variant", VARIANTS)
+def test_linear_split_k_and_decode_shapes(variant):
+    # few output tiles and a long K: the K loop is split over workgroups (with and without the
+    # scratch workspace the Python wrapper provides); M <= 16 with K % 1024 == 0: streaming kernel
+    import torch_int._CUDA as C
+    for (M, N, K) in [(128, 640, 4096), (100, 520, 2048), (512, 1280, 5120), (40, 256, 8192),
+                      (1, 4096, 2048), (4, 4112, 1024), (16, 5120, 3072), (9, 4100, 5120)]:
+        _say(f"linear-splitk/decode {variant} M={M} N={N} K={K}")
+        _linear_case(C, variant, M, N, K, seed=21)
+
+
+def test_split_k_matches_unsplit_through_the_c_abi():
+    # same call with and without a workspace must give identical bytes
+    import torch_int._CUDA as C
+    g = torch.Generator().manual_seed(3)
+    M, N, K = 128, 640, 4096
+    x, w, b = _s8(g, M, K).to(DEV), _s8(g, N, K).to(DEV), _s8(g, N).to(DEV)
+    need = C._lib.ti_linear_workspace_bytes(M, N, K)
+    assert need > 0
+    outs = []
+    for ws_bytes in (0, need):
+        ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=DEV)
+        out = torch.empty((M, N), dtype=torch.int8, device=DEV)
+        rc = C._lib.ti_linear_a8_w8_b8_o8(x.data_ptr(), w.data_ptr(), b.data_ptr(), out.data_ptr(), M, N, K,
+                                          0.002, 0.01, ws.data_ptr() if ws_bytes else None, ws_bytes,
+                                          torch.cuda.current_stream().cuda_stream)
+        assert rc == 0
+        outs.append(out.cpu())
+    assert torch.equal(outs[0], outs[1])
+    assert torch.equal(outs[0], orc.linear_a8_w8_b8_o8(x.cpu(), w.cpu(), b.cpu(), 0.002, 0.01))
+
+
 def test_linear_opt125m_config():
     # BASELINE config 1: x [4,512,768], W [768,768], bias [768], alpha 1e-3, beta 1e-2, seed 0
     import torch_int._CUDA as C
@@ -297,6 +329,59 @@ def test_ln_q_full_size_and_in_place():
                                       torch.cuda.current_stream().cuda_stream)
     assert rc == 0
     assert torch.equal(d_res.cpu(), r_ref) and torch.equal(q.cpu(), q_ref)
+
+
+# ------------------------------------------------------------------ fused chains of the OPT blocks
+
+def test_fused_add_layernorm_q():
+    import torch_int._hip_ext as X
+    for i, shape in enumerate([(7, 768), (4, 6, 5120), (3, 9216), (5, 1023), (2, 20000), (3, 1)]):
+        _say(f"add_layernorm_q shape={shape}")
+        g = torch.Generator().manual_seed(400 + i)
+        H = shape[-1]
+        x, res = torch.randn(shape, generator=g), torch.randn(shape, generator=g) * 3
+        gamma = (1 + 0.02 * torch.randn(H, generator=g)) * 25
+        beta = 0.5 * torch.randn(H, generator=g)
+        r_ref, q_ref = orc.add_layernorm_q(x, res, gamma, beta, 1e-5)
+        d_res = res.to(DEV)
+        q = X.add_layernorm_q(x.to(DEV), d_res, gamma.to(DEV), beta.to(DEV), 1e-5)
+        assert torch.equal(d_res.cpu(), r_ref) and torch.equal(r_ref, res + x)  # residual updated in place
+        assert (q.cpu() != q_ref).sum().item() == 0
+        _, q_ref2 = orc.add_layernorm_q(None, res, gamma, beta, 1e-5)
+        d_res = res.to(DEV)
+        q2 = X.add_layernorm_q(None, d_res, gamma.to(DEV), beta.to(DEV), 1e-5)
+        assert torch.equal(d_res.cpu(), res) and (q2.cpu() != q_ref2).sum().item() == 0
+        # upstream chain (nn/fused.py:13-18) on the GPU: one LSB, rarely
+        y = torch.nn.functional.layer_norm(res.to(DEV), (H,), gamma.to(DEV), beta.to(DEV), 1e-5)
+        q_t = y.round().clamp(-128, 127).to(torch.int8)
+        assert (q2.int() - q_t.int()).abs().max().item() <= 1
+        assert (q2 != q_t).float().mean().item() <= 0.01 + 1.0 / q2.numel()
+
+
+def test_fused_attn_softmax_q():
+    import torch_int._hip_ext as X
+    neg = torch.finfo(torch.float32).min
+    for i, (B, H, T, S) in enumerate([(2, 4, 16, 16), (1, 3, 5, 513), (2, 2, 33, 100), (1, 2, 1, 2049),
+                                      (1, 1, 4, 4100), (4, 40, 64, 512)]):
+        _say(f"attn_softmax_q B={B} H={H} T={T} S={S}")
+        g = torch.Generator().manual_seed(500 + i)
+        scores = torch.randn(B * H, T, S, generator=g) * 6
+        mask = torch.zeros(B, 1, T, S)
+        mask.masked_fill_(torch.arange(S)[None, :] > torch.arange(S - T, S)[:, None], neg)  # causal
+        mask[0, 0, :, : S // 7] = neg                                                       # padding
+        for m in (mask, None):
+            ref = orc.attn_softmax_q(scores, m, H)
+            out = X.attn_softmax_q(scores.to(DEV), m.to(DEV) if m is not None else None, H)
+            assert out.dtype == torch.int8 and out.shape == scores.shape
+            assert (out.cpu() != ref).sum().item() == 0
+            # upstream chain (models/opt.py:144-178) on the GPU
+            s = scores.to(DEV).view(B, H, T, S)
+            if m is not None:
+                s = torch.clamp_min(s + m.to(DEV), neg)
+            q_t = (torch.softmax(s.view(B * H, T, S), -1) * 127).round().to(torch.int8)
+            assert (out.int() - q_t.int()).abs().max().item() <= 1
+            assert (out != q_t).float().mean().item() <= 1e-3 + 1.0 / out.numel()
+            assert int(out.min()) >= 0
 
 
 def test_runs_are_deterministic():

@@ -98,8 +98,12 @@ def _capture(layer):
     mods = {"ln1": layer.self_attn_layer_norm, "q": a.q_proj, "k": a.k_proj, "v": a.v_proj, "qk": a.qk_bmm,
             "pv": a.pv_bmm, "out": a.out_proj, "ln2": layer.final_layer_norm, "fc1": layer.fc1, "fc2": layer.fc2}
     for name, m in mods.items():
+        def pre(mod, inp, name=name):
+            rec[name + "_in"] = tuple(t.detach().clone() for t in inp)  # before any in-place update
+
         def hook(mod, inp, out, name=name):
             rec[name] = (tuple(t.detach().clone() for t in inp), out.detach().clone())
+        handles.append(m.register_forward_pre_hook(pre))
         handles.append(m.register_forward_hook(hook))
     return rec, handles
 
@@ -156,7 +160,7 @@ def test_decoder_layer_opt13b_shape():
     # fp32 library pieces: LayerNormQ (int8 within one LSB) and softmax -> int8 probabilities
     _say("  check layer norms and softmax")
     for name, ln in (("ln1", layer.self_attn_layer_norm), ("ln2", layer.final_layer_norm)):
-        x, y = rec[name][0][0].cpu(), rec[name][1].cpu()
+        x, y = rec[name][0][0].cpu(), rec[name][1].cpu()  # post-hook input: residual after the in-place add
         ref = ln(x)
         assert (y.int() - ref.int()).abs().max() <= 1 and (y != ref).float().mean() < 1e-3, name
     probs_gpu = p_in[heads].float() / 127
@@ -165,7 +169,8 @@ def test_decoder_layer_opt13b_shape():
     assert (probs_gpu.cpu() - probs_cpu).abs().max() <= 0.5 / 127 + 1e-3
     # residual algebra: out = hidden + attn_out + fc2_out, in that order, in fp32
     r1 = hidden.to(DEV) + rec["out"][1]
-    assert torch.equal(rec["ln2"][0][0], r1)
+    assert torch.equal(rec["ln2_in"][0], hidden.to(DEV))  # the layer norm receives the residual ...
+    assert torch.equal(rec["ln2"][0][0], r1)              # ... and has added the attention output in place
     assert torch.equal(out[0], r1 + rec["fc2"][1])
 
 

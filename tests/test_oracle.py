@@ -268,3 +268,47 @@ def test_ln_q_invariants():
     r_all, q_all = orc.dq_add_layernorm_q(inp, 0.01, res, gamma, beta * 0, 1e-5)
     r_one, q_one = orc.dq_add_layernorm_q(inp[4:5], 0.01, res[4:5], gamma, beta * 0, 1e-5)
     assert torch.equal(r_all[4:5], r_one) and torch.equal(q_all[4:5], q_one)
+
+
+# ------------------------------------------------------------------ fused chains of the OPT blocks
+
+def test_add_layernorm_q_against_torch():
+    # upstream models/opt.py:281-283 + nn/fused.py:13-18, restated with torch ops
+    g = torch.Generator().manual_seed(11)
+    for shape in [(6, 768), (2, 5120), (3, 1023), (4, 1)]:
+        H = shape[-1]
+        x, res = torch.randn(shape, generator=g), torch.randn(shape, generator=g) * 2
+        gamma = (1 + 0.02 * torch.randn(H, generator=g)) * 30
+        beta = torch.randn(H, generator=g)
+        r, q = orc.add_layernorm_q(x, res, gamma, beta, 1e-5)
+        assert torch.equal(r, res + x)
+        ref = torch.nn.functional.layer_norm(res + x, (H,), gamma, beta, 1e-5).round().clamp(-128, 127).to(torch.int8)
+        assert (q.int() - ref.int()).abs().max().item() <= 1
+        assert (q != ref).float().mean().item() <= 0.01 + 1.0 / q.numel()
+        r0, q0 = orc.add_layernorm_q(None, res + x, gamma, beta, 1e-5)
+        assert torch.equal(q0, q)  # adding first or passing the sum is the same thing
+
+
+def test_attn_softmax_q_against_torch():
+    # upstream models/opt.py:144-178, restated with torch ops
+    neg = torch.finfo(torch.float32).min
+    g = torch.Generator().manual_seed(12)
+    for (B, H, T, S) in [(2, 3, 8, 8), (1, 2, 5, 131), (2, 2, 16, 512), (1, 1, 3, 1)]:
+        scores = torch.randn(B * H, T, S, generator=g) * 8
+        mask = torch.zeros(B, 1, T, S)
+        mask.masked_fill_(torch.arange(S)[None, :] > torch.arange(S - T, S)[:, None] + (S < T) * T, neg)
+        for m in (mask, None):
+            q = orc.attn_softmax_q(scores, m, H)
+            s = scores.view(B, H, T, S)
+            if m is not None:
+                s = torch.clamp_min(s + m, neg)
+            p = torch.softmax(s.double(), -1)  # fp64 route
+            ref = (p * 127).round().to(torch.int8).view(B * H, T, S)
+            assert (q.int() - ref.int()).abs().max().item() <= 1
+            assert (q != ref).float().mean().item() <= 1e-3 + 1.0 / q.numel()
+            assert int(q.min()) >= 0 and int(q.max()) <= 127
+            # every row sums to 127 up to rounding of its entries
+            assert (q.int().sum(-1) - 127).abs().max().item() <= S // 2 + 1
+    # a fully masked row degenerates to the uniform distribution, like softmax of equal inputs
+    q = orc.attn_softmax_q(torch.randn(1, 1, 8, generator=g), torch.full((1, 1, 1, 8), neg), 1)
+    assert q.tolist() == [[[16] * 8]]  # round(127 / 8) = 16

@@ -59,6 +59,8 @@ static int run_gemm(const char* op, int kind, const void* a, const void* b, cons
   p.N = (int)N;
   p.K = (int)K;
   p.batch = (int)batch;
+  p.lda = (int)K;
+  p.ldb = (int)K;
   p.strideA = M * K;
   p.strideB = N * K;
   p.strideC = M * N;
@@ -162,6 +164,36 @@ int ti_dq_add_layernorm_q(const int32_t* input, float input_scale, const float* 
   if (int rc = check_ptr(op, "q_out", q_out, 1, nonempty)) return rc;
   return launch_dq_add_layernorm_q(input, input_scale, residual, gamma, beta, eps, r_out, q_out, rows, H,
                                    static_cast<hipStream_t>(stream));
+}
+
+int ti_add_layernorm_q(const float* x, float* residual, const float* gamma, const float* beta, float eps,
+                       int8_t* q_out, int64_t rows, int64_t H, void* stream) {
+  g_err[0] = 0;
+  const char* op = "add_layernorm_q";
+  if (rows < 0 || H < 0 || rows > 0x7fffffffLL || H > 0x7fffffffLL)
+    return fail(TI_ERR_INVALID_ARG, "%s: rows and H must be in [0, 2^31) (rows=%lld H=%lld)", op, (long long)rows,
+                (long long)H);
+  const bool nonempty = rows > 0 && H > 0;
+  if (int rc = check_ptr(op, "x", x, 4, nonempty && x != nullptr)) return rc;
+  if (int rc = check_ptr(op, "residual", residual, 4, nonempty)) return rc;
+  if (int rc = check_ptr(op, "gamma", gamma, 4, nonempty)) return rc;
+  if (int rc = check_ptr(op, "beta", beta, 4, nonempty)) return rc;
+  if (int rc = check_ptr(op, "q_out", q_out, 1, nonempty)) return rc;
+  return launch_add_layernorm_q(x, residual, gamma, beta, eps, q_out, rows, H, static_cast<hipStream_t>(stream));
+}
+
+int ti_attn_softmax_q(const float* scores, const float* mask, int8_t* probs, int64_t batch, int64_t heads, int64_t T,
+                      int64_t S, void* stream) {
+  g_err[0] = 0;
+  const char* op = "attn_softmax_q";
+  if (batch < 0 || heads < 0 || T < 0 || S < 0 || T > 0x7fffffffLL || S > 0x7fffffffLL || heads > 0x7fffffffLL ||
+      batch > 0x7fffffffLL)
+    return fail(TI_ERR_INVALID_ARG, "%s: sizes must be in [0, 2^31)", op);
+  const bool nonempty = batch > 0 && heads > 0 && T > 0 && S > 0;
+  if (int rc = check_ptr(op, "scores", scores, 4, nonempty)) return rc;
+  if (int rc = check_ptr(op, "mask", mask, 4, nonempty && mask != nullptr)) return rc;
+  if (int rc = check_ptr(op, "probs", probs, 1, nonempty)) return rc;
+  return launch_attn_softmax_q(scores, mask, probs, batch, heads, T, S, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

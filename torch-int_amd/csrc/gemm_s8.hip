@@ -376,14 +376,14 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe_kernel(GemmParams p, int
       if (slab * 16 < BM) {
         const int chunk = pos ^ ((prow >> 2) & 3);
         const int gr = m0 + prow < M ? m0 + prow : M - 1;  // edge rows re-read the last row; never stored
-        src[j] = (const TI_GLOBAL_AS int8_t*)(A + (size_t)gr * K + chunk * 16);
+        src[j] = (const TI_GLOBAL_AS int8_t*)(A + (size_t)gr * p.lda + chunk * 16);
       } else {
         const int br = prow - BM;
         const int chunk = pos ^ ((br >> 2) & 3);
         int lr = br;
         if (SWAP) lr = (br & ~31) | ((br & 4) << 2) | ((br & 24) >> 1) | (br & 3);  // MFMA row 8q+4h+j -> 16h+4q+j
         const int gr = n0 + lr < N ? n0 + lr : N - 1;
-        src[j] = (const TI_GLOBAL_AS int8_t*)(B + (size_t)gr * K + chunk * 16);
+        src[j] = (const TI_GLOBAL_AS int8_t*)(B + (size_t)gr * p.ldb + chunk * 16);
       }
     }
   };
@@ -853,8 +853,86 @@ static int launch_pipe(const GemmParams& p, hipStream_t stream) {
   return TI_OK;
 }
 
+// ---------------------------------------------------------------------------
+// Split-K: when a problem has too few output tiles to fill the chip, K is cut
+// into `splits` slices that run as the batches of one launch of the pipelined
+// kernel (raw int32 output into a workspace [splits][M][N]); this kernel then
+// adds the slices and applies the epilogue.  Integer partial sums make the
+// result independent of the split.
 template <int KIND>
-static int launch_kind(const GemmParams& p, hipStream_t stream) {
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmParams p, const int* __restrict__ ws, int splits) {
+  using E = Epi<KIND>;
+  using Out = typename E::Out;
+  using BiasT = typename E::Bias;
+  const long long total = (long long)p.M * p.N;
+  const long long i0 = ((long long)blockIdx.x * 256 + threadIdx.x) * 4;
+  if (i0 >= total) return;
+  const BiasT* bias = reinterpret_cast<const BiasT*>(p.bias);
+  Out* C = reinterpret_cast<Out*>(p.C);
+  if ((p.N & 3) == 0) {  // four consecutive columns of one row
+    v4i acc = *reinterpret_cast<const v4i*>(ws + i0);
+    for (int s = 1; s < splits; ++s) acc += *reinterpret_cast<const v4i*>(ws + (long long)s * total + i0);
+    const int n = (int)(i0 % p.N);
+    Out o[4];
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      BiasT bv = BiasT(0);
+      if (E::kHasBias) bv = bias[n + v];
+      o[v] = E::apply(acc[v], E::bias_term(bv, p.beta), p.alpha);
+    }
+    if (sizeof(Out) == 4) {
+      using W = typename std::conditional<sizeof(Out) == 4, Out, int>::type;
+      v4i w4 = {__builtin_bit_cast(int, (W)o[0]), __builtin_bit_cast(int, (W)o[1]), __builtin_bit_cast(int, (W)o[2]),
+                __builtin_bit_cast(int, (W)o[3])};
+      *reinterpret_cast<v4i*>(C + i0) = w4;
+    } else {
+      *reinterpret_cast<unsigned*>(C + i0) = (unsigned)(unsigned char)o[0] | ((unsigned)(unsigned char)o[1] << 8) |
+                                             ((unsigned)(unsigned char)o[2] << 16) |
+                                             ((unsigned)(unsigned char)o[3] << 24);
+    }
+  } else {
+    for (int v = 0; v < 4 && i0 + v < total; ++v) {
+      int acc = 0;
+      for (int s = 0; s < splits; ++s) acc += ws[(long long)s * total + i0 + v];
+      BiasT bv = BiasT(0);
+      if (E::kHasBias) bv = bias[(i0 + v) % p.N];
+      C[i0 + v] = E::apply(acc, E::bias_term(bv, p.beta), p.alpha);
+    }
+  }
+}
+
+// Number of K slices for an (M,N,K) linear on this chip; 1 = do not split.  A small cost
+// model: chip time of the GEMM at the utilisation the tile count allows, plus the time
+// to write and re-read the int32 partial tiles.
+static int choose_splits(long long M, long long N, long long K) {
+  if (M <= 16 || M > 1024 || K % PBK != 0 || K < 1024) return 1;
+  const double slots = num_cus();  // one 128x128 workgroup per CU already gets most of a CU's rate
+  const double tiles = (double)((M + 127) / 128) * (double)((N + 127) / 128);
+  const double ops = 2.0 * M * N * K, bytes = (double)K * (M + N);
+  const double t0 = ops / 2.0e15 > bytes / 5.0e12 ? ops / 2.0e15 : bytes / 5.0e12;
+  const long long steps = K / PBK;
+  int best = 1;
+  double best_t = 1e30;
+  for (int s = 1; s <= 16; ++s) {
+    if (steps % s != 0 || steps / s < 4) continue;
+    const double util = tiles * s / slots < 1.0 ? tiles * s / slots : 1.0;
+    double t = t0 / util;
+    if (s > 1) t += 2.0 * s * M * N * 4.0 / 4.0e12 + 3.0e-6;
+    if (t < best_t * 0.97) {  // prefer fewer slices unless the gain is clear
+      best_t = t;
+      best = s;
+    }
+  }
+  return best;
+}
+
+long long gemm_workspace_bytes(long long M, long long N, long long K) {
+  const int s = choose_splits(M, N, K);
+  return s > 1 ? (long long)s * M * N * 4 : 0;
+}
+
+template <int KIND>
+static int launch_kind(const GemmParams& p, void* workspace, long long workspace_bytes, hipStream_t stream) {
   using Out = typename Epi<KIND>::Out;
   const bool aligned = (p.K % 16 == 0) && ((reinterpret_cast<uintptr_t>(p.A) & 15) == 0) &&
                        ((reinterpret_cast<uintptr_t>(p.B) & 15) == 0) &&
@@ -908,6 +986,28 @@ static int launch_kind(const GemmParams& p, hipStream_t stream) {
     if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "gemm launch: %s", hipGetErrorString(e));
     return TI_OK;
   }
+  if (p.batch == 1 && p.lda == p.K && p.ldb == p.K) {
+    const int splits = choose_splits(p.M, p.N, p.K);
+    const long long need = (long long)splits * p.M * p.N * 4;
+    if (splits > 1 && workspace != nullptr && workspace_bytes >= need &&
+        (reinterpret_cast<uintptr_t>(workspace) & 15) == 0) {
+      GemmParams q = p;  // the K slices are the batches of one raw-int32 GEMM into the workspace
+      q.K = p.K / splits;
+      q.batch = splits;
+      q.strideA = q.K;
+      q.strideB = q.K;
+      q.strideC = (long long)p.M * p.N;
+      q.C = workspace;
+      q.bias = nullptr;
+      if (int rc = launch_pipe<PipeCfg<128, 128, 2, 2, 4, EPI_S32_RAW, false>>(q, stream)) return rc;
+      const long long quads = ((long long)p.M * p.N + 3) / 4;
+      hipLaunchKernelGGL(splitk_reduce_kernel<KIND>, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream, p,
+                         static_cast<const int*>(workspace), splits);
+      hipError_t e = hipGetLastError();
+      if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "split-K reduce launch: %s", hipGetErrorString(e));
+      return TI_OK;
+    }
+  }
   // 8-bit outputs take the orientation whose lanes own 16 consecutive columns.
   constexpr bool SWAP = sizeof(Out) == 1;
   const long long t256 = (long long)((p.M + 255) / 256) * ((p.N + 255) / 256) * p.batch;
@@ -921,19 +1021,17 @@ static int launch_kind(const GemmParams& p, hipStream_t stream) {
   return launch_tile<TileCfg<64, 64, 2, 2, KIND, SWAP>>(p, stream);
 }
 
-long long gemm_workspace_bytes(long long, long long, long long) { return 0; }
-
-int launch_gemm(int kind, const GemmParams& p, void*, long long, hipStream_t stream) {
+int launch_gemm(int kind, const GemmParams& p, void* ws, long long ws_bytes, hipStream_t stream) {
   if (p.M == 0 || p.N == 0 || p.batch == 0) return TI_OK;
   switch (kind) {
-    case EPI_S32_BIAS: return launch_kind<EPI_S32_BIAS>(p, stream);
-    case EPI_S32_SCALED: return launch_kind<EPI_S32_SCALED>(p, stream);
-    case EPI_F32_BIAS: return launch_kind<EPI_F32_BIAS>(p, stream);
-    case EPI_S8_BIAS: return launch_kind<EPI_S8_BIAS>(p, stream);
-    case EPI_S8_RELU: return launch_kind<EPI_S8_RELU>(p, stream);
-    case EPI_F32_SCALE: return launch_kind<EPI_F32_SCALE>(p, stream);
-    case EPI_S8_SCALE: return launch_kind<EPI_S8_SCALE>(p, stream);
-    case EPI_S32_RAW: return launch_kind<EPI_S32_RAW>(p, stream);
+    case EPI_S32_BIAS: return launch_kind<EPI_S32_BIAS>(p, ws, ws_bytes, stream);
+    case EPI_S32_SCALED: return launch_kind<EPI_S32_SCALED>(p, ws, ws_bytes, stream);
+    case EPI_F32_BIAS: return launch_kind<EPI_F32_BIAS>(p, ws, ws_bytes, stream);
+    case EPI_S8_BIAS: return launch_kind<EPI_S8_BIAS>(p, ws, ws_bytes, stream);
+    case EPI_S8_RELU: return launch_kind<EPI_S8_RELU>(p, ws, ws_bytes, stream);
+    case EPI_F32_SCALE: return launch_kind<EPI_F32_SCALE>(p, ws, ws_bytes, stream);
+    case EPI_S8_SCALE: return launch_kind<EPI_S8_SCALE>(p, ws, ws_bytes, stream);
+    case EPI_S32_RAW: return launch_kind<EPI_S32_RAW>(p, ws, ws_bytes, stream);
   }
   return fail(TI_ERR_INVALID_ARG, "unknown epilogue kind %d", kind);
 }

@@ -36,8 +36,13 @@ __device__ __forceinline__ int pack_s8x4(float y0, float y1, float y2, float y3)
   return (int)(b0 | (b1 << 8) | (b2 << 16) | (b3 << 24));
 }
 
+// What is normalised: MODE_DQ_ADD  r = res + scale * float(in)   (int32 in; dq_add_layernorm_q)
+//                     MODE_ADD     r = res + x                   (fp32 x passed through `in`)
+//                     MODE_PLAIN   r = x                         (fp32 x passed through `res`; r is not stored)
+enum LnMode : int { MODE_DQ_ADD = 0, MODE_ADD = 1, MODE_PLAIN = 2 };
+
 // H % 4 == 0, H <= NC * 1024, all row starts 16-byte aligned.
-template <int NC>
+template <int NC, int MODE>
 __global__ __launch_bounds__(256) void ln_q_rows_kernel(const int32_t* __restrict__ in, float scale,
                                                         const float* res,  // may alias r_out
                                                         const float* __restrict__ gamma,
@@ -58,13 +63,21 @@ __global__ __launch_bounds__(256) void ln_q_rows_kernel(const int32_t* __restric
   for (int i = 0; i < NC; ++i) {
     const int c = t + i * 256;
     if (c < nchunks) {
-      v4i x = in4[c];
       v4f a = res4[c];
       v4f v;
+      if (MODE == MODE_DQ_ADD) {
+        v4i x = in4[c];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) v[j] = __builtin_fmaf(scale, (float)x[j], a[j]);
+        for (int j = 0; j < 4; ++j) v[j] = __builtin_fmaf(scale, (float)x[j], a[j]);
+      } else if (MODE == MODE_ADD) {
+        v4f x = reinterpret_cast<const v4f*>(in4)[c];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] = a[j] + x[j];
+      } else {
+        v = a;
+      }
       r[i] = v;
-      rout4[c] = v;
+      if (MODE != MODE_PLAIN) rout4[c] = v;
 #pragma unroll
       for (int j = 0; j < 4; ++j) s = s + v[j];
     }
@@ -106,7 +119,8 @@ __global__ __launch_bounds__(256) void ln_q_rows_kernel(const int32_t* __restric
 __global__ __launch_bounds__(256) void ln_q_rows_generic_kernel(const int32_t* __restrict__ in, float scale,
                                                                 const float* res, const float* __restrict__ gamma,
                                                                 const float* __restrict__ beta, float eps,
-                                                                float* r_out, int8_t* __restrict__ q_out, int H) {
+                                                                float* r_out, int8_t* __restrict__ q_out, int H,
+                                                                int mode) {
   __shared__ float red[4];
   const long long row = blockIdx.x;
   const int t = threadIdx.x;
@@ -115,11 +129,17 @@ __global__ __launch_bounds__(256) void ln_q_rows_generic_kernel(const int32_t* _
   float* ro = r_out + row * H;
   int8_t* q = q_out + row * H;
   const int nchunks = (H + 3) >> 2;
+  const float* xf = reinterpret_cast<const float*>(x);
+  auto value = [&](int i) {
+    if (mode == MODE_DQ_ADD) return __builtin_fmaf(scale, (float)x[i], a[i]);
+    if (mode == MODE_ADD) return a[i] + xf[i];
+    return a[i];
+  };
   float s = 0.0f;
   for (int c = t; c < nchunks; c += 256)
     for (int j = 0; j < 4; ++j) {
       const int i = c * 4 + j;
-      if (i < H) s = s + __builtin_fmaf(scale, (float)x[i], a[i]);
+      if (i < H) s = s + value(i);
     }
   const float fH = (float)H;
   const float mu = block_sum_256(s, red) / fH;
@@ -128,7 +148,7 @@ __global__ __launch_bounds__(256) void ln_q_rows_generic_kernel(const int32_t* _
     for (int j = 0; j < 4; ++j) {
       const int i = c * 4 + j;
       if (i < H) {
-        float d = __builtin_fmaf(scale, (float)x[i], a[i]) - mu;
+        float d = value(i) - mu;
         float sq = d * d;
         s2 = s2 + sq;
       }
@@ -141,34 +161,45 @@ __global__ __launch_bounds__(256) void ln_q_rows_generic_kernel(const int32_t* _
     for (int j = 0; j < 4; ++j) {
       const int i = c * 4 + j;
       if (i < H) {
-        float v = __builtin_fmaf(scale, (float)x[i], a[i]);
+        float v = value(i);
         float y = __builtin_fmaf((v - mu) * rstd, gamma[i], beta[i]);
-        ro[i] = v;
+        if (mode != MODE_PLAIN) ro[i] = v;
         q[i] = (int8_t)rne_s8(y);
       }
     }
 }
 
 template <int NC>
-static void launch_rows(const int32_t* in, float scale, const float* res, const float* gamma, const float* beta,
-                        float eps, float* r_out, int8_t* q_out, long long rows, int H, hipStream_t stream) {
-  hipLaunchKernelGGL(ln_q_rows_kernel<NC>, dim3((unsigned)rows), dim3(256), 0, stream, in, scale, res, gamma,
-                     beta, eps, r_out, q_out, H);
+static void launch_rows(int mode, const int32_t* in, float scale, const float* res, const float* gamma,
+                        const float* beta, float eps, float* r_out, int8_t* q_out, long long rows, int H,
+                        hipStream_t stream) {
+  const dim3 grid((unsigned)rows), block(256);
+  if (mode == MODE_DQ_ADD)
+    hipLaunchKernelGGL((ln_q_rows_kernel<NC, MODE_DQ_ADD>), grid, block, 0, stream, in, scale, res, gamma, beta, eps,
+                       r_out, q_out, H);
+  else if (mode == MODE_ADD)
+    hipLaunchKernelGGL((ln_q_rows_kernel<NC, MODE_ADD>), grid, block, 0, stream, in, scale, res, gamma, beta, eps,
+                       r_out, q_out, H);
+  else
+    hipLaunchKernelGGL((ln_q_rows_kernel<NC, MODE_PLAIN>), grid, block, 0, stream, in, scale, res, gamma, beta, eps,
+                       r_out, q_out, H);
 }
 
-int launch_dq_add_layernorm_q(const int32_t* in, float scale, const float* res, const float* gamma,
-                              const float* beta, float eps, float* r_out, int8_t* q_out, long long rows,
-                              long long H, hipStream_t stream) {
+static int launch_ln_mode(int mode, const void* in, float scale, const float* res, const float* gamma,
+                          const float* beta, float eps, float* r_out, int8_t* q_out, long long rows, long long H,
+                          hipStream_t stream) {
   if (rows == 0 || H == 0) return TI_OK;
   auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
-  const bool fast = (H % 4 == 0) && H <= 16 * 1024 && al16(in) && al16(res) && al16(gamma) && al16(beta) &&
-                    al16(r_out) && ((reinterpret_cast<uintptr_t>(q_out) & 3) == 0);
+  const bool fast = (H % 4 == 0) && H <= 16 * 1024 && (mode == MODE_PLAIN || al16(in)) && al16(res) && al16(gamma) &&
+                    al16(beta) && (mode == MODE_PLAIN || al16(r_out)) &&
+                    ((reinterpret_cast<uintptr_t>(q_out) & 3) == 0);
   const int h = (int)H;
+  const int32_t* in32 = static_cast<const int32_t*>(in);
   if (fast) {
     const int nc = (int)((H + 1023) / 1024);
-#define TI_LN_CASE(n)                                                                     \
-  case n:                                                                                 \
-    launch_rows<n>(in, scale, res, gamma, beta, eps, r_out, q_out, rows, h, stream);      \
+#define TI_LN_CASE(n)                                                                              \
+  case n:                                                                                          \
+    launch_rows<n>(mode, in32, scale, res, gamma, beta, eps, r_out, q_out, rows, h, stream);       \
     break;
     switch (nc) {
       TI_LN_CASE(1) TI_LN_CASE(2) TI_LN_CASE(3) TI_LN_CASE(4) TI_LN_CASE(5) TI_LN_CASE(6) TI_LN_CASE(7)
@@ -177,12 +208,26 @@ int launch_dq_add_layernorm_q(const int32_t* in, float scale, const float* res, 
     }
 #undef TI_LN_CASE
   } else {
-    hipLaunchKernelGGL(ln_q_rows_generic_kernel, dim3((unsigned)rows), dim3(256), 0, stream, in, scale, res,
-                       gamma, beta, eps, r_out, q_out, h);
+    hipLaunchKernelGGL(ln_q_rows_generic_kernel, dim3((unsigned)rows), dim3(256), 0, stream, in32, scale, res, gamma,
+                       beta, eps, r_out, q_out, h, mode);
   }
   hipError_t e = hipGetLastError();
-  if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "dq_add_layernorm_q launch: %s", hipGetErrorString(e));
+  if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "layernorm_q launch: %s", hipGetErrorString(e));
   return TI_OK;
+}
+
+int launch_dq_add_layernorm_q(const int32_t* in, float scale, const float* res, const float* gamma,
+                              const float* beta, float eps, float* r_out, int8_t* q_out, long long rows,
+                              long long H, hipStream_t stream) {
+  return launch_ln_mode(MODE_DQ_ADD, in, scale, res, gamma, beta, eps, r_out, q_out, rows, H, stream);
+}
+
+// x == nullptr: q = LayerNormQ(residual); else residual += x (in place) and q = LayerNormQ(residual).
+int launch_add_layernorm_q(const float* x, float* residual, const float* gamma, const float* beta, float eps,
+                           int8_t* q_out, long long rows, long long H, hipStream_t stream) {
+  if (x == nullptr)
+    return launch_ln_mode(MODE_PLAIN, nullptr, 1.0f, residual, gamma, beta, eps, nullptr, q_out, rows, H, stream);
+  return launch_ln_mode(MODE_ADD, x, 1.0f, residual, gamma, beta, eps, residual, q_out, rows, H, stream);
 }
 
 }  // namespace ti

@@ -137,6 +137,7 @@ struct GemmParams {
   const void* bias;
   void* C;
   int M, N, K, batch;
+  int lda, ldb;                         // bytes between consecutive rows of A and B (>= K)
   long long strideA, strideB, strideC;  // elements between consecutive batches
   float alpha, beta;
 };
@@ -150,5 +151,12 @@ long long gemm_workspace_bytes(long long M, long long N, long long K);
 int launch_dq_add_layernorm_q(const int32_t* in, float scale, const float* res, const float* gamma,
                               const float* beta, float eps, float* r_out, int8_t* q_out,
                               long long rows, long long H, hipStream_t stream);
+
+int launch_add_layernorm_q(const float* x, float* residual, const float* gamma, const float* beta, float eps,
+                           int8_t* q_out, long long rows, long long H, hipStream_t stream);
+
+// softmax_q.hip
+int launch_attn_softmax_q(const float* scores, const float* mask, int8_t* out, long long batch, long long heads,
+                          long long T, long long S, hipStream_t stream);
 
 }  // namespace ti

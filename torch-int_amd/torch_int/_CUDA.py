@@ -87,7 +87,7 @@ def _load_fastcall():
 
 
 _fast = _load_fastcall()
-_workspaces = {}  # (device index, stream) -> zero-initialised uint8 tensor used as split-K scratch
+_workspaces = {}  # (device index, stream) -> uint8 tensor used as split-K scratch
 _raw_stream = torch._C._cuda_getCurrentRawStream
 _current_device = torch.cuda.current_device
 _empty = torch.empty
@@ -127,15 +127,18 @@ def _status(op, rc):
         _fail(op, f"{msg} (status {rc})")
 
 
+_ws_bytes = _lib.ti_linear_workspace_bytes
+
+
 def _workspace(dev_index, stream, nbytes):
-    """Split-K scratch: zero-filled once; the kernels leave it zeroed.  One per (device, stream) so
-    that calls on different streams never share it."""
+    """Split-K scratch (int32 partial tiles; contents need no initialisation).  One buffer per
+    (device, stream), grown on demand, so that calls on different streams never share it."""
     if nbytes <= 0:
         return 0, 0
     key = (dev_index, stream)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
-        ws = torch.zeros(int(nbytes), dtype=torch.uint8, device=torch.device("cuda", dev_index))
+        ws = torch.empty(int(nbytes), dtype=torch.uint8, device=torch.device("cuda", dev_index))
         _workspaces[key] = ws
     return ws.data_ptr(), ws.numel()
 
@@ -172,7 +175,8 @@ def _linear(op, kind, x, w, bias, bias_dtype, out_dtype, alpha, beta):
         torch.cuda.set_device(idx)
     try:
         stream = _raw_stream(idx)
-        ws_ptr, ws_bytes = 0, 0  # no kernel uses split-K scratch yet (ti_linear_workspace_bytes() == 0)
+        # split-K scratch is only ever wanted for mid-sized M (see choose_splits in csrc/gemm_s8.hip)
+        ws_ptr, ws_bytes = _workspace(idx, stream, _ws_bytes(M, N, K)) if 16 < M <= 1024 else (0, 0)
         if _fast is not None:
             rc = _fast.linear(kind, x.data_ptr(), w.data_ptr(), bias.data_ptr(), out.data_ptr(), M, N, K,
                               alpha, beta, ws_ptr, ws_bytes, stream)

@@ -1,0 +1,82 @@
+"""Fused element-wise kernels of the OPT blocks that upstream runs as chains of torch ops.
+
+These are *not* part of the reference's ``torch_int._CUDA`` surface; the modules in
+``torch_int.nn.fused`` and ``torch_int.models.opt`` call them when their input is an fp32
+tensor on a HIP device and fall back to the upstream torch-op chain otherwise.
+
+* :func:`add_layernorm_q` -- ``residual.add_(x)`` + ``LayerNormQ`` (upstream models/opt.py:281-283,
+  nn/fused.py:13-18) in one pass.
+* :func:`attn_softmax_q` -- mask add, clamp to finfo.min, softmax, ``*127``, round, int8 cast
+  (upstream models/opt.py:144-178) in one pass.
+"""
+import ctypes
+
+import torch
+
+from . import _CUDA
+
+_lib = _CUDA._lib
+_vp, _i64, _f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_float
+_lib.ti_add_layernorm_q.argtypes = [_vp, _vp, _vp, _vp, _f32, _vp, _i64, _i64, _vp]
+_lib.ti_add_layernorm_q.restype = ctypes.c_int
+_lib.ti_attn_softmax_q.argtypes = [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]
+_lib.ti_attn_softmax_q.restype = ctypes.c_int
+_raw_stream = torch._C._cuda_getCurrentRawStream
+
+
+def _ok(t, dtype):
+    return isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == dtype and t.is_contiguous()
+
+
+def can_fuse_layernorm(x, weight, bias):
+    """True when the fused kernel applies: fp32 contiguous HIP tensors, last dim = len(weight)."""
+    return (_ok(x, torch.float32) and _ok(weight, torch.float32) and _ok(bias, torch.float32)
+            and x.dim() >= 1 and x.shape[-1] == weight.numel() == bias.numel() and x.numel() > 0)
+
+
+def add_layernorm_q(x, residual, weight, bias, eps):
+    """``residual += x`` in place (skipped when ``x`` is None), returns int8
+    ``clamp(round(layer_norm(residual) * weight + bias), -128, 127)``."""
+    op = "add_layernorm_q"
+    if not can_fuse_layernorm(residual, weight, bias):
+        raise RuntimeError(f"torch_int._hip_ext.{op}: needs contiguous fp32 HIP tensors")
+    if x is not None and not (_ok(x, torch.float32) and x.shape == residual.shape and x.device == residual.device):
+        raise RuntimeError(f"torch_int._hip_ext.{op}: x must be a contiguous fp32 tensor shaped like residual")
+    dev = residual.device
+    H = residual.shape[-1]
+    q = torch.empty(residual.shape, dtype=torch.int8, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.ti_add_layernorm_q(x.data_ptr() if x is not None else None, residual.data_ptr(),
+                                     weight.data_ptr(), bias.data_ptr(), float(eps), q.data_ptr(),
+                                     residual.numel() // H, H, _raw_stream(dev.index) or None)
+    if rc:
+        raise RuntimeError(f"torch_int._hip_ext.{op}: {_lib.ti_last_error().decode()} (status {rc})")
+    return q
+
+
+def can_fuse_softmax(scores, mask, bsz, heads):
+    if not (_ok(scores, torch.float32) and scores.dim() == 3 and scores.shape[0] == bsz * heads and scores.numel() > 0):
+        return False
+    if mask is None:
+        return True
+    return (_ok(mask, torch.float32) and mask.device == scores.device
+            and tuple(mask.shape) == (bsz, 1, scores.shape[1], scores.shape[2]))
+
+
+def attn_softmax_q(scores, mask, heads):
+    """scores fp32 [bsz*heads, T, S], mask fp32 [bsz, 1, T, S] or None ->
+    int8 ``round(127 * softmax(max(scores + mask, finfo.min), dim=-1))``."""
+    op = "attn_softmax_q"
+    BH, T, S = scores.shape
+    bsz = BH // heads
+    if bsz * heads != BH or not can_fuse_softmax(scores, mask, bsz, heads):
+        raise RuntimeError(f"torch_int._hip_ext.{op}: needs contiguous fp32 HIP tensors, scores [bsz*heads,T,S], "
+                           f"mask [bsz,1,T,S]")
+    dev = scores.device
+    out = torch.empty((BH, T, S), dtype=torch.int8, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.ti_attn_softmax_q(scores.data_ptr(), mask.data_ptr() if mask is not None else None, out.data_ptr(),
+                                    bsz, heads, T, S, _raw_stream(dev.index) or None)
+    if rc:
+        raise RuntimeError(f"torch_int._hip_ext.{op}: {_lib.ti_last_error().decode()} (status {rc})")
+    return out

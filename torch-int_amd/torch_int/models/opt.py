@@ -14,6 +14,7 @@ from typing import List, Optional, Tuple
 import torch
 from torch import nn
 
+from .. import _hip_ext
 from ..nn.bmm import BMM_S8T_S8N_F32T, BMM_S8T_S8N_S8T
 from ..nn.fused import LayerNormQ
 from ..nn.linear import W8A8B8O8Linear, W8A8B8O8LinearReLU, W8A8BFP32OFP32Linear
@@ -95,27 +96,31 @@ class Int8OPTAttention(nn.Module):
         if scores.size() != (bsz * H, tgt_len, src_len):
             raise ValueError(f"Attention weights should be of size {(bsz * H, tgt_len, src_len)}, but is"
                              f" {scores.size()}")
-        if attention_mask is not None:
-            if attention_mask.size() != (bsz, 1, tgt_len, src_len):
-                raise ValueError(f"Attention mask should be of size {(bsz, 1, tgt_len, src_len)}, but is"
-                                 f" {attention_mask.size()}")
-            scores = scores.view(bsz, H, tgt_len, src_len) + attention_mask
-            scores = torch.clamp_min(scores, torch.finfo(scores.dtype).min)
-            scores = scores.view(bsz * H, tgt_len, src_len)
-        probs = nn.functional.softmax(scores, dim=-1)
-
-        if layer_head_mask is not None:
-            if layer_head_mask.size() != (H,):
-                raise ValueError(f"Head mask for a single layer should be of size {(H,)}, but is"
-                                 f" {layer_head_mask.size()}")
-            probs = (layer_head_mask.view(1, -1, 1, 1) * probs.view(bsz, H, tgt_len, src_len)
-                     ).view(bsz * H, tgt_len, src_len)
-        probs_out = probs.view(bsz, H, tgt_len, src_len) if output_attentions else None
-
-        # P.V with V transposed to [bsz*H, d, src]: (P V) = P . (V^T)^T.  The probabilities are
-        # scaled and rounded in place, so with output_attentions the returned view holds
-        # round(127 p), which is what upstream returns too (models/opt.py:166-178).
-        probs_q = probs.mul_(127).round_().to(torch.int8)
+        if attention_mask is not None and attention_mask.size() != (bsz, 1, tgt_len, src_len):
+            raise ValueError(f"Attention mask should be of size {(bsz, 1, tgt_len, src_len)}, but is"
+                             f" {attention_mask.size()}")
+        if layer_head_mask is not None and layer_head_mask.size() != (H,):
+            raise ValueError(f"Head mask for a single layer should be of size {(H,)}, but is"
+                             f" {layer_head_mask.size()}")
+        if layer_head_mask is None and _hip_ext.can_fuse_softmax(scores, attention_mask, bsz, H):
+            # mask add, clamp, softmax, *127, round and int8 cast in one kernel
+            probs_q = _hip_ext.attn_softmax_q(scores, attention_mask, H)
+            probs_out = probs_q.view(bsz, H, tgt_len, src_len).float() if output_attentions else None
+        else:
+            if attention_mask is not None:
+                scores = scores.view(bsz, H, tgt_len, src_len) + attention_mask
+                scores = torch.clamp_min(scores, torch.finfo(scores.dtype).min)
+                scores = scores.view(bsz * H, tgt_len, src_len)
+            probs = nn.functional.softmax(scores, dim=-1)
+            if layer_head_mask is not None:
+                probs = (layer_head_mask.view(1, -1, 1, 1) * probs.view(bsz, H, tgt_len, src_len)
+                         ).view(bsz * H, tgt_len, src_len)
+            probs_out = probs.view(bsz, H, tgt_len, src_len) if output_attentions else None
+            # The probabilities are scaled and rounded in place, so with output_attentions the
+            # returned view holds round(127 p), which is what upstream returns too
+            # (models/opt.py:166-178).
+            probs_q = probs.mul_(127).round_().to(torch.int8)
+        # P.V with V transposed to [bsz*H, d, src]: (P V) = P . (V^T)^T
         value_t = value.transpose(1, 2).contiguous()
         ctx = self.pv_bmm(probs_q, value_t)  # int8 [bsz*H, tgt, d]
         if ctx.size() != (bsz * H, tgt_len, d):
@@ -160,8 +165,7 @@ class Int8OPTDecoderLayer(nn.Module):
         x, attn_weights, present = self.self_attn(
             hidden_states=x, past_key_value=past_key_value, attention_mask=attention_mask,
             layer_head_mask=layer_head_mask, output_attentions=output_attentions)
-        residual.add_(x.to(residual.dtype))
-        x = self.final_layer_norm(residual)
+        x = self.final_layer_norm(residual, add=x)  # residual += x, then LayerNormQ
         x = self.fc2(self.fc1(x))
         residual.add_(x.to(residual.dtype))
         outputs = (residual,)

@@ -2,6 +2,7 @@
 import torch
 import torch.nn.functional as F
 
+from .. import _hip_ext
 from ..functional.fused import dq_add_layernorm_q_cpp
 
 
@@ -18,7 +19,15 @@ class LayerNormQ(_QuantLayerNormBase):
     """fp -> int8: LayerNorm in fp32, round half-even, clamp to [-128, 127].
     ``from_float`` folds the output scale into weight and bias."""
 
-    def forward(self, x):
+    def forward(self, x, add=None):
+        """int8 LayerNorm of ``x``.  With ``add`` given, ``x`` is first updated in place
+        (``x.add_(add)``, the residual update of the decoder layer) -- fused into the same
+        kernel when ``x`` is a contiguous fp32 HIP tensor."""
+        if _hip_ext.can_fuse_layernorm(x, self.weight, self.bias) and (
+                add is None or (add.dtype == x.dtype and add.shape == x.shape and add.is_contiguous())):
+            return _hip_ext.add_layernorm_q(add, x, self.weight, self.bias, self.eps)  # one pass, same maths
+        if add is not None:
+            x.add_(add.to(x.dtype))
         y = F.layer_norm(x.to(self.weight.dtype), x.shape[-1:], self.weight, self.bias, self.eps)
         return y.round().clamp(-128, 127).to(torch.int8)
 
