@@ -519,6 +519,257 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe_kernel(GemmParams p, int
   __builtin_amdgcn_s_waitcnt(0x0F70);  // the trailing filler copies must land before the LDS is released
 }
 
+// ---------------------------------------------------------------------------
+// Variant of the pipelined persistent kernel built from 16x16 blocks
+// (v_mfma_i32_16x16x64_i8: one instruction covers the whole 64-byte K step).
+// Its output tile can be any multiple of 16 per wave, which gives tile counts
+// that divide the chip evenly where 256x256 does not: OPT-13B widths are
+// multiples of 160, and 2048x5120 outputs make exactly 256 tiles of 256x160.
+//
+// Same LDS stage layout, swizzle, copy stream and barrier scheme as
+// gemm_pipe_kernel.  Differences: a wave copies (BM+BN)/NWAVES panel rows per
+// step, the last copy instruction with only part of its lanes enabled when
+// that is not a multiple of 16; fragments of step g+1 are read while step g
+// multiplies; the weight rows always feed the MFMA row operand, so a lane ends
+// with four consecutive output columns of one row per block (4-byte s8 or
+// 16-byte 32-bit stores).
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int STAGES_, int KIND_>
+struct Pipe16Cfg {
+  static constexpr int BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, KIND = KIND_, STAGES = STAGES_;
+  static constexpr int NWAVES = WAVES_M * WAVES_N;
+  static constexpr int NT = NWAVES * 64;
+  static constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
+  static constexpr int TM = WTM / 16, TN = WTN / 16;
+  static constexpr int STAGE_BYTES = (BM + BN) * PBK;
+  static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
+  static constexpr int RPW = (BM + BN) / NWAVES;  // panel rows a wave copies per step
+  static constexpr int TAIL_ROWS = RPW % 16;
+  static constexpr int COPIES = RPW / 16 + (TAIL_ROWS ? 1 : 0);
+  static_assert(WTM % 16 == 0 && WTN % 16 == 0, "wave tile must be made of 16x16 blocks");
+  static_assert((BM + BN) % NWAVES == 0 && RPW % 4 == 0, "a wave must copy whole groups of four rows");
+  static_assert(LDS_BYTES <= 160 * 1024 && STAGES >= 3, "LDS budget");
+};
+
+template <class Cfg>
+__global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe16_kernel(GemmParams p, int tiles_m, int tiles_n, int items) {
+  using E = Epi<Cfg::KIND>;
+  using Out = typename E::Out;
+  using BiasT = typename E::Bias;
+  constexpr int BM = Cfg::BM, BN = Cfg::BN, TM = Cfg::TM, TN = Cfg::TN, COPIES = Cfg::COPIES, S = Cfg::STAGES;
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave_m = wave / Cfg::WAVES_N, wave_n = wave % Cfg::WAVES_N;
+  const int M = p.M, N = p.N, K = p.K;
+  const int KT = K / PBK;
+  const int tiles = tiles_m * tiles_n;
+  const int first = blockIdx.x, stride = gridDim.x;
+  const int my_items = (items - first + stride - 1) / stride;
+  const int G = my_items * KT;
+
+  // ---- copy stream: copy j of this wave fills panel rows wave*RPW + 16j .. +15 of [A panel | B panel]
+  const TI_GLOBAL_AS int8_t* src[COPIES];
+  auto set_copy_item = [&](int item) {
+    const int b = item / tiles;
+    int tile_m, tile_n;
+    tile_of_workgroup(item - b * tiles, tiles_m, tiles_n, tile_m, tile_n);
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int8_t* A = p.A + (long long)b * p.strideA;
+    const int8_t* B = p.B + (long long)b * p.strideB;
+#pragma unroll
+    for (int j = 0; j < COPIES; ++j) {
+      int prow = wave * Cfg::RPW + j * 16 + (lane >> 2);
+      prow = prow < BM + BN ? prow : BM + BN - 1;  // lanes beyond a partial last copy are disabled anyway
+      const int pos = lane & 3;
+      if (prow < BM) {
+        const int chunk = pos ^ ((prow >> 2) & 3);
+        const int gr = m0 + prow < M ? m0 + prow : M - 1;  // edge rows re-read the last row; never stored
+        src[j] = (const TI_GLOBAL_AS int8_t*)(A + (size_t)gr * p.lda + chunk * 16);
+      } else {
+        const int br = prow - BM;
+        const int chunk = pos ^ ((br >> 2) & 3);
+        const int gr = n0 + br < N ? n0 + br : N - 1;
+        src[j] = (const TI_GLOBAL_AS int8_t*)(B + (size_t)gr * p.ldb + chunk * 16);
+      }
+    }
+  };
+  int c_item = first, c_kt = 0, c_g = 0, c_live = 1;
+  auto issue_copies = [&]() {
+    TI_LDS_AS char* dst = (TI_LDS_AS char*)smem + (c_g % S) * Cfg::STAGE_BYTES + wave * Cfg::RPW * PBK;
+#pragma unroll
+    for (int j = 0; j < COPIES; ++j) {
+      if (Cfg::TAIL_ROWS == 0 || j + 1 < COPIES || lane < Cfg::TAIL_ROWS * 4)
+        __builtin_amdgcn_global_load_lds((const TI_GLOBAL_AS void*)(src[j] + c_kt * PBK),
+                                         (TI_LDS_AS void*)(dst + j * 1024), 16, 0, 0);
+    }
+    c_kt += c_live;
+    ++c_g;
+  };
+  auto advance_copy_item = [&]() {  // call when c_live && c_kt == KT
+    if (c_g < G) {
+      c_kt = 0;
+      c_item += stride;
+      set_copy_item(c_item);
+    } else {
+      c_live = 0;
+      c_kt = KT - 1;
+    }
+  };
+
+  // ---- fragment addressing: lane reads panel row (lane & 15), chunk (lane >> 4)
+  const int r = lane & 15, g4 = lane >> 4;
+  const int fpos = (g4 ^ (r >> 2)) & 3;
+  const int a_frag = (wave_m * Cfg::WTM + r) * PBK + (fpos << 4);
+  const int b_frag = BM * PBK + (wave_n * Cfg::WTN + r) * PBK + (fpos << 4);
+
+  v4i acc[TM][TN];
+  auto zero_acc = [&]() {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) acc[i][j] = v4i{0, 0, 0, 0};
+  };
+  auto read_frags = [&](int gs, v4i (&fa)[TM], v4i (&fb)[TN]) {
+    const char* st = smem + (gs % S) * Cfg::STAGE_BYTES;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) fa[i] = *reinterpret_cast<const v4i*>(st + a_frag + i * 16 * PBK);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) fb[j] = *reinterpret_cast<const v4i*>(st + b_frag + j * 16 * PBK);
+  };
+  auto mma = [&](v4i (&fa)[TM], v4i (&fb)[TN]) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[j], fa[i], acc[i][j], 0, 0, 0);
+  };
+  auto interleave = [&]() {  // one LDS read after each of the first TM+TN MFMAs
+#pragma unroll
+    for (int i = 0; i < TM + TN; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - (TM + TN), 0);
+  };
+
+  set_copy_item(c_item);
+#pragma unroll
+  for (int s = 0; s < S - 1; ++s) {
+    issue_copies();
+    if (c_live && c_kt == KT) advance_copy_item();
+  }
+  wait_copies_then_barrier<(S - 2) * COPIES>();
+
+  v4i fa0[TM], fb0[TN], fa1[TM], fb1[TN];
+  read_frags(0, fa0, fb0);
+  zero_acc();
+
+  int item = first, kt = 0, gs = 0;  // multiply cursor
+  // One K step: multiply the fragments in (fc, fd) while those of the next step load into (fn, fm).
+  auto step = [&](v4i (&fc)[TM], v4i (&fd)[TN], v4i (&fn)[TM], v4i (&fm)[TN], auto last) {
+    constexpr bool LAST = decltype(last)::value;
+    wait_copies_then_barrier<(S - 3) * COPIES>();  // step gs+1 landed; every wave is done with step gs-1
+    issue_copies();                                // step gs+S-1 into the stage step gs-1 used
+    if (!LAST) read_frags(gs + 1, fn, fm);
+    mma(fc, fd);
+    if (!LAST) interleave();
+    ++gs;
+  };
+  auto finish_item = [&]() {
+    const int b = item / tiles;
+    int tile_m, tile_n;
+    tile_of_workgroup(item - b * tiles, tiles_m, tiles_n, tile_m, tile_n);
+    int lane_here = lane;  // opaque copy: keeps the epilogue's address arithmetic out of the mainloop
+    asm volatile("" : "+v"(lane_here));
+    const int er = lane_here & 15, eg = lane_here >> 4;
+    Out* __restrict__ C = reinterpret_cast<Out*>(p.C) + (long long)b * p.strideC;
+    const BiasT* __restrict__ bias = reinterpret_cast<const BiasT*>(p.bias);
+    const bool vec_ok = (N & 3) == 0;
+    const bool bias_al = (reinterpret_cast<uintptr_t>(bias) & 15) == 0;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int nb = tile_n * BN + wave_n * Cfg::WTN + j * 16 + 4 * eg;
+      float bt[4];
+      if (E::kHasBias && vec_ok && bias_al && nb + 4 <= N) {
+        BiasT bv[4];
+        if (sizeof(BiasT) == 1) {
+          const int w = *reinterpret_cast<const int*>(bias + nb);
+          __builtin_memcpy(bv, &w, 4);
+        } else {
+          const v4i w = *reinterpret_cast<const v4i*>(bias + nb);
+          __builtin_memcpy(bv, &w, 16);
+        }
+#pragma unroll
+        for (int v = 0; v < 4; ++v) bt[v] = E::bias_term(bv[v], p.beta);
+      } else {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          BiasT bv = BiasT(0);
+          if (E::kHasBias && nb + v < N) bv = bias[nb + v];
+          bt[v] = E::bias_term(bv, p.beta);
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const int m = tile_m * BM + wave_m * Cfg::WTM + i * 16 + er;
+        if (m >= M) continue;
+        Out o[4];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) o[v] = E::apply(acc[i][j][v], bt[v], p.alpha);
+        Out* dst = C + (long long)m * N + nb;
+        if (vec_ok && nb + 4 <= N) {
+          if (sizeof(Out) == 4) {
+            using W = typename std::conditional<sizeof(Out) == 4, Out, int>::type;
+            v4i w4 = {__builtin_bit_cast(int, (W)o[0]), __builtin_bit_cast(int, (W)o[1]),
+                      __builtin_bit_cast(int, (W)o[2]), __builtin_bit_cast(int, (W)o[3])};
+            *reinterpret_cast<v4i*>(dst) = w4;
+          } else {
+            *reinterpret_cast<unsigned*>(dst) = (unsigned)(unsigned char)o[0] | ((unsigned)(unsigned char)o[1] << 8) |
+                                                ((unsigned)(unsigned char)o[2] << 16) |
+                                                ((unsigned)(unsigned char)o[3] << 24);
+          }
+        } else {
+#pragma unroll
+          for (int v = 0; v < 4; ++v)
+            if (nb + v < N) dst[v] = o[v];
+        }
+      }
+    }
+    item += stride;
+    kt = 0;
+    zero_acc();
+  };
+
+  while (gs < G) {
+    // steps until the multiply or the copy cursor reaches the end of its work item
+    int n = KT - kt;
+    if (c_live && KT - c_kt < n) n = KT - c_kt;
+    const bool item_done = kt + n == KT;
+    int plain = item_done ? n - 1 : n;  // steps that also load the next step's fragments
+    for (; plain >= 2; plain -= 2) {
+      step(fa0, fb0, fa1, fb1, std::false_type{});
+      step(fa1, fb1, fa0, fb0, std::false_type{});
+    }
+    if (plain == 1) {
+      step(fa0, fb0, fa1, fb1, std::false_type{});
+#pragma unroll
+      for (int i = 0; i < TM; ++i) fa0[i] = fa1[i];
+#pragma unroll
+      for (int j = 0; j < TN; ++j) fb0[j] = fb1[j];
+    }
+    if (item_done) step(fa0, fb0, fa1, fb1, std::true_type{});
+    kt += n;
+    if (c_live && c_kt == KT) advance_copy_item();
+    if (item_done) {
+      finish_item();
+      if (gs < G) read_frags(gs, fa0, fb0);
+    }
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // the trailing filler copies must land before the LDS is released
+}
+
 // Epilogue of the M <= 16 kernels: the lane holds row m and columns nb .. nb+3.
 template <int KIND>
 __device__ __forceinline__ void store_skinny_tile(v4i acc, const GemmParams& p, int batch, int m, int nb) {
@@ -831,10 +1082,9 @@ static int num_cus() {
   return n;
 }
 
-template <class Cfg>
-static int launch_pipe(const GemmParams& p, hipStream_t stream) {
+template <class Cfg, class Kern>
+static int launch_persistent(Kern kern, const GemmParams& p, hipStream_t stream) {
   static bool attr_set = false;
-  auto kern = gemm_pipe_kernel<Cfg>;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
@@ -859,6 +1109,15 @@ static int launch_pipe(const GemmParams& p, hipStream_t stream) {
 // kernel (raw int32 output into a workspace [splits][M][N]); this kernel then
 // adds the slices and applies the epilogue.  Integer partial sums make the
 // result independent of the split.
+template <class Cfg>
+static int launch_pipe(const GemmParams& p, hipStream_t stream) {
+  return launch_persistent<Cfg>(gemm_pipe_kernel<Cfg>, p, stream);
+}
+template <class Cfg>
+static int launch_pipe16(const GemmParams& p, hipStream_t stream) {
+  return launch_persistent<Cfg>(gemm_pipe16_kernel<Cfg>, p, stream);
+}
+
 template <int KIND>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmParams p, const int* __restrict__ ws, int splits) {
   using E = Epi<KIND>;
@@ -1013,7 +1272,20 @@ static int launch_kind(const GemmParams& p, void* workspace, long long workspace
   const long long t256 = (long long)((p.M + 255) / 256) * ((p.N + 255) / 256) * p.batch;
   const long long t128 = (long long)((p.M + 127) / 128) * ((p.N + 127) / 128) * p.batch;
   if (p.K % PBK == 0 && p.K >= PBK) {
-    if (t256 >= 160) return launch_pipe<PipeCfg<256, 256, 2, 4, 4, KIND, SWAP>>(p, stream);
+    if (t256 >= 160) {
+      // 256x160 tiles (16x16 blocks) when the width allows it and they fill the CUs more evenly.
+      // Measured at full occupancy the 16x16-block kernel reaches 0.78 of the 256x256 kernel's rate
+      // (one barrier per 20 short MFMAs instead of per 16 long ones), so it only pays off when the
+      // 256x256 grid would leave more than a fifth of the CUs idle (e.g. 2048x5120: 160 tiles).
+      const long long cus = num_cus();
+      const long long t160 = (long long)((p.M + 255) / 256) * ((p.N + 159) / 160) * p.batch;
+      const double e256 = (double)t256 / (double)(((t256 + cus - 1) / cus) * cus);
+      const double e160 = 0.78 * (double)t160 / (double)(((t160 + cus - 1) / cus) * cus);
+      static const int force = getenv("TI_TILE") ? atoi(getenv("TI_TILE")) : 0;  // experiments: 1 = 256x256, 2 = 256x160
+      if ((p.N % 160 == 0 && e160 > e256 && force != 1) || force == 2)
+        return launch_pipe16<Pipe16Cfg<256, 160, 4, 2, 5, KIND>>(p, stream);
+      return launch_pipe<PipeCfg<256, 256, 2, 4, 4, KIND, SWAP>>(p, stream);
+    }
     if (t128 >= 128) return launch_pipe<PipeCfg<128, 128, 2, 2, 4, KIND, SWAP>>(p, stream);
   }
   if (t256 >= 160) return launch_tile<TileCfg<256, 256, 2, 4, KIND, SWAP>>(p, stream);
