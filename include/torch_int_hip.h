@@ -130,6 +130,14 @@ int ti_add_layernorm_q(const float* x, float* residual, const float* gamma, cons
 int ti_attn_softmax_q(const float* scores, const float* mask, int8_t* probs, int64_t batch, int64_t heads,
                       int64_t T, int64_t S, void* stream);
 
+/* dst[b, y, x, :] = src[b, x, y, :] for int8 [B, X, Y, D]: the head split / merge
+ * `view(B,T,H,d).transpose(1,2).contiguous()` (torch_int/models/opt.py:80-81,189-196). */
+int ti_permute_0213_s8(const int8_t* src, int8_t* dst, int64_t B, int64_t X, int64_t Y, int64_t D, void* stream);
+
+/* dst[b, c, r] = src[b, r, c] for int8 [B, R, C]: `value_states.transpose(1, 2).contiguous()`
+ * (torch_int/models/opt.py:180). */
+int ti_transpose_last2_s8(const int8_t* src, int8_t* dst, int64_t B, int64_t R, int64_t C, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -384,6 +384,24 @@ def test_fused_attn_softmax_q():
             assert int(out.min()) >= 0
 
 
+def test_int8_layout_kernels():
+    import torch_int._hip_ext as X
+    g = torch.Generator().manual_seed(9)
+    for (B, T, H, d) in [(4, 512, 40, 128), (2, 37, 4, 64), (1, 1, 3, 24), (3, 5, 7, 20)]:
+        _say(f"split/merge heads B={B} T={T} H={H} d={d}")
+        t = _s8(g, B, T, H * d).to(DEV)
+        ref = t.view(B, T, H, d).transpose(1, 2).contiguous()
+        out = X.split_heads(t, B, T, H, d)
+        assert out.is_contiguous() and torch.equal(out, ref)
+        back = X.merge_heads(out.view(B * H, T, d), B, H, T, d)
+        assert back.shape == (B, T, H * d) and torch.equal(back, t)
+    for (B, R, C) in [(160, 512, 128), (8, 513, 128), (3, 70, 50), (2, 1, 128), (5, 64, 1), (1, 200, 333)]:
+        _say(f"transpose_last2 B={B} R={R} C={C}")
+        t = _s8(g, B, R, C).to(DEV)
+        out = X.transpose_last2(t)
+        assert out.is_contiguous() and torch.equal(out, t.transpose(1, 2).contiguous())
+
+
 def test_runs_are_deterministic():
     # identical bytes on repeated launches (an LDS race would show up here)
     import torch_int._CUDA as C

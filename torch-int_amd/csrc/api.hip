@@ -196,4 +196,28 @@ int ti_attn_softmax_q(const float* scores, const float* mask, int8_t* probs, int
   return launch_attn_softmax_q(scores, mask, probs, batch, heads, T, S, static_cast<hipStream_t>(stream));
 }
 
+int ti_permute_0213_s8(const int8_t* src, int8_t* dst, int64_t B, int64_t X, int64_t Y, int64_t D, void* stream) {
+  g_err[0] = 0;
+  const char* op = "permute_0213_s8";
+  const int64_t lim = 0x7fffffffLL;
+  if (B < 0 || X < 0 || Y < 0 || D < 0 || X > lim || Y > lim || D > lim || B > lim)
+    return fail(TI_ERR_INVALID_ARG, "%s: sizes must be in [0, 2^31)", op);
+  const bool nonempty = B > 0 && X > 0 && Y > 0 && D > 0;
+  if (int rc = check_ptr(op, "src", src, 1, nonempty)) return rc;
+  if (int rc = check_ptr(op, "dst", dst, 1, nonempty)) return rc;
+  return launch_permute_0213_s8(src, dst, B, X, Y, D, static_cast<hipStream_t>(stream));
+}
+
+int ti_transpose_last2_s8(const int8_t* src, int8_t* dst, int64_t B, int64_t R, int64_t C, void* stream) {
+  g_err[0] = 0;
+  const char* op = "transpose_last2_s8";
+  const int64_t lim = 0x7fffffffLL;
+  if (B < 0 || R < 0 || C < 0 || R > lim || C > lim || B > 65535 || (R + 63) / 64 > 65535)
+    return fail(TI_ERR_INVALID_ARG, "%s: needs 0 <= B <= 65535, R < 2^22, C < 2^31", op);
+  const bool nonempty = B > 0 && R > 0 && C > 0;
+  if (int rc = check_ptr(op, "src", src, 1, nonempty)) return rc;
+  if (int rc = check_ptr(op, "dst", dst, 1, nonempty)) return rc;
+  return launch_transpose_last2_s8(src, dst, B, R, C, static_cast<hipStream_t>(stream));
+}
+
 }  // extern "C"

@@ -1,0 +1,112 @@
+// int8 layout changes of the attention block, as single coalesced passes:
+//   permute_0213:  [B, X, Y, D] -> [B, Y, X, D]   (rows of D bytes move intact: the
+//                  head split / merge  view(B,T,H,d).transpose(1,2).contiguous())
+//   transpose_last2: [B, R, C] -> [B, C, R]        (byte transpose: V -> V^T)
+#include "ti_common.h"
+
+namespace ti {
+
+// one thread per 16-byte chunk of the output; D % 16 == 0, 16-byte aligned pointers
+__global__ __launch_bounds__(256) void permute_0213_v16_kernel(const v4i* __restrict__ src, v4i* __restrict__ dst,
+                                                               int X, int Y, int chunks, long long total) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const int c = (int)(i % chunks);
+  long long row = i / chunks;            // output row index: (b, y, x)
+  const int x = (int)(row % X);
+  row /= X;
+  const int y = (int)(row % Y);
+  const long long b = row / Y;
+  dst[i] = src[((b * X + x) * Y + y) * chunks + c];
+}
+
+__global__ __launch_bounds__(256) void permute_0213_bytes_kernel(const int8_t* __restrict__ src,
+                                                                 int8_t* __restrict__ dst, int X, int Y, int D,
+                                                                 long long total) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const int c = (int)(i % D);
+  long long row = i / D;
+  const int x = (int)(row % X);
+  row /= X;
+  const int y = (int)(row % Y);
+  const long long b = row / Y;
+  dst[i] = src[((b * X + x) * Y + y) * D + c];
+}
+
+// 64x64 byte tiles through LDS; any R, C
+__global__ __launch_bounds__(256) void transpose_last2_kernel(const int8_t* __restrict__ src, int8_t* __restrict__ dst,
+                                                              int R, int C) {
+  __shared__ int8_t tile[64][64 + 4];
+  const long long base = (long long)blockIdx.z * R * C;
+  const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+  const int t = threadIdx.x;
+  // load: thread t covers row t/4, bytes (t%4)*16 .. +15
+  {
+    const int r = r0 + (t >> 2), cb = c0 + (t & 3) * 16;
+    if (r < R) {
+      const int8_t* s = src + base + (long long)r * C + cb;
+      if (cb + 16 <= C && ((reinterpret_cast<uintptr_t>(s) & 15) == 0)) {
+        v4i v = *reinterpret_cast<const v4i*>(s);
+        int8_t b[16];
+        __builtin_memcpy(b, &v, 16);
+#pragma unroll
+        for (int j = 0; j < 16; ++j) tile[t >> 2][(t & 3) * 16 + j] = b[j];
+      } else {
+        for (int j = 0; j < 16; ++j)
+          if (cb + j < C) tile[t >> 2][(t & 3) * 16 + j] = s[j];
+      }
+    }
+  }
+  __syncthreads();
+  // store: thread t covers output row (column of the tile) t/4, bytes (t%4)*16 .. +15 along R
+  {
+    const int c = c0 + (t >> 2), rb = r0 + (t & 3) * 16;
+    if (c < C) {
+      int8_t b[16];
+#pragma unroll
+      for (int j = 0; j < 16; ++j) b[j] = tile[(t & 3) * 16 + j][t >> 2];
+      int8_t* d = dst + base + (long long)c * R + rb;
+      if (rb + 16 <= R && ((reinterpret_cast<uintptr_t>(d) & 15) == 0)) {
+        v4i v;
+        __builtin_memcpy(&v, b, 16);
+        *reinterpret_cast<v4i*>(d) = v;
+      } else {
+        for (int j = 0; j < 16; ++j)
+          if (rb + j < R) d[j] = b[j];
+      }
+    }
+  }
+}
+
+int launch_permute_0213_s8(const int8_t* src, int8_t* dst, long long B, long long X, long long Y, long long D,
+                           hipStream_t stream) {
+  const long long bytes = B * X * Y * D;
+  if (bytes == 0) return TI_OK;
+  const bool v16 = (D % 16 == 0) && ((reinterpret_cast<uintptr_t>(src) & 15) == 0) &&
+                   ((reinterpret_cast<uintptr_t>(dst) & 15) == 0);
+  if (v16) {
+    const long long total = bytes / 16;
+    hipLaunchKernelGGL(permute_0213_v16_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
+                       reinterpret_cast<const v4i*>(src), reinterpret_cast<v4i*>(dst), (int)X, (int)Y, (int)(D / 16),
+                       total);
+  } else {
+    hipLaunchKernelGGL(permute_0213_bytes_kernel, dim3((unsigned)((bytes + 255) / 256)), dim3(256), 0, stream, src,
+                       dst, (int)X, (int)Y, (int)D, bytes);
+  }
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "permute launch: %s", hipGetErrorString(e));
+  return TI_OK;
+}
+
+int launch_transpose_last2_s8(const int8_t* src, int8_t* dst, long long B, long long R, long long C,
+                              hipStream_t stream) {
+  if (B * R * C == 0) return TI_OK;
+  dim3 grid((unsigned)((C + 63) / 64), (unsigned)((R + 63) / 64), (unsigned)B);
+  hipLaunchKernelGGL(transpose_last2_kernel, grid, dim3(256), 0, stream, src, dst, (int)R, (int)C);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "transpose launch: %s", hipGetErrorString(e));
+  return TI_OK;
+}
+
+}  // namespace ti

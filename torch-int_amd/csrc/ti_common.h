@@ -159,4 +159,10 @@ int launch_add_layernorm_q(const float* x, float* residual, const float* gamma, 
 int launch_attn_softmax_q(const float* scores, const float* mask, int8_t* out, long long batch, long long heads,
                           long long T, long long S, hipStream_t stream);
 
+// permute.hip
+int launch_permute_0213_s8(const int8_t* src, int8_t* dst, long long B, long long X, long long Y, long long D,
+                           hipStream_t stream);
+int launch_transpose_last2_s8(const int8_t* src, int8_t* dst, long long B, long long R, long long C,
+                              hipStream_t stream);
+
 }  // namespace ti

@@ -21,6 +21,10 @@ _lib.ti_add_layernorm_q.argtypes = [_vp, _vp, _vp, _vp, _f32, _vp, _i64, _i64, _
 _lib.ti_add_layernorm_q.restype = ctypes.c_int
 _lib.ti_attn_softmax_q.argtypes = [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]
 _lib.ti_attn_softmax_q.restype = ctypes.c_int
+_lib.ti_permute_0213_s8.argtypes = [_vp, _vp, _i64, _i64, _i64, _i64, _vp]
+_lib.ti_permute_0213_s8.restype = ctypes.c_int
+_lib.ti_transpose_last2_s8.argtypes = [_vp, _vp, _i64, _i64, _i64, _vp]
+_lib.ti_transpose_last2_s8.restype = ctypes.c_int
 _raw_stream = torch._C._cuda_getCurrentRawStream
 
 
@@ -79,4 +83,44 @@ def attn_softmax_q(scores, mask, heads):
                                     bsz, heads, T, S, _raw_stream(dev.index) or None)
     if rc:
         raise RuntimeError(f"torch_int._hip_ext.{op}: {_lib.ti_last_error().decode()} (status {rc})")
+    return out
+
+
+def split_heads(t, bsz, seq_len, heads, head_dim):
+    """int8 [bsz, seq, heads*head_dim] -> contiguous [bsz, heads, seq, head_dim]
+    (``view(bsz, seq, heads, d).transpose(1, 2).contiguous()``)."""
+    if not (_ok(t, torch.int8) and t.numel() == bsz * seq_len * heads * head_dim and t.numel() > 0):
+        return t.view(bsz, seq_len, heads, head_dim).transpose(1, 2).contiguous()
+    out = torch.empty((bsz, heads, seq_len, head_dim), dtype=torch.int8, device=t.device)
+    with torch.cuda.device(t.device):
+        rc = _lib.ti_permute_0213_s8(t.data_ptr(), out.data_ptr(), bsz, seq_len, heads, head_dim,
+                                     _raw_stream(t.device.index) or None)
+    if rc:
+        raise RuntimeError(f"torch_int._hip_ext.split_heads: {_lib.ti_last_error().decode()} (status {rc})")
+    return out
+
+
+def merge_heads(t, bsz, heads, seq_len, head_dim):
+    """int8 [bsz*heads, seq, head_dim] -> contiguous [bsz, seq, heads*head_dim]."""
+    if not (_ok(t, torch.int8) and t.numel() == bsz * seq_len * heads * head_dim and t.numel() > 0):
+        return t.view(bsz, heads, seq_len, head_dim).transpose(1, 2).reshape(bsz, seq_len, heads * head_dim).contiguous()
+    out = torch.empty((bsz, seq_len, heads * head_dim), dtype=torch.int8, device=t.device)
+    with torch.cuda.device(t.device):
+        rc = _lib.ti_permute_0213_s8(t.data_ptr(), out.data_ptr(), bsz, heads, seq_len, head_dim,
+                                     _raw_stream(t.device.index) or None)
+    if rc:
+        raise RuntimeError(f"torch_int._hip_ext.merge_heads: {_lib.ti_last_error().decode()} (status {rc})")
+    return out
+
+
+def transpose_last2(t):
+    """int8 [B, R, C] -> contiguous [B, C, R]."""
+    if not (_ok(t, torch.int8) and t.dim() == 3 and t.numel() > 0 and t.shape[0] <= 65535):
+        return t.transpose(1, 2).contiguous()
+    B, R, C = t.shape
+    out = torch.empty((B, C, R), dtype=torch.int8, device=t.device)
+    with torch.cuda.device(t.device):
+        rc = _lib.ti_transpose_last2_s8(t.data_ptr(), out.data_ptr(), B, R, C, _raw_stream(t.device.index) or None)
+    if rc:
+        raise RuntimeError(f"torch_int._hip_ext.transpose_last2: {_lib.ti_last_error().decode()} (status {rc})")
     return out

@@ -62,7 +62,10 @@ class Int8OPTAttention(nn.Module):
         return q
 
     def _shape(self, tensor: torch.Tensor, seq_len: int, bsz: int):
-        return tensor.view(bsz, seq_len, self.num_heads, self.head_dim).transpose(1, 2).contiguous()
+        """[bsz, seq, embed] -> contiguous [bsz, heads, seq, head_dim]."""
+        if seq_len < 0:
+            seq_len = tensor.numel() // (bsz * self.embed_dim)
+        return _hip_ext.split_heads(tensor, bsz, seq_len, self.num_heads, self.head_dim)
 
     @torch.no_grad()
     def forward(self, hidden_states: torch.Tensor, key_value_states: Optional[torch.Tensor] = None,
@@ -121,11 +124,11 @@ class Int8OPTAttention(nn.Module):
             # (models/opt.py:166-178).
             probs_q = probs.mul_(127).round_().to(torch.int8)
         # P.V with V transposed to [bsz*H, d, src]: (P V) = P . (V^T)^T
-        value_t = value.transpose(1, 2).contiguous()
+        value_t = _hip_ext.transpose_last2(value)
         ctx = self.pv_bmm(probs_q, value_t)  # int8 [bsz*H, tgt, d]
         if ctx.size() != (bsz * H, tgt_len, d):
             raise ValueError(f"`attn_output` should be of size {(bsz, H, tgt_len, d)}, but is {ctx.size()}")
-        ctx = ctx.view(bsz, H, tgt_len, d).transpose(1, 2).reshape(bsz, tgt_len, self.embed_dim).contiguous()
+        ctx = _hip_ext.merge_heads(ctx, bsz, H, tgt_len, d)
         return self.out_proj(ctx), probs_out, present
 
 
