@@ -302,7 +302,7 @@ static float exp_nonpos(float x) {
 }
 
 /* The chain between the two attention products (torch_int/models/opt.py:144-178):
- * s = max(scores + mask, -FLT_MAX); p = softmax(s) over the last dim; probs = int8(rint(127 p)).
+ * s = max(scores + mask, -FLT_MAX); e = exp(s - max s); probs = int8(rint(e * (127 / sum e))).
  * scores [batch*heads, T, S], mask [batch, 1, T, S] or NULL.  Reduction order: chunk c
  * (elements 4c..4c+3) belongs to lane c mod 64, a lane visits its elements in ascending order,
  * lanes combine with a xor butterfly (offsets 32..1). */
@@ -349,7 +349,8 @@ void orc_attn_softmax_q(const float* scores, const float* mask, int8_t* probs, i
       memcpy(cur, nxt, sizeof(cur));
     }
     float s = cur[0];
-    for (int64_t i = 0; i < S; ++i) probs[row * S + i] = (int8_t)(int)rintf((v[i] / s) * 127.0f);
+    float scale = 127.0f / s; /* one division per row */
+    for (int64_t i = 0; i < S; ++i) probs[row * S + i] = (int8_t)(int)rintf(v[i] * scale);
     free(v);
   }
 }

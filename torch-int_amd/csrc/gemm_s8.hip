@@ -317,9 +317,10 @@ __global__ __launch_bounds__(Cfg::NT) void gemm_tile_kernel(GemmParams p, int ti
 
 static constexpr int PBK = 64;
 
-template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int STAGES_, int KIND_, bool SWAP_>
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int STAGES_, int KIND_, bool SWAP_, int MIN_WAVES_ = 2>
 struct PipeCfg {
   static constexpr int BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, KIND = KIND_;
+  static constexpr int MIN_WAVES = MIN_WAVES_;  // waves per SIMD the register budget is sized for
   static constexpr int STAGES = STAGES_;
   static constexpr bool SWAP = SWAP_;
   static constexpr int NWAVES = WAVES_M * WAVES_N;
@@ -342,7 +343,7 @@ __device__ __forceinline__ void wait_copies_then_barrier() {
 
 // items = tiles_m * tiles_n * batch work items; item -> (batch, tile) with the tile index minor.
 template <class Cfg>
-__global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe_kernel(GemmParams p, int tiles_m, int tiles_n, int items) {
+__global__ __launch_bounds__(Cfg::NT, Cfg::MIN_WAVES) void gemm_pipe_kernel(GemmParams p, int tiles_m, int tiles_n, int items) {
   constexpr int BM = Cfg::BM, BN = Cfg::BN, TM = Cfg::TM, TN = Cfg::TN, COPIES = Cfg::COPIES;
   constexpr int S = Cfg::STAGES;
   constexpr bool SWAP = Cfg::SWAP;
@@ -1272,7 +1273,9 @@ static int launch_kind(const GemmParams& p, void* workspace, long long workspace
   const long long t256 = (long long)((p.M + 255) / 256) * ((p.N + 255) / 256) * p.batch;
   const long long t128 = (long long)((p.M + 127) / 128) * ((p.N + 127) / 128) * p.batch;
   if (p.K % PBK == 0 && p.K >= PBK) {
-    if (t256 >= 160) {
+    // a 256-wide tile on a narrow or short output would mostly multiply padding
+    const bool wide = p.N > 128 && p.M > 128;
+    if (t256 >= 160 && wide) {
       // 256x160 tiles (16x16 blocks) when the width allows it and they fill the CUs more evenly.
       // Measured at full occupancy the 16x16-block kernel reaches 0.78 of the 256x256 kernel's rate
       // (one barrier per 20 short MFMAs instead of per 16 long ones), so it only pays off when the

@@ -101,6 +101,7 @@ __global__ __launch_bounds__(256) void attn_softmax_q_kernel(const float* __rest
     }
   }
   s = wave_sum(s);
+  const float scale = 127.0f / s;  // one division per row; probabilities are e * scale
   int* dst = reinterpret_cast<int*>(out + row * S);
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
@@ -109,7 +110,7 @@ __global__ __launch_bounds__(256) void attn_softmax_q_kernel(const float* __rest
       unsigned w = 0;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const float pq = __builtin_rintf((v[i][j] / s) * 127.0f);  // in [0, 127]
+        const float pq = __builtin_rintf(v[i][j] * scale);  // in [0, 127]
         w |= (unsigned)(int)pq << (8 * j);
       }
       dst[c] = (int)w;
@@ -152,10 +153,11 @@ __global__ __launch_bounds__(256) void attn_softmax_q_generic_kernel(const float
     for (int j = 0; j < 4; ++j)
       if (c * 4 + j < S) s = s + exp_nonpos(value(c * 4 + j) - m);
   s = wave_sum(s);
+  const float scale = 127.0f / s;
   for (int c = lane; c < nchunks; c += 64)
     for (int j = 0; j < 4; ++j)
       if (c * 4 + j < S)
-        out[row * S + c * 4 + j] = (int8_t)(int)__builtin_rintf((exp_nonpos(value(c * 4 + j) - m) / s) * 127.0f);
+        out[row * S + c * 4 + j] = (int8_t)(int)__builtin_rintf(exp_nonpos(value(c * 4 + j) - m) * scale);
 }
 
 int launch_attn_softmax_q(const float* scores, const float* mask, int8_t* out, long long batch, long long heads,
