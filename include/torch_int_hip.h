@@ -48,8 +48,9 @@ const char* ti_last_error(void);
 int ti_init(void);
 
 /* Bytes of scratch the linear entry points can use for (M,N,K) to split the K
- * loop over workgroups when M is small (decode).  Passing a smaller or NULL
- * workspace is always legal and only selects a non-split kernel. */
+ * loop over workgroups when the output has too few tiles to fill the chip
+ * (16 < M <= 1024 with a long K); 0 when no split is worthwhile.  Passing a
+ * smaller or NULL workspace is always legal and only selects a non-split kernel. */
 int64_t ti_linear_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
 /* ---- W8A8 linear: out[M,N] = epilogue(x[M,K] . w[N,K]^T, bias[N]) ---- */
@@ -129,6 +130,13 @@ int ti_add_layernorm_q(const float* x, float* residual, const float* gamma, cons
  * attention products (torch_int/models/opt.py:144-178). */
 int ti_attn_softmax_q(const float* scores, const float* mask, int8_t* probs, int64_t batch, int64_t heads,
                       int64_t T, int64_t S, void* stream);
+
+/* c[b,M,N] = s8(rint(clamp(alpha * a[b,M,K] . bm[b,K,N], -128, 127))) with bm ROW-major (not transposed):
+ * the P.V product on V as the KV cache stores it, replacing `value_states.transpose(1, 2).contiguous()`
+ * followed by bmm_s8t_s8n_s8t (torch_int/models/opt.py:180-182) when few query rows are live
+ * (incremental decoding).  Any M works, 16 rows per pass over bm; any K and N (no multiple-of-16 rule). */
+int ti_bmm_s8t_s8t_s8t(const int8_t* a, const int8_t* bm, int8_t* c, int64_t batch, int64_t M, int64_t N, int64_t K,
+                       float alpha, void* stream);
 
 /* dst[b, y, x, :] = src[b, x, y, :] for int8 [B, X, Y, D]: the head split / merge
  * `view(B,T,H,d).transpose(1,2).contiguous()` (torch_int/models/opt.py:80-81,189-196). */

@@ -235,3 +235,8 @@ def attn_softmax_q(scores, mask, heads):
         mp = _p(mask)
     _load().orc_attn_softmax_q(_p(scores), mp, _p(out), _i64(batch), _i64(heads), _i64(T), _i64(S))
     return out
+
+
+def bmm_s8t_s8t_s8t(a, b, alpha):
+    """P.V with V row-major: a [B,M,K], b [B,K,N] (ti_bmm_s8t_s8t_s8t) = bmm_s8t_s8n_s8t on b transposed."""
+    return bmm_s8t_s8n_s8t(a, b.transpose(1, 2).contiguous(), alpha)

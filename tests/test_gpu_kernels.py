@@ -227,7 +227,8 @@ def test_bmm_shapes():
     # upstream minimum shapes (tests/test_bmm_shape.py:8,19), kernel test shapes
     # (tests/test_bmm.py:8,114), ragged, decode-like (M=1, src_len not a multiple of 16)
     shapes = [(1, 1, 4, 16), (1, 1, 16, 16), (1, 512, 32, 512), (1, 512, 12288, 512), (3, 70, 50, 96),
-              (5, 33, 129, 128), (8, 1, 513, 128), (8, 1, 128, 513), (2, 130, 130, 528), (16, 128, 128, 128)]
+              (5, 33, 129, 128), (8, 1, 513, 128), (8, 1, 128, 513), (2, 130, 130, 528), (16, 128, 128, 128),
+              (12, 1, 517, 128), (3, 4, 33, 64), (2, 16, 1030, 256), (2, 300, 132, 64), (3, 5, 20, 32)]
     for i, (B, M, N, K) in enumerate(shapes):
         _say(f"bmm B={B} M={M} N={N} K={K}")
         _bmm_case(C, B, M, N, K, seed=200 + i)
@@ -400,6 +401,29 @@ def test_int8_layout_kernels():
         t = _s8(g, B, R, C).to(DEV)
         out = X.transpose_last2(t)
         assert out.is_contiguous() and torch.equal(out, t.transpose(1, 2).contiguous())
+
+
+def test_bmm_rowmajor_rhs_for_decode():
+    # P.V on V as the KV cache stores it: [B, M, K] x [B, K, N], any K and N
+    import torch_int._hip_ext as X
+    g = torch.Generator().manual_seed(41)
+    shapes = [(288, 1, 128, 517), (16, 1, 128, 2500), (8, 4, 128, 33), (3, 16, 100, 50), (2, 37, 64, 300),
+              (2, 2, 130, 70), (3, 1, 7, 5), (2, 3, 16, 0), (1, 16, 256, 1024)]
+    for (B, M, N, K) in shapes:
+        _say(f"bmm_s8t_s8t_s8t B={B} M={M} N={N} K={K}")
+        a = _s8(g, B, M, K, lo=0)
+        b = _s8(g, B, K, N)
+        alpha = _scal(g, 2e-4, 4e-3)
+        out = X.bmm_s8t_s8t_s8t(a.to(DEV), b.to(DEV), alpha).cpu()
+        assert torch.equal(out, orc.bmm_s8t_s8t_s8t(a, b, alpha)), (B, M, N, K)
+    # an operand pair whose rows are not dword aligned takes the byte path
+    a, b = _s8(g, 2, 3, 40), _s8(g, 2, 41, 24)
+    bd = b.to(DEV)[:, 1:, :].contiguous()
+    odd = torch.empty(2 * 40 * 24 + 1, dtype=torch.int8, device=DEV)[1:].view(2, 40, 24)
+    odd.copy_(bd)
+    assert odd.data_ptr() % 4 != 0
+    out = X.bmm_s8t_s8t_s8t(a.to(DEV), odd, 0.001).cpu()
+    assert torch.equal(out, orc.bmm_s8t_s8t_s8t(a, b[:, 1:, :].contiguous(), 0.001))
 
 
 def test_runs_are_deterministic():

@@ -196,6 +196,18 @@ int ti_attn_softmax_q(const float* scores, const float* mask, int8_t* probs, int
   return launch_attn_softmax_q(scores, mask, probs, batch, heads, T, S, static_cast<hipStream_t>(stream));
 }
 
+int ti_bmm_s8t_s8t_s8t(const int8_t* a, const int8_t* b, int8_t* c, int64_t batch, int64_t M, int64_t N, int64_t K,
+                       float alpha, void* stream) {
+  g_err[0] = 0;
+  const char* op = "bmm_s8t_s8t_s8t";
+  if (int rc = check_dims(op, batch, M, N, K)) return rc;
+  const bool nonempty = batch > 0 && M > 0 && N > 0;
+  if (int rc = check_ptr(op, "a", a, 1, nonempty && K > 0)) return rc;
+  if (int rc = check_ptr(op, "b", b, 1, nonempty && K > 0)) return rc;
+  if (int rc = check_ptr(op, "c", c, 1, nonempty)) return rc;
+  return launch_bmm_s8t_s8t_s8t(a, b, c, batch, M, N, K, alpha, static_cast<hipStream_t>(stream));
+}
+
 int ti_permute_0213_s8(const int8_t* src, int8_t* dst, int64_t B, int64_t X, int64_t Y, int64_t D, void* stream) {
   g_err[0] = 0;
   const char* op = "permute_0213_s8";

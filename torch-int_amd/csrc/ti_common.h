@@ -165,4 +165,8 @@ int launch_permute_0213_s8(const int8_t* src, int8_t* dst, long long B, long lon
 int launch_transpose_last2_s8(const int8_t* src, int8_t* dst, long long B, long long R, long long C,
                               hipStream_t stream);
 
+// bmm_rowmajor.hip
+int launch_bmm_s8t_s8t_s8t(const int8_t* a, const int8_t* b, int8_t* c, long long batch, long long M, long long N,
+                           long long K, float alpha, hipStream_t stream);
+
 }  // namespace ti

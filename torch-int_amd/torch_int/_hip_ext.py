@@ -8,6 +8,10 @@ tensor on a HIP device and fall back to the upstream torch-op chain otherwise.
   nn/fused.py:13-18) in one pass.
 * :func:`attn_softmax_q` -- mask add, clamp to finfo.min, softmax, ``*127``, round, int8 cast
   (upstream models/opt.py:144-178) in one pass.
+* :func:`split_heads`, :func:`merge_heads`, :func:`transpose_last2` -- the int8 layout changes around
+  the two attention products (upstream models/opt.py:80-81, 180, 189-196).
+* :func:`bmm_s8t_s8t_s8t` -- P.V on V as the KV cache stores it (no transposed copy), for the few
+  query rows of incremental decoding.
 """
 import ctypes
 
@@ -25,6 +29,8 @@ _lib.ti_permute_0213_s8.argtypes = [_vp, _vp, _i64, _i64, _i64, _i64, _vp]
 _lib.ti_permute_0213_s8.restype = ctypes.c_int
 _lib.ti_transpose_last2_s8.argtypes = [_vp, _vp, _i64, _i64, _i64, _vp]
 _lib.ti_transpose_last2_s8.restype = ctypes.c_int
+_lib.ti_bmm_s8t_s8t_s8t.argtypes = [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _f32, _vp]
+_lib.ti_bmm_s8t_s8t_s8t.restype = ctypes.c_int
 _raw_stream = torch._C._cuda_getCurrentRawStream
 
 
@@ -89,6 +95,8 @@ def attn_softmax_q(scores, mask, heads):
 def split_heads(t, bsz, seq_len, heads, head_dim):
     """int8 [bsz, seq, heads*head_dim] -> contiguous [bsz, heads, seq, head_dim]
     (``view(bsz, seq, heads, d).transpose(1, 2).contiguous()``)."""
+    if (seq_len == 1 or heads == 1) and t.is_contiguous():
+        return t.view(bsz, heads, seq_len, head_dim)  # the permutation moves nothing
     if not (_ok(t, torch.int8) and t.numel() == bsz * seq_len * heads * head_dim and t.numel() > 0):
         return t.view(bsz, seq_len, heads, head_dim).transpose(1, 2).contiguous()
     out = torch.empty((bsz, heads, seq_len, head_dim), dtype=torch.int8, device=t.device)
@@ -102,6 +110,8 @@ def split_heads(t, bsz, seq_len, heads, head_dim):
 
 def merge_heads(t, bsz, heads, seq_len, head_dim):
     """int8 [bsz*heads, seq, head_dim] -> contiguous [bsz, seq, heads*head_dim]."""
+    if (seq_len == 1 or heads == 1) and t.is_contiguous():
+        return t.view(bsz, seq_len, heads * head_dim)
     if not (_ok(t, torch.int8) and t.numel() == bsz * seq_len * heads * head_dim and t.numel() > 0):
         return t.view(bsz, heads, seq_len, head_dim).transpose(1, 2).reshape(bsz, seq_len, heads * head_dim).contiguous()
     out = torch.empty((bsz, seq_len, heads * head_dim), dtype=torch.int8, device=t.device)
@@ -123,4 +133,25 @@ def transpose_last2(t):
         rc = _lib.ti_transpose_last2_s8(t.data_ptr(), out.data_ptr(), B, R, C, _raw_stream(t.device.index) or None)
     if rc:
         raise RuntimeError(f"torch_int._hip_ext.transpose_last2: {_lib.ti_last_error().decode()} (status {rc})")
+    return out
+
+
+def can_bmm_rowmajor(a, b):
+    return (_ok(a, torch.int8) and _ok(b, torch.int8) and a.dim() == 3 and b.dim() == 3 and a.device == b.device
+            and a.shape[0] == b.shape[0] and a.shape[2] == b.shape[1] and a.shape[0] <= 65535)
+
+
+def bmm_s8t_s8t_s8t(a, b, alpha):
+    """int8 a [B, M, K], int8 b [B, K, N] (row-major, *not* transposed) -> int8
+    ``clamp(round(alpha * a @ b), -128, 127)`` [B, M, N].  Streams b once per 16 rows of a."""
+    if not can_bmm_rowmajor(a, b):
+        raise RuntimeError("torch_int._hip_ext.bmm_s8t_s8t_s8t: needs contiguous int8 HIP tensors a [B,M,K], b [B,K,N]")
+    B, M, K = a.shape
+    N = b.shape[2]
+    out = torch.empty((B, M, N), dtype=torch.int8, device=a.device)
+    with torch.cuda.device(a.device):
+        rc = _lib.ti_bmm_s8t_s8t_s8t(a.data_ptr(), b.data_ptr(), out.data_ptr(), B, M, N, K, float(alpha),
+                                     _raw_stream(a.device.index) or None)
+    if rc:
+        raise RuntimeError(f"torch_int._hip_ext.bmm_s8t_s8t_s8t: {_lib.ti_last_error().decode()} (status {rc})")
     return out

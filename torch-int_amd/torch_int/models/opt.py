@@ -123,9 +123,12 @@ class Int8OPTAttention(nn.Module):
             # returned view holds round(127 p), which is what upstream returns too
             # (models/opt.py:166-178).
             probs_q = probs.mul_(127).round_().to(torch.int8)
-        # P.V with V transposed to [bsz*H, d, src]: (P V) = P . (V^T)^T
-        value_t = _hip_ext.transpose_last2(value)
-        ctx = self.pv_bmm(probs_q, value_t)  # int8 [bsz*H, tgt, d]
+        if tgt_len <= 16 and type(self.pv_bmm) is BMM_S8T_S8N_S8T and _hip_ext.can_bmm_rowmajor(probs_q, value):
+            # few query rows (incremental decoding): stream V once, as the cache stores it
+            ctx = _hip_ext.bmm_s8t_s8t_s8t(probs_q, value, self.pv_bmm._scalar("a"))
+        else:
+            # P.V with V transposed to [bsz*H, d, src]: (P V) = P . (V^T)^T
+            ctx = self.pv_bmm(probs_q, _hip_ext.transpose_last2(value))  # int8 [bsz*H, tgt, d]
         if ctx.size() != (bsz * H, tgt_len, d):
             raise ValueError(f"`attn_output` should be of size {(bsz, H, tgt_len, d)}, but is {ctx.size()}")
         ctx = _hip_ext.merge_heads(ctx, bsz, H, tgt_len, d)
