@@ -9,10 +9,16 @@ divided by the wall time of a step, in TOPS.
 
 Also reported on the same JSON line:
   roofline      the MFMA-bound part of the sweep (M >= 2048): ops per launch / mean launch
-                duration measured with HIP events on the launch stream, against 5.0 POP/s;
+                duration, against 5.0 POP/s.  The top-level figures come from HIP events
+                recorded around those launches inside the timed steps; `sustained` repeats
+                the measurement with the reference's own protocol (benchmark/utils.py:81-96:
+                100 warm-up launches, then a window of at least 200 ms of back-to-back
+                launches of one case), where the clock has settled under the power limit;
   cpu_baseline  the reference's CPU integer emulation (torch int32 matmul + the fp32
                 epilogue) timed on this box's host cores on a bounded sample;
-  cases         per-case microseconds, TOPS, GB/s and the binding roofline;
+  cases         per-case microseconds (sustained protocol; the HBM-bound cases rotate
+                through enough weight copies to defeat the 256 MB last-level cache), TOPS,
+                GB/s and the binding roofline;
   hbm_kernels   attention BMMs and dq_add_layernorm_q against the 8 TB/s HBM roofline;
   decoder_layer_ms   Int8OPTDecoderLayer at OPT-13B shape (batch 4, seq 512).
 """
@@ -64,28 +70,37 @@ def build_sweep(torch, C, dev):
             for v in VARIANTS:
                 alpha = float(torch.empty(1).uniform_(1e-4, 1e-2, generator=g))
                 beta = float(torch.empty(1).uniform_(1e-4, 1e-2, generator=g))
-                if v == "b32_o32":
-                    fn = (lambda x=x, w=w, b=bias[v]: C.linear_a8_w8_b32_o32(x, w, b))
-                elif v == "bfp32_ofp32":
-                    fn = (lambda x=x, w=w, b=bias[v], a=alpha, be=beta: C.linear_a8_w8_bfp32_ofp32(x, w, b, a, be))
-                elif v == "b8_o8":
-                    fn = (lambda x=x, w=w, b=bias[v], a=alpha, be=beta: C.linear_a8_w8_b8_o8(x, w, b, a, be))
-                else:
-                    fn = (lambda x=x, w=w, b=bias[v], a=alpha, be=beta: C.linear_relu_a8_w8_b8_o8(x, w, b, a, be))
-                cases.append({"variant": v, "M": M, "N": N, "K": K, "fn": fn,
+                def make(w, v=v, x=x, b=bias[v], a=alpha, be=beta):
+                    if v == "b32_o32":
+                        return lambda: C.linear_a8_w8_b32_o32(x, w, b)
+                    if v == "bfp32_ofp32":
+                        return lambda: C.linear_a8_w8_bfp32_ofp32(x, w, b, a, be)
+                    if v == "b8_o8":
+                        return lambda: C.linear_a8_w8_b8_o8(x, w, b, a, be)
+                    return lambda: C.linear_relu_a8_w8_b8_o8(x, w, b, a, be)
+                cases.append({"variant": v, "M": M, "N": N, "K": K, "fn": make(w), "make": make, "w": w,
                               "ops": 2.0 * M * N * K, "bytes": float(gemm_bytes(M, N, K, v))})
     return cases
 
 
-def event_time_ms(torch, fn, iters, warm=2):
-    """Mean duration of fn() in ms, HIP events on the current (launch) stream."""
-    for _ in range(warm):
-        fn()
+def sustained_ms(torch, fns, window_ms=200.0, warm_launches=100):
+    """Mean launch duration in ms under upstream's protocol (benchmark/utils.py:81-96): 100 warm-up
+    launches, then back-to-back launches between two HIP events on the launch stream, enough of them
+    to fill `window_ms`.  `fns` is a list of equivalent closures (e.g. one per weight copy) used round-robin."""
+    n = len(fns)
+    for i in range(warm_launches):
+        fns[i % n]()
     start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    torch.cuda.synchronize()
     start.record()
-    for _ in range(iters):
-        fn()
+    for i in range(10):
+        fns[i % n]()
+    end.record()
+    torch.cuda.synchronize()
+    est = max(start.elapsed_time(end) / 10, 1e-3)
+    iters = max(20, int(window_ms / est) + 1)
+    start.record()
+    for i in range(iters):
+        fns[i % n]()
     end.record()
     torch.cuda.synchronize()
     return start.elapsed_time(end) / iters
@@ -115,18 +130,27 @@ def cpu_baseline(torch):
 
 
 def hbm_kernels(torch, C, dev):
+    """Attention products and LayerNorm-quant against the HBM roofline (algorithmic bytes / duration).
+    Inputs rotate through enough copies (> 256 MB) that reads cannot be served from the last-level cache."""
     out = []
     g = torch.Generator().manual_seed(1)
+
+    def rot(t, total_bytes):
+        n = max(2, -(-320 * 2 ** 20 // total_bytes))
+        return [t] + [t.clone() for _ in range(n - 1)]
+
     for S in (512,):
         q = torch.randint(-127, 128, (160, S, 128), dtype=torch.int8, generator=g).to(dev)
         k = torch.randint(-127, 128, (160, S, 128), dtype=torch.int8, generator=g).to(dev)
         p = torch.randint(0, 128, (160, S, S), dtype=torch.int8, generator=g).to(dev)
         vt = torch.randint(-127, 128, (160, 128, S), dtype=torch.int8, generator=g).to(dev)
-        ms = event_time_ms(torch, lambda: C.bmm_s8t_s8n_f32t(q, k, 0.002), 50)
+        ks = rot(k, 2 * k.numel())
+        ms = sustained_ms(torch, [lambda k=k: C.bmm_s8t_s8n_f32t(q, k, 0.002) for k in ks], window_ms=60.0)
         by = 160.0 * (2 * S * 128 + 4 * S * S)
         out.append({"kernel": "bmm_s8t_s8n_f32t", "shape": [160, S, S, 128], "us": ms * 1e3,
                     "GBps": by / ms / 1e6, "frac": by / ms / 1e6 / PEAK_HBM_GBS})
-        ms = event_time_ms(torch, lambda: C.bmm_s8t_s8n_s8t(p, vt, 0.002), 50)
+        ps = rot(p, p.numel())
+        ms = sustained_ms(torch, [lambda p=p: C.bmm_s8t_s8n_s8t(p, vt, 0.002) for p in ps], window_ms=60.0)
         by = 160.0 * (S * S + 128 * S + S * 128)
         out.append({"kernel": "bmm_s8t_s8n_s8t", "shape": [160, S, 128, S], "us": ms * 1e3,
                     "GBps": by / ms / 1e6, "frac": by / ms / 1e6 / PEAK_HBM_GBS})
@@ -134,7 +158,9 @@ def hbm_kernels(torch, C, dev):
     inp = torch.randint(-65536, 65536, (rows, H), dtype=torch.int32, generator=g).to(dev)
     res = torch.randn(rows, H, generator=g).to(dev)
     gamma, beta = torch.ones(H, device=dev), torch.zeros(H, device=dev)
-    ms = event_time_ms(torch, lambda: C.dq_add_layernorm_q(inp, 0.01, res, gamma, beta, 1e-5), 100)
+    pairs = list(zip(rot(inp, 8 * inp.numel()), rot(res, 8 * res.numel())))
+    ms = sustained_ms(torch, [lambda i=i, r=r: C.dq_add_layernorm_q(i, 0.01, r, gamma, beta, 1e-5) for i, r in pairs],
+                      window_ms=60.0)
     by = 13.0 * rows * H + 8 * H
     out.append({"kernel": "dq_add_layernorm_q", "shape": [rows, H], "us": ms * 1e3,
                 "GBps": by / ms / 1e6, "frac": by / ms / 1e6 / PEAK_HBM_GBS})
@@ -160,7 +186,7 @@ def decoder_layer_ms(torch, dev):
     mask = torch.zeros(T, T, device=dev).masked_fill(
         torch.triu(torch.ones(T, T, dtype=torch.bool, device=dev), 1), torch.finfo(torch.float32).min)
     mask = mask[None, None].expand(B, 1, T, T).contiguous()
-    return event_time_ms(torch, lambda: layer(hidden.clone(), attention_mask=mask), 10)
+    return sustained_ms(torch, [lambda: layer(hidden.clone(), attention_mask=mask)], window_ms=300.0, warm_launches=20)
 
 
 def main():
@@ -184,18 +210,31 @@ def main():
     cases = build_sweep(torch, C, dev)
     sweep_ops = sum(c["ops"] for c in cases)
 
-    def step():
+    heavy = [i for i, c in enumerate(cases) if c["M"] >= 2048]   # the MFMA-bound launches
+    marks = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in heavy]
+             for _ in range(args.steps)]
+
+    def step(ev=None):
+        k = 0
         for c in cases:
-            c["fn"]()
+            if ev is not None and c["M"] >= 2048:
+                ev[k][0].record()
+                c["fn"]()
+                ev[k][1].record()
+                k += 1
+            else:
+                c["fn"]()
 
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
+    for i in range(args.steps):
+        step(marks[i])
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    heavy_ms = sum(a.elapsed_time(b) for ev in marks for (a, b) in ev) / max(args.steps, 1)   # per step
+    heavy_ops = sum(cases[i]["ops"] for i in heavy)
     value = sweep_ops / (ms_per_step * 1e-3) / 1e12
 
     result = {
@@ -208,30 +247,42 @@ def main():
                    "launches_per_step": len(cases), "ops_per_step": sweep_ops},
     }
 
+    in_sweep = heavy_ops / heavy_ms / 1e9
+    result["roofline"] = {
+        "bound": "mfma", "achieved": in_sweep, "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
+        "frac": in_sweep / PEAK_INT8_TOPS, "traffic": TRAFFIC_NOTE,
+        "kernel": "gemm_pipe_kernel<256x256x64, 4 stages> and its 256x160 sibling (all M>=2048 cases of the sweep)",
+        "ops_per_launch": heavy_ops / len(heavy), "avg_launch_ms": heavy_ms / len(heavy), "launches": len(heavy),
+        "protocol": "HIP events around each M>=2048 launch inside the timed steps"}
+
     if not args.sweep_only:
-        # per-case launch durations (HIP events on the launch stream)
+        # per-case launch durations, upstream's protocol; HBM-bound cases rotate weight copies (> 256 MB in total)
         table = []
         mfma_ops = mfma_ms = 0.0
-        n_mfma = 0
+        copies = {}
         for c in cases:
-            iters = 20 if c["M"] >= 2048 else 50
-            ms = event_time_ms(torch, c["fn"], iters)
+            bound = "mfma" if c["M"] >= 2048 else "hbm"
+            fns = [c["fn"]]
+            if bound == "hbm":
+                key = (c["N"], c["K"])
+                if key not in copies:
+                    n_copies = -(-320 * 2 ** 20 // (c["N"] * c["K"]))
+                    copies[key] = [c["w"]] + [c["w"].clone() for _ in range(n_copies - 1)]
+                fns = [c["make"](w) for w in copies[key]]
+            ms = sustained_ms(torch, fns, window_ms=200.0 if bound == "mfma" else 60.0)
             tops = c["ops"] / ms / 1e9
             gbs = c["bytes"] / ms / 1e6
-            bound = "mfma" if c["M"] >= 2048 else "hbm"
             frac = tops / PEAK_INT8_TOPS if bound == "mfma" else gbs / PEAK_HBM_GBS
             table.append({"variant": c["variant"], "M": c["M"], "N": c["N"], "K": c["K"], "us": round(ms * 1e3, 2),
                           "TOPS": round(tops, 1), "GBps": round(gbs, 1), "bound": bound, "frac": round(frac, 4)})
             if bound == "mfma":
                 mfma_ops += c["ops"]
                 mfma_ms += ms
-                n_mfma += 1
-        achieved = mfma_ops / mfma_ms / 1e9
-        result["roofline"] = {
-            "bound": "mfma", "achieved": achieved, "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
-            "frac": achieved / PEAK_INT8_TOPS, "traffic": TRAFFIC_NOTE,
-            "kernel": "gemm_pipe_kernel<256x256x64, 4 stages> (all M>=2048 cases of the sweep)",
-            "ops_per_launch": mfma_ops / n_mfma, "avg_launch_ms": mfma_ms / n_mfma, "launches": n_mfma}
+        del copies
+        sustained = mfma_ops / mfma_ms / 1e9
+        result["roofline"]["sustained"] = {
+            "achieved": sustained, "frac": sustained / PEAK_INT8_TOPS, "avg_launch_ms": mfma_ms / len(heavy),
+            "protocol": "per case: 100 warm-up launches, then >= 200 ms of back-to-back launches between two HIP events"}
         result["cases"] = table
         result["hbm_kernels"] = hbm_kernels(torch, C, dev)
         result["decoder_layer_ms"] = decoder_layer_ms(torch, dev)

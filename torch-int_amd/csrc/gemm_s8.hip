@@ -1161,28 +1161,42 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmParams p, const 
   }
 }
 
-// Number of K slices for an (M,N,K) linear on this chip; 1 = do not split.  A small cost
-// model: chip time of the GEMM at the utilisation the tile count allows, plus the time
-// to write and re-read the int32 partial tiles.
-static int choose_splits(long long M, long long N, long long K) {
+// Number of K slices for an (M,N,K) linear on this chip (1 = do not split) and the tile edge
+// (128 or 256) of the raw-int32 GEMM that computes the slices.  A small cost model fitted to
+// measurements at OPT-13B/66B widths with cache-cold weights: a 256x256 workgroup takes about
+// 0.85 us per K step with a CU to itself; a 128x128 workgroup 0.35 us alone and 0.70 us when two
+// share a CU; 8 us per round for pipeline fill and epilogue; the int32 partial tiles are written
+// once and read once (they mostly stay in the last-level cache), plus the second launch.
+static int choose_splits(long long M, long long N, long long K, int* tile_edge = nullptr) {
+  if (tile_edge) *tile_edge = 128;
   if (M <= 16 || M > 1024 || K % PBK != 0 || K < 1024) return 1;
-  const double slots = num_cus();  // one 128x128 workgroup per CU already gets most of a CU's rate
-  const double tiles = (double)((M + 127) / 128) * (double)((N + 127) / 128);
-  const double ops = 2.0 * M * N * K, bytes = (double)K * (M + N);
-  const double t0 = ops / 2.0e15 > bytes / 5.0e12 ? ops / 2.0e15 : bytes / 5.0e12;
+  const double cus = num_cus();
   const long long steps = K / PBK;
-  int best = 1;
+  int best = 1, best_edge = 128;
   double best_t = 1e30;
-  for (int s = 1; s <= 16; ++s) {
-    if (steps % s != 0 || steps / s < 4) continue;
-    const double util = tiles * s / slots < 1.0 ? tiles * s / slots : 1.0;
-    double t = t0 / util;
-    if (s > 1) t += 2.0 * s * M * N * 4.0 / 4.0e12 + 3.0e-6;
-    if (t < best_t * 0.97) {  // prefer fewer slices unless the gain is clear
-      best_t = t;
-      best = s;
+  for (int edge = 128; edge <= 256; edge += 128) {
+    const double tiles = (double)((M + edge - 1) / edge) * (double)((N + edge - 1) / edge);
+    for (int s = 1; s <= 16; ++s) {
+      if (steps % s != 0 || steps / s < 4) continue;
+      const double wgs = tiles * s;
+      double rounds, step_us;
+      if (edge == 256) {
+        rounds = (double)(long long)((wgs + cus - 1) / cus);
+        step_us = 0.85;
+      } else {
+        rounds = (double)(long long)((wgs + 2 * cus - 1) / (2 * cus));
+        step_us = wgs <= cus ? 0.35 : 0.70;
+      }
+      double t = rounds * ((double)(steps / s) * step_us + 8.0);
+      if (s > 1) t += (double)(s + 1) * M * N * 4.0 / 8.0e6 + 3.0;  // bytes / (8 TB/s) in us
+      if (t < best_t * 0.97) {  // prefer fewer slices and the smaller tile unless the gain is clear
+        best_t = t;
+        best = s;
+        best_edge = edge;
+      }
     }
   }
+  if (tile_edge) *tile_edge = best_edge;
   return best;
 }
 
@@ -1245,7 +1259,8 @@ static int launch_kind(const GemmParams& p, void* workspace, long long workspace
     return TI_OK;
   }
   if (p.batch == 1 && p.lda == p.K && p.ldb == p.K) {
-    const int splits = choose_splits(p.M, p.N, p.K);
+    int edge = 128;
+    const int splits = choose_splits(p.M, p.N, p.K, &edge);
     const long long need = (long long)splits * p.M * p.N * 4;
     if (splits > 1 && workspace != nullptr && workspace_bytes >= need &&
         (reinterpret_cast<uintptr_t>(workspace) & 15) == 0) {
@@ -1257,7 +1272,9 @@ static int launch_kind(const GemmParams& p, void* workspace, long long workspace
       q.strideC = (long long)p.M * p.N;
       q.C = workspace;
       q.bias = nullptr;
-      if (int rc = launch_pipe<PipeCfg<128, 128, 2, 2, 4, EPI_S32_RAW, false>>(q, stream)) return rc;
+      if (int rc = edge == 256 ? launch_pipe<PipeCfg<256, 256, 2, 4, 4, EPI_S32_RAW, false>>(q, stream)
+                               : launch_pipe<PipeCfg<128, 128, 2, 2, 4, EPI_S32_RAW, false>>(q, stream))
+        return rc;
       const long long quads = ((long long)p.M * p.N + 3) / 4;
       hipLaunchKernelGGL(splitk_reduce_kernel<KIND>, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream, p,
                          static_cast<const int*>(workspace), splits);
