@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Headline benchmark: the W8A8 linear-kernel sweep at OPT-13B shapes on one MI355X.
 
-One "step" is one pass over BASELINE config 2: (N,K) in {(5120,5120), (20480,5120),
+One "step" is one pass over the linear-kernel sweep: (N,K) in {(5120,5120), (20480,5120),
 (5120,20480)} x M in {1,16,128,512,2048,8192} x the four variants (s32 bias/out, fp32
 bias/out, s8 bias/out, fused-ReLU s8 out) = 72 GEMM launches on synthetic int8 data that
 is resident in HBM before the clock starts.  `value` = 2*M*N*K summed over the sweep,
@@ -23,6 +23,7 @@ Also reported on the same JSON line:
   decoder_layer_ms   Int8OPTDecoderLayer at OPT-13B shape (batch 4, seq 512).
 """
 import argparse
+import ctypes
 import json
 import os
 import sys
@@ -35,10 +36,12 @@ for _p in (os.path.join(ROOT, "torch-int_amd"), ROOT):
 
 PEAK_INT8_TOPS = 5000.0   # MI355X dense INT8 MFMA, TOP/s
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
-# HBM bytes per launch of the dominant kernel need rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE), which
-# cannot be taken from inside this process; the measured figure is kept in profiles/ (1.44 GB for the
-# 8192x20480x5120 s8 case against 0.31 GB algorithmic).
-TRAFFIC_NOTE = None
+# HBM-side bytes per launch of the dominant kernel come from rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) of
+# this script's own sweep, which cannot be taken from inside the process: 417 768 KiB x 2.000 fetched +
+# 183 193 KiB written per launch, averaged over the 16 launches per step that reach the 256x256 kernel
+# (commands and calibration in profiles/gemm_pipe_256x256_linear_8192x20480x5120.md).
+TRAFFIC_BYTES = 1.043e9
+DOMINANT = "pipe_256x256"
 SHAPES = [(5120, 5120), (20480, 5120), (5120, 20480)]   # (N, K): qkv/out_proj, fc1, fc2
 MS = [1, 16, 128, 512, 2048, 8192]
 VARIANTS = ["b32_o32", "bfp32_ofp32", "b8_o8", "relu_b8_o8"]
@@ -209,6 +212,11 @@ def main():
 
     cases = build_sweep(torch, C, dev)
     sweep_ops = sum(c["ops"] for c in cases)
+    C._lib.ti_last_kernel.restype = ctypes.c_char_p
+    for c in cases:   # one untimed call each: which kernel family does the library pick for this case?
+        c["fn"]()
+        c["kernel"] = C._lib.ti_last_kernel().decode()
+    torch.cuda.synchronize()
 
     heavy = [i for i, c in enumerate(cases) if c["M"] >= 2048]   # the MFMA-bound launches
     marks = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in heavy]
@@ -235,6 +243,10 @@ def main():
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
     heavy_ms = sum(a.elapsed_time(b) for ev in marks for (a, b) in ev) / max(args.steps, 1)   # per step
     heavy_ops = sum(cases[i]["ops"] for i in heavy)
+    # the dominant kernel: the 256x256 pipelined GEMM (whatever cases the library routes to it)
+    dom = [k for k, i in enumerate(heavy) if cases[i]["kernel"] == DOMINANT]
+    dom_ms = sum(ev[k][0].elapsed_time(ev[k][1]) for ev in marks for k in dom) / max(args.steps, 1)
+    dom_ops = sum(cases[heavy[k]]["ops"] for k in dom)
     value = sweep_ops / (ms_per_step * 1e-3) / 1e12
 
     result = {
@@ -247,13 +259,16 @@ def main():
                    "launches_per_step": len(cases), "ops_per_step": sweep_ops},
     }
 
-    in_sweep = heavy_ops / heavy_ms / 1e9
+    achieved = dom_ops / dom_ms / 1e9
     result["roofline"] = {
-        "bound": "mfma", "achieved": in_sweep, "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
-        "frac": in_sweep / PEAK_INT8_TOPS, "traffic": TRAFFIC_NOTE,
-        "kernel": "gemm_pipe_kernel<256x256x64, 4 stages> and its 256x160 sibling (all M>=2048 cases of the sweep)",
-        "ops_per_launch": heavy_ops / len(heavy), "avg_launch_ms": heavy_ms / len(heavy), "launches": len(heavy),
-        "protocol": "HIP events around each M>=2048 launch inside the timed steps"}
+        "bound": "mfma", "achieved": achieved, "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
+        "frac": achieved / PEAK_INT8_TOPS, "traffic": TRAFFIC_BYTES,
+        "kernel": "gemm_pipe_kernel<PipeCfg<256,256,2,4,4,KIND,...>> (the sweep cases the library routes to it: "
+                  + ", ".join(sorted({f"{cases[heavy[k]]['M']}x{cases[heavy[k]]['N']}x{cases[heavy[k]]['K']}" for k in dom})) + ")",
+        "ops_per_launch": dom_ops / len(dom), "avg_launch_ms": dom_ms / len(dom), "launches_per_step": len(dom),
+        "protocol": "HIP events around each of these launches inside the timed steps",
+        "all_mfma_bound_cases": {"achieved": heavy_ops / heavy_ms / 1e9, "frac": heavy_ops / heavy_ms / 1e9 / PEAK_INT8_TOPS,
+                                 "launches_per_step": len(heavy), "avg_launch_ms": heavy_ms / len(heavy)}}
 
     if not args.sweep_only:
         # per-case launch durations, upstream's protocol; HBM-bound cases rotate weight copies (> 256 MB in total)
@@ -273,16 +288,18 @@ def main():
             tops = c["ops"] / ms / 1e9
             gbs = c["bytes"] / ms / 1e6
             frac = tops / PEAK_INT8_TOPS if bound == "mfma" else gbs / PEAK_HBM_GBS
-            table.append({"variant": c["variant"], "M": c["M"], "N": c["N"], "K": c["K"], "us": round(ms * 1e3, 2),
+            table.append({"variant": c["variant"], "M": c["M"], "N": c["N"], "K": c["K"], "kernel": c["kernel"],
+                          "us": round(ms * 1e3, 2),
                           "TOPS": round(tops, 1), "GBps": round(gbs, 1), "bound": bound, "frac": round(frac, 4)})
-            if bound == "mfma":
+            if c["kernel"] == DOMINANT and bound == "mfma":
                 mfma_ops += c["ops"]
                 mfma_ms += ms
         del copies
         sustained = mfma_ops / mfma_ms / 1e9
         result["roofline"]["sustained"] = {
-            "achieved": sustained, "frac": sustained / PEAK_INT8_TOPS, "avg_launch_ms": mfma_ms / len(heavy),
-            "protocol": "per case: 100 warm-up launches, then >= 200 ms of back-to-back launches between two HIP events"}
+            "achieved": sustained, "frac": sustained / PEAK_INT8_TOPS, "avg_launch_ms": mfma_ms / len(dom),
+            "protocol": "same cases, each alone: 100 warm-up launches, then >= 200 ms of back-to-back launches "
+                        "between two HIP events (upstream benchmark/utils.py:81-96)"}
         result["cases"] = table
         result["hbm_kernels"] = hbm_kernels(torch, C, dev)
         result["decoder_layer_ms"] = decoder_layer_ms(torch, dev)

@@ -53,6 +53,11 @@ int ti_init(void);
  * smaller or NULL workspace is always legal and only selects a non-split kernel. */
 int64_t ti_linear_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
+/* Diagnostics: the kernel family the calling thread's last linear / bmm_s8t_s8n_* call launched
+ * ("pipe_256x256", "pipe16_256x160", "pipe_128x128", "splitk_256x256", "splitk_128x128", "stream",
+ * "skinny", "tile_*", "scalar"; "" before the first call).  Benchmarks use it to label their rows. */
+const char* ti_last_kernel(void);
+
 /* ---- W8A8 linear: out[M,N] = epilogue(x[M,K] . w[N,K]^T, bias[N]) ---- */
 
 /* replaces linear_a8_w8_b32_o32 (torch_int/kernels/linear.cu:13-136;

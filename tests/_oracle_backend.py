@@ -41,7 +41,7 @@ def oracle_backend(fast_matmul=False):
 
 
 def randomize_int8_layer(layer, gen, scale_lo=1e-4, scale_hi=1e-2):
-    """BASELINE config 4 initialisation of an Int8OPTDecoderLayer: int8 weights and biases
+    """Decoder-layer benchmark initialisation of an Int8OPTDecoderLayer: int8 weights and biases
     uniform in [-127,127], fp32 biases ~N(0,1), per-tensor scales ~U(lo,hi), LayerNorm
     gamma ~N(1,0.02), beta ~N(0,0.02)."""
     def u():

@@ -137,7 +137,7 @@ def test_split_k_matches_unsplit_through_the_c_abi():
 
 
 def test_linear_opt125m_config():
-    # BASELINE config 1: x [4,512,768], W [768,768], bias [768], alpha 1e-3, beta 1e-2, seed 0
+    # the single-linear benchmark configuration at OPT-125m width: x [4,512,768], W [768,768], bias [768], alpha 1e-3, beta 1e-2, seed 0
     import torch_int._CUDA as C
     _say("linear C1")
     out = _linear_case(C, "b8_o8", 2048, 768, 768, seed=0, alpha=0.001, beta=0.01)
@@ -246,7 +246,7 @@ def test_bmm_literal_fixture_from_upstream_tests():
 
 @pytest.mark.parametrize("S", [128, 512])
 def test_bmm_attention_config(S):
-    # BASELINE config 3 at a reduced batch*heads (the full 160 is covered by properties below)
+    # the attention-product benchmark configuration at a reduced batch*heads (the full 160 is covered by properties below)
     import torch_int._CUDA as C
     BH, d = 8, 128
     _say(f"attention bmm S={S}")
@@ -255,7 +255,7 @@ def test_bmm_attention_config(S):
 
 
 def test_bmm_full_size_properties():
-    # B*H = 160, S = 512, d = 128 (BASELINE config 3): size-independent checks
+    # B*H = 160, S = 512, d = 128 (the attention-product benchmark configuration): size-independent checks
     import torch_int._CUDA as C
     g = torch.Generator().manual_seed(9)
     BH, S, d = 160, 512, 128

@@ -34,7 +34,7 @@ def _rel_err(a, b):
 @torch.no_grad()
 def test_linear_and_bmm_modules_on_gpu():
     g = torch.Generator().manual_seed(0)
-    x = torch.randint(-127, 128, (4, 512, 768), dtype=torch.int8, generator=g)  # BASELINE config 1 input
+    x = torch.randint(-127, 128, (4, 512, 768), dtype=torch.int8, generator=g)  # the OPT-125m single-linear benchmark input
     for cls in (W8A8B8O8Linear, W8A8B8O8LinearReLU, W8A8B32O32Linear, W8A8B32O32LinearWithoutScaling,
                 W8A8BFP32OFP32Linear):
         _say("module", cls.__name__)
@@ -110,7 +110,7 @@ def _capture(layer):
 
 @torch.no_grad()
 def test_decoder_layer_opt13b_shape():
-    """BASELINE config 4: hidden 5120, 40 heads, FFN 20480, batch 4, seq 512, causal mask.
+    """The decoder-layer benchmark configuration: hidden 5120, 40 heads, FFN 20480, batch 4, seq 512, causal mask.
 
     With per-tensor scales drawn from U(1e-4, 1e-2) nearly every int8 activation saturates,
     so the layer as a whole amplifies a one-LSB difference after the fp32 softmax/LayerNorm

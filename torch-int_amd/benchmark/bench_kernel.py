@@ -5,6 +5,9 @@ Examples
   python torch-int_amd/benchmark/bench_kernel.py --op linear_b8_o8 --shape 8192 20480 5120
   python torch-int_amd/benchmark/bench_kernel.py --op bmm_f32t --shape 160 512 512 128
   python torch-int_amd/benchmark/bench_kernel.py --op ln_q --shape 2048 5120
+  python torch-int_amd/benchmark/bench_kernel.py --op softmax_q --shape 4 40 512 512        # batch heads T S
+  python torch-int_amd/benchmark/bench_kernel.py --op bmm_s8t_rowmajor --shape 288 1 128 544
+  python torch-int_amd/benchmark/bench_kernel.py --op linear_b8_o8 --shape 1 20480 5120 --rotate 4   # cache-cold weights
   python torch-int_amd/benchmark/bench_kernel.py --op copy --shape 268435456      # bytes; counter calibration
   rocprofv3 --kernel-trace --stats --output-format csv -d out -- python3 .../bench_kernel.py --op ...
 
@@ -21,6 +24,7 @@ sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), ".."
 
 import torch  # noqa: E402
 import torch_int._CUDA as C  # noqa: E402
+import torch_int._hip_ext as X  # noqa: E402
 
 LINEAR = {
     "linear_b32_o32": (torch.int32, 4, 4),
@@ -33,12 +37,15 @@ LINEAR = {
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--op", required=True, choices=list(LINEAR) + ["bmm_f32t", "bmm_s8t", "bmm_s32t", "ln_q", "copy"])
+    ap.add_argument("--op", required=True, choices=list(LINEAR) + ["bmm_f32t", "bmm_s8t", "bmm_s32t", "bmm_s8t_rowmajor", "ln_q", "add_ln_q",
+                                               "softmax_q", "copy"])
     ap.add_argument("--shape", type=int, nargs="+", required=True)
     ap.add_argument("--iters", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--alpha", type=float, default=0.001)
     ap.add_argument("--beta", type=float, default=0.01)
+    ap.add_argument("--rotate", type=int, default=1,
+                    help="copies of the large read-only operand used round-robin (defeats the 256 MB last-level cache)")
     args = ap.parse_args()
     dev = torch.device("cuda:0")
     g = torch.Generator(device=dev).manual_seed(0)
@@ -50,7 +57,8 @@ def main():
     if args.op in LINEAR:
         M, N, K = args.shape
         bdt, bb, ob = LINEAR[args.op]
-        x, w = s8(M, K), s8(N, K)
+        x, ws = s8(M, K), [s8(N, K) for _ in range(args.rotate)]
+        w = ws[0]
         bias = torch.randn(N, device=dev, generator=g) if bdt == torch.float32 else \
             torch.randint(-127, 128, (N,), device=dev, generator=g).to(bdt)
         fn = {"linear_b32_o32": lambda: C.linear_a8_w8_b32_o32(x, w, bias),
@@ -59,6 +67,19 @@ def main():
               "linear_b8_o8": lambda: C.linear_a8_w8_b8_o8(x, w, bias, args.alpha, args.beta),
               "linear_relu_b8_o8": lambda: C.linear_relu_a8_w8_b8_o8(x, w, bias, args.alpha, args.beta)}[args.op]
         ops, nbytes = 2.0 * M * N * K, M * K + N * K + N * bb + M * N * ob
+        if args.rotate > 1:
+            variants, kind = [], args.op
+            for w in ws:
+                variants.append({"linear_b32_o32": lambda w=w: C.linear_a8_w8_b32_o32(x, w, bias),
+                                 "linear_b32_o32_scaled": lambda w=w: C.linear_a8_w8_b32_o32_with_scaling(x, w, bias, args.alpha, args.beta),
+                                 "linear_bfp32_ofp32": lambda w=w: C.linear_a8_w8_bfp32_ofp32(x, w, bias, args.alpha, 1.0),
+                                 "linear_b8_o8": lambda w=w: C.linear_a8_w8_b8_o8(x, w, bias, args.alpha, args.beta),
+                                 "linear_relu_b8_o8": lambda w=w: C.linear_relu_a8_w8_b8_o8(x, w, bias, args.alpha, args.beta)}[kind])
+            state = {"i": 0}
+
+            def fn():
+                state["i"] = (state["i"] + 1) % len(variants)
+                return variants[state["i"]]()
     elif args.op.startswith("bmm"):
         B, M, N, K = args.shape
         a, b = s8(B, M, K, lo=0 if args.op == "bmm_s8t" else -127), s8(B, N, K)
@@ -66,6 +87,26 @@ def main():
               "bmm_s8t": lambda: C.bmm_s8t_s8n_s8t(a, b, args.alpha),
               "bmm_s32t": lambda: C.bmm_s8t_s8n_s32t(a, b)}[args.op]
         ops, nbytes = 2.0 * B * M * N * K, B * (M * K + N * K + M * N * (1 if args.op == "bmm_s8t" else 4))
+    elif args.op == "bmm_s8t_rowmajor":
+        B, M, N, K = args.shape
+        a, b = s8(B, M, K, lo=0), s8(B, K, N)
+        fn = lambda: X.bmm_s8t_s8t_s8t(a, b, args.alpha)  # noqa: E731
+        ops, nbytes = 2.0 * B * M * N * K, B * (M * K + N * K + M * N)
+    elif args.op == "softmax_q":
+        batch, heads, T, S = args.shape
+        scores = torch.randn(batch * heads, T, S, device=dev, generator=g) * 4
+        mask = torch.zeros(T, S, device=dev).masked_fill(
+            torch.triu(torch.ones(T, S, dtype=torch.bool, device=dev), 1 + S - T), torch.finfo(torch.float32).min)
+        mask = mask[None, None].expand(batch, 1, T, S).contiguous()
+        fn = lambda: X.attn_softmax_q(scores, mask, heads)  # noqa: E731
+        nbytes = 5.0 * batch * heads * T * S + 4.0 * batch * T * S
+    elif args.op == "add_ln_q":
+        rows, H = args.shape
+        x = torch.randn(rows, H, device=dev, generator=g)
+        res = torch.randn(rows, H, device=dev, generator=g)
+        gamma, beta = torch.ones(H, device=dev), torch.zeros(H, device=dev)
+        fn = lambda: X.add_layernorm_q(x, res, gamma, beta, 1e-5)  # noqa: E731
+        nbytes = 13.0 * rows * H + 8 * H
     elif args.op == "ln_q":
         rows, H = args.shape
         inp = torch.randint(-65536, 65536, (rows, H), dtype=torch.int32, device=dev, generator=g)

@@ -196,6 +196,8 @@ int ti_attn_softmax_q(const float* scores, const float* mask, int8_t* probs, int
   return launch_attn_softmax_q(scores, mask, probs, batch, heads, T, S, static_cast<hipStream_t>(stream));
 }
 
+const char* ti_last_kernel(void) { return last_gemm_kernel(); }
+
 int ti_bmm_s8t_s8t_s8t(const int8_t* a, const int8_t* b, int8_t* c, int64_t batch, int64_t M, int64_t N, int64_t K,
                        float alpha, void* stream) {
   g_err[0] = 0;

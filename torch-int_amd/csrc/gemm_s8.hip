@@ -1205,6 +1205,9 @@ long long gemm_workspace_bytes(long long M, long long N, long long K) {
   return s > 1 ? (long long)s * M * N * 4 : 0;
 }
 
+static thread_local const char* g_last_kernel = "";
+const char* last_gemm_kernel() { return g_last_kernel; }
+
 template <int KIND>
 static int launch_kind(const GemmParams& p, void* workspace, long long workspace_bytes, hipStream_t stream) {
   using Out = typename Epi<KIND>::Out;
@@ -1212,6 +1215,7 @@ static int launch_kind(const GemmParams& p, void* workspace, long long workspace
                        ((reinterpret_cast<uintptr_t>(p.B) & 15) == 0) &&
                        (p.strideA % 16 == 0) && (p.strideB % 16 == 0);  // the stores check C themselves
   if (!aligned) {
+    g_last_kernel = "scalar";
     const long long total = (long long)p.M * p.N;
     dim3 grid((unsigned)((total + 255) / 256), 1, p.batch);
     hipLaunchKernelGGL(gemm_scalar_kernel<KIND>, grid, dim3(256), 0, stream, p);
@@ -1220,6 +1224,7 @@ static int launch_kind(const GemmParams& p, void* workspace, long long workspace
     return TI_OK;
   }
   if (p.M <= 16 && p.K % SBK == 0 && (long long)((p.N + 15) / 16) * p.batch >= 256) {
+    g_last_kernel = "stream";
     const int spb = (p.N + 15) / 16;
     const long long strips = (long long)spb * p.batch;
     if (strips > 0x7fffffffLL) return fail(TI_ERR_INVALID_ARG, "too many output strips (%lld)", strips);
@@ -1243,6 +1248,7 @@ static int launch_kind(const GemmParams& p, void* workspace, long long workspace
     return launch(gemm_stream_kernel<KIND, 16, 2>, 32, 2);
   }
   if (p.M <= 16) {
+    g_last_kernel = "skinny";
     const int nw = skinny_waves(p);
     dim3 grid((p.N + 15) / 16, 1, p.batch);
     const size_t lds = (size_t)(nw - 1) * 256 * sizeof(int);
@@ -1264,6 +1270,7 @@ static int launch_kind(const GemmParams& p, void* workspace, long long workspace
     const long long need = (long long)splits * p.M * p.N * 4;
     if (splits > 1 && workspace != nullptr && workspace_bytes >= need &&
         (reinterpret_cast<uintptr_t>(workspace) & 15) == 0) {
+      g_last_kernel = edge == 256 ? "splitk_256x256" : "splitk_128x128";
       GemmParams q = p;  // the K slices are the batches of one raw-int32 GEMM into the workspace
       q.K = p.K / splits;
       q.batch = splits;
@@ -1299,15 +1306,27 @@ static int launch_kind(const GemmParams& p, void* workspace, long long workspace
       const long long t160 = (long long)((p.M + 255) / 256) * ((p.N + 159) / 160) * p.batch;
       const double e256 = (double)t256 / (double)(((t256 + cus - 1) / cus) * cus);
       const double e160 = 0.78 * (double)t160 / (double)(((t160 + cus - 1) / cus) * cus);
-      static const int force = getenv("TI_TILE") ? atoi(getenv("TI_TILE")) : 0;  // experiments: 1 = 256x256, 2 = 256x160
-      if ((p.N % 160 == 0 && e160 > e256 && force != 1) || force == 2)
+      if (p.N % 160 == 0 && e160 > e256) {
+        g_last_kernel = "pipe16_256x160";
         return launch_pipe16<Pipe16Cfg<256, 160, 4, 2, 5, KIND>>(p, stream);
+      }
+      g_last_kernel = "pipe_256x256";
       return launch_pipe<PipeCfg<256, 256, 2, 4, 4, KIND, SWAP>>(p, stream);
     }
-    if (t128 >= 128) return launch_pipe<PipeCfg<128, 128, 2, 2, 4, KIND, SWAP>>(p, stream);
+    if (t128 >= 128) {
+      g_last_kernel = "pipe_128x128";
+      return launch_pipe<PipeCfg<128, 128, 2, 2, 4, KIND, SWAP>>(p, stream);
+    }
   }
-  if (t256 >= 160) return launch_tile<TileCfg<256, 256, 2, 4, KIND, SWAP>>(p, stream);
-  if (t128 >= 128) return launch_tile<TileCfg<128, 128, 2, 2, KIND, SWAP>>(p, stream);
+  if (t256 >= 160) {
+    g_last_kernel = "tile_256x256";
+    return launch_tile<TileCfg<256, 256, 2, 4, KIND, SWAP>>(p, stream);
+  }
+  if (t128 >= 128) {
+    g_last_kernel = "tile_128x128";
+    return launch_tile<TileCfg<128, 128, 2, 2, KIND, SWAP>>(p, stream);
+  }
+  g_last_kernel = "tile_64x64";
   return launch_tile<TileCfg<64, 64, 2, 2, KIND, SWAP>>(p, stream);
 }
 

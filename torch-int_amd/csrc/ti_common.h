@@ -146,6 +146,7 @@ struct GemmParams {
 int launch_gemm(int kind, const GemmParams& p, void* workspace, long long workspace_bytes,
                 hipStream_t stream);
 long long gemm_workspace_bytes(long long M, long long N, long long K);
+const char* last_gemm_kernel();  // kernel family of the calling thread's last launch_gemm ("" before the first)
 
 // ln_q.hip
 int launch_dq_add_layernorm_q(const int32_t* in, float scale, const float* res, const float* gamma,
