@@ -104,6 +104,23 @@ def test_linear_large_tiles(variant):
         _linear_case(C, variant, M, N, K, seed=7)
 
 
+def test_every_gemm_kernel_family_is_reached_and_exact():
+    # one shape per dispatch branch; the library reports which kernel family it launched
+    import ctypes
+    import torch_int._CUDA as C
+    C._lib.ti_last_kernel.restype = ctypes.c_char_p
+    expect = [((2048, 5120, 256), "pipe16_256x160"), ((2000, 9216, 192), "pipe16_256x288"),
+              ((4096, 2816, 128), "pipe_256x256"), ((1024, 2048, 64), "pipe_128x128"),
+              ((1024, 5120, 5120), "splitk_256x256"), ((128, 640, 4096), "splitk_128x128"),
+              ((16, 5120, 3072), "stream"), ((3, 100, 272), "skinny"), ((300, 200, 48), "tile_64x64"),
+              ((2100, 5000, 272), "tile_256x256"), ((1024, 2048, 80), "tile_128x128"), ((70, 50, 37), "scalar")]
+    for (M, N, K), family in expect:
+        for variant in ("b8_o8", "bfp32_ofp32"):
+            _say(f"family {family} {variant} M={M} N={N} K={K}")
+            _linear_case(C, variant, M, N, K, seed=55)
+            assert C._lib.ti_last_kernel().decode() == family, (M, N, K, C._lib.ti_last_kernel())
+
+
 @pytest.mark.parametrize("variant", VARIANTS)
 def test_linear_split_k_and_decode_shapes(variant):
     # few output tiles and a long K: the K loop is split over workgroups (with and without the

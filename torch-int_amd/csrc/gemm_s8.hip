@@ -546,6 +546,10 @@ struct Pipe16Cfg {
   static constexpr int RPW = (BM + BN) / NWAVES;  // panel rows a wave copies per step
   static constexpr int TAIL_ROWS = RPW % 16;
   static constexpr int COPIES = RPW / 16 + (TAIL_ROWS ? 1 : 0);
+  // Registers: 4 per accumulator block, 4 per fragment.  When two full sets of fragments would not fit
+  // next to the accumulators, the weight fragments are kept in one set and reloaded block by block,
+  // each right after the MFMAs that consumed it.
+  static constexpr bool SINGLE_B = 4 * TM * TN + 8 * (TM + TN) >= 224;
   static_assert(WTM % 16 == 0 && WTN % 16 == 0, "wave tile must be made of 16x16 blocks");
   static_assert((BM + BN) % NWAVES == 0 && RPW % 4 == 0, "a wave must copy whole groups of four rows");
   static_assert(LDS_BYTES <= 160 * 1024 && STAGES >= 3, "LDS budget");
@@ -673,9 +677,25 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe16_kernel(GemmParams p, i
     constexpr bool LAST = decltype(last)::value;
     wait_copies_then_barrier<(S - 3) * COPIES>();  // step gs+1 landed; every wave is done with step gs-1
     issue_copies();                                // step gs+S-1 into the stage step gs-1 used
-    if (!LAST) read_frags(gs + 1, fn, fm);
-    mma(fc, fd);
-    if (!LAST) interleave();
+    if constexpr (Cfg::SINGLE_B) {
+      // the weight fragments live in fb0 only (fd / fm are ignored)
+      const char* st = smem + ((gs + 1) % S) * Cfg::STAGE_BYTES;
+      if (!LAST) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fn[i] = *reinterpret_cast<const v4i*>(st + a_frag + i * 16 * PBK);
+      }
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+          acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb0[j], fc[i], acc[i][j], 0, 0, 0);
+        if (!LAST) fb0[j] = *reinterpret_cast<const v4i*>(st + b_frag + j * 16 * PBK);
+      }
+    } else {
+      if (!LAST) read_frags(gs + 1, fn, fm);
+      mma(fc, fd);
+      if (!LAST) interleave();
+    }
     ++gs;
   };
   auto finish_item = [&]() {
@@ -757,8 +777,10 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe16_kernel(GemmParams p, i
       step(fa0, fb0, fa1, fb1, std::false_type{});
 #pragma unroll
       for (int i = 0; i < TM; ++i) fa0[i] = fa1[i];
+      if (!Cfg::SINGLE_B) {
 #pragma unroll
-      for (int j = 0; j < TN; ++j) fb0[j] = fb1[j];
+        for (int j = 0; j < TN; ++j) fb0[j] = fb1[j];
+      }
     }
     if (item_done) step(fa0, fb0, fa1, fb1, std::true_type{});
     kt += n;
@@ -1298,17 +1320,24 @@ static int launch_kind(const GemmParams& p, void* workspace, long long workspace
     // a 256-wide tile on a narrow or short output would mostly multiply padding
     const bool wide = p.N > 128 && p.M > 128;
     if (t256 >= 160 && wide) {
-      // 256x160 tiles (16x16 blocks) when the width allows it and they fill the CUs more evenly.
-      // Measured at full occupancy the 16x16-block kernel reaches 0.78 of the 256x256 kernel's rate
-      // (one barrier per 20 short MFMAs instead of per 16 long ones), so it only pays off when the
-      // 256x256 grid would leave more than a fifth of the CUs idle (e.g. 2048x5120: 160 tiles).
+      // 256x160 or 256x288 tiles (16x16 blocks) when the width allows it and they fill the CUs more
+      // evenly.  Measured at full occupancy the 16x16-block kernel reaches 0.78 (256x160: one barrier
+      // per 20 short MFMAs) or 0.9 (256x288: 36 per barrier) of the 256x256 kernel's rate, so it only
+      // pays off when the 256x256 grid would leave CUs idle (e.g. 2048x5120: 160 tiles of 256x256 but
+      // 256 of 256x160; 2048x9216: 288 tiles of 256x256 = two rounds, but exactly 256 of 256x288).
       const long long cus = num_cus();
-      const long long t160 = (long long)((p.M + 255) / 256) * ((p.N + 159) / 160) * p.batch;
-      const double e256 = (double)t256 / (double)(((t256 + cus - 1) / cus) * cus);
-      const double e160 = 0.78 * (double)t160 / (double)(((t160 + cus - 1) / cus) * cus);
-      if (p.N % 160 == 0 && e160 > e256) {
+      auto fill = [&](long long tiles) { return (double)tiles / (double)(((tiles + cus - 1) / cus) * cus); };
+      const long long rows256 = (p.M + 255) / 256;
+      const double e256 = fill(t256);
+      const double e160 = p.N % 160 == 0 ? 0.78 * fill(rows256 * (p.N / 160) * p.batch) : 0.0;
+      const double e288 = p.N % 288 == 0 ? 0.9 * fill(rows256 * (p.N / 288) * p.batch) : 0.0;
+      if (e160 > e256 && e160 >= e288) {
         g_last_kernel = "pipe16_256x160";
         return launch_pipe16<Pipe16Cfg<256, 160, 4, 2, 5, KIND>>(p, stream);
+      }
+      if (e288 > e256) {
+        g_last_kernel = "pipe16_256x288";
+        return launch_pipe16<Pipe16Cfg<256, 288, 4, 2, 4, KIND>>(p, stream);
       }
       g_last_kernel = "pipe_256x256";
       return launch_pipe<PipeCfg<256, 256, 2, 4, 4, KIND, SWAP>>(p, stream);
