@@ -109,6 +109,37 @@ def test_unscaled_and_fp32_linear_modules():
         assert torch.equal(f(x).view(12, 16), orc.linear_a8_w8_bfp32_ofp32(x.view(12, 32), f.weight, f.bias, 0.004, 1))
 
 
+def test_weight_only_linear_modules():
+    # W8A16Linear / W8FakeA8Linear (upstream nn/linear.py:232-337): pure torch, no INT8 kernel involved
+    from torch_int.nn.linear import W8A16Linear, W8FakeA8Linear
+    torch.manual_seed(0)
+    lin = torch.nn.Linear(64, 48)
+    x = torch.randn(5, 7, 64)
+    y_gt = lin(x)
+    for quant in ("per_channel", "per_tensor"):
+        m = W8A16Linear.from_float(_clone_linear(lin), weight_quant=quant)
+        assert m.weight.dtype == torch.int8 and m.bias.dtype == torch.float16 and m.bias.shape == (48,)
+        assert set(m.state_dict()) == {"weight", "bias", "weight_scales"}
+        y = m(x.clone())
+        assert y.shape == y_gt.shape
+        assert ((y - y_gt) ** 2).mean() / (y_gt ** 2).mean() < 1e-3, quant
+    with pytest.raises(ValueError):
+        W8A16Linear.from_float(_clone_linear(lin), weight_quant="per_row")
+    for act in ("per_token", "per_tensor"):
+        m = W8FakeA8Linear.from_float(_clone_linear(lin), act_quant=act)
+        y = m(x.clone())
+        assert ((y - y_gt) ** 2).mean() / (y_gt ** 2).mean() < 2e-3, act
+    with pytest.raises(ValueError):
+        W8FakeA8Linear(8, 8, act_quant="per_block")
+    m = W8A16Linear(16, 8, bias=False)
+    assert m.bias is None and m(torch.randn(3, 16)).shape == (3, 8)
+    # the fake-quantised activations lie on the int8 grid of their row scale
+    t = torch.randn(4, 64)
+    scale = t.abs().max(dim=-1, keepdim=True)[0] / 127
+    q = W8FakeA8Linear(64, 8).activation_fake_quantizer(t.clone()) / scale
+    assert torch.allclose(q, q.round(), atol=1e-4) and q.abs().max() <= 127.001
+
+
 def test_bmm_modules_and_from_scale():
     g = torch.Generator().manual_seed(3)
     a, b = _s8(g, 2, 5, 16), _s8(g, 2, 7, 16)

@@ -1,4 +1,5 @@
-"""W8A8 linear layers (upstream ``torch_int/nn/linear.py:16-229``).
+"""W8A8 linear layers (upstream ``torch_int/nn/linear.py:16-229``) and the two weight-only
+layers ``W8A16Linear`` / ``W8FakeA8Linear`` (``:232-337``).
 
 Every class keeps upstream's constructor signature, buffer names/shapes/dtypes
 (``weight`` int8 [out, in], ``bias`` [1, out], 0-dim fp32 ``a``/``b``) and
@@ -8,7 +9,9 @@ Every class keeps upstream's constructor signature, buffer names/shapes/dtypes
 import torch
 
 from .. import _CUDA
-from ..functional.quantization import quantize_per_tensor_absmax
+from ..functional.quantization import (fake_quantize_activation_per_tensor_absmax,
+                                       fake_quantize_activation_per_token_absmax,
+                                       quantize_per_tensor_absmax, quantize_weight_per_channel_absmax)
 from ._scalars import ScalarCacheMixin
 
 
@@ -143,4 +146,88 @@ class W8A8BFP32OFP32Linear(_W8A8Base):
         q.bias = module.bias.to(torch.float32)
         q.a = input_scale * w_scale
         q.input_scale, q.weight_scale = input_scale, w_scale
+        return q
+
+
+class _W8FloatActivationBase(torch.nn.Module):
+    """Shared part of the weight-only layers: int8 ``weight`` [out, in], fp16 ``bias`` [1, out] (or None)
+    and fp16 ``weight_scales``; the forward pass dequantises the weight and runs a floating-point linear
+    (upstream ``torch_int/nn/linear.py:232-337``).  These layers do not touch the INT8 kernels."""
+
+    def __init__(self, in_features, out_features, bias=True):
+        super().__init__()
+        self.in_features = in_features
+        self.out_features = out_features
+        self.register_buffer("weight", torch.randint(-127, 127, (out_features, in_features), dtype=torch.int8))
+        self.register_buffer("bias", torch.zeros((1, out_features), dtype=torch.float16) if bias else None)
+        self.register_buffer("weight_scales", torch.ones(out_features, dtype=torch.float16))
+
+    def to(self, *args, **kwargs):
+        super().to(*args, **kwargs)
+        device = torch._C._nn._parse_to(*args, **kwargs)[0]
+        if device is not None:  # the int8 weight follows device moves, never a dtype cast
+            self.weight = self.weight.to(device)
+        return self
+
+    def _dequantized_weight(self, dtype):
+        w = self.weight.to(dtype)
+        s = self.weight_scales.to(dtype)
+        # one scale per output channel ([out] or [out, 1]) or a single per-tensor scale
+        return w.mul_(s.reshape(-1, 1) if s.numel() == self.out_features else s.reshape(()))
+
+    def _bias_for(self, x):
+        return None if self.bias is None else self.bias.to(x.dtype).reshape(-1)
+
+    def extra_repr(self):
+        return f"{self.in_features}, {self.out_features}, bias={self.bias is not None}"
+
+
+class W8A16Linear(_W8FloatActivationBase):
+    """int8 weights, floating-point activations: y = x @ (weight * weight_scales)^T + bias."""
+
+    @torch.no_grad()
+    def forward(self, x):
+        return torch.nn.functional.linear(x, self._dequantized_weight(x.dtype), self._bias_for(x))
+
+    @staticmethod
+    def from_float(module, weight_quant="per_channel"):
+        assert isinstance(module, torch.nn.Linear)
+        q = W8A16Linear(module.in_features, module.out_features, module.bias is not None)
+        if weight_quant == "per_channel":
+            q.weight, q.weight_scales = quantize_weight_per_channel_absmax(module.weight)
+        elif weight_quant == "per_tensor":
+            q.weight, q.weight_scales = quantize_per_tensor_absmax(module.weight)
+        else:
+            raise ValueError('weight_quant must be "per_channel" or "per_tensor"')
+        if module.bias is not None:
+            q.bias = module.bias.to(torch.float16)
+        return q
+
+
+class W8FakeA8Linear(_W8FloatActivationBase):
+    """int8 weights, activations fake-quantised to the int8 grid (per token or per tensor) and kept in
+    floating point: the accuracy-simulation layer.  The activation tensor is quantised in place."""
+
+    def __init__(self, in_features, out_features, bias=True, act_quant="per_token"):
+        super().__init__(in_features, out_features, bias)
+        if act_quant == "per_token":
+            self.activation_fake_quantizer = fake_quantize_activation_per_token_absmax
+        elif act_quant == "per_tensor":
+            self.activation_fake_quantizer = fake_quantize_activation_per_tensor_absmax
+        else:
+            raise ValueError('act_quant must be "per_token" or "per_tensor"')
+
+    @torch.no_grad()
+    def forward(self, x):
+        w = self._dequantized_weight(x.dtype)
+        x = self.activation_fake_quantizer(x)
+        return torch.nn.functional.linear(x, w, self._bias_for(x))
+
+    @staticmethod
+    def from_float(module, act_quant="per_token"):
+        assert isinstance(module, torch.nn.Linear)
+        q = W8FakeA8Linear(module.in_features, module.out_features, module.bias is not None, act_quant)
+        q.weight, q.weight_scales = quantize_weight_per_channel_absmax(module.weight)
+        if module.bias is not None:
+            q.bias = module.bias.to(torch.float16)
         return q
