@@ -121,6 +121,13 @@ int ti_dq_add_layernorm_q(const int32_t* input, float input_scale, const float* 
 /* ---- fused element-wise chains of the OPT blocks (no counterpart in the reference's native
  * module: upstream runs these as sequences of torch ops) ---- */
 
+/* inout[m,n] = inout[m,n] + fmaf(alpha, acc, beta*bias[n]): linear_a8_w8_bfp32_ofp32 whose result is added
+ * (one fp32 add, after the linear's own rounding) into a tensor that is already there.  Replaces
+ * `residual.add_(fc2(x))` (torch_int/models/opt.py:287-289) without the intermediate [M,N] tensor. */
+int ti_linear_a8_w8_bfp32_ofp32_acc(const int8_t* x, const int8_t* w, const float* bias, float* inout,
+                                    int64_t M, int64_t N, int64_t K, float alpha, float beta,
+                                    void* workspace, int64_t workspace_bytes, void* stream);
+
 /* x != NULL: residual[row,i] += x[row,i] (in place), then
  *            q_out = s8(clamp(rint(LN(residual[row,:])[i] * gamma[i] + beta[i]), -128, 127));
  * x == NULL: the same without the add (residual is only read).

@@ -240,3 +240,8 @@ def attn_softmax_q(scores, mask, heads):
 def bmm_s8t_s8t_s8t(a, b, alpha):
     """P.V with V row-major: a [B,M,K], b [B,K,N] (ti_bmm_s8t_s8t_s8t) = bmm_s8t_s8n_s8t on b transposed."""
     return bmm_s8t_s8n_s8t(a, b.transpose(1, 2).contiguous(), alpha)
+
+
+def linear_a8_w8_bfp32_ofp32_acc(x, w, bias, alpha, beta, inout, acc_fn=gemm_acc):
+    """ti_linear_a8_w8_bfp32_ofp32_acc: the fp32 linear, rounded, then one fp32 add into ``inout`` (returns a new tensor)."""
+    return inout + linear_a8_w8_bfp32_ofp32(x, w, bias, alpha, beta, acc_fn=acc_fn).view(inout.shape)

@@ -420,6 +420,40 @@ def test_int8_layout_kernels():
         assert out.is_contiguous() and torch.equal(out, t.transpose(1, 2).contiguous())
 
 
+def test_linear_accumulate_into_output():
+    # inout += alpha*acc + bias in the GEMM epilogue, through every kernel family the fp32 linear can take
+    import ctypes
+    import torch_int._CUDA as C
+    C._lib.ti_last_kernel.restype = ctypes.c_char_p
+    g = torch.Generator().manual_seed(63)
+    seen = set()
+    for (M, N, K) in [(2048, 5120, 256), (2000, 9216, 192), (4096, 2816, 128), (1024, 2048, 64), (1024, 5120, 5120),
+                      (128, 640, 4096), (16, 5120, 3072), (3, 100, 272), (300, 200, 48), (2100, 5000, 272),
+                      (70, 50, 37), (4, 64, 0)]:
+        _say(f"linear += M={M} N={N} K={K}")
+        x, w = _s8(g, M, K), _s8(g, N, K)
+        bias, resid = torch.randn(N, generator=g), torch.randn(M, N, generator=g) * 3
+        alpha = _scal(g, 1e-4, 1e-2)
+        ref = orc.linear_a8_w8_bfp32_ofp32_acc(x, w, bias, alpha, 1.0, resid)
+        inout = resid.to(DEV)
+        out = C._linear_a8_w8_bfp32_ofp32_acc(x.to(DEV), w.to(DEV), bias.to(DEV), alpha, 1.0, inout)
+        assert out.data_ptr() == inout.data_ptr()
+        assert _ulp_diff(out.cpu(), ref) == 0, (M, N, K)
+        seen.add(C._lib.ti_last_kernel().decode())
+    assert {"pipe16_256x160", "pipe16_256x288", "pipe_256x256", "pipe_128x128", "splitk_256x256", "splitk_128x128",
+            "stream", "skinny", "tile_64x64", "tile_256x256", "scalar"} <= seen, seen
+    # the module route: W8A8BFP32OFP32Linear(x, add_to=residual)
+    from torch_int.nn.linear import W8A8BFP32OFP32Linear
+    m = W8A8BFP32OFP32Linear(256, 320, alpha=0.003)
+    m.bias = torch.randn(1, 320, generator=g)
+    x = _s8(g, 2, 5, 256)
+    resid = torch.randn(2, 5, 320, generator=g)
+    ref = orc.linear_a8_w8_bfp32_ofp32_acc(x.view(-1, 256), m.weight, m.bias, 0.003, 1.0, resid)
+    m = m.to(DEV)
+    r = resid.to(DEV)
+    assert m(x.to(DEV), add_to=r) is r and _ulp_diff(r.cpu(), ref) == 0
+
+
 def test_bmm_rowmajor_rhs_for_decode():
     # P.V on V as the KV cache stores it: [B, M, K] x [B, K, N], any K and N
     import torch_int._hip_ext as X

@@ -148,7 +148,13 @@ def test_decoder_layer_opt13b_shape():
         check_linear(name, orc.linear_a8_w8_b8_o8, lin, (lin.a.item(), lin.b.item()))
     check_linear("out", orc.linear_a8_w8_bfp32_ofp32, a.out_proj, (a.out_proj.a.item(), 1))
     check_linear("fc1", orc.linear_relu_a8_w8_b8_o8, layer.fc1, (layer.fc1.a.item(), layer.fc1.b.item()))
-    check_linear("fc2", orc.linear_a8_w8_bfp32_ofp32, layer.fc2, (layer.fc2.a.item(), 1))
+    # fc2 adds its result into the residual stream in the GEMM epilogue: its "output" is the updated residual
+    _say("  check fc2 (+= residual)")
+    r1 = hidden.to(DEV) + rec["out"][1]
+    x = rec["fc2"][0][0].cpu().view(B * T, -1)[rows].contiguous()
+    ref = orc.linear_a8_w8_bfp32_ofp32_acc(x, layer.fc2.weight, layer.fc2.bias, layer.fc2.a.item(), 1,
+                                           r1.cpu().view(B * T, -1)[rows].contiguous(), acc_fn=orc.gemm_acc_torch)
+    assert torch.equal(rec["fc2"][1].cpu().view(B * T, -1)[rows], ref)
     heads = torch.tensor([0, 39, 77, 159])
     _say("  check qk / pv")
     (q_in, k_in), s_out = rec["qk"]
@@ -168,10 +174,9 @@ def test_decoder_layer_opt13b_shape():
     probs_cpu = torch.softmax(torch.clamp_min(scores, torch.finfo(torch.float32).min), -1)
     assert (probs_gpu.cpu() - probs_cpu).abs().max() <= 0.5 / 127 + 1e-3
     # residual algebra: out = hidden + attn_out + fc2_out, in that order, in fp32
-    r1 = hidden.to(DEV) + rec["out"][1]
     assert torch.equal(rec["ln2_in"][0], hidden.to(DEV))  # the layer norm receives the residual ...
     assert torch.equal(rec["ln2"][0][0], r1)              # ... and has added the attention output in place
-    assert torch.equal(out[0], r1 + rec["fc2"][1])
+    assert torch.equal(out[0], rec["fc2"][1])             # fc2 has added its result to that, in place
 
 
 @torch.no_grad()

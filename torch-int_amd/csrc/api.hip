@@ -114,6 +114,13 @@ int ti_linear_a8_w8_bfp32_ofp32(const int8_t* x, const int8_t* w, const float* b
                   ws_bytes, stream);
 }
 
+int ti_linear_a8_w8_bfp32_ofp32_acc(const int8_t* x, const int8_t* w, const float* bias, float* inout, int64_t M,
+                                    int64_t N, int64_t K, float alpha, float beta, void* ws, int64_t ws_bytes,
+                                    void* stream) {
+  return run_gemm("linear_a8_w8_bfp32_ofp32_acc", EPI_F32_BIAS_ACC, x, w, bias, 4, inout, 4, 1, M, N, K, alpha, beta,
+                  ws, ws_bytes, stream);
+}
+
 int ti_linear_a8_w8_b8_o8(const int8_t* x, const int8_t* w, const int8_t* bias, int8_t* out, int64_t M,
                           int64_t N, int64_t K, float alpha, float beta, void* ws, int64_t ws_bytes,
                           void* stream) {

@@ -34,6 +34,7 @@ static PyObject* fc_linear(PyObject* self, PyObject* const* a, Py_ssize_t n) {
     case 2: rc = ti_linear_a8_w8_bfp32_ofp32(x, w, b, o, M, N, K, alpha, beta, ws, wsb, st); break;
     case 3: rc = ti_linear_a8_w8_b8_o8(x, w, b, o, M, N, K, alpha, beta, ws, wsb, st); break;
     case 4: rc = ti_linear_relu_a8_w8_b8_o8(x, w, b, o, M, N, K, alpha, beta, ws, wsb, st); break;
+    case 8: rc = ti_linear_a8_w8_bfp32_ofp32_acc(x, w, b, o, M, N, K, alpha, beta, ws, wsb, st); break;
     default:
       PyErr_SetString(PyExc_ValueError, "unknown linear kind");
       return NULL;

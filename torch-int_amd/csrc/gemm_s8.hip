@@ -138,10 +138,10 @@ __device__ __forceinline__ void store_tile(v16i (&acc)[Cfg::TM][Cfg::TN], const 
           } else {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-              Out o0 = E::apply(acc[i][j][4 * q + 0], bt[4 * q + 0], alpha);
-              Out o1 = E::apply(acc[i][j][4 * q + 1], bt[4 * q + 1], alpha);
-              Out o2 = E::apply(acc[i][j][4 * q + 2], bt[4 * q + 2], alpha);
-              Out o3 = E::apply(acc[i][j][4 * q + 3], bt[4 * q + 3], alpha);
+              Out o0 = merge_old<E>(E::apply(acc[i][j][4 * q + 0], bt[4 * q + 0], alpha), dst + 4 * q + 0);
+              Out o1 = merge_old<E>(E::apply(acc[i][j][4 * q + 1], bt[4 * q + 1], alpha), dst + 4 * q + 1);
+              Out o2 = merge_old<E>(E::apply(acc[i][j][4 * q + 2], bt[4 * q + 2], alpha), dst + 4 * q + 2);
+              Out o3 = merge_old<E>(E::apply(acc[i][j][4 * q + 3], bt[4 * q + 3], alpha), dst + 4 * q + 3);
               v4i w = {__builtin_bit_cast(int, o0), __builtin_bit_cast(int, o1),
                        __builtin_bit_cast(int, o2), __builtin_bit_cast(int, o3)};
               *reinterpret_cast<v4i*>(dst + 4 * q) = w;
@@ -150,7 +150,7 @@ __device__ __forceinline__ void store_tile(v16i (&acc)[Cfg::TM][Cfg::TN], const 
         } else {
 #pragma unroll
           for (int v = 0; v < 16; ++v)
-            if (nb + v < N) dst[v] = E::apply(acc[i][j][v], bt[v], alpha);
+            if (nb + v < N) dst[v] = merge_old<E>(E::apply(acc[i][j][v], bt[v], alpha), dst + v);
         }
       }
     }
@@ -167,7 +167,11 @@ __device__ __forceinline__ void store_tile(v16i (&acc)[Cfg::TM][Cfg::TN], const 
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const int m = m0 + wave_m * Cfg::WTM + i * 32 + 8 * (v >> 2) + 4 * half + (v & 3);
-          if (m < M && n < N) C[(long long)m * N + n] = E::apply(acc[i][j][v], bt, alpha);
+          if (m < M && n < N) {
+            Out fresh = E::apply(acc[i][j][v], bt, alpha);
+            if constexpr (E::kAccumulate) fresh = C[(long long)m * N + n] + fresh;
+            C[(long long)m * N + n] = fresh;
+          }
         }
       }
     }
@@ -709,9 +713,38 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe16_kernel(GemmParams p, i
     const BiasT* __restrict__ bias = reinterpret_cast<const BiasT*>(p.bias);
     const bool vec_ok = (N & 3) == 0 && (reinterpret_cast<uintptr_t>(C) & 15) == 0;
     const bool bias_al = (reinterpret_cast<uintptr_t>(bias) & 15) == 0;
+    // accumulate-into-output kind: fetch what the tile holds now, the loads in flight together before the
+    // first use -- the whole wave tile when its TM*TN*4 registers fit, else one column block at a time
+    constexpr bool HOLD_ALL = E::kAccumulate && TM * TN <= 24;
+    constexpr int HJ = E::kAccumulate ? (HOLD_ALL ? TN : 1) : 1;
+    typename std::conditional<E::kAccumulate, v4f, char>::type held[E::kAccumulate ? TM : 1][HJ];
+    auto fetch_held = [&](int j, int slot) {
+      if constexpr (E::kAccumulate) {
+        const int nb = tile_n * BN + wave_n * Cfg::WTN + j * 16 + 4 * eg;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+          const int m = tile_m * BM + wave_m * Cfg::WTM + i * 16 + er;
+          const float* src = reinterpret_cast<const float*>(C) + ((long long)(m < M ? m : M - 1) * N + nb);
+          v4f h = {0.f, 0.f, 0.f, 0.f};
+          if (vec_ok && nb + 4 <= N) {
+            h = *reinterpret_cast<const v4f*>(src);
+          } else {
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+              if (nb + v < N) h[v] = src[v];
+          }
+          held[i][slot] = h;
+        }
+      }
+    };
+    if constexpr (HOLD_ALL) {
+#pragma unroll
+      for (int j = 0; j < TN; ++j) fetch_held(j, j);
+    }
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       const int nb = tile_n * BN + wave_n * Cfg::WTN + j * 16 + 4 * eg;
+      if constexpr (E::kAccumulate && !HOLD_ALL) fetch_held(j, 0);
       float bt[4];
       if (E::kHasBias && vec_ok && bias_al && nb + 4 <= N) {
         BiasT bv[4];
@@ -740,6 +773,10 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe16_kernel(GemmParams p, i
 #pragma unroll
         for (int v = 0; v < 4; ++v) o[v] = E::apply(acc[i][j][v], bt[v], p.alpha);
         Out* dst = C + (long long)m * N + nb;
+        if constexpr (E::kAccumulate) {
+#pragma unroll
+          for (int v = 0; v < 4; ++v) o[v] = held[i][HOLD_ALL ? j : 0][v] + o[v];
+        }
         if (vec_ok && nb + 4 <= N) {
           if (sizeof(Out) == 4) {
             using W = typename std::conditional<sizeof(Out) == 4, Out, int>::type;
@@ -810,6 +847,11 @@ __device__ __forceinline__ void store_skinny_tile(v4i acc, const GemmParams& p, 
     o[v] = E::apply(acc[v], E::bias_term(bv, p.beta), p.alpha);
   }
   Out* dst = C + (long long)m * N + nb;
+  if constexpr (E::kAccumulate) {
+#pragma unroll
+    for (int v = 0; v < 4; ++v)
+      if (nb + v < N) o[v] = merge_old<E>(o[v], dst + v);
+  }
   const bool whole = (N % 4 == 0) && nb + 4 <= N && (reinterpret_cast<uintptr_t>(C) & 15) == 0;
   if (whole && sizeof(Out) == 4) {
     using W = typename std::conditional<sizeof(Out) == 4, Out, int>::type;
@@ -1070,7 +1112,7 @@ __global__ __launch_bounds__(256) void gemm_scalar_kernel(GemmParams p) {
   BiasT bv = BiasT(0);
   if (E::kHasBias) bv = reinterpret_cast<const BiasT*>(p.bias)[n];
   Out* C = reinterpret_cast<Out*>(p.C) + (long long)blockIdx.z * p.strideC;
-  C[idx] = E::apply(acc, E::bias_term(bv, p.beta), p.alpha);
+  C[idx] = merge_old<E>(E::apply(acc, E::bias_term(bv, p.beta), p.alpha), C + idx);
 }
 
 // ------------------------------------------------------------------ host side
@@ -1160,7 +1202,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmParams p, const 
     for (int v = 0; v < 4; ++v) {
       BiasT bv = BiasT(0);
       if (E::kHasBias) bv = bias[n + v];
-      o[v] = E::apply(acc[v], E::bias_term(bv, p.beta), p.alpha);
+      o[v] = merge_old<E>(E::apply(acc[v], E::bias_term(bv, p.beta), p.alpha), C + i0 + v);
     }
     if (sizeof(Out) == 4) {
       using W = typename std::conditional<sizeof(Out) == 4, Out, int>::type;
@@ -1178,7 +1220,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmParams p, const 
       for (int s = 0; s < splits; ++s) acc += ws[(long long)s * total + i0 + v];
       BiasT bv = BiasT(0);
       if (E::kHasBias) bv = bias[(i0 + v) % p.N];
-      C[i0 + v] = E::apply(acc, E::bias_term(bv, p.beta), p.alpha);
+      C[i0 + v] = merge_old<E>(E::apply(acc, E::bias_term(bv, p.beta), p.alpha), C + i0 + v);
     }
   }
 }
@@ -1255,13 +1297,17 @@ static int launch_kind(const GemmParams& p, void* workspace, long long workspace
     // stages and as many resident workgroups as the LDS allows.
     auto launch = [&](auto kern, int rows, int per_cu) -> int {
       const int lds = 2 * rows * SBK + S_RED;
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-      if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+      static bool attr_set = false;  // one flag per kernel instantiation (the lambda is generic)
+      if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+        attr_set = true;
+      }
       const long long slots = (long long)cus * per_cu;
       hipLaunchKernelGGL(kern, dim3((unsigned)(strips < slots ? strips : slots)), dim3(256), lds, stream, p, spb,
                          (int)strips);
-      e = hipGetLastError();
+      hipError_t e = hipGetLastError();
       if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "gemm launch: %s", hipGetErrorString(e));
       return TI_OK;
     };
@@ -1370,6 +1416,7 @@ int launch_gemm(int kind, const GemmParams& p, void* ws, long long ws_bytes, hip
     case EPI_F32_SCALE: return launch_kind<EPI_F32_SCALE>(p, ws, ws_bytes, stream);
     case EPI_S8_SCALE: return launch_kind<EPI_S8_SCALE>(p, ws, ws_bytes, stream);
     case EPI_S32_RAW: return launch_kind<EPI_S32_RAW>(p, ws, ws_bytes, stream);
+    case EPI_F32_BIAS_ACC: return launch_kind<EPI_F32_BIAS_ACC>(p, ws, ws_bytes, stream);
   }
   return fail(TI_ERR_INVALID_ARG, "unknown epilogue kind %d", kind);
 }

@@ -26,6 +26,7 @@ enum EpiKind : int {
   EPI_F32_SCALE = 5,   // out = a * acc
   EPI_S8_SCALE = 6,    // out = s8(rint(clamp(a * acc)))
   EPI_S32_RAW = 7,     // out = acc
+  EPI_F32_BIAS_ACC = 8,  // out = out + fma(a, acc, b*bias)   (fp32; adds into the tensor already there)
 };
 
 // round-half-even then v_cvt_i32_f32, which saturates to int32 and maps NaN to 0
@@ -55,6 +56,7 @@ struct Epi<EPI_S32_BIAS> {
   using Out = int32_t;
   using Bias = int32_t;
   static constexpr bool kHasBias = true;
+  static constexpr bool kAccumulate = false;
   // the "bias term" is carried as raw bits so one code path serves all kinds
   static __device__ __forceinline__ float bias_term(Bias b, float) { return __int_as_float(b); }
   static __device__ __forceinline__ Out apply(int acc, float bt, float) {
@@ -66,6 +68,7 @@ struct Epi<EPI_S32_SCALED> {
   using Out = int32_t;
   using Bias = int32_t;
   static constexpr bool kHasBias = true;
+  static constexpr bool kAccumulate = false;
   static __device__ __forceinline__ float bias_term(Bias b, float beta) { return beta * (float)b; }
   static __device__ __forceinline__ Out apply(int acc, float bt, float alpha) {
     return rne_sat_s32(__builtin_fmaf(alpha, (float)acc, bt));
@@ -76,6 +79,7 @@ struct Epi<EPI_F32_BIAS> {
   using Out = float;
   using Bias = float;
   static constexpr bool kHasBias = true;
+  static constexpr bool kAccumulate = false;
   static __device__ __forceinline__ float bias_term(Bias b, float beta) { return beta * b; }
   static __device__ __forceinline__ Out apply(int acc, float bt, float alpha) {
     return __builtin_fmaf(alpha, (float)acc, bt);
@@ -86,6 +90,7 @@ struct Epi<EPI_S8_BIAS> {
   using Out = int8_t;
   using Bias = int8_t;
   static constexpr bool kHasBias = true;
+  static constexpr bool kAccumulate = false;
   static __device__ __forceinline__ float bias_term(Bias b, float beta) { return beta * (float)(int)b; }
   static __device__ __forceinline__ Out apply(int acc, float bt, float alpha) {
     return (int8_t)rne_s8(__builtin_fmaf(alpha, (float)acc, bt));
@@ -96,6 +101,7 @@ struct Epi<EPI_S8_RELU> {
   using Out = int8_t;
   using Bias = int8_t;
   static constexpr bool kHasBias = true;
+  static constexpr bool kAccumulate = false;
   static __device__ __forceinline__ float bias_term(Bias b, float beta) { return beta * (float)(int)b; }
   static __device__ __forceinline__ Out apply(int acc, float bt, float alpha) {
     // relu then clamp == integer clamp to [0, 127] after rounding (NaN -> 0 either way)
@@ -107,6 +113,7 @@ struct Epi<EPI_F32_SCALE> {
   using Out = float;
   using Bias = float;
   static constexpr bool kHasBias = false;
+  static constexpr bool kAccumulate = false;
   static __device__ __forceinline__ float bias_term(Bias, float) { return 0.0f; }
   static __device__ __forceinline__ Out apply(int acc, float, float alpha) { return alpha * (float)acc; }
 };
@@ -115,6 +122,7 @@ struct Epi<EPI_S8_SCALE> {
   using Out = int8_t;
   using Bias = int8_t;
   static constexpr bool kHasBias = false;
+  static constexpr bool kAccumulate = false;
   static __device__ __forceinline__ float bias_term(Bias, float) { return 0.0f; }
   static __device__ __forceinline__ Out apply(int acc, float, float alpha) {
     return (int8_t)rne_s8(alpha * (float)acc);
@@ -125,9 +133,32 @@ struct Epi<EPI_S32_RAW> {
   using Out = int32_t;
   using Bias = int32_t;
   static constexpr bool kHasBias = false;
+  static constexpr bool kAccumulate = false;
   static __device__ __forceinline__ float bias_term(Bias, float) { return 0.0f; }
   static __device__ __forceinline__ Out apply(int acc, float, float) { return acc; }
 };
+
+template <>
+struct Epi<EPI_F32_BIAS_ACC> {
+  using Out = float;
+  using Bias = float;
+  static constexpr bool kHasBias = true;
+  static constexpr bool kAccumulate = true;  // the stores add to what the output already holds
+  static __device__ __forceinline__ float bias_term(Bias b, float beta) { return beta * b; }
+  static __device__ __forceinline__ Out apply(int acc, float bt, float alpha) {
+    return __builtin_fmaf(alpha, (float)acc, bt);
+  }
+};
+
+// `fresh` for the ordinary kinds; `*where + fresh` (one fp32 add, the linear's own result rounded first)
+// for the accumulate-into-output kind.
+template <class E>
+__device__ __forceinline__ typename E::Out merge_old(typename E::Out fresh, const typename E::Out* where) {
+  if constexpr (E::kAccumulate)
+    return *where + fresh;
+  else
+    return fresh;
+}
 
 // Problem description handed to every GEMM kernel.  A is [batch, M, K], B is
 // [batch, N, K], C is [batch, M, N], all packed; bias is [N] (shared by batches).

@@ -38,6 +38,7 @@ _SIGNATURES = {
     "ti_linear_a8_w8_b32_o32_with_scaling": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _f32, _f32, _vp, _i64, _vp],
     "ti_linear_a8_w8_bfp32_ofp32": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _f32, _f32, _vp, _i64, _vp],
     "ti_linear_a8_w8_b8_o8": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _f32, _f32, _vp, _i64, _vp],
+    "ti_linear_a8_w8_bfp32_ofp32_acc": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _f32, _f32, _vp, _i64, _vp],
     "ti_linear_relu_a8_w8_b8_o8": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _f32, _f32, _vp, _i64, _vp],
     "ti_bmm_s8t_s8n_f32t": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _f32, _vp],
     "ti_bmm_s8t_s8n_s8t": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _f32, _vp],
@@ -94,10 +95,10 @@ _empty = torch.empty
 _I8, _I32, _F32 = torch.int8, torch.int32, torch.float32
 
 # kind codes shared with csrc/ti_common.h (EpiKind) and csrc/fastcall.c
-_K_B32, _K_B32S, _K_F32, _K_S8, _K_RELU, _K_BMM_F32, _K_BMM_S8, _K_BMM_S32 = range(8)
+_K_B32, _K_B32S, _K_F32, _K_S8, _K_RELU, _K_BMM_F32, _K_BMM_S8, _K_BMM_S32, _K_F32_ACC = range(9)
 _LINEAR_CTYPES = {_K_B32: _lib.ti_linear_a8_w8_b32_o32, _K_B32S: _lib.ti_linear_a8_w8_b32_o32_with_scaling,
                   _K_F32: _lib.ti_linear_a8_w8_bfp32_ofp32, _K_S8: _lib.ti_linear_a8_w8_b8_o8,
-                  _K_RELU: _lib.ti_linear_relu_a8_w8_b8_o8}
+                  _K_RELU: _lib.ti_linear_relu_a8_w8_b8_o8, _K_F32_ACC: _lib.ti_linear_a8_w8_bfp32_ofp32_acc}
 _BMM_CTYPES = {_K_BMM_F32: _lib.ti_bmm_s8t_s8n_f32t, _K_BMM_S8: _lib.ti_bmm_s8t_s8n_s8t,
                _K_BMM_S32: _lib.ti_bmm_s8t_s8n_s32t}
 
@@ -143,7 +144,7 @@ def _workspace(dev_index, stream, nbytes):
     return ws.data_ptr(), ws.numel()
 
 
-def _linear(op, kind, x, w, bias, bias_dtype, out_dtype, alpha, beta):
+def _linear(op, kind, x, w, bias, bias_dtype, out_dtype, alpha, beta, inout=None):
     # fast accept path first; the slow path below names what is wrong
     if not (type(x) is torch.Tensor and type(w) is torch.Tensor and x.dtype is _I8 and w.dtype is _I8
             and x.dim() == 2 and w.dim() == 2 and x.is_cuda and w.device == x.device
@@ -165,7 +166,13 @@ def _linear(op, kind, x, w, bias, bias_dtype, out_dtype, alpha, beta):
         _fail(op, f"bias must be {bias_dtype}, got {bias.dtype}")
     if not bias.is_contiguous():
         bias = bias.contiguous()
-    out = _empty((M, N), dtype=out_dtype, device=dev)
+    if inout is None:
+        out = _empty((M, N), dtype=out_dtype, device=dev)
+    else:  # the accumulate-into-output variant writes where the caller says
+        out = inout
+        if not (type(out) is torch.Tensor and out.dtype is out_dtype and out.device == dev and out.is_contiguous()
+                and out.numel() == M * N and out.dim() >= 1 and out.shape[-1] == N):
+            _fail(op, f"the tensor to add into must be a contiguous {out_dtype} tensor of {M}x{N} elements on {dev}")
     if M == 0 or N == 0:
         return out
     idx = dev.index
@@ -206,6 +213,13 @@ def linear_a8_w8_b32_o32_with_scaling(input, weight, bias, alpha, beta):
 def linear_a8_w8_bfp32_ofp32(input, weight, bias, alpha, beta):
     """fp32 [M,N] = alpha*acc + beta*bias, fp32 bias  (upstream linear.cu:246-365)."""
     return _linear("linear_a8_w8_bfp32_ofp32", _K_F32, input, weight, bias, _F32, _F32, float(alpha), float(beta))
+
+
+def _linear_a8_w8_bfp32_ofp32_acc(input, weight, bias, alpha, beta, inout):
+    """inout += alpha*acc + beta*bias, in place (no counterpart upstream; used by the OPT decoder layer for
+    ``residual.add_(fc2(x))``).  Returns ``inout``."""
+    return _linear("linear_a8_w8_bfp32_ofp32_acc", _K_F32_ACC, input, weight, bias, _F32, _F32, float(alpha),
+                   float(beta), inout)
 
 
 def linear_a8_w8_b8_o8(input, weight, bias, alpha, beta):

@@ -172,8 +172,11 @@ class Int8OPTDecoderLayer(nn.Module):
             hidden_states=x, past_key_value=past_key_value, attention_mask=attention_mask,
             layer_head_mask=layer_head_mask, output_attentions=output_attentions)
         x = self.final_layer_norm(residual, add=x)  # residual += x, then LayerNormQ
-        x = self.fc2(self.fc1(x))
-        residual.add_(x.to(residual.dtype))
+        x = self.fc1(x)
+        if type(self.fc2) is W8A8BFP32OFP32Linear:
+            self.fc2(x, add_to=residual)  # residual += fc2(x), added in the GEMM epilogue when residual is fp32
+        else:
+            residual.add_(self.fc2(x).to(residual.dtype))
         outputs = (residual,)
         if output_attentions:
             outputs += (attn_weights,)
