@@ -143,12 +143,20 @@ int ti_add_layernorm_q(const float* x, float* residual, const float* gamma, cons
 int ti_attn_softmax_q(const float* scores, const float* mask, int8_t* probs, int64_t batch, int64_t heads,
                       int64_t T, int64_t S, void* stream);
 
+/* bmm_s8t_s8n_f32t whose operands need not be packed along the batch dimension: stride_a / stride_b are the
+ * elements between consecutive batches of a / b (0 = packed; each [M,K] / [N,K] matrix itself stays packed).
+ * Lets Q.K^T read K from a KV-cache buffer that has spare room after every head
+ * (torch_int/models/opt.py:128-133 concatenates the cache instead). */
+int ti_bmm_s8t_s8n_f32t_strided(const int8_t* a, const int8_t* b, float* c, int64_t batch, int64_t M, int64_t N,
+                                int64_t K, int64_t stride_a, int64_t stride_b, float alpha, void* stream);
+
 /* c[b,M,N] = s8(rint(clamp(alpha * a[b,M,K] . bm[b,K,N], -128, 127))) with bm ROW-major (not transposed):
  * the P.V product on V as the KV cache stores it, replacing `value_states.transpose(1, 2).contiguous()`
  * followed by bmm_s8t_s8n_s8t (torch_int/models/opt.py:180-182) when few query rows are live
- * (incremental decoding).  Any M works, 16 rows per pass over bm; any K and N (no multiple-of-16 rule). */
+ * (incremental decoding).  Any M works, 16 rows per pass over bm; any K and N (no multiple-of-16 rule).
+ * stride_b = elements between consecutive batches of bm (0 = packed K*N). */
 int ti_bmm_s8t_s8t_s8t(const int8_t* a, const int8_t* bm, int8_t* c, int64_t batch, int64_t M, int64_t N, int64_t K,
-                       float alpha, void* stream);
+                       int64_t stride_b, float alpha, void* stream);
 
 /* dst[b, y, x, :] = src[b, x, y, :] for int8 [B, X, Y, D]: the head split / merge
  * `view(B,T,H,d).transpose(1,2).contiguous()` (torch_int/models/opt.py:80-81,189-196). */
@@ -157,6 +165,13 @@ int ti_permute_0213_s8(const int8_t* src, int8_t* dst, int64_t B, int64_t X, int
 /* dst[b, c, r] = src[b, r, c] for int8 [B, R, C]: `value_states.transpose(1, 2).contiguous()`
  * (torch_int/models/opt.py:180). */
 int ti_transpose_last2_s8(const int8_t* src, int8_t* dst, int64_t B, int64_t R, int64_t C, void* stream);
+
+/* k_buf[bh, S + t, :] = k_new[bh, t, :] and v_buf[bh, S + t, :] = v_new[bh, t, :] for t < T: appends the new
+ * tokens' keys and values ([BH, T, D] packed) to cache buffers [BH, cap, D] that hold S positions, in one launch.
+ * Replaces the two `torch.cat([past, new], dim=2)` of torch_int/models/opt.py:128-133, which copy the whole
+ * cache at every decode step. */
+int ti_kv_append_s8(const int8_t* k_new, const int8_t* v_new, int8_t* k_buf, int8_t* v_buf, int64_t BH, int64_t T,
+                    int64_t D, int64_t cap, int64_t S, void* stream);
 
 #ifdef __cplusplus
 }

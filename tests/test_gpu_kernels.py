@@ -467,6 +467,17 @@ def test_bmm_rowmajor_rhs_for_decode():
         alpha = _scal(g, 2e-4, 4e-3)
         out = X.bmm_s8t_s8t_s8t(a.to(DEV), b.to(DEV), alpha).cpu()
         assert torch.equal(out, orc.bmm_s8t_s8t_s8t(a, b, alpha)), (B, M, N, K)
+    # operands that live in a buffer with spare rows after every batch (a KV cache with room to grow)
+    for (B, M, S, d, cap) in [(288, 1, 517, 128, 656), (6, 4, 33, 64, 48), (3, 16, 100, 32, 101)]:
+        _say(f"batch-strided products B={B} M={M} S={S} d={d} cap={cap}")
+        p_, q_ = _s8(g, B, M, S, lo=0), _s8(g, B, M, d)
+        kbuf, vbuf = _s8(g, B, cap, d), _s8(g, B, cap, d)
+        kd, vd = kbuf.to(DEV)[:, :S], vbuf.to(DEV)[:, :S]
+        assert not kd.is_contiguous() or B == 1
+        out = X.bmm_s8t_s8t_s8t(p_.to(DEV), vd, 0.002).cpu()
+        assert torch.equal(out, orc.bmm_s8t_s8t_s8t(p_, vbuf[:, :S].contiguous(), 0.002))
+        sc = X.bmm_s8t_s8n_f32t_strided(q_.to(DEV), kd, 0.003).cpu()
+        assert _ulp_diff(sc, orc.bmm_s8t_s8n_f32t(q_, kbuf[:, :S].contiguous(), 0.003)) == 0
     # an operand pair whose rows are not dword aligned takes the byte path
     a, b = _s8(g, 2, 3, 40), _s8(g, 2, 41, 24)
     bd = b.to(DEV)[:, 1:, :].contiguous()
@@ -475,6 +486,22 @@ def test_bmm_rowmajor_rhs_for_decode():
     assert odd.data_ptr() % 4 != 0
     out = X.bmm_s8t_s8t_s8t(a.to(DEV), odd, 0.001).cpu()
     assert torch.equal(out, orc.bmm_s8t_s8t_s8t(a, b[:, 1:, :].contiguous(), 0.001))
+
+
+def test_kv_append_kernel():
+    import torch_int._hip_ext as X
+    g = torch.Generator().manual_seed(17)
+    for (B, H, cap, d, S, T) in [(4, 72, 656, 128, 544, 1), (2, 3, 40, 64, 7, 5), (1, 2, 9, 24, 8, 1), (2, 2, 16, 20, 0, 16)]:
+        _say(f"kv_append B={B} H={H} cap={cap} d={d} S={S} T={T}")
+        kbuf, vbuf = _s8(g, B, H, cap, d), _s8(g, B, H, cap, d)
+        kn, vn = _s8(g, B, H, T, d), _s8(g, B, H, T, d)
+        kd, vd = kbuf.to(DEV), vbuf.to(DEV)
+        X.kv_append(kn.to(DEV), vn.to(DEV), kd, vd, S)
+        kbuf[:, :, S:S + T] = kn
+        vbuf[:, :, S:S + T] = vn
+        assert torch.equal(kd.cpu(), kbuf) and torch.equal(vd.cpu(), vbuf)
+    with pytest.raises(RuntimeError):
+        X.kv_append(kn.to(DEV), vn.to(DEV), kd, vd, 1)   # 1 + 16 positions do not fit 16
 
 
 def test_runs_are_deterministic():

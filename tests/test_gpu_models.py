@@ -201,3 +201,26 @@ def test_causal_lm_prefill_and_decode_on_gpu():
     step = glm(ids[:, -1:].to(DEV), past_key_values=out.past_key_values, use_cache=True)
     assert step.past_key_values[0][0].shape[2] == 49
     assert _rel_err(step.logits.cpu(), ref_step.logits) <= 2e-3
+    _say("three more decode steps on the in-place cache, and the same steps with concatenation")
+    from torch_int.models.opt import Int8OPTAttention
+    toks = torch.randint(2, 512, (2, 3), generator=g).to(DEV)
+
+    def run(past):
+        logits = []
+        for t in range(3):
+            o = glm(toks[:, t:t + 1], past_key_values=past, use_cache=True)
+            past = o.past_key_values
+            logits.append(o.logits)
+        return logits, past
+    a_logits, a_past = run(step.past_key_values)
+    assert not a_past[0][0].is_contiguous() and a_past[0][0].data_ptr() == step.past_key_values[0][0].data_ptr()
+    Int8OPTAttention.kv_cache_in_place = False
+    try:
+        b_logits, b_past = run(tuple((k.contiguous(), v.contiguous()) for k, v in step.past_key_values))
+    finally:
+        Int8OPTAttention.kv_cache_in_place = True
+    assert b_past[0][0].is_contiguous() and b_past[0][0].shape[2] == 52
+    for x, y in zip(a_logits, b_logits):
+        assert torch.equal(x, y)                       # same kernels' arithmetic on either layout
+    for (k1, v1), (k2, v2) in zip(a_past, b_past):
+        assert torch.equal(k1, k2) and torch.equal(v1, v2)

@@ -440,3 +440,59 @@ def test_causal_lm_prefill_then_decode():
         loss = lm(ids, labels=ids).loss
     assert torch.allclose(step.logits[:, 0], full.logits[:, 16], rtol=1e-4, atol=1e-4)
     assert loss.dim() == 0 and torch.isfinite(loss)
+
+
+def test_kv_cache_append_in_place_semantics():
+    # _kv_append must behave like torch.cat for every caller, however the cache tensors are reused
+    from torch_int.models.opt import _kv_append
+    g = torch.Generator().manual_seed(5)
+
+    def rnd(*shape):
+        return torch.randint(-127, 128, shape, dtype=torch.int8, generator=g)
+    past, t1, t2, t3 = rnd(2, 3, 10, 8), rnd(2, 3, 1, 8), rnd(2, 3, 1, 8), rnd(2, 3, 2, 8)
+    a = _kv_append(past, t1)                       # no buffer yet: copies into one with spare room
+    assert torch.equal(a, torch.cat([past, t1], 2)) and not a.is_contiguous() and a._ti_kv.buf.shape[2] >= 11 + 64
+    b = _kv_append(a, t2)                          # appended behind a, same storage
+    assert b.data_ptr() == a.data_ptr() and torch.equal(b, torch.cat([past, t1, t2], 2))
+    assert torch.equal(a, torch.cat([past, t1], 2))
+    c = _kv_append(a, t3)                          # a second continuation of a: must not disturb b
+    assert c.data_ptr() != b.data_ptr()
+    assert torch.equal(c, torch.cat([past, t1, t3], 2)) and torch.equal(b, torch.cat([past, t1, t2], 2))
+    d = _kv_append(b[:, :, :11], t3)               # a slice made by the caller carries no buffer: plain copy
+    assert torch.equal(d, torch.cat([past, t1, t3], 2)) and torch.equal(b, torch.cat([past, t1, t2], 2))
+    e = b
+    for _ in range(200):                           # growth beyond the spare room re-allocates, values survive
+        e = _kv_append(e, t1)
+    assert e.shape[2] == 212 and torch.equal(e[:, :, :12], b) and torch.equal(e[:, :, -1:], t1)
+    f = _kv_append(b.index_select(0, torch.tensor([1, 0])), t2)   # beam-search style re-ordering
+    assert torch.equal(f, torch.cat([b.index_select(0, torch.tensor([1, 0])), t2], 2))
+
+
+def test_decode_with_in_place_cache_matches_concatenation():
+    from torch_int.models.opt import Int8OPTAttention
+    cfg = OPTConfigLite(hidden_size=64, num_hidden_layers=2, ffn_dim=128, num_attention_heads=4, vocab_size=97,
+                        max_position_embeddings=64)
+    torch.manual_seed(3)
+    lm = Int8OPTForCausalLM(cfg).eval()
+    g = torch.Generator().manual_seed(4)
+    for layer in lm.model.decoder.layers:
+        randomize_int8_layer(layer, g, 2e-3, 8e-3)
+    ids = torch.randint(2, 97, (2, 9), generator=g)
+    outs = {}
+    with oracle_backend():
+        for mode in (True, False):
+            Int8OPTAttention.kv_cache_in_place = mode
+            try:
+                o = lm(ids[:, :5], use_cache=True)
+                steps = [o.logits]
+                for t in range(5, 9):
+                    o = lm(ids[:, t:t + 1], past_key_values=o.past_key_values, use_cache=True)
+                    steps.append(o.logits)
+                outs[mode] = (steps, o.past_key_values)
+            finally:
+                Int8OPTAttention.kv_cache_in_place = True
+    for x, y in zip(outs[True][0], outs[False][0]):
+        assert torch.equal(x, y)
+    for (k1, v1), (k2, v2) in zip(outs[True][1], outs[False][1]):
+        assert k1.shape[2] == 20 and torch.equal(k1, k2) and torch.equal(v1, v2)  # 5 tokens padded to 16, then 4 steps
+        assert not k1.is_contiguous() and k2.is_contiguous()

@@ -41,9 +41,16 @@ static int check_ptr(const char* op, const char* name, const void* p, size_t ali
 
 static int run_gemm(const char* op, int kind, const void* a, const void* b, const void* bias, size_t bias_elt,
                     void* c, size_t out_elt, int64_t batch, int64_t M, int64_t N, int64_t K, float alpha,
-                    float beta, void* ws, int64_t ws_bytes, void* stream) {
+                    float beta, void* ws, int64_t ws_bytes, void* stream, int64_t stride_a = 0,
+                    int64_t stride_b = 0) {
   g_err[0] = 0;
   if (int rc = check_dims(op, batch, M, N, K)) return rc;
+  // batch strides (elements between consecutive batches of a / b); 0 = packed
+  if (stride_a == 0) stride_a = M * K;
+  if (stride_b == 0) stride_b = N * K;
+  if (stride_a < M * K || stride_b < N * K)
+    return fail(TI_ERR_INVALID_ARG, "%s: batch strides (%lld, %lld) are smaller than one batch (%lld, %lld)", op,
+                (long long)stride_a, (long long)stride_b, (long long)(M * K), (long long)(N * K));
   const bool nonempty = batch > 0 && M > 0 && N > 0;
   if (int rc = check_ptr(op, "input", a, 1, nonempty && K > 0)) return rc;
   if (int rc = check_ptr(op, "weight", b, 1, nonempty && K > 0)) return rc;
@@ -61,8 +68,8 @@ static int run_gemm(const char* op, int kind, const void* a, const void* b, cons
   p.batch = (int)batch;
   p.lda = (int)K;
   p.ldb = (int)K;
-  p.strideA = M * K;
-  p.strideB = N * K;
+  p.strideA = stride_a;
+  p.strideB = stride_b;
   p.strideC = M * N;
   p.alpha = alpha;
   p.beta = beta;
@@ -205,16 +212,26 @@ int ti_attn_softmax_q(const float* scores, const float* mask, int8_t* probs, int
 
 const char* ti_last_kernel(void) { return last_gemm_kernel(); }
 
+int ti_bmm_s8t_s8n_f32t_strided(const int8_t* a, const int8_t* b, float* c, int64_t batch, int64_t M, int64_t N,
+                                int64_t K, int64_t stride_a, int64_t stride_b, float alpha, void* stream) {
+  return run_gemm("bmm_s8t_s8n_f32t_strided", EPI_F32_SCALE, a, b, nullptr, 0, c, 4, batch, M, N, K, alpha, 0.0f,
+                  nullptr, 0, stream, stride_a, stride_b);
+}
+
 int ti_bmm_s8t_s8t_s8t(const int8_t* a, const int8_t* b, int8_t* c, int64_t batch, int64_t M, int64_t N, int64_t K,
-                       float alpha, void* stream) {
+                       int64_t stride_b, float alpha, void* stream) {
   g_err[0] = 0;
   const char* op = "bmm_s8t_s8t_s8t";
   if (int rc = check_dims(op, batch, M, N, K)) return rc;
+  if (stride_b == 0) stride_b = K * N;
+  if (stride_b < K * N)
+    return fail(TI_ERR_INVALID_ARG, "%s: batch stride %lld is smaller than one K x N matrix (%lld)", op,
+                (long long)stride_b, (long long)(K * N));
   const bool nonempty = batch > 0 && M > 0 && N > 0;
   if (int rc = check_ptr(op, "a", a, 1, nonempty && K > 0)) return rc;
   if (int rc = check_ptr(op, "b", b, 1, nonempty && K > 0)) return rc;
   if (int rc = check_ptr(op, "c", c, 1, nonempty)) return rc;
-  return launch_bmm_s8t_s8t_s8t(a, b, c, batch, M, N, K, alpha, static_cast<hipStream_t>(stream));
+  return launch_bmm_s8t_s8t_s8t(a, b, c, batch, M, N, K, stride_b, alpha, static_cast<hipStream_t>(stream));
 }
 
 int ti_permute_0213_s8(const int8_t* src, int8_t* dst, int64_t B, int64_t X, int64_t Y, int64_t D, void* stream) {
@@ -227,6 +244,23 @@ int ti_permute_0213_s8(const int8_t* src, int8_t* dst, int64_t B, int64_t X, int
   if (int rc = check_ptr(op, "src", src, 1, nonempty)) return rc;
   if (int rc = check_ptr(op, "dst", dst, 1, nonempty)) return rc;
   return launch_permute_0213_s8(src, dst, B, X, Y, D, static_cast<hipStream_t>(stream));
+}
+
+int ti_kv_append_s8(const int8_t* k_new, const int8_t* v_new, int8_t* k_buf, int8_t* v_buf, int64_t BH, int64_t T,
+                    int64_t D, int64_t cap, int64_t S, void* stream) {
+  g_err[0] = 0;
+  const char* op = "kv_append_s8";
+  const int64_t lim = 0x7fffffffLL;
+  if (BH < 0 || T < 0 || D < 0 || cap < 0 || S < 0 || BH > lim || T > lim || D > lim || cap > lim)
+    return fail(TI_ERR_INVALID_ARG, "%s: sizes must be in [0, 2^31)", op);
+  if (S + T > cap) return fail(TI_ERR_INVALID_ARG, "%s: %lld + %lld positions do not fit a capacity of %lld", op,
+                               (long long)S, (long long)T, (long long)cap);
+  const bool nonempty = BH > 0 && T > 0 && D > 0;
+  if (int rc = check_ptr(op, "k_new", k_new, 1, nonempty)) return rc;
+  if (int rc = check_ptr(op, "v_new", v_new, 1, nonempty)) return rc;
+  if (int rc = check_ptr(op, "k_buf", k_buf, 1, nonempty)) return rc;
+  if (int rc = check_ptr(op, "v_buf", v_buf, 1, nonempty)) return rc;
+  return launch_kv_append_s8(k_new, v_new, k_buf, v_buf, BH, T, D, cap, S, static_cast<hipStream_t>(stream));
 }
 
 int ti_transpose_last2_s8(const int8_t* src, int8_t* dst, int64_t B, int64_t R, int64_t C, void* stream) {

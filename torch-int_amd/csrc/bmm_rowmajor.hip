@@ -17,7 +17,7 @@ constexpr int RM_BN = 128;   // output columns per workgroup
 template <int MR, bool FAST>
 __global__ __launch_bounds__(256) void bmm_rowmajor_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ B,
                                                            int8_t* __restrict__ C, int M, int N, int K, int tiles_n,
-                                                           int groups_m, float alpha) {
+                                                           int groups_m, long long stride_b, float alpha) {
   __shared__ int8_t a_s[MR][RM_KC];
   __shared__ int red[4][MR][RM_BN];
   const int t = threadIdx.x, cq = t & 31, ks = t >> 5, wave = t >> 6;
@@ -42,7 +42,7 @@ __global__ __launch_bounds__(256) void bmm_rowmajor_kernel(const int8_t* __restr
       for (int k = t; k < kc; k += 256) a_s[m][k] = live ? arow[k] : (int8_t)0;
     }
     __syncthreads();
-    const int8_t* bbase = B + ((b * K + kc0) * (long long)N + n);
+    const int8_t* bbase = B + (b * stride_b + kc0 * (long long)N + n);
     constexpr int U = 8;  // rows of bm in flight per thread
     for (int k0 = ks; k0 < kc; k0 += 8 * U) {
       int w[U][4];
@@ -110,30 +110,31 @@ __global__ __launch_bounds__(256) void bmm_rowmajor_kernel(const int8_t* __restr
 
 template <int MR>
 static void launch_rm(bool fast, dim3 grid, hipStream_t stream, const int8_t* a, const int8_t* b, int8_t* c, int M,
-                      int N, int K, int tiles_n, int groups_m, float alpha) {
+                      int N, int K, int tiles_n, int groups_m, long long stride_b, float alpha) {
   if (fast)
     hipLaunchKernelGGL((bmm_rowmajor_kernel<MR, true>), grid, dim3(256), 0, stream, a, b, c, M, N, K, tiles_n,
-                       groups_m, alpha);
+                       groups_m, stride_b, alpha);
   else
     hipLaunchKernelGGL((bmm_rowmajor_kernel<MR, false>), grid, dim3(256), 0, stream, a, b, c, M, N, K, tiles_n,
-                       groups_m, alpha);
+                       groups_m, stride_b, alpha);
 }
 
 int launch_bmm_s8t_s8t_s8t(const int8_t* a, const int8_t* b, int8_t* c, long long batch, long long M, long long N,
-                           long long K, float alpha, hipStream_t stream) {
+                           long long K, long long stride_b, float alpha, hipStream_t stream) {
   if (batch == 0 || M == 0 || N == 0) return TI_OK;
   const int mr = M == 1 ? 1 : (M <= 4 ? 4 : 16);
   const long long tiles_n = (N + RM_BN - 1) / RM_BN, groups_m = (M + mr - 1) / mr;
   const long long wgs = tiles_n * groups_m * batch;
   if (wgs > 0x7fffffffLL) return fail(TI_ERR_INVALID_ARG, "bmm_s8t_s8t_s8t: too many output tiles (%lld)", wgs);
-  const bool fast = (N % 4 == 0) && (reinterpret_cast<uintptr_t>(b) % 4 == 0) && (reinterpret_cast<uintptr_t>(c) % 4 == 0);
+  const bool fast = (N % 4 == 0) && (stride_b % 4 == 0) && (reinterpret_cast<uintptr_t>(b) % 4 == 0) &&
+                    (reinterpret_cast<uintptr_t>(c) % 4 == 0);
   const dim3 grid((unsigned)wgs);
   if (mr == 1)
-    launch_rm<1>(fast, grid, stream, a, b, c, (int)M, (int)N, (int)K, (int)tiles_n, (int)groups_m, alpha);
+    launch_rm<1>(fast, grid, stream, a, b, c, (int)M, (int)N, (int)K, (int)tiles_n, (int)groups_m, stride_b, alpha);
   else if (mr == 4)
-    launch_rm<4>(fast, grid, stream, a, b, c, (int)M, (int)N, (int)K, (int)tiles_n, (int)groups_m, alpha);
+    launch_rm<4>(fast, grid, stream, a, b, c, (int)M, (int)N, (int)K, (int)tiles_n, (int)groups_m, stride_b, alpha);
   else
-    launch_rm<16>(fast, grid, stream, a, b, c, (int)M, (int)N, (int)K, (int)tiles_n, (int)groups_m, alpha);
+    launch_rm<16>(fast, grid, stream, a, b, c, (int)M, (int)N, (int)K, (int)tiles_n, (int)groups_m, stride_b, alpha);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "bmm_s8t_s8t_s8t launch: %s", hipGetErrorString(e));
   return TI_OK;

@@ -85,6 +85,20 @@ static PyObject* fc_ln_q(PyObject* self, PyObject* const* a, Py_ssize_t n) {
   return PyLong_FromLong(ti_dq_add_layernorm_q(in, scale, res, g, b, eps, ro, qo, rows, H, st));
 }
 
+/* kv_append(k_new, v_new, k_buf, v_buf, BH, T, D, cap, S, stream) -> status */
+static PyObject* fc_kv_append(PyObject* self, PyObject* const* a, Py_ssize_t n) {
+  (void)self;
+  if (n != 10) {
+    PyErr_SetString(PyExc_TypeError, "kv_append expects 10 arguments");
+    return NULL;
+  }
+  void *kn = as_ptr(a[0]), *vn = as_ptr(a[1]), *kb = as_ptr(a[2]), *vb = as_ptr(a[3]);
+  int64_t BH = as_i64(a[4]), T = as_i64(a[5]), D = as_i64(a[6]), cap = as_i64(a[7]), S = as_i64(a[8]);
+  void* st = as_ptr(a[9]);
+  if (PyErr_Occurred()) return NULL;
+  return PyLong_FromLong(ti_kv_append_s8(kn, vn, kb, vb, BH, T, D, cap, S, st));
+}
+
 static PyObject* fc_last_error(PyObject* self, PyObject* noargs) {
   (void)self;
   (void)noargs;
@@ -95,6 +109,7 @@ static PyMethodDef methods[] = {
     {"linear", (PyCFunction)(void (*)(void))fc_linear, METH_FASTCALL, "forward to ti_linear_*"},
     {"bmm", (PyCFunction)(void (*)(void))fc_bmm, METH_FASTCALL, "forward to ti_bmm_*"},
     {"ln_q", (PyCFunction)(void (*)(void))fc_ln_q, METH_FASTCALL, "forward to ti_dq_add_layernorm_q"},
+    {"kv_append", (PyCFunction)(void (*)(void))fc_kv_append, METH_FASTCALL, "forward to ti_kv_append_s8"},
     {"last_error", fc_last_error, METH_NOARGS, "ti_last_error()"},
     {NULL, NULL, 0, NULL}};
 

@@ -2,6 +2,7 @@
 //   permute_0213:  [B, X, Y, D] -> [B, Y, X, D]   (rows of D bytes move intact: the
 //                  head split / merge  view(B,T,H,d).transpose(1,2).contiguous())
 //   transpose_last2: [B, R, C] -> [B, C, R]        (byte transpose: V -> V^T)
+//   kv_append:     kbuf[bh, S + t, :] = knew[bh, t, :] and the same for V, one launch for both caches
 #include "ti_common.h"
 
 namespace ti {
@@ -77,6 +78,44 @@ __global__ __launch_bounds__(256) void transpose_last2_kernel(const int8_t* __re
       }
     }
   }
+}
+
+// rows of D bytes: row r = (bh, t) of the new tokens goes to row (bh * cap + S + t) of the cache buffer;
+// blockIdx.y selects K (0) or V (1).  CH = bytes moved per thread (16 when D and the pointers allow, else 1).
+template <int CH>
+__global__ __launch_bounds__(256) void kv_append_kernel(const int8_t* __restrict__ knew, const int8_t* __restrict__ vnew,
+                                                        int8_t* __restrict__ kbuf, int8_t* __restrict__ vbuf, int T,
+                                                        int per_row, long long cap, long long S, long long total) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const int c = (int)(i % per_row);
+  const long long row = i / per_row;
+  const long long bh = row / T, t = row % T;
+  const int8_t* src = (blockIdx.y ? vnew : knew) + (row * per_row + c) * CH;
+  int8_t* dst = (blockIdx.y ? vbuf : kbuf) + (((bh * cap + S + t) * per_row) + c) * CH;
+  if (CH == 16)
+    *reinterpret_cast<v4i*>(dst) = *reinterpret_cast<const v4i*>(src);
+  else
+    *dst = *src;
+}
+
+int launch_kv_append_s8(const int8_t* knew, const int8_t* vnew, int8_t* kbuf, int8_t* vbuf, long long BH, long long T,
+                        long long D, long long cap, long long S, hipStream_t stream) {
+  const long long bytes = BH * T * D;
+  if (bytes == 0) return TI_OK;
+  const uintptr_t all = reinterpret_cast<uintptr_t>(knew) | reinterpret_cast<uintptr_t>(vnew) |
+                        reinterpret_cast<uintptr_t>(kbuf) | reinterpret_cast<uintptr_t>(vbuf);
+  if (D % 16 == 0 && (all & 15) == 0) {
+    const long long total = bytes / 16;
+    hipLaunchKernelGGL(kv_append_kernel<16>, dim3((unsigned)((total + 255) / 256), 2), dim3(256), 0, stream, knew, vnew,
+                       kbuf, vbuf, (int)T, (int)(D / 16), cap, S, total);
+  } else {
+    hipLaunchKernelGGL(kv_append_kernel<1>, dim3((unsigned)((bytes + 255) / 256), 2), dim3(256), 0, stream, knew, vnew,
+                       kbuf, vbuf, (int)T, (int)D, cap, S, bytes);
+  }
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "kv_append launch: %s", hipGetErrorString(e));
+  return TI_OK;
 }
 
 int launch_permute_0213_s8(const int8_t* src, int8_t* dst, long long B, long long X, long long Y, long long D,

@@ -196,9 +196,11 @@ int launch_permute_0213_s8(const int8_t* src, int8_t* dst, long long B, long lon
                            hipStream_t stream);
 int launch_transpose_last2_s8(const int8_t* src, int8_t* dst, long long B, long long R, long long C,
                               hipStream_t stream);
+int launch_kv_append_s8(const int8_t* knew, const int8_t* vnew, int8_t* kbuf, int8_t* vbuf, long long BH, long long T,
+                        long long D, long long cap, long long S, hipStream_t stream);
 
 // bmm_rowmajor.hip
 int launch_bmm_s8t_s8t_s8t(const int8_t* a, const int8_t* b, int8_t* c, long long batch, long long M, long long N,
-                           long long K, float alpha, hipStream_t stream);
+                           long long K, long long stride_b, float alpha, hipStream_t stream);
 
 }  // namespace ti

@@ -29,9 +29,31 @@ _lib.ti_permute_0213_s8.argtypes = [_vp, _vp, _i64, _i64, _i64, _i64, _vp]
 _lib.ti_permute_0213_s8.restype = ctypes.c_int
 _lib.ti_transpose_last2_s8.argtypes = [_vp, _vp, _i64, _i64, _i64, _vp]
 _lib.ti_transpose_last2_s8.restype = ctypes.c_int
-_lib.ti_bmm_s8t_s8t_s8t.argtypes = [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _f32, _vp]
+_lib.ti_bmm_s8t_s8t_s8t.argtypes = [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _f32, _vp]
 _lib.ti_bmm_s8t_s8t_s8t.restype = ctypes.c_int
+_lib.ti_bmm_s8t_s8n_f32t_strided.argtypes = [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _vp]
+_lib.ti_bmm_s8t_s8n_f32t_strided.restype = ctypes.c_int
+_lib.ti_kv_append_s8.argtypes = [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp]
+_lib.ti_kv_append_s8.restype = ctypes.c_int
 _raw_stream = torch._C._cuda_getCurrentRawStream
+_fast = _CUDA._fast if getattr(_CUDA._fast, "kv_append", None) is not None else None
+
+
+class _NoSwitch:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SWITCH = _NoSwitch()
+_current_device = torch.cuda.current_device
+
+
+def _on(dev):
+    """Context that makes ``dev`` current; free when it already is (the usual case)."""
+    return _NO_SWITCH if dev.index == _current_device() else torch.cuda.device(dev)
 
 
 def _ok(t, dtype):
@@ -44,18 +66,20 @@ def can_fuse_layernorm(x, weight, bias):
             and x.dim() >= 1 and x.shape[-1] == weight.numel() == bias.numel() and x.numel() > 0)
 
 
-def add_layernorm_q(x, residual, weight, bias, eps):
+def add_layernorm_q(x, residual, weight, bias, eps, checked=False):
     """``residual += x`` in place (skipped when ``x`` is None), returns int8
-    ``clamp(round(layer_norm(residual) * weight + bias), -128, 127)``."""
+    ``clamp(round(layer_norm(residual) * weight + bias), -128, 127)``.  ``checked=True``: the caller has
+    already established the conditions below (the modules do, via the ``can_*`` predicates)."""
     op = "add_layernorm_q"
-    if not can_fuse_layernorm(residual, weight, bias):
-        raise RuntimeError(f"torch_int._hip_ext.{op}: needs contiguous fp32 HIP tensors")
-    if x is not None and not (_ok(x, torch.float32) and x.shape == residual.shape and x.device == residual.device):
-        raise RuntimeError(f"torch_int._hip_ext.{op}: x must be a contiguous fp32 tensor shaped like residual")
+    if not checked:
+        if not can_fuse_layernorm(residual, weight, bias):
+            raise RuntimeError(f"torch_int._hip_ext.{op}: needs contiguous fp32 HIP tensors")
+        if x is not None and not (_ok(x, torch.float32) and x.shape == residual.shape and x.device == residual.device):
+            raise RuntimeError(f"torch_int._hip_ext.{op}: x must be a contiguous fp32 tensor shaped like residual")
     dev = residual.device
     H = residual.shape[-1]
     q = torch.empty(residual.shape, dtype=torch.int8, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         rc = _lib.ti_add_layernorm_q(x.data_ptr() if x is not None else None, residual.data_ptr(),
                                      weight.data_ptr(), bias.data_ptr(), float(eps), q.data_ptr(),
                                      residual.numel() // H, H, _raw_stream(dev.index) or None)
@@ -73,18 +97,18 @@ def can_fuse_softmax(scores, mask, bsz, heads):
             and tuple(mask.shape) == (bsz, 1, scores.shape[1], scores.shape[2]))
 
 
-def attn_softmax_q(scores, mask, heads):
+def attn_softmax_q(scores, mask, heads, checked=False):
     """scores fp32 [bsz*heads, T, S], mask fp32 [bsz, 1, T, S] or None ->
     int8 ``round(127 * softmax(max(scores + mask, finfo.min), dim=-1))``."""
     op = "attn_softmax_q"
     BH, T, S = scores.shape
     bsz = BH // heads
-    if bsz * heads != BH or not can_fuse_softmax(scores, mask, bsz, heads):
+    if not checked and (bsz * heads != BH or not can_fuse_softmax(scores, mask, bsz, heads)):
         raise RuntimeError(f"torch_int._hip_ext.{op}: needs contiguous fp32 HIP tensors, scores [bsz*heads,T,S], "
                            f"mask [bsz,1,T,S]")
     dev = scores.device
     out = torch.empty((BH, T, S), dtype=torch.int8, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         rc = _lib.ti_attn_softmax_q(scores.data_ptr(), mask.data_ptr() if mask is not None else None, out.data_ptr(),
                                     bsz, heads, T, S, _raw_stream(dev.index) or None)
     if rc:
@@ -100,7 +124,7 @@ def split_heads(t, bsz, seq_len, heads, head_dim):
     if not (_ok(t, torch.int8) and t.numel() == bsz * seq_len * heads * head_dim and t.numel() > 0):
         return t.view(bsz, seq_len, heads, head_dim).transpose(1, 2).contiguous()
     out = torch.empty((bsz, heads, seq_len, head_dim), dtype=torch.int8, device=t.device)
-    with torch.cuda.device(t.device):
+    with _on(t.device):
         rc = _lib.ti_permute_0213_s8(t.data_ptr(), out.data_ptr(), bsz, seq_len, heads, head_dim,
                                      _raw_stream(t.device.index) or None)
     if rc:
@@ -115,7 +139,7 @@ def merge_heads(t, bsz, heads, seq_len, head_dim):
     if not (_ok(t, torch.int8) and t.numel() == bsz * seq_len * heads * head_dim and t.numel() > 0):
         return t.view(bsz, heads, seq_len, head_dim).transpose(1, 2).reshape(bsz, seq_len, heads * head_dim).contiguous()
     out = torch.empty((bsz, seq_len, heads * head_dim), dtype=torch.int8, device=t.device)
-    with torch.cuda.device(t.device):
+    with _on(t.device):
         rc = _lib.ti_permute_0213_s8(t.data_ptr(), out.data_ptr(), bsz, heads, seq_len, head_dim,
                                      _raw_stream(t.device.index) or None)
     if rc:
@@ -129,29 +153,88 @@ def transpose_last2(t):
         return t.transpose(1, 2).contiguous()
     B, R, C = t.shape
     out = torch.empty((B, C, R), dtype=torch.int8, device=t.device)
-    with torch.cuda.device(t.device):
+    with _on(t.device):
         rc = _lib.ti_transpose_last2_s8(t.data_ptr(), out.data_ptr(), B, R, C, _raw_stream(t.device.index) or None)
     if rc:
         raise RuntimeError(f"torch_int._hip_ext.transpose_last2: {_lib.ti_last_error().decode()} (status {rc})")
     return out
 
 
+def _batch_strided(t):
+    """int8 HIP tensor [B, R, C] whose [R, C] matrices are packed; the batch stride may exceed R*C
+    (a view into a buffer with spare rows, such as a KV cache with room to grow)."""
+    return (isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == torch.int8 and t.dim() == 3
+            and (t.shape[2] == 1 or t.stride(2) == 1) and (t.shape[1] == 1 or t.stride(1) == t.shape[2])
+            and (t.shape[0] == 1 or t.stride(0) >= t.shape[1] * t.shape[2]))
+
+
 def can_bmm_rowmajor(a, b):
-    return (_ok(a, torch.int8) and _ok(b, torch.int8) and a.dim() == 3 and b.dim() == 3 and a.device == b.device
+    return (_ok(a, torch.int8) and _batch_strided(b) and a.dim() == 3 and a.device == b.device
             and a.shape[0] == b.shape[0] and a.shape[2] == b.shape[1] and a.shape[0] <= 65535)
 
 
-def bmm_s8t_s8t_s8t(a, b, alpha):
-    """int8 a [B, M, K], int8 b [B, K, N] (row-major, *not* transposed) -> int8
+def bmm_s8t_s8t_s8t(a, b, alpha, checked=False):
+    """int8 a [B, M, K], int8 b [B, K, N] (row-major, *not* transposed; batch stride free) -> int8
     ``clamp(round(alpha * a @ b), -128, 127)`` [B, M, N].  Streams b once per 16 rows of a."""
-    if not can_bmm_rowmajor(a, b):
-        raise RuntimeError("torch_int._hip_ext.bmm_s8t_s8t_s8t: needs contiguous int8 HIP tensors a [B,M,K], b [B,K,N]")
+    if not checked and not can_bmm_rowmajor(a, b):
+        raise RuntimeError("torch_int._hip_ext.bmm_s8t_s8t_s8t: needs int8 HIP tensors a [B,M,K] (contiguous), "
+                           "b [B,K,N] (each matrix packed)")
     B, M, K = a.shape
     N = b.shape[2]
     out = torch.empty((B, M, N), dtype=torch.int8, device=a.device)
-    with torch.cuda.device(a.device):
-        rc = _lib.ti_bmm_s8t_s8t_s8t(a.data_ptr(), b.data_ptr(), out.data_ptr(), B, M, N, K, float(alpha),
-                                     _raw_stream(a.device.index) or None)
+    with _on(a.device):
+        rc = _lib.ti_bmm_s8t_s8t_s8t(a.data_ptr(), b.data_ptr(), out.data_ptr(), B, M, N, K,
+                                     b.stride(0) if B > 1 else 0, float(alpha), _raw_stream(a.device.index) or None)
     if rc:
         raise RuntimeError(f"torch_int._hip_ext.bmm_s8t_s8t_s8t: {_lib.ti_last_error().decode()} (status {rc})")
     return out
+
+
+def can_bmm_strided(a, b):
+    return (_batch_strided(a) and _batch_strided(b) and a.device == b.device and a.shape[0] == b.shape[0]
+            and a.shape[2] == b.shape[2] and a.shape[0] <= 65535 and a.numel() > 0 and b.numel() > 0)
+
+
+def bmm_s8t_s8n_f32t_strided(a, b, alpha, checked=False):
+    """``_CUDA.bmm_s8t_s8n_f32t`` for operands that are packed per matrix but not along the batch dimension:
+    a [B, M, K], b [B, N, K] -> fp32 alpha * a @ b^T [B, M, N]."""
+    if not checked and not can_bmm_strided(a, b):
+        raise RuntimeError("torch_int._hip_ext.bmm_s8t_s8n_f32t_strided: needs int8 HIP tensors a [B,M,K], b [B,N,K] "
+                           "whose matrices are packed")
+    B, M, K = a.shape
+    N = b.shape[1]
+    out = torch.empty((B, M, N), dtype=torch.float32, device=a.device)
+    with _on(a.device):
+        rc = _lib.ti_bmm_s8t_s8n_f32t_strided(a.data_ptr(), b.data_ptr(), out.data_ptr(), B, M, N, K,
+                                              a.stride(0) if B > 1 else 0, b.stride(0) if B > 1 else 0, float(alpha),
+                                              _raw_stream(a.device.index) or None)
+    if rc:
+        raise RuntimeError(f"torch_int._hip_ext.bmm_s8t_s8n_f32t_strided: {_lib.ti_last_error().decode()} (status {rc})")
+    return out
+
+
+def can_kv_append(k_new, v_new, k_buf, v_buf):
+    """int8 HIP tensors: new [B, H, T, d] contiguous, buffers [B, H, cap, d] contiguous, all on one device."""
+    return (_ok(k_new, torch.int8) and _ok(v_new, torch.int8) and _ok(k_buf, torch.int8) and _ok(v_buf, torch.int8)
+            and k_new.dim() == 4 and k_new.shape == v_new.shape and k_buf.shape == v_buf.shape
+            and k_buf.shape[:2] == k_new.shape[:2] and k_buf.shape[3] == k_new.shape[3]
+            and k_new.device == v_new.device == k_buf.device == v_buf.device)
+
+
+def kv_append(k_new, v_new, k_buf, v_buf, filled, checked=False):
+    """k_buf[:, :, filled:filled+T] = k_new and the same for v, one launch."""
+    if not checked and not can_kv_append(k_new, v_new, k_buf, v_buf):
+        raise RuntimeError("torch_int._hip_ext.kv_append: needs contiguous int8 HIP tensors new [B,H,T,d], buffers [B,H,cap,d]")
+    B, H, T, d = k_new.shape
+    cap = k_buf.shape[2]
+    dev = k_new.device
+    with _on(dev):
+        stream = _raw_stream(dev.index)
+        if _fast is not None:
+            rc = _fast.kv_append(k_new.data_ptr(), v_new.data_ptr(), k_buf.data_ptr(), v_buf.data_ptr(), B * H, T, d,
+                                 cap, filled, stream)
+        else:
+            rc = _lib.ti_kv_append_s8(k_new.data_ptr(), v_new.data_ptr(), k_buf.data_ptr(), v_buf.data_ptr(), B * H, T,
+                                      d, cap, filled, stream or None)
+    if rc:
+        raise RuntimeError(f"torch_int._hip_ext.kv_append: {_lib.ti_last_error().decode()} (status {rc})")

@@ -20,11 +20,83 @@ from ..nn.fused import LayerNormQ
 from ..nn.linear import W8A8B8O8Linear, W8A8B8O8LinearReLU, W8A8BFP32OFP32Linear
 
 
+class _KVBuffer:
+    """Backing store of one growing K or V cache tensor: ``buf`` is [bsz, heads, capacity, head_dim] and the
+    first ``filled`` positions hold tokens.  The tensors handed out as ``past_key_value`` are views
+    ``buf[:, :, :n]`` that carry a reference to this object."""
+    __slots__ = ("buf", "filled")
+
+    def __init__(self, buf, filled):
+        self.buf, self.filled = buf, filled
+
+
+def _kv_room(past, new):
+    """The buffer behind ``past`` when ``new`` can be written right after it, else None."""
+    kv = getattr(past, "_ti_kv", None)
+    S, T = past.shape[2], new.shape[2]
+    if (kv is not None and kv.filled == S and S + T <= kv.buf.shape[2] and past.data_ptr() == kv.buf.data_ptr()
+            and past.stride() == kv.buf.stride() and past.shape[:2] == new.shape[:2] and past.shape[3] == new.shape[3]
+            and past.dtype == new.dtype and past.device == new.device):
+        return kv
+    return None
+
+
+def _kv_fresh(past, T):
+    """A new buffer holding ``past`` with room for T + max(64, a quarter of the length) further positions."""
+    S = past.shape[2]
+    cap = -(-(S + T + max(64, (S + T) // 4)) // 16) * 16
+    buf = torch.empty((past.shape[0], past.shape[1], cap, past.shape[3]), dtype=past.dtype, device=past.device)
+    buf[:, :, :S].copy_(past)
+    return _KVBuffer(buf, S)
+
+
+def _kv_view(kv, n):
+    out = kv.buf[:, :, :n]
+    out._ti_kv = kv
+    return out
+
+
+def _kv_append(past, new):
+    """``torch.cat([past, new], dim=2)`` for [bsz, heads, len, head_dim] cache tensors without re-copying the
+    past: when ``past`` is a view handed out by an earlier call and nothing was appended after it, ``new`` is
+    written into the spare room behind it and a longer view of the same buffer is returned; the values
+    ``past`` shows never change.  Otherwise (first decode step, a cache that was re-indexed or sliced by the
+    caller, a second continuation of the same past, no room left) the result is built in a fresh buffer."""
+    S, T = past.shape[2], new.shape[2]
+    kv = _kv_room(past, new) or _kv_fresh(past, T)
+    kv.buf[:, :, S:S + T].copy_(new)
+    kv.filled = S + T
+    return _kv_view(kv, S + T)
+
+
+def _kv_append_pair(past_k, past_v, new_k, new_v):
+    """``_kv_append`` for the key and the value cache of one layer, with a single copy kernel when both live
+    in HIP buffers of the same shape."""
+    S, T = past_k.shape[2], new_k.shape[2]
+    if past_v.shape[2] != S or new_v.shape[2] != T:
+        return _kv_append(past_k, new_k), _kv_append(past_v, new_v)
+    kk = _kv_room(past_k, new_k) or _kv_fresh(past_k, T)
+    vv = _kv_room(past_v, new_v) or _kv_fresh(past_v, T)
+    if _hip_ext.can_kv_append(new_k, new_v, kk.buf, vv.buf):
+        _hip_ext.kv_append(new_k, new_v, kk.buf, vv.buf, S, checked=True)
+    else:
+        kk.buf[:, :, S:S + T].copy_(new_k)
+        vv.buf[:, :, S:S + T].copy_(new_v)
+    kk.filled = vv.filled = S + T
+    return _kv_view(kk, S + T), _kv_view(vv, S + T)
+
+
 class Int8OPTAttention(nn.Module):
     """Multi-head self-attention with int8 projections and int8 Q.K^T / P.V products.
 
     upstream: ``torch_int/models/opt.py:22-199``.
+
+    ``kv_cache_in_place`` (class attribute, default True): the (key, value) tensors returned for
+    ``past_key_value`` reuse one buffer with spare room, so a decode step appends its token instead of
+    re-copying the whole cache (see ``_kv_append``).  They are then views that are packed per head but not
+    across heads; set it to False to get upstream's freshly concatenated contiguous tensors.
     """
+    kv_cache_in_place = True
 
     def __init__(self, embed_dim: int, num_heads: int):
         super().__init__()
@@ -86,16 +158,24 @@ class Int8OPTAttention(nn.Module):
             key = self._shape(self.k_proj(kv_src), -1, bsz)
             value = self._shape(self.v_proj(kv_src), -1, bsz)
             if not cross and past_key_value is not None:
-                key = torch.cat([past_key_value[0], key], dim=2)
-                value = torch.cat([past_key_value[1], value], dim=2)
+                if self.kv_cache_in_place:
+                    key, value = _kv_append_pair(past_key_value[0], past_key_value[1], key, value)
+                else:
+                    key = torch.cat([past_key_value[0], key], dim=2)
+                    value = torch.cat([past_key_value[1], value], dim=2)
         present = (key, value)
 
         query = self._shape(query, tgt_len, bsz).view(bsz * H, -1, d)
-        key = key.view(bsz * H, -1, d)
-        value = value.view(bsz * H, -1, d)
+        # cache views are packed per head; [bsz, H] merges into one batch dimension either way
+        key = key.view(bsz * H, -1, d) if key.is_contiguous() else key.reshape(bsz * H, key.shape[2], d)
+        value = value.view(bsz * H, -1, d) if value.is_contiguous() else value.reshape(bsz * H, value.shape[2], d)
         src_len = key.size(1)
 
-        scores = self.qk_bmm(query, key)  # fp32 [bsz*H, tgt, src]
+        if (not key.is_contiguous() and type(self.qk_bmm) is BMM_S8T_S8N_F32T
+                and _hip_ext.can_bmm_strided(query, key)):
+            scores = _hip_ext.bmm_s8t_s8n_f32t_strided(query, key, self.qk_bmm._scalar("a"), checked=True)
+        else:
+            scores = self.qk_bmm(query, key.contiguous())  # fp32 [bsz*H, tgt, src]
         if scores.size() != (bsz * H, tgt_len, src_len):
             raise ValueError(f"Attention weights should be of size {(bsz * H, tgt_len, src_len)}, but is"
                              f" {scores.size()}")
@@ -107,7 +187,7 @@ class Int8OPTAttention(nn.Module):
                              f" {layer_head_mask.size()}")
         if layer_head_mask is None and _hip_ext.can_fuse_softmax(scores, attention_mask, bsz, H):
             # mask add, clamp, softmax, *127, round and int8 cast in one kernel
-            probs_q = _hip_ext.attn_softmax_q(scores, attention_mask, H)
+            probs_q = _hip_ext.attn_softmax_q(scores, attention_mask, H, checked=True)
             probs_out = probs_q.view(bsz, H, tgt_len, src_len).float() if output_attentions else None
         else:
             if attention_mask is not None:
@@ -125,10 +205,10 @@ class Int8OPTAttention(nn.Module):
             probs_q = probs.mul_(127).round_().to(torch.int8)
         if tgt_len <= 16 and type(self.pv_bmm) is BMM_S8T_S8N_S8T and _hip_ext.can_bmm_rowmajor(probs_q, value):
             # few query rows (incremental decoding): stream V once, as the cache stores it
-            ctx = _hip_ext.bmm_s8t_s8t_s8t(probs_q, value, self.pv_bmm._scalar("a"))
+            ctx = _hip_ext.bmm_s8t_s8t_s8t(probs_q, value, self.pv_bmm._scalar("a"), checked=True)
         else:
             # P.V with V transposed to [bsz*H, d, src]: (P V) = P . (V^T)^T
-            ctx = self.pv_bmm(probs_q, _hip_ext.transpose_last2(value))  # int8 [bsz*H, tgt, d]
+            ctx = self.pv_bmm(probs_q, _hip_ext.transpose_last2(value.contiguous()))  # int8 [bsz*H, tgt, d]
         if ctx.size() != (bsz * H, tgt_len, d):
             raise ValueError(f"`attn_output` should be of size {(bsz, H, tgt_len, d)}, but is {ctx.size()}")
         ctx = _hip_ext.merge_heads(ctx, bsz, H, tgt_len, d)

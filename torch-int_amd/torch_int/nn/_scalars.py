@@ -10,13 +10,17 @@ import torch
 
 class ScalarCacheMixin:
     def _scalar(self, name):
-        buf = getattr(self, name)
-        if not torch.is_tensor(buf):
-            return float(buf)
-        cache = self.__dict__.setdefault("_scalar_cache", {})
-        key = (id(buf), buf._version)
+        buf = self._buffers.get(name)  # skips nn.Module.__getattr__: this runs several times per kernel launch
+        if buf is None:
+            buf = getattr(self, name)
+            if not torch.is_tensor(buf):
+                return float(buf)
+        cache = self.__dict__.get("_scalar_cache")
+        if cache is None:
+            cache = self.__dict__["_scalar_cache"] = {}
         hit = cache.get(name)
-        if hit is None or hit[0] != key:
-            hit = (key, float(buf.item()))
-            cache[name] = hit
-        return hit[1]
+        if hit is not None and hit[0] is buf and hit[1] == buf._version:
+            return hit[2]
+        value = float(buf.item())
+        cache[name] = (buf, buf._version, value)
+        return value

@@ -14,9 +14,9 @@ class _ScaledBMM(ScalarCacheMixin, torch.nn.Module):
         super().__init__()
         self.register_buffer("a", torch.tensor(alpha))
 
-    @torch.no_grad()
     def forward(self, a, b):
-        """a: int8 [B, M, K]; b: int8 [B, N, K]; returns [B, M, N]."""
+        """a: int8 [B, M, K]; b: int8 [B, N, K]; returns [B, M, N].  (Integer inputs, outputs from
+        torch.empty: nothing can require grad, so no torch.no_grad() context per call.)"""
         return getattr(_CUDA, self._kernel)(a, b, self._scalar("a"))
 
     @staticmethod
@@ -49,6 +49,5 @@ class BMM_S8T_S8N_F32T(_ScaledBMM):
 class BMM_S8T_S8N_S32T(torch.nn.Module):
     """int32 output: the raw accumulators."""
 
-    @torch.no_grad()
     def forward(self, a, b):
         return _CUDA.bmm_s8t_s8n_s32t(a, b)

@@ -24,8 +24,9 @@ class LayerNormQ(_QuantLayerNormBase):
         (``x.add_(add)``, the residual update of the decoder layer) -- fused into the same
         kernel when ``x`` is a contiguous fp32 HIP tensor."""
         if _hip_ext.can_fuse_layernorm(x, self.weight, self.bias) and (
-                add is None or (add.dtype == x.dtype and add.shape == x.shape and add.is_contiguous())):
-            return _hip_ext.add_layernorm_q(add, x, self.weight, self.bias, self.eps)  # one pass, same maths
+                add is None or (add.dtype == x.dtype and add.shape == x.shape and add.device == x.device
+                                and add.is_contiguous())):
+            return _hip_ext.add_layernorm_q(add, x, self.weight, self.bias, self.eps, checked=True)  # one pass, same maths
         if add is not None:
             x.add_(add.to(x.dtype))
         y = F.layer_norm(x.to(self.weight.dtype), x.shape[-1:], self.weight, self.bias, self.eps)

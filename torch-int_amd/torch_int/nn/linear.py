@@ -43,8 +43,19 @@ class _W8A8Base(ScalarCacheMixin, torch.nn.Module):
     def _run(self, x):
         raise NotImplementedError
 
-    @torch.no_grad()
+    def _wb(self):
+        """(weight, bias) without the cost of two nn.Module.__getattr__ calls; from_float may have left
+        either as a Parameter (it assigns the float module's tensors), hence the fallback."""
+        b = self._buffers
+        w, bias = b.get("weight"), b.get("bias")
+        return (w if w is not None else self.weight), (bias if bias is not None else self.bias)
+
+    # No torch.no_grad() here (upstream decorates forward): the inputs are integer tensors and the outputs
+    # come from torch.empty, so nothing can require grad, and the context manager costs a microsecond or two
+    # on a path where a decode-sized kernel takes about five.
     def forward(self, x):
+        if x.dim() == 2:
+            return self._run(x)
         lead = x.shape[:-1]
         y = self._run(x.reshape(-1, x.shape[-1]))
         return y.view(*lead, -1)
@@ -62,7 +73,8 @@ class W8A8B8O8Linear(_W8A8Base):
         self._register_scales(alpha, beta)
 
     def _run(self, x):
-        return _CUDA.linear_a8_w8_b8_o8(x, self.weight, self.bias, self._scalar("a"), self._scalar("b"))
+        w, bias = self._wb()
+        return _CUDA.linear_a8_w8_b8_o8(x, w, bias, self._scalar("a"), self._scalar("b"))
 
     @classmethod
     def from_float(cls, module, input_scale, output_scale):
@@ -78,7 +90,8 @@ class W8A8B8O8LinearReLU(W8A8B8O8Linear):
     """As W8A8B8O8Linear with a fused ReLU: outputs in [0, 127] (fc1)."""
 
     def _run(self, x):
-        return _CUDA.linear_relu_a8_w8_b8_o8(x, self.weight, self.bias, self._scalar("a"), self._scalar("b"))
+        w, bias = self._wb()
+        return _CUDA.linear_relu_a8_w8_b8_o8(x, w, bias, self._scalar("a"), self._scalar("b"))
 
 
 class W8A8B32O32LinearWithoutScaling(_W8A8Base):
@@ -135,11 +148,11 @@ class W8A8BFP32OFP32Linear(_W8A8Base):
         return self
 
     def _run(self, x):
-        if self.bias.dtype != torch.float32:
-            self.bias = self.bias.to(torch.float32)
-        return _CUDA.linear_a8_w8_bfp32_ofp32(x, self.weight, self.bias, self._scalar("a"), 1)
+        w, bias = self._wb()
+        if bias.dtype != torch.float32:
+            self.bias = bias = bias.to(torch.float32)
+        return _CUDA.linear_a8_w8_bfp32_ofp32(x, w, bias, self._scalar("a"), 1)
 
-    @torch.no_grad()
     def forward(self, x, add_to=None):
         """``add_to`` (not in upstream): a contiguous fp32 tensor shaped like the output; the result is added
         into it in place by the GEMM epilogue (``add_to.add_(linear(x))`` without the intermediate) and
@@ -153,11 +166,12 @@ class W8A8BFP32OFP32Linear(_W8A8Base):
                 and add_to.shape == x.shape[:-1] + (self.out_features,) and add_to.numel() <= 4096 * self.out_features
                 and hasattr(_CUDA, "_linear_a8_w8_bfp32_ofp32_acc"))
         if not fits:
-            return add_to.add_(super().forward(x).to(add_to.dtype))
-        if self.bias.dtype != torch.float32:
-            self.bias = self.bias.to(torch.float32)
-        _CUDA._linear_a8_w8_bfp32_ofp32_acc(x.reshape(-1, x.shape[-1]), self.weight, self.bias, self._scalar("a"), 1,
-                                            add_to)
+            with torch.no_grad():
+                return add_to.add_(super().forward(x).to(add_to.dtype))
+        w, bias = self._wb()
+        if bias.dtype != torch.float32:
+            self.bias = bias = bias.to(torch.float32)
+        _CUDA._linear_a8_w8_bfp32_ofp32_acc(x.reshape(-1, x.shape[-1]), w, bias, self._scalar("a"), 1, add_to)
         return add_to
 
     @classmethod
