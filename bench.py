@@ -276,22 +276,23 @@ def main():
         mfma_ops = mfma_ms = 0.0
         copies = {}
         for c in cases:
-            bound = "mfma" if c["M"] >= 2048 else "hbm"
+            # the binding roofline by arithmetic intensity (ridge = 5000 TOP/s / 8000 GB/s = 625 ops per byte)
+            bound = "mfma" if c["ops"] / c["bytes"] >= PEAK_INT8_TOPS * 1e3 / PEAK_HBM_GBS else "hbm"
             fns = [c["fn"]]
-            if bound == "hbm":
+            if c["M"] < 2048:   # weights dominate the traffic: keep them out of the last-level cache
                 key = (c["N"], c["K"])
                 if key not in copies:
                     n_copies = -(-320 * 2 ** 20 // (c["N"] * c["K"]))
                     copies[key] = [c["w"]] + [c["w"].clone() for _ in range(n_copies - 1)]
                 fns = [c["make"](w) for w in copies[key]]
-            ms = sustained_ms(torch, fns, window_ms=200.0 if bound == "mfma" else 60.0)
+            ms = sustained_ms(torch, fns, window_ms=200.0 if c["M"] >= 2048 else 60.0)
             tops = c["ops"] / ms / 1e9
             gbs = c["bytes"] / ms / 1e6
             frac = tops / PEAK_INT8_TOPS if bound == "mfma" else gbs / PEAK_HBM_GBS
             table.append({"variant": c["variant"], "M": c["M"], "N": c["N"], "K": c["K"], "kernel": c["kernel"],
                           "us": round(ms * 1e3, 2),
                           "TOPS": round(tops, 1), "GBps": round(gbs, 1), "bound": bound, "frac": round(frac, 4)})
-            if c["kernel"] == DOMINANT and bound == "mfma":
+            if c["kernel"] == DOMINANT and c["M"] >= 2048:
                 mfma_ops += c["ops"]
                 mfma_ms += ms
         del copies
