@@ -61,6 +61,18 @@ def test_c_abi_rejects_bad_arguments_without_a_device():
     # beyond the 32-bit tiling limits
     rc = lib.ti_linear_a8_w8_b32_o32(p, p, p, p, 1 << 20, 4, 1 << 20, None, 0, None)
     assert rc == 1 and b"limits" in lib.ti_last_error()
+    # batch strides smaller than one matrix; a cache append that does not fit; the row-major product's stride
+    i64 = ctypes.c_int64
+    lib.ti_bmm_s8t_s8n_f32t_strided.argtypes = [ctypes.c_void_p] * 3 + [i64] * 6 + [ctypes.c_float, ctypes.c_void_p]
+    rc = lib.ti_bmm_s8t_s8n_f32t_strided(p, p, p, 2, 1, 4, 16, 8, 64, 1.0, None)
+    assert rc == 1 and b"batch strides" in lib.ti_last_error()
+    lib.ti_kv_append_s8.argtypes = [ctypes.c_void_p] * 4 + [i64] * 5 + [ctypes.c_void_p]
+    rc = lib.ti_kv_append_s8(p, p, p, p, 2, 3, 16, 10, 8, None)
+    assert rc == 1 and b"do not fit" in lib.ti_last_error()
+    lib.ti_bmm_s8t_s8t_s8t.argtypes = [ctypes.c_void_p] * 3 + [i64] * 5 + [ctypes.c_float, ctypes.c_void_p]
+    rc = lib.ti_bmm_s8t_s8t_s8t(p, p, p, 2, 1, 4, 16, 8, 1.0, None)
+    assert rc == 1 and b"batch stride" in lib.ti_last_error()
+    assert lib.ti_kv_append_s8(None, None, None, None, 0, 1, 16, 8, 0, None) == 0
     # empty problems succeed without touching pointers or a device
     assert lib.ti_linear_a8_w8_b8_o8(None, None, None, None, 0, 16, 16, 1.0, 1.0, None, 0, None) == 0
     assert lib.ti_dq_add_layernorm_q(None, 1.0, None, None, None, 1e-5, None, None, 0, 128, None) == 0
