@@ -85,6 +85,16 @@ int ti_linear_a8_w8_b8_o8(const int8_t* x, const int8_t* w, const int8_t* bias, 
                           int64_t M, int64_t N, int64_t K, float alpha, float beta,
                           void* workspace, int64_t workspace_bytes, void* stream);
 
+/* `count` (<= 4) linear_a8_w8_b8_o8 problems that share the input x[M,K] and the shape: out[i] =
+ * s8(rint(clamp(alpha[i]*(x . w[i]^T) + beta[i]*bias[i]))).  w, bias, out, alpha, beta are HOST arrays of
+ * `count` device pointers / scalars.  The q, k and v projections of one attention block
+ * (torch_int/models/opt.py:108-126 calls them one after the other); for M <= 16 with K % 1024 == 0 all
+ * weights are streamed by a single launch, other shapes run problem by problem.  Results are those of
+ * `count` separate calls. */
+int ti_linear_a8_w8_b8_o8_group(const int8_t* x, const int8_t* const* w, const int8_t* const* bias,
+                                int8_t* const* out, const float* alpha, const float* beta, int64_t count,
+                                int64_t M, int64_t N, int64_t K, void* stream);
+
 /* replaces linear_relu_a8_w8_b8_o8 (linear.cu:476-625; linear.h:28-33):
  * out = s8(rint(min(max(alpha*acc + beta*bias, 0), 127))). */
 int ti_linear_relu_a8_w8_b8_o8(const int8_t* x, const int8_t* w, const int8_t* bias, int8_t* out,

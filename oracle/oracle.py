@@ -245,3 +245,8 @@ def bmm_s8t_s8t_s8t(a, b, alpha):
 def linear_a8_w8_bfp32_ofp32_acc(x, w, bias, alpha, beta, inout, acc_fn=gemm_acc):
     """ti_linear_a8_w8_bfp32_ofp32_acc: the fp32 linear, rounded, then one fp32 add into ``inout`` (returns a new tensor)."""
     return inout + linear_a8_w8_bfp32_ofp32(x, w, bias, alpha, beta, acc_fn=acc_fn).view(inout.shape)
+
+
+def linear_a8_w8_b8_o8_group(x, weights, biases, alphas, betas):
+    """ti_linear_a8_w8_b8_o8_group: the separate linears, one after the other."""
+    return tuple(linear_a8_w8_b8_o8(x, w, b, a, be) for w, b, a, be in zip(weights, biases, alphas, betas))

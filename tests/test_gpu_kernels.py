@@ -488,6 +488,28 @@ def test_bmm_rowmajor_rhs_for_decode():
     assert torch.equal(out, orc.bmm_s8t_s8t_s8t(a, b[:, 1:, :].contiguous(), 0.001))
 
 
+def test_grouped_qkv_linear():
+    import ctypes
+    import torch_int._CUDA as C
+    import torch_int._hip_ext as X
+    C._lib.ti_last_kernel.restype = ctypes.c_char_p
+    g = torch.Generator().manual_seed(29)
+    for (M, N, K, n, family) in [(4, 5120, 5120, 3, "stream_group"), (1, 2048, 1024, 3, "stream_group"),
+                                 (16, 1536, 2048, 4, "stream_group"), (9, 4100, 3072, 2, "stream_group"),
+                                 (4, 640, 1024, 3, None), (40, 512, 256, 3, None), (3, 100, 272, 1, None)]:
+        _say(f"grouped linear M={M} N={N} K={K} n={n}")
+        x = _s8(g, M, K)
+        ws, bs = [_s8(g, N, K) for _ in range(n)], [_s8(g, N) for _ in range(n)]
+        al, be = [_scal(g, 1e-4, 1e-2) for _ in range(n)], [_scal(g, 1e-4, 1e-2) for _ in range(n)]
+        ref = orc.linear_a8_w8_b8_o8_group(x, ws, bs, al, be)
+        out = X.linear_a8_w8_b8_o8_group(x.to(DEV), [w.to(DEV) for w in ws], [b.to(DEV) for b in bs], al, be)
+        assert len(out) == n
+        for o, r_ in zip(out, ref):
+            assert torch.equal(o.cpu(), r_), (M, N, K)
+        if family:
+            assert C._lib.ti_last_kernel().decode() == family
+
+
 def test_kv_append_kernel():
     import torch_int._hip_ext as X
     g = torch.Generator().manual_seed(17)

@@ -135,6 +135,49 @@ int ti_linear_a8_w8_b8_o8(const int8_t* x, const int8_t* w, const int8_t* bias, 
                   ws_bytes, stream);
 }
 
+int ti_linear_a8_w8_b8_o8_group(const int8_t* x, const int8_t* const* w, const int8_t* const* bias, int8_t* const* out,
+                                const float* alpha, const float* beta, int64_t count, int64_t M, int64_t N,
+                                int64_t K, void* stream) {
+  g_err[0] = 0;
+  const char* op = "linear_a8_w8_b8_o8_group";
+  if (count < 0 || count > 4) return fail(TI_ERR_INVALID_ARG, "%s: 0 to 4 problems per group, got %lld", op, (long long)count);
+  if (int rc = check_dims(op, 1, M, N, K)) return rc;
+  const bool nonempty = count > 0 && M > 0 && N > 0;
+  if (!nonempty) return TI_OK;
+  if (w == nullptr || bias == nullptr || out == nullptr || alpha == nullptr || beta == nullptr)
+    return fail(TI_ERR_INVALID_ARG, "%s: a per-problem array is NULL", op);
+  if (int rc = check_ptr(op, "input", x, 1, K > 0)) return rc;
+  GemmGroup grp{};
+  grp.count = (int)count;
+  for (int i = 0; i < count; ++i) {
+    if (int rc = check_ptr(op, "weight", w[i], 1, K > 0)) return rc;
+    if (int rc = check_ptr(op, "bias", bias[i], 1, true)) return rc;
+    if (int rc = check_ptr(op, "output", out[i], 1, true)) return rc;
+    grp.B[i] = w[i];
+    grp.bias[i] = bias[i];
+    grp.C[i] = out[i];
+    grp.alpha[i] = alpha[i];
+    grp.beta[i] = beta[i];
+  }
+  GemmParams p;
+  p.A = x;
+  p.B = grp.B[0];
+  p.bias = grp.bias[0];
+  p.C = grp.C[0];
+  p.M = (int)M;
+  p.N = (int)N;
+  p.K = (int)K;
+  p.batch = 1;
+  p.lda = (int)K;
+  p.ldb = (int)K;
+  p.strideA = M * K;
+  p.strideB = N * K;
+  p.strideC = M * N;
+  p.alpha = grp.alpha[0];
+  p.beta = grp.beta[0];
+  return launch_gemm_group_s8(p, grp, static_cast<hipStream_t>(stream));
+}
+
 int ti_linear_relu_a8_w8_b8_o8(const int8_t* x, const int8_t* w, const int8_t* bias, int8_t* out, int64_t M,
                                int64_t N, int64_t K, float alpha, float beta, void* ws, int64_t ws_bytes,
                                void* stream) {

@@ -85,6 +85,25 @@ static PyObject* fc_ln_q(PyObject* self, PyObject* const* a, Py_ssize_t n) {
   return PyLong_FromLong(ti_dq_add_layernorm_q(in, scale, res, g, b, eps, ro, qo, rows, H, st));
 }
 
+/* linear_group3(x, w0, w1, w2, b0, b1, b2, o0, o1, o2, M, N, K, a0, a1, a2, be0, be1, be2, stream) -> status */
+static PyObject* fc_linear_group3(PyObject* self, PyObject* const* a, Py_ssize_t n) {
+  (void)self;
+  if (n != 20) {
+    PyErr_SetString(PyExc_TypeError, "linear_group3 expects 20 arguments");
+    return NULL;
+  }
+  const int8_t* x = (const int8_t*)as_ptr(a[0]);
+  const int8_t* w[3] = {(const int8_t*)as_ptr(a[1]), (const int8_t*)as_ptr(a[2]), (const int8_t*)as_ptr(a[3])};
+  const int8_t* b[3] = {(const int8_t*)as_ptr(a[4]), (const int8_t*)as_ptr(a[5]), (const int8_t*)as_ptr(a[6])};
+  int8_t* o[3] = {(int8_t*)as_ptr(a[7]), (int8_t*)as_ptr(a[8]), (int8_t*)as_ptr(a[9])};
+  int64_t M = as_i64(a[10]), N = as_i64(a[11]), K = as_i64(a[12]);
+  float al[3] = {as_f32(a[13]), as_f32(a[14]), as_f32(a[15])};
+  float be[3] = {as_f32(a[16]), as_f32(a[17]), as_f32(a[18])};
+  void* st = as_ptr(a[19]);
+  if (PyErr_Occurred()) return NULL;
+  return PyLong_FromLong(ti_linear_a8_w8_b8_o8_group(x, w, b, o, al, be, 3, M, N, K, st));
+}
+
 /* kv_append(k_new, v_new, k_buf, v_buf, BH, T, D, cap, S, stream) -> status */
 static PyObject* fc_kv_append(PyObject* self, PyObject* const* a, Py_ssize_t n) {
   (void)self;
@@ -109,6 +128,7 @@ static PyMethodDef methods[] = {
     {"linear", (PyCFunction)(void (*)(void))fc_linear, METH_FASTCALL, "forward to ti_linear_*"},
     {"bmm", (PyCFunction)(void (*)(void))fc_bmm, METH_FASTCALL, "forward to ti_bmm_*"},
     {"ln_q", (PyCFunction)(void (*)(void))fc_ln_q, METH_FASTCALL, "forward to ti_dq_add_layernorm_q"},
+    {"linear_group3", (PyCFunction)(void (*)(void))fc_linear_group3, METH_FASTCALL, "forward to ti_linear_a8_w8_b8_o8_group"},
     {"kv_append", (PyCFunction)(void (*)(void))fc_kv_append, METH_FASTCALL, "forward to ti_kv_append_s8"},
     {"last_error", fc_last_error, METH_NOARGS, "ti_last_error()"},
     {NULL, NULL, 0, NULL}};

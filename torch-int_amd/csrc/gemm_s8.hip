@@ -966,8 +966,11 @@ static constexpr int SBK = 1024;
 static constexpr int S_RED = 3 * 256 * 4;  // partial tiles of waves 1..3
 
 // MX = activation rows staged per block (1, 4 or 16 >= M); S = LDS stages.
-template <int KIND, int MX, int S>
-__global__ __launch_bounds__(256) void gemm_stream_kernel(GemmParams p, int strips_per_batch, int strips) {
+// GROUPED: the "batches" are the problems of a GemmGroup (same activations and shape; weight, bias,
+// output and scales per problem) instead of slices of one strided tensor.
+template <int KIND, int MX, int S, bool GROUPED = false>
+__global__ __launch_bounds__(256) void gemm_stream_kernel(GemmParams p, int strips_per_batch, int strips,
+                                                          GemmGroup grp) {
   constexpr int ROWS = 16 + MX;              // row copies per block
   constexpr int COPIES = (ROWS + 3) / 4;     // per wave; indices past ROWS repeat the last row copy
   constexpr int STAGE = ROWS * SBK;
@@ -987,8 +990,8 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(GemmParams p, int stri
   auto set_copy_strip = [&](int strip) {
     const int b = strip / strips_per_batch;
     const int n0 = (strip - b * strips_per_batch) * 16;
-    const int8_t* A = p.A + (long long)b * p.strideA;
-    const int8_t* B = p.B + (long long)b * p.strideB;
+    const int8_t* A = GROUPED ? p.A : p.A + (long long)b * p.strideA;
+    const int8_t* B = GROUPED ? grp.B[b] : p.B + (long long)b * p.strideB;
 #pragma unroll
     for (int i = 0; i < COPIES; ++i) {
       int q = wave + 4 * i;
@@ -1071,7 +1074,16 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(GemmParams p, int stri
 #pragma unroll
           for (int v = 0; v < 4; ++v) acc[v] += red[w * 256 + v * 64 + lane];
         const int b = strip / strips_per_batch;
-        if (r < M) store_skinny_tile<KIND>(acc, p, b, r, (strip - b * strips_per_batch) * 16 + 4 * g);
+        if (GROUPED) {
+          GemmParams q = p;  // problem b of the group as a one-batch problem
+          q.bias = grp.bias[b];
+          q.C = grp.C[b];
+          q.alpha = grp.alpha[b];
+          q.beta = grp.beta[b];
+          if (r < M) store_skinny_tile<KIND>(acc, q, 0, r, (strip - b * strips_per_batch) * 16 + 4 * g);
+        } else if (r < M) {
+          store_skinny_tile<KIND>(acc, p, b, r, (strip - b * strips_per_batch) * 16 + 4 * g);
+        }
       }
       // the next write to red[] is at least one workgroup barrier (top of the next block) away
       acc = v4i{0, 0, 0, 0};
@@ -1306,7 +1318,7 @@ static int launch_kind(const GemmParams& p, void* workspace, long long workspace
       }
       const long long slots = (long long)cus * per_cu;
       hipLaunchKernelGGL(kern, dim3((unsigned)(strips < slots ? strips : slots)), dim3(256), lds, stream, p, spb,
-                         (int)strips);
+                         (int)strips, GemmGroup{});
       hipError_t e = hipGetLastError();
       if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "gemm launch: %s", hipGetErrorString(e));
       return TI_OK;
@@ -1403,6 +1415,50 @@ static int launch_kind(const GemmParams& p, void* workspace, long long workspace
   }
   g_last_kernel = "tile_64x64";
   return launch_tile<TileCfg<64, 64, 2, 2, KIND, SWAP>>(p, stream);
+}
+
+// q/k/v-style group of s8 linears.  Decode shapes (M <= 16, K % 1024 == 0, enough strips) take one launch
+// of the streaming kernel over all the weights; anything else runs problem by problem.
+int launch_gemm_group_s8(const GemmParams& shape, const GemmGroup& grp, hipStream_t stream) {
+  constexpr int KIND = EPI_S8_BIAS;
+  if (shape.M == 0 || shape.N == 0 || grp.count == 0) return TI_OK;
+  bool aligned = (shape.K % SBK == 0) && shape.K > 0 && (reinterpret_cast<uintptr_t>(shape.A) & 15) == 0;
+  for (int i = 0; i < grp.count; ++i) aligned = aligned && (reinterpret_cast<uintptr_t>(grp.B[i]) & 15) == 0;
+  const int spb = (shape.N + 15) / 16;
+  const long long strips = (long long)spb * grp.count;
+  if (aligned && shape.M <= 16 && strips >= 256) {
+    g_last_kernel = "stream_group";
+    const int cus = num_cus();
+    auto launch = [&](auto kern, int rows, int per_cu) -> int {
+      const int lds = 2 * rows * SBK + S_RED;
+      static bool attr_set = false;
+      if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+        attr_set = true;
+      }
+      const long long slots = (long long)cus * per_cu;
+      hipLaunchKernelGGL(kern, dim3((unsigned)(strips < slots ? strips : slots)), dim3(256), lds, stream, shape, spb,
+                         (int)strips, grp);
+      hipError_t e = hipGetLastError();
+      if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "gemm launch: %s", hipGetErrorString(e));
+      return TI_OK;
+    };
+    if (shape.M == 1) return launch(gemm_stream_kernel<KIND, 1, 2, true>, 17, 4);
+    if (shape.M <= 4) return launch(gemm_stream_kernel<KIND, 4, 2, true>, 20, 3);
+    return launch(gemm_stream_kernel<KIND, 16, 2, true>, 32, 2);
+  }
+  for (int i = 0; i < grp.count; ++i) {
+    GemmParams q = shape;
+    q.B = grp.B[i];
+    q.bias = grp.bias[i];
+    q.C = grp.C[i];
+    q.alpha = grp.alpha[i];
+    q.beta = grp.beta[i];
+    if (int rc = launch_kind<KIND>(q, nullptr, 0, stream)) return rc;
+  }
+  return TI_OK;
 }
 
 int launch_gemm(int kind, const GemmParams& p, void* ws, long long ws_bytes, hipStream_t stream) {

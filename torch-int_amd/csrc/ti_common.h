@@ -173,6 +173,17 @@ struct GemmParams {
   float alpha, beta;
 };
 
+// Up to four linears that share the activation matrix and the shape (the q/k/v projections of one
+// attention block) run as one launch: problem i has its own weight, bias, output and scales.
+struct GemmGroup {
+  const int8_t* B[4];
+  const void* bias[4];
+  void* C[4];
+  float alpha[4], beta[4];
+  int count;
+};
+int launch_gemm_group_s8(const GemmParams& shape, const GemmGroup& grp, hipStream_t stream);
+
 // Launchers (gemm_s8.hip).  `kind` is an EpiKind.  Returns a TI_* status.
 int launch_gemm(int kind, const GemmParams& p, void* workspace, long long workspace_bytes,
                 hipStream_t stream);

@@ -35,8 +35,13 @@ _lib.ti_bmm_s8t_s8n_f32t_strided.argtypes = [_vp, _vp, _vp, _i64, _i64, _i64, _i
 _lib.ti_bmm_s8t_s8n_f32t_strided.restype = ctypes.c_int
 _lib.ti_kv_append_s8.argtypes = [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp]
 _lib.ti_kv_append_s8.restype = ctypes.c_int
+_pp = ctypes.POINTER(ctypes.c_void_p)
+_lib.ti_linear_a8_w8_b8_o8_group.argtypes = [_vp, _pp, _pp, _pp, ctypes.POINTER(_f32), ctypes.POINTER(_f32), _i64, _i64,
+                                            _i64, _i64, _vp]
+_lib.ti_linear_a8_w8_b8_o8_group.restype = ctypes.c_int
 _raw_stream = torch._C._cuda_getCurrentRawStream
 _fast = _CUDA._fast if getattr(_CUDA._fast, "kv_append", None) is not None else None
+_fast_group3 = getattr(_CUDA._fast, "linear_group3", None)
 
 
 class _NoSwitch:
@@ -238,3 +243,47 @@ def kv_append(k_new, v_new, k_buf, v_buf, filled, checked=False):
                                       d, cap, filled, stream or None)
     if rc:
         raise RuntimeError(f"torch_int._hip_ext.kv_append: {_lib.ti_last_error().decode()} (status {rc})")
+
+
+def can_linear_group(x, weights, biases):
+    """One int8 HIP activation matrix [M, K] (contiguous) and up to four contiguous int8 weights [N, K] of one
+    shape with int8 biases of N elements, all on one device."""
+    if not (_ok(x, torch.int8) and x.dim() == 2 and 1 <= len(weights) == len(biases) <= 4 and x.numel() > 0):
+        return False
+    N, K = weights[0].shape[0], x.shape[1]
+    for w, b in zip(weights, biases):
+        if not (_ok(w, torch.int8) and _ok(b, torch.int8) and w.dim() == 2 and w.shape[0] == N and w.shape[1] == K
+                and b.numel() == N and w.device == x.device and b.device == x.device):
+            return False
+    return True
+
+
+def linear_a8_w8_b8_o8_group(x, weights, biases, alphas, betas, checked=False):
+    """``[_CUDA.linear_a8_w8_b8_o8(x, w, b, a, be) for ...]`` as one call: a tuple of int8 [M, N] outputs (views
+    of one allocation).  For decode-sized M the weights are streamed by a single kernel launch."""
+    if not checked and not can_linear_group(x, weights, biases):
+        raise RuntimeError("torch_int._hip_ext.linear_a8_w8_b8_o8_group: needs a contiguous int8 HIP input [M,K] and "
+                           "1-4 contiguous int8 weights [N,K] / biases [N] of one shape on the same device")
+    n = len(weights)
+    M, K = x.shape
+    N = weights[0].shape[0]
+    out = torch.empty((n, M, N), dtype=torch.int8, device=x.device)
+    step = M * N
+    base = out.data_ptr()
+    with _on(x.device):
+        stream = _raw_stream(x.device.index)
+        if n == 3 and _fast_group3 is not None:
+            rc = _fast_group3(x.data_ptr(), weights[0].data_ptr(), weights[1].data_ptr(), weights[2].data_ptr(),
+                              biases[0].data_ptr(), biases[1].data_ptr(), biases[2].data_ptr(), base, base + step,
+                              base + 2 * step, M, N, K, float(alphas[0]), float(alphas[1]), float(alphas[2]),
+                              float(betas[0]), float(betas[1]), float(betas[2]), stream)
+        else:
+            arr = ctypes.c_void_p * n
+            farr = _f32 * n
+            rc = _lib.ti_linear_a8_w8_b8_o8_group(
+                x.data_ptr(), arr(*[w.data_ptr() for w in weights]), arr(*[b.data_ptr() for b in biases]),
+                arr(*[base + i * step for i in range(n)]), farr(*[float(a) for a in alphas]),
+                farr(*[float(b) for b in betas]), n, M, N, K, stream or None)
+    if rc:
+        raise RuntimeError(f"torch_int._hip_ext.linear_a8_w8_b8_o8_group: {_lib.ti_last_error().decode()} (status {rc})")
+    return out.unbind(0)

@@ -133,6 +133,23 @@ class Int8OPTAttention(nn.Module):
         q.pv_bmm = BMM_S8T_S8N_S8T.from_scale(1.0 / 127, v_output_scale, out_input_scale)
         return q
 
+    def _qkv_grouped(self, hidden_states):
+        """(q, k, v) projections [bsz, tgt, embed] from one grouped call, or None when the three layers are not
+        plain W8A8B8O8Linear of one shape on contiguous HIP tensors."""
+        q, k, v = self.q_proj, self.k_proj, self.v_proj
+        if not (type(q) is W8A8B8O8Linear and type(k) is W8A8B8O8Linear and type(v) is W8A8B8O8Linear):
+            return None
+        x = hidden_states.reshape(-1, hidden_states.shape[-1])
+        (wq, bq), (wk, bk), (wv, bv) = q._wb(), k._wb(), v._wb()
+        weights, biases = (wq, wk, wv), (bq.reshape(-1), bk.reshape(-1), bv.reshape(-1))
+        if not _hip_ext.can_linear_group(x, weights, biases):
+            return None
+        outs = _hip_ext.linear_a8_w8_b8_o8_group(
+            x, weights, biases, (q._scalar("a"), k._scalar("a"), v._scalar("a")),
+            (q._scalar("b"), k._scalar("b"), v._scalar("b")), checked=True)
+        lead = hidden_states.shape[:-1]
+        return tuple(o.view(*lead, -1) for o in outs)
+
     def _shape(self, tensor: torch.Tensor, seq_len: int, bsz: int):
         """[bsz, seq, embed] -> contiguous [bsz, heads, seq, head_dim]."""
         if seq_len < 0:
@@ -150,13 +167,16 @@ class Int8OPTAttention(nn.Module):
         bsz, tgt_len, _ = hidden_states.size()
         H, d = self.num_heads, self.head_dim
 
-        query = self.q_proj(hidden_states)
+        grouped = None
+        if not cross and bsz * tgt_len <= 16 and hidden_states.is_cuda:
+            grouped = self._qkv_grouped(hidden_states)  # decode: one launch streams all three weights
+        query = self.q_proj(hidden_states) if grouped is None else grouped[0]
         if cross and past_key_value is not None:
             key, value = past_key_value
         else:
             kv_src = key_value_states if cross else hidden_states
-            key = self._shape(self.k_proj(kv_src), -1, bsz)
-            value = self._shape(self.v_proj(kv_src), -1, bsz)
+            key = self._shape(self.k_proj(kv_src) if grouped is None else grouped[1], -1, bsz)
+            value = self._shape(self.v_proj(kv_src) if grouped is None else grouped[2], -1, bsz)
             if not cross and past_key_value is not None:
                 if self.kv_cache_in_place:
                     key, value = _kv_append_pair(past_key_value[0], past_key_value[1], key, value)
