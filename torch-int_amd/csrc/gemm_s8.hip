@@ -180,9 +180,6 @@ __device__ __forceinline__ void store_tile(v16i (&acc)[Cfg::TM][Cfg::TN], const 
 
 template <class Cfg>
 __global__ __launch_bounds__(Cfg::NT) void gemm_tile_kernel(GemmParams p, int tiles_m, int tiles_n) {
-  using E = Epi<Cfg::KIND>;
-  using Out = typename E::Out;
-  using BiasT = typename E::Bias;
   constexpr int BM = Cfg::BM, BN = Cfg::BN, NT = Cfg::NT, TM = Cfg::TM, TN = Cfg::TN;
   constexpr bool SWAP = Cfg::SWAP;
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -881,9 +878,6 @@ __device__ __forceinline__ void store_skinny_tile(v4i acc, const GemmParams& p, 
 // keeps NBLK KiB of weights in flight.
 template <int NBLK, int KIND>
 __global__ __launch_bounds__(1024) void gemm_skinny_kernel(GemmParams p) {
-  using E = Epi<KIND>;
-  using Out = typename E::Out;
-  using BiasT = typename E::Bias;
   extern __shared__ int red[];  // [NW - 1][256]
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1129,16 +1123,26 @@ __global__ __launch_bounds__(256) void gemm_scalar_kernel(GemmParams p) {
 
 // ------------------------------------------------------------------ host side
 
+// Raises a kernel's dynamic-LDS limit once per device.  `done` is the caller's per-instantiation bit mask of
+// devices already handled (benign race: setting the attribute twice is harmless).
+template <class Kern>
+static int allow_lds(Kern kern, int bytes, unsigned long long& done) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) dev = 0;
+  const unsigned long long bit = 1ull << (dev & 63);
+  if (done & bit) return TI_OK;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     bytes);
+  if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+  done |= bit;
+  return TI_OK;
+}
+
 template <class Cfg>
 static int launch_tile(const GemmParams& p, hipStream_t stream) {
-  static bool attr_set = false;  // benign race: setting the attribute twice is harmless
+  static unsigned long long lds_ok = 0;
   auto kern = gemm_tile_kernel<Cfg>;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
-    if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    attr_set = true;
-  }
+  if (int rc = allow_lds(kern, Cfg::LDS_BYTES, lds_ok)) return rc;
   const int tiles_m = (p.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (p.N + Cfg::BN - 1) / Cfg::BN;
   dim3 grid(tiles_m * tiles_n, 1, p.batch);
   hipLaunchKernelGGL(kern, grid, dim3(Cfg::NT), Cfg::LDS_BYTES, stream, p, tiles_m, tiles_n);
@@ -1161,13 +1165,8 @@ static int num_cus() {
 
 template <class Cfg, class Kern>
 static int launch_persistent(Kern kern, const GemmParams& p, hipStream_t stream) {
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
-    if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    attr_set = true;
-  }
+  static unsigned long long lds_ok = 0;
+  if (int rc = allow_lds(kern, Cfg::LDS_BYTES, lds_ok)) return rc;
   const int tiles_m = (p.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (p.N + Cfg::BN - 1) / Cfg::BN;
   const long long items = (long long)tiles_m * tiles_n * p.batch;
   if (items > 0x7fffffffLL) return fail(TI_ERR_INVALID_ARG, "too many output tiles (%lld)", items);
@@ -1309,13 +1308,8 @@ static int launch_kind(const GemmParams& p, void* workspace, long long workspace
     // stages and as many resident workgroups as the LDS allows.
     auto launch = [&](auto kern, int rows, int per_cu) -> int {
       const int lds = 2 * rows * SBK + S_RED;
-      static bool attr_set = false;  // one flag per kernel instantiation (the lambda is generic)
-      if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-        if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-        attr_set = true;
-      }
+      static unsigned long long lds_ok = 0;  // one mask per kernel instantiation (the lambda is generic)
+      if (int rc = allow_lds(kern, lds, lds_ok)) return rc;
       const long long slots = (long long)cus * per_cu;
       hipLaunchKernelGGL(kern, dim3((unsigned)(strips < slots ? strips : slots)), dim3(256), lds, stream, p, spb,
                          (int)strips, GemmGroup{});
@@ -1431,13 +1425,8 @@ int launch_gemm_group_s8(const GemmParams& shape, const GemmGroup& grp, hipStrea
     const int cus = num_cus();
     auto launch = [&](auto kern, int rows, int per_cu) -> int {
       const int lds = 2 * rows * SBK + S_RED;
-      static bool attr_set = false;
-      if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-        if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-        attr_set = true;
-      }
+      static unsigned long long lds_ok = 0;
+      if (int rc = allow_lds(kern, lds, lds_ok)) return rc;
       const long long slots = (long long)cus * per_cu;
       hipLaunchKernelGGL(kern, dim3((unsigned)(strips < slots ? strips : slots)), dim3(256), lds, stream, shape, spb,
                          (int)strips, grp);
