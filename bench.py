@@ -189,7 +189,9 @@ def decoder_layer_ms(torch, dev):
     mask = torch.zeros(T, T, device=dev).masked_fill(
         torch.triu(torch.ones(T, T, dtype=torch.bool, device=dev), 1), torch.finfo(torch.float32).min)
     mask = mask[None, None].expand(B, 1, T, T).contiguous()
-    return sustained_ms(torch, [lambda: layer(hidden.clone(), attention_mask=mask)], window_ms=300.0, warm_launches=20)
+    # the layer updates its input in place (as upstream does); timing it on the same tensor again and again keeps
+    # a 42 MB copy out of the measurement, and LayerNorm keeps the growing residual in range
+    return sustained_ms(torch, [lambda: layer(hidden, attention_mask=mask)], window_ms=300.0, warm_launches=20)
 
 
 def main():

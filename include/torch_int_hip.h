@@ -85,6 +85,15 @@ int ti_linear_a8_w8_b8_o8(const int8_t* x, const int8_t* w, const int8_t* bias, 
                           int64_t M, int64_t N, int64_t K, float alpha, float beta,
                           void* workspace, int64_t workspace_bytes, void* stream);
 
+/* linear_a8_w8_b8_o8 whose [M, N] result is stored head-major: with M = B*T rows and N = H*head_dim columns,
+ * element (b*T + t, h*head_dim + dd) goes to out[b][h][t][dd] of a packed [B, H, T, head_dim] tensor.  The
+ * values are those of ti_linear_a8_w8_b8_o8; this replaces the `view(B,T,H,d).transpose(1,2).contiguous()`
+ * that follows the q/k/v projections (torch_int/models/opt.py:80-81).  T divides M, head_dim divides N and is
+ * a multiple of 16. */
+int ti_linear_a8_w8_b8_o8_heads(const int8_t* x, const int8_t* w, const int8_t* bias, int8_t* out, int64_t M,
+                                int64_t N, int64_t K, float alpha, float beta, int64_t T, int64_t head_dim,
+                                void* workspace, int64_t workspace_bytes, void* stream);
+
 /* `count` (<= 4) linear_a8_w8_b8_o8 problems that share the input x[M,K] and the shape: out[i] =
  * s8(rint(clamp(alpha[i]*(x . w[i]^T) + beta[i]*bias[i]))).  w, bias, out, alpha, beta are HOST arrays of
  * `count` device pointers / scalars.  The q, k and v projections of one attention block

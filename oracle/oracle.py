@@ -250,3 +250,9 @@ def linear_a8_w8_bfp32_ofp32_acc(x, w, bias, alpha, beta, inout, acc_fn=gemm_acc
 def linear_a8_w8_b8_o8_group(x, weights, biases, alphas, betas):
     """ti_linear_a8_w8_b8_o8_group: the separate linears, one after the other."""
     return tuple(linear_a8_w8_b8_o8(x, w, b, a, be) for w, b, a, be in zip(weights, biases, alphas, betas))
+
+
+def linear_a8_w8_b8_o8_heads(x, w, bias, alpha, beta, bsz, seq_len, heads, head_dim):
+    """ti_linear_a8_w8_b8_o8_heads: the plain linear, then the head split as torch writes it."""
+    y = linear_a8_w8_b8_o8(x, w, bias, alpha, beta)
+    return y.view(bsz, seq_len, heads, head_dim).transpose(1, 2).contiguous()

@@ -488,6 +488,33 @@ def test_bmm_rowmajor_rhs_for_decode():
     assert torch.equal(out, orc.bmm_s8t_s8t_s8t(a, b[:, 1:, :].contiguous(), 0.001))
 
 
+def test_head_major_projection_through_every_kernel_family():
+    # the s8 linear whose stores write [bsz, heads, seq, d]: same values as the plain linear, permuted
+    import ctypes
+    import torch_int._CUDA as C
+    import torch_int._hip_ext as X
+    C._lib.ti_last_kernel.restype = ctypes.c_char_p
+    g = torch.Generator().manual_seed(71)
+    seen = set()
+    # (bsz, seq, heads, d, K)
+    for (B, T, H, d, K) in [(4, 512, 40, 128, 256), (2, 1000, 72, 128, 192), (8, 512, 22, 128, 128), (2, 512, 16, 128, 64),
+                            (2, 512, 40, 128, 5120), (2, 64, 5, 128, 4096), (1, 16, 40, 128, 3072), (1, 3, 5, 32, 272),
+                            (3, 100, 5, 48, 48), (3, 700, 39, 128, 272), (2, 35, 3, 16, 37)]:
+        M, N = B * T, H * d
+        _say(f"head-major linear bsz={B} seq={T} heads={H} d={d} K={K}")
+        x, w, b = _s8(g, M, K), _s8(g, N, K), _s8(g, N)
+        alpha, beta = _scal(g, 1e-4, 1e-2), _scal(g, 1e-4, 1e-2)
+        ref = orc.linear_a8_w8_b8_o8_heads(x, w, b, alpha, beta, B, T, H, d)
+        out = X.linear_a8_w8_b8_o8_heads(x.to(DEV), w.to(DEV), b.to(DEV), alpha, beta, B, T, H, d)
+        assert out.shape == (B, H, T, d) and out.is_contiguous()
+        assert torch.equal(out.cpu(), ref), (B, T, H, d, K)
+        seen.add(C._lib.ti_last_kernel().decode())
+    assert {"pipe16_256x160", "pipe16_256x288", "pipe_256x256", "pipe_128x128", "splitk_256x256", "splitk_128x128",
+            "stream", "skinny", "tile_64x64", "tile_256x256", "scalar"} <= seen, seen
+    with pytest.raises(RuntimeError):
+        X.linear_a8_w8_b8_o8_heads(x.to(DEV), w.to(DEV), b.to(DEV), alpha, beta, 2, 35, 6, 8)   # d not a multiple of 16
+
+
 def test_grouped_qkv_linear():
     import ctypes
     import torch_int._CUDA as C

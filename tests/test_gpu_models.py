@@ -144,8 +144,17 @@ def test_decoder_layer_opt13b_shape():
             assert (y != ref).sum().item() == 0, name
 
     a = layer.self_attn
+    # q/k/v are written head-major by their GEMMs (the projection modules' forward is bypassed): what the two
+    # attention products received must be the plain linears of the first LayerNorm's output, head-split
+    x_qkv = rec["ln1"][1].cpu().view(B * T, -1)[rows].contiguous()
+    (q_in, k_in), _ = rec["qk"]
+    (_, vt_in), _ = rec["pv"]
+    got = {"q": q_in, "k": k_in, "v": vt_in.transpose(1, 2)}
     for name, lin in (("q", a.q_proj), ("k", a.k_proj), ("v", a.v_proj)):
-        check_linear(name, orc.linear_a8_w8_b8_o8, lin, (lin.a.item(), lin.b.item()))
+        _say("  check", name)
+        y = got[name].reshape(B, H, T, D // H).permute(0, 2, 1, 3).reshape(B * T, D).cpu()[rows]
+        ref = orc.linear_a8_w8_b8_o8(x_qkv, lin.weight, lin.bias, lin.a.item(), lin.b.item(), acc_fn=orc.gemm_acc_torch)
+        assert torch.equal(y, ref), name
     check_linear("out", orc.linear_a8_w8_bfp32_ofp32, a.out_proj, (a.out_proj.a.item(), 1))
     check_linear("fc1", orc.linear_relu_a8_w8_b8_o8, layer.fc1, (layer.fc1.a.item(), layer.fc1.b.item()))
     # fc2 adds its result into the residual stream in the GEMM epilogue: its "output" is the updated residual

@@ -42,7 +42,7 @@ static int check_ptr(const char* op, const char* name, const void* p, size_t ali
 static int run_gemm(const char* op, int kind, const void* a, const void* b, const void* bias, size_t bias_elt,
                     void* c, size_t out_elt, int64_t batch, int64_t M, int64_t N, int64_t K, float alpha,
                     float beta, void* ws, int64_t ws_bytes, void* stream, int64_t stride_a = 0,
-                    int64_t stride_b = 0) {
+                    int64_t stride_b = 0, int64_t out_T = 0, int64_t out_d = 0) {
   g_err[0] = 0;
   if (int rc = check_dims(op, batch, M, N, K)) return rc;
   // batch strides (elements between consecutive batches of a / b); 0 = packed
@@ -73,6 +73,15 @@ static int run_gemm(const char* op, int kind, const void* a, const void* b, cons
   p.strideC = M * N;
   p.alpha = alpha;
   p.beta = beta;
+  if (out_T != 0 || out_d != 0) {
+    if (out_T <= 0 || out_d <= 0 || M % out_T != 0 || N % out_d != 0 || out_d % 16 != 0)
+      return fail(TI_ERR_INVALID_ARG,
+                  "%s: head-major output needs T > 0 dividing M and head_dim > 0 dividing N, a multiple of 16 "
+                  "(got M=%lld N=%lld T=%lld head_dim=%lld)",
+                  op, (long long)M, (long long)N, (long long)out_T, (long long)out_d);
+    p.out_T = (int)out_T;
+    p.out_d = (int)out_d;
+  }
   return launch_gemm(kind, p, ws, ws_bytes, static_cast<hipStream_t>(stream));
 }
 
@@ -133,6 +142,13 @@ int ti_linear_a8_w8_b8_o8(const int8_t* x, const int8_t* w, const int8_t* bias, 
                           void* stream) {
   return run_gemm("linear_a8_w8_b8_o8", EPI_S8_BIAS, x, w, bias, 1, out, 1, 1, M, N, K, alpha, beta, ws,
                   ws_bytes, stream);
+}
+
+int ti_linear_a8_w8_b8_o8_heads(const int8_t* x, const int8_t* w, const int8_t* bias, int8_t* out, int64_t M,
+                                int64_t N, int64_t K, float alpha, float beta, int64_t T, int64_t head_dim,
+                                void* ws, int64_t ws_bytes, void* stream) {
+  return run_gemm("linear_a8_w8_b8_o8_heads", EPI_S8_BIAS, x, w, bias, 1, out, 1, 1, M, N, K, alpha, beta, ws,
+                  ws_bytes, stream, 0, 0, T, head_dim);
 }
 
 int ti_linear_a8_w8_b8_o8_group(const int8_t* x, const int8_t* const* w, const int8_t* const* bias, int8_t* const* out,

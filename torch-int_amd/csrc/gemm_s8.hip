@@ -122,7 +122,7 @@ __device__ __forceinline__ void store_tile(v16i (&acc)[Cfg::TM][Cfg::TN], const 
       for (int i = 0; i < TM; ++i) {
         const int m = m0 + wave_m * Cfg::WTM + i * 32 + frow;
         if (m >= M) continue;
-        Out* dst = C + (long long)m * N + nb;
+        Out* dst = C + out_index(p, m, nb);
         if (vec_ok && nb + 16 <= N) {
           if constexpr (sizeof(Out) == 1) {
             v4i w;
@@ -169,8 +169,9 @@ __device__ __forceinline__ void store_tile(v16i (&acc)[Cfg::TM][Cfg::TN], const 
           const int m = m0 + wave_m * Cfg::WTM + i * 32 + 8 * (v >> 2) + 4 * half + (v & 3);
           if (m < M && n < N) {
             Out fresh = E::apply(acc[i][j][v], bt, alpha);
-            if constexpr (E::kAccumulate) fresh = C[(long long)m * N + n] + fresh;
-            C[(long long)m * N + n] = fresh;
+            Out* at = C + out_index(p, m, n);
+            if constexpr (E::kAccumulate) fresh = *at + fresh;
+            *at = fresh;
           }
         }
       }
@@ -721,7 +722,7 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe16_kernel(GemmParams p, i
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
           const int m = tile_m * BM + wave_m * Cfg::WTM + i * 16 + er;
-          const float* src = reinterpret_cast<const float*>(C) + ((long long)(m < M ? m : M - 1) * N + nb);
+          const float* src = reinterpret_cast<const float*>(C) + out_index(p, m < M ? m : M - 1, nb < N ? nb : 0);
           v4f h = {0.f, 0.f, 0.f, 0.f};
           if (vec_ok && nb + 4 <= N) {
             h = *reinterpret_cast<const v4f*>(src);
@@ -769,7 +770,7 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe16_kernel(GemmParams p, i
         Out o[4];
 #pragma unroll
         for (int v = 0; v < 4; ++v) o[v] = E::apply(acc[i][j][v], bt[v], p.alpha);
-        Out* dst = C + (long long)m * N + nb;
+        Out* dst = C + out_index(p, m, nb < N ? nb : 0);
         if constexpr (E::kAccumulate) {
 #pragma unroll
           for (int v = 0; v < 4; ++v) o[v] = held[i][HOLD_ALL ? j : 0][v] + o[v];
@@ -843,7 +844,7 @@ __device__ __forceinline__ void store_skinny_tile(v4i acc, const GemmParams& p, 
     if (E::kHasBias && nb + v < N) bv = bias[nb + v];
     o[v] = E::apply(acc[v], E::bias_term(bv, p.beta), p.alpha);
   }
-  Out* dst = C + (long long)m * N + nb;
+  Out* dst = C + out_index(p, m, nb < N ? nb : 0);
   if constexpr (E::kAccumulate) {
 #pragma unroll
     for (int v = 0; v < 4; ++v)
@@ -1118,7 +1119,8 @@ __global__ __launch_bounds__(256) void gemm_scalar_kernel(GemmParams p) {
   BiasT bv = BiasT(0);
   if (E::kHasBias) bv = reinterpret_cast<const BiasT*>(p.bias)[n];
   Out* C = reinterpret_cast<Out*>(p.C) + (long long)blockIdx.z * p.strideC;
-  C[idx] = merge_old<E>(E::apply(acc, E::bias_term(bv, p.beta), p.alpha), C + idx);
+  Out* at = C + out_index(p, m, n);
+  *at = merge_old<E>(E::apply(acc, E::bias_term(bv, p.beta), p.alpha), at);
 }
 
 // ------------------------------------------------------------------ host side
@@ -1208,22 +1210,22 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmParams p, const 
     v4i acc = *reinterpret_cast<const v4i*>(ws + i0);
     for (int s = 1; s < splits; ++s) acc += *reinterpret_cast<const v4i*>(ws + (long long)s * total + i0);
     const int n = (int)(i0 % p.N);
+    Out* dst = C + out_index(p, (int)(i0 / p.N), n);
     Out o[4];
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
       BiasT bv = BiasT(0);
       if (E::kHasBias) bv = bias[n + v];
-      o[v] = merge_old<E>(E::apply(acc[v], E::bias_term(bv, p.beta), p.alpha), C + i0 + v);
+      o[v] = merge_old<E>(E::apply(acc[v], E::bias_term(bv, p.beta), p.alpha), dst + v);
     }
     if (sizeof(Out) == 4) {
       using W = typename std::conditional<sizeof(Out) == 4, Out, int>::type;
       v4i w4 = {__builtin_bit_cast(int, (W)o[0]), __builtin_bit_cast(int, (W)o[1]), __builtin_bit_cast(int, (W)o[2]),
                 __builtin_bit_cast(int, (W)o[3])};
-      *reinterpret_cast<v4i*>(C + i0) = w4;
+      *reinterpret_cast<v4i*>(dst) = w4;
     } else {
-      *reinterpret_cast<unsigned*>(C + i0) = (unsigned)(unsigned char)o[0] | ((unsigned)(unsigned char)o[1] << 8) |
-                                             ((unsigned)(unsigned char)o[2] << 16) |
-                                             ((unsigned)(unsigned char)o[3] << 24);
+      *reinterpret_cast<unsigned*>(dst) = (unsigned)(unsigned char)o[0] | ((unsigned)(unsigned char)o[1] << 8) |
+                                          ((unsigned)(unsigned char)o[2] << 16) | ((unsigned)(unsigned char)o[3] << 24);
     }
   } else {
     for (int v = 0; v < 4 && i0 + v < total; ++v) {
@@ -1231,7 +1233,8 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmParams p, const 
       for (int s = 0; s < splits; ++s) acc += ws[(long long)s * total + i0 + v];
       BiasT bv = BiasT(0);
       if (E::kHasBias) bv = bias[(i0 + v) % p.N];
-      C[i0 + v] = merge_old<E>(E::apply(acc, E::bias_term(bv, p.beta), p.alpha), C + i0 + v);
+      Out* at = C + out_index(p, (int)((i0 + v) / p.N), (int)((i0 + v) % p.N));
+      *at = merge_old<E>(E::apply(acc, E::bias_term(bv, p.beta), p.alpha), at);
     }
   }
 }
@@ -1353,6 +1356,7 @@ static int launch_kind(const GemmParams& p, void* workspace, long long workspace
       q.strideC = (long long)p.M * p.N;
       q.C = workspace;
       q.bias = nullptr;
+      q.out_T = q.out_d = 0;  // the partial products are plain [splits][M][N]; only the reduction permutes
       if (int rc = edge == 256 ? launch_pipe<PipeCfg<256, 256, 2, 4, 4, EPI_S32_RAW, false>>(q, stream)
                                : launch_pipe<PipeCfg<128, 128, 2, 2, 4, EPI_S32_RAW, false>>(q, stream))
         return rc;

@@ -171,7 +171,20 @@ struct GemmParams {
   int lda, ldb;                         // bytes between consecutive rows of A and B (>= K)
   long long strideA, strideB, strideC;  // elements between consecutive batches
   float alpha, beta;
+  // Head-major output (out_d > 0): row m = (b, t) with t < out_T, column n = (h, dd) with dd < out_d is
+  // stored as element [b][h][t][dd] of a packed [M/out_T, N/out_d, out_T, out_d] tensor -- the layout the
+  // attention products want, written by the projection itself.  0 = plain row-major [M, N].
+  int out_T = 0, out_d = 0;
 };
+
+// Offset of output element (m, n) of one batch; consecutive n stay consecutive inside a head, so vector
+// stores of VEC columns starting at a multiple of VEC are unaffected when out_d % VEC == 0.
+__device__ __forceinline__ long long out_index(const GemmParams& p, int m, int n) {
+  if (p.out_d == 0) return (long long)m * p.N + n;
+  const int b = m / p.out_T, t = m - b * p.out_T;
+  const int h = n / p.out_d, dd = n - h * p.out_d;
+  return (((long long)b * (p.N / p.out_d) + h) * p.out_T + t) * p.out_d + dd;
+}
 
 // Up to four linears that share the activation matrix and the shape (the q/k/v projections of one
 // attention block) run as one launch: problem i has its own weight, bias, output and scales.

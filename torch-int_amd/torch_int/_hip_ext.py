@@ -35,6 +35,8 @@ _lib.ti_bmm_s8t_s8n_f32t_strided.argtypes = [_vp, _vp, _vp, _i64, _i64, _i64, _i
 _lib.ti_bmm_s8t_s8n_f32t_strided.restype = ctypes.c_int
 _lib.ti_kv_append_s8.argtypes = [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp]
 _lib.ti_kv_append_s8.restype = ctypes.c_int
+_lib.ti_linear_a8_w8_b8_o8_heads.argtypes = [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _f32, _f32, _i64, _i64, _vp, _i64, _vp]
+_lib.ti_linear_a8_w8_b8_o8_heads.restype = ctypes.c_int
 _pp = ctypes.POINTER(ctypes.c_void_p)
 _lib.ti_linear_a8_w8_b8_o8_group.argtypes = [_vp, _pp, _pp, _pp, ctypes.POINTER(_f32), ctypes.POINTER(_f32), _i64, _i64,
                                             _i64, _i64, _vp]
@@ -287,3 +289,31 @@ def linear_a8_w8_b8_o8_group(x, weights, biases, alphas, betas, checked=False):
     if rc:
         raise RuntimeError(f"torch_int._hip_ext.linear_a8_w8_b8_o8_group: {_lib.ti_last_error().decode()} (status {rc})")
     return out.unbind(0)
+
+
+def can_linear_heads(x, w, bias, bsz, seq_len, heads, head_dim):
+    return (_ok(x, torch.int8) and _ok(w, torch.int8) and _ok(bias, torch.int8) and x.dim() == 2 and w.dim() == 2
+            and x.shape[1] == w.shape[1] and x.shape[0] == bsz * seq_len and w.shape[0] == heads * head_dim
+            and bias.numel() == w.shape[0] and head_dim % 16 == 0 and x.numel() > 0
+            and w.device == x.device and bias.device == x.device)
+
+
+def linear_a8_w8_b8_o8_heads(x, w, bias, alpha, beta, bsz, seq_len, heads, head_dim, checked=False):
+    """``_CUDA.linear_a8_w8_b8_o8(x, w, bias, alpha, beta).view(bsz, seq, heads, d).transpose(1, 2).contiguous()``
+    with the permutation done by the GEMM's stores: int8 [bsz, heads, seq, head_dim]."""
+    if not checked and not can_linear_heads(x, w, bias, bsz, seq_len, heads, head_dim):
+        raise RuntimeError("torch_int._hip_ext.linear_a8_w8_b8_o8_heads: needs contiguous int8 HIP tensors x [bsz*seq,K], "
+                           "w [heads*d,K], bias [heads*d] with d a multiple of 16")
+    M, K = x.shape
+    N = w.shape[0]
+    out = torch.empty((bsz, heads, seq_len, head_dim), dtype=torch.int8, device=x.device)
+    idx = x.device.index
+    with _on(x.device):
+        stream = _raw_stream(idx)
+        ws_ptr, ws_bytes = _CUDA._workspace(idx, stream, _CUDA._ws_bytes(M, N, K)) if 16 < M <= 1024 else (0, 0)
+        rc = _lib.ti_linear_a8_w8_b8_o8_heads(x.data_ptr(), w.data_ptr(), bias.data_ptr(), out.data_ptr(), M, N, K,
+                                              float(alpha), float(beta), seq_len, head_dim, ws_ptr or None, ws_bytes,
+                                              stream or None)
+    if rc:
+        raise RuntimeError(f"torch_int._hip_ext.linear_a8_w8_b8_o8_heads: {_lib.ti_last_error().decode()} (status {rc})")
+    return out

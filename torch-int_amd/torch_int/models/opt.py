@@ -150,6 +150,24 @@ class Int8OPTAttention(nn.Module):
         lead = hidden_states.shape[:-1]
         return tuple(o.view(*lead, -1) for o in outs)
 
+    def _qkv_head_major(self, hidden_states, bsz, tgt_len):
+        """(q, k, v), each int8 [bsz, heads, tgt, head_dim] written in that layout by the projection GEMMs
+        themselves, or None when the layers or tensors do not qualify."""
+        q, k, v = self.q_proj, self.k_proj, self.v_proj
+        if not (type(q) is W8A8B8O8Linear and type(k) is W8A8B8O8Linear and type(v) is W8A8B8O8Linear):
+            return None
+        x = hidden_states.reshape(-1, hidden_states.shape[-1])
+        H, d = self.num_heads, self.head_dim
+        out = []
+        for lin in (q, k, v):
+            w, b = lin._wb()
+            b = b.reshape(-1)
+            if not _hip_ext.can_linear_heads(x, w, b, bsz, tgt_len, H, d):
+                return None
+            out.append(_hip_ext.linear_a8_w8_b8_o8_heads(x, w, b, lin._scalar("a"), lin._scalar("b"), bsz, tgt_len, H, d,
+                                                         checked=True))
+        return tuple(out)
+
     def _shape(self, tensor: torch.Tensor, seq_len: int, bsz: int):
         """[bsz, seq, embed] -> contiguous [bsz, heads, seq, head_dim]."""
         if seq_len < 0:
@@ -167,16 +185,28 @@ class Int8OPTAttention(nn.Module):
         bsz, tgt_len, _ = hidden_states.size()
         H, d = self.num_heads, self.head_dim
 
-        grouped = None
-        if not cross and bsz * tgt_len <= 16 and hidden_states.is_cuda:
-            grouped = self._qkv_grouped(hidden_states)  # decode: one launch streams all three weights
-        query = self.q_proj(hidden_states) if grouped is None else grouped[0]
+        # Self-attention on HIP tensors takes the q/k/v projections from one of two fused forms: a single
+        # grouped launch for decode-sized inputs, or projections whose stores already produce the
+        # [bsz, heads, seq, head_dim] layout; both give the values of the plain layers.
+        proj = None  # (q, k, v), each [bsz, H, tgt, d]
+        if not cross and hidden_states.is_cuda:
+            if bsz * tgt_len <= 16:
+                flat = self._qkv_grouped(hidden_states)
+                if flat is not None:
+                    proj = tuple(self._shape(t, tgt_len, bsz) for t in flat)
+            else:
+                proj = self._qkv_head_major(hidden_states, bsz, tgt_len)
+        if proj is not None:
+            query4, key, value = proj
+        else:
+            query4 = self._shape(self.q_proj(hidden_states), tgt_len, bsz)
         if cross and past_key_value is not None:
             key, value = past_key_value
         else:
-            kv_src = key_value_states if cross else hidden_states
-            key = self._shape(self.k_proj(kv_src) if grouped is None else grouped[1], -1, bsz)
-            value = self._shape(self.v_proj(kv_src) if grouped is None else grouped[2], -1, bsz)
+            if proj is None:
+                kv_src = key_value_states if cross else hidden_states
+                key = self._shape(self.k_proj(kv_src), -1, bsz)
+                value = self._shape(self.v_proj(kv_src), -1, bsz)
             if not cross and past_key_value is not None:
                 if self.kv_cache_in_place:
                     key, value = _kv_append_pair(past_key_value[0], past_key_value[1], key, value)
@@ -185,7 +215,7 @@ class Int8OPTAttention(nn.Module):
                     value = torch.cat([past_key_value[1], value], dim=2)
         present = (key, value)
 
-        query = self._shape(query, tgt_len, bsz).view(bsz * H, -1, d)
+        query = query4.view(bsz * H, -1, d)
         # cache views are packed per head; [bsz, H] merges into one batch dimension either way
         key = key.view(bsz * H, -1, d) if key.is_contiguous() else key.reshape(bsz * H, key.shape[2], d)
         value = value.view(bsz * H, -1, d) if value.is_contiguous() else value.reshape(bsz * H, value.shape[2], d)
