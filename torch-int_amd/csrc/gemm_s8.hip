@@ -169,7 +169,8 @@ __device__ __forceinline__ void store_tile(v16i (&acc)[Cfg::TM][Cfg::TN], const 
           const int m = m0 + wave_m * Cfg::WTM + i * 32 + 8 * (v >> 2) + 4 * half + (v & 3);
           if (m < M && n < N) {
             Out fresh = E::apply(acc[i][j][v], bt, alpha);
-            Out* at = C + out_index(p, m, n);
+            // plain row-major only: head-major output exists for 8-bit outputs, which take the branch above
+            Out* at = C + ((long long)m * N + n);
             if constexpr (E::kAccumulate) fresh = *at + fresh;
             *at = fresh;
           }

@@ -173,7 +173,7 @@ struct GemmParams {
   float alpha, beta;
   // Head-major output (out_d > 0): row m = (b, t) with t < out_T, column n = (h, dd) with dd < out_d is
   // stored as element [b][h][t][dd] of a packed [M/out_T, N/out_d, out_T, out_d] tensor -- the layout the
-  // attention products want, written by the projection itself.  0 = plain row-major [M, N].
+  // attention products want, written by the projection itself.  0 = plain row-major [M, N].  8-bit outputs only.
   int out_T = 0, out_d = 0;
 };
 
