@@ -104,6 +104,66 @@ static PyObject* fc_linear_group3(PyObject* self, PyObject* const* a, Py_ssize_t
   return PyLong_FromLong(ti_linear_a8_w8_b8_o8_group(x, w, b, o, al, be, 3, M, N, K, st));
 }
 
+/* add_ln_q(x|0, residual, gamma, beta, eps, q_out, rows, H, stream) -> status */
+static PyObject* fc_add_ln_q(PyObject* self, PyObject* const* a, Py_ssize_t n) {
+  (void)self;
+  if (n != 9) {
+    PyErr_SetString(PyExc_TypeError, "add_ln_q expects 9 arguments");
+    return NULL;
+  }
+  void *x = as_ptr(a[0]), *res = as_ptr(a[1]), *g = as_ptr(a[2]), *b = as_ptr(a[3]);
+  float eps = as_f32(a[4]);
+  void* q = as_ptr(a[5]);
+  int64_t rows = as_i64(a[6]), H = as_i64(a[7]);
+  void* st = as_ptr(a[8]);
+  if (PyErr_Occurred()) return NULL;
+  return PyLong_FromLong(ti_add_layernorm_q(x, res, g, b, eps, q, rows, H, st));
+}
+
+/* softmax_q(scores, mask|0, probs, batch, heads, T, S, stream) -> status */
+static PyObject* fc_softmax_q(PyObject* self, PyObject* const* a, Py_ssize_t n) {
+  (void)self;
+  if (n != 8) {
+    PyErr_SetString(PyExc_TypeError, "softmax_q expects 8 arguments");
+    return NULL;
+  }
+  void *sc = as_ptr(a[0]), *mk = as_ptr(a[1]), *pr = as_ptr(a[2]);
+  int64_t B = as_i64(a[3]), Hh = as_i64(a[4]), T = as_i64(a[5]), S = as_i64(a[6]);
+  void* st = as_ptr(a[7]);
+  if (PyErr_Occurred()) return NULL;
+  return PyLong_FromLong(ti_attn_softmax_q(sc, mk, pr, B, Hh, T, S, st));
+}
+
+/* bmm_f32t_strided(a, b, c, batch, M, N, K, stride_a, stride_b, alpha, stream) -> status */
+static PyObject* fc_bmm_f32t_strided(PyObject* self, PyObject* const* a, Py_ssize_t n) {
+  (void)self;
+  if (n != 11) {
+    PyErr_SetString(PyExc_TypeError, "bmm_f32t_strided expects 11 arguments");
+    return NULL;
+  }
+  void *pa = as_ptr(a[0]), *pb = as_ptr(a[1]), *pc = as_ptr(a[2]);
+  int64_t B = as_i64(a[3]), M = as_i64(a[4]), N = as_i64(a[5]), K = as_i64(a[6]), sa = as_i64(a[7]), sb = as_i64(a[8]);
+  float alpha = as_f32(a[9]);
+  void* st = as_ptr(a[10]);
+  if (PyErr_Occurred()) return NULL;
+  return PyLong_FromLong(ti_bmm_s8t_s8n_f32t_strided(pa, pb, pc, B, M, N, K, sa, sb, alpha, st));
+}
+
+/* bmm_rowmajor(a, b, c, batch, M, N, K, stride_b, alpha, stream) -> status */
+static PyObject* fc_bmm_rowmajor(PyObject* self, PyObject* const* a, Py_ssize_t n) {
+  (void)self;
+  if (n != 10) {
+    PyErr_SetString(PyExc_TypeError, "bmm_rowmajor expects 10 arguments");
+    return NULL;
+  }
+  void *pa = as_ptr(a[0]), *pb = as_ptr(a[1]), *pc = as_ptr(a[2]);
+  int64_t B = as_i64(a[3]), M = as_i64(a[4]), N = as_i64(a[5]), K = as_i64(a[6]), sb = as_i64(a[7]);
+  float alpha = as_f32(a[8]);
+  void* st = as_ptr(a[9]);
+  if (PyErr_Occurred()) return NULL;
+  return PyLong_FromLong(ti_bmm_s8t_s8t_s8t(pa, pb, pc, B, M, N, K, sb, alpha, st));
+}
+
 /* kv_append(k_new, v_new, k_buf, v_buf, BH, T, D, cap, S, stream) -> status */
 static PyObject* fc_kv_append(PyObject* self, PyObject* const* a, Py_ssize_t n) {
   (void)self;
@@ -128,6 +188,10 @@ static PyMethodDef methods[] = {
     {"linear", (PyCFunction)(void (*)(void))fc_linear, METH_FASTCALL, "forward to ti_linear_*"},
     {"bmm", (PyCFunction)(void (*)(void))fc_bmm, METH_FASTCALL, "forward to ti_bmm_*"},
     {"ln_q", (PyCFunction)(void (*)(void))fc_ln_q, METH_FASTCALL, "forward to ti_dq_add_layernorm_q"},
+    {"add_ln_q", (PyCFunction)(void (*)(void))fc_add_ln_q, METH_FASTCALL, "forward to ti_add_layernorm_q"},
+    {"softmax_q", (PyCFunction)(void (*)(void))fc_softmax_q, METH_FASTCALL, "forward to ti_attn_softmax_q"},
+    {"bmm_f32t_strided", (PyCFunction)(void (*)(void))fc_bmm_f32t_strided, METH_FASTCALL, "forward to ti_bmm_s8t_s8n_f32t_strided"},
+    {"bmm_rowmajor", (PyCFunction)(void (*)(void))fc_bmm_rowmajor, METH_FASTCALL, "forward to ti_bmm_s8t_s8t_s8t"},
     {"linear_group3", (PyCFunction)(void (*)(void))fc_linear_group3, METH_FASTCALL, "forward to ti_linear_a8_w8_b8_o8_group"},
     {"kv_append", (PyCFunction)(void (*)(void))fc_kv_append, METH_FASTCALL, "forward to ti_kv_append_s8"},
     {"last_error", fc_last_error, METH_NOARGS, "ti_last_error()"},

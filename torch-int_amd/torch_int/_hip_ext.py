@@ -44,6 +44,10 @@ _lib.ti_linear_a8_w8_b8_o8_group.restype = ctypes.c_int
 _raw_stream = torch._C._cuda_getCurrentRawStream
 _fast = _CUDA._fast if getattr(_CUDA._fast, "kv_append", None) is not None else None
 _fast_group3 = getattr(_CUDA._fast, "linear_group3", None)
+_fast_add_ln_q = getattr(_CUDA._fast, "add_ln_q", None)
+_fast_softmax_q = getattr(_CUDA._fast, "softmax_q", None)
+_fast_bmm_strided = getattr(_CUDA._fast, "bmm_f32t_strided", None)
+_fast_bmm_rowmajor = getattr(_CUDA._fast, "bmm_rowmajor", None)
 
 
 class _NoSwitch:
@@ -87,9 +91,14 @@ def add_layernorm_q(x, residual, weight, bias, eps, checked=False):
     H = residual.shape[-1]
     q = torch.empty(residual.shape, dtype=torch.int8, device=dev)
     with _on(dev):
-        rc = _lib.ti_add_layernorm_q(x.data_ptr() if x is not None else None, residual.data_ptr(),
-                                     weight.data_ptr(), bias.data_ptr(), float(eps), q.data_ptr(),
-                                     residual.numel() // H, H, _raw_stream(dev.index) or None)
+        if _fast_add_ln_q is not None:
+            rc = _fast_add_ln_q(x.data_ptr() if x is not None else 0, residual.data_ptr(), weight.data_ptr(),
+                                bias.data_ptr(), float(eps), q.data_ptr(), residual.numel() // H, H,
+                                _raw_stream(dev.index))
+        else:
+            rc = _lib.ti_add_layernorm_q(x.data_ptr() if x is not None else None, residual.data_ptr(),
+                                         weight.data_ptr(), bias.data_ptr(), float(eps), q.data_ptr(),
+                                         residual.numel() // H, H, _raw_stream(dev.index) or None)
     if rc:
         raise RuntimeError(f"torch_int._hip_ext.{op}: {_lib.ti_last_error().decode()} (status {rc})")
     return q
@@ -116,8 +125,12 @@ def attn_softmax_q(scores, mask, heads, checked=False):
     dev = scores.device
     out = torch.empty((BH, T, S), dtype=torch.int8, device=dev)
     with _on(dev):
-        rc = _lib.ti_attn_softmax_q(scores.data_ptr(), mask.data_ptr() if mask is not None else None, out.data_ptr(),
-                                    bsz, heads, T, S, _raw_stream(dev.index) or None)
+        if _fast_softmax_q is not None:
+            rc = _fast_softmax_q(scores.data_ptr(), mask.data_ptr() if mask is not None else 0, out.data_ptr(), bsz,
+                                 heads, T, S, _raw_stream(dev.index))
+        else:
+            rc = _lib.ti_attn_softmax_q(scores.data_ptr(), mask.data_ptr() if mask is not None else None,
+                                        out.data_ptr(), bsz, heads, T, S, _raw_stream(dev.index) or None)
     if rc:
         raise RuntimeError(f"torch_int._hip_ext.{op}: {_lib.ti_last_error().decode()} (status {rc})")
     return out
@@ -190,8 +203,13 @@ def bmm_s8t_s8t_s8t(a, b, alpha, checked=False):
     N = b.shape[2]
     out = torch.empty((B, M, N), dtype=torch.int8, device=a.device)
     with _on(a.device):
-        rc = _lib.ti_bmm_s8t_s8t_s8t(a.data_ptr(), b.data_ptr(), out.data_ptr(), B, M, N, K,
-                                     b.stride(0) if B > 1 else 0, float(alpha), _raw_stream(a.device.index) or None)
+        if _fast_bmm_rowmajor is not None:
+            rc = _fast_bmm_rowmajor(a.data_ptr(), b.data_ptr(), out.data_ptr(), B, M, N, K,
+                                    b.stride(0) if B > 1 else 0, float(alpha), _raw_stream(a.device.index))
+        else:
+            rc = _lib.ti_bmm_s8t_s8t_s8t(a.data_ptr(), b.data_ptr(), out.data_ptr(), B, M, N, K,
+                                         b.stride(0) if B > 1 else 0, float(alpha),
+                                         _raw_stream(a.device.index) or None)
     if rc:
         raise RuntimeError(f"torch_int._hip_ext.bmm_s8t_s8t_s8t: {_lib.ti_last_error().decode()} (status {rc})")
     return out
@@ -212,9 +230,14 @@ def bmm_s8t_s8n_f32t_strided(a, b, alpha, checked=False):
     N = b.shape[1]
     out = torch.empty((B, M, N), dtype=torch.float32, device=a.device)
     with _on(a.device):
-        rc = _lib.ti_bmm_s8t_s8n_f32t_strided(a.data_ptr(), b.data_ptr(), out.data_ptr(), B, M, N, K,
-                                              a.stride(0) if B > 1 else 0, b.stride(0) if B > 1 else 0, float(alpha),
-                                              _raw_stream(a.device.index) or None)
+        if _fast_bmm_strided is not None:
+            rc = _fast_bmm_strided(a.data_ptr(), b.data_ptr(), out.data_ptr(), B, M, N, K,
+                                   a.stride(0) if B > 1 else 0, b.stride(0) if B > 1 else 0, float(alpha),
+                                   _raw_stream(a.device.index))
+        else:
+            rc = _lib.ti_bmm_s8t_s8n_f32t_strided(a.data_ptr(), b.data_ptr(), out.data_ptr(), B, M, N, K,
+                                                  a.stride(0) if B > 1 else 0, b.stride(0) if B > 1 else 0,
+                                                  float(alpha), _raw_stream(a.device.index) or None)
     if rc:
         raise RuntimeError(f"torch_int._hip_ext.bmm_s8t_s8n_f32t_strided: {_lib.ti_last_error().decode()} (status {rc})")
     return out
