@@ -524,6 +524,216 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MIN_WAVES) void gemm_pipe_kernel(Gemm
 }
 
 // ---------------------------------------------------------------------------
+// The same persistent pipeline with K steps of 128 bytes and two LDS stages.
+// A panel row of one step is one whole 128-byte cache line, so every line of
+// the operands crosses the L2 -> L1 path once (with 64-byte steps each line is
+// requested again one step later, after 64 KiB of other lines have passed
+// through the L1), and there is one workgroup barrier per 128 bytes of K.
+//
+// LDS stage = [A panel BM x 128][B panel BN x 128]; chunk c of panel row r at
+// chunk position c ^ ((r >> 1) & 7).  One copy instruction fills 1 KiB = 8
+// panel rows, lane l landing at row l/8, position l%8.
+//
+// One K step = four 32-byte slices.  Fragments of slice s+1 are read while
+// slice s multiplies.  After the reads of the last slice: wait for them and for
+// this wave's copies of the next step, pass the barrier (next stage complete,
+// this stage no longer read by anyone), issue the copies two steps ahead into
+// the stage just released, read the first slice of the next step and multiply
+// the last slice of this one.
+static constexpr int QBK = 128;
+
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int KIND_, bool SWAP_>
+struct Pipe2Cfg {
+  static constexpr int BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, KIND = KIND_;
+  static constexpr bool SWAP = SWAP_;
+  static constexpr int NWAVES = WAVES_M * WAVES_N;
+  static constexpr int NT = NWAVES * 64;
+  static constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
+  static constexpr int TM = WTM / 32, TN = WTN / 32;
+  static constexpr int STAGE_BYTES = (BM + BN) * QBK;
+  static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
+  static constexpr int COPIES = (BM + BN) / 8 / NWAVES;  // copy instructions per wave per step
+  static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be made of 32x32 blocks");
+  static_assert((BM + BN) % (8 * NWAVES) == 0 && (BM / 8) % COPIES == 0, "a wave copies 1 KiB slabs of one panel");
+  static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
+};
+
+template <class Cfg>
+__global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe2_kernel(GemmParams p, int tiles_m, int tiles_n, int items) {
+  constexpr int BM = Cfg::BM, BN = Cfg::BN, TM = Cfg::TM, TN = Cfg::TN, COPIES = Cfg::COPIES;
+  constexpr bool SWAP = Cfg::SWAP;
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave_m = wave / Cfg::WAVES_N, wave_n = wave % Cfg::WAVES_N;
+  const int M = p.M, N = p.N, K = p.K;
+  const int KT = K / QBK;
+  const int tiles = tiles_m * tiles_n;
+  const int first = blockIdx.x, stride = gridDim.x;
+  const int my_items = (items - first + stride - 1) / stride;  // >= 1 (grid <= items)
+  const int G = my_items * KT;                                  // K steps this workgroup multiplies
+
+  // ---- copy stream: copy j of this wave fills stage bytes [(wave*COPIES + j) * 1024, +1024)
+  const bool copies_a = wave * COPIES * 8 < BM;  // this wave fills A panel rows (else B panel rows)
+  const TI_GLOBAL_AS int8_t* src[COPIES];
+  auto set_copy_item = [&](int item) {
+    const int b = item / tiles;
+    int tile_m, tile_n;
+    tile_of_workgroup(item - b * tiles, tiles_m, tiles_n, tile_m, tile_n);
+    const int first_row = copies_a ? tile_m * BM : tile_n * BN;  // of the panel in its operand
+    const int last_row = (copies_a ? M : N) - 1;                 // edge rows re-read the last row; never stored
+    const size_t ld = copies_a ? p.lda : p.ldb;
+    const int8_t* origin = copies_a ? p.A + (long long)b * p.strideA : p.B + (long long)b * p.strideB;
+#pragma unroll
+    for (int j = 0; j < COPIES; ++j) {
+      const int prow = (wave * COPIES + j) * 8 + (lane >> 3) - (copies_a ? 0 : BM);  // row inside the panel
+      const int chunk = (lane & 7) ^ ((prow >> 1) & 7);
+      int lr = prow;
+      if (SWAP && !copies_a) lr = (prow & ~31) | ((prow & 4) << 2) | ((prow & 24) >> 1) | (prow & 3);  // MFMA row 8q+4h+j -> 16h+4q+j
+      const int gr = first_row + lr < last_row ? first_row + lr : last_row;
+      src[j] = (const TI_GLOBAL_AS int8_t*)(origin + (size_t)gr * ld + chunk * 16);
+    }
+  };
+  // Copy cursor (work item, K step inside it, global step).  Past the last item it keeps
+  // re-copying the final K step into the stage that is free anyway, so that one step of
+  // copies is in flight at every barrier and the wait counts never change.
+  int c_item = first, c_kt = 0, c_g = 0, c_live = 1;
+  auto issue_copies = [&]() {
+    TI_LDS_AS char* dst = (TI_LDS_AS char*)smem + (c_g & 1) * Cfg::STAGE_BYTES + wave * COPIES * 1024;
+#pragma unroll
+    for (int j = 0; j < COPIES; ++j)
+      __builtin_amdgcn_global_load_lds((const TI_GLOBAL_AS void*)(src[j] + c_kt * QBK), (TI_LDS_AS void*)(dst + j * 1024),
+                                       16, 0, 0);
+    c_kt += c_live;
+    ++c_g;
+  };
+  auto advance_copy_item = [&]() {  // call when c_live && c_kt == KT
+    if (c_g < G) {
+      c_kt = 0;
+      c_item += stride;
+      set_copy_item(c_item);
+    } else {
+      c_live = 0;
+      c_kt = KT - 1;
+    }
+  };
+
+  // ---- fragment addressing: lane reads panel row (lane & 31), chunk 2*slice + (lane >> 5)
+  const int frow = lane & 31;
+  const int fpos = ((lane >> 5) ^ (frow >> 1)) & 7;  // chunk position for slice 0
+  const int a_frag = (wave_m * Cfg::WTM + frow) * QBK + (fpos << 4);
+  const int b_frag = BM * QBK + (wave_n * Cfg::WTN + frow) * QBK + (fpos << 4);
+
+  v16i acc[TM][TN];
+  auto zero_acc = [&]() {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+  };
+  auto read_frags = [&](int g, int slice, v4i (&fa)[TM], v4i (&fb)[TN]) {
+    const char* s = smem + (g & 1) * Cfg::STAGE_BYTES;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+      fa[i] = *reinterpret_cast<const v4i*>(s + ((a_frag ^ (slice << 5)) + i * 32 * QBK));
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+      fb[j] = *reinterpret_cast<const v4i*>(s + ((b_frag ^ (slice << 5)) + j * 32 * QBK));
+  };
+  auto mma = [&](v4i (&fa)[TM], v4i (&fb)[TN]) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        acc[i][j] = SWAP ? __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[j], fa[i], acc[i][j], 0, 0, 0)
+                         : __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+  };
+  // scheduling hint: one LDS read after each of the first TM+TN MFMAs of a group
+  auto interleave = [&]() {
+#pragma unroll
+    for (int i = 0; i < TM + TN; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 DS read
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - (TM + TN), 0);
+  };
+
+  // ---- prologue: two steps of copies, wait for the first
+  set_copy_item(c_item);
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    issue_copies();
+    if (c_live && c_kt == KT) advance_copy_item();
+  }
+  wait_copies_then_barrier<COPIES>();
+
+  v4i fa0[TM], fb0[TN], fa1[TM], fb1[TN];
+  read_frags(0, 0, fa0, fb0);
+  zero_acc();
+
+  int item = first, kt = 0, g = 0;  // multiply cursor
+  // One K step.  LAST = last K step of a work item: the next item's first fragments are
+  // read after the epilogue instead, so they do not occupy registers during it.
+  auto step = [&](auto last) {
+    constexpr bool LAST = decltype(last)::value;
+    read_frags(g, 1, fa1, fb1);
+    mma(fa0, fb0);
+    interleave();
+    read_frags(g, 2, fa0, fb0);
+    mma(fa1, fb1);
+    interleave();
+    read_frags(g, 3, fa1, fb1);
+    mma(fa0, fb0);
+    interleave();
+    // the lgkmcnt wait is what allows this stage to be overwritten after the barrier
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    issue_copies();  // step g+2 into the stage this step used
+    if (!LAST) read_frags(g + 1, 0, fa0, fb0);
+    mma(fa1, fb1);
+    if (!LAST) interleave();
+  };
+  auto finish_item = [&]() {
+    const int b = item / tiles;
+    int tile_m, tile_n;
+    tile_of_workgroup(item - b * tiles, tiles_m, tiles_n, tile_m, tile_n);
+    // opaque copy of the lane id: keeps the epilogue's address arithmetic inside the loop
+    int lane_here = lane;
+    asm volatile("" : "+v"(lane_here));
+    store_tile<Cfg>(acc, p, b, tile_m * BM, tile_n * BN, wave_m, wave_n, lane_here);
+    item += stride;
+    kt = 0;
+    zero_acc();
+  };
+
+  while (g < G) {
+    // steps until the multiply or the copy cursor reaches the end of its work item
+    int n = KT - kt;
+    if (c_live && KT - c_kt < n) n = KT - c_kt;
+    const bool item_done = kt + n == KT;
+    const int plain = item_done ? n - 1 : n;
+    for (int i = 0; i < plain; ++i) {
+      step(std::false_type{});
+      ++g;
+    }
+    if (item_done) {
+      step(std::true_type{});
+      ++g;
+    }
+    kt += n;
+    if (c_live && c_kt == KT) advance_copy_item();
+    if (item_done) {
+      finish_item();
+      if (g < G) read_frags(g, 0, fa0, fb0);
+    }
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // the trailing filler copies must land before the LDS is released
+}
+
+// ---------------------------------------------------------------------------
 // Variant of the pipelined persistent kernel built from 16x16 blocks
 // (v_mfma_i32_16x16x64_i8: one instruction covers the whole 64-byte K step).
 // Its output tile can be any multiple of 16 per wave, which gives tile counts
@@ -1193,6 +1403,10 @@ static int launch_pipe(const GemmParams& p, hipStream_t stream) {
   return launch_persistent<Cfg>(gemm_pipe_kernel<Cfg>, p, stream);
 }
 template <class Cfg>
+static int launch_pipe2(const GemmParams& p, hipStream_t stream) {
+  return launch_persistent<Cfg>(gemm_pipe2_kernel<Cfg>, p, stream);
+}
+template <class Cfg>
 static int launch_pipe16(const GemmParams& p, hipStream_t stream) {
   return launch_persistent<Cfg>(gemm_pipe16_kernel<Cfg>, p, stream);
 }
@@ -1358,8 +1572,9 @@ static int launch_kind(const GemmParams& p, void* workspace, long long workspace
       q.C = workspace;
       q.bias = nullptr;
       q.out_T = q.out_d = 0;  // the partial products are plain [splits][M][N]; only the reduction permutes
-      if (int rc = edge == 256 ? launch_pipe<PipeCfg<256, 256, 2, 4, 4, EPI_S32_RAW, false>>(q, stream)
-                               : launch_pipe<PipeCfg<128, 128, 2, 2, 4, EPI_S32_RAW, false>>(q, stream))
+      if (int rc = edge != 256          ? launch_pipe<PipeCfg<128, 128, 2, 2, 4, EPI_S32_RAW, false>>(q, stream)
+                   : q.K % QBK == 0 ? launch_pipe2<Pipe2Cfg<256, 256, 2, 4, EPI_S32_RAW, false>>(q, stream)
+                                    : launch_pipe<PipeCfg<256, 256, 2, 4, 4, EPI_S32_RAW, false>>(q, stream))
         return rc;
       const long long quads = ((long long)p.M * p.N + 3) / 4;
       hipLaunchKernelGGL(splitk_reduce_kernel<KIND>, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream, p,
@@ -1397,6 +1612,7 @@ static int launch_kind(const GemmParams& p, void* workspace, long long workspace
         return launch_pipe16<Pipe16Cfg<256, 288, 4, 2, 4, KIND>>(p, stream);
       }
       g_last_kernel = "pipe_256x256";
+      if (p.K % QBK == 0) return launch_pipe2<Pipe2Cfg<256, 256, 2, 4, KIND, SWAP>>(p, stream);  // whole cache lines per row
       return launch_pipe<PipeCfg<256, 256, 2, 4, 4, KIND, SWAP>>(p, stream);
     }
     if (t128 >= 128) {
