@@ -75,6 +75,36 @@ __device__ __forceinline__ void tile_of_workgroup(int pid, int tiles_m, int tile
   tn = in / gsz;
 }
 
+// 4x4 transpose across the four lanes of a quad: lane b (0..3) enters with x[k] = its own element k
+// and leaves with x[k] = element b of lane k.  Two exchange rounds (partner lane ^ 2, then lane ^ 1)
+// over the DPP quad permutes; every lane of the wave must take part.
+__device__ __forceinline__ void quad_transpose(int (&x)[4], int lane) {
+  const bool hi = lane & 2;
+  int s0 = hi ? x[0] : x[2];
+  int s1 = hi ? x[1] : x[3];
+  int r0 = __builtin_amdgcn_mov_dpp(s0, 0x4E, 0xf, 0xf, true);  // quad_perm [2,3,0,1]
+  int r1 = __builtin_amdgcn_mov_dpp(s1, 0x4E, 0xf, 0xf, true);
+  if (hi) {
+    x[0] = r0;
+    x[1] = r1;
+  } else {
+    x[2] = r0;
+    x[3] = r1;
+  }
+  const bool odd = lane & 1;
+  s0 = odd ? x[0] : x[1];
+  s1 = odd ? x[2] : x[3];
+  r0 = __builtin_amdgcn_mov_dpp(s0, 0xB1, 0xf, 0xf, true);  // quad_perm [1,0,3,2]
+  r1 = __builtin_amdgcn_mov_dpp(s1, 0xB1, 0xf, 0xf, true);
+  if (odd) {
+    x[0] = r0;
+    x[2] = r1;
+  } else {
+    x[1] = r0;
+    x[3] = r1;
+  }
+}
+
 // Applies the epilogue to a wavefront's accumulators and stores them.
 template <class Cfg>
 __device__ __forceinline__ void store_tile(v16i (&acc)[Cfg::TM][Cfg::TN], const GemmParams& p, int batch, int m0,
@@ -162,6 +192,39 @@ __device__ __forceinline__ void store_tile(v16i (&acc)[Cfg::TM][Cfg::TN], const 
       BiasT bv = BiasT(0);
       if (E::kHasBias && n < N) bv = bias[n];
       const float bt = E::bias_term(bv, beta);
+      // 32-bit outputs of a block that lies inside the matrix: the lanes of a quad swap their four
+      // rows x four columns, so that a lane ends with four consecutive columns of one row and a store
+      // instruction writes eight whole 128-byte lines instead of two
+      const int nq = n0 + wave_n * Cfg::WTN + j * 32;  // first column of the block
+      if constexpr (sizeof(Out) == 4) {
+       if ((N & 3) == 0 && nq + 32 <= N && (reinterpret_cast<uintptr_t>(C) & 15) == 0) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            int x[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) x[k] = __builtin_bit_cast(int, E::apply(acc[i][j][4 * q + k], bt, alpha));
+            quad_transpose(x, lane);
+            const int m = m0 + wave_m * Cfg::WTM + i * 32 + 8 * q + 4 * half + (lane & 3);
+            if (m < M) {
+              Out* at = C + ((long long)m * N + nq + (frow & ~3));
+              if constexpr (E::kAccumulate) {
+                const v4i old = *reinterpret_cast<const v4i*>(at);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                  const int was = old[k], add = x[k];  // plain values: the casts below must not see vector elements
+                  x[k] = __builtin_bit_cast(int, __builtin_bit_cast(Out, was) + __builtin_bit_cast(Out, add));
+                }
+              }
+              v4i w = {x[0], x[1], x[2], x[3]};
+              *reinterpret_cast<v4i*>(at) = w;
+            }
+          }
+        }
+        continue;
+       }
+      }
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
 #pragma unroll
