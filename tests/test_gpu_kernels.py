@@ -109,7 +109,9 @@ def test_every_gemm_kernel_family_is_reached_and_exact():
     import ctypes
     import torch_int._CUDA as C
     C._lib.ti_last_kernel.restype = ctypes.c_char_p
-    expect = [((2048, 5120, 256), "pipe16_256x160"), ((2000, 9216, 192), "pipe16_256x288"),
+    expect = [((2048, 5120, 256), "pipe16_256x160"), ((2048, 5120, 192), "pipe16_256x160"),
+              ((2000, 9216, 192), "pipe16_256x288"), ((2000, 9216, 384), "pipe16_256x288"),
+              ((4096, 2816, 192), "pipe_256x256"),
               ((4096, 2816, 128), "pipe_256x256"), ((1024, 2048, 64), "pipe_128x128"),
               ((1024, 5120, 5120), "splitk_256x256"), ((128, 640, 4096), "splitk_128x128"),
               ((16, 5120, 3072), "stream"), ((3, 100, 272), "skinny"), ((300, 200, 48), "tile_64x64"),
@@ -427,7 +429,8 @@ def test_linear_accumulate_into_output():
     C._lib.ti_last_kernel.restype = ctypes.c_char_p
     g = torch.Generator().manual_seed(63)
     seen = set()
-    for (M, N, K) in [(2048, 5120, 256), (2000, 9216, 192), (4096, 2816, 128), (1024, 2048, 64), (1024, 5120, 5120),
+    for (M, N, K) in [(2048, 5120, 256), (2048, 5120, 64), (2000, 9216, 192), (2000, 9216, 128), (4096, 2816, 128),
+                      (4096, 2816, 320), (1024, 2048, 64), (1024, 5120, 5120),
                       (128, 640, 4096), (16, 5120, 3072), (3, 100, 272), (300, 200, 48), (2100, 5000, 272),
                       (70, 50, 37), (4, 64, 0)]:
         _say(f"linear += M={M} N={N} K={K}")
@@ -497,7 +500,8 @@ def test_head_major_projection_through_every_kernel_family():
     g = torch.Generator().manual_seed(71)
     seen = set()
     # (bsz, seq, heads, d, K)
-    for (B, T, H, d, K) in [(4, 512, 40, 128, 256), (2, 1000, 72, 128, 192), (8, 512, 22, 128, 128), (2, 512, 16, 128, 64),
+    for (B, T, H, d, K) in [(4, 512, 40, 128, 256), (4, 512, 40, 128, 192), (2, 1000, 72, 128, 192), (2, 1000, 72, 128, 256),
+                            (8, 512, 22, 128, 128), (8, 512, 22, 128, 192), (2, 512, 16, 128, 64),
                             (2, 512, 40, 128, 5120), (2, 64, 5, 128, 4096), (1, 16, 40, 128, 3072), (1, 3, 5, 32, 272),
                             (3, 100, 5, 48, 48), (3, 700, 39, 128, 272), (2, 35, 3, 16, 37)]:
         M, N = B * T, H * d

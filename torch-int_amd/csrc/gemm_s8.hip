@@ -831,6 +831,105 @@ struct Pipe16Cfg {
   static_assert(LDS_BYTES <= 160 * 1024 && STAGES >= 3, "LDS budget");
 };
 
+// Epilogue of the 16x16-block kernels: the lane holds row (lane & 15) and four consecutive columns
+// 4 * (lane >> 4) .. +3 of every block.
+template <class Cfg>
+__device__ __forceinline__ void store_tile16(v4i (&acc)[Cfg::TM][Cfg::TN], const GemmParams& p, int b, int tile_m,
+                                             int tile_n, int wave_m, int wave_n, int lane_here) {
+  using E = Epi<Cfg::KIND>;
+  using Out = typename E::Out;
+  using BiasT = typename E::Bias;
+  constexpr int BM = Cfg::BM, BN = Cfg::BN, TM = Cfg::TM, TN = Cfg::TN;
+  const int M = p.M, N = p.N;
+  const int er = lane_here & 15, eg = lane_here >> 4;
+  Out* __restrict__ C = reinterpret_cast<Out*>(p.C) + (long long)b * p.strideC;
+  const BiasT* __restrict__ bias = reinterpret_cast<const BiasT*>(p.bias);
+  const bool vec_ok = (N & 3) == 0 && (reinterpret_cast<uintptr_t>(C) & 15) == 0;
+  const bool bias_al = (reinterpret_cast<uintptr_t>(bias) & 15) == 0;
+  // accumulate-into-output kind: fetch what the tile holds now, the loads in flight together before the
+  // first use -- the whole wave tile when its TM*TN*4 registers fit, else one column block at a time
+  constexpr bool HOLD_ALL = E::kAccumulate && TM * TN <= 24;
+  constexpr int HJ = E::kAccumulate ? (HOLD_ALL ? TN : 1) : 1;
+  typename std::conditional<E::kAccumulate, v4f, char>::type held[E::kAccumulate ? TM : 1][HJ];
+  auto fetch_held = [&](int j, int slot) {
+    if constexpr (E::kAccumulate) {
+      const int nb = tile_n * BN + wave_n * Cfg::WTN + j * 16 + 4 * eg;
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const int m = tile_m * BM + wave_m * Cfg::WTM + i * 16 + er;
+        const float* src = reinterpret_cast<const float*>(C) + out_index(p, m < M ? m : M - 1, nb < N ? nb : 0);
+        v4f h = {0.f, 0.f, 0.f, 0.f};
+        if (vec_ok && nb + 4 <= N) {
+          h = *reinterpret_cast<const v4f*>(src);
+        } else {
+#pragma unroll
+          for (int v = 0; v < 4; ++v)
+            if (nb + v < N) h[v] = src[v];
+        }
+        held[i][slot] = h;
+      }
+    }
+  };
+  if constexpr (HOLD_ALL) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) fetch_held(j, j);
+  }
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int nb = tile_n * BN + wave_n * Cfg::WTN + j * 16 + 4 * eg;
+    if constexpr (E::kAccumulate && !HOLD_ALL) fetch_held(j, 0);
+    float bt[4];
+    if (E::kHasBias && vec_ok && bias_al && nb + 4 <= N) {
+      BiasT bv[4];
+      if (sizeof(BiasT) == 1) {
+        const int w = *reinterpret_cast<const int*>(bias + nb);
+        __builtin_memcpy(bv, &w, 4);
+      } else {
+        const v4i w = *reinterpret_cast<const v4i*>(bias + nb);
+        __builtin_memcpy(bv, &w, 16);
+      }
+#pragma unroll
+      for (int v = 0; v < 4; ++v) bt[v] = E::bias_term(bv[v], p.beta);
+    } else {
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        BiasT bv = BiasT(0);
+        if (E::kHasBias && nb + v < N) bv = bias[nb + v];
+        bt[v] = E::bias_term(bv, p.beta);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int m = tile_m * BM + wave_m * Cfg::WTM + i * 16 + er;
+      if (m >= M) continue;
+      Out o[4];
+#pragma unroll
+      for (int v = 0; v < 4; ++v) o[v] = E::apply(acc[i][j][v], bt[v], p.alpha);
+      Out* dst = C + out_index(p, m, nb < N ? nb : 0);
+      if constexpr (E::kAccumulate) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) o[v] = held[i][HOLD_ALL ? j : 0][v] + o[v];
+      }
+      if (vec_ok && nb + 4 <= N) {
+        if (sizeof(Out) == 4) {
+          using W = typename std::conditional<sizeof(Out) == 4, Out, int>::type;
+          v4i w4 = {__builtin_bit_cast(int, (W)o[0]), __builtin_bit_cast(int, (W)o[1]),
+                    __builtin_bit_cast(int, (W)o[2]), __builtin_bit_cast(int, (W)o[3])};
+          *reinterpret_cast<v4i*>(dst) = w4;
+        } else {
+          *reinterpret_cast<unsigned*>(dst) = (unsigned)(unsigned char)o[0] | ((unsigned)(unsigned char)o[1] << 8) |
+                                              ((unsigned)(unsigned char)o[2] << 16) |
+                                              ((unsigned)(unsigned char)o[3] << 24);
+        }
+      } else {
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+          if (nb + v < N) dst[v] = o[v];
+      }
+    }
+  }
+}
+
 template <class Cfg>
 __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe16_kernel(GemmParams p, int tiles_m, int tiles_n, int items) {
   using E = Epi<Cfg::KIND>;
@@ -980,93 +1079,7 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe16_kernel(GemmParams p, i
     tile_of_workgroup(item - b * tiles, tiles_m, tiles_n, tile_m, tile_n);
     int lane_here = lane;  // opaque copy: keeps the epilogue's address arithmetic out of the mainloop
     asm volatile("" : "+v"(lane_here));
-    const int er = lane_here & 15, eg = lane_here >> 4;
-    Out* __restrict__ C = reinterpret_cast<Out*>(p.C) + (long long)b * p.strideC;
-    const BiasT* __restrict__ bias = reinterpret_cast<const BiasT*>(p.bias);
-    const bool vec_ok = (N & 3) == 0 && (reinterpret_cast<uintptr_t>(C) & 15) == 0;
-    const bool bias_al = (reinterpret_cast<uintptr_t>(bias) & 15) == 0;
-    // accumulate-into-output kind: fetch what the tile holds now, the loads in flight together before the
-    // first use -- the whole wave tile when its TM*TN*4 registers fit, else one column block at a time
-    constexpr bool HOLD_ALL = E::kAccumulate && TM * TN <= 24;
-    constexpr int HJ = E::kAccumulate ? (HOLD_ALL ? TN : 1) : 1;
-    typename std::conditional<E::kAccumulate, v4f, char>::type held[E::kAccumulate ? TM : 1][HJ];
-    auto fetch_held = [&](int j, int slot) {
-      if constexpr (E::kAccumulate) {
-        const int nb = tile_n * BN + wave_n * Cfg::WTN + j * 16 + 4 * eg;
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-          const int m = tile_m * BM + wave_m * Cfg::WTM + i * 16 + er;
-          const float* src = reinterpret_cast<const float*>(C) + out_index(p, m < M ? m : M - 1, nb < N ? nb : 0);
-          v4f h = {0.f, 0.f, 0.f, 0.f};
-          if (vec_ok && nb + 4 <= N) {
-            h = *reinterpret_cast<const v4f*>(src);
-          } else {
-#pragma unroll
-            for (int v = 0; v < 4; ++v)
-              if (nb + v < N) h[v] = src[v];
-          }
-          held[i][slot] = h;
-        }
-      }
-    };
-    if constexpr (HOLD_ALL) {
-#pragma unroll
-      for (int j = 0; j < TN; ++j) fetch_held(j, j);
-    }
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int nb = tile_n * BN + wave_n * Cfg::WTN + j * 16 + 4 * eg;
-      if constexpr (E::kAccumulate && !HOLD_ALL) fetch_held(j, 0);
-      float bt[4];
-      if (E::kHasBias && vec_ok && bias_al && nb + 4 <= N) {
-        BiasT bv[4];
-        if (sizeof(BiasT) == 1) {
-          const int w = *reinterpret_cast<const int*>(bias + nb);
-          __builtin_memcpy(bv, &w, 4);
-        } else {
-          const v4i w = *reinterpret_cast<const v4i*>(bias + nb);
-          __builtin_memcpy(bv, &w, 16);
-        }
-#pragma unroll
-        for (int v = 0; v < 4; ++v) bt[v] = E::bias_term(bv[v], p.beta);
-      } else {
-#pragma unroll
-        for (int v = 0; v < 4; ++v) {
-          BiasT bv = BiasT(0);
-          if (E::kHasBias && nb + v < N) bv = bias[nb + v];
-          bt[v] = E::bias_term(bv, p.beta);
-        }
-      }
-#pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        const int m = tile_m * BM + wave_m * Cfg::WTM + i * 16 + er;
-        if (m >= M) continue;
-        Out o[4];
-#pragma unroll
-        for (int v = 0; v < 4; ++v) o[v] = E::apply(acc[i][j][v], bt[v], p.alpha);
-        Out* dst = C + out_index(p, m, nb < N ? nb : 0);
-        if constexpr (E::kAccumulate) {
-#pragma unroll
-          for (int v = 0; v < 4; ++v) o[v] = held[i][HOLD_ALL ? j : 0][v] + o[v];
-        }
-        if (vec_ok && nb + 4 <= N) {
-          if (sizeof(Out) == 4) {
-            using W = typename std::conditional<sizeof(Out) == 4, Out, int>::type;
-            v4i w4 = {__builtin_bit_cast(int, (W)o[0]), __builtin_bit_cast(int, (W)o[1]),
-                      __builtin_bit_cast(int, (W)o[2]), __builtin_bit_cast(int, (W)o[3])};
-            *reinterpret_cast<v4i*>(dst) = w4;
-          } else {
-            *reinterpret_cast<unsigned*>(dst) = (unsigned)(unsigned char)o[0] | ((unsigned)(unsigned char)o[1] << 8) |
-                                                ((unsigned)(unsigned char)o[2] << 16) |
-                                                ((unsigned)(unsigned char)o[3] << 24);
-          }
-        } else {
-#pragma unroll
-          for (int v = 0; v < 4; ++v)
-            if (nb + v < N) dst[v] = o[v];
-        }
-      }
-    }
+    store_tile16<Cfg>(acc, p, b, tile_m, tile_n, wave_m, wave_n, lane_here);
     item += stride;
     kt = 0;
     zero_acc();
@@ -1097,6 +1110,203 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe16_kernel(GemmParams p, i
     if (item_done) {
       finish_item();
       if (gs < G) read_frags(gs, fa0, fb0);
+    }
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // the trailing filler copies must land before the LDS is released
+}
+
+// The 16x16-block kernel with K steps of 128 bytes and two LDS stages (see gemm_pipe2_kernel for the
+// stage layout and the step structure; a step here is two 64-byte slices, one MFMA deep each).
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int KIND_>
+struct Pipe16QCfg {
+  static constexpr int BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, KIND = KIND_;
+  static constexpr int NWAVES = WAVES_M * WAVES_N;
+  static constexpr int NT = NWAVES * 64;
+  static constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
+  static constexpr int TM = WTM / 16, TN = WTN / 16;
+  static constexpr int STAGE_BYTES = (BM + BN) * QBK;
+  static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
+  static constexpr int RPW = (BM + BN) / NWAVES;  // panel rows a wave copies per step
+  static constexpr int TAIL_ROWS = RPW % 8;
+  static constexpr int COPIES = RPW / 8 + (TAIL_ROWS ? 1 : 0);
+  static constexpr bool SINGLE_B = 4 * TM * TN + 8 * (TM + TN) >= 224;  // as in Pipe16Cfg
+  static_assert(WTM % 16 == 0 && WTN % 16 == 0, "wave tile must be made of 16x16 blocks");
+  static_assert((BM + BN) % NWAVES == 0 && RPW % 2 == 0, "a wave must copy whole pairs of rows");
+  static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
+};
+
+template <class Cfg>
+__global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe16q_kernel(GemmParams p, int tiles_m, int tiles_n, int items) {
+  constexpr int BM = Cfg::BM, BN = Cfg::BN, TM = Cfg::TM, TN = Cfg::TN, COPIES = Cfg::COPIES;
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave_m = wave / Cfg::WAVES_N, wave_n = wave % Cfg::WAVES_N;
+  const int M = p.M, N = p.N, K = p.K;
+  const int KT = K / QBK;
+  const int tiles = tiles_m * tiles_n;
+  const int first = blockIdx.x, stride = gridDim.x;
+  const int my_items = (items - first + stride - 1) / stride;
+  const int G = my_items * KT;
+
+  // ---- copy stream: copy j of this wave fills panel rows wave*RPW + 8j .. +7 of [A panel | B panel]
+  const TI_GLOBAL_AS int8_t* src[COPIES];
+  auto set_copy_item = [&](int item) {
+    const int b = item / tiles;
+    int tile_m, tile_n;
+    tile_of_workgroup(item - b * tiles, tiles_m, tiles_n, tile_m, tile_n);
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int8_t* A = p.A + (long long)b * p.strideA;
+    const int8_t* B = p.B + (long long)b * p.strideB;
+#pragma unroll
+    for (int j = 0; j < COPIES; ++j) {
+      int prow = wave * Cfg::RPW + j * 8 + (lane >> 3);
+      prow = prow < BM + BN ? prow : BM + BN - 1;  // lanes beyond a partial last copy are disabled anyway
+      const int pos = lane & 7;
+      if (prow < BM) {
+        const int chunk = pos ^ ((prow >> 1) & 7);
+        const int gr = m0 + prow < M ? m0 + prow : M - 1;  // edge rows re-read the last row; never stored
+        src[j] = (const TI_GLOBAL_AS int8_t*)(A + (size_t)gr * p.lda + chunk * 16);
+      } else {
+        const int br = prow - BM;
+        const int chunk = pos ^ ((br >> 1) & 7);
+        const int gr = n0 + br < N ? n0 + br : N - 1;
+        src[j] = (const TI_GLOBAL_AS int8_t*)(B + (size_t)gr * p.ldb + chunk * 16);
+      }
+    }
+  };
+  int c_item = first, c_kt = 0, c_g = 0, c_live = 1;
+  auto issue_copies = [&]() {
+    TI_LDS_AS char* dst = (TI_LDS_AS char*)smem + (c_g & 1) * Cfg::STAGE_BYTES + wave * Cfg::RPW * QBK;
+#pragma unroll
+    for (int j = 0; j < COPIES; ++j) {
+      if (Cfg::TAIL_ROWS == 0 || j + 1 < COPIES || lane < Cfg::TAIL_ROWS * 8)
+        __builtin_amdgcn_global_load_lds((const TI_GLOBAL_AS void*)(src[j] + c_kt * QBK),
+                                         (TI_LDS_AS void*)(dst + j * 1024), 16, 0, 0);
+    }
+    c_kt += c_live;
+    ++c_g;
+  };
+  auto advance_copy_item = [&]() {  // call when c_live && c_kt == KT
+    if (c_g < G) {
+      c_kt = 0;
+      c_item += stride;
+      set_copy_item(c_item);
+    } else {
+      c_live = 0;
+      c_kt = KT - 1;
+    }
+  };
+
+  // ---- fragment addressing: lane reads panel row (lane & 15), chunk 4*slice + (lane >> 4)
+  const int r = lane & 15, g4 = lane >> 4;
+  const int fpos = (g4 ^ (r >> 1)) & 7;  // chunk position for slice 0
+  const int a_frag = (wave_m * Cfg::WTM + r) * QBK + (fpos << 4);
+  const int b_frag = BM * QBK + (wave_n * Cfg::WTN + r) * QBK + (fpos << 4);
+
+  v4i acc[TM][TN];
+  auto zero_acc = [&]() {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) acc[i][j] = v4i{0, 0, 0, 0};
+  };
+  auto read_a = [&](int gs, int slice, v4i (&fa)[TM]) {
+    const char* st = smem + (gs & 1) * Cfg::STAGE_BYTES;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) fa[i] = *reinterpret_cast<const v4i*>(st + ((a_frag ^ (slice << 6)) + i * 16 * QBK));
+  };
+  auto read_b1 = [&](int gs, int slice, int j) {
+    const char* st = smem + (gs & 1) * Cfg::STAGE_BYTES;
+    return *reinterpret_cast<const v4i*>(st + ((b_frag ^ (slice << 6)) + j * 16 * QBK));
+  };
+  auto read_frags = [&](int gs, int slice, v4i (&fa)[TM], v4i (&fb)[TN]) {
+    read_a(gs, slice, fa);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) fb[j] = read_b1(gs, slice, j);
+  };
+  auto interleave = [&]() {  // one LDS read after each of the first TM+TN MFMAs
+#pragma unroll
+    for (int i = 0; i < TM + TN; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - (TM + TN), 0);
+  };
+  // Multiplies the fragments (fc, fd) while those of (gs_next, slice_next) load into (fn, fm); with
+  // SINGLE_B the weight fragments live in fd only and are replaced block by block.
+  auto mma_and_fetch = [&](v4i (&fc)[TM], v4i (&fd)[TN], v4i (&fn)[TM], v4i (&fm)[TN], int gs_next, int slice_next,
+                           auto fetch) {
+    constexpr bool FETCH = decltype(fetch)::value;
+    if constexpr (Cfg::SINGLE_B) {
+      if (FETCH) read_a(gs_next, slice_next, fn);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+          acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fd[j], fc[i], acc[i][j], 0, 0, 0);
+        if (FETCH) fd[j] = read_b1(gs_next, slice_next, j);
+      }
+    } else {
+      if (FETCH) read_frags(gs_next, slice_next, fn, fm);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fd[j], fc[i], acc[i][j], 0, 0, 0);
+      if (FETCH) interleave();
+    }
+  };
+
+  set_copy_item(c_item);
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    issue_copies();
+    if (c_live && c_kt == KT) advance_copy_item();
+  }
+  wait_copies_then_barrier<COPIES>();
+
+  v4i fa0[TM], fb0[TN], fa1[TM], fb1[TN];  // fb1 is unused with SINGLE_B
+  read_frags(0, 0, fa0, fb0);
+  zero_acc();
+
+  int item = first, kt = 0, gs = 0;  // multiply cursor
+  auto step = [&](auto last) {
+    constexpr bool LAST = decltype(last)::value;
+    mma_and_fetch(fa0, fb0, fa1, Cfg::SINGLE_B ? fb0 : fb1, gs, 1, std::true_type{});
+    // the lgkmcnt wait is what allows this stage to be overwritten after the barrier
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    issue_copies();  // step gs+2 into the stage this step used
+    mma_and_fetch(fa1, Cfg::SINGLE_B ? fb0 : fb1, fa0, fb0, gs + 1, 0, std::integral_constant<bool, !LAST>{});
+    ++gs;
+  };
+  auto finish_item = [&]() {
+    const int b = item / tiles;
+    int tile_m, tile_n;
+    tile_of_workgroup(item - b * tiles, tiles_m, tiles_n, tile_m, tile_n);
+    int lane_here = lane;  // opaque copy: keeps the epilogue's address arithmetic out of the mainloop
+    asm volatile("" : "+v"(lane_here));
+    store_tile16<Cfg>(acc, p, b, tile_m, tile_n, wave_m, wave_n, lane_here);
+    item += stride;
+    kt = 0;
+    zero_acc();
+  };
+
+  while (gs < G) {
+    // steps until the multiply or the copy cursor reaches the end of its work item
+    int n = KT - kt;
+    if (c_live && KT - c_kt < n) n = KT - c_kt;
+    const bool item_done = kt + n == KT;
+    const int plain = item_done ? n - 1 : n;
+    for (int i = 0; i < plain; ++i) step(std::false_type{});
+    if (item_done) step(std::true_type{});
+    kt += n;
+    if (c_live && c_kt == KT) advance_copy_item();
+    if (item_done) {
+      finish_item();
+      if (gs < G) read_frags(gs, 0, fa0, fb0);
     }
   }
   __builtin_amdgcn_s_waitcnt(0x0F70);  // the trailing filler copies must land before the LDS is released
@@ -1470,6 +1680,10 @@ static int launch_pipe2(const GemmParams& p, hipStream_t stream) {
   return launch_persistent<Cfg>(gemm_pipe2_kernel<Cfg>, p, stream);
 }
 template <class Cfg>
+static int launch_pipe16q(const GemmParams& p, hipStream_t stream) {
+  return launch_persistent<Cfg>(gemm_pipe16q_kernel<Cfg>, p, stream);
+}
+template <class Cfg>
 static int launch_pipe16(const GemmParams& p, hipStream_t stream) {
   return launch_persistent<Cfg>(gemm_pipe16_kernel<Cfg>, p, stream);
 }
@@ -1656,22 +1870,27 @@ static int launch_kind(const GemmParams& p, void* workspace, long long workspace
     const bool wide = p.N > 128 && p.M > 128;
     if (t256 >= 160 && wide) {
       // 256x160 or 256x288 tiles (16x16 blocks) when the width allows it and they fill the CUs more
-      // evenly.  Measured at full occupancy the 16x16-block kernel reaches 0.78 (256x160: one barrier
-      // per 20 short MFMAs) or 0.9 (256x288: 36 per barrier) of the 256x256 kernel's rate, so it only
-      // pays off when the 256x256 grid would leave CUs idle (e.g. 2048x5120: 160 tiles of 256x256 but
-      // 256 of 256x160; 2048x9216: 288 tiles of 256x256 = two rounds, but exactly 256 of 256x288).
+      // evenly (e.g. 2048x5120: 160 tiles of 256x256 but 256 of 256x160; 2048x9216: 288 tiles of 256x256 =
+      // two rounds, but exactly 256 of 256x288).  Rates relative to the 256x256 kernel at full occupancy,
+      // measured: with 128-byte steps 0.88 (256x160; 0.85 with 32-bit stores) and 0.95 (256x288); with
+      // 64-byte steps (K not a multiple of 128) 0.78 and 0.9.
       const long long cus = num_cus();
       auto fill = [&](long long tiles) { return (double)tiles / (double)(((tiles + cus - 1) / cus) * cus); };
       const long long rows256 = (p.M + 255) / 256;
+      const bool wide_step = p.K % QBK == 0;
+      const double f160 = !wide_step ? 0.78 : sizeof(Out) == 1 ? 0.88 : 0.85;
+      const double f288 = wide_step ? 0.95 : 0.9;
       const double e256 = fill(t256);
-      const double e160 = p.N % 160 == 0 ? 0.78 * fill(rows256 * (p.N / 160) * p.batch) : 0.0;
-      const double e288 = p.N % 288 == 0 ? 0.9 * fill(rows256 * (p.N / 288) * p.batch) : 0.0;
+      const double e160 = p.N % 160 == 0 ? f160 * fill(rows256 * (p.N / 160) * p.batch) : 0.0;
+      const double e288 = p.N % 288 == 0 ? f288 * fill(rows256 * (p.N / 288) * p.batch) : 0.0;
       if (e160 > e256 && e160 >= e288) {
         g_last_kernel = "pipe16_256x160";
+        if (wide_step) return launch_pipe16q<Pipe16QCfg<256, 160, 4, 2, KIND>>(p, stream);
         return launch_pipe16<Pipe16Cfg<256, 160, 4, 2, 5, KIND>>(p, stream);
       }
       if (e288 > e256) {
         g_last_kernel = "pipe16_256x288";
+        if (wide_step) return launch_pipe16q<Pipe16QCfg<256, 288, 4, 2, KIND>>(p, stream);
         return launch_pipe16<Pipe16Cfg<256, 288, 4, 2, 4, KIND>>(p, stream);
       }
       g_last_kernel = "pipe_256x256";
