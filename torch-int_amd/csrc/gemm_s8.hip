@@ -848,7 +848,7 @@ __device__ __forceinline__ void store_tile16(v4i (&acc)[Cfg::TM][Cfg::TN], const
   const bool bias_al = (reinterpret_cast<uintptr_t>(bias) & 15) == 0;
   // accumulate-into-output kind: fetch what the tile holds now, the loads in flight together before the
   // first use -- the whole wave tile when its TM*TN*4 registers fit, else one column block at a time
-  constexpr bool HOLD_ALL = E::kAccumulate && TM * TN <= 24;
+  constexpr bool HOLD_ALL = E::kAccumulate && TM * TN <= 12;
   constexpr int HJ = E::kAccumulate ? (HOLD_ALL ? TN : 1) : 1;
   typename std::conditional<E::kAccumulate, v4f, char>::type held[E::kAccumulate ? TM : 1][HJ];
   auto fetch_held = [&](int j, int slot) {
