@@ -36,12 +36,15 @@ for _p in (os.path.join(ROOT, "torch-int_amd"), ROOT):
 
 PEAK_INT8_TOPS = 5000.0   # MI355X dense INT8 MFMA, TOP/s
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
-# HBM-side bytes per launch of the dominant kernel come from rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) of
-# this script's own sweep, which cannot be taken from inside the process: 417 768 KiB x 2.000 fetched +
-# 183 193 KiB written per launch, averaged over the 16 launches per step that reach the 256x256 kernel
-# (commands and calibration in profiles/gemm_pipe_256x256_linear_8192x20480x5120.md).
-TRAFFIC_BYTES = 1.043e9
-DOMINANT = "pipe_256x256"
+# Kernel families the large (M >= 2048) sweep cases are routed to, by the label ti_last_kernel() reports: the
+# kernel template behind the label at these shapes (K is a multiple of 128 everywhere in the sweep) and the HBM-side
+# bytes per launch, averaged over the sweep launches that reach it.  The byte counts cannot be taken from inside
+# the process: they come from rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) of this script's own sweep; commands,
+# raw counter values and the calibration against a plain copy kernel are in profiles/.
+FAMILIES = {
+    "pipe_256x256": {"kernel": "gemm_pipe2_kernel<Pipe2Cfg<256,256,2,4,KIND,SWAP>>", "traffic": None},
+    "pipe16_256x160": {"kernel": "gemm_pipe16q_kernel<Pipe16QCfg<256,160,4,2,KIND>>", "traffic": None},
+}
 SHAPES = [(5120, 5120), (20480, 5120), (5120, 20480)]   # (N, K): qkv/out_proj, fc1, fc2
 MS = [1, 16, 128, 512, 2048, 8192]
 VARIANTS = ["b32_o32", "bfp32_ofp32", "b8_o8", "relu_b8_o8"]
@@ -245,10 +248,18 @@ def main():
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
     heavy_ms = sum(a.elapsed_time(b) for ev in marks for (a, b) in ev) / max(args.steps, 1)   # per step
     heavy_ops = sum(cases[i]["ops"] for i in heavy)
-    # the dominant kernel: the 256x256 pipelined GEMM (whatever cases the library routes to it)
-    dom = [k for k, i in enumerate(heavy) if cases[i]["kernel"] == DOMINANT]
-    dom_ms = sum(ev[k][0].elapsed_time(ev[k][1]) for ev in marks for k in dom) / max(args.steps, 1)
-    dom_ops = sum(cases[heavy[k]]["ops"] for k in dom)
+    # the dominant kernel: the family that takes the largest share of the timed launches
+    fam = {}
+    for k, i in enumerate(heavy):
+        t = sum(ev[k][0].elapsed_time(ev[k][1]) for ev in marks) / max(args.steps, 1)
+        f = fam.setdefault(cases[i]["kernel"], {"ms": 0.0, "ops": 0.0, "idx": []})
+        f["ms"] += t
+        f["ops"] += cases[i]["ops"]
+        f["idx"].append(k)
+    DOMINANT = max(fam, key=lambda name: fam[name]["ms"])
+    dom = fam[DOMINANT]["idx"]
+    dom_ms = fam[DOMINANT]["ms"]
+    dom_ops = fam[DOMINANT]["ops"]
     value = sweep_ops / (ms_per_step * 1e-3) / 1e12
 
     result = {
@@ -264,13 +275,18 @@ def main():
     achieved = dom_ops / dom_ms / 1e9
     result["roofline"] = {
         "bound": "mfma", "achieved": achieved, "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
-        "frac": achieved / PEAK_INT8_TOPS, "traffic": TRAFFIC_BYTES,
-        "kernel": "gemm_pipe_kernel<PipeCfg<256,256,2,4,4,KIND,...>> (the sweep cases the library routes to it: "
+        "frac": achieved / PEAK_INT8_TOPS, "traffic": FAMILIES.get(DOMINANT, {}).get("traffic"),
+        "kernel": FAMILIES.get(DOMINANT, {}).get("kernel", DOMINANT) + " (the sweep cases the library routes to it: "
                   + ", ".join(sorted({f"{cases[heavy[k]]['M']}x{cases[heavy[k]]['N']}x{cases[heavy[k]]['K']}" for k in dom})) + ")",
+        "family": DOMINANT,
         "ops_per_launch": dom_ops / len(dom), "avg_launch_ms": dom_ms / len(dom), "launches_per_step": len(dom),
         "protocol": "HIP events around each of these launches inside the timed steps",
         "all_mfma_bound_cases": {"achieved": heavy_ops / heavy_ms / 1e9, "frac": heavy_ops / heavy_ms / 1e9 / PEAK_INT8_TOPS,
-                                 "launches_per_step": len(heavy), "avg_launch_ms": heavy_ms / len(heavy)}}
+                                 "launches_per_step": len(heavy), "avg_launch_ms": heavy_ms / len(heavy)},
+        "families": {name: {"kernel": FAMILIES.get(name, {}).get("kernel", name), "launches_per_step": len(f["idx"]),
+                            "avg_launch_ms": f["ms"] / len(f["idx"]), "achieved": f["ops"] / f["ms"] / 1e9,
+                            "frac": f["ops"] / f["ms"] / 1e9 / PEAK_INT8_TOPS,
+                            "traffic": FAMILIES.get(name, {}).get("traffic")} for name, f in fam.items()}}
 
     if not args.sweep_only:
         # per-case launch durations, upstream's protocol; HBM-bound cases rotate weight copies (> 256 MB in total)

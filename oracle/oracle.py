@@ -242,6 +242,21 @@ def bmm_s8t_s8t_s8t(a, b, alpha):
     return bmm_s8t_s8n_s8t(a, b.transpose(1, 2).contiguous(), alpha)
 
 
+def decode_attn_s8(q, k_new, v_new, k_buf, v_buf, filled, mask, heads, alpha_qk, alpha_pv):
+    """ti_decode_attn_s8: the chain of upstream's decode step (torch_int/models/opt.py:128-190) on
+    [BH, T, d] q / k_new / v_new and cache buffers [BH, cap, d] holding ``filled`` positions.  Returns
+    (ctx, probs, k_buf', v_buf') with the new rows appended in copies of the buffers."""
+    T = q.shape[1]
+    S = filled + T
+    k_buf, v_buf = k_buf.clone(), v_buf.clone()
+    k_buf[:, filled:S] = k_new
+    v_buf[:, filled:S] = v_new
+    scores = bmm_s8t_s8n_f32t(q, k_buf[:, :S].contiguous(), alpha_qk)
+    probs = attn_softmax_q(scores, mask, heads)
+    ctx = bmm_s8t_s8t_s8t(probs, v_buf[:, :S].contiguous(), alpha_pv)
+    return ctx, probs, k_buf, v_buf
+
+
 def linear_a8_w8_bfp32_ofp32_acc(x, w, bias, alpha, beta, inout, acc_fn=gemm_acc):
     """ti_linear_a8_w8_bfp32_ofp32_acc: the fp32 linear, rounded, then one fp32 add into ``inout`` (returns a new tensor)."""
     return inout + linear_a8_w8_bfp32_ofp32(x, w, bias, alpha, beta, acc_fn=acc_fn).view(inout.shape)

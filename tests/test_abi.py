@@ -73,6 +73,23 @@ def test_c_abi_rejects_bad_arguments_without_a_device():
     rc = lib.ti_bmm_s8t_s8t_s8t(p, p, p, 2, 1, 4, 16, 8, 1.0, None)
     assert rc == 1 and b"batch stride" in lib.ti_last_error()
     assert lib.ti_kv_append_s8(None, None, None, None, 0, 1, 16, 8, 0, None) == 0
+    # decode attention: shape limits, the pairing of the new rows, alignment; (T, S, head_dim) support query
+    lib.ti_decode_attn_s8.argtypes = [ctypes.c_void_p] * 8 + [i64] * 6 + [ctypes.c_float] * 2 + [ctypes.c_void_p]
+    lib.ti_decode_attn_supported.argtypes = [i64] * 3
+    assert lib.ti_decode_attn_supported(1, 2048, 128) == 1 and lib.ti_decode_attn_supported(4, 2048, 128) == 1
+    assert lib.ti_decode_attn_supported(5, 16, 128) == 0 and lib.ti_decode_attn_supported(1, 16, 96) == 0
+    assert lib.ti_decode_attn_supported(4, 1 << 20, 128) == 0 and lib.ti_decode_attn_supported(1, 0, 128) == 0
+    rc = lib.ti_decode_attn_s8(p, p, p, p, p, None, p, None, 4, 5, 128, 64, 32, 2, 1.0, 1.0, None)
+    assert rc == 1 and b"unsupported shape" in lib.ti_last_error()
+    rc = lib.ti_decode_attn_s8(p, p, None, p, p, None, p, None, 4, 1, 128, 64, 32, 2, 1.0, 1.0, None)
+    assert rc == 1 and b"both" in lib.ti_last_error()
+    rc = lib.ti_decode_attn_s8(p, p, p, p, p, None, p, None, 4, 1, 128, 16, 32, 2, 1.0, 1.0, None)
+    assert rc == 1 and b"do not fit" in lib.ti_last_error()
+    rc = lib.ti_decode_attn_s8(p, p, p, p, p, None, p, None, 3, 1, 128, 64, 32, 2, 1.0, 1.0, None)
+    assert rc == 1 and b"multiple of heads" in lib.ti_last_error()
+    rc = lib.ti_decode_attn_s8(p + 4, p, p, p, p, None, p, None, 4, 1, 128, 64, 32, 2, 1.0, 1.0, None)
+    assert rc == 2 and b"aligned" in lib.ti_last_error()
+    assert lib.ti_decode_attn_s8(None, None, None, None, None, None, None, None, 0, 1, 128, 64, 32, 2, 1.0, 1.0, None) == 0
     # empty problems succeed without touching pointers or a device
     assert lib.ti_linear_a8_w8_b8_o8(None, None, None, None, 0, 16, 16, 1.0, 1.0, None, 0, None) == 0
     assert lib.ti_dq_add_layernorm_q(None, 1.0, None, None, None, 1e-5, None, None, 0, 128, None) == 0

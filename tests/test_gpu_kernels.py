@@ -557,6 +557,49 @@ def test_kv_append_kernel():
         X.kv_append(kn.to(DEV), vn.to(DEV), kd, vd, 1)   # 1 + 16 positions do not fit 16
 
 
+def test_decode_attention_matches_the_separate_kernels_and_the_oracle():
+    # one launch = append + Q.K^T + softmax-quant + P.V of a decode step, bit for bit
+    import torch_int._hip_ext as X
+    import torch_int._CUDA as C
+    g = torch.Generator().manual_seed(29)
+    neg = torch.finfo(torch.float32).min
+    # (batch, heads, cap, d, filled, T, masked)
+    cases = [(4, 72, 656, 128, 543, 1, True), (1, 40, 2064, 128, 2047, 1, False), (2, 12, 96, 64, 70, 1, True),
+             (2, 5, 48, 128, 0, 1, False), (2, 3, 600, 128, 513, 4, True), (1, 2, 80, 64, 61, 3, False),
+             (3, 2, 40, 128, 7, 2, True)]
+    for (B, H, cap, d, S0, T, masked) in cases:
+        _say(f"decode_attn B={B} H={H} cap={cap} d={d} filled={S0} T={T} mask={masked}")
+        S = S0 + T
+        kbuf, vbuf = _s8(g, B * H, cap, d), _s8(g, B * H, cap, d)
+        q, kn, vn = _s8(g, B * H, T, d), _s8(g, B * H, T, d), _s8(g, B * H, T, d)
+        a_qk, a_pv = _scal(g, 1e-4, 2e-3), _scal(g, 1e-3, 1e-2)
+        mask = None
+        if masked:   # padding on the left of some batch rows plus causality among the new tokens
+            mask = torch.zeros(B, 1, T, S)
+            mask[0, :, :, :min(3, S0)] = neg
+            for t in range(T):
+                mask[:, :, t, S0 + t + 1:] = neg
+        ref_ctx, ref_p, ref_k, ref_v = orc.decode_attn_s8(q, kn, vn, kbuf, vbuf, S0, mask, H, a_qk, a_pv)
+        kd, vd = kbuf.view(B, H, cap, d).to(DEV), vbuf.view(B, H, cap, d).to(DEV)
+        args = (q.view(B, H, T, d).to(DEV), kn.view(B, H, T, d).to(DEV), vn.view(B, H, T, d).to(DEV), kd, vd, S0,
+                mask.to(DEV) if masked else None)
+        assert X.can_decode_attention(*args)
+        ctx, probs = X.decode_attention(*args, a_qk, a_pv, want_probs=True)
+        assert torch.equal(probs.cpu(), ref_p), "probabilities"
+        assert torch.equal(ctx.cpu(), ref_ctx), "context"
+        assert torch.equal(kd.cpu().view(B * H, cap, d), ref_k) and torch.equal(vd.cpu().view(B * H, cap, d), ref_v)
+        # and against the kernels it replaces, on the device
+        kc = kd.view(B * H, cap, d)[:, :S].contiguous()
+        sc = C.bmm_s8t_s8n_f32t(q.to(DEV), kc, a_qk)
+        pq = X.attn_softmax_q(sc, args[6], H)
+        assert torch.equal(pq, probs)
+        assert torch.equal(X.bmm_s8t_s8t_s8t(pq, vd.view(B * H, cap, d)[:, :S], a_pv), ctx)
+        ctx2, none = X.decode_attention(*args, a_qk, a_pv)   # same cache rows again, no probabilities wanted
+        assert none is None and torch.equal(ctx2, ctx)
+    assert not X.can_decode_attention(args[0], args[1], args[2], kd, vd, cap, None)        # no room
+    assert not X.can_decode_attention(args[0][:, :, :, :32].contiguous(), args[1], args[2], kd, vd, 0, None)
+
+
 def test_runs_are_deterministic():
     # identical bytes on repeated launches (an LDS race would show up here)
     import torch_int._CUDA as C

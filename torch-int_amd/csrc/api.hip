@@ -322,6 +322,39 @@ int ti_kv_append_s8(const int8_t* k_new, const int8_t* v_new, int8_t* k_buf, int
   return launch_kv_append_s8(k_new, v_new, k_buf, v_buf, BH, T, D, cap, S, static_cast<hipStream_t>(stream));
 }
 
+int ti_decode_attn_supported(int64_t T, int64_t S, int64_t D) { return decode_attn_supported(T, S, D) ? 1 : 0; }
+
+int ti_decode_attn_s8(const int8_t* q, const int8_t* k_new, const int8_t* v_new, int8_t* k_buf, int8_t* v_buf,
+                      const float* mask, int8_t* ctx, int8_t* probs_out, int64_t BH, int64_t T, int64_t D, int64_t cap,
+                      int64_t S, int64_t heads, float alpha_qk, float alpha_pv, void* stream) {
+  g_err[0] = 0;
+  const char* op = "decode_attn_s8";
+  const int64_t lim = 0x7fffffffLL;
+  if (BH < 0 || T < 0 || D < 0 || cap < 0 || S < 0 || heads < 1 || BH > lim || cap > lim || heads > lim)
+    return fail(TI_ERR_INVALID_ARG, "%s: sizes must be in [0, 2^31) and heads >= 1", op);
+  if (BH % heads != 0) return fail(TI_ERR_INVALID_ARG, "%s: BH = %lld is not a multiple of heads = %lld", op,
+                                   (long long)BH, (long long)heads);
+  if ((k_new == nullptr) != (v_new == nullptr))
+    return fail(TI_ERR_INVALID_ARG, "%s: k_new and v_new must both be given or both be NULL", op);
+  if (S > cap) return fail(TI_ERR_INVALID_ARG, "%s: %lld positions do not fit a capacity of %lld", op, (long long)S,
+                           (long long)cap);
+  if (k_new != nullptr && S < T)
+    return fail(TI_ERR_INVALID_ARG, "%s: S = %lld counts the %lld appended positions", op, (long long)S, (long long)T);
+  if (BH == 0) return TI_OK;
+  if (!decode_attn_supported(T, S, D))
+    return fail(TI_ERR_INVALID_ARG, "%s: unsupported shape T=%lld S=%lld head_dim=%lld (needs 1 <= T <= 4, head_dim 64 or "
+                "128, S >= 1 and scores that fit the LDS)", op, (long long)T, (long long)S, (long long)D);
+  if (int rc = check_ptr(op, "q", q, 16, true)) return rc;
+  if (int rc = check_ptr(op, "k_new", k_new, 16, k_new != nullptr)) return rc;
+  if (int rc = check_ptr(op, "v_new", v_new, 16, v_new != nullptr)) return rc;
+  if (int rc = check_ptr(op, "k_buf", k_buf, 16, true)) return rc;
+  if (int rc = check_ptr(op, "v_buf", v_buf, 16, true)) return rc;
+  if (int rc = check_ptr(op, "mask", mask, 4, mask != nullptr)) return rc;
+  if (int rc = check_ptr(op, "ctx", ctx, 1, true)) return rc;
+  return launch_decode_attn_s8(q, k_new, v_new, k_buf, v_buf, mask, ctx, probs_out, BH, T, D, cap, S, heads, alpha_qk,
+                               alpha_pv, static_cast<hipStream_t>(stream));
+}
+
 int ti_transpose_last2_s8(const int8_t* src, int8_t* dst, int64_t B, int64_t R, int64_t C, void* stream) {
   g_err[0] = 0;
   const char* op = "transpose_last2_s8";

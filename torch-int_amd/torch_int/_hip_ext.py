@@ -35,6 +35,11 @@ _lib.ti_bmm_s8t_s8n_f32t_strided.argtypes = [_vp, _vp, _vp, _i64, _i64, _i64, _i
 _lib.ti_bmm_s8t_s8n_f32t_strided.restype = ctypes.c_int
 _lib.ti_kv_append_s8.argtypes = [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp]
 _lib.ti_kv_append_s8.restype = ctypes.c_int
+_lib.ti_decode_attn_supported.argtypes = [_i64, _i64, _i64]
+_lib.ti_decode_attn_supported.restype = ctypes.c_int
+_lib.ti_decode_attn_s8.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32,
+                                   _f32, _vp]
+_lib.ti_decode_attn_s8.restype = ctypes.c_int
 _lib.ti_linear_a8_w8_b8_o8_heads.argtypes = [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _f32, _f32, _i64, _i64, _vp, _i64, _vp]
 _lib.ti_linear_a8_w8_b8_o8_heads.restype = ctypes.c_int
 _pp = ctypes.POINTER(ctypes.c_void_p)
@@ -268,6 +273,51 @@ def kv_append(k_new, v_new, k_buf, v_buf, filled, checked=False):
                                       d, cap, filled, stream or None)
     if rc:
         raise RuntimeError(f"torch_int._hip_ext.kv_append: {_lib.ti_last_error().decode()} (status {rc})")
+
+
+def decode_attention_shape_ok(T, S, d):
+    """Whether ``decode_attention`` takes T query rows over S cache positions of head size d."""
+    return bool(_lib.ti_decode_attn_supported(T, S, d))
+
+
+def can_decode_attention(q, k_new, v_new, k_buf, v_buf, filled, mask):
+    """int8 HIP tensors on one device: q / k_new / v_new [B, H, T, d] contiguous with 1 <= T <= 4 and d 64 or 128,
+    cache buffers [B, H, cap, d] contiguous holding ``filled`` positions with room for T more; mask None or fp32
+    [B, 1, T, filled + T] contiguous; and scores that fit the LDS."""
+    if not (_ok(q, torch.int8) and q.dim() == 4 and can_kv_append(k_new, v_new, k_buf, v_buf)
+            and q.shape == k_new.shape and q.device == k_new.device and q.numel() > 0):
+        return False
+    B, H, T, d = q.shape
+    S = filled + T
+    if S > k_buf.shape[2] or not _lib.ti_decode_attn_supported(T, S, d):
+        return False
+    if any(t.data_ptr() % 16 for t in (q, k_new, v_new, k_buf, v_buf)):
+        return False
+    return mask is None or (_ok(mask, torch.float32) and mask.shape == (B, 1, T, S) and mask.device == q.device)
+
+
+def decode_attention(q, k_new, v_new, k_buf, v_buf, filled, mask, alpha_qk, alpha_pv, want_probs=False,
+                     checked=False):
+    """The attention of a decode step in one launch: writes k_new / v_new behind the ``filled`` positions of the
+    cache buffers and returns (ctx int8 [B*H, T, d], probs int8 [B*H, T, filled+T] or None) with
+    ctx = bmm_s8t_s8t_s8t(round(127 softmax(alpha_qk q k^T + mask)), v, alpha_pv), bit for bit what the separate
+    Q.K^T, softmax and P.V kernels return."""
+    if not checked and not can_decode_attention(q, k_new, v_new, k_buf, v_buf, filled, mask):
+        raise RuntimeError("torch_int._hip_ext.decode_attention: needs contiguous int8 HIP q/k_new/v_new [B,H,T,d] "
+                           "(T <= 4, d 64 or 128), cache buffers [B,H,cap,d] with room, and an fp32 mask [B,1,T,S] or None")
+    B, H, T, d = q.shape
+    S = filled + T
+    dev = q.device
+    ctx = torch.empty((B * H, T, d), dtype=torch.int8, device=dev)
+    probs = torch.empty((B * H, T, S), dtype=torch.int8, device=dev) if want_probs else None
+    with _on(dev):
+        rc = _lib.ti_decode_attn_s8(q.data_ptr(), k_new.data_ptr(), v_new.data_ptr(), k_buf.data_ptr(), v_buf.data_ptr(),
+                                    mask.data_ptr() if mask is not None else None, ctx.data_ptr(),
+                                    probs.data_ptr() if probs is not None else None, B * H, T, d, k_buf.shape[2], S, H,
+                                    alpha_qk, alpha_pv, _raw_stream(dev.index) or None)
+    if rc:
+        raise RuntimeError(f"torch_int._hip_ext.decode_attention: {_lib.ti_last_error().decode()} (status {rc})")
+    return ctx, probs
 
 
 def can_linear_group(x, weights, biases):

@@ -175,6 +175,31 @@ class Int8OPTAttention(nn.Module):
         return _hip_ext.split_heads(tensor, bsz, seq_len, self.num_heads, self.head_dim)
 
     @torch.no_grad()
+    def _decode_fused(self, query4, key, value, past_key_value, attention_mask, output_attentions):
+        """The whole attention of a decode step (cache append, Q.K^T, softmax-quant, P.V) as one kernel launch,
+        or None when the shapes, the cache or the product modules do not allow it; same values as the separate
+        steps of ``forward``."""
+        past_k, past_v = past_key_value
+        if not (type(self.qk_bmm) is BMM_S8T_S8N_F32T and type(self.pv_bmm) is BMM_S8T_S8N_S8T
+                and past_k.dim() == 4 and past_v.shape == past_k.shape):
+            return None
+        bsz, H, T, d = query4.shape
+        S0 = past_k.shape[2]
+        if not _hip_ext.decode_attention_shape_ok(T, S0 + T, d):
+            return None
+        kk = _kv_room(past_k, key) or _kv_fresh(past_k, T)
+        vv = _kv_room(past_v, value) or _kv_fresh(past_v, T)
+        if not _hip_ext.can_decode_attention(query4, key, value, kk.buf, vv.buf, S0, attention_mask):
+            return None   # (a buffer made above is simply dropped; the caller builds its own)
+        ctx, probs = _hip_ext.decode_attention(query4, key, value, kk.buf, vv.buf, S0, attention_mask,
+                                               self.qk_bmm._scalar("a"), self.pv_bmm._scalar("a"),
+                                               want_probs=output_attentions, checked=True)
+        kk.filled = vv.filled = S0 + T
+        present = (_kv_view(kk, S0 + T), _kv_view(vv, S0 + T))
+        probs_out = probs.view(bsz, H, T, S0 + T).float() if output_attentions else None
+        ctx = _hip_ext.merge_heads(ctx, bsz, H, T, d)
+        return self.out_proj(ctx), probs_out, present
+
     def forward(self, hidden_states: torch.Tensor, key_value_states: Optional[torch.Tensor] = None,
                 past_key_value: Optional[Tuple[torch.Tensor]] = None,
                 attention_mask: Optional[torch.Tensor] = None,
@@ -208,6 +233,10 @@ class Int8OPTAttention(nn.Module):
                 key = self._shape(self.k_proj(kv_src), -1, bsz)
                 value = self._shape(self.v_proj(kv_src), -1, bsz)
             if not cross and past_key_value is not None:
+                if self.kv_cache_in_place and proj is not None and tgt_len <= 4 and layer_head_mask is None:
+                    fused = self._decode_fused(query4, key, value, past_key_value, attention_mask, output_attentions)
+                    if fused is not None:
+                        return fused
                 if self.kv_cache_in_place:
                     key, value = _kv_append_pair(past_key_value[0], past_key_value[1], key, value)
                 else:
