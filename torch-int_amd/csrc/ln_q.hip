@@ -42,7 +42,10 @@ __device__ __forceinline__ int pack_s8x4(float y0, float y1, float y2, float y3)
 enum LnMode : int { MODE_DQ_ADD = 0, MODE_ADD = 1, MODE_PLAIN = 2 };
 
 // H % 4 == 0, H <= NC * 1024, all row starts 16-byte aligned.
-template <int NC, int MODE>
+// EARLY: gamma and beta are fetched together with the row instead of after the two reductions; with only
+// a few rows in flight (decode) the kernel is a chain of memory latencies and this removes one of them,
+// with many rows the extra registers would only cost occupancy.
+template <int NC, int MODE, bool EARLY = false>
 __global__ __launch_bounds__(256) void ln_q_rows_kernel(const int32_t* __restrict__ in, float scale,
                                                         const float* res,  // may alias r_out
                                                         const float* __restrict__ gamma,
@@ -57,6 +60,19 @@ __global__ __launch_bounds__(256) void ln_q_rows_kernel(const int32_t* __restric
   v4f* rout4 = reinterpret_cast<v4f*>(r_out + row * H);
   int* q4 = reinterpret_cast<int*>(q_out + row * H);
 
+  const v4f* g4 = reinterpret_cast<const v4f*>(gamma);
+  const v4f* b4 = reinterpret_cast<const v4f*>(beta);
+  v4f ge[EARLY ? NC : 1], be[EARLY ? NC : 1];
+  if constexpr (EARLY) {
+#pragma unroll
+    for (int i = 0; i < NC; ++i) {
+      const int c = t + i * 256;
+      if (c < nchunks) {
+        ge[i] = g4[c];
+        be[i] = b4[c];
+      }
+    }
+  }
   v4f r[NC];
   float s = 0.0f;
 #pragma unroll
@@ -99,13 +115,18 @@ __global__ __launch_bounds__(256) void ln_q_rows_kernel(const int32_t* __restric
   }
   const float var = block_sum_256(s2, red) / fH;
   const float rstd = 1.0f / __builtin_sqrtf(var + eps);
-  const v4f* g4 = reinterpret_cast<const v4f*>(gamma);
-  const v4f* b4 = reinterpret_cast<const v4f*>(beta);
 #pragma unroll
   for (int i = 0; i < NC; ++i) {
     const int c = t + i * 256;
     if (c < nchunks) {
-      v4f g = g4[c], b = b4[c];
+      v4f g, b;
+      if constexpr (EARLY) {
+        g = ge[i];
+        b = be[i];
+      } else {
+        g = g4[c];
+        b = b4[c];
+      }
       float y[4];
 #pragma unroll
       for (int j = 0; j < 4; ++j) y[j] = __builtin_fmaf((r[i][j] - mu) * rstd, g[j], b[j]);
@@ -174,15 +195,22 @@ static void launch_rows(int mode, const int32_t* in, float scale, const float* r
                         const float* beta, float eps, float* r_out, int8_t* q_out, long long rows, int H,
                         hipStream_t stream) {
   const dim3 grid((unsigned)rows), block(256);
-  if (mode == MODE_DQ_ADD)
-    hipLaunchKernelGGL((ln_q_rows_kernel<NC, MODE_DQ_ADD>), grid, block, 0, stream, in, scale, res, gamma, beta, eps,
-                       r_out, q_out, H);
-  else if (mode == MODE_ADD)
-    hipLaunchKernelGGL((ln_q_rows_kernel<NC, MODE_ADD>), grid, block, 0, stream, in, scale, res, gamma, beta, eps,
-                       r_out, q_out, H);
-  else
-    hipLaunchKernelGGL((ln_q_rows_kernel<NC, MODE_PLAIN>), grid, block, 0, stream, in, scale, res, gamma, beta, eps,
-                       r_out, q_out, H);
+  const bool early = rows <= 64;  // fewer rows than CUs: latency-bound
+#define TI_LN_LAUNCH(MODE)                                                                                     \
+  if (early)                                                                                                   \
+    hipLaunchKernelGGL((ln_q_rows_kernel<NC, MODE, true>), grid, block, 0, stream, in, scale, res, gamma, beta, eps, \
+                       r_out, q_out, H);                                                                       \
+  else                                                                                                         \
+    hipLaunchKernelGGL((ln_q_rows_kernel<NC, MODE, false>), grid, block, 0, stream, in, scale, res, gamma, beta, eps, \
+                       r_out, q_out, H)
+  if (mode == MODE_DQ_ADD) {
+    TI_LN_LAUNCH(MODE_DQ_ADD);
+  } else if (mode == MODE_ADD) {
+    TI_LN_LAUNCH(MODE_ADD);
+  } else {
+    TI_LN_LAUNCH(MODE_PLAIN);
+  }
+#undef TI_LN_LAUNCH
 }
 
 static int launch_ln_mode(int mode, const void* in, float scale, const float* res, const float* gamma,
