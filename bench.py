@@ -8,9 +8,11 @@ is resident in HBM before the clock starts.  `value` = 2*M*N*K summed over the s
 divided by the wall time of a step, in TOPS.
 
 Also reported on the same JSON line:
-  roofline      the MFMA-bound part of the sweep (M >= 2048): ops per launch / mean launch
-                duration, against 5.0 POP/s.  The top-level figures come from HIP events
-                recorded around those launches inside the timed steps; `sustained` repeats
+  roofline      the dominant kernel of the sweep (the kernel family with the largest share of
+                the launch time): ops per launch / mean launch duration over the launches the
+                library routes to it, against 5.0 POP/s, with the other MFMA kernel family and
+                all MFMA-bound launches beside it.  The top-level figures come from HIP events
+                recorded around the launches inside the timed steps; `sustained` repeats
                 the measurement with the reference's own protocol (benchmark/utils.py:81-96:
                 100 warm-up launches, then a window of at least 200 ms of back-to-back
                 launches of one case), where the clock has settled under the power limit;
@@ -42,8 +44,10 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
 # the process: they come from rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) of this script's own sweep; commands,
 # raw counter values and the calibration against a plain copy kernel are in profiles/.
 FAMILIES = {
-    "pipe_256x256": {"kernel": "gemm_pipe2_kernel<Pipe2Cfg<256,256,2,4,KIND,SWAP>>", "traffic": None},
-    "pipe16_256x160": {"kernel": "gemm_pipe16q_kernel<Pipe16QCfg<256,160,4,2,KIND>>", "traffic": None},
+    # 273 944 KiB x 2.000 fetched + 76 686 KiB written per launch, mean over its 24 launches per step
+    "pipe16_256x160": {"kernel": "gemm_pipe16q_kernel<Pipe16QCfg<256,160,4,2,KIND>>", "traffic": 0.640e9},
+    # 614 682 KiB x 2.000 fetched + 417 713 KiB written per launch, mean over its 4 launches per step
+    "pipe_256x256": {"kernel": "gemm_pipe2_kernel<Pipe2Cfg<256,256,2,4,KIND,SWAP>>", "traffic": 1.687e9},
 }
 SHAPES = [(5120, 5120), (20480, 5120), (5120, 20480)]   # (N, K): qkv/out_proj, fc1, fc2
 MS = [1, 16, 128, 512, 2048, 8192]
@@ -223,14 +227,16 @@ def main():
         c["kernel"] = C._lib.ti_last_kernel().decode()
     torch.cuda.synchronize()
 
-    heavy = [i for i, c in enumerate(cases) if c["M"] >= 2048]   # the MFMA-bound launches
+    # launches bracketed by HIP events: everything from M = 512 up (all the cases the tiled MFMA kernels take)
+    heavy = [i for i, c in enumerate(cases) if c["M"] >= 512]
+    ridge = PEAK_INT8_TOPS * 1e3 / PEAK_HBM_GBS   # ops per byte above which the MFMA roofline binds
     marks = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in heavy]
              for _ in range(args.steps)]
 
     def step(ev=None):
         k = 0
         for c in cases:
-            if ev is not None and c["M"] >= 2048:
+            if ev is not None and c["M"] >= 512:
                 ev[k][0].record()
                 c["fn"]()
                 ev[k][1].record()
@@ -246,8 +252,9 @@ def main():
         step(marks[i])
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
-    heavy_ms = sum(a.elapsed_time(b) for ev in marks for (a, b) in ev) / max(args.steps, 1)   # per step
-    heavy_ops = sum(cases[i]["ops"] for i in heavy)
+    bound_k = [k for k, i in enumerate(heavy) if cases[i]["ops"] / cases[i]["bytes"] >= ridge]
+    heavy_ms = sum(ev[k][0].elapsed_time(ev[k][1]) for ev in marks for k in bound_k) / max(args.steps, 1)   # per step
+    heavy_ops = sum(cases[heavy[k]]["ops"] for k in bound_k)
     # the dominant kernel: the family that takes the largest share of the timed launches
     fam = {}
     for k, i in enumerate(heavy):
@@ -282,7 +289,7 @@ def main():
         "ops_per_launch": dom_ops / len(dom), "avg_launch_ms": dom_ms / len(dom), "launches_per_step": len(dom),
         "protocol": "HIP events around each of these launches inside the timed steps",
         "all_mfma_bound_cases": {"achieved": heavy_ops / heavy_ms / 1e9, "frac": heavy_ops / heavy_ms / 1e9 / PEAK_INT8_TOPS,
-                                 "launches_per_step": len(heavy), "avg_launch_ms": heavy_ms / len(heavy)},
+                                 "launches_per_step": len(bound_k), "avg_launch_ms": heavy_ms / len(bound_k)},
         "families": {name: {"kernel": FAMILIES.get(name, {}).get("kernel", name), "launches_per_step": len(f["idx"]),
                             "avg_launch_ms": f["ms"] / len(f["idx"]), "achieved": f["ops"] / f["ms"] / 1e9,
                             "frac": f["ops"] / f["ms"] / 1e9 / PEAK_INT8_TOPS,
@@ -303,14 +310,14 @@ def main():
                     n_copies = -(-320 * 2 ** 20 // (c["N"] * c["K"]))
                     copies[key] = [c["w"]] + [c["w"].clone() for _ in range(n_copies - 1)]
                 fns = [c["make"](w) for w in copies[key]]
-            ms = sustained_ms(torch, fns, window_ms=200.0 if c["M"] >= 2048 else 60.0)
+            ms = sustained_ms(torch, fns, window_ms=200.0 if c["M"] >= 512 and c["kernel"] == DOMINANT or c["M"] >= 2048 else 60.0)
             tops = c["ops"] / ms / 1e9
             gbs = c["bytes"] / ms / 1e6
             frac = tops / PEAK_INT8_TOPS if bound == "mfma" else gbs / PEAK_HBM_GBS
             table.append({"variant": c["variant"], "M": c["M"], "N": c["N"], "K": c["K"], "kernel": c["kernel"],
                           "us": round(ms * 1e3, 2),
                           "TOPS": round(tops, 1), "GBps": round(gbs, 1), "bound": bound, "frac": round(frac, 4)})
-            if c["kernel"] == DOMINANT and c["M"] >= 2048:
+            if c["kernel"] == DOMINANT and c["M"] >= 512:
                 mfma_ops += c["ops"]
                 mfma_ms += ms
         del copies

@@ -99,7 +99,7 @@ def test_linear_shapes(variant):
 def test_linear_large_tiles(variant):
     # enough 256x256 tiles to select the large-tile kernel, with ragged M and N
     import torch_int._CUDA as C
-    for (M, N, K) in [(2048, 5120, 256), (2100, 5000, 272), (4096, 2560, 128)]:
+    for (M, N, K) in [(2048, 5120, 256), (2100, 5000, 272), (4096, 2560, 128), (4000, 2816, 1024)]:
         _say(f"linear-large {variant} M={M} N={N} K={K}")
         _linear_case(C, variant, M, N, K, seed=7)
 
@@ -431,7 +431,7 @@ def test_linear_accumulate_into_output():
     g = torch.Generator().manual_seed(63)
     seen = set()
     for (M, N, K) in [(2048, 5120, 256), (2048, 5120, 64), (2000, 9216, 192), (2000, 9216, 128), (4096, 2816, 128),
-                      (4096, 2816, 320), (1024, 2048, 64), (1024, 5120, 5120), (4, 4608, 16384),
+                      (4096, 2816, 1024), (1024, 2048, 64), (1024, 5120, 5120), (4, 4608, 16384),
                       (128, 640, 4096), (16, 5120, 3072), (3, 100, 272), (300, 200, 48), (2100, 5000, 272),
                       (70, 50, 37), (4, 64, 0)]:
         _say(f"linear += M={M} N={N} K={K}")

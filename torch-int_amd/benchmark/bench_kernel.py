@@ -38,7 +38,7 @@ LINEAR = {
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--op", required=True, choices=list(LINEAR) + ["bmm_f32t", "bmm_s8t", "bmm_s32t", "bmm_s8t_rowmajor", "ln_q", "add_ln_q",
-                                               "softmax_q", "copy"])
+                                               "softmax_q", "decode_attn", "copy"])
     ap.add_argument("--shape", type=int, nargs="+", required=True)
     ap.add_argument("--iters", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
@@ -100,6 +100,20 @@ def main():
         mask = mask[None, None].expand(batch, 1, T, S).contiguous()
         fn = lambda: X.attn_softmax_q(scores, mask, heads)  # noqa: E731
         nbytes = 5.0 * batch * heads * T * S + 4.0 * batch * T * S
+    elif args.op == "decode_attn":
+        # one decode step's attention: batch, heads, cached positions, head size, new tokens; --rotate cache copies
+        batch, heads, filled, d, T = args.shape
+        cap = -(-(filled + T + 64) // 16) * 16
+        caches = [(s8(batch, heads, cap, d), s8(batch, heads, cap, d)) for _ in range(args.rotate)]
+        q, kn, vn = s8(batch, heads, T, d), s8(batch, heads, T, d), s8(batch, heads, T, d)
+        mask = torch.zeros(batch, 1, T, filled + T, device=dev)
+        state = {"i": 0}
+
+        def fn():
+            state["i"] = (state["i"] + 1) % len(caches)
+            kb, vb = caches[state["i"]]
+            return X.decode_attention(q, kn, vn, kb, vb, filled, mask, 0.001, 0.004)
+        nbytes = 2.0 * batch * heads * (filled + T) * d
     elif args.op == "add_ln_q":
         rows, H = args.shape
         x = torch.randn(rows, H, device=dev, generator=g)

@@ -197,7 +197,9 @@ __device__ __forceinline__ void store_tile(v16i (&acc)[Cfg::TM][Cfg::TN], const 
       // instruction writes eight whole 128-byte lines instead of two
       const int nq = n0 + wave_n * Cfg::WTN + j * 32;  // first column of the block
       if constexpr (sizeof(Out) == 4) {
-       if ((N & 3) == 0 && nq + 32 <= N && (reinterpret_cast<uintptr_t>(C) & 15) == 0) {
+       // (short K, e.g. Q.K^T with K = head size: the epilogue is most of the kernel and the plain stores,
+       // which need no lane exchanges, are faster)
+       if (p.K >= 1024 && (N & 3) == 0 && nq + 32 <= N && (reinterpret_cast<uintptr_t>(C) & 15) == 0) {
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
 #pragma unroll
