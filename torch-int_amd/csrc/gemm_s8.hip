@@ -934,9 +934,6 @@ __device__ __forceinline__ void store_tile16(v4i (&acc)[Cfg::TM][Cfg::TN], const
 
 template <class Cfg>
 __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe16_kernel(GemmParams p, int tiles_m, int tiles_n, int items) {
-  using E = Epi<Cfg::KIND>;
-  using Out = typename E::Out;
-  using BiasT = typename E::Bias;
   constexpr int BM = Cfg::BM, BN = Cfg::BN, TM = Cfg::TM, TN = Cfg::TN, COPIES = Cfg::COPIES, S = Cfg::STAGES;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
