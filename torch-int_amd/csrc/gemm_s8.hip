@@ -1769,29 +1769,8 @@ static int choose_splits(long long M, long long N, long long K, int* tile_edge =
   return best;
 }
 
-// K slices for the streaming (M <= 16) kernel.  A strip of 16 weight rows is one work item; when a matrix
-// has few, long strips (N small, K large: fc2, out_proj) the CUs end up with unequal numbers of them.
-// Cost in units of one 1 KiB-deep block per CU: the most loaded CU's items times their depth (+0.5 per item
-// for the reduction between the waves), +4 for the second launch that adds the slices.
-static int choose_stream_splits(long long M, long long N, long long K) {
-  if (M > 16 || K % SBK != 0) return 1;
-  const long long strips = (N + 15) / 16, blocks = K / SBK, cus = num_cus();
-  if (strips < 256) return 1;
-  int best = 1;
-  double best_c = (double)((strips + cus - 1) / cus) * ((double)blocks + 0.5);
-  for (int sp = 2; sp <= 8; ++sp) {
-    if (blocks % sp != 0 || blocks / sp < 2) continue;
-    const double c = (double)((strips * sp + cus - 1) / cus) * ((double)(blocks / sp) + 0.5) + 4.0;
-    if (c < best_c * 0.9) {
-      best_c = c;
-      best = sp;
-    }
-  }
-  return best;
-}
-
 long long gemm_workspace_bytes(long long M, long long N, long long K) {
-  const int s = M <= 16 ? choose_stream_splits(M, N, K) : choose_splits(M, N, K);
+  const int s = choose_splits(M, N, K);
   return s > 1 ? (long long)s * M * N * 4 : 0;
 }
 
@@ -1812,30 +1791,6 @@ static int launch_kind(const GemmParams& p, void* workspace, long long workspace
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "gemm launch: %s", hipGetErrorString(e));
     return TI_OK;
-  }
-  if (p.M <= 16 && p.batch == 1 && p.lda == p.K && p.ldb == p.K && KIND != EPI_S32_RAW) {
-    const int splits = choose_stream_splits(p.M, p.N, p.K);
-    const long long need = (long long)splits * p.M * p.N * 4;
-    if (splits > 1 && workspace != nullptr && workspace_bytes >= need &&
-        (reinterpret_cast<uintptr_t>(workspace) & 15) == 0) {
-      GemmParams q = p;  // the K slices are the batches of one raw-int32 product into the workspace
-      q.K = p.K / splits;
-      q.batch = splits;
-      q.strideA = q.K;
-      q.strideB = q.K;
-      q.strideC = (long long)p.M * p.N;
-      q.C = workspace;
-      q.bias = nullptr;
-      q.out_T = q.out_d = 0;
-      if (int rc = launch_kind<EPI_S32_RAW>(q, nullptr, 0, stream)) return rc;
-      g_last_kernel = "stream_splitk";
-      const long long quads = ((long long)p.M * p.N + 3) / 4;
-      hipLaunchKernelGGL(splitk_reduce_kernel<KIND>, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream, p,
-                         static_cast<const int*>(workspace), splits);
-      hipError_t e = hipGetLastError();
-      if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "split-K reduce launch: %s", hipGetErrorString(e));
-      return TI_OK;
-    }
   }
   if (p.M <= 16 && p.K % SBK == 0 && (long long)((p.N + 15) / 16) * p.batch >= 256) {
     g_last_kernel = "stream";

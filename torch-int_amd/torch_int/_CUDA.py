@@ -190,8 +190,8 @@ def _linear(op, kind, x, w, bias, bias_dtype, out_dtype, alpha, beta, inout=None
         torch.cuda.set_device(idx)
     try:
         stream = _raw_stream(idx)
-        # split-K scratch is only ever wanted up to mid-sized M (see the split choosers in csrc/gemm_s8.hip)
-        ws_ptr, ws_bytes = _workspace(idx, stream, _ws_bytes(M, N, K)) if M <= 1024 else (0, 0)
+        # split-K scratch is only ever wanted for mid-sized M (see choose_splits in csrc/gemm_s8.hip)
+        ws_ptr, ws_bytes = _workspace(idx, stream, _ws_bytes(M, N, K)) if 16 < M <= 1024 else (0, 0)
         if _fast is not None:
             rc = _fast.linear(kind, x.data_ptr(), w.data_ptr(), bias.data_ptr(), out.data_ptr(), M, N, K,
                               alpha, beta, ws_ptr, ws_bytes, stream)
