@@ -205,6 +205,17 @@ int ti_decode_attn_s8(const int8_t* q, const int8_t* k_new, const int8_t* v_new,
                       const float* mask, int8_t* ctx, int8_t* probs_out, int64_t BH, int64_t T, int64_t D, int64_t cap,
                       int64_t S, int64_t heads, float alpha_qk, float alpha_pv, void* stream);
 
+/* probs[bh, t, :] = int8 round(127 * softmax(max(alpha * q[bh, t, :] . k[bh, :, :]^T + mask, most negative float)))
+ * in one launch: ti_bmm_s8t_s8n_f32t followed by ti_attn_softmax_q (torch_int/models/opt.py:137-178) without the
+ * fp32 score tensor in between; the same bits.  q is [BH, T, D] with stride_q elements between batches, k is
+ * [BH, S, D] with stride_k, rows packed; mask fp32 [BH/heads, 1, T, S] or NULL; probs [BH, T, S] packed.
+ * Limits: D = 128, S a multiple of 16 in [16, 512]: ti_attn_qk_softmax_q_supported(T, S, D) says whether a shape
+ * is accepted. */
+int ti_attn_qk_softmax_q_supported(int64_t T, int64_t S, int64_t D);
+int ti_attn_qk_softmax_q(const int8_t* q, const int8_t* k, const float* mask, int8_t* probs, int64_t BH, int64_t T,
+                         int64_t S, int64_t D, int64_t stride_q, int64_t stride_k, int64_t heads, float alpha,
+                         void* stream);
+
 #ifdef __cplusplus
 }
 #endif

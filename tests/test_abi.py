@@ -90,6 +90,19 @@ def test_c_abi_rejects_bad_arguments_without_a_device():
     rc = lib.ti_decode_attn_s8(p + 4, p, p, p, p, None, p, None, 4, 1, 128, 64, 32, 2, 1.0, 1.0, None)
     assert rc == 2 and b"aligned" in lib.ti_last_error()
     assert lib.ti_decode_attn_s8(None, None, None, None, None, None, None, None, 0, 1, 128, 64, 32, 2, 1.0, 1.0, None) == 0
+    # fused Q.K^T + softmax-quant: shape limits, batch strides, alignment
+    lib.ti_attn_qk_softmax_q.argtypes = [ctypes.c_void_p] * 4 + [i64] * 7 + [ctypes.c_float, ctypes.c_void_p]
+    lib.ti_attn_qk_softmax_q_supported.argtypes = [i64] * 3
+    assert lib.ti_attn_qk_softmax_q_supported(512, 512, 128) == 1 and lib.ti_attn_qk_softmax_q_supported(1, 16, 128) == 1
+    assert lib.ti_attn_qk_softmax_q_supported(512, 528, 128) == 0 and lib.ti_attn_qk_softmax_q_supported(512, 40, 128) == 0
+    assert lib.ti_attn_qk_softmax_q_supported(512, 512, 64) == 0
+    rc = lib.ti_attn_qk_softmax_q(p, p, None, p, 4, 64, 520, 128, 64 * 128, 520 * 128, 2, 1.0, None)
+    assert rc == 1 and b"unsupported shape" in lib.ti_last_error()
+    rc = lib.ti_attn_qk_softmax_q(p, p, None, p, 4, 64, 64, 128, 64 * 128, 63 * 128, 2, 1.0, None)
+    assert rc == 1 and b"batch strides" in lib.ti_last_error()
+    rc = lib.ti_attn_qk_softmax_q(p, p + 8, None, p, 4, 64, 64, 128, 64 * 128, 64 * 128, 2, 1.0, None)
+    assert rc == 2 and b"aligned" in lib.ti_last_error()
+    assert lib.ti_attn_qk_softmax_q(None, None, None, None, 0, 64, 64, 128, 0, 0, 2, 1.0, None) == 0
     # empty problems succeed without touching pointers or a device
     assert lib.ti_linear_a8_w8_b8_o8(None, None, None, None, 0, 16, 16, 1.0, 1.0, None, 0, None) == 0
     assert lib.ti_dq_add_layernorm_q(None, 1.0, None, None, None, 1e-5, None, None, 0, 128, None) == 0

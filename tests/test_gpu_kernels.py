@@ -601,6 +601,42 @@ def test_decode_attention_matches_the_separate_kernels_and_the_oracle():
     assert not X.can_decode_attention(args[0][:, :, :, :32].contiguous(), args[1], args[2], kd, vd, 0, None)
 
 
+def test_fused_qk_softmax_matches_the_two_kernels_and_the_oracle():
+    # Q.K^T + mask + softmax + quantise in one launch: the bytes of bmm_s8t_s8n_f32t followed by attn_softmax_q
+    import torch_int._hip_ext as X
+    import torch_int._CUDA as C
+    g = torch.Generator().manual_seed(83)
+    neg = torch.finfo(torch.float32).min
+    # (batch, heads, T, S, mask kind)
+    cases = [(4, 40, 512, 512, "causal"), (2, 3, 100, 96, "pad"), (1, 4, 64, 16, None), (2, 2, 70, 272, "causal"),
+             (1, 2, 1, 512, None), (3, 1, 130, 144, "pad"), (1, 2, 300, 304, "causal")]
+    for (B, H, T, S, kind) in cases:
+        _say(f"qk_softmax B={B} H={H} T={T} S={S} mask={kind}")
+        q, k = _s8(g, B * H, T, 128), _s8(g, B * H, S, 128)
+        alpha = _scal(g, 2e-4, 2e-3)
+        mask = None
+        if kind is not None:
+            mask = torch.zeros(B, 1, T, S)
+            if kind == "causal":
+                mask += torch.zeros(T, S).masked_fill(torch.arange(S)[None, :] > torch.arange(T)[:, None] + (S - T), neg)
+            mask[0, :, :, :5] = neg      # left padding of the first batch row (adds up with causality, may overflow to -inf)
+        ref = orc.attn_softmax_q(orc.bmm_s8t_s8n_f32t(q, k, alpha), mask, H)
+        qd, kd, md = q.to(DEV), k.to(DEV), (mask.to(DEV) if mask is not None else None)
+        assert X.can_attn_qk_softmax_q(qd, kd, md, B, H)
+        out = X.attn_qk_softmax_q(qd, kd, md, alpha, H)
+        assert out.shape == (B * H, T, S) and out.dtype == torch.int8
+        assert torch.equal(out.cpu(), ref), (B, H, T, S, kind, (out.cpu() != ref).sum().item())
+        two = X.attn_softmax_q(C.bmm_s8t_s8n_f32t(qd, kd, alpha), md, H)
+        assert torch.equal(out, two)
+        # keys read in place from a longer cache buffer (batch stride > S * 128)
+        buf = torch.zeros(B * H, S + 48, 128, dtype=torch.int8, device=DEV)
+        buf[:, :S] = kd
+        assert X.can_attn_qk_softmax_q(qd, buf[:, :S], md, B, H)
+        assert torch.equal(X.attn_qk_softmax_q(qd, buf[:, :S], md, alpha, H), out)
+    assert not X.can_attn_qk_softmax_q(qd, kd[:, :40], None, B, H)          # S not a multiple of 16
+    assert not X.can_attn_qk_softmax_q(qd[:, :, :64].contiguous(), kd[:, :, :64].contiguous(), None, B, H)
+
+
 def test_runs_are_deterministic():
     # identical bytes on repeated launches (an LDS race would show up here)
     import torch_int._CUDA as C

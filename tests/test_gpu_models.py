@@ -126,9 +126,21 @@ def test_decoder_layer_opt13b_shape():
     mask = causal_mask(B, T, T)
     gl = copy.deepcopy(layer).to(DEV)
     rec, handles = _capture(gl)
+    # at this shape Q.K^T and the softmax run as one kernel (the qk_bmm module is bypassed): record its operands
+    import torch_int._hip_ext as X
+    fused = X.attn_qk_softmax_q
+
+    def spy(q, k, m, alpha, heads, checked=False):
+        p = fused(q, k, m, alpha, heads, checked=checked)
+        rec["qk"] = ((q.detach().clone(), k.detach().clone()), p.detach().clone(), alpha)
+        return p
+    X.attn_qk_softmax_q = spy
     _say("decoder layer OPT-13B shape: GPU forward")
     h_gpu = hidden.to(DEV)
-    out = gl(h_gpu, attention_mask=mask.to(DEV), use_cache=True)
+    try:
+        out = gl(h_gpu, attention_mask=mask.to(DEV), use_cache=True)
+    finally:
+        X.attn_qk_softmax_q = fused
     assert out[0] is h_gpu and out[0].shape == (B, T, D) and torch.isfinite(out[0]).all()
     for h in handles:
         h.remove()
@@ -147,7 +159,7 @@ def test_decoder_layer_opt13b_shape():
     # q/k/v are written head-major by their GEMMs (the projection modules' forward is bypassed): what the two
     # attention products received must be the plain linears of the first LayerNorm's output, head-split
     x_qkv = rec["ln1"][1].cpu().view(B * T, -1)[rows].contiguous()
-    (q_in, k_in), _ = rec["qk"]
+    (q_in, k_in), _, _ = rec["qk"]
     (_, vt_in), _ = rec["pv"]
     got = {"q": q_in, "k": k_in, "v": vt_in.transpose(1, 2)}
     for name, lin in (("q", a.q_proj), ("k", a.k_proj), ("v", a.v_proj)):
@@ -166,10 +178,14 @@ def test_decoder_layer_opt13b_shape():
     assert torch.equal(rec["fc2"][1].cpu().view(B * T, -1)[rows], ref)
     heads = torch.tensor([0, 39, 77, 159])
     _say("  check qk / pv")
-    (q_in, k_in), s_out = rec["qk"]
-    assert s_out.shape == (B * H, T, T)
-    assert torch.equal(s_out[heads].cpu(), orc.bmm_s8t_s8n_f32t(q_in[heads].cpu(), k_in[heads].cpu(), a.qk_bmm.a.item()))
+    (q_in, k_in), p_out, alpha_qk = rec["qk"]
+    assert p_out.shape == (B * H, T, T) and alpha_qk == a.qk_bmm.a.item()
+    s_ref = orc.bmm_s8t_s8n_f32t(q_in[heads].cpu(), k_in[heads].cpu(), alpha_qk)   # heads of batch 0, 0, 1, 3
+    for i, hd in enumerate(heads.tolist()):   # the fused kernel = the oracle's product, then its softmax-quantiser
+        ref_p = orc.attn_softmax_q(s_ref[i:i + 1], mask[hd // H:hd // H + 1], 1)
+        assert torch.equal(p_out[hd:hd + 1].cpu(), ref_p), hd
     (p_in, v_in), c_out = rec["pv"]
+    assert torch.equal(p_in, p_out)
     assert c_out.shape == (B * H, T, D // H) and int(p_in.min()) >= 0
     assert torch.equal(c_out[heads].cpu(), orc.bmm_s8t_s8n_s8t(p_in[heads].cpu(), v_in[heads].cpu(), a.pv_bmm.a.item()))
     # fp32 library pieces: LayerNormQ (int8 within one LSB) and softmax -> int8 probabilities
@@ -179,7 +195,7 @@ def test_decoder_layer_opt13b_shape():
         ref = ln(x)
         assert (y.int() - ref.int()).abs().max() <= 1 and (y != ref).float().mean() < 1e-3, name
     probs_gpu = p_in[heads].float() / 127
-    scores = s_out[heads].cpu().view(4, T, T) + mask[0, 0]
+    scores = s_ref.view(4, T, T) + mask[0, 0]
     probs_cpu = torch.softmax(torch.clamp_min(scores, torch.finfo(torch.float32).min), -1)
     assert (probs_gpu.cpu() - probs_cpu).abs().max() <= 0.5 / 127 + 1e-3
     # residual algebra: out = hidden + attn_out + fc2_out, in that order, in fp32

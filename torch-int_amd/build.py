@@ -12,7 +12,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "torch_int", "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libtorch_int_hip.so")
-SOURCES = ["api.hip", "gemm_s8.hip", "ln_q.hip", "softmax_q.hip", "permute.hip", "bmm_rowmajor.hip", "decode_attn.hip"]
+SOURCES = ["api.hip", "gemm_s8.hip", "ln_q.hip", "softmax_q.hip", "permute.hip", "bmm_rowmajor.hip", "decode_attn.hip", "attn_fused.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [

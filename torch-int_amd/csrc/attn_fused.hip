@@ -1,0 +1,249 @@
+// Q.K^T fused with the mask, the softmax and the int8 quantisation of the probabilities, for prefill with
+// up to 512 key positions and head size 128: probs = round(127 softmax(max(alpha q.k^T + mask, lowest))).
+// The fp32 scores (4 bytes per query-key pair written and read again by the two-kernel form) never leave
+// the registers.  Arithmetic and summation order are those of attn_softmax_q on the scores of
+// bmm_s8t_s8n_f32t, so the bytes are the same.
+//
+// One workgroup of four waves per (batch * head, block of 64 query rows).  The 64 query rows and all S key
+// rows are copied to LDS once (128-byte rows, chunk c of row r at position c ^ ((r >> 1) & 7)).  A wave owns
+// 16 query rows and all S keys: S/16 blocks of v_mfma_i32_16x16x64_i8 (keys as the row operand), after which
+// lane (r, g) = (lane & 15, lane >> 4) holds, for block j, the scores of query row r and keys 16j + 4g .. +3.
+// A score row is therefore spread over four lanes, each holding whole chunks of four consecutive keys, which is
+// what the reference summation order is made of: chunk c belongs to partial sum c % 64, partial sums meet in a
+// xor butterfly 32, 16, 8, 4, 2, 1.  Chunk c = 4j + g, so partial sum index = 4 (j % 16) + g: levels 32..4 of
+// the butterfly combine values of one lane (j ^ 8, j ^ 4, j ^ 2, j ^ 1), levels 2 and 1 are the lane exchanges
+// lane ^ 32 and lane ^ 16.
+#include "ti_common.h"
+#include "softmax_math.h"
+
+namespace ti {
+
+#define TI_GLOBAL_AS __attribute__((address_space(1)))
+#define TI_LDS_AS __attribute__((address_space(3)))
+
+constexpr int AF_ROWS = 64;   // query rows per workgroup
+constexpr int AF_D = 128;     // head size
+constexpr int AF_MAX_S = 512;
+
+// NB = key blocks of 16 the registers are sized for (S <= 16 * NB).
+template <int NB>
+__global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t* __restrict__ q,
+                                                                   const int8_t* __restrict__ k,
+                                                                   const float* __restrict__ mask,
+                                                                   int8_t* __restrict__ probs, int T, int S,
+                                                                   long long stride_q, long long stride_k, int heads,
+                                                                   int row_blocks, float alpha) {
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const long long bh = blockIdx.x / row_blocks;
+  const int t0 = (blockIdx.x % row_blocks) * AF_ROWS;
+  const int nb = S >> 4;
+
+  // ---- copies: slab i = 8 rows of [Q tile (64 rows) | K panel (S rows)], 1 KiB per wave instruction
+  const int8_t* qb = q + bh * stride_q;
+  const int8_t* kb = k + bh * stride_k;
+  const int slabs = (AF_ROWS + S) >> 3;
+  for (int i = wave; i < slabs; i += 4) {
+    const int row = i * 8 + (lane >> 3);  // row of the stacked panels
+    const int pos = lane & 7;
+    const int8_t* src;
+    if (row < AF_ROWS) {
+      const int t = t0 + row < T ? t0 + row : T - 1;  // rows past the end repeat the last one; never stored
+      src = qb + (long long)t * AF_D + ((pos ^ ((row >> 1) & 7)) << 4);
+    } else {
+      const int kr = row - AF_ROWS;
+      src = kb + (long long)kr * AF_D + ((pos ^ ((kr >> 1) & 7)) << 4);
+    }
+    __builtin_amdgcn_global_load_lds((const TI_GLOBAL_AS void*)src, (TI_LDS_AS void*)((TI_LDS_AS char*)smem + i * 1024),
+                                     16, 0, 0);
+  }
+  asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+
+  // ---- scores: acc[j] = q rows (16 of this wave) x key block j
+  const int r = lane & 15, g = lane >> 4;
+  const int sw = (r >> 1) & 7;
+  const char* qs = smem + (wave * 16 + r) * AF_D;
+  const char* ks = smem + AF_ROWS * AF_D + r * AF_D;
+  v4i qf[2];
+#pragma unroll
+  for (int s = 0; s < 2; ++s) qf[s] = *reinterpret_cast<const v4i*>(qs + (((4 * s + g) ^ sw) << 4));
+  v4i acc[NB];
+#pragma unroll
+  for (int j = 0; j < NB; ++j) {
+    acc[j] = v4i{0, 0, 0, 0};
+    if (j < nb) {
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        const v4i kf = *reinterpret_cast<const v4i*>(ks + j * 16 * AF_D + (((4 * s + g) ^ sw) << 4));
+        acc[j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(kf, qf[s], acc[j], 0, 0, 0);
+      }
+    }
+  }
+
+  __syncthreads();  // all waves have read their fragments: the K panel may be overwritten (see the stores below)
+
+  // ---- x = max(alpha * acc + mask, lowest); row maximum.  The mask values of eight blocks are fetched
+  // while the previous eight are consumed.
+  const int t = t0 + wave * 16 + r;
+  const int tc = t < T ? t : T - 1;
+  const float* mrow = mask != nullptr ? mask + (((bh / heads) * T + tc) * (long long)S) : nullptr;
+  const float lowest = -3.402823466e+38f;
+  float m = lowest;
+  constexpr int MG = NB < 8 ? NB : 8;  // blocks per mask group
+  v4f mk[2][MG];
+  auto fetch_mask = [&](int j0, v4f (&dst)[MG]) {
+#pragma unroll
+    for (int u = 0; u < MG; ++u) {
+      const int j = j0 + u;
+      dst[u] = v4f{0.f, 0.f, 0.f, 0.f};
+      if (mrow != nullptr && j < nb) dst[u] = *reinterpret_cast<const v4f*>(mrow + 16 * j + 4 * g);
+    }
+  };
+  fetch_mask(0, mk[0]);
+#pragma unroll
+  for (int j0 = 0; j0 < NB; j0 += MG) {
+    const int cur = (j0 / MG) & 1;
+    if (j0 + MG < NB) fetch_mask(j0 + MG, mk[cur ^ 1]);
+#pragma unroll
+    for (int u = 0; u < MG; ++u) {
+      const int j = j0 + u;
+      if (j < nb) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          float x = Epi<EPI_F32_SCALE>::apply(acc[j][v], 0.0f, alpha);
+          if (mrow != nullptr) x = x + mk[cur][u][v];
+          x = x > lowest ? x : lowest;
+          m = m > x ? m : x;
+          acc[j][v] = __float_as_int(x);
+        }
+      }
+    }
+  }
+  {
+    float o = __shfl_xor(m, 16, 64);
+    m = m > o ? m : o;
+    o = __shfl_xor(m, 32, 64);
+    m = m > o ? m : o;
+  }
+
+  // ---- e = exp(x - m); partial sums in the reference order.  exp_nonpos returns exactly 0 below -87, so a
+  // block in which no lane of the wave has anything above that (masked-out keys) skips the evaluation.
+  unsigned live = 0;  // bit j: block j has non-zero probabilities somewhere in the wave
+  float part[16];
+#pragma unroll
+  for (int jj = 0; jj < 16; ++jj) {
+    float p = 0.0f;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int j = jj + 16 * h;
+      if (j < NB && j < nb) {
+        bool any = false;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) any = any || (__int_as_float(acc[j][v]) - m > -87.0f);
+        if (__builtin_amdgcn_ballot_w64(any) != 0) {
+          live |= 1u << j;
+#pragma unroll
+          for (int v = 0; v < 4; ++v) {
+            const float e = exp_nonpos(__int_as_float(acc[j][v]) - m);
+            acc[j][v] = __float_as_int(e);
+            p = p + e;
+          }
+        } else {
+          // every e is 0: p + 0 = p, nothing to add
+          acc[j] = v4i{0, 0, 0, 0};
+        }
+      }
+    }
+    part[jj] = p;
+  }
+#pragma unroll
+  for (int w = 8; w >= 1; w >>= 1)
+#pragma unroll
+    for (int jj = 0; jj < w; ++jj) part[jj] = part[jj] + part[jj + w];
+  float sum = part[0];
+  sum = sum + __shfl_xor(sum, 32, 64);
+  sum = sum + __shfl_xor(sum, 16, 64);
+  const float scale = 127.0f / sum;
+
+  // ---- probabilities: four consecutive keys per lane and block = one dword, staged through the part of the
+  // K panel this wave may reuse (every wave is past the barrier above, so nobody reads the panel any more) and
+  // written out as whole rows, 16 bytes per lane.  Row pitch S + 16 keeps the dword writes off each other's banks.
+  const int pitch = S + 16;
+  char* stage = smem + AF_ROWS * AF_D + wave * 16 * pitch;
+#pragma unroll
+  for (int j = 0; j < NB; ++j) {
+    if (j < nb) {
+      unsigned w = 0;
+      if (live >> j & 1) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const float pq = __builtin_rintf(__int_as_float(acc[j][v]) * scale);  // in [0, 127]
+          w |= (unsigned)(int)pq << (8 * v);
+        }
+      }
+      *reinterpret_cast<unsigned*>(stage + r * pitch + 16 * j + 4 * g) = w;
+    }
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the wave's own LDS writes are done; its reads below follow
+  const int cpr = S >> 4;                              // 16-byte chunks per row
+  int8_t* pbase = probs + (bh * T + t0 + wave * 16) * (long long)S;
+  for (int idx = lane; idx < 16 * cpr; idx += 64) {
+    const int row = idx / cpr, c16 = idx - row * cpr;
+    if (t0 + wave * 16 + row < T)
+      *reinterpret_cast<v4i*>(pbase + (long long)row * S + c16 * 16) =
+          *reinterpret_cast<const v4i*>(stage + row * pitch + c16 * 16);
+  }
+}
+
+bool attn_qk_softmax_q_supported(long long T, long long S, long long D) {
+  return T >= 1 && D == AF_D && S >= 16 && S <= AF_MAX_S && S % 16 == 0;
+}
+
+template <int NB>
+static int launch_af(dim3 grid, size_t lds, hipStream_t stream, const int8_t* q, const int8_t* k, const float* mask,
+                     int8_t* probs, int T, int S, long long stride_q, long long stride_k, int heads, int row_blocks,
+                     float alpha) {
+  auto kern = attn_qk_softmax_q_kernel<NB>;
+  static unsigned long long lds_ok = 0;  // bit per device: the large dynamic LDS size has been allowed
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return fail(TI_ERR_LAUNCH, "attn_qk_softmax_q: no current device");
+  if (dev < 64 && !(lds_ok >> dev & 1)) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (AF_ROWS + AF_MAX_S) * AF_D);
+    if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "attn_qk_softmax_q: LDS limit: %s", hipGetErrorString(e));
+    lds_ok |= 1ull << dev;
+  }
+  hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, q, k, mask, probs, T, S, stride_q, stride_k, heads, row_blocks,
+                     alpha);
+  return TI_OK;
+}
+
+int launch_attn_qk_softmax_q(const int8_t* q, const int8_t* k, const float* mask, int8_t* probs, long long BH,
+                             long long T, long long S, long long D, long long stride_q, long long stride_k,
+                             long long heads, float alpha, hipStream_t stream) {
+  if (BH == 0 || T == 0) return TI_OK;
+  if (!attn_qk_softmax_q_supported(T, S, D))
+    return fail(TI_ERR_INVALID_ARG, "attn_qk_softmax_q: unsupported shape (T=%lld S=%lld head_dim=%lld)", T, S, D);
+  const long long row_blocks = (T + AF_ROWS - 1) / AF_ROWS;
+  if (BH * row_blocks > 0x7fffffffLL || T > 0x7fffffffLL)
+    return fail(TI_ERR_INVALID_ARG, "attn_qk_softmax_q: too many row blocks (%lld)", BH * row_blocks);
+  const dim3 grid((unsigned)(BH * row_blocks));
+  const size_t lds = (size_t)(AF_ROWS + S) * AF_D;
+  int rc;
+  if (S <= 128)
+    rc = launch_af<8>(grid, lds, stream, q, k, mask, probs, (int)T, (int)S, stride_q, stride_k, (int)heads,
+                      (int)row_blocks, alpha);
+  else if (S <= 256)
+    rc = launch_af<16>(grid, lds, stream, q, k, mask, probs, (int)T, (int)S, stride_q, stride_k, (int)heads,
+                       (int)row_blocks, alpha);
+  else
+    rc = launch_af<32>(grid, lds, stream, q, k, mask, probs, (int)T, (int)S, stride_q, stride_k, (int)heads,
+                       (int)row_blocks, alpha);
+  if (rc) return rc;
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "attn_qk_softmax_q launch: %s", hipGetErrorString(e));
+  return TI_OK;
+}
+
+}  // namespace ti

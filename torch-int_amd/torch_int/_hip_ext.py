@@ -35,6 +35,10 @@ _lib.ti_bmm_s8t_s8n_f32t_strided.argtypes = [_vp, _vp, _vp, _i64, _i64, _i64, _i
 _lib.ti_bmm_s8t_s8n_f32t_strided.restype = ctypes.c_int
 _lib.ti_kv_append_s8.argtypes = [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp]
 _lib.ti_kv_append_s8.restype = ctypes.c_int
+_lib.ti_attn_qk_softmax_q_supported.argtypes = [_i64, _i64, _i64]
+_lib.ti_attn_qk_softmax_q_supported.restype = ctypes.c_int
+_lib.ti_attn_qk_softmax_q.argtypes = [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _vp]
+_lib.ti_attn_qk_softmax_q.restype = ctypes.c_int
 _lib.ti_decode_attn_supported.argtypes = [_i64, _i64, _i64]
 _lib.ti_decode_attn_supported.restype = ctypes.c_int
 _lib.ti_decode_attn_s8.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32,
@@ -273,6 +277,42 @@ def kv_append(k_new, v_new, k_buf, v_buf, filled, checked=False):
                                       d, cap, filled, stream or None)
     if rc:
         raise RuntimeError(f"torch_int._hip_ext.kv_append: {_lib.ti_last_error().decode()} (status {rc})")
+
+
+def can_attn_qk_softmax_q(q, k, mask, bsz, heads):
+    """int8 HIP q [bsz*heads, T, 128] contiguous and k [bsz*heads, S, 128] with packed rows (any batch stride that is
+    a multiple of 16), S a multiple of 16 up to 512; mask None or fp32 [bsz, 1, T, S] contiguous."""
+    if not (_ok(q, torch.int8) and type(k) is torch.Tensor and k.dtype is torch.int8 and k.is_cuda and q.dim() == 3
+            and k.dim() == 3 and q.shape[0] == k.shape[0] == bsz * heads and q.shape[2] == k.shape[2]
+            and k.device == q.device and q.numel() > 0):
+        return False
+    T, S, d = q.shape[1], k.shape[1], q.shape[2]
+    if not _lib.ti_attn_qk_softmax_q_supported(T, S, d):
+        return False
+    if k.stride(2) != 1 or k.stride(1) != d or k.stride(0) < S * d or k.stride(0) % 16 or q.data_ptr() % 16 or \
+            k.data_ptr() % 16:
+        return False
+    return mask is None or (_ok(mask, torch.float32) and mask.shape == (bsz, 1, T, S) and mask.device == q.device
+                            and mask.data_ptr() % 16 == 0)
+
+
+def attn_qk_softmax_q(q, k, mask, alpha, heads, checked=False):
+    """int8 round(127 softmax(alpha q k^T + mask)) [bsz*heads, T, S] in one launch: the values of
+    ``attn_softmax_q(bmm_s8t_s8n_f32t(q, k, alpha), mask, heads)`` without the fp32 scores in memory."""
+    if not checked and not can_attn_qk_softmax_q(q, k, mask, q.shape[0] // heads, heads):
+        raise RuntimeError("torch_int._hip_ext.attn_qk_softmax_q: needs int8 HIP q [B*H,T,128] / k [B*H,S,128] (S a "
+                           "multiple of 16 up to 512) and an fp32 mask [B,1,T,S] or None")
+    BH, T, d = q.shape
+    S = k.shape[1]
+    dev = q.device
+    probs = torch.empty((BH, T, S), dtype=torch.int8, device=dev)
+    with _on(dev):
+        rc = _lib.ti_attn_qk_softmax_q(q.data_ptr(), k.data_ptr(), mask.data_ptr() if mask is not None else None,
+                                       probs.data_ptr(), BH, T, S, d, T * d, k.stride(0), heads, alpha,
+                                       _raw_stream(dev.index) or None)
+    if rc:
+        raise RuntimeError(f"torch_int._hip_ext.attn_qk_softmax_q: {_lib.ti_last_error().decode()} (status {rc})")
+    return probs
 
 
 def decode_attention_shape_ok(T, S, d):

@@ -250,12 +250,18 @@ class Int8OPTAttention(nn.Module):
         value = value.view(bsz * H, -1, d) if value.is_contiguous() else value.reshape(bsz * H, value.shape[2], d)
         src_len = key.size(1)
 
-        if (not key.is_contiguous() and type(self.qk_bmm) is BMM_S8T_S8N_F32T
+        probs_q = None
+        if (layer_head_mask is None and tgt_len > 16 and type(self.qk_bmm) is BMM_S8T_S8N_F32T
+                and _hip_ext.can_attn_qk_softmax_q(query, key, attention_mask, bsz, H)):
+            # Q.K^T, mask, clamp, softmax, *127, round and int8 cast in one kernel: the fp32 scores stay in registers
+            probs_q = _hip_ext.attn_qk_softmax_q(query, key, attention_mask, self.qk_bmm._scalar("a"), H, checked=True)
+            probs_out = probs_q.view(bsz, H, tgt_len, src_len).float() if output_attentions else None
+        elif (not key.is_contiguous() and type(self.qk_bmm) is BMM_S8T_S8N_F32T
                 and _hip_ext.can_bmm_strided(query, key)):
             scores = _hip_ext.bmm_s8t_s8n_f32t_strided(query, key, self.qk_bmm._scalar("a"), checked=True)
         else:
             scores = self.qk_bmm(query, key.contiguous())  # fp32 [bsz*H, tgt, src]
-        if scores.size() != (bsz * H, tgt_len, src_len):
+        if probs_q is None and scores.size() != (bsz * H, tgt_len, src_len):
             raise ValueError(f"Attention weights should be of size {(bsz * H, tgt_len, src_len)}, but is"
                              f" {scores.size()}")
         if attention_mask is not None and attention_mask.size() != (bsz, 1, tgt_len, src_len):
@@ -264,7 +270,9 @@ class Int8OPTAttention(nn.Module):
         if layer_head_mask is not None and layer_head_mask.size() != (H,):
             raise ValueError(f"Head mask for a single layer should be of size {(H,)}, but is"
                              f" {layer_head_mask.size()}")
-        if layer_head_mask is None and _hip_ext.can_fuse_softmax(scores, attention_mask, bsz, H):
+        if probs_q is not None:
+            pass
+        elif layer_head_mask is None and _hip_ext.can_fuse_softmax(scores, attention_mask, bsz, H):
             # mask add, clamp, softmax, *127, round and int8 cast in one kernel
             probs_q = _hip_ext.attn_softmax_q(scores, attention_mask, H, checked=True)
             probs_out = probs_q.view(bsz, H, tgt_len, src_len).float() if output_attentions else None
