@@ -113,8 +113,8 @@ __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t*
         for (int v = 0; v < 4; ++v) {
           float x = Epi<EPI_F32_SCALE>::apply(acc[j][v], 0.0f, alpha);
           if (mrow != nullptr) x = x + mk[cur][u][v];
-          x = x > lowest ? x : lowest;
-          m = m > x ? m : x;
+          x = __builtin_fmaxf(x, lowest);  // = x > lowest ? x : lowest, NaN included
+          m = __builtin_fmaxf(m, x);
           acc[j][v] = __float_as_int(x);
         }
       }
@@ -138,10 +138,9 @@ __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t*
     for (int h = 0; h < 2; ++h) {
       const int j = jj + 16 * h;
       if (j < NB && j < nb) {
-        bool any = false;
-#pragma unroll
-        for (int v = 0; v < 4; ++v) any = any || (__int_as_float(acc[j][v]) - m > -87.0f);
-        if (__builtin_amdgcn_ballot_w64(any) != 0) {
+        const float top = __builtin_fmaxf(__builtin_fmaxf(__int_as_float(acc[j][0]), __int_as_float(acc[j][1])),
+                                          __builtin_fmaxf(__int_as_float(acc[j][2]), __int_as_float(acc[j][3])));
+        if (__builtin_amdgcn_ballot_w64(top - m > -87.0f) != 0) {
           live |= 1u << j;
 #pragma unroll
           for (int v = 0; v < 4; ++v) {
