@@ -178,6 +178,24 @@ static PyObject* fc_kv_append(PyObject* self, PyObject* const* a, Py_ssize_t n) 
   return PyLong_FromLong(ti_kv_append_s8(kn, vn, kb, vb, BH, T, D, cap, S, st));
 }
 
+/* decode_attn(q, k_new, v_new, k_buf, v_buf, mask, ctx, probs, BH, T, D, cap, S, heads, alpha_qk, alpha_pv, stream) -> status */
+static PyObject* fc_decode_attn(PyObject* self, PyObject* const* a, Py_ssize_t n) {
+  (void)self;
+  if (n != 17) {
+    PyErr_SetString(PyExc_TypeError, "decode_attn expects 17 arguments");
+    return NULL;
+  }
+  void *q = as_ptr(a[0]), *kn = as_ptr(a[1]), *vn = as_ptr(a[2]), *kb = as_ptr(a[3]), *vb = as_ptr(a[4]);
+  void *mask = as_ptr(a[5]), *ctx = as_ptr(a[6]), *probs = as_ptr(a[7]);
+  int64_t BH = as_i64(a[8]), T = as_i64(a[9]), D = as_i64(a[10]), cap = as_i64(a[11]), S = as_i64(a[12]);
+  int64_t heads = as_i64(a[13]);
+  double aqk = PyFloat_AsDouble(a[14]), apv = PyFloat_AsDouble(a[15]);
+  void* st = as_ptr(a[16]);
+  if (PyErr_Occurred()) return NULL;
+  return PyLong_FromLong(ti_decode_attn_s8(q, kn, vn, kb, vb, mask, ctx, probs, BH, T, D, cap, S, heads, (float)aqk,
+                                           (float)apv, st));
+}
+
 static PyObject* fc_last_error(PyObject* self, PyObject* noargs) {
   (void)self;
   (void)noargs;
@@ -194,6 +212,7 @@ static PyMethodDef methods[] = {
     {"bmm_rowmajor", (PyCFunction)(void (*)(void))fc_bmm_rowmajor, METH_FASTCALL, "forward to ti_bmm_s8t_s8t_s8t"},
     {"linear_group3", (PyCFunction)(void (*)(void))fc_linear_group3, METH_FASTCALL, "forward to ti_linear_a8_w8_b8_o8_group"},
     {"kv_append", (PyCFunction)(void (*)(void))fc_kv_append, METH_FASTCALL, "forward to ti_kv_append_s8"},
+    {"decode_attn", (PyCFunction)(void (*)(void))fc_decode_attn, METH_FASTCALL, "forward to ti_decode_attn_s8"},
     {"last_error", fc_last_error, METH_NOARGS, "ti_last_error()"},
     {NULL, NULL, 0, NULL}};
 

@@ -52,6 +52,7 @@ _lib.ti_linear_a8_w8_b8_o8_group.argtypes = [_vp, _pp, _pp, _pp, ctypes.POINTER(
 _lib.ti_linear_a8_w8_b8_o8_group.restype = ctypes.c_int
 _raw_stream = torch._C._cuda_getCurrentRawStream
 _fast = _CUDA._fast if getattr(_CUDA._fast, "kv_append", None) is not None else None
+_fast_decode_attn = getattr(_CUDA._fast, "decode_attn", None)
 _fast_group3 = getattr(_CUDA._fast, "linear_group3", None)
 _fast_add_ln_q = getattr(_CUDA._fast, "add_ln_q", None)
 _fast_softmax_q = getattr(_CUDA._fast, "softmax_q", None)
@@ -351,10 +352,17 @@ def decode_attention(q, k_new, v_new, k_buf, v_buf, filled, mask, alpha_qk, alph
     ctx = torch.empty((B * H, T, d), dtype=torch.int8, device=dev)
     probs = torch.empty((B * H, T, S), dtype=torch.int8, device=dev) if want_probs else None
     with _on(dev):
-        rc = _lib.ti_decode_attn_s8(q.data_ptr(), k_new.data_ptr(), v_new.data_ptr(), k_buf.data_ptr(), v_buf.data_ptr(),
-                                    mask.data_ptr() if mask is not None else None, ctx.data_ptr(),
-                                    probs.data_ptr() if probs is not None else None, B * H, T, d, k_buf.shape[2], S, H,
-                                    alpha_qk, alpha_pv, _raw_stream(dev.index) or None)
+        stream = _raw_stream(dev.index)
+        if _fast_decode_attn is not None:
+            rc = _fast_decode_attn(q.data_ptr(), k_new.data_ptr(), v_new.data_ptr(), k_buf.data_ptr(), v_buf.data_ptr(),
+                                   mask.data_ptr() if mask is not None else 0, ctx.data_ptr(),
+                                   probs.data_ptr() if probs is not None else 0, B * H, T, d, k_buf.shape[2], S, H,
+                                   alpha_qk, alpha_pv, stream)
+        else:
+            rc = _lib.ti_decode_attn_s8(q.data_ptr(), k_new.data_ptr(), v_new.data_ptr(), k_buf.data_ptr(),
+                                        v_buf.data_ptr(), mask.data_ptr() if mask is not None else None, ctx.data_ptr(),
+                                        probs.data_ptr() if probs is not None else None, B * H, T, d, k_buf.shape[2],
+                                        S, H, alpha_qk, alpha_pv, stream or None)
     if rc:
         raise RuntimeError(f"torch_int._hip_ext.decode_attention: {_lib.ti_last_error().decode()} (status {rc})")
     return ctx, probs
