@@ -192,6 +192,16 @@ int ti_transpose_last2_s8(const int8_t* src, int8_t* dst, int64_t B, int64_t R, 
 int ti_kv_append_s8(const int8_t* k_new, const int8_t* v_new, int8_t* k_buf, int8_t* v_buf, int64_t BH, int64_t T,
                     int64_t D, int64_t cap, int64_t S, void* stream);
 
+/* The attention of a prefill step in one launch (torch_int/models/opt.py:137-196): ctx[b, t, h*D:(h+1)*D] =
+ * s8(alpha_pv * sum_s p[t, s] * v[s, :]) with p the int8 probabilities of ti_attn_qk_softmax_q, i.e. the chain
+ * ti_bmm_s8t_s8n_f32t, ti_attn_softmax_q, ti_bmm_s8t_s8n_s8t and the head merge `transpose(1,2).reshape(...)`,
+ * same bits, without the score and probability tensors.  vt is V transposed, [BH, D, S] packed (what
+ * ti_transpose_last2_s8 makes, as upstream's `value_states.transpose(1,2).contiguous()`); ctx is [BH/heads, T,
+ * heads*D] packed.  Limits: D = 128, S a multiple of 64 in [64, 512]. */
+int ti_attn_prefill_s8(const int8_t* q, const int8_t* k, const int8_t* vt, const float* mask, int8_t* ctx, int64_t BH,
+                       int64_t T, int64_t S, int64_t D, int64_t stride_q, int64_t stride_k, int64_t heads,
+                       float alpha_qk, float alpha_pv, void* stream);
+
 /* One launch for the attention of an incremental decoding step (torch_int/models/opt.py:128-190 with T new
  * tokens and a KV cache): appends k_new / v_new ([BH, T, D] packed) at positions S-T .. S-1 of the cache buffers
  * ([BH, cap, D], S positions after the append; pass NULL for both to attend over a cache that already holds

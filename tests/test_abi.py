@@ -103,6 +103,12 @@ def test_c_abi_rejects_bad_arguments_without_a_device():
     rc = lib.ti_attn_qk_softmax_q(p, p + 8, None, p, 4, 64, 64, 128, 64 * 128, 64 * 128, 2, 1.0, None)
     assert rc == 2 and b"aligned" in lib.ti_last_error()
     assert lib.ti_attn_qk_softmax_q(None, None, None, None, 0, 64, 64, 128, 0, 0, 2, 1.0, None) == 0
+    lib.ti_attn_prefill_s8.argtypes = [ctypes.c_void_p] * 5 + [i64] * 7 + [ctypes.c_float] * 2 + [ctypes.c_void_p]
+    rc = lib.ti_attn_prefill_s8(p, p, p, None, p, 4, 64, 80, 128, 64 * 128, 80 * 128, 2, 1.0, 1.0, None)
+    assert rc == 1 and b"multiple of 64" in lib.ti_last_error()
+    rc = lib.ti_attn_prefill_s8(p, p, None, None, p, 4, 64, 64, 128, 64 * 128, 64 * 128, 2, 1.0, 1.0, None)
+    assert rc == 1 and b"vt is NULL" in lib.ti_last_error()
+    assert lib.ti_attn_prefill_s8(None, None, None, None, None, 0, 64, 64, 128, 0, 0, 2, 1.0, 1.0, None) == 0
     # empty problems succeed without touching pointers or a device
     assert lib.ti_linear_a8_w8_b8_o8(None, None, None, None, 0, 16, 16, 1.0, 1.0, None, 0, None) == 0
     assert lib.ti_dq_add_layernorm_q(None, 1.0, None, None, None, 1e-5, None, None, 0, 128, None) == 0

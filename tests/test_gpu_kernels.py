@@ -637,6 +637,33 @@ def test_fused_qk_softmax_matches_the_two_kernels_and_the_oracle():
     assert not X.can_attn_qk_softmax_q(qd[:, :, :64].contiguous(), kd[:, :, :64].contiguous(), None, B, H)
 
 
+def test_fused_prefill_attention_matches_the_chain():
+    # Q.K^T + softmax-quant + P.V + head merge in one launch against the oracle's chain of the separate operators
+    import torch_int._hip_ext as X
+    g = torch.Generator().manual_seed(97)
+    neg = torch.finfo(torch.float32).min
+    for (B, H, T, S, kind) in [(4, 40, 512, 512, "causal"), (2, 3, 100, 128, "pad"), (1, 4, 64, 64, None),
+                               (2, 2, 70, 256, "causal"), (1, 2, 300, 320, "causal"), (1, 1, 5, 448, None)]:
+        _say(f"attn_prefill B={B} H={H} T={T} S={S} mask={kind}")
+        q, k, v = _s8(g, B * H, T, 128), _s8(g, B * H, S, 128), _s8(g, B * H, S, 128)
+        a_qk, a_pv = _scal(g, 2e-4, 2e-3), _scal(g, 2e-3, 2e-2)
+        mask = None
+        if kind is not None:
+            mask = torch.zeros(B, 1, T, S)
+            if kind == "causal":
+                mask += torch.zeros(T, S).masked_fill(torch.arange(S)[None, :] > torch.arange(T)[:, None] + (S - T), neg)
+            mask[0, :, :, :5] = neg
+        probs = orc.attn_softmax_q(orc.bmm_s8t_s8n_f32t(q, k, a_qk), mask, H)
+        ref = orc.bmm_s8t_s8t_s8t(probs, v, a_pv).view(B, H, T, 128).transpose(1, 2).reshape(B, T, H * 128)
+        qd, kd, md = q.to(DEV), k.to(DEV), (mask.to(DEV) if mask is not None else None)
+        vt = X.transpose_last2(v.to(DEV))
+        assert X.can_attn_prefill(qd, kd, vt, md, B, H)
+        out = X.attn_prefill(qd, kd, vt, md, a_qk, a_pv, H)
+        assert out.shape == (B, T, H * 128) and out.dtype == torch.int8
+        assert torch.equal(out.cpu(), ref), (B, H, T, S, kind, (out.cpu() != ref).sum().item())
+    assert not X.can_attn_prefill(qd, kd[:, :432], vt[:, :, :432].contiguous(), None, B, H)   # S % 64 != 0
+
+
 def test_runs_are_deterministic():
     # identical bytes on repeated launches (an LDS race would show up here)
     import torch_int._CUDA as C

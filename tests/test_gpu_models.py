@@ -128,19 +128,22 @@ def test_decoder_layer_opt13b_shape():
     rec, handles = _capture(gl)
     # at this shape Q.K^T and the softmax run as one kernel (the qk_bmm module is bypassed): record its operands
     import torch_int._hip_ext as X
-    fused = X.attn_qk_softmax_q
+    fused = X.attn_prefill
 
-    def spy(q, k, m, alpha, heads, checked=False):
-        p = fused(q, k, m, alpha, heads, checked=checked)
-        rec["qk"] = ((q.detach().clone(), k.detach().clone()), p.detach().clone(), alpha)
-        return p
-    X.attn_qk_softmax_q = spy
+    def spy(q, k, vt, m, a_qk, a_pv, heads, checked=False):
+        # the same operands through the two-stage form (probabilities, then P.V): what the checks below look at
+        c = fused(q, k, vt, m, a_qk, a_pv, heads, checked=checked)
+        p = X.attn_qk_softmax_q(q, k, m, a_qk, heads)
+        rec["qk"] = ((q.detach().clone(), k.detach().clone()), p, a_qk)
+        rec["pv"] = ((p, vt.detach().clone()), c.detach().clone())
+        return c
+    X.attn_prefill = spy
     _say("decoder layer OPT-13B shape: GPU forward")
     h_gpu = hidden.to(DEV)
     try:
         out = gl(h_gpu, attention_mask=mask.to(DEV), use_cache=True)
     finally:
-        X.attn_qk_softmax_q = fused
+        X.attn_prefill = fused
     assert out[0] is h_gpu and out[0].shape == (B, T, D) and torch.isfinite(out[0]).all()
     for h in handles:
         h.remove()
@@ -186,8 +189,9 @@ def test_decoder_layer_opt13b_shape():
         assert torch.equal(p_out[hd:hd + 1].cpu(), ref_p), hd
     (p_in, v_in), c_out = rec["pv"]
     assert torch.equal(p_in, p_out)
-    assert c_out.shape == (B * H, T, D // H) and int(p_in.min()) >= 0
-    assert torch.equal(c_out[heads].cpu(), orc.bmm_s8t_s8n_s8t(p_in[heads].cpu(), v_in[heads].cpu(), a.pv_bmm.a.item()))
+    assert c_out.shape == (B, T, D) and int(p_in.min()) >= 0   # the fused kernel's context, heads already merged
+    c_heads = c_out.view(B, T, H, D // H).permute(0, 2, 1, 3).reshape(B * H, T, D // H)
+    assert torch.equal(c_heads[heads].cpu(), orc.bmm_s8t_s8n_s8t(p_in[heads].cpu(), v_in[heads].cpu(), a.pv_bmm.a.item()))
     # fp32 library pieces: LayerNormQ (int8 within one LSB) and softmax -> int8 probabilities
     _say("  check layer norms and softmax")
     for name, ln in (("ln1", layer.self_attn_layer_norm), ("ln2", layer.final_layer_norm)):

@@ -38,7 +38,7 @@ LINEAR = {
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--op", required=True, choices=list(LINEAR) + ["bmm_f32t", "bmm_s8t", "bmm_s32t", "bmm_s8t_rowmajor", "ln_q", "add_ln_q",
-                                               "softmax_q", "qk_softmax_q", "decode_attn", "copy"])
+                                               "softmax_q", "qk_softmax_q", "attn_prefill", "decode_attn", "copy"])
     ap.add_argument("--shape", type=int, nargs="+", required=True)
     ap.add_argument("--iters", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
@@ -110,6 +110,16 @@ def main():
         fn = lambda: X.attn_qk_softmax_q(q, k, mask, args.alpha, heads)  # noqa: E731
         ops = 2.0 * batch * heads * T * S * 128
         nbytes = batch * heads * (T * 128 + S * 128 + T * S) + 4.0 * batch * T * S
+    elif args.op == "attn_prefill":
+        # Q.K^T + softmax-quant + P.V + head merge in one launch: batch, heads, query rows, key rows (head size 128)
+        batch, heads, T, S = args.shape
+        q, k, vt = s8(batch * heads, T, 128), s8(batch * heads, S, 128), s8(batch * heads, 128, S)
+        mask = torch.zeros(T, S, device=dev).masked_fill(
+            torch.triu(torch.ones(T, S, dtype=torch.bool, device=dev), 1 + S - T), torch.finfo(torch.float32).min)
+        mask = mask[None, None].expand(batch, 1, T, S).contiguous()
+        fn = lambda: X.attn_prefill(q, k, vt, mask, args.alpha, 0.004, heads)  # noqa: E731
+        ops = 4.0 * batch * heads * T * S * 128
+        nbytes = batch * heads * (2 * T * 128 + 2 * S * 128) + 4.0 * batch * T * S
     elif args.op == "decode_attn":
         # one decode step's attention: batch, heads, cached positions, head size, new tokens; --rotate cache copies
         batch, heads, filled, d, T = args.shape

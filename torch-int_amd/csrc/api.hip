@@ -347,8 +347,34 @@ int ti_attn_qk_softmax_q(const int8_t* q, const int8_t* k, const float* mask, in
   if (int rc = check_ptr(op, "k", k, 16, true)) return rc;
   if (int rc = check_ptr(op, "mask", mask, 16, mask != nullptr)) return rc;
   if (int rc = check_ptr(op, "probs", probs, 16, true)) return rc;
-  return launch_attn_qk_softmax_q(q, k, mask, probs, BH, T, S, D, stride_q, stride_k, heads, alpha,
-                                  static_cast<hipStream_t>(stream));
+  return launch_attn_qk_softmax_q(q, k, mask, probs, BH, T, S, D, stride_q, stride_k, heads, alpha, nullptr, nullptr,
+                                  0.0f, static_cast<hipStream_t>(stream));
+}
+
+int ti_attn_prefill_s8(const int8_t* q, const int8_t* k, const int8_t* vt, const float* mask, int8_t* ctx, int64_t BH,
+                       int64_t T, int64_t S, int64_t D, int64_t stride_q, int64_t stride_k, int64_t heads,
+                       float alpha_qk, float alpha_pv, void* stream) {
+  g_err[0] = 0;
+  const char* op = "attn_prefill_s8";
+  const int64_t lim = 0x7fffffffLL;
+  if (BH < 0 || T < 0 || S < 0 || D < 0 || heads < 1 || BH > lim || T > lim || heads > lim)
+    return fail(TI_ERR_INVALID_ARG, "%s: sizes must be in [0, 2^31) and heads >= 1", op);
+  if (BH % heads != 0) return fail(TI_ERR_INVALID_ARG, "%s: BH = %lld is not a multiple of heads = %lld", op,
+                                   (long long)BH, (long long)heads);
+  if (BH == 0 || T == 0) return TI_OK;
+  if (!attn_qk_softmax_q_supported(T, S, D) || S % 64 != 0)
+    return fail(TI_ERR_INVALID_ARG, "%s: unsupported shape T=%lld S=%lld head_dim=%lld (needs head_dim 128 and S a "
+                "multiple of 64 in [64, 512])", op, (long long)T, (long long)S, (long long)D);
+  if (stride_q < T * D || stride_k < S * D || stride_q % 16 != 0 || stride_k % 16 != 0)
+    return fail(TI_ERR_INVALID_ARG, "%s: batch strides (%lld, %lld) must be multiples of 16 and cover one matrix", op,
+                (long long)stride_q, (long long)stride_k);
+  if (int rc = check_ptr(op, "q", q, 16, true)) return rc;
+  if (int rc = check_ptr(op, "k", k, 16, true)) return rc;
+  if (int rc = check_ptr(op, "vt", vt, 16, true)) return rc;
+  if (int rc = check_ptr(op, "mask", mask, 16, mask != nullptr)) return rc;
+  if (int rc = check_ptr(op, "ctx", ctx, 4, true)) return rc;
+  return launch_attn_qk_softmax_q(q, k, mask, nullptr, BH, T, S, D, stride_q, stride_k, heads, alpha_qk, vt, ctx,
+                                  alpha_pv, static_cast<hipStream_t>(stream));
 }
 
 int ti_decode_attn_supported(int64_t T, int64_t S, int64_t D) { return decode_attn_supported(T, S, D) ? 1 : 0; }

@@ -26,13 +26,22 @@ constexpr int AF_D = 128;     // head size
 constexpr int AF_MAX_S = 512;
 
 // NB = key blocks of 16 the registers are sized for (S <= 16 * NB).
-template <int NB>
+// PV: instead of storing the probabilities, multiply them with V right away (S a multiple of 64): vt is V
+// transposed, [batch*heads, 128, S]; it is copied into the LDS the K panel occupied while the softmax runs
+// (row pitch S + 16 against bank conflicts).  The probabilities of a 64-key slice sit in a lane as four dwords
+// (keys 16i + 4g .. +3, i = 0..3); used as they are for the 16 operand bytes of lane (r, g), they fix a
+// permutation of the 64 keys inside the slice, and the V fragments are gathered with the same permutation (four
+// 4-byte reads), so the integer sum over the slice is the same.  The context rows are written already merged:
+// ctx is [batch, T, heads * 128].
+template <int NB, bool PV>
 __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t* __restrict__ q,
                                                                    const int8_t* __restrict__ k,
                                                                    const float* __restrict__ mask,
                                                                    int8_t* __restrict__ probs, int T, int S,
                                                                    long long stride_q, long long stride_k, int heads,
-                                                                   int row_blocks, float alpha) {
+                                                                   int row_blocks, float alpha,
+                                                                   const int8_t* __restrict__ vt,
+                                                                   int8_t* __restrict__ ctx, float alpha_pv) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -82,6 +91,20 @@ __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t*
   }
 
   __syncthreads();  // all waves have read their fragments: the K panel may be overwritten (see the stores below)
+  const int pitch = S + 16;
+  // V^T panel: 128 rows of pitch bytes, ending where the K panel ended (it starts inside the dead Q tile)
+  char* vts = smem + (AF_ROWS + S) * AF_D - AF_D * pitch;
+  if constexpr (PV) {
+    const int8_t* vb = vt + bh * (long long)AF_D * S;
+    const int instrs = (AF_D * pitch) >> 10;  // 1 KiB each
+    for (int i = wave; i < instrs; i += 4) {
+      const int o = i * 1024 + lane * 16;
+      int row = o / pitch, col = o - row * pitch;
+      col = col < S ? col : 0;  // the 16 pad bytes of a row receive a copy of its first chunk; never read
+      __builtin_amdgcn_global_load_lds((const TI_GLOBAL_AS void*)(vb + (long long)row * S + col),
+                                       (TI_LDS_AS void*)((TI_LDS_AS char*)vts + i * 1024), 16, 0, 0);
+    }
+  }
 
   // ---- x = max(alpha * acc + mask, lowest); row maximum.  The mask values of eight blocks are fetched
   // while the previous eight are consumed.
@@ -165,33 +188,68 @@ __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t*
   sum = sum + __shfl_xor(sum, 16, 64);
   const float scale = 127.0f / sum;
 
-  // ---- probabilities: four consecutive keys per lane and block = one dword, staged through the part of the
-  // K panel this wave may reuse (every wave is past the barrier above, so nobody reads the panel any more) and
-  // written out as whole rows, 16 bytes per lane.  Row pitch S + 16 keeps the dword writes off each other's banks.
-  const int pitch = S + 16;
-  char* stage = smem + AF_ROWS * AF_D + wave * 16 * pitch;
+  // ---- probabilities: four consecutive keys per lane and block = one dword
+  unsigned pw[NB];
 #pragma unroll
   for (int j = 0; j < NB; ++j) {
-    if (j < nb) {
-      unsigned w = 0;
-      if (live >> j & 1) {
+    unsigned w = 0;
+    if (j < nb && (live >> j & 1)) {
 #pragma unroll
-        for (int v = 0; v < 4; ++v) {
-          const float pq = __builtin_rintf(__int_as_float(acc[j][v]) * scale);  // in [0, 127]
-          w |= (unsigned)(int)pq << (8 * v);
+      for (int v = 0; v < 4; ++v) {
+        const float pq = __builtin_rintf(__int_as_float(acc[j][v]) * scale);  // in [0, 127]
+        w |= (unsigned)(int)pq << (8 * v);
+      }
+    }
+    pw[j] = w;
+  }
+  if constexpr (!PV) {
+    // staged through the part of the K panel this wave may reuse (every wave is past the barrier above, so
+    // nobody reads the panel any more) and written out as whole rows, 16 bytes per lane
+    char* stage = smem + AF_ROWS * AF_D + wave * 16 * pitch;
+#pragma unroll
+    for (int j = 0; j < NB; ++j)
+      if (j < nb) *reinterpret_cast<unsigned*>(stage + r * pitch + 16 * j + 4 * g) = pw[j];
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the wave's own LDS writes are done; its reads below follow
+    const int cpr = S >> 4;                              // 16-byte chunks per row
+    int8_t* pbase = probs + (bh * T + t0 + wave * 16) * (long long)S;
+    for (int idx = lane; idx < 16 * cpr; idx += 64) {
+      const int row = idx / cpr, c16 = idx - row * cpr;
+      if (t0 + wave * 16 + row < T)
+        *reinterpret_cast<v4i*>(pbase + (long long)row * S + c16 * 16) =
+            *reinterpret_cast<const v4i*>(stage + row * pitch + c16 * 16);
+    }
+  } else {
+    // ---- context = P . V: all V^T copies of the workgroup must have landed
+    asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+    v4i o[AF_D / 16];
+#pragma unroll
+    for (int c = 0; c < AF_D / 16; ++c) o[c] = v4i{0, 0, 0, 0};
+    const char* vrow = vts + r * pitch + 4 * g;  // V^T row (= head-dim index) r of block c is 16c + r
+#pragma unroll
+    for (int sl = 0; sl < NB / 4; ++sl) {
+      if (4 * sl < nb) {
+        const v4i pa = {(int)pw[4 * sl], (int)pw[4 * sl + 1], (int)pw[4 * sl + 2], (int)pw[4 * sl + 3]};
+#pragma unroll
+        for (int c = 0; c < AF_D / 16; ++c) {
+          const char* src = vrow + c * 16 * pitch + 64 * sl;
+          const v4i vf = {*reinterpret_cast<const int*>(src), *reinterpret_cast<const int*>(src + 16),
+                          *reinterpret_cast<const int*>(src + 32), *reinterpret_cast<const int*>(src + 48)};
+          o[c] = __builtin_amdgcn_mfma_i32_16x16x64_i8(vf, pa, o[c], 0, 0, 0);
         }
       }
-      *reinterpret_cast<unsigned*>(stage + r * pitch + 16 * j + 4 * g) = w;
     }
-  }
-  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the wave's own LDS writes are done; its reads below follow
-  const int cpr = S >> 4;                              // 16-byte chunks per row
-  int8_t* pbase = probs + (bh * T + t0 + wave * 16) * (long long)S;
-  for (int idx = lane; idx < 16 * cpr; idx += 64) {
-    const int row = idx / cpr, c16 = idx - row * cpr;
-    if (t0 + wave * 16 + row < T)
-      *reinterpret_cast<v4i*>(pbase + (long long)row * S + c16 * 16) =
-          *reinterpret_cast<const v4i*>(stage + row * pitch + c16 * 16);
+    if (t < T) {
+      const long long b = bh / heads, h = bh - b * heads;
+      int* crow = reinterpret_cast<int*>(ctx + ((b * T + t) * heads + h) * (long long)AF_D) + g;
+#pragma unroll
+      for (int c = 0; c < AF_D / 16; ++c) {
+        unsigned w = 0;
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+          w |= (unsigned)(unsigned char)Epi<EPI_S8_SCALE>::apply(o[c][v], 0.0f, alpha_pv) << (8 * v);
+        crow[4 * c] = (int)w;
+      }
+    }
   }
 }
 
@@ -199,11 +257,11 @@ bool attn_qk_softmax_q_supported(long long T, long long S, long long D) {
   return T >= 1 && D == AF_D && S >= 16 && S <= AF_MAX_S && S % 16 == 0;
 }
 
-template <int NB>
+template <int NB, bool PV>
 static int launch_af(dim3 grid, size_t lds, hipStream_t stream, const int8_t* q, const int8_t* k, const float* mask,
                      int8_t* probs, int T, int S, long long stride_q, long long stride_k, int heads, int row_blocks,
-                     float alpha) {
-  auto kern = attn_qk_softmax_q_kernel<NB>;
+                     float alpha, const int8_t* vt, int8_t* ctx, float alpha_pv) {
+  auto kern = attn_qk_softmax_q_kernel<NB, PV>;
   static unsigned long long lds_ok = 0;  // bit per device: the large dynamic LDS size has been allowed
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return fail(TI_ERR_LAUNCH, "attn_qk_softmax_q: no current device");
@@ -214,15 +272,17 @@ static int launch_af(dim3 grid, size_t lds, hipStream_t stream, const int8_t* q,
     lds_ok |= 1ull << dev;
   }
   hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, q, k, mask, probs, T, S, stride_q, stride_k, heads, row_blocks,
-                     alpha);
+                     alpha, vt, ctx, alpha_pv);
   return TI_OK;
 }
 
+// vt == nullptr: probabilities into probs.  Otherwise context into ctx ([batch, T, heads*128]); needs S % 64 == 0.
 int launch_attn_qk_softmax_q(const int8_t* q, const int8_t* k, const float* mask, int8_t* probs, long long BH,
                              long long T, long long S, long long D, long long stride_q, long long stride_k,
-                             long long heads, float alpha, hipStream_t stream) {
+                             long long heads, float alpha, const int8_t* vt, int8_t* ctx, float alpha_pv,
+                             hipStream_t stream) {
   if (BH == 0 || T == 0) return TI_OK;
-  if (!attn_qk_softmax_q_supported(T, S, D))
+  if (!attn_qk_softmax_q_supported(T, S, D) || (vt != nullptr && S % 64 != 0))
     return fail(TI_ERR_INVALID_ARG, "attn_qk_softmax_q: unsupported shape (T=%lld S=%lld head_dim=%lld)", T, S, D);
   const long long row_blocks = (T + AF_ROWS - 1) / AF_ROWS;
   if (BH * row_blocks > 0x7fffffffLL || T > 0x7fffffffLL)
@@ -230,15 +290,19 @@ int launch_attn_qk_softmax_q(const int8_t* q, const int8_t* k, const float* mask
   const dim3 grid((unsigned)(BH * row_blocks));
   const size_t lds = (size_t)(AF_ROWS + S) * AF_D;
   int rc;
-  if (S <= 128)
-    rc = launch_af<8>(grid, lds, stream, q, k, mask, probs, (int)T, (int)S, stride_q, stride_k, (int)heads,
-                      (int)row_blocks, alpha);
-  else if (S <= 256)
-    rc = launch_af<16>(grid, lds, stream, q, k, mask, probs, (int)T, (int)S, stride_q, stride_k, (int)heads,
-                       (int)row_blocks, alpha);
-  else
-    rc = launch_af<32>(grid, lds, stream, q, k, mask, probs, (int)T, (int)S, stride_q, stride_k, (int)heads,
-                       (int)row_blocks, alpha);
+#define TI_AF(NB, PV)                                                                                              \
+  rc = launch_af<NB, PV>(grid, lds, stream, q, k, mask, probs, (int)T, (int)S, stride_q, stride_k, (int)heads,    \
+                         (int)row_blocks, alpha, vt, ctx, alpha_pv)
+  if (vt == nullptr) {
+    if (S <= 128) TI_AF(8, false);
+    else if (S <= 256) TI_AF(16, false);
+    else TI_AF(32, false);
+  } else {
+    if (S <= 128) TI_AF(8, true);
+    else if (S <= 256) TI_AF(16, true);
+    else TI_AF(32, true);
+  }
+#undef TI_AF
   if (rc) return rc;
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "attn_qk_softmax_q launch: %s", hipGetErrorString(e));

@@ -223,7 +223,8 @@ int launch_transpose_last2_s8(const int8_t* src, int8_t* dst, long long B, long 
 bool attn_qk_softmax_q_supported(long long T, long long S, long long D);
 int launch_attn_qk_softmax_q(const int8_t* q, const int8_t* k, const float* mask, int8_t* probs, long long BH,
                              long long T, long long S, long long D, long long stride_q, long long stride_k,
-                             long long heads, float alpha, hipStream_t stream);
+                             long long heads, float alpha, const int8_t* vt, int8_t* ctx, float alpha_pv,
+                             hipStream_t stream);
 bool decode_attn_supported(long long T, long long S, long long D);
 int launch_decode_attn_s8(const int8_t* q, const int8_t* k_new, const int8_t* v_new, int8_t* k_buf, int8_t* v_buf,
                           const float* mask, int8_t* ctx, int8_t* probs_out, long long BH, long long T, long long D,

@@ -39,6 +39,8 @@ _lib.ti_attn_qk_softmax_q_supported.argtypes = [_i64, _i64, _i64]
 _lib.ti_attn_qk_softmax_q_supported.restype = ctypes.c_int
 _lib.ti_attn_qk_softmax_q.argtypes = [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _vp]
 _lib.ti_attn_qk_softmax_q.restype = ctypes.c_int
+_lib.ti_attn_prefill_s8.argtypes = [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _f32, _vp]
+_lib.ti_attn_prefill_s8.restype = ctypes.c_int
 _lib.ti_decode_attn_supported.argtypes = [_i64, _i64, _i64]
 _lib.ti_decode_attn_supported.restype = ctypes.c_int
 _lib.ti_decode_attn_s8.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32,
@@ -314,6 +316,32 @@ def attn_qk_softmax_q(q, k, mask, alpha, heads, checked=False):
     if rc:
         raise RuntimeError(f"torch_int._hip_ext.attn_qk_softmax_q: {_lib.ti_last_error().decode()} (status {rc})")
     return probs
+
+
+def can_attn_prefill(q, k, vt, mask, bsz, heads):
+    """``can_attn_qk_softmax_q`` plus: S a multiple of 64 and vt = V transposed, int8 [bsz*heads, 128, S] contiguous."""
+    return (can_attn_qk_softmax_q(q, k, mask, bsz, heads) and k.shape[1] % 64 == 0 and _ok(vt, torch.int8)
+            and vt.shape == (q.shape[0], q.shape[2], k.shape[1]) and vt.device == q.device and vt.data_ptr() % 16 == 0)
+
+
+def attn_prefill(q, k, vt, mask, alpha_qk, alpha_pv, heads, checked=False):
+    """Prefill attention in one launch: int8 context [bsz, T, heads*128] =
+    merge_heads(bmm_s8t_s8n_s8t(attn_qk_softmax_q(q, k, mask, alpha_qk), vt, alpha_pv)), the same bits, without the
+    score and probability tensors."""
+    if not checked and not can_attn_prefill(q, k, vt, mask, q.shape[0] // heads, heads):
+        raise RuntimeError("torch_int._hip_ext.attn_prefill: needs int8 HIP q [B*H,T,128], k [B*H,S,128], vt [B*H,128,S] "
+                           "(S a multiple of 64 up to 512) and an fp32 mask [B,1,T,S] or None")
+    BH, T, d = q.shape
+    S = k.shape[1]
+    dev = q.device
+    ctx = torch.empty((BH // heads, T, heads * d), dtype=torch.int8, device=dev)
+    with _on(dev):
+        rc = _lib.ti_attn_prefill_s8(q.data_ptr(), k.data_ptr(), vt.data_ptr(),
+                                     mask.data_ptr() if mask is not None else None, ctx.data_ptr(), BH, T, S, d, T * d,
+                                     k.stride(0), heads, alpha_qk, alpha_pv, _raw_stream(dev.index) or None)
+    if rc:
+        raise RuntimeError(f"torch_int._hip_ext.attn_prefill: {_lib.ti_last_error().decode()} (status {rc})")
+    return ctx
 
 
 def decode_attention_shape_ok(T, S, d):

@@ -250,6 +250,15 @@ class Int8OPTAttention(nn.Module):
         value = value.view(bsz * H, -1, d) if value.is_contiguous() else value.reshape(bsz * H, value.shape[2], d)
         src_len = key.size(1)
 
+        if (layer_head_mask is None and not output_attentions and tgt_len > 16 and src_len % 64 == 0
+                and type(self.qk_bmm) is BMM_S8T_S8N_F32T and type(self.pv_bmm) is BMM_S8T_S8N_S8T
+                and _hip_ext.can_attn_qk_softmax_q(query, key, attention_mask, bsz, H) and value.is_cuda):
+            # the whole attention (Q.K^T, softmax-quant, P.V, head merge) in one kernel on V transposed
+            vt = _hip_ext.transpose_last2(value.contiguous())
+            if _hip_ext.can_attn_prefill(query, key, vt, attention_mask, bsz, H):
+                ctx = _hip_ext.attn_prefill(query, key, vt, attention_mask, self.qk_bmm._scalar("a"),
+                                            self.pv_bmm._scalar("a"), H, checked=True)
+                return self.out_proj(ctx), None, present
         probs_q = None
         if (layer_head_mask is None and tgt_len > 16 and type(self.qk_bmm) is BMM_S8T_S8N_F32T
                 and _hip_ext.can_attn_qk_softmax_q(query, key, attention_mask, bsz, H)):
