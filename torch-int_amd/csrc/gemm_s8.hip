@@ -1730,42 +1730,49 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmParams p, const 
   }
 }
 
-// Number of K slices for an (M,N,K) linear on this chip (1 = do not split) and the tile edge
-// (128 or 256) of the raw-int32 GEMM that computes the slices.  A small cost model fitted to
-// measurements at OPT-13B/66B widths with cache-cold weights: a 256x256 workgroup takes about
-// 0.85 us per K step with a CU to itself; a 128x128 workgroup 0.35 us alone and 0.70 us when two
+// Number of K slices for an (M,N,K) linear on this chip (1 = do not split) and the tile of the
+// raw-int32 GEMM that computes the slices.  A small cost model fitted to measurements at OPT-13B/66B
+// widths with cache-cold weights, per 64-byte K step: a 256x256 workgroup takes about 0.85 us with a CU
+// to itself, 256x160 0.55 us, 256x288 0.92 us; a 128x128 workgroup 0.35 us alone and 0.70 us when two
 // share a CU; 8 us per round for pipeline fill and epilogue; the int32 partial tiles are written
-// once and read once (they mostly stay in the last-level cache), plus the second launch.
-static int choose_splits(long long M, long long N, long long K, int* tile_edge = nullptr) {
-  if (tile_edge) *tile_edge = 128;
+// once and read once (they mostly stay in the last-level cache), plus the second launch.  The
+// unsplit candidates are in the race too, so that a shape whose 256x160 or 256x288 tiles already fill
+// the chip is left to the ordinary dispatch.
+enum SplitTile { SPLIT_128 = 0, SPLIT_256 = 1, SPLIT_256x160 = 2, SPLIT_256x288 = 3 };
+static int choose_splits(long long M, long long N, long long K, int* tile_kind = nullptr) {
+  if (tile_kind) *tile_kind = SPLIT_128;
   if (M <= 16 || M > 1024 || K % PBK != 0 || K < 1024) return 1;
   const double cus = num_cus();
   const long long steps = K / PBK;
-  int best = 1, best_edge = 128;
+  int best = 1, best_kind = SPLIT_128;
   double best_t = 1e30;
-  for (int edge = 128; edge <= 256; edge += 128) {
-    const double tiles = (double)((M + edge - 1) / edge) * (double)((N + edge - 1) / edge);
+  for (int kind = SPLIT_128; kind <= SPLIT_256x288; ++kind) {
+    const int bm = kind == SPLIT_128 ? 128 : 256;
+    const int bn = kind == SPLIT_128 ? 128 : kind == SPLIT_256 ? 256 : kind == SPLIT_256x160 ? 160 : 288;
+    if (kind >= SPLIT_256x160 && N % bn != 0) continue;
+    const double tiles = (double)((M + bm - 1) / bm) * (double)((N + bn - 1) / bn);
     for (int s = 1; s <= 16; ++s) {
       if (steps % s != 0 || steps / s < 4) continue;
+      if (kind >= SPLIT_256x160 && (K / s) % QBK != 0) continue;  // these tiles step 128 bytes at a time
       const double wgs = tiles * s;
       double rounds, step_us;
-      if (edge == 256) {
-        rounds = (double)(long long)((wgs + cus - 1) / cus);
-        step_us = 0.85;
-      } else {
+      if (kind == SPLIT_128) {
         rounds = (double)(long long)((wgs + 2 * cus - 1) / (2 * cus));
         step_us = wgs <= cus ? 0.35 : 0.70;
+      } else {
+        rounds = (double)(long long)((wgs + cus - 1) / cus);
+        step_us = kind == SPLIT_256 ? 0.85 : kind == SPLIT_256x160 ? 0.55 : 0.92;
       }
       double t = rounds * ((double)(steps / s) * step_us + 8.0);
-      if (s > 1) t += (double)(s + 1) * M * N * 4.0 / 8.0e6 + 3.0;  // bytes / (8 TB/s) in us
+      if (s > 1) t += (double)(2 * s + 1) * M * N * 4.0 / 8.0e6 + 3.0;  // partials out and back in, at 8 TB/s, in us
       if (t < best_t * 0.97) {  // prefer fewer slices and the smaller tile unless the gain is clear
         best_t = t;
         best = s;
-        best_edge = edge;
+        best_kind = kind;
       }
     }
   }
-  if (tile_edge) *tile_edge = best_edge;
+  if (tile_kind) *tile_kind = best_kind;
   return best;
 }
 
@@ -1833,12 +1840,15 @@ static int launch_kind(const GemmParams& p, void* workspace, long long workspace
     return TI_OK;
   }
   if (p.batch == 1 && p.lda == p.K && p.ldb == p.K) {
-    int edge = 128;
-    const int splits = choose_splits(p.M, p.N, p.K, &edge);
+    int tile = SPLIT_128;
+    const int splits = choose_splits(p.M, p.N, p.K, &tile);
     const long long need = (long long)splits * p.M * p.N * 4;
     if (splits > 1 && workspace != nullptr && workspace_bytes >= need &&
         (reinterpret_cast<uintptr_t>(workspace) & 15) == 0) {
-      g_last_kernel = edge == 256 ? "splitk_256x256" : "splitk_128x128";
+      g_last_kernel = tile == SPLIT_128      ? "splitk_128x128"
+                      : tile == SPLIT_256    ? "splitk_256x256"
+                      : tile == SPLIT_256x160 ? "splitk_256x160"
+                                              : "splitk_256x288";
       GemmParams q = p;  // the K slices are the batches of one raw-int32 GEMM into the workspace
       q.K = p.K / splits;
       q.batch = splits;
@@ -1848,10 +1858,13 @@ static int launch_kind(const GemmParams& p, void* workspace, long long workspace
       q.C = workspace;
       q.bias = nullptr;
       q.out_T = q.out_d = 0;  // the partial products are plain [splits][M][N]; only the reduction permutes
-      if (int rc = edge != 256          ? launch_pipe<PipeCfg<128, 128, 2, 2, 4, EPI_S32_RAW, false>>(q, stream)
-                   : q.K % QBK == 0 ? launch_pipe2<Pipe2Cfg<256, 256, 2, 4, EPI_S32_RAW, false>>(q, stream)
-                                    : launch_pipe<PipeCfg<256, 256, 2, 4, 4, EPI_S32_RAW, false>>(q, stream))
-        return rc;
+      int rc;
+      if (tile == SPLIT_128) rc = launch_pipe<PipeCfg<128, 128, 2, 2, 4, EPI_S32_RAW, false>>(q, stream);
+      else if (tile == SPLIT_256x160) rc = launch_pipe16q<Pipe16QCfg<256, 160, 4, 2, EPI_S32_RAW>>(q, stream);
+      else if (tile == SPLIT_256x288) rc = launch_pipe16q<Pipe16QCfg<256, 288, 4, 2, EPI_S32_RAW>>(q, stream);
+      else if (q.K % QBK == 0) rc = launch_pipe2<Pipe2Cfg<256, 256, 2, 4, EPI_S32_RAW, false>>(q, stream);
+      else rc = launch_pipe<PipeCfg<256, 256, 2, 4, 4, EPI_S32_RAW, false>>(q, stream);
+      if (rc) return rc;
       const long long quads = ((long long)p.M * p.N + 3) / 4;
       hipLaunchKernelGGL(splitk_reduce_kernel<KIND>, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream, p,
                          static_cast<const int*>(workspace), splits);
