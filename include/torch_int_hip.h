@@ -98,11 +98,21 @@ int ti_linear_a8_w8_b8_o8_heads(const int8_t* x, const int8_t* w, const int8_t* 
  * s8(rint(clamp(alpha[i]*(x . w[i]^T) + beta[i]*bias[i]))).  w, bias, out, alpha, beta are HOST arrays of
  * `count` device pointers / scalars.  The q, k and v projections of one attention block
  * (torch_int/models/opt.py:108-126 calls them one after the other); for M <= 16 with K % 1024 == 0 all
- * weights are streamed by a single launch, other shapes run problem by problem.  Results are those of
+ * weights are streamed by a single launch, for M > 128 with N % 160 == 0 or N % 288 == 0 and K % 128 == 0 the
+ * problems are the batches of one persistent tiled launch, other shapes run problem by problem.  Results are those of
  * `count` separate calls. */
 int ti_linear_a8_w8_b8_o8_group(const int8_t* x, const int8_t* const* w, const int8_t* const* bias,
                                 int8_t* const* out, const float* alpha, const float* beta, int64_t count,
                                 int64_t M, int64_t N, int64_t K, void* stream);
+
+/* ti_linear_a8_w8_b8_o8_group with every output stored head-major as by ti_linear_a8_w8_b8_o8_heads: the
+ * q, k and v projections of a prefill (torch_int/models/opt.py:108-126 followed by the `_shape` permutations,
+ * :80-81) as one call.  When N is a multiple of 160 or 288, K of 128 and M > 128, the problems run as the
+ * batches of one persistent launch; other shapes run problem by problem.  Results are those of `count`
+ * separate calls. */
+int ti_linear_a8_w8_b8_o8_group_heads(const int8_t* x, const int8_t* const* w, const int8_t* const* bias,
+                                      int8_t* const* out, const float* alpha, const float* beta, int64_t count,
+                                      int64_t M, int64_t N, int64_t K, int64_t T, int64_t head_dim, void* stream);
 
 /* replaces linear_relu_a8_w8_b8_o8 (linear.cu:476-625; linear.h:28-33):
  * out = s8(rint(min(max(alpha*acc + beta*bias, 0), 127))). */

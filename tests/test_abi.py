@@ -109,6 +109,17 @@ def test_c_abi_rejects_bad_arguments_without_a_device():
     rc = lib.ti_attn_prefill_s8(p, p, None, None, p, 4, 64, 64, 128, 64 * 128, 64 * 128, 2, 1.0, 1.0, None)
     assert rc == 1 and b"vt is NULL" in lib.ti_last_error()
     assert lib.ti_attn_prefill_s8(None, None, None, None, None, 0, 64, 64, 128, 0, 0, 2, 1.0, 1.0, None) == 0
+    # grouped head-major linears: head split, group size, per-problem arrays
+    pp, fp = ctypes.POINTER(ctypes.c_void_p), ctypes.POINTER(ctypes.c_float)
+    lib.ti_linear_a8_w8_b8_o8_group_heads.argtypes = [ctypes.c_void_p, pp, pp, pp, fp, fp] + [i64] * 6 + [ctypes.c_void_p]
+    ptrs, scal = (ctypes.c_void_p * 3)(p, p, p), (ctypes.c_float * 3)(1.0, 1.0, 1.0)
+    rc = lib.ti_linear_a8_w8_b8_o8_group_heads(p, ptrs, ptrs, ptrs, scal, scal, 3, 8, 32, 16, 3, 16, None)
+    assert rc == 1 and b"multiple of T" in lib.ti_last_error()
+    rc = lib.ti_linear_a8_w8_b8_o8_group_heads(p, ptrs, ptrs, ptrs, scal, scal, 5, 8, 32, 16, 4, 16, None)
+    assert rc == 1 and b"0 to 4 problems" in lib.ti_last_error()
+    rc = lib.ti_linear_a8_w8_b8_o8_group_heads(p, None, ptrs, ptrs, scal, scal, 3, 8, 32, 16, 4, 16, None)
+    assert rc == 1 and b"NULL" in lib.ti_last_error()
+    assert lib.ti_linear_a8_w8_b8_o8_group_heads(p, ptrs, ptrs, ptrs, scal, scal, 0, 8, 32, 16, 4, 16, None) == 0
     # empty problems succeed without touching pointers or a device
     assert lib.ti_linear_a8_w8_b8_o8(None, None, None, None, 0, 16, 16, 1.0, 1.0, None, 0, None) == 0
     assert lib.ti_dq_add_layernorm_q(None, 1.0, None, None, None, 1e-5, None, None, 0, 128, None) == 0

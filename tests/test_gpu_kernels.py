@@ -545,6 +545,42 @@ def test_grouped_qkv_linear():
             assert C._lib.ti_last_kernel().decode() == family
 
 
+def test_grouped_prefill_linears_one_launch():
+    # q/k/v-style groups at prefill sizes: plain and head-major stores, the one-launch kernels and the loop
+    import ctypes
+    import torch_int._CUDA as C
+    import torch_int._hip_ext as X
+    C._lib.ti_last_kernel.restype = ctypes.c_char_p
+    g = torch.Generator().manual_seed(31)
+    # (bsz, seq, heads, d, K, problems, family)
+    for (B, T, H, d, K, n, family) in [(4, 512, 40, 128, 256, 3, "pipe16_256x160_group"),
+                                       (2, 1000, 72, 128, 128, 3, "pipe16_256x288_group"),
+                                       (2, 100, 5, 128, 384, 2, "pipe16_256x160_group"),
+                                       (1, 300, 9, 32, 640, 4, "pipe16_256x288_group"),
+                                       (3, 171, 10, 16, 128, 3, "pipe16_256x160_group"),
+                                       (2, 100, 6, 128, 128, 3, None), (2, 60, 5, 128, 128, 3, None),
+                                       (2, 100, 5, 128, 192, 3, None)]:
+        M, N = B * T, H * d
+        _say(f"grouped prefill linear M={M} N={N} K={K} n={n}")
+        x = _s8(g, M, K)
+        ws, bs = [_s8(g, N, K) for _ in range(n)], [_s8(g, N) for _ in range(n)]
+        al, be = [_scal(g, 1e-4, 1e-2) for _ in range(n)], [_scal(g, 1e-4, 1e-2) for _ in range(n)]
+        xd, wd, bd = x.to(DEV), [w.to(DEV) for w in ws], [b.to(DEV) for b in bs]
+        ref = orc.linear_a8_w8_b8_o8_group(x, ws, bs, al, be)
+        out = X.linear_a8_w8_b8_o8_group(xd, wd, bd, al, be)
+        if family:
+            assert C._lib.ti_last_kernel().decode() == family
+        for o, r_ in zip(out, ref):
+            assert torch.equal(o.cpu(), r_), (M, N, K)
+        out = X.linear_a8_w8_b8_o8_group_heads(xd, wd, bd, al, be, B, T, H, d)
+        if family:
+            assert C._lib.ti_last_kernel().decode() == family
+        assert X.linear_group_is_one_launch(M, N, K) == (family is not None)
+        for o, r_ in zip(out, ref):
+            assert o.shape == (B, H, T, d) and o.is_contiguous()
+            assert torch.equal(o.cpu(), r_.view(B, T, H, d).transpose(1, 2)), (M, N, K)
+
+
 def test_kv_append_kernel():
     import torch_int._hip_ext as X
     g = torch.Generator().manual_seed(17)

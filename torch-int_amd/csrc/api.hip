@@ -151,11 +151,10 @@ int ti_linear_a8_w8_b8_o8_heads(const int8_t* x, const int8_t* w, const int8_t* 
                   ws_bytes, stream, 0, 0, T, head_dim);
 }
 
-int ti_linear_a8_w8_b8_o8_group(const int8_t* x, const int8_t* const* w, const int8_t* const* bias, int8_t* const* out,
-                                const float* alpha, const float* beta, int64_t count, int64_t M, int64_t N,
-                                int64_t K, void* stream) {
+static int linear_group(const char* op, const int8_t* x, const int8_t* const* w, const int8_t* const* bias,
+                        int8_t* const* out, const float* alpha, const float* beta, int64_t count, int64_t M, int64_t N,
+                        int64_t K, int64_t T, int64_t head_dim, void* stream) {
   g_err[0] = 0;
-  const char* op = "linear_a8_w8_b8_o8_group";
   if (count < 0 || count > 4) return fail(TI_ERR_INVALID_ARG, "%s: 0 to 4 problems per group, got %lld", op, (long long)count);
   if (int rc = check_dims(op, 1, M, N, K)) return rc;
   const bool nonempty = count > 0 && M > 0 && N > 0;
@@ -191,7 +190,26 @@ int ti_linear_a8_w8_b8_o8_group(const int8_t* x, const int8_t* const* w, const i
   p.strideC = M * N;
   p.alpha = grp.alpha[0];
   p.beta = grp.beta[0];
+  p.out_T = (int)T;
+  p.out_d = (int)head_dim;
   return launch_gemm_group_s8(p, grp, static_cast<hipStream_t>(stream));
+}
+
+int ti_linear_a8_w8_b8_o8_group(const int8_t* x, const int8_t* const* w, const int8_t* const* bias, int8_t* const* out,
+                                const float* alpha, const float* beta, int64_t count, int64_t M, int64_t N,
+                                int64_t K, void* stream) {
+  return linear_group("linear_a8_w8_b8_o8_group", x, w, bias, out, alpha, beta, count, M, N, K, 0, 0, stream);
+}
+
+int ti_linear_a8_w8_b8_o8_group_heads(const int8_t* x, const int8_t* const* w, const int8_t* const* bias,
+                                      int8_t* const* out, const float* alpha, const float* beta, int64_t count,
+                                      int64_t M, int64_t N, int64_t K, int64_t T, int64_t head_dim, void* stream) {
+  const char* op = "linear_a8_w8_b8_o8_group_heads";
+  g_err[0] = 0;
+  if (T <= 0 || head_dim <= 0 || M % T != 0 || N % head_dim != 0 || head_dim % 16 != 0)
+    return fail(TI_ERR_INVALID_ARG, "%s: M=%lld must be a multiple of T=%lld, N=%lld of head_dim=%lld, head_dim of 16",
+                op, (long long)M, (long long)T, (long long)N, (long long)head_dim);
+  return linear_group(op, x, w, bias, out, alpha, beta, count, M, N, K, T, head_dim, stream);
 }
 
 int ti_linear_relu_a8_w8_b8_o8(const int8_t* x, const int8_t* w, const int8_t* bias, int8_t* out, int64_t M,

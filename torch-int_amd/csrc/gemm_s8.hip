@@ -1116,9 +1116,12 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe16_kernel(GemmParams p, i
 
 // The 16x16-block kernel with K steps of 128 bytes and two LDS stages (see gemm_pipe2_kernel for the
 // stage layout and the step structure; a step here is two 64-byte slices, one MFMA deep each).
-template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int KIND_>
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int KIND_, bool GROUPED_ = false>
 struct Pipe16QCfg {
   static constexpr int BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, KIND = KIND_;
+  // GROUPED: the "batches" are the problems of a GemmGroup (same activations and shape; weight, bias,
+  // output and scales per problem), so that q/k/v projections run as one persistent launch
+  static constexpr bool GROUPED = GROUPED_;
   static constexpr int NWAVES = WAVES_M * WAVES_N;
   static constexpr int NT = NWAVES * 64;
   static constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
@@ -1135,7 +1138,8 @@ struct Pipe16QCfg {
 };
 
 template <class Cfg>
-__global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe16q_kernel(GemmParams p, int tiles_m, int tiles_n, int items) {
+__global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe16q_kernel(GemmParams p, int tiles_m, int tiles_n, int items,
+                                                                  GemmGroup grp) {
   constexpr int BM = Cfg::BM, BN = Cfg::BN, TM = Cfg::TM, TN = Cfg::TN, COPIES = Cfg::COPIES;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
@@ -1157,8 +1161,8 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe16q_kernel(GemmParams p, 
     int tile_m, tile_n;
     tile_of_workgroup(item - b * tiles, tiles_m, tiles_n, tile_m, tile_n);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
-    const int8_t* A = p.A + (long long)b * p.strideA;
-    const int8_t* B = p.B + (long long)b * p.strideB;
+    const int8_t* A = Cfg::GROUPED ? p.A : p.A + (long long)b * p.strideA;
+    const int8_t* B = Cfg::GROUPED ? grp.B[b] : p.B + (long long)b * p.strideB;
 #pragma unroll
     for (int j = 0; j < COPIES; ++j) {
       int prow = wave * Cfg::RPW + j * 8 + (lane >> 3);
@@ -1287,7 +1291,16 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe16q_kernel(GemmParams p, 
     tile_of_workgroup(item - b * tiles, tiles_m, tiles_n, tile_m, tile_n);
     int lane_here = lane;  // opaque copy: keeps the epilogue's address arithmetic out of the mainloop
     asm volatile("" : "+v"(lane_here));
-    store_tile16<Cfg>(acc, p, b, tile_m, tile_n, wave_m, wave_n, lane_here);
+    if constexpr (Cfg::GROUPED) {
+      GemmParams q = p;  // problem b of the group as a one-batch problem
+      q.bias = grp.bias[b];
+      q.C = grp.C[b];
+      q.alpha = grp.alpha[b];
+      q.beta = grp.beta[b];
+      store_tile16<Cfg>(acc, q, 0, tile_m, tile_n, wave_m, wave_n, lane_here);
+    } else {
+      store_tile16<Cfg>(acc, p, b, tile_m, tile_n, wave_m, wave_n, lane_here);
+    }
     item += stride;
     kt = 0;
     zero_acc();
@@ -1648,8 +1661,8 @@ static int num_cus() {
   return n;
 }
 
-template <class Cfg, class Kern>
-static int launch_persistent(Kern kern, const GemmParams& p, hipStream_t stream) {
+template <class Cfg, class Kern, class... Extra>
+static int launch_persistent(Kern kern, const GemmParams& p, hipStream_t stream, Extra... extra) {
   static unsigned long long lds_ok = 0;
   if (int rc = allow_lds(kern, Cfg::LDS_BYTES, lds_ok)) return rc;
   const int tiles_m = (p.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (p.N + Cfg::BN - 1) / Cfg::BN;
@@ -1658,7 +1671,7 @@ static int launch_persistent(Kern kern, const GemmParams& p, hipStream_t stream)
   // one resident workgroup per LDS-sized slot; a multiple of 8 keeps the XCD mapping of tile ids
   const long long slots = (long long)num_cus() * ((160 * 1024) / Cfg::LDS_BYTES);
   const int grid = (int)(items < slots ? items : slots);
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, p, tiles_m, tiles_n, (int)items);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, p, tiles_m, tiles_n, (int)items, extra...);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "gemm launch: %s", hipGetErrorString(e));
   return TI_OK;
@@ -1679,8 +1692,8 @@ static int launch_pipe2(const GemmParams& p, hipStream_t stream) {
   return launch_persistent<Cfg>(gemm_pipe2_kernel<Cfg>, p, stream);
 }
 template <class Cfg>
-static int launch_pipe16q(const GemmParams& p, hipStream_t stream) {
-  return launch_persistent<Cfg>(gemm_pipe16q_kernel<Cfg>, p, stream);
+static int launch_pipe16q(const GemmParams& p, hipStream_t stream, const GemmGroup& grp = GemmGroup{}) {
+  return launch_persistent<Cfg>(gemm_pipe16q_kernel<Cfg>, p, stream, grp);
 }
 template <class Cfg>
 static int launch_pipe16(const GemmParams& p, hipStream_t stream) {
@@ -1931,8 +1944,9 @@ static int launch_kind(const GemmParams& p, void* workspace, long long workspace
 int launch_gemm_group_s8(const GemmParams& shape, const GemmGroup& grp, hipStream_t stream) {
   constexpr int KIND = EPI_S8_BIAS;
   if (shape.M == 0 || shape.N == 0 || grp.count == 0) return TI_OK;
-  bool aligned = (shape.K % SBK == 0) && shape.K > 0 && (reinterpret_cast<uintptr_t>(shape.A) & 15) == 0;
-  for (int i = 0; i < grp.count; ++i) aligned = aligned && (reinterpret_cast<uintptr_t>(grp.B[i]) & 15) == 0;
+  bool ptr_ok = (reinterpret_cast<uintptr_t>(shape.A) & 15) == 0;
+  for (int i = 0; i < grp.count; ++i) ptr_ok = ptr_ok && (reinterpret_cast<uintptr_t>(grp.B[i]) & 15) == 0;
+  const bool aligned = ptr_ok && (shape.K % SBK == 0) && shape.K > 0;
   const int spb = (shape.N + 15) / 16;
   const long long strips = (long long)spb * grp.count;
   if (aligned && shape.M <= 16 && strips >= 256) {
@@ -1952,6 +1966,26 @@ int launch_gemm_group_s8(const GemmParams& shape, const GemmGroup& grp, hipStrea
     if (shape.M == 1) return launch(gemm_stream_kernel<KIND, 1, 2, true>, 17, 4);
     if (shape.M <= 4) return launch(gemm_stream_kernel<KIND, 4, 2, true>, 20, 3);
     return launch(gemm_stream_kernel<KIND, 16, 2, true>, 32, 2);
+  }
+  // Prefill shapes whose width the 256x160 or 256x288 tiles divide: the problems are the batches of one
+  // persistent launch, so the pipeline fill and the epilogue of one projection overlap the next one's work.
+  if (ptr_ok && shape.M > 128 && shape.K % QBK == 0 && shape.K >= QBK && grp.count > 1 && shape.lda == shape.K &&
+      shape.ldb == shape.K) {
+    const long long cus = num_cus();
+    auto fill = [&](long long tiles) { return (double)tiles / (double)(((tiles + cus - 1) / cus) * cus); };
+    const long long rows256 = (shape.M + 255) / 256;
+    const double e160 = shape.N % 160 == 0 ? 0.88 * fill(rows256 * (shape.N / 160) * grp.count) : 0.0;
+    const double e288 = shape.N % 288 == 0 ? 0.95 * fill(rows256 * (shape.N / 288) * grp.count) : 0.0;
+    if (e160 > 0.0 || e288 > 0.0) {
+      GemmParams q = shape;
+      q.batch = grp.count;
+      if (e160 >= e288) {
+        g_last_kernel = "pipe16_256x160_group";
+        return launch_pipe16q<Pipe16QCfg<256, 160, 4, 2, KIND, true>>(q, stream, grp);
+      }
+      g_last_kernel = "pipe16_256x288_group";
+      return launch_pipe16q<Pipe16QCfg<256, 288, 4, 2, KIND, true>>(q, stream, grp);
+    }
   }
   for (int i = 0; i < grp.count; ++i) {
     GemmParams q = shape;

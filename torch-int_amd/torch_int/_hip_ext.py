@@ -52,6 +52,9 @@ _pp = ctypes.POINTER(ctypes.c_void_p)
 _lib.ti_linear_a8_w8_b8_o8_group.argtypes = [_vp, _pp, _pp, _pp, ctypes.POINTER(_f32), ctypes.POINTER(_f32), _i64, _i64,
                                             _i64, _i64, _vp]
 _lib.ti_linear_a8_w8_b8_o8_group.restype = ctypes.c_int
+_lib.ti_linear_a8_w8_b8_o8_group_heads.argtypes = [_vp, _pp, _pp, _pp, ctypes.POINTER(_f32), ctypes.POINTER(_f32), _i64,
+                                                   _i64, _i64, _i64, _i64, _i64, _vp]
+_lib.ti_linear_a8_w8_b8_o8_group_heads.restype = ctypes.c_int
 _raw_stream = torch._C._cuda_getCurrentRawStream
 _fast = _CUDA._fast if getattr(_CUDA._fast, "kv_append", None) is not None else None
 _fast_decode_attn = getattr(_CUDA._fast, "decode_attn", None)
@@ -437,6 +440,44 @@ def linear_a8_w8_b8_o8_group(x, weights, biases, alphas, betas, checked=False):
                 farr(*[float(b) for b in betas]), n, M, N, K, stream or None)
     if rc:
         raise RuntimeError(f"torch_int._hip_ext.linear_a8_w8_b8_o8_group: {_lib.ti_last_error().decode()} (status {rc})")
+    return out.unbind(0)
+
+
+def linear_group_is_one_launch(M, N, K):
+    """Whether the library runs a group of [M,K] x [N,K] linears as ONE launch (otherwise it loops over the
+    problems, without the split-K workspace that separate calls would get)."""
+    if M <= 16:
+        return K % 1024 == 0
+    return M > 128 and K >= 128 and K % 128 == 0 and (N % 160 == 0 or N % 288 == 0)
+
+
+def linear_a8_w8_b8_o8_group_heads(x, weights, biases, alphas, betas, bsz, seq_len, heads, head_dim, checked=False):
+    """``[linear_a8_w8_b8_o8_heads(x, w, b, a, be, bsz, seq_len, heads, head_dim) for ...]`` as one call: a tuple
+    of int8 [bsz, heads, seq, head_dim] outputs (views of one allocation).  The q/k/v projections of a prefill:
+    widths the 256x160 or 256x288 tiles divide run as one persistent launch over all the problems."""
+    if not checked and not (can_linear_group(x, weights, biases)
+                            and all(can_linear_heads(x, w, b, bsz, seq_len, heads, head_dim)
+                                    for w, b in zip(weights, biases))):
+        raise RuntimeError("torch_int._hip_ext.linear_a8_w8_b8_o8_group_heads: needs a contiguous int8 HIP input "
+                           "[bsz*seq,K] and 1-4 contiguous int8 weights [heads*d,K] / biases [heads*d] of one shape "
+                           "on the same device, d a multiple of 16")
+    n = len(weights)
+    M, K = x.shape
+    N = weights[0].shape[0]
+    out = torch.empty((n, bsz, heads, seq_len, head_dim), dtype=torch.int8, device=x.device)
+    step = M * N
+    base = out.data_ptr()
+    arr = ctypes.c_void_p * n
+    farr = _f32 * n
+    with _on(x.device):
+        stream = _raw_stream(x.device.index)
+        rc = _lib.ti_linear_a8_w8_b8_o8_group_heads(
+            x.data_ptr(), arr(*[w.data_ptr() for w in weights]), arr(*[b.data_ptr() for b in biases]),
+            arr(*[base + i * step for i in range(n)]), farr(*[float(a) for a in alphas]),
+            farr(*[float(b) for b in betas]), n, M, N, K, seq_len, head_dim, stream or None)
+    if rc:
+        raise RuntimeError(f"torch_int._hip_ext.linear_a8_w8_b8_o8_group_heads: {_lib.ti_last_error().decode()} "
+                           f"(status {rc})")
     return out.unbind(0)
 
 

@@ -158,15 +158,19 @@ class Int8OPTAttention(nn.Module):
             return None
         x = hidden_states.reshape(-1, hidden_states.shape[-1])
         H, d = self.num_heads, self.head_dim
-        out = []
-        for lin in (q, k, v):
-            w, b = lin._wb()
-            b = b.reshape(-1)
-            if not _hip_ext.can_linear_heads(x, w, b, bsz, tgt_len, H, d):
-                return None
-            out.append(_hip_ext.linear_a8_w8_b8_o8_heads(x, w, b, lin._scalar("a"), lin._scalar("b"), bsz, tgt_len, H, d,
-                                                         checked=True))
-        return tuple(out)
+        wb = [lin._wb() for lin in (q, k, v)]
+        weights, biases = [w for w, _ in wb], [b.reshape(-1) for _, b in wb]
+        if not all(_hip_ext.can_linear_heads(x, w, b, bsz, tgt_len, H, d) for w, b in zip(weights, biases)):
+            return None
+        if (_hip_ext.can_linear_group(x, weights, biases)
+                and _hip_ext.linear_group_is_one_launch(x.shape[0], weights[0].shape[0], x.shape[1])):
+            # one call; widths the 16x16-block tiles divide run as a single persistent launch
+            return _hip_ext.linear_a8_w8_b8_o8_group_heads(
+                x, weights, biases, [lin._scalar("a") for lin in (q, k, v)], [lin._scalar("b") for lin in (q, k, v)],
+                bsz, tgt_len, H, d, checked=True)
+        return tuple(_hip_ext.linear_a8_w8_b8_o8_heads(x, w, b, lin._scalar("a"), lin._scalar("b"), bsz, tgt_len, H, d,
+                                                       checked=True)
+                     for lin, w, b in zip((q, k, v), weights, biases))
 
     def _shape(self, tensor: torch.Tensor, seq_len: int, bsz: int):
         """[bsz, seq, embed] -> contiguous [bsz, heads, seq, head_dim]."""
