@@ -253,3 +253,46 @@ def test_causal_lm_prefill_and_decode_on_gpu():
         assert torch.equal(x, y)                       # same kernels' arithmetic on either layout
     for (k1, v1), (k2, v2) in zip(a_past, b_past):
         assert torch.equal(k1, k2) and torch.equal(v1, v2)
+
+
+@torch.no_grad()
+def test_side_stream_and_graph_replay_of_a_decoder_layer():
+    """The launches go to torch's current stream: a layer run on a side stream, and one captured into a
+    graph and replayed (with eager work and synchronisations between the replays), give the bits of the
+    plain eager run."""
+    g = torch.Generator().manual_seed(5)
+    D, H, F, B, T = 640, 5, 1280, 3, 128  # widths the grouped projection and the fused attention take
+    layer = randomize_int8_layer(Int8OPTDecoderLayer(D, H, F), g).to(DEV)
+    hidden0 = torch.randn(B, T, D, generator=g).to(DEV)
+    mask = causal_mask(B, T, T).to(DEV)
+    for _ in range(2):  # warm-up: first-use attribute calls, scalar caches, workspaces
+        eager = layer(hidden0.clone(), attention_mask=mask, use_cache=True)
+    torch.cuda.synchronize()
+
+    _say("layer on a side stream")
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        layer(hidden0.clone(), attention_mask=mask, use_cache=True)  # this stream's own workspace
+        out = layer(hidden0.clone(), attention_mask=mask, use_cache=True)
+    side.synchronize()
+    assert torch.equal(out[0], eager[0]) and torch.equal(out[1][0], eager[1][0]) and torch.equal(out[1][1], eager[1][1])
+
+    _say("layer captured into a graph")
+    static_in = hidden0.clone()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        layer(static_in.clone(), attention_mask=mask, use_cache=True)
+    side.synchronize()
+    with torch.cuda.graph(graph, stream=side):
+        static_out = layer(static_in, attention_mask=mask, use_cache=True)  # updates static_in in place
+    for i in range(3):
+        _say("replay", i)
+        other = torch.randn(B, T, D, generator=g).to(DEV) if i == 1 else hidden0
+        ref = layer(other.clone(), attention_mask=mask, use_cache=True)  # eager work between the replays
+        torch.cuda.synchronize()
+        static_in.copy_(other)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(static_out[0], ref[0]), i
+        assert torch.equal(static_out[1][0], ref[1][0]) and torch.equal(static_out[1][1], ref[1][1]), i
