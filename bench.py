@@ -117,25 +117,28 @@ def sustained_ms(torch, fns, window_ms=200.0, warm_launches=100):
 
 
 def cpu_baseline(torch):
-    """torch CPU int32 matmul + the oracle's fp32 epilogue (the reference's integer emulation),
-    on an M=256 slice of the q/k/v/out_proj shape, all four variants."""
+    """torch CPU int32 matmul + the oracle's fp32 epilogue (the reference's integer emulation), on an M=256
+    slice of each of the sweep's three (N, K) shapes, all four variants: 10-20 s of CPU work."""
     from oracle import oracle as orc
     g = torch.Generator().manual_seed(0)
-    M, N, K = 256, 5120, 5120
-    x = torch.randint(-127, 128, (M, K), dtype=torch.int8, generator=g)
-    w = torch.randint(-127, 128, (N, K), dtype=torch.int8, generator=g)
-    b8 = torch.randint(-127, 128, (N,), dtype=torch.int8, generator=g)
-    b32 = torch.randint(-65535, 65535, (N,), dtype=torch.int32, generator=g)
-    bf = torch.randn(N, generator=g)
-    t0 = time.perf_counter()
-    orc.linear_a8_w8_b32_o32(x, w, b32, acc_fn=orc.gemm_acc_torch)
-    orc.linear_a8_w8_bfp32_ofp32(x, w, bf, 0.001, 1.0, acc_fn=orc.gemm_acc_torch)
-    orc.linear_a8_w8_b8_o8(x, w, b8, 0.001, 0.01, acc_fn=orc.gemm_acc_torch)
-    orc.linear_relu_a8_w8_b8_o8(x, w, b8, 0.001, 0.01, acc_fn=orc.gemm_acc_torch)
-    dt = time.perf_counter() - t0
-    ops = 4 * 2.0 * M * N * K
+    M = 256
+    ops = dt = 0.0
+    for N, K in SHAPES:
+        x = torch.randint(-127, 128, (M, K), dtype=torch.int8, generator=g)
+        w = torch.randint(-127, 128, (N, K), dtype=torch.int8, generator=g)
+        b8 = torch.randint(-127, 128, (N,), dtype=torch.int8, generator=g)
+        b32 = torch.randint(-65535, 65535, (N,), dtype=torch.int32, generator=g)
+        bf = torch.randn(N, generator=g)
+        t0 = time.perf_counter()
+        orc.linear_a8_w8_b32_o32(x, w, b32, acc_fn=orc.gemm_acc_torch)
+        orc.linear_a8_w8_bfp32_ofp32(x, w, bf, 0.001, 1.0, acc_fn=orc.gemm_acc_torch)
+        orc.linear_a8_w8_b8_o8(x, w, b8, 0.001, 0.01, acc_fn=orc.gemm_acc_torch)
+        orc.linear_relu_a8_w8_b8_o8(x, w, b8, 0.001, 0.01, acc_fn=orc.gemm_acc_torch)
+        dt += time.perf_counter() - t0
+        ops += 4 * 2.0 * M * N * K
+    shapes = ", ".join(f"{N}x{K}" for N, K in SHAPES)
     return {"value": ops / dt / 1e12, "unit": "TOPS", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": f"4 variants x (M={M}, N={N}, K={K}) torch int32 matmul + fp32 epilogue, "
+            "sample": f"4 variants x M={M} rows of each (N,K) in {{{shapes}}}: torch int32 matmul + fp32 epilogue, "
                       f"{dt:.1f} s, host cpu_count={os.cpu_count()}"}
 
 
