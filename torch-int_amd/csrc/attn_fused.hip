@@ -45,8 +45,11 @@ __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t*
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const long long bh = blockIdx.x / row_blocks;
-  const int t0 = (blockIdx.x % row_blocks) * AF_ROWS;
+  // Workgroups are dispatched in blockIdx order: the last row blocks first (under a causal mask they have the
+  // most live keys), one per (batch, head), then the next ones, so that the light blocks fill the tail.
+  const int n_bh = gridDim.x / row_blocks;
+  const long long bh = blockIdx.x % n_bh;
+  const int t0 = (row_blocks - 1 - (int)(blockIdx.x / n_bh)) * AF_ROWS;
   const int nb = S >> 4;
 
   // ---- copies: slab i = 8 rows of [Q tile (64 rows) | K panel (S rows)], 1 KiB per wave instruction
