@@ -100,7 +100,7 @@ def test_linear_large_tiles(variant):
     # enough 256x256 tiles to select the large-tile kernel, with ragged M and N
     import torch_int._CUDA as C
     for (M, N, K) in [(2048, 5120, 256), (2100, 5000, 272), (4096, 2560, 128), (4000, 2816, 1024), (4090, 2790, 256),
-                      (2010, 5120, 384), (1990, 9216, 128)]:
+                      (2010, 5120, 384), (1990, 9216, 128), (2040, 5120, 128), (2048, 2560, 640)]:
         _say(f"linear-large {variant} M={M} N={N} K={K}")
         _linear_case(C, variant, M, N, K, seed=7)
 

@@ -1127,7 +1127,10 @@ struct Pipe16QCfg {
   static constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
   static constexpr int TM = WTM / 16, TN = WTN / 16;
   static constexpr int STAGE_BYTES = (BM + BN) * QBK;
-  static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
+  // three stages when the LDS holds them (256x160): copies then run two to three K steps ahead of their use,
+  // which covers the latency of operands that come from HBM instead of the last-level cache
+  static constexpr int STAGES = 3 * STAGE_BYTES <= 160 * 1024 ? 3 : 2;
+  static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
   static constexpr int RPW = (BM + BN) / NWAVES;  // panel rows a wave copies per step
   static constexpr int TAIL_ROWS = RPW % 8;
   static constexpr int COPIES = RPW / 8 + (TAIL_ROWS ? 1 : 0);
@@ -1180,9 +1183,11 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe16q_kernel(GemmParams p, 
       }
     }
   };
-  int c_item = first, c_kt = 0, c_g = 0, c_live = 1;
+  constexpr int STAGES = Cfg::STAGES;
+  auto next_slot = [](int slot) { return slot + 1 == STAGES ? 0 : slot + 1; };
+  int c_item = first, c_kt = 0, c_g = 0, c_live = 1, c_slot = 0;
   auto issue_copies = [&]() {
-    TI_LDS_AS char* dst = (TI_LDS_AS char*)smem + (c_g & 1) * Cfg::STAGE_BYTES + wave * Cfg::RPW * QBK;
+    TI_LDS_AS char* dst = (TI_LDS_AS char*)smem + c_slot * Cfg::STAGE_BYTES + wave * Cfg::RPW * QBK;
 #pragma unroll
     for (int j = 0; j < COPIES; ++j) {
       if (Cfg::TAIL_ROWS == 0 || j + 1 < COPIES || lane < Cfg::TAIL_ROWS * 8)
@@ -1191,6 +1196,7 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe16q_kernel(GemmParams p, 
     }
     c_kt += c_live;
     ++c_g;
+    c_slot = next_slot(c_slot);
   };
   auto advance_copy_item = [&]() {  // call when c_live && c_kt == KT
     if (c_g < G) {
@@ -1216,19 +1222,19 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe16q_kernel(GemmParams p, 
 #pragma unroll
       for (int j = 0; j < TN; ++j) acc[i][j] = v4i{0, 0, 0, 0};
   };
-  auto read_a = [&](int gs, int slice, v4i (&fa)[TM]) {
-    const char* st = smem + (gs & 1) * Cfg::STAGE_BYTES;
+  auto read_a = [&](int slot, int slice, v4i (&fa)[TM]) {
+    const char* st = smem + slot * Cfg::STAGE_BYTES;
 #pragma unroll
     for (int i = 0; i < TM; ++i) fa[i] = *reinterpret_cast<const v4i*>(st + ((a_frag ^ (slice << 6)) + i * 16 * QBK));
   };
-  auto read_b1 = [&](int gs, int slice, int j) {
-    const char* st = smem + (gs & 1) * Cfg::STAGE_BYTES;
+  auto read_b1 = [&](int slot, int slice, int j) {
+    const char* st = smem + slot * Cfg::STAGE_BYTES;
     return *reinterpret_cast<const v4i*>(st + ((b_frag ^ (slice << 6)) + j * 16 * QBK));
   };
-  auto read_frags = [&](int gs, int slice, v4i (&fa)[TM], v4i (&fb)[TN]) {
-    read_a(gs, slice, fa);
+  auto read_frags = [&](int slot, int slice, v4i (&fa)[TM], v4i (&fb)[TN]) {
+    read_a(slot, slice, fa);
 #pragma unroll
-    for (int j = 0; j < TN; ++j) fb[j] = read_b1(gs, slice, j);
+    for (int j = 0; j < TN; ++j) fb[j] = read_b1(slot, slice, j);
   };
   auto interleave = [&]() {  // one LDS read after each of the first TM+TN MFMAs
 #pragma unroll
@@ -1238,7 +1244,7 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe16q_kernel(GemmParams p, 
     }
     __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - (TM + TN), 0);
   };
-  // Multiplies the fragments (fc, fd) while those of (gs_next, slice_next) load into (fn, fm); with
+  // Multiplies the fragments (fc, fd) while those of (stage gs_next, slice_next) load into (fn, fm); with
   // SINGLE_B the weight fragments live in fd only and are replaced block by block.
   auto mma_and_fetch = [&](v4i (&fc)[TM], v4i (&fd)[TN], v4i (&fn)[TM], v4i (&fm)[TN], int gs_next, int slice_next,
                            auto fetch) {
@@ -1265,24 +1271,27 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe16q_kernel(GemmParams p, 
 
   set_copy_item(c_item);
 #pragma unroll
-  for (int s = 0; s < 2; ++s) {
+  for (int s = 0; s < STAGES; ++s) {
     issue_copies();
     if (c_live && c_kt == KT) advance_copy_item();
   }
-  wait_copies_then_barrier<COPIES>();
+  wait_copies_then_barrier<(STAGES - 1) * COPIES>();  // step 0 has landed
 
   v4i fa0[TM], fb0[TN], fa1[TM], fb1[TN];  // fb1 is unused with SINGLE_B
   read_frags(0, 0, fa0, fb0);
   zero_acc();
 
-  int item = first, kt = 0, gs = 0;  // multiply cursor
+  int item = first, kt = 0, gs = 0, slot = 0;  // multiply cursor; slot = gs % STAGES
   auto step = [&](auto last) {
     constexpr bool LAST = decltype(last)::value;
-    mma_and_fetch(fa0, fb0, fa1, Cfg::SINGLE_B ? fb0 : fb1, gs, 1, std::true_type{});
-    // the lgkmcnt wait is what allows this stage to be overwritten after the barrier
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    issue_copies();  // step gs+2 into the stage this step used
-    mma_and_fetch(fa1, Cfg::SINGLE_B ? fb0 : fb1, fa0, fb0, gs + 1, 0, std::integral_constant<bool, !LAST>{});
+    mma_and_fetch(fa0, fb0, fa1, Cfg::SINGLE_B ? fb0 : fb1, slot, 1, std::true_type{});
+    // Step gs+1 has landed once at most the copies of the steps after it are outstanding (loads complete in
+    // order; stores of an epilogue in between only make the count conservative).  The lgkmcnt wait is what
+    // allows this stage to be overwritten after the barrier.
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"((STAGES - 2) * COPIES) : "memory");
+    issue_copies();  // step gs+STAGES into the stage this step used
+    slot = next_slot(slot);
+    mma_and_fetch(fa1, Cfg::SINGLE_B ? fb0 : fb1, fa0, fb0, slot, 0, std::integral_constant<bool, !LAST>{});
     ++gs;
   };
   auto finish_item = [&]() {
@@ -1318,7 +1327,7 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe16q_kernel(GemmParams p, 
     if (c_live && c_kt == KT) advance_copy_item();
     if (item_done) {
       finish_item();
-      if (gs < G) read_frags(gs, 0, fa0, fb0);
+      if (gs < G) read_frags(slot, 0, fa0, fb0);
     }
   }
   __builtin_amdgcn_s_waitcnt(0x0F70);  // the trailing filler copies must land before the LDS is released
@@ -1897,13 +1906,13 @@ static int launch_kind(const GemmParams& p, void* workspace, long long workspace
       // 256x160 or 256x288 tiles (16x16 blocks) when the width allows it and they fill the CUs more
       // evenly (e.g. 2048x5120: 160 tiles of 256x256 but 256 of 256x160; 2048x9216: 288 tiles of 256x256 =
       // two rounds, but exactly 256 of 256x288).  Rates relative to the 256x256 kernel at full occupancy,
-      // measured: with 128-byte steps 0.88 (256x160; 0.85 with 32-bit stores) and 0.95 (256x288); with
-      // 64-byte steps (K not a multiple of 128) 0.78 and 0.9.
+      // measured: with 128-byte steps 0.94 (256x160, three LDS stages) and 0.95 (256x288); with 64-byte steps
+      // (K not a multiple of 128) 0.78 and 0.9.
       const long long cus = num_cus();
       auto fill = [&](long long tiles) { return (double)tiles / (double)(((tiles + cus - 1) / cus) * cus); };
       const long long rows256 = (p.M + 255) / 256;
       const bool wide_step = p.K % QBK == 0;
-      const double f160 = !wide_step ? 0.78 : sizeof(Out) == 1 ? 0.88 : 0.85;
+      const double f160 = wide_step ? 0.94 : 0.78;
       const double f288 = wide_step ? 0.95 : 0.9;
       const double e256 = fill(t256);
       const double e160 = p.N % 160 == 0 ? f160 * fill(rows256 * (p.N / 160) * p.batch) : 0.0;
