@@ -276,6 +276,17 @@ def test_bmm_attention_config(S):
     _bmm_case(C, BH, S, d, S, seed=32, prob_lhs=True)   # P.V^T^T
 
 
+def test_bmm_long_prefill_pv_tile():
+    # P.V of a long prefill (N = 128, many row tiles): the 256x128 three-stage kernel, ragged M included
+    import ctypes
+    import torch_int._CUDA as C
+    C._lib.ti_last_kernel.restype = ctypes.c_char_p
+    for (B, M, K) in [(64, 2048, 256), (70, 1900, 384), (260, 520, 128)]:
+        _say(f"long P.V B={B} M={M} N=128 K={K}")
+        _bmm_case(C, B, M, 128, K, seed=77, prob_lhs=True)
+        assert C._lib.ti_last_kernel().decode() == "pipe16_256x128", (B, M, K)
+
+
 def test_bmm_full_size_properties():
     # B*H = 160, S = 512, d = 128 (the attention-product benchmark configuration): size-independent checks
     import torch_int._CUDA as C

@@ -1931,6 +1931,11 @@ static int launch_kind(const GemmParams& p, void* workspace, long long workspace
       if (p.K % QBK == 0) return launch_pipe2<Pipe2Cfg<256, 256, 2, 4, KIND, SWAP>>(p, stream);  // whole cache lines per row
       return launch_pipe<PipeCfg<256, 256, 2, 4, 4, KIND, SWAP>>(p, stream);
     }
+    // 128-wide outputs with many rows (P.V of a long prefill): 256x128 tiles, three stages of 128-byte steps
+    if (p.N == 128 && p.K % QBK == 0 && p.M >= 512 && (long long)((p.M + 255) / 256) * p.batch >= 2 * num_cus()) {
+      g_last_kernel = "pipe16_256x128";
+      return launch_pipe16q<Pipe16QCfg<256, 128, 4, 2, KIND>>(p, stream);
+    }
     if (t128 >= 128) {
       g_last_kernel = "pipe_128x128";
       return launch_pipe<PipeCfg<128, 128, 2, 2, 4, KIND, SWAP>>(p, stream);
