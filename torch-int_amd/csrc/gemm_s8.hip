@@ -1786,6 +1786,15 @@ static int choose_splits(long long M, long long N, long long K, int* tile_kind =
         step_us = kind == SPLIT_256 ? 0.85 : kind == SPLIT_256x160 ? 0.55 : 0.92;
       }
       double t = rounds * ((double)(steps / s) * step_us + 8.0);
+      // The weights come from HBM: a workgroup keeps about `ahead` K steps of its weight rows in flight, and what
+      // all resident workgroups have in flight over a 2 us round trip bounds the streaming rate (5 TB/s at most).
+      const double ahead = kind == SPLIT_128 ? 4.0 : kind == SPLIT_256x160 ? 2.5 : 1.5;
+      const double step_bytes = (double)bn * (kind == SPLIT_128 ? 64.0 : 128.0);
+      const double resident = wgs < cus * (kind == SPLIT_128 ? 2 : 1) ? wgs : cus * (kind == SPLIT_128 ? 2 : 1);
+      double rate = resident * ahead * step_bytes / 2.0;  // bytes per us
+      if (rate > 5.0e6) rate = 5.0e6;
+      const double t_stream = (double)N * (double)K / rate + 8.0;
+      if (t < t_stream) t = t_stream;
       if (s > 1) t += (double)(2 * s + 1) * M * N * 4.0 / 8.0e6 + 3.0;  // partials out and back in, at 8 TB/s, in us
       if (t < best_t * 0.97) {  // prefer fewer slices and the smaller tile unless the gain is clear
         best_t = t;
