@@ -85,6 +85,20 @@ int ti_linear_a8_w8_b8_o8(const int8_t* x, const int8_t* w, const int8_t* bias, 
                           int64_t M, int64_t N, int64_t K, float alpha, float beta,
                           void* workspace, int64_t workspace_bytes, void* stream);
 
+/* ti_linear_a8_w8_b8_o8 for callers that cannot allocate device memory or pass a workspace (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.
+ * Same arguments minus the workspace, same bytes out.  The split-K partial products go to a buffer of
+ * TI_NOALLOC_SCRATCH_BYTES that is part of the library's device image (one copy per GPU, held until the
+ * process ends); the call allocates and frees nothing.  Shapes whose split needs more
+ * (ti_linear_workspace_bytes(M, N, K) > TI_NOALLOC_SCRATCH_BYTES) are refused with TI_ERR_INVALID_ARG.
+ * Every call on a GPU shares that GPU's buffer: calls that may overlap in time on one GPU (different
+ * streams, different threads) race and must be serialised by the caller.  The buffer needs no clearing
+ * between calls (every partial product is written before it is read).  ti_init() resolves the buffer's address
+ * for the current device; without it the first call on a device does. */
+#define TI_NOALLOC_SCRATCH_BYTES (40 * 1024 * 1024)
+int ti_linear_a8_w8_b8_o8_noalloc(const int8_t* x, const int8_t* w, const int8_t* bias, int8_t* out,
+                                  int64_t M, int64_t N, int64_t K, float alpha, float beta, void* stream);
+
 /* linear_a8_w8_b8_o8 whose [M, N] result is stored head-major: with M = B*T rows and N = H*head_dim columns,
  * element (b*T + t, h*head_dim + dd) goes to out[b][h][t][dd] of a packed [B, H, T, head_dim] tensor.  The
  * values are those of ti_linear_a8_w8_b8_o8; this replaces the `view(B,T,H,d).transpose(1,2).contiguous()`

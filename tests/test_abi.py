@@ -58,6 +58,11 @@ def test_c_abi_rejects_bad_arguments_without_a_device():
     # misaligned int32 output
     rc = lib.ti_bmm_s8t_s8n_s32t(p, p, p + 1, 1, 1, 4, 16, None)
     assert rc == 2 and b"aligned" in lib.ti_last_error()
+    # the no-allocation linear refuses a shape whose split-K scratch exceeds its built-in buffer (before any device call)
+    lib.ti_linear_a8_w8_b8_o8_noalloc.argtypes = ([ctypes.c_void_p] * 4 + [ctypes.c_int64] * 3 + [ctypes.c_float] * 2
+                                                  + [ctypes.c_void_p])
+    rc = lib.ti_linear_a8_w8_b8_o8_noalloc(p, p, p, p, 512, 9216, 9216, 1.0, 1.0, None)
+    assert rc == 1 and b"scratch" in lib.ti_last_error()
     # beyond the 32-bit tiling limits
     rc = lib.ti_linear_a8_w8_b32_o32(p, p, p, p, 1 << 20, 4, 1 << 20, None, 0, None)
     assert rc == 1 and b"limits" in lib.ti_last_error()

@@ -1,10 +1,19 @@
 // extern "C" surface of libtorch_int_hip.so: argument validation and dispatch.
 // Declarations and the contract of each entry point live in
 // include/torch_int_hip.h.
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
 #include "ti_common.h"
+
+// Split-K scratch of ti_linear_a8_w8_b8_o8_noalloc: int32 partial products [slices][M][N].  One copy of the
+// array lives on every GPU the library runs on, from the moment the code object is loaded there until the
+// process ends.  In host code this name is only a handle for hipGetSymbolAddress; kernels and copies get the
+// device address that scratch_address() returns.  (No `used` attribute here: with it the device compiler emits
+// the array before it has seen the host code that names it, keeps the symbol local to the code object, and the
+// runtime's lookup in hipGetSymbolAddress aborts the process.)
+static __device__ __align__(256) unsigned char scratch[TI_NOALLOC_SCRATCH_BYTES];
 
 namespace ti {
 
@@ -16,6 +25,30 @@ int fail(int code, const char* fmt, ...) {
   vsnprintf(g_err, sizeof(g_err), fmt, ap);
   va_end(ap);
   return code;
+}
+
+// Device address of `scratch` on the current device (each GPU has its own copy at its own address), looked
+// up once per device.  Racing first calls store the same value.
+static constexpr int kMaxDevices = 64;
+static std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+static int scratch_address(const char* op, void** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(TI_ERR_NO_DEVICE, "%s: hipGetDevice: %s", op, hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices)
+    return fail(TI_ERR_NO_DEVICE, "%s: device index %d is beyond the %d devices the scratch table covers", op, dev,
+                kMaxDevices);
+  void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (ptr == nullptr) {
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr)
+      return fail(TI_ERR_NO_DEVICE, "%s: hipGetSymbolAddress(scratch) on device %d: %s", op, dev,
+                  hipGetErrorString(e));
+    g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+  }
+  *out = ptr;
+  return TI_OK;
 }
 
 static int check_dims(const char* op, int64_t batch, int64_t M, int64_t N, int64_t K) {
@@ -105,7 +138,8 @@ int ti_init(void) {
   if (e != hipSuccess) return fail(TI_ERR_NO_DEVICE, "hipGetDeviceProperties: %s", hipGetErrorString(e));
   if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
     return fail(TI_ERR_NO_DEVICE, "device %d is %s; this library holds gfx950 code only", dev, prop.gcnArchName);
-  return TI_OK;
+  void* ptr = nullptr;  // resolve the no-allocation entry point's scratch here, outside any capture or hot loop
+  return scratch_address("ti_init", &ptr);
 }
 
 int64_t ti_linear_workspace_bytes(int64_t M, int64_t N, int64_t K) { return gemm_workspace_bytes(M, N, K); }
@@ -142,6 +176,25 @@ int ti_linear_a8_w8_b8_o8(const int8_t* x, const int8_t* w, const int8_t* bias, 
                           void* stream) {
   return run_gemm("linear_a8_w8_b8_o8", EPI_S8_BIAS, x, w, bias, 1, out, 1, 1, M, N, K, alpha, beta, ws,
                   ws_bytes, stream);
+}
+
+int ti_linear_a8_w8_b8_o8_noalloc(const int8_t* x, const int8_t* w, const int8_t* bias, int8_t* out, int64_t M,
+                                  int64_t N, int64_t K, float alpha, float beta, void* stream) {
+  const char* op = "linear_a8_w8_b8_o8_noalloc";
+  g_err[0] = 0;
+  if (int rc = check_dims(op, 1, M, N, K)) return rc;
+  const int64_t need = gemm_workspace_bytes(M, N, K);
+  if (need > (int64_t)TI_NOALLOC_SCRATCH_BYTES)
+    return fail(TI_ERR_INVALID_ARG,
+                "%s: M=%lld N=%lld K=%lld needs %lld bytes of split-K scratch, the built-in buffer holds %lld; "
+                "call ti_linear_a8_w8_b8_o8 with a workspace of your own",
+                op, (long long)M, (long long)N, (long long)K, (long long)need, (long long)TI_NOALLOC_SCRATCH_BYTES);
+  void* ws = nullptr;
+  if (need > 0) {
+    if (int rc = scratch_address(op, &ws)) return rc;
+  }
+  // the partial products are written in full before the reduction reads them: nothing to clear
+  return run_gemm(op, EPI_S8_BIAS, x, w, bias, 1, out, 1, 1, M, N, K, alpha, beta, ws, need > 0 ? need : 0, stream);
 }
 
 int ti_linear_a8_w8_b8_o8_heads(const int8_t* x, const int8_t* w, const int8_t* bias, int8_t* out, int64_t M,
