@@ -210,6 +210,7 @@ def main():
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-ceiling", action="store_true", help="skip the matrix-pipe ceiling loops")
     ap.add_argument("--sweep-only", action="store_true", help="skip the per-case, HBM-kernel and layer sections")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -298,6 +299,17 @@ def main():
                             "frac": f["ops"] / f["ms"] / 1e9 / PEAK_INT8_TOPS,
                             "traffic": FAMILIES.get(name, {}).get("traffic")} for name, f in fam.items()}}
 
+    if not args.no_ceiling:
+        # what the matrix pipe of this board sustains on constant / random operand bytes (diagnostic loops, no GEMM)
+        import torch_int._hip_ext as X
+        m = X.measure_mfma_ceiling(window_ms=250.0)
+        result["roofline"]["measured_ceiling"] = {
+            "unit": "TOP/s", "constant": m["mfma_only_constant"], "random": m["mfma_only_random"],
+            "lds_fed": m["lds_fed_random"], "all": m,
+            "frac_of_lds_fed": achieved / m["lds_fed_random"],
+            "note": "back-to-back launches of ti_diag_mfma_loop over 250 ms windows: v_mfma_i32_32x32x32_i8 only "
+                    "(constant / random operand bytes), and with LDS fragment reads, global->LDS copies and a barrier "
+                    "per step on random bytes (lds_fed); the published peak stays the denominator of frac"}
     if not args.sweep_only:
         # per-case launch durations, upstream's protocol; HBM-bound cases rotate weight copies (> 256 MB in total)
         table = []

@@ -58,6 +58,16 @@ int64_t ti_linear_workspace_bytes(int64_t M, int64_t N, int64_t K);
  * "skinny", "tile_*", "scalar"; "" before the first call).  Benchmarks use it to label their rows. */
 const char* ti_last_kernel(void);
 
+/* Diagnostic (no counterpart in the reference; computes nothing): one launch that issues the instruction mix of
+ * the tiled GEMM mainloop `iters` times per wave on the first MiB of `data` (device memory, at least 1 MiB, 16-byte
+ * aligned), so that a benchmark can measure what the matrix pipe of this board sustains for a given operand
+ * pattern (fill `data` with a constant or with random bytes).  mode 0: v_mfma_i32_32x32x32_i8 only; 1: plus the
+ * LDS fragment reads; 2: plus global->LDS copies from an L2-resident source and a workgroup barrier per step.
+ * `sink` is one int32 of device memory (written only if the accumulators hit a magic value).
+ * ti_diag_mfma_loop_ops(iters) = integer operations one such launch performs on the current device. */
+int ti_diag_mfma_loop(int mode, const int8_t* data, int64_t data_bytes, int64_t iters, int32_t* sink, void* stream);
+int64_t ti_diag_mfma_loop_ops(int64_t iters);
+
 /* ---- W8A8 linear: out[M,N] = epilogue(x[M,K] . w[N,K]^T, bias[N]) ---- */
 
 /* replaces linear_a8_w8_b32_o32 (torch_int/kernels/linear.cu:13-136;

@@ -724,3 +724,20 @@ def test_runs_are_deterministic():
     for _ in range(5):
         assert torch.equal(C.linear_a8_w8_b8_o8(x, w, b, 0.002, 0.01), first)
         assert torch.equal(C.linear_a8_w8_b32_o32(x, w, b.to(torch.int32)), first32)
+
+
+def test_diag_mfma_loop_runs_and_reports_its_work():
+    # the diagnostic loop behind bench.py's measured ceiling: every mode launches, exits and counts its operations
+    import torch_int._hip_ext as X
+    data = torch.randint(-127, 128, (1 << 20,), dtype=torch.int8, device=DEV)
+    sink = torch.zeros(1, dtype=torch.int32, device=DEV)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    for mode in (0, 1, 2):
+        _say(f"diag_mfma_loop mode {mode}")
+        ops = X.diag_mfma_loop(mode, data, 200, sink)
+        torch.cuda.synchronize()
+        assert ops == cus * 8 * 200 * 16 * 65536
+    with pytest.raises(RuntimeError):
+        X.diag_mfma_loop(3, data, 200, sink)
+    with pytest.raises(RuntimeError):
+        X.diag_mfma_loop(0, data[: 1 << 19], 200, sink)

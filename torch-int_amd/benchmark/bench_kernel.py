@@ -9,6 +9,9 @@ Examples
   python torch-int_amd/benchmark/bench_kernel.py --op bmm_s8t_rowmajor --shape 288 1 128 544
   python torch-int_amd/benchmark/bench_kernel.py --op linear_b8_o8 --shape 1 20480 5120 --rotate 4   # cache-cold weights
   python torch-int_amd/benchmark/bench_kernel.py --op copy --shape 268435456      # bytes; counter calibration
+  python torch-int_amd/benchmark/bench_kernel.py --op mfma_loop --shape 2 20000 --pattern random --iters 200
+      # matrix-pipe ceiling: mode (0 MFMA only, 1 + LDS reads, 2 + LDS-DMA copies and barrier), steps per wave
+  python torch-int_amd/benchmark/bench_kernel.py --op mfma_ceiling --shape 250    # all six figures, 250 ms windows
   rocprofv3 --kernel-trace --stats --output-format csv -d out -- python3 .../bench_kernel.py --op ...
 
 Prints one JSON line: mean microseconds per call (HIP events on the launch stream), algorithmic
@@ -38,7 +41,8 @@ LINEAR = {
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--op", required=True, choices=list(LINEAR) + ["bmm_f32t", "bmm_s8t", "bmm_s32t", "bmm_s8t_rowmajor", "ln_q", "add_ln_q",
-                                               "softmax_q", "qk_softmax_q", "attn_prefill", "decode_attn", "copy"])
+                                               "softmax_q", "qk_softmax_q", "attn_prefill", "decode_attn", "copy",
+                                               "mfma_loop", "mfma_ceiling"])
     ap.add_argument("--shape", type=int, nargs="+", required=True)
     ap.add_argument("--iters", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
@@ -46,8 +50,14 @@ def main():
     ap.add_argument("--beta", type=float, default=0.01)
     ap.add_argument("--rotate", type=int, default=1,
                     help="copies of the large read-only operand used round-robin (defeats the 256 MB last-level cache)")
+    ap.add_argument("--pattern", choices=["constant", "random"], default="random",
+                    help="operand bytes of --op mfma_loop")
     args = ap.parse_args()
     dev = torch.device("cuda:0")
+    if args.op == "mfma_ceiling":
+        print(json.dumps({"op": args.op, "window_ms": args.shape[0], "TOPS": X.measure_mfma_ceiling(float(args.shape[0]))}),
+              flush=True)
+        return
     g = torch.Generator(device=dev).manual_seed(0)
 
     def s8(*shape, lo=-127):
@@ -148,6 +158,13 @@ def main():
         gamma, beta = torch.ones(H, device=dev), torch.zeros(H, device=dev)
         fn = lambda: C.dq_add_layernorm_q(inp, 0.01, res, gamma, beta, 1e-5)  # noqa: E731
         nbytes = 13.0 * rows * H + 8 * H
+    elif args.op == "mfma_loop":
+        mode, steps = args.shape
+        data = (torch.full((1 << 20,), 1, dtype=torch.int8, device=dev) if args.pattern == "constant"
+                else s8(1 << 20))
+        sink = torch.zeros(1, dtype=torch.int32, device=dev)
+        ops = float(X.diag_mfma_loop(mode, data, steps, sink))
+        fn = lambda: X.diag_mfma_loop(mode, data, steps, sink)  # noqa: E731
     else:  # plain device copy of a known size: reference reading for FETCH_SIZE / WRITE_SIZE
         n, = args.shape
         src = torch.empty(n, dtype=torch.uint8, device=dev).random_(generator=g)

@@ -12,7 +12,12 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "torch_int", "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libtorch_int_hip.so")
-SOURCES = ["api.hip", "gemm_s8.hip", "ln_q.hip", "softmax_q.hip", "permute.hip", "bmm_rowmajor.hip", "decode_attn.hip", "attn_fused.hip"]
+# (source, extra defines, object name).  The GEMM kernels are compiled once per epilogue kind (EpiKind 0..8 of
+# csrc/ti_common.h), each kind in a translation unit of its own, so that they build in parallel.
+SOURCES = [(s, [], s[:-4] + ".o") for s in
+           ["api.hip", "gemm_s8.hip", "ln_q.hip", "softmax_q.hip", "permute.hip", "bmm_rowmajor.hip", "decode_attn.hip",
+            "attn_fused.hip", "diag_mfma.hip"]]
+SOURCES += [("gemm_s8_kinds.hip", [f"-DTI_KIND={k}"], f"gemm_s8_kind{k}.o") for k in range(9)]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -43,9 +48,10 @@ def build(verbose=True, extra_flags=()):
     obj_dir = os.path.join(HERE, "build")
     os.makedirs(obj_dir, exist_ok=True)
 
-    def compile_one(src):
-        obj = os.path.join(obj_dir, os.path.splitext(src)[0] + ".o")
-        cmd = [HIPCC, *FLAGS, *extra_flags, "-c", os.path.join(CSRC, src), "-o", obj]
+    def compile_one(item):
+        src, defines, name = item
+        obj = os.path.join(obj_dir, name)
+        cmd = [HIPCC, *FLAGS, *defines, *extra_flags, "-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         subprocess.check_call(cmd)

@@ -1,0 +1,119 @@
+// Diagnostic, not part of any operator: loops that issue the instruction mix of the tiled INT8 GEMM mainloop
+// on operands that never change, to measure what the matrix pipe sustains on this board with a given operand
+// pattern (the caller fills `data`: a constant byte, or uniformly random bytes).  No result is produced; the
+// accumulators are only folded into a value that is never stored unless it hits a magic number.
+//
+// One workgroup of 8 waves per CU, two waves per SIMD, as the 256x256-tile kernel runs.  Per step a wave issues
+// 16 v_mfma_i32_32x32x32_i8 (a 128x64 wave tile over 64 bytes of K) and, depending on the mode,
+//   mode 0  nothing else                                       -> the matrix pipe alone
+//   mode 1  + 12 ds_read_b128 fragment reads, waited for       -> operands fed from LDS
+//   mode 2  + 4 x 1 KiB global->LDS copies from a source that stays in L2 (1 MiB shared by all
+//             workgroups), a wait that leaves the newest three steps of copies in flight, and a
+//             workgroup barrier                                 -> the whole mainloop without the epilogue
+#include "ti_common.h"
+
+namespace ti {
+
+#define TI_GLOBAL_AS __attribute__((address_space(1)))
+#define TI_LDS_AS __attribute__((address_space(3)))
+
+static constexpr int kDiagLds = 128 * 1024;
+
+template <int MODE>
+__global__ __launch_bounds__(512, 2) void mfma_loop_kernel(const int8_t* __restrict__ data, int iters, int* sink) {
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const char* g = reinterpret_cast<const char*>(data);
+  // the lower half of the LDS holds the bytes the fragment reads fetch; the upper half receives the copies
+  for (int i = threadIdx.x; i < 65536 / 16; i += 512)
+    *reinterpret_cast<v4i*>(smem + i * 16) = *reinterpret_cast<const v4i*>(g + (size_t)i * 16);
+  __syncthreads();
+  v16i acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) acc[i][j] = 0;
+  v4i a[2][8], b[2][4];
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+#pragma unroll
+    for (int r = 0; r < 8; ++r)
+      a[s][r] = *reinterpret_cast<const v4i*>(g + ((size_t)(wave * 12 + r) * 64 + lane) * 16 + s * 131072);
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      b[s][r] = *reinterpret_cast<const v4i*>(g + ((size_t)(wave * 12 + 8 + r) * 64 + lane) * 16 + s * 131072);
+  }
+  const int rd_base = lane * 16 + (wave & 3) * 1024;
+  const size_t goff = (size_t)(blockIdx.x % 8) * 131072 + wave * 4096 + lane * 16;  // 1 MiB in all: stays in L2
+#define TI_MF(ai, bi, ci, S) \
+  asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+v"(acc[ci]) : "v"(a[S][ai]), "v"(b[S][bi]))
+#define TI_RD(dst, off)                                                                          \
+  if (MODE >= 1) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(rd_base), "n"(off))
+#define TI_STEP(S, T)                                                                                          \
+  {                                                                                                            \
+    if (MODE == 2) {                                                                                           \
+      _Pragma("unroll") for (int j = 0; j < 4; ++j) __builtin_amdgcn_global_load_lds(                         \
+          (const TI_GLOBAL_AS void*)(g + goff + j * 1024),                                                     \
+          (TI_LDS_AS void*)((TI_LDS_AS char*)smem + 65536 + (S * 8 + wave) * 4096 + j * 1024), 16, 0, 0); \
+    }                                                                                                          \
+    TI_MF(0, 0, 0, S); TI_RD(a[T][0], 0);     TI_MF(1, 0, 1, S); TI_RD(a[T][1], 4096);                         \
+    TI_MF(2, 0, 2, S); TI_RD(a[T][2], 8192);  TI_MF(3, 0, 3, S); TI_RD(a[T][3], 12288);                        \
+    TI_MF(0, 1, 4, S); TI_RD(b[T][0], 16384); TI_MF(1, 1, 5, S); TI_RD(b[T][1], 20480);                        \
+    TI_MF(2, 1, 6, S); TI_RD(a[T][4], 24576); TI_MF(3, 1, 7, S); TI_RD(a[T][5], 28672);                        \
+    TI_MF(4, 2, 0, S); TI_RD(a[T][6], 32768); TI_MF(5, 2, 1, S); TI_RD(a[T][7], 36864);                        \
+    TI_MF(6, 2, 2, S); TI_RD(b[T][2], 40960); TI_MF(7, 2, 3, S); TI_RD(b[T][3], 45056);                        \
+    TI_MF(4, 3, 4, S); TI_MF(5, 3, 5, S); TI_MF(6, 3, 6, S); TI_MF(7, 3, 7, S);                                \
+    if (MODE >= 1) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                                          \
+    if (MODE == 2) asm volatile("s_waitcnt vmcnt(12)\n\ts_barrier" ::: "memory");                              \
+  }
+  for (int it = 0; it < iters; it += 2) {
+    TI_STEP(0, 1)
+    TI_STEP(1, 0)
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  int s = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) s += acc[i][j];
+  if (s == 0x12345678) sink[0] = 1;
+#undef TI_STEP
+#undef TI_RD
+#undef TI_MF
+}
+
+static int diag_grid() {
+  int dev = 0, count = 0;
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || count <= 0)
+    count = 256;
+  return count;
+}
+
+long long diag_mfma_loop_ops(long long iters) {
+  // workgroups x 8 waves x steps x 16 instructions x (32 x 32 x 32 multiply-adds = 2 ops each)
+  return (long long)diag_grid() * 8 * iters * 16 * 65536;
+}
+
+template <int MODE>
+static int launch_mfma_loop(const int8_t* data, int iters, int* sink, hipStream_t stream) {
+  auto kern = mfma_loop_kernel<MODE>;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     kDiagLds);
+  if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+  hipLaunchKernelGGL(kern, dim3(diag_grid()), dim3(512), kDiagLds, stream, data, iters, sink);
+  e = hipGetLastError();
+  if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "mfma loop launch: %s", hipGetErrorString(e));
+  return TI_OK;
+}
+
+int launch_diag_mfma_loop(int mode, const int8_t* data, long long iters, int* sink, hipStream_t stream) {
+  switch (mode) {
+    case 0: return launch_mfma_loop<0>(data, (int)iters, sink, stream);
+    case 1: return launch_mfma_loop<1>(data, (int)iters, sink, stream);
+    case 2: return launch_mfma_loop<2>(data, (int)iters, sink, stream);
+  }
+  return fail(TI_ERR_INVALID_ARG, "diag_mfma_loop: mode must be 0, 1 or 2 (got %d)", mode);
+}
+
+}  // namespace ti

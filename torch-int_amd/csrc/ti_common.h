@@ -233,6 +233,10 @@ int launch_decode_attn_s8(const int8_t* q, const int8_t* k_new, const int8_t* v_
 int launch_kv_append_s8(const int8_t* knew, const int8_t* vnew, int8_t* kbuf, int8_t* vbuf, long long BH, long long T,
                         long long D, long long cap, long long S, hipStream_t stream);
 
+// diag_mfma.hip
+int launch_diag_mfma_loop(int mode, const int8_t* data, long long iters, int* sink, hipStream_t stream);
+long long diag_mfma_loop_ops(long long iters);
+
 // bmm_rowmajor.hip
 int launch_bmm_s8t_s8t_s8t(const int8_t* a, const int8_t* b, int8_t* c, long long batch, long long M, long long N,
                            long long K, long long stride_b, float alpha, hipStream_t stream);

@@ -55,6 +55,10 @@ _lib.ti_linear_a8_w8_b8_o8_group.restype = ctypes.c_int
 _lib.ti_linear_a8_w8_b8_o8_group_heads.argtypes = [_vp, _pp, _pp, _pp, ctypes.POINTER(_f32), ctypes.POINTER(_f32), _i64,
                                                    _i64, _i64, _i64, _i64, _i64, _vp]
 _lib.ti_linear_a8_w8_b8_o8_group_heads.restype = ctypes.c_int
+_lib.ti_diag_mfma_loop.argtypes = [ctypes.c_int, _vp, _i64, _i64, _vp, _vp]
+_lib.ti_diag_mfma_loop.restype = ctypes.c_int
+_lib.ti_diag_mfma_loop_ops.argtypes = [_i64]
+_lib.ti_diag_mfma_loop_ops.restype = _i64
 _raw_stream = torch._C._cuda_getCurrentRawStream
 _fast = _CUDA._fast if getattr(_CUDA._fast, "kv_append", None) is not None else None
 _fast_decode_attn = getattr(_CUDA._fast, "decode_attn", None)
@@ -506,4 +510,50 @@ def linear_a8_w8_b8_o8_heads(x, w, bias, alpha, beta, bsz, seq_len, heads, head_
                                               stream or None)
     if rc:
         raise RuntimeError(f"torch_int._hip_ext.linear_a8_w8_b8_o8_heads: {_lib.ti_last_error().decode()} (status {rc})")
+    return out
+
+
+def diag_mfma_loop(mode, data, iters, sink):
+    """Diagnostic launch (computes nothing): the mainloop's instruction mix ``iters`` times per wave on the bytes of
+    ``data`` (uint8 / int8 HIP tensor of at least 1 MiB); mode 0 = MFMA only, 1 = + LDS fragment reads, 2 = + global->LDS
+    copies and a barrier per step.  ``sink`` is an int32 HIP tensor of one element.  Returns the integer operations
+    the launch performs."""
+    if not (isinstance(data, torch.Tensor) and data.is_cuda and data.is_contiguous() and data.element_size() == 1):
+        raise RuntimeError("torch_int._hip_ext.diag_mfma_loop: data must be a contiguous one-byte HIP tensor")
+    if not (_ok(sink, torch.int32) and sink.numel() >= 1 and sink.device == data.device):
+        raise RuntimeError("torch_int._hip_ext.diag_mfma_loop: sink must be an int32 HIP tensor on the same device")
+    with _on(data.device):
+        rc = _lib.ti_diag_mfma_loop(int(mode), data.data_ptr(), data.numel(), int(iters), sink.data_ptr(),
+                                    _raw_stream(data.device.index) or None)
+        ops = int(_lib.ti_diag_mfma_loop_ops(int(iters)))
+    if rc:
+        raise RuntimeError(f"torch_int._hip_ext.diag_mfma_loop: {_lib.ti_last_error().decode()} (status {rc})")
+    return ops
+
+
+def measure_mfma_ceiling(window_ms=250.0, iters=20000):
+    """What the int8 matrix pipe of the current device sustains, in TOP/s, for the three loop modes of
+    ``diag_mfma_loop`` on constant and on uniformly random operand bytes: back-to-back launches between two HIP
+    events for at least ``window_ms`` per figure (after the same again as warm-up, so the clocks have settled under
+    the board's power limit)."""
+    dev = torch.device("cuda", torch.cuda.current_device())
+    sink = torch.zeros(1, dtype=torch.int32, device=dev)
+    patterns = {"constant": torch.full((1 << 20,), 1, dtype=torch.int8, device=dev),
+                "random": torch.randint(-127, 128, (1 << 20,), dtype=torch.int8, device=dev)}
+    out = {}
+    for mode, label in ((0, "mfma_only"), (1, "lds_reads"), (2, "lds_fed")):
+        for pname, data in patterns.items():
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            ops = diag_mfma_loop(mode, data, iters, sink)
+            end.record()
+            torch.cuda.synchronize()
+            n = max(2, int(window_ms / max(start.elapsed_time(end), 1e-3)) + 1)
+            for timed in (False, True):
+                start.record()
+                for _ in range(n):
+                    diag_mfma_loop(mode, data, iters, sink)
+                end.record()
+                torch.cuda.synchronize()
+            out[f"{label}_{pname}"] = ops * n / start.elapsed_time(end) / 1e9
     return out
