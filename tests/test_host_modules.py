@@ -9,6 +9,9 @@ import pytest
 import torch
 from torch import nn
 
+from _float_opt import FloatOPTAttention as _FloatOPTAttention
+from _float_opt import FloatOPTDecoderLayer as _FloatOPTDecoderLayer
+from _float_opt import clone_linear as _clone_linear
 from _oracle_backend import causal_mask, oracle_backend, randomize_int8_layer
 from oracle import oracle as orc
 from torch_int.models.opt import (Int8OPTAttention, Int8OPTDecoder, Int8OPTDecoderLayer, Int8OPTForCausalLM,
@@ -206,66 +209,6 @@ def test_linear_from_float_algebra_and_accuracy():
         assert m.bias.dtype == torch.int32
         r2 = ((y_gt - m(q_x).float() * y_scale) ** 2).mean() / (y_gt ** 2).mean()
         assert r2 < 1e-3, r2.item()
-
-
-def _clone_linear(lin):
-    c = nn.Linear(lin.in_features, lin.out_features)
-    c.load_state_dict(lin.state_dict())
-    return c.requires_grad_(False)
-
-
-class _FloatOPTAttention(nn.Module):
-    """Plain fp32 OPT self-attention (attribute names the int8 converter reads)."""
-
-    def __init__(self, embed_dim, num_heads):
-        super().__init__()
-        self.embed_dim, self.num_heads, self.head_dim = embed_dim, num_heads, embed_dim // num_heads
-        self.scaling = self.head_dim ** -0.5
-        self.q_proj, self.k_proj = nn.Linear(embed_dim, embed_dim), nn.Linear(embed_dim, embed_dim)
-        self.v_proj, self.out_proj = nn.Linear(embed_dim, embed_dim), nn.Linear(embed_dim, embed_dim)
-
-    def forward(self, x, mask=None):
-        B, T, D = x.shape
-        H, d = self.num_heads, self.head_dim
-        q = (self.q_proj(x) * self.scaling).view(B, T, H, d).transpose(1, 2)
-        k = self.k_proj(x).view(B, T, H, d).transpose(1, 2)
-        v = self.v_proj(x).view(B, T, H, d).transpose(1, 2)
-        s = q @ k.transpose(-1, -2)
-        if mask is not None:
-            s = s + mask
-        p = torch.softmax(s, -1)
-        return self.out_proj((p @ v).transpose(1, 2).reshape(B, T, D))
-
-
-class _FloatOPTDecoderLayer(nn.Module):
-    def __init__(self, embed_dim, num_heads, ffn_dim):
-        super().__init__()
-        self.embed_dim = embed_dim
-        self.self_attn = _FloatOPTAttention(embed_dim, num_heads)
-        self.self_attn_layer_norm, self.final_layer_norm = nn.LayerNorm(embed_dim), nn.LayerNorm(embed_dim)
-        self.fc1, self.fc2 = nn.Linear(embed_dim, ffn_dim), nn.Linear(ffn_dim, embed_dim)
-
-    def forward(self, x, mask=None, record=None):
-        h = self.self_attn_layer_norm(x)
-        if record is not None:
-            record["attn_input_scale"] = h.abs().max().item() / 127
-            a = self.self_attn
-            record["q_output_scale"] = a.q_proj(h).abs().max().item() / 127
-            record["k_output_scale"] = a.k_proj(h).abs().max().item() / 127
-            record["v_output_scale"] = a.v_proj(h).abs().max().item() / 127
-            B, T, D = h.shape
-            q = (a.q_proj(h) * a.scaling).view(B, T, a.num_heads, a.head_dim).transpose(1, 2)
-            k = a.k_proj(h).view(B, T, a.num_heads, a.head_dim).transpose(1, 2)
-            v = a.v_proj(h).view(B, T, a.num_heads, a.head_dim).transpose(1, 2)
-            s = q @ k.transpose(-1, -2) + (mask if mask is not None else 0)
-            ctx = (torch.softmax(s, -1) @ v).transpose(1, 2).reshape(B, T, D)
-            record["out_input_scale"] = ctx.abs().max().item() / 127
-        x = x + self.self_attn(h, mask)
-        h = self.final_layer_norm(x)
-        if record is not None:
-            record["fc1_input_scale"] = h.abs().max().item() / 127
-            record["fc2_input_scale"] = torch.relu(self.fc1(h)).abs().max().item() / 127
-        return x + self.fc2(torch.relu(self.fc1(h)))
 
 
 @torch.no_grad()
@@ -496,3 +439,25 @@ def test_decode_with_in_place_cache_matches_concatenation():
     for (k1, v1), (k2, v2) in zip(outs[True][1], outs[False][1]):
         assert k1.shape[2] == 20 and torch.equal(k1, k2) and torch.equal(v1, v2)  # 5 tokens padded to 16, then 4 steps
         assert not k1.is_contiguous() and k2.is_contiguous()
+
+
+def test_causal_lm_ties_lm_head_and_loads_a_checkpoint_without_it():
+    # upstream's post_init ties lm_head to the token embedding; exported checkpoints store the tensor once
+    cfg = OPTConfigLite(hidden_size=32, num_hidden_layers=1, ffn_dim=64, num_attention_heads=4, vocab_size=60,
+                        max_position_embeddings=64)
+    torch.manual_seed(0)
+    lm = Int8OPTForCausalLM(cfg)
+    assert lm.lm_head.weight is lm.model.decoder.embed_tokens.weight
+    sd = {k: v.clone() for k, v in lm.state_dict().items() if k != "lm_head.weight"}
+    torch.manual_seed(1)
+    other = Int8OPTForCausalLM(cfg)
+    res = other.load_state_dict(sd, strict=True)
+    assert not res.missing_keys and not res.unexpected_keys
+    assert torch.equal(other.lm_head.weight, lm.model.decoder.embed_tokens.weight)
+    assert other.lm_head.weight is other.model.decoder.embed_tokens.weight
+    # a checkpoint that does carry an untied head keeps it apart when the config says so
+    cfg2 = OPTConfigLite(hidden_size=32, num_hidden_layers=1, ffn_dim=64, num_attention_heads=4, vocab_size=60,
+                         max_position_embeddings=64)
+    cfg2.tie_word_embeddings = False
+    untied = Int8OPTForCausalLM(cfg2)
+    assert untied.lm_head.weight is not untied.model.decoder.embed_tokens.weight

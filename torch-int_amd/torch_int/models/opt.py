@@ -570,6 +570,17 @@ class Int8OPTForCausalLM(nn.Module):
         self.config = config
         self.model = Int8OPTModel(config)
         self.lm_head = nn.Linear(config.word_embed_proj_dim, config.vocab_size, bias=False)
+        # Upstream's post_init ties the output projection to the token embedding (OPTConfig.tie_word_embeddings
+        # defaults to True), and exported checkpoints then carry no ``lm_head.weight``.
+        if getattr(config, "tie_word_embeddings", True):
+            self.lm_head.weight = self.model.decoder.embed_tokens.weight
+        self._register_load_state_dict_pre_hook(self._fill_tied_lm_head)
+
+    def _fill_tied_lm_head(self, state_dict, prefix, *unused):
+        """A state dict without ``lm_head.weight`` (tied weights are stored once) loads the embedding there."""
+        head, emb = prefix + "lm_head.weight", prefix + "model.decoder.embed_tokens.weight"
+        if head not in state_dict and emb in state_dict and self.lm_head.weight.shape == state_dict[emb].shape:
+            state_dict[head] = state_dict[emb]
 
     @staticmethod
     def from_float(module, decoder_layer_scales):
