@@ -171,6 +171,18 @@ int ti_dq_add_layernorm_q(const int32_t* input, float input_scale, const float* 
                           const float* gamma, const float* beta, float eps,
                           float* r_out, int8_t* q_out, int64_t rows, int64_t H, void* stream);
 
+/* dq_add_layernorm_q on an fp16 residual stream with fp16 gamma and beta (the reference's op is ATen and takes
+ * them: torch_int/kernels/fused.cu:17-24, called that way by benchmark/bench_dq_add_ln_q.py:37-45).  residual,
+ * gamma, beta and r_out point to IEEE binary16 values.  The arithmetic is fp32 and rounds where the reference's
+ * chain of torch ops on fp16 tensors rounds:
+ *   r_out = f16(fmaf(input_scale, float(f16(input)), float(residual)))     (|input| >= 65520 -> infinity)
+ *   y     = f16(LN(float(r_out))[i] * float(gamma[i]) + float(beta[i]))
+ *   q_out = s8(rint(clamp(float(y), -128, 127)))
+ * r_out may alias residual. */
+int ti_dq_add_layernorm_q_f16(const int32_t* input, float input_scale, const void* residual, const void* gamma,
+                              const void* beta, float eps, void* r_out, int8_t* q_out, int64_t rows, int64_t H,
+                              void* stream);
+
 /* ---- fused element-wise chains of the OPT blocks (no counterpart in the reference's native
  * module: upstream runs these as sequences of torch ops) ---- */
 
@@ -188,6 +200,12 @@ int ti_linear_a8_w8_bfp32_ofp32_acc(const int8_t* x, const int8_t* w, const floa
  * LayerNormQ.forward on fp32 input (torch_int/nn/fused.py:13-18). */
 int ti_add_layernorm_q(const float* x, float* residual, const float* gamma, const float* beta, float eps,
                        int8_t* q_out, int64_t rows, int64_t H, void* stream);
+
+/* ti_add_layernorm_q on an fp16 residual stream with fp16 x, gamma and beta (LayerNormQ of a model converted
+ * with .half(), torch_int/nn/fused.py:13-18): residual = f16(float(residual) + float(x)) in place when x != NULL,
+ * then y = f16(LN(float(residual)) * gamma + beta), q_out = s8(rint(clamp(float(y), -128, 127))). */
+int ti_add_layernorm_q_f16(const void* x, void* residual, const void* gamma, const void* beta, float eps,
+                           int8_t* q_out, int64_t rows, int64_t H, void* stream);
 
 /* probs[b*heads+h, t, s] = s8(rint(127 * softmax_s(max(scores[b*heads+h,t,s] + mask[b,0,t,s], -FLT_MAX))));
  * scores [batch*heads, T, S] fp32, mask [batch, 1, T, S] fp32 or NULL.

@@ -200,6 +200,49 @@ def dq_add_layernorm_q(inp, input_scale, residual, gamma, beta, eps):
     return r, q
 
 
+def _ln_f16(mode, inp, scale, residual, gamma, beta, eps):
+    residual = _chk(residual, torch.float16, "residual")
+    gamma = _chk(gamma, torch.float16, "gamma")
+    beta = _chk(beta, torch.float16, "beta")
+    H = residual.shape[-1]
+    rows = residual.numel() // H if H else 0
+    assert gamma.numel() == H and beta.numel() == H
+    r = torch.empty_like(residual)
+    q = torch.empty(residual.shape, dtype=torch.int8)
+    _load().orc_layernorm_q_f16(ctypes.c_int(mode), _p(inp) if inp is not None else None, _f32(scale), _p(residual),
+                                _p(gamma), _p(beta), _f32(eps), _p(r), _p(q), _i64(rows), _i64(H))
+    return r, q
+
+
+def dq_add_layernorm_q_f16(inp, input_scale, residual, gamma, beta, eps):
+    """dq_add_layernorm_q on fp16 residual / gamma / beta: (fp16 residual output, int8)."""
+    inp = _chk(inp, torch.int32, "input")
+    assert inp.shape == residual.shape
+    return _ln_f16(0, inp, input_scale, residual, gamma, beta, eps)
+
+
+def add_layernorm_q_f16(x, residual, gamma, beta, eps):
+    """add_layernorm_q on fp16 tensors; x may be None."""
+    if x is None:
+        return _ln_f16(2, None, 1.0, residual, gamma, beta, eps)
+    x = _chk(x, torch.float16, "x")
+    assert x.shape == residual.shape
+    return _ln_f16(1, x, 1.0, residual, gamma, beta, eps)
+
+
+def f16_round_trip(x):
+    """fp32 tensor -> (uint16 bit patterns of the oracle's fp16 conversion, and their fp32 values)."""
+    x = _chk(x, torch.float32, "x")
+    lib = _load()
+    lib.orc_f16_of_f32.restype = ctypes.c_uint16
+    lib.orc_f16_of_f32.argtypes = [ctypes.c_float]
+    lib.orc_f32_of_f16.restype = ctypes.c_float
+    lib.orc_f32_of_f16.argtypes = [ctypes.c_uint16]
+    bits = [lib.orc_f16_of_f32(float(v)) for v in x.reshape(-1).tolist()]
+    back = [lib.orc_f32_of_f16(b) for b in bits]
+    return torch.tensor(bits, dtype=torch.int32), torch.tensor(back, dtype=torch.float32)
+
+
 # ---- fused chains of the OPT blocks (ti_add_layernorm_q / ti_attn_softmax_q) ----
 
 def add_layernorm_q(x, residual, gamma, beta, eps):

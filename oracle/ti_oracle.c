@@ -258,6 +258,79 @@ void orc_dq_add_layernorm_q(const int32_t* in, float scale, const float* res,
   }
 }
 
+/* IEEE binary16 <-> binary32 in integer arithmetic (gcc 11 on x86 has no _Float16): round to nearest even,
+ * subnormals kept, overflow to infinity -- what a GPU's fp32->fp16 conversion and torch's .half() do. */
+float orc_f32_of_f16(uint16_t h) {
+  uint32_t sign = (uint32_t)(h & 0x8000u) << 16, e = (h >> 10) & 31u, m = h & 0x3ffu, bits;
+  if (e == 31u) {
+    bits = sign | 0x7f800000u | (m << 13);
+  } else if (e != 0u) {
+    bits = sign | ((e + 112u) << 23) | (m << 13);
+  } else if (m == 0u) {
+    bits = sign;
+  } else { /* subnormal: m * 2^-24 */
+    int shift = 0;
+    while (!(m & 0x400u)) { m <<= 1; ++shift; }
+    bits = sign | ((uint32_t)(113 - shift) << 23) | ((m & 0x3ffu) << 13);
+  }
+  float f;
+  memcpy(&f, &bits, 4);
+  return f;
+}
+
+uint16_t orc_f16_of_f32(float f) {
+  uint32_t x;
+  memcpy(&x, &f, 4);
+  uint16_t sign = (uint16_t)((x >> 16) & 0x8000u);
+  uint32_t absx = x & 0x7fffffffu;
+  if (absx >= 0x7f800000u) return (uint16_t)(sign | (absx > 0x7f800000u ? 0x7e00u : 0x7c00u)); /* NaN, inf */
+  if (absx >= 0x477ff000u) return (uint16_t)(sign | 0x7c00u); /* rounds to >= 65520: overflow */
+  if (absx < 0x33000001u) return sign;                        /* <= 2^-25: rounds to zero (the tie goes to even) */
+  int32_t e = (int32_t)(absx >> 23) - 127;
+  uint32_t man = (absx & 0x7fffffu) | 0x800000u; /* 24 bits */
+  int drop = e >= -14 ? 13 : 13 + (-14 - e);     /* bits to discard */
+  uint32_t kept = man >> drop, rest = man & ((1u << drop) - 1u), half = 1u << (drop - 1);
+  if (rest > half || (rest == half && (kept & 1u))) ++kept;
+  /* normal: kept has 11 bits (or 12 after a carry); subnormal: kept is the 10-bit field (a carry makes it normal) */
+  uint32_t out = e >= -14 ? ((uint32_t)(e + 14) << 10) + kept : kept;
+  return (uint16_t)(sign | out);
+}
+
+static inline float round_f16(float x) { return orc_f32_of_f16(orc_f16_of_f32(x)); }
+
+/* dq_add_layernorm_q and the add + LayerNormQ chain on fp16 tensors (torch_int/kernels/fused.cu:17-24 called
+ * with fp16 residual / gamma / beta as in benchmark/bench_dq_add_ln_q.py:37-45; torch_int/nn/fused.py:13-18 on a
+ * model converted with .half()).  The torch ops compute in fp32 and round each tensor they produce to fp16:
+ *   r = f16(fmaf(s, f32(f16(in)), f32(res)))   or   r = f16(f32(res) + f32(x))   or   r = res (x == NULL, mode 2)
+ *     (torch.add casts its int32 operand to the common dtype, fp16, before the fp32 arithmetic: observed on the
+ *      device, where it matches on every element; |in| >= 65520 becomes infinity)
+ *   y = f16(fmaf((f32(r) - mean) * rstd, f32(gamma), f32(beta)))   mean / rstd from the fixed tree over f32(r)
+ *   q = s8(rne(clamp(f32(y), -128, 127)))
+ * mode 0: dequantise + add (`in` int32); 1: add (`in` fp16 x); 2: plain.  r_out may be NULL in mode 2. */
+void orc_layernorm_q_f16(int mode, const void* in, float scale, const uint16_t* res, const uint16_t* gamma,
+                         const uint16_t* beta, float eps, uint16_t* r_out, int8_t* q_out, int64_t rows, int64_t H) {
+#pragma omp parallel for schedule(static)
+  for (int64_t row = 0; row < rows; ++row) {
+    float* r = (float*)malloc(sizeof(float) * (size_t)(H > 0 ? H : 1));
+    for (int64_t i = 0; i < H; ++i) {
+      float a = orc_f32_of_f16(res[row * H + i]);
+      if (mode == 0) r[i] = round_f16(fmaf(scale, round_f16(f32_of_i32(((const int32_t*)in)[row * H + i])), a));
+      else if (mode == 1) r[i] = round_f16(a + orc_f32_of_f16(((const uint16_t*)in)[row * H + i]));
+      else r[i] = a;
+    }
+    float fH = (float)H;
+    float mu = tree_sum(r, H, 0, 0.0f) / fH;
+    float var = tree_sum(r, H, 1, mu) / fH;
+    float rstd = 1.0f / sqrtf(var + eps);
+    for (int64_t i = 0; i < H; ++i) {
+      float y = fmaf((r[i] - mu) * rstd, orc_f32_of_f16(gamma[i]), orc_f32_of_f16(beta[i]));
+      q_out[row * H + i] = sat_rne_s8(round_f16(y));
+      if (r_out) r_out[row * H + i] = orc_f16_of_f32(r[i]);
+    }
+    free(r);
+  }
+}
+
 /* ------------------------------------------- fused chains of the OPT blocks */
 
 /* residual.add_(x) followed by LayerNormQ (torch_int/models/opt.py:281-283 and

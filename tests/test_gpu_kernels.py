@@ -741,3 +741,64 @@ def test_diag_mfma_loop_runs_and_reports_its_work():
         X.diag_mfma_loop(3, data, 200, sink)
     with pytest.raises(RuntimeError):
         X.diag_mfma_loop(0, data[: 1 << 19], 200, sink)
+
+
+def test_ln_q_fp16_residual_stream():
+    # dq_add_layernorm_q and add + LayerNormQ with fp16 residual / gamma / beta: bit-exact against the oracle's
+    # restatement, and within one LSB of the chain of torch ops on the same fp16 tensors on the device
+    import torch_int._CUDA as C
+    import torch_int._hip_ext as X
+    from torch_int.functional.fused import dq_add_layernorm_q_py
+    for i, shape in enumerate([(2, 3, 4), (7, 768), (4, 5, 5120), (3, 9216), (2, 12288), (5, 1023), (3, 1), (2, 16384),
+                               (2, 20000), (1, 18), (4, 512, 5120)]):
+        _say(f"ln_q fp16 shape={shape}")
+        g = torch.Generator().manual_seed(600 + i)
+        H = shape[-1]
+        inp = torch.randint(-60000, 60000, shape, dtype=torch.int32, generator=g)   # fp16 holds these (see below)
+        res = torch.randn(shape, generator=g).half()
+        gamma = ((1 + 0.02 * torch.randn(H, generator=g)) * 20).half()
+        beta = (0.4 * torch.randn(H, generator=g)).half()
+        s = _scal(g, 1e-4, 1e-2)
+        r_ref, q_ref = orc.dq_add_layernorm_q_f16(inp, s, res, gamma, beta, 1e-5)
+        r, q = C.dq_add_layernorm_q(inp.to(DEV), s, res.to(DEV), gamma.to(DEV), beta.to(DEV), 1e-5)
+        assert r.dtype == torch.float16 and q.dtype == torch.int8 and r.shape == shape and q.shape == shape
+        assert torch.equal(r.cpu().view(torch.int16), r_ref.view(torch.int16)), f"r {shape}"
+        assert (q.cpu() != q_ref).sum().item() == 0, f"q {shape}"
+        r_t, q_t = dq_add_layernorm_q_py(inp.to(DEV), s, res.to(DEV), gamma.to(DEV), beta.to(DEV), 1e-5)
+        assert r_t.dtype == torch.float16 and (r != r_t).float().mean().item() <= 1e-3 + 1.0 / r.numel()
+        assert (q.int() - q_t.int()).abs().max().item() <= 1
+        assert (q != q_t).float().mean().item() <= 0.01 + 1.0 / q.numel()
+        # residual.add_(x) + LayerNormQ on the fp16 stream, and LayerNormQ alone
+        x = torch.randn(shape, generator=g).half()
+        r2_ref, q2_ref = orc.add_layernorm_q_f16(x, res, gamma, beta, 1e-5)
+        d_res = res.to(DEV)
+        q2 = X.add_layernorm_q(x.to(DEV), d_res, gamma.to(DEV), beta.to(DEV), 1e-5)
+        assert torch.equal(d_res.cpu().view(torch.int16), r2_ref.view(torch.int16)) and (q2.cpu() != q2_ref).sum().item() == 0
+        q3 = X.add_layernorm_q(None, d_res, gamma.to(DEV), beta.to(DEV), 1e-5)
+        assert torch.equal(q3, q2) and torch.equal(d_res.cpu().view(torch.int16), r2_ref.view(torch.int16))
+    # int32 values beyond fp16's range become infinity, as in torch's own add: same bits as the oracle, NaN rows -> 0
+    inp = torch.tensor([[65519, 65520, -70000, 5], [1, 2, 3, 4]], dtype=torch.int32)
+    res4, g4, b4 = torch.randn(2, 4, generator=g).half(), torch.ones(4).half(), torch.zeros(4).half()
+    r_ref, q_ref = orc.dq_add_layernorm_q_f16(inp, 0.001, res4, g4, b4, 1e-5)
+    r, q = C.dq_add_layernorm_q(inp.to(DEV), 0.001, res4.to(DEV), g4.to(DEV), b4.to(DEV), 1e-5)
+    assert torch.isinf(r_ref[0, 1]) and torch.isinf(r_ref[0, 2]) and not torch.isinf(r_ref[0, 0])
+    assert torch.equal(r.cpu().view(torch.int16), r_ref.view(torch.int16)) and torch.equal(q.cpu(), q_ref)
+    assert torch.equal(r.cpu(), torch.add(res4.to(DEV), inp.to(DEV), alpha=0.001).cpu())
+    with pytest.raises(RuntimeError, match="share one dtype"):
+        C.dq_add_layernorm_q(inp.to(DEV), 0.001, res4.to(DEV), g4.float().to(DEV), b4.to(DEV), 1e-5)
+    # the modules: a LayerNormQ converted with .half(), and an fp16 input of an fp32 layer (promoted first)
+    from torch_int.nn.fused import LayerNormQ
+    ln = LayerNormQ(768)
+    ln.weight, ln.bias = torch.randn(768, generator=g) * 20, torch.randn(768, generator=g)
+    x16 = torch.randn(5, 768, generator=g).half()
+    q32 = copy_to(ln, DEV)(x16.to(DEV))
+    _, ref32 = orc.add_layernorm_q(None, x16.float(), ln.weight, ln.bias, 1e-5)
+    assert torch.equal(q32.cpu(), ref32)
+    q16 = copy_to(ln, DEV).half()(x16.to(DEV))
+    _, ref16 = orc.add_layernorm_q_f16(None, x16, ln.weight.half(), ln.bias.half(), 1e-5)
+    assert torch.equal(q16.cpu(), ref16)
+
+
+def copy_to(module, dev):
+    import copy
+    return copy.deepcopy(module).to(dev)

@@ -312,3 +312,60 @@ def test_attn_softmax_q_against_torch():
     # a fully masked row degenerates to the uniform distribution, like softmax of equal inputs
     q = orc.attn_softmax_q(torch.randn(1, 1, 8, generator=g), torch.full((1, 1, 1, 8), neg), 1)
     assert q.tolist() == [[[16] * 8]]  # round(127 / 8) = 16
+
+
+# ------------------------------------------------------------------ fp16 residual stream
+
+def test_f16_conversion_matches_numpy():
+    g = torch.Generator().manual_seed(0)
+    x = torch.cat([torch.randn(3000, generator=g) * torch.logspace(-9, 5.2, 3000),
+                   torch.tensor([0.0, -0.0, 65504.0, 65519.9, 65520.0, 65536.0, 1e9, -1e9, float("inf"), -float("inf"),
+                                 2.0 ** -24, 2.0 ** -25, 2.0 ** -25 * 1.0001, 2.0 ** -14, 2.0 ** -14 * 0.9999, 6.1e-5,
+                                 5.96e-8, 1.0009765625, 1.00048828125, 1.00146484375])])   # ties, subnormals, overflow
+    bits, back = orc.f16_round_trip(x)
+    with np.errstate(over="ignore"):
+        ref = x.numpy().astype(np.float16)
+    assert np.array_equal(bits.numpy().astype(np.uint16), ref.view(np.uint16))
+    assert np.array_equal(back.numpy(), ref.astype(np.float32))
+
+
+@pytest.mark.parametrize("shape", [(2, 3, 4), (5, 768), (3, 1023), (2, 5120)])
+def test_ln_q_f16_against_torch_ops_in_fp32(shape):
+    # the GPU chain of ATen ops on fp16 tensors computes in fp32 and rounds every tensor it produces to fp16
+    g = torch.Generator().manual_seed(sum(shape))
+    H = shape[-1]
+    inp = torch.randint(-60000, 60000, shape, dtype=torch.int32, generator=g)
+    res = torch.randn(shape, generator=g).half()
+    gamma = ((1 + 0.02 * torch.randn(H, generator=g)) * 20).half()
+    beta = (0.4 * torch.randn(H, generator=g)).half()
+    s = 0.0037
+    r, q = orc.dq_add_layernorm_q_f16(inp, s, res, gamma, beta, 1e-5)
+    assert r.dtype == torch.float16 and q.dtype == torch.int8
+    # torch.add casts the int32 operand to the common dtype (fp16) before the fp32 arithmetic
+    r_t = torch.add(res.float(), inp.half().float(), alpha=s).half()
+    # identical but for a double-rounding tie now and then (torch's fp32 add is within 1 ulp of the fma)
+    assert (r != r_t).float().mean() < 1e-3 and ((r.float() - r_t.float()).abs() <= r_t.float().abs() * 2 ** -10).all()
+    y_t = torch.nn.functional.layer_norm(r.float(), (H,), gamma.float(), beta.float(), 1e-5).half()
+    q_t = y_t.float().clamp(-128, 127).round().to(torch.int8)
+    assert (q.int() - q_t.int()).abs().max() <= 1 and (q != q_t).float().mean() <= 0.01 + 1.0 / q.numel()
+    # the add + LayerNormQ chain, with and without the add
+    x = torch.randn(shape, generator=g).half()
+    r2, q2 = orc.add_layernorm_q_f16(x, res, gamma, beta, 1e-5)
+    assert torch.equal(r2, (res.float() + x.float()).half())
+    y_t = torch.nn.functional.layer_norm(r2.float(), (H,), gamma.float(), beta.float(), 1e-5).half()
+    q_t = y_t.float().clamp(-128, 127).round().to(torch.int8)
+    assert (q2.int() - q_t.int()).abs().max() <= 1 and (q2 != q_t).float().mean() <= 0.01 + 1.0 / q2.numel()
+    r3, q3 = orc.add_layernorm_q_f16(None, r2, gamma, beta, 1e-5)
+    assert torch.equal(r3, r2) and torch.equal(q3, q2)
+
+
+def test_ln_q_f16_rounds_the_normalised_value_to_half_before_the_integer():
+    # one row where fp16 rounding of y decides the integer: y = 65.47 -> fp16 65.5 -> 66 (fp32 alone gives 65)
+    H = 4
+    res = torch.tensor([[1.0, -1.0, 1.0, -1.0]]).half()          # mean 0, variance 1
+    gamma = torch.tensor([65.47, 64.47, 1.0, 1.0]).half()
+    beta = torch.zeros(H).half()
+    _, q = orc.add_layernorm_q_f16(None, res, gamma, beta, 0.0)
+    g32 = gamma.float()
+    y = (res.float()[0] * g32)
+    assert q[0].tolist() == y.half().float().round().to(torch.int8).tolist()

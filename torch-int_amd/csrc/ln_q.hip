@@ -3,6 +3,12 @@
 // one pass over HBM (13 bytes per element: 4 in + 4 residual in + 4 residual
 // out + 1 int8 out).
 //
+// The residual stream, gamma and beta are fp32 or, all three, fp16 (element type T).  With fp16 the arithmetic
+// stays fp32 and rounds where a chain of torch ops on fp16 tensors rounds: the int32 input is converted to fp16
+// first (torch.add casts it to the common dtype; magnitudes from 65520 up become infinity), the updated residual
+// is rounded to fp16 before it is normalised (LayerNorm sees the stored tensor), and the LayerNorm output is
+// rounded to fp16 before it is rounded to an integer.  9 bytes per element then.
+//
 // One 256-lane workgroup per row.  The row lives in registers between the
 // three phases (sum, sum of squared deviations, normalise), so each input
 // byte is read once.  The fp32 reduction order is fixed:
@@ -28,6 +34,28 @@ __device__ __forceinline__ float block_sum_256(float s, float* red) {
   return ((red[0] + red[1]) + red[2]) + red[3];
 }
 
+typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+
+// four consecutive elements (chunk c) of a row as fp32 / stored from fp32
+__device__ __forceinline__ v4f load4(const float* row, int c) { return reinterpret_cast<const v4f*>(row)[c]; }
+__device__ __forceinline__ v4f load4(const _Float16* row, int c) {
+  const v4h h = reinterpret_cast<const v4h*>(row)[c];
+  return v4f{(float)h[0], (float)h[1], (float)h[2], (float)h[3]};
+}
+__device__ __forceinline__ void store4(float* row, int c, v4f v) { reinterpret_cast<v4f*>(row)[c] = v; }
+__device__ __forceinline__ void store4(_Float16* row, int c, v4f v) {
+  reinterpret_cast<v4h*>(row)[c] = v4h{(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
+}
+// The value a tensor of element type T holds after the fp32 value `x` is stored to it (round to nearest even
+// for fp16).  The empty asm keeps the fp32 result of the preceding operation a value of its own: without it the
+// compiler merges an fma and the conversion into one mixed-precision instruction that rounds the exact sum
+// straight to fp16, which differs from "fp32 operation, then conversion" when the fp32 result is a tie.
+template <class T>
+__device__ __forceinline__ float as_stored(float x) {
+  if constexpr (sizeof(T) == 2) asm volatile("" : "+v"(x));
+  return (float)(T)x;
+}
+
 __device__ __forceinline__ int pack_s8x4(float y0, float y1, float y2, float y3) {
   unsigned b0 = (unsigned char)(int8_t)rne_s8(y0);
   unsigned b1 = (unsigned char)(int8_t)rne_s8(y1);
@@ -45,31 +73,30 @@ enum LnMode : int { MODE_DQ_ADD = 0, MODE_ADD = 1, MODE_PLAIN = 2 };
 // EARLY: gamma and beta are fetched together with the row instead of after the two reductions; with only
 // a few rows in flight (decode) the kernel is a chain of memory latencies and this removes one of them,
 // with many rows the extra registers would only cost occupancy.
-template <int NC, int MODE, bool EARLY = false>
-__global__ __launch_bounds__(256) void ln_q_rows_kernel(const int32_t* __restrict__ in, float scale,
-                                                        const float* res,  // may alias r_out
-                                                        const float* __restrict__ gamma,
-                                                        const float* __restrict__ beta, float eps,
-                                                        float* r_out, int8_t* __restrict__ q_out, int H) {
+template <int NC, int MODE, bool EARLY, class T>
+__global__ __launch_bounds__(256) void ln_q_rows_kernel(const void* __restrict__ in, float scale,
+                                                        const T* res,  // may alias r_out
+                                                        const T* __restrict__ gamma,
+                                                        const T* __restrict__ beta, float eps,
+                                                        T* r_out, int8_t* __restrict__ q_out, int H) {
   __shared__ float red[4];
   const long long row = blockIdx.x;
   const int t = threadIdx.x;
   const int nchunks = H >> 2;
-  const v4i* in4 = reinterpret_cast<const v4i*>(in + row * H);
-  const v4f* res4 = reinterpret_cast<const v4f*>(res + row * H);
-  v4f* rout4 = reinterpret_cast<v4f*>(r_out + row * H);
+  const v4i* in4 = reinterpret_cast<const v4i*>(static_cast<const int32_t*>(in) + row * H);  // MODE_DQ_ADD
+  const T* x_row = static_cast<const T*>(in) + row * H;                                        // MODE_ADD
+  const T* res_row = res + row * H;
+  T* rout_row = r_out + row * H;
   int* q4 = reinterpret_cast<int*>(q_out + row * H);
 
-  const v4f* g4 = reinterpret_cast<const v4f*>(gamma);
-  const v4f* b4 = reinterpret_cast<const v4f*>(beta);
   v4f ge[EARLY ? NC : 1], be[EARLY ? NC : 1];
   if constexpr (EARLY) {
 #pragma unroll
     for (int i = 0; i < NC; ++i) {
       const int c = t + i * 256;
       if (c < nchunks) {
-        ge[i] = g4[c];
-        be[i] = b4[c];
+        ge[i] = load4(gamma, c);
+        be[i] = load4(beta, c);
       }
     }
   }
@@ -79,21 +106,21 @@ __global__ __launch_bounds__(256) void ln_q_rows_kernel(const int32_t* __restric
   for (int i = 0; i < NC; ++i) {
     const int c = t + i * 256;
     if (c < nchunks) {
-      v4f a = res4[c];
+      v4f a = load4(res_row, c);
       v4f v;
       if (MODE == MODE_DQ_ADD) {
         v4i x = in4[c];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) v[j] = __builtin_fmaf(scale, (float)x[j], a[j]);
+        for (int j = 0; j < 4; ++j) v[j] = as_stored<T>(__builtin_fmaf(scale, as_stored<T>((float)x[j]), a[j]));
       } else if (MODE == MODE_ADD) {
-        v4f x = reinterpret_cast<const v4f*>(in4)[c];
+        v4f x = load4(x_row, c);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) v[j] = a[j] + x[j];
+        for (int j = 0; j < 4; ++j) v[j] = as_stored<T>(a[j] + x[j]);
       } else {
         v = a;
       }
       r[i] = v;
-      if (MODE != MODE_PLAIN) rout4[c] = v;
+      if (MODE != MODE_PLAIN) store4(rout_row, c, v);
 #pragma unroll
       for (int j = 0; j < 4; ++j) s = s + v[j];
     }
@@ -124,12 +151,12 @@ __global__ __launch_bounds__(256) void ln_q_rows_kernel(const int32_t* __restric
         g = ge[i];
         b = be[i];
       } else {
-        g = g4[c];
-        b = b4[c];
+        g = load4(gamma, c);
+        b = load4(beta, c);
       }
       float y[4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) y[j] = __builtin_fmaf((r[i][j] - mu) * rstd, g[j], b[j]);
+      for (int j = 0; j < 4; ++j) y[j] = as_stored<T>(__builtin_fmaf((r[i][j] - mu) * rstd, g[j], b[j]));
       q4[c] = pack_s8x4(y[0], y[1], y[2], y[3]);
     }
   }
@@ -137,24 +164,25 @@ __global__ __launch_bounds__(256) void ln_q_rows_kernel(const int32_t* __restric
 
 // Any H and alignment: same reduction tree, scalar accesses, the row is
 // recomputed from the inputs in each phase instead of being kept in registers.
-__global__ __launch_bounds__(256) void ln_q_rows_generic_kernel(const int32_t* __restrict__ in, float scale,
-                                                                const float* res, const float* __restrict__ gamma,
-                                                                const float* __restrict__ beta, float eps,
-                                                                float* r_out, int8_t* __restrict__ q_out, int H,
+template <class T>
+__global__ __launch_bounds__(256) void ln_q_rows_generic_kernel(const void* __restrict__ in, float scale,
+                                                                const T* res, const T* __restrict__ gamma,
+                                                                const T* __restrict__ beta, float eps,
+                                                                T* r_out, int8_t* __restrict__ q_out, int H,
                                                                 int mode) {
   __shared__ float red[4];
   const long long row = blockIdx.x;
   const int t = threadIdx.x;
-  const int32_t* x = in + row * H;
-  const float* a = res + row * H;
-  float* ro = r_out + row * H;
+  const int32_t* x = static_cast<const int32_t*>(in) + row * H;
+  const T* xf = static_cast<const T*>(in) + row * H;
+  const T* a = res + row * H;
+  T* ro = r_out + row * H;
   int8_t* q = q_out + row * H;
   const int nchunks = (H + 3) >> 2;
-  const float* xf = reinterpret_cast<const float*>(x);
   auto value = [&](int i) {
-    if (mode == MODE_DQ_ADD) return __builtin_fmaf(scale, (float)x[i], a[i]);
-    if (mode == MODE_ADD) return a[i] + xf[i];
-    return a[i];
+    if (mode == MODE_DQ_ADD) return as_stored<T>(__builtin_fmaf(scale, as_stored<T>((float)x[i]), (float)a[i]));
+    if (mode == MODE_ADD) return as_stored<T>((float)a[i] + (float)xf[i]);
+    return (float)a[i];
   };
   float s = 0.0f;
   for (int c = t; c < nchunks; c += 256)
@@ -183,25 +211,24 @@ __global__ __launch_bounds__(256) void ln_q_rows_generic_kernel(const int32_t* _
       const int i = c * 4 + j;
       if (i < H) {
         float v = value(i);
-        float y = __builtin_fmaf((v - mu) * rstd, gamma[i], beta[i]);
-        if (mode != MODE_PLAIN) ro[i] = v;
+        float y = as_stored<T>(__builtin_fmaf((v - mu) * rstd, (float)gamma[i], (float)beta[i]));
+        if (mode != MODE_PLAIN) ro[i] = (T)v;
         q[i] = (int8_t)rne_s8(y);
       }
     }
 }
 
-template <int NC>
-static void launch_rows(int mode, const int32_t* in, float scale, const float* res, const float* gamma,
-                        const float* beta, float eps, float* r_out, int8_t* q_out, long long rows, int H,
-                        hipStream_t stream) {
+template <int NC, class T>
+static void launch_rows(int mode, const void* in, float scale, const T* res, const T* gamma, const T* beta, float eps,
+                        T* r_out, int8_t* q_out, long long rows, int H, hipStream_t stream) {
   const dim3 grid((unsigned)rows), block(256);
   const bool early = rows <= 64;  // fewer rows than CUs: latency-bound
-#define TI_LN_LAUNCH(MODE)                                                                                     \
-  if (early)                                                                                                   \
-    hipLaunchKernelGGL((ln_q_rows_kernel<NC, MODE, true>), grid, block, 0, stream, in, scale, res, gamma, beta, eps, \
-                       r_out, q_out, H);                                                                       \
-  else                                                                                                         \
-    hipLaunchKernelGGL((ln_q_rows_kernel<NC, MODE, false>), grid, block, 0, stream, in, scale, res, gamma, beta, eps, \
+#define TI_LN_LAUNCH(MODE)                                                                                        \
+  if (early)                                                                                                      \
+    hipLaunchKernelGGL((ln_q_rows_kernel<NC, MODE, true, T>), grid, block, 0, stream, in, scale, res, gamma, beta, eps, \
+                       r_out, q_out, H);                                                                          \
+  else                                                                                                            \
+    hipLaunchKernelGGL((ln_q_rows_kernel<NC, MODE, false, T>), grid, block, 0, stream, in, scale, res, gamma, beta, eps, \
                        r_out, q_out, H)
   if (mode == MODE_DQ_ADD) {
     TI_LN_LAUNCH(MODE_DQ_ADD);
@@ -213,21 +240,22 @@ static void launch_rows(int mode, const int32_t* in, float scale, const float* r
 #undef TI_LN_LAUNCH
 }
 
-static int launch_ln_mode(int mode, const void* in, float scale, const float* res, const float* gamma,
-                          const float* beta, float eps, float* r_out, int8_t* q_out, long long rows, long long H,
-                          hipStream_t stream) {
+template <class T>
+static int launch_ln_mode(int mode, const void* in, float scale, const T* res, const T* gamma, const T* beta, float eps,
+                          T* r_out, int8_t* q_out, long long rows, long long H, hipStream_t stream) {
   if (rows == 0 || H == 0) return TI_OK;
-  auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
-  const bool fast = (H % 4 == 0) && H <= 16 * 1024 && (mode == MODE_PLAIN || al16(in)) && al16(res) && al16(gamma) &&
-                    al16(beta) && (mode == MODE_PLAIN || al16(r_out)) &&
-                    ((reinterpret_cast<uintptr_t>(q_out) & 3) == 0);
+  // a chunk of four elements is one load: 16 bytes of fp32, 8 bytes of fp16 (16 bytes of the int32 input)
+  constexpr uintptr_t kAlign = 4 * sizeof(T) - 1;
+  auto al = [](const void* p, uintptr_t mask) { return (reinterpret_cast<uintptr_t>(p) & mask) == 0; };
+  const uintptr_t in_mask = mode == MODE_DQ_ADD ? 15 : kAlign;
+  const bool fast = (H % 4 == 0) && H <= 16 * 1024 && (mode == MODE_PLAIN || al(in, in_mask)) && al(res, kAlign) &&
+                    al(gamma, kAlign) && al(beta, kAlign) && (mode == MODE_PLAIN || al(r_out, kAlign)) && al(q_out, 3);
   const int h = (int)H;
-  const int32_t* in32 = static_cast<const int32_t*>(in);
   if (fast) {
     const int nc = (int)((H + 1023) / 1024);
-#define TI_LN_CASE(n)                                                                              \
-  case n:                                                                                          \
-    launch_rows<n>(mode, in32, scale, res, gamma, beta, eps, r_out, q_out, rows, h, stream);       \
+#define TI_LN_CASE(n)                                                                                \
+  case n:                                                                                            \
+    launch_rows<n, T>(mode, in, scale, res, gamma, beta, eps, r_out, q_out, rows, h, stream);        \
     break;
     switch (nc) {
       TI_LN_CASE(1) TI_LN_CASE(2) TI_LN_CASE(3) TI_LN_CASE(4) TI_LN_CASE(5) TI_LN_CASE(6) TI_LN_CASE(7)
@@ -236,7 +264,7 @@ static int launch_ln_mode(int mode, const void* in, float scale, const float* re
     }
 #undef TI_LN_CASE
   } else {
-    hipLaunchKernelGGL(ln_q_rows_generic_kernel, dim3((unsigned)rows), dim3(256), 0, stream, in32, scale, res, gamma,
+    hipLaunchKernelGGL(ln_q_rows_generic_kernel<T>, dim3((unsigned)rows), dim3(256), 0, stream, in, scale, res, gamma,
                        beta, eps, r_out, q_out, h, mode);
   }
   hipError_t e = hipGetLastError();
@@ -247,15 +275,35 @@ static int launch_ln_mode(int mode, const void* in, float scale, const float* re
 int launch_dq_add_layernorm_q(const int32_t* in, float scale, const float* res, const float* gamma,
                               const float* beta, float eps, float* r_out, int8_t* q_out, long long rows,
                               long long H, hipStream_t stream) {
-  return launch_ln_mode(MODE_DQ_ADD, in, scale, res, gamma, beta, eps, r_out, q_out, rows, H, stream);
+  return launch_ln_mode<float>(MODE_DQ_ADD, in, scale, res, gamma, beta, eps, r_out, q_out, rows, H, stream);
 }
 
 // x == nullptr: q = LayerNormQ(residual); else residual += x (in place) and q = LayerNormQ(residual).
 int launch_add_layernorm_q(const float* x, float* residual, const float* gamma, const float* beta, float eps,
                            int8_t* q_out, long long rows, long long H, hipStream_t stream) {
   if (x == nullptr)
-    return launch_ln_mode(MODE_PLAIN, nullptr, 1.0f, residual, gamma, beta, eps, nullptr, q_out, rows, H, stream);
-  return launch_ln_mode(MODE_ADD, x, 1.0f, residual, gamma, beta, eps, residual, q_out, rows, H, stream);
+    return launch_ln_mode<float>(MODE_PLAIN, nullptr, 1.0f, residual, gamma, beta, eps, nullptr, q_out, rows, H, stream);
+  return launch_ln_mode<float>(MODE_ADD, x, 1.0f, residual, gamma, beta, eps, residual, q_out, rows, H, stream);
+}
+
+// The same two operations on an fp16 residual stream with fp16 gamma and beta (pointers to IEEE binary16).
+int launch_dq_add_layernorm_q_f16(const int32_t* in, float scale, const void* res, const void* gamma, const void* beta,
+                                  float eps, void* r_out, int8_t* q_out, long long rows, long long H,
+                                  hipStream_t stream) {
+  using H16 = _Float16;
+  return launch_ln_mode<H16>(MODE_DQ_ADD, in, scale, static_cast<const H16*>(res), static_cast<const H16*>(gamma),
+                             static_cast<const H16*>(beta), eps, static_cast<H16*>(r_out), q_out, rows, H, stream);
+}
+
+int launch_add_layernorm_q_f16(const void* x, void* residual, const void* gamma, const void* beta, float eps,
+                               int8_t* q_out, long long rows, long long H, hipStream_t stream) {
+  using H16 = _Float16;
+  H16* r = static_cast<H16*>(residual);
+  if (x == nullptr)
+    return launch_ln_mode<H16>(MODE_PLAIN, nullptr, 1.0f, r, static_cast<const H16*>(gamma),
+                               static_cast<const H16*>(beta), eps, nullptr, q_out, rows, H, stream);
+  return launch_ln_mode<H16>(MODE_ADD, x, 1.0f, r, static_cast<const H16*>(gamma), static_cast<const H16*>(beta), eps, r,
+                             q_out, rows, H, stream);
 }
 
 }  // namespace ti

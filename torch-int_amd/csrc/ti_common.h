@@ -211,6 +211,12 @@ int launch_dq_add_layernorm_q(const int32_t* in, float scale, const float* res, 
 int launch_add_layernorm_q(const float* x, float* residual, const float* gamma, const float* beta, float eps,
                            int8_t* q_out, long long rows, long long H, hipStream_t stream);
 
+int launch_dq_add_layernorm_q_f16(const int32_t* in, float scale, const void* res, const void* gamma, const void* beta,
+                                  float eps, void* r_out, int8_t* q_out, long long rows, long long H,
+                                  hipStream_t stream);
+int launch_add_layernorm_q_f16(const void* x, void* residual, const void* gamma, const void* beta, float eps,
+                               int8_t* q_out, long long rows, long long H, hipStream_t stream);
+
 // softmax_q.hip
 int launch_attn_softmax_q(const float* scores, const float* mask, int8_t* out, long long batch, long long heads,
                           long long T, long long S, hipStream_t stream);

@@ -44,6 +44,7 @@ _SIGNATURES = {
     "ti_bmm_s8t_s8n_s8t": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _f32, _vp],
     "ti_bmm_s8t_s8n_s32t": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],
     "ti_dq_add_layernorm_q": [_vp, _f32, _vp, _vp, _vp, _f32, _vp, _vp, _i64, _i64, _vp],
+    "ti_dq_add_layernorm_q_f16": [_vp, _f32, _vp, _vp, _vp, _f32, _vp, _vp, _i64, _i64, _vp],
 }
 
 
@@ -287,24 +288,34 @@ def bmm_s8t_s8n_s32t(A, B):
 
 
 def dq_add_layernorm_q(input, input_scale, residual_input, gamma, beta, epsilon):
-    """(residual_output fp32, ln_output int8)  (upstream fused.cu:5-25).
+    """(residual_output, ln_output int8)  (upstream fused.cu:5-25).
 
     residual_output = residual_input + input_scale * input;
     ln_output = int8(round(clamp(layer_norm(residual_output) * gamma + beta, -128, 127))).
+    residual_input, gamma and beta are fp32, or all three fp16 (as upstream's benchmark/bench_dq_add_ln_q.py:37-45
+    calls it); residual_output has the residual's dtype.  With fp16 the arithmetic is fp32 and rounds to fp16 where
+    upstream's chain of ATen ops does (the updated residual, the LayerNorm output).
     """
     op = "dq_add_layernorm_q"
     _check(op, "input", input, _I32, None)
     dev = input.device
     if input.dim() < 1:
         _fail(op, "input must have at least one dimension")
-    _check(op, "residual_input", residual_input, _F32, None, dev)
+    fdt = residual_input.dtype if isinstance(residual_input, torch.Tensor) else None
+    if fdt is not torch.float16:
+        fdt = _F32
+    _check(op, "residual_input", residual_input, fdt, None, dev)
     if residual_input.shape != input.shape:
         _fail(op, f"input is {tuple(input.shape)} but residual_input is {tuple(residual_input.shape)}")
     H = input.shape[-1]
     gamma = gamma.detach() if isinstance(gamma, torch.Tensor) else gamma
     beta = beta.detach() if isinstance(beta, torch.Tensor) else beta
-    _check(op, "gamma", gamma, _F32, 1, dev)
-    _check(op, "beta", beta, _F32, 1, dev)
+    for name, t in (("gamma", gamma), ("beta", beta)):
+        if isinstance(t, torch.Tensor) and t.dtype is not fdt and t.dtype in (_F32, torch.float16):
+            _fail(op, f"{name} is {t.dtype} but residual_input is {fdt}: residual_input, gamma and beta must share one "
+                      "dtype (float32 or float16)")
+    _check(op, "gamma", gamma, fdt, 1, dev)
+    _check(op, "beta", beta, fdt, 1, dev)
     if gamma.numel() != H or beta.numel() != H:
         _fail(op, f"gamma/beta must have {H} elements, got {gamma.numel()} and {beta.numel()}")
     r_out = torch.empty_like(residual_input)
@@ -320,7 +331,10 @@ def dq_add_layernorm_q(input, input_scale, residual_input, gamma, beta, epsilon)
         stream = _raw_stream(idx)
         args = (input.data_ptr(), float(input_scale), residual_input.data_ptr(), gamma.data_ptr(), beta.data_ptr(),
                 float(epsilon), r_out.data_ptr(), q_out.data_ptr(), input.numel() // H, H)
-        rc = _fast.ln_q(*args, stream) if _fast is not None else _lib.ti_dq_add_layernorm_q(*args, stream or None)
+        if fdt is torch.float16:
+            rc = _lib.ti_dq_add_layernorm_q_f16(*args, stream or None)
+        else:
+            rc = _fast.ln_q(*args, stream) if _fast is not None else _lib.ti_dq_add_layernorm_q(*args, stream or None)
     finally:
         if switch:
             torch.cuda.set_device(prev)

@@ -23,6 +23,8 @@ _lib = _CUDA._lib
 _vp, _i64, _f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_float
 _lib.ti_add_layernorm_q.argtypes = [_vp, _vp, _vp, _vp, _f32, _vp, _i64, _i64, _vp]
 _lib.ti_add_layernorm_q.restype = ctypes.c_int
+_lib.ti_add_layernorm_q_f16.argtypes = [_vp, _vp, _vp, _vp, _f32, _vp, _i64, _i64, _vp]
+_lib.ti_add_layernorm_q_f16.restype = ctypes.c_int
 _lib.ti_attn_softmax_q.argtypes = [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]
 _lib.ti_attn_softmax_q.restype = ctypes.c_int
 _lib.ti_permute_0213_s8.argtypes = [_vp, _vp, _i64, _i64, _i64, _i64, _vp]
@@ -91,8 +93,9 @@ def _ok(t, dtype):
 
 
 def can_fuse_layernorm(x, weight, bias):
-    """True when the fused kernel applies: fp32 contiguous HIP tensors, last dim = len(weight)."""
-    return (_ok(x, torch.float32) and _ok(weight, torch.float32) and _ok(bias, torch.float32)
+    """True when the fused kernel applies: contiguous HIP tensors that are all fp32 or all fp16, last dim = len(weight)."""
+    dt = x.dtype if isinstance(x, torch.Tensor) else None
+    return (dt in (torch.float32, torch.float16) and _ok(x, dt) and _ok(weight, dt) and _ok(bias, dt)
             and x.dim() >= 1 and x.shape[-1] == weight.numel() == bias.numel() and x.numel() > 0)
 
 
@@ -103,14 +106,18 @@ def add_layernorm_q(x, residual, weight, bias, eps, checked=False):
     op = "add_layernorm_q"
     if not checked:
         if not can_fuse_layernorm(residual, weight, bias):
-            raise RuntimeError(f"torch_int._hip_ext.{op}: needs contiguous fp32 HIP tensors")
-        if x is not None and not (_ok(x, torch.float32) and x.shape == residual.shape and x.device == residual.device):
-            raise RuntimeError(f"torch_int._hip_ext.{op}: x must be a contiguous fp32 tensor shaped like residual")
+            raise RuntimeError(f"torch_int._hip_ext.{op}: needs contiguous HIP tensors, all fp32 or all fp16")
+        if x is not None and not (_ok(x, residual.dtype) and x.shape == residual.shape and x.device == residual.device):
+            raise RuntimeError(f"torch_int._hip_ext.{op}: x must be a contiguous tensor shaped and typed like residual")
     dev = residual.device
     H = residual.shape[-1]
     q = torch.empty(residual.shape, dtype=torch.int8, device=dev)
     with _on(dev):
-        if _fast_add_ln_q is not None:
+        if residual.dtype is torch.float16:
+            rc = _lib.ti_add_layernorm_q_f16(x.data_ptr() if x is not None else None, residual.data_ptr(),
+                                             weight.data_ptr(), bias.data_ptr(), float(eps), q.data_ptr(),
+                                             residual.numel() // H, H, _raw_stream(dev.index) or None)
+        elif _fast_add_ln_q is not None:
             rc = _fast_add_ln_q(x.data_ptr() if x is not None else 0, residual.data_ptr(), weight.data_ptr(),
                                 bias.data_ptr(), float(eps), q.data_ptr(), residual.numel() // H, H,
                                 _raw_stream(dev.index))

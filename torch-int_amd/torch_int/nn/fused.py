@@ -29,7 +29,10 @@ class LayerNormQ(_QuantLayerNormBase):
             return _hip_ext.add_layernorm_q(add, x, self.weight, self.bias, self.eps, checked=True)  # one pass, same maths
         if add is not None:
             x.add_(add.to(x.dtype))
-        y = F.layer_norm(x.to(self.weight.dtype), x.shape[-1:], self.weight, self.bias, self.eps)
+        x = x.to(self.weight.dtype)  # upstream nn/fused.py:14: an fp16 input of an fp32 layer is promoted first
+        if _hip_ext.can_fuse_layernorm(x, self.weight, self.bias):
+            return _hip_ext.add_layernorm_q(None, x, self.weight, self.bias, self.eps, checked=True)
+        y = F.layer_norm(x, x.shape[-1:], self.weight, self.bias, self.eps)
         return y.round().clamp(-128, 127).to(torch.int8)
 
     @staticmethod
