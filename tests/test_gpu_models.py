@@ -296,3 +296,28 @@ def test_side_stream_and_graph_replay_of_a_decoder_layer():
         torch.cuda.synchronize()
         assert torch.equal(static_out[0], ref[0]), i
         assert torch.equal(static_out[1][0], ref[1][0]) and torch.equal(static_out[1][1], ref[1][1]), i
+
+
+@torch.no_grad()
+def test_fused_softmax_switch_restores_the_torch_chain():
+    """Int8OPTAttention.fused_softmax = False: probabilities from upstream's chain of torch ops; the layer's int8
+    tensors then differ from the fused path by at most one LSB on a small fraction, and the fp32 output agrees."""
+    from torch_int.models.opt import Int8OPTAttention
+    g = torch.Generator().manual_seed(9)
+    D, H, F, B, T = 640, 5, 1280, 2, 128
+    layer = randomize_int8_layer(Int8OPTDecoderLayer(D, H, F), g, 2e-4, 2e-3).to(DEV)
+    hidden = torch.randn(B, T, D, generator=g).to(DEV)
+    mask = causal_mask(B, T, T).to(DEV)
+    fused = layer(hidden.clone(), attention_mask=mask, use_cache=True, output_attentions=True)
+    Int8OPTAttention.fused_softmax = False
+    try:
+        plain = layer(hidden.clone(), attention_mask=mask, use_cache=True, output_attentions=True)
+        step = layer(hidden[:, :1].clone(), attention_mask=torch.zeros(B, 1, 1, T + 1, device=DEV), use_cache=True,
+                     past_key_value=plain[2])
+    finally:
+        Int8OPTAttention.fused_softmax = True
+    assert step[1][0].shape[2] == T + 1
+    p_f, p_p = fused[1], plain[1]          # round(127 p) as fp32, [B, H, T, T]
+    assert (p_f - p_p).abs().max() <= 1 and (p_f != p_p).float().mean() < 5e-3
+    assert torch.equal(fused[2][0], plain[2][0]) and torch.equal(fused[2][1], plain[2][1])   # K / V: before the softmax
+    assert _rel_err(fused[0], plain[0]) < 2e-2

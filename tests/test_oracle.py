@@ -124,6 +124,28 @@ def test_int_to_float_conversion_rounds_to_nearest_even():
     assert out.tolist() == [2.0 ** 24, 2.0 ** 24 + 4, -(2.0 ** 24), 2.0 ** 31, -(2.0 ** 31)]
 
 
+def test_f32t_and_s8t_epilogues_are_one_rounded_multiply():
+    # alpha * f32(acc): one fp32 product of the (already rounded) converted accumulator, against exact rationals
+    rng = np.random.default_rng(1)
+    acc = torch.from_numpy(np.concatenate([rng.integers(-2 ** 31, 2 ** 31, 1500), rng.integers(-40000, 40000, 1500)])
+                           .astype(np.int32))
+    alpha = 0.0186   # the scale of upstream's literal test (tests/test_bmm.py:99)
+    out = orc.epi_f32t(acc, alpha)
+    out8 = orc.epi_s8t(acc, alpha)
+    a32 = Fraction(float(np.float32(alpha)))
+    for i in range(acc.numel()):
+        conv = Fraction(float(np.float32(int(acc[i]))))          # int32 -> fp32, first rounding
+        want = _round_to_f32(a32 * conv)
+        assert out[i].item() == want, i
+        t = Fraction(want)
+        lo = max(min(t, Fraction(127)), Fraction(-128))           # clamp, then round half to even
+        fl = lo.numerator // lo.denominator
+        rem = lo - fl
+        if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and fl % 2 == 1):
+            fl += 1
+        assert out8[i].item() == fl, i
+
+
 def test_s8_epilogue_identity_ties_and_saturation():
     acc = torch.arange(-140, 141, dtype=torch.int32).view(1, -1)
     n = acc.numel()

@@ -97,6 +97,10 @@ class Int8OPTAttention(nn.Module):
     across heads; set it to False to get upstream's freshly concatenated contiguous tensors.
     """
     kv_cache_in_place = True
+    # False: the probabilities come from upstream's own chain of torch ops between the two products (mask add,
+    # clamp, softmax, * 127, round, int8 cast; models/opt.py:144-178) instead of the fused kernels, whose
+    # e * (127 / sum) differs from (e / sum) * 127 by one LSB on a small fraction of the probabilities.
+    fused_softmax = True
 
     def __init__(self, embed_dim: int, num_heads: int):
         super().__init__()
@@ -237,7 +241,8 @@ class Int8OPTAttention(nn.Module):
                 key = self._shape(self.k_proj(kv_src), -1, bsz)
                 value = self._shape(self.v_proj(kv_src), -1, bsz)
             if not cross and past_key_value is not None:
-                if self.kv_cache_in_place and proj is not None and tgt_len <= 4 and layer_head_mask is None:
+                if (self.kv_cache_in_place and self.fused_softmax and proj is not None and tgt_len <= 4
+                        and layer_head_mask is None):
                     fused = self._decode_fused(query4, key, value, past_key_value, attention_mask, output_attentions)
                     if fused is not None:
                         return fused
@@ -254,8 +259,8 @@ class Int8OPTAttention(nn.Module):
         value = value.view(bsz * H, -1, d) if value.is_contiguous() else value.reshape(bsz * H, value.shape[2], d)
         src_len = key.size(1)
 
-        if (layer_head_mask is None and not output_attentions and tgt_len > 16 and src_len % 64 == 0
-                and type(self.qk_bmm) is BMM_S8T_S8N_F32T and type(self.pv_bmm) is BMM_S8T_S8N_S8T
+        if (self.fused_softmax and layer_head_mask is None and not output_attentions and tgt_len > 16
+                and src_len % 64 == 0 and type(self.qk_bmm) is BMM_S8T_S8N_F32T and type(self.pv_bmm) is BMM_S8T_S8N_S8T
                 and _hip_ext.can_attn_qk_softmax_q(query, key, attention_mask, bsz, H) and value.is_cuda):
             # the whole attention (Q.K^T, softmax-quant, P.V, head merge) in one kernel on V transposed
             vt = _hip_ext.transpose_last2(value.contiguous())
@@ -264,7 +269,7 @@ class Int8OPTAttention(nn.Module):
                                             self.pv_bmm._scalar("a"), H, checked=True)
                 return self.out_proj(ctx), None, present
         probs_q = None
-        if (layer_head_mask is None and tgt_len > 16 and type(self.qk_bmm) is BMM_S8T_S8N_F32T
+        if (self.fused_softmax and layer_head_mask is None and tgt_len > 16 and type(self.qk_bmm) is BMM_S8T_S8N_F32T
                 and _hip_ext.can_attn_qk_softmax_q(query, key, attention_mask, bsz, H)):
             # Q.K^T, mask, clamp, softmax, *127, round and int8 cast in one kernel: the fp32 scores stay in registers
             probs_q = _hip_ext.attn_qk_softmax_q(query, key, attention_mask, self.qk_bmm._scalar("a"), H, checked=True)
@@ -285,7 +290,7 @@ class Int8OPTAttention(nn.Module):
                              f" {layer_head_mask.size()}")
         if probs_q is not None:
             pass
-        elif layer_head_mask is None and _hip_ext.can_fuse_softmax(scores, attention_mask, bsz, H):
+        elif self.fused_softmax and layer_head_mask is None and _hip_ext.can_fuse_softmax(scores, attention_mask, bsz, H):
             # mask add, clamp, softmax, *127, round and int8 cast in one kernel
             probs_q = _hip_ext.attn_softmax_q(scores, attention_mask, H, checked=True)
             probs_out = probs_q.view(bsz, H, tgt_len, src_len).float() if output_attentions else None
