@@ -59,7 +59,7 @@ struct TileCfg {
 // with a private L2) own a contiguous run of tiles and (ii) consecutive tiles
 // walk down GROUP rows of tiles before moving to the next column, which keeps
 // the A rows and B rows a run touches small enough to stay in that L2.
-__device__ __forceinline__ void tile_of_workgroup(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
+__device__ __forceinline__ void tile_of_workgroup(int pid, int tiles_m, int tiles_n, int& tm, int& tn, int GROUP = 8) {
   const int total = tiles_m * tiles_n;
   const int NXCD = 8;
   int per = (total + NXCD - 1) / NXCD;
@@ -67,7 +67,6 @@ __device__ __forceinline__ void tile_of_workgroup(int pid, int tiles_m, int tile
   if (tall == 0) tall = NXCD;
   int xcd = pid % NXCD, local = pid / NXCD;
   int id = (xcd < tall) ? xcd * per + local : tall * per + (xcd - tall) * (per - 1) + local;
-  const int GROUP = 8;
   int width = GROUP * tiles_n;
   int g = id / width;
   int first = g * GROUP;
@@ -435,7 +434,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MIN_WAVES) void gemm_pipe_kernel(Gemm
   auto set_copy_item = [&](int item) {
     const int b = item / tiles;
     int tile_m, tile_n;
-    tile_of_workgroup(item - b * tiles, tiles_m, tiles_n, tile_m, tile_n);
+    tile_of_workgroup(item - b * tiles, tiles_m, tiles_n, tile_m, tile_n, p.band);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int8_t* A = p.A + (long long)b * p.strideA;
     const int8_t* B = p.B + (long long)b * p.strideB;
@@ -555,7 +554,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MIN_WAVES) void gemm_pipe_kernel(Gemm
   auto finish_item = [&]() {
     const int b = item / tiles;
     int tile_m, tile_n;
-    tile_of_workgroup(item - b * tiles, tiles_m, tiles_n, tile_m, tile_n);
+    tile_of_workgroup(item - b * tiles, tiles_m, tiles_n, tile_m, tile_n, p.band);
     // opaque copy of the lane id: keeps the epilogue's address arithmetic inside the loop
     // (hoisted, it would occupy registers during the whole mainloop)
     int lane_here = lane;
@@ -648,7 +647,7 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe2_kernel(GemmParams p, in
   auto set_copy_item = [&](int item) {
     const int b = item / tiles;
     int tile_m, tile_n;
-    tile_of_workgroup(item - b * tiles, tiles_m, tiles_n, tile_m, tile_n);
+    tile_of_workgroup(item - b * tiles, tiles_m, tiles_n, tile_m, tile_n, p.band);
     const int first_row = copies_a ? tile_m * BM : tile_n * BN;  // of the panel in its operand
     const int last_row = (copies_a ? M : N) - 1;                 // edge rows re-read the last row; never stored
     const size_t ld = copies_a ? p.lda : p.ldb;
@@ -766,7 +765,7 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe2_kernel(GemmParams p, in
   auto finish_item = [&]() {
     const int b = item / tiles;
     int tile_m, tile_n;
-    tile_of_workgroup(item - b * tiles, tiles_m, tiles_n, tile_m, tile_n);
+    tile_of_workgroup(item - b * tiles, tiles_m, tiles_n, tile_m, tile_n, p.band);
     // opaque copy of the lane id: keeps the epilogue's address arithmetic inside the loop
     int lane_here = lane;
     asm volatile("" : "+v"(lane_here));
@@ -835,6 +834,27 @@ struct Pipe16Cfg {
   static_assert(LDS_BYTES <= 160 * 1024 && STAGES >= 3, "LDS budget");
 };
 
+// 4x4 transpose of dwords across the four 16-lane rows of a wave: lane (r, g) = r + 16 g enters with x[k] and
+// leaves with x[k] = what lane (r, k) held in x[g].  Two v_permlane32_swap and two v_permlane16_swap; every lane
+// of the wave must take part.
+__device__ __forceinline__ void row_transpose4(int (&x)[4]) {
+  auto a = __builtin_amdgcn_permlane32_swap((unsigned)x[0], (unsigned)x[2], false, false);  // rows 2,3 of x0 <-> rows 0,1 of x2
+  auto b = __builtin_amdgcn_permlane32_swap((unsigned)x[1], (unsigned)x[3], false, false);
+  auto c = __builtin_amdgcn_permlane16_swap(a[0], b[0], false, false);  // odd rows of the first <-> even rows of the second
+  auto d = __builtin_amdgcn_permlane16_swap(a[1], b[1], false, false);
+  x[0] = (int)c[0];
+  x[1] = (int)c[1];
+  x[2] = (int)d[0];
+  x[3] = (int)d[1];
+}
+
+// four int8 values (already clamped to [-128, 127], held in ints) as one dword, first value in the low byte
+__device__ __forceinline__ int pack_s8x4_ints(int a, int b, int c, int d) {
+  const unsigned lo = __builtin_amdgcn_perm((unsigned)b, (unsigned)a, 0x0c0c0400u);  // a.byte0 | b.byte0 << 8
+  const unsigned hi = __builtin_amdgcn_perm((unsigned)d, (unsigned)c, 0x0c0c0400u);
+  return (int)__builtin_amdgcn_perm(hi, lo, 0x05040100u);
+}
+
 // Epilogue of the 16x16-block kernels: the lane holds row (lane & 15) and four consecutive columns
 // 4 * (lane >> 4) .. +3 of every block.
 template <class Cfg>
@@ -850,6 +870,61 @@ __device__ __forceinline__ void store_tile16(v4i (&acc)[Cfg::TM][Cfg::TN], const
   const BiasT* __restrict__ bias = reinterpret_cast<const BiasT*>(p.bias);
   const bool vec_ok = (N & 3) == 0 && (reinterpret_cast<uintptr_t>(C) & 15) == 0;
   const bool bias_al = (reinterpret_cast<uintptr_t>(bias) & 15) == 0;
+  if constexpr (sizeof(Out) == 1 && TN >= 4) {
+    // 8-bit outputs of a wave tile that lies inside the matrix: the four lanes that share an output row swap
+    // their 4-byte pieces of four column blocks, so that a lane ends with the 16 consecutive bytes of one block
+    // and a store instruction writes 64 contiguous bytes of each of 16 rows instead of 16: a quarter of the
+    // write requests.  (A condition on the tile, not the lane: all lanes of the wave take the swaps.)
+    const int nw = tile_n * BN + wave_n * Cfg::WTN;  // first column of the wave tile
+    if ((N & 15) == 0 && (reinterpret_cast<uintptr_t>(C) & 15) == 0 && nw + Cfg::WTN <= N && (p.out_d & 15) == 0) {
+      // groups of four column blocks (the last group may be shorter and keeps its 4-byte stores)
+#pragma unroll
+      for (int j0 = 0; j0 < TN; j0 += 4) {
+        constexpr int kFull = 4;
+        const int nblk = TN - j0 < kFull ? TN - j0 : kFull;  // compile-time after unrolling
+        float bt[4][4];
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+          if (jj >= nblk) continue;
+          const int nb = nw + (j0 + jj) * 16 + 4 * eg;
+          BiasT bv[4] = {BiasT(0), BiasT(0), BiasT(0), BiasT(0)};
+          if (E::kHasBias) {
+            if ((reinterpret_cast<uintptr_t>(bias) & 3) == 0) {
+              const int w = *reinterpret_cast<const int*>(bias + nb);
+              __builtin_memcpy(bv, &w, 4);
+            } else {
+#pragma unroll
+              for (int v = 0; v < 4; ++v) bv[v] = bias[nb + v];
+            }
+          }
+#pragma unroll
+          for (int v = 0; v < 4; ++v) bt[jj][v] = E::bias_term(bv[v], p.beta);
+        }
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+          const int m = tile_m * BM + wave_m * Cfg::WTM + i * 16 + er;
+          int x[4] = {0, 0, 0, 0};
+#pragma unroll
+          for (int jj = 0; jj < 4; ++jj) {
+            if (jj >= nblk) continue;
+            x[jj] = pack_s8x4_ints(E::apply_int(acc[i][j0 + jj][0], bt[jj][0], p.alpha),
+                                   E::apply_int(acc[i][j0 + jj][1], bt[jj][1], p.alpha),
+                                   E::apply_int(acc[i][j0 + jj][2], bt[jj][2], p.alpha),
+                                   E::apply_int(acc[i][j0 + jj][3], bt[jj][3], p.alpha));
+          }
+          if (nblk == 4) {
+            row_transpose4(x);  // lane (er, eg) now holds block j0 + eg of its row, columns 0..15
+            if (m < M) *reinterpret_cast<v4i*>(C + out_index(p, m, nw + (j0 + eg) * 16)) = v4i{x[0], x[1], x[2], x[3]};
+          } else {
+#pragma unroll
+            for (int jj = 0; jj < 4; ++jj)
+              if (jj < nblk && m < M) *reinterpret_cast<int*>(C + out_index(p, m, nw + (j0 + jj) * 16 + 4 * eg)) = x[jj];
+          }
+        }
+      }
+      return;
+    }
+  }
   // accumulate-into-output kind: fetch what the tile holds now, the loads in flight together before the
   // first use -- the whole wave tile when its TM*TN*4 registers fit, else one column block at a time
   constexpr bool HOLD_ALL = E::kAccumulate && TM * TN <= 12;
@@ -955,7 +1030,7 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe16_kernel(GemmParams p, i
   auto set_copy_item = [&](int item) {
     const int b = item / tiles;
     int tile_m, tile_n;
-    tile_of_workgroup(item - b * tiles, tiles_m, tiles_n, tile_m, tile_n);
+    tile_of_workgroup(item - b * tiles, tiles_m, tiles_n, tile_m, tile_n, p.band);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int8_t* A = p.A + (long long)b * p.strideA;
     const int8_t* B = p.B + (long long)b * p.strideB;
@@ -1077,7 +1152,7 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe16_kernel(GemmParams p, i
   auto finish_item = [&]() {
     const int b = item / tiles;
     int tile_m, tile_n;
-    tile_of_workgroup(item - b * tiles, tiles_m, tiles_n, tile_m, tile_n);
+    tile_of_workgroup(item - b * tiles, tiles_m, tiles_n, tile_m, tile_n, p.band);
     int lane_here = lane;  // opaque copy: keeps the epilogue's address arithmetic out of the mainloop
     asm volatile("" : "+v"(lane_here));
     store_tile16<Cfg>(acc, p, b, tile_m, tile_n, wave_m, wave_n, lane_here);
@@ -1118,7 +1193,7 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe16_kernel(GemmParams p, i
 
 // The 16x16-block kernel with K steps of 128 bytes and two LDS stages (see gemm_pipe2_kernel for the
 // stage layout and the step structure; a step here is two 64-byte slices, one MFMA deep each).
-template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int KIND_, bool GROUPED_ = false>
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int KIND_, bool GROUPED_ = false, int MAX_STAGES_ = 3>
 struct Pipe16QCfg {
   static constexpr int BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, KIND = KIND_;
   // GROUPED: the "batches" are the problems of a GemmGroup (same activations and shape; weight, bias,
@@ -1131,7 +1206,7 @@ struct Pipe16QCfg {
   static constexpr int STAGE_BYTES = (BM + BN) * QBK;
   // three stages when the LDS holds them (256x160): copies then run two to three K steps ahead of their use,
   // which covers the latency of operands that come from HBM instead of the last-level cache
-  static constexpr int STAGES = 3 * STAGE_BYTES <= 160 * 1024 ? 3 : 2;
+  static constexpr int STAGES = (MAX_STAGES_ >= 3 && 3 * STAGE_BYTES <= 160 * 1024) ? 3 : 2;
   static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
   static constexpr int RPW = (BM + BN) / NWAVES;  // panel rows a wave copies per step
   static constexpr int TAIL_ROWS = RPW % 8;
@@ -1164,7 +1239,7 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe16q_kernel(GemmParams p, 
   auto set_copy_item = [&](int item) {
     const int b = item / tiles;
     int tile_m, tile_n;
-    tile_of_workgroup(item - b * tiles, tiles_m, tiles_n, tile_m, tile_n);
+    tile_of_workgroup(item - b * tiles, tiles_m, tiles_n, tile_m, tile_n, p.band);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int8_t* A = Cfg::GROUPED ? p.A : p.A + (long long)b * p.strideA;
     const int8_t* B = Cfg::GROUPED ? grp.B[b] : p.B + (long long)b * p.strideB;
@@ -1289,7 +1364,9 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe16q_kernel(GemmParams p, 
     mma_and_fetch(fa0, fb0, fa1, Cfg::SINGLE_B ? fb0 : fb1, slot, 1, std::true_type{});
     // Step gs+1 has landed once at most the copies of the steps after it are outstanding (loads complete in
     // order; stores of an epilogue in between only make the count conservative).  The lgkmcnt wait is what
-    // allows this stage to be overwritten after the barrier.
+    // allows this stage to be overwritten after the barrier.  (Allowing for the epilogue's stores in the first
+    // waits of the next tile, through a uniform branch around the wait, was measured slower: 184 against 178 us
+    // at 8192x5120x5120.)
     asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"((STAGES - 2) * COPIES) : "memory");
     issue_copies();  // step gs+STAGES into the stage this step used
     slot = next_slot(slot);
@@ -1299,7 +1376,7 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe16q_kernel(GemmParams p, 
   auto finish_item = [&]() {
     const int b = item / tiles;
     int tile_m, tile_n;
-    tile_of_workgroup(item - b * tiles, tiles_m, tiles_n, tile_m, tile_n);
+    tile_of_workgroup(item - b * tiles, tiles_m, tiles_n, tile_m, tile_n, p.band);
     int lane_here = lane;  // opaque copy: keeps the epilogue's address arithmetic out of the mainloop
     asm volatile("" : "+v"(lane_here));
     if constexpr (Cfg::GROUPED) {
@@ -1676,7 +1753,12 @@ static int num_cus() {
 }
 
 template <class Cfg, class Kern, class... Extra>
-static int launch_persistent(Kern kern, const GemmParams& p, hipStream_t stream, Extra... extra) {
+static int launch_persistent(Kern kern, const GemmParams& p_in, hipStream_t stream, Extra... extra) {
+  GemmParams p = p_in;
+  // An XCD's 32 resident workgroups cover band x (32 / band) tiles per round and fetch band * BM + (32 / band) * BN
+  // panel rows for them: 8 x 4 is the minimum for square tiles, 4 x 8 for tiles that are much taller than wide
+  // (256x160: 2304 rows against 2688; measured 1 % faster, 5 % with 32-bit outputs at N = 20480).
+  p.band = 3 * Cfg::BN <= 2 * Cfg::BM ? 4 : 8;
   static std::atomic<unsigned long long> lds_ok{0};
   if (int rc = allow_lds(kern, Cfg::LDS_BYTES, lds_ok)) return rc;
   const int tiles_m = (p.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (p.N + Cfg::BN - 1) / Cfg::BN;

@@ -92,9 +92,11 @@ struct Epi<EPI_S8_BIAS> {
   static constexpr bool kHasBias = true;
   static constexpr bool kAccumulate = false;
   static __device__ __forceinline__ float bias_term(Bias b, float beta) { return beta * (float)(int)b; }
-  static __device__ __forceinline__ Out apply(int acc, float bt, float alpha) {
-    return (int8_t)rne_s8(__builtin_fmaf(alpha, (float)acc, bt));
+  // the output value as an int in [-128, 127] (for epilogues that pack bytes themselves)
+  static __device__ __forceinline__ int apply_int(int acc, float bt, float alpha) {
+    return rne_s8(__builtin_fmaf(alpha, (float)acc, bt));
   }
+  static __device__ __forceinline__ Out apply(int acc, float bt, float alpha) { return (int8_t)apply_int(acc, bt, alpha); }
 };
 template <>
 struct Epi<EPI_S8_RELU> {
@@ -103,10 +105,11 @@ struct Epi<EPI_S8_RELU> {
   static constexpr bool kHasBias = true;
   static constexpr bool kAccumulate = false;
   static __device__ __forceinline__ float bias_term(Bias b, float beta) { return beta * (float)(int)b; }
-  static __device__ __forceinline__ Out apply(int acc, float bt, float alpha) {
+  static __device__ __forceinline__ int apply_int(int acc, float bt, float alpha) {
     // relu then clamp == integer clamp to [0, 127] after rounding (NaN -> 0 either way)
-    return (int8_t)rne_clamp<0>(__builtin_fmaf(alpha, (float)acc, bt));
+    return rne_clamp<0>(__builtin_fmaf(alpha, (float)acc, bt));
   }
+  static __device__ __forceinline__ Out apply(int acc, float bt, float alpha) { return (int8_t)apply_int(acc, bt, alpha); }
 };
 template <>
 struct Epi<EPI_F32_SCALE> {
@@ -124,9 +127,8 @@ struct Epi<EPI_S8_SCALE> {
   static constexpr bool kHasBias = false;
   static constexpr bool kAccumulate = false;
   static __device__ __forceinline__ float bias_term(Bias, float) { return 0.0f; }
-  static __device__ __forceinline__ Out apply(int acc, float, float alpha) {
-    return (int8_t)rne_s8(alpha * (float)acc);
-  }
+  static __device__ __forceinline__ int apply_int(int acc, float, float alpha) { return rne_s8(alpha * (float)acc); }
+  static __device__ __forceinline__ Out apply(int acc, float bt, float alpha) { return (int8_t)apply_int(acc, bt, alpha); }
 };
 template <>
 struct Epi<EPI_S32_RAW> {
@@ -175,6 +177,8 @@ struct GemmParams {
   // stored as element [b][h][t][dd] of a packed [M/out_T, N/out_d, out_T, out_d] tensor -- the layout the
   // attention products want, written by the projection itself.  0 = plain row-major [M, N].  8-bit outputs only.
   int out_T = 0, out_d = 0;
+  // Tile rows an XCD's run of tiles walks down before it moves to the next tile column (see tile_of_workgroup).
+  int band = 8;
 };
 
 // Offset of output element (m, n) of one batch; consecutive n stay consecutive inside a head, so vector
