@@ -104,8 +104,9 @@ def test_c_abi_rejects_bad_arguments_without_a_device():
     lib.ti_attn_qk_softmax_q.argtypes = [ctypes.c_void_p] * 4 + [i64] * 7 + [ctypes.c_float, ctypes.c_void_p]
     lib.ti_attn_qk_softmax_q_supported.argtypes = [i64] * 3
     assert lib.ti_attn_qk_softmax_q_supported(512, 512, 128) == 1 and lib.ti_attn_qk_softmax_q_supported(1, 16, 128) == 1
-    assert lib.ti_attn_qk_softmax_q_supported(512, 528, 128) == 0 and lib.ti_attn_qk_softmax_q_supported(512, 40, 128) == 0
-    assert lib.ti_attn_qk_softmax_q_supported(512, 512, 64) == 0
+    assert lib.ti_attn_qk_softmax_q_supported(512, 528, 128) == 1 and lib.ti_attn_qk_softmax_q_supported(512, 40, 128) == 0
+    assert lib.ti_attn_qk_softmax_q_supported(512, 512, 64) == 1 and lib.ti_attn_qk_softmax_q_supported(2048, 4096, 64) == 1
+    assert lib.ti_attn_qk_softmax_q_supported(512, 4112, 128) == 0 and lib.ti_attn_qk_softmax_q_supported(512, 512, 96) == 0
     rc = lib.ti_attn_qk_softmax_q(p, p, None, p, 4, 64, 520, 128, 64 * 128, 520 * 128, 2, 1.0, None)
     assert rc == 1 and b"unsupported shape" in lib.ti_last_error()
     rc = lib.ti_attn_qk_softmax_q(p, p, None, p, 4, 64, 64, 128, 64 * 128, 63 * 128, 2, 1.0, None)
@@ -114,8 +115,8 @@ def test_c_abi_rejects_bad_arguments_without_a_device():
     assert rc == 2 and b"aligned" in lib.ti_last_error()
     assert lib.ti_attn_qk_softmax_q(None, None, None, None, 0, 64, 64, 128, 0, 0, 2, 1.0, None) == 0
     lib.ti_attn_prefill_s8.argtypes = [ctypes.c_void_p] * 5 + [i64] * 7 + [ctypes.c_float] * 2 + [ctypes.c_void_p]
-    rc = lib.ti_attn_prefill_s8(p, p, p, None, p, 4, 64, 80, 128, 64 * 128, 80 * 128, 2, 1.0, 1.0, None)
-    assert rc == 1 and b"multiple of 64" in lib.ti_last_error()
+    rc = lib.ti_attn_prefill_s8(p, p, p, None, p, 4, 64, 72, 128, 64 * 128, 72 * 128, 2, 1.0, 1.0, None)
+    assert rc == 1 and b"multiple of 16" in lib.ti_last_error()
     rc = lib.ti_attn_prefill_s8(p, p, None, None, p, 4, 64, 64, 128, 64 * 128, 64 * 128, 2, 1.0, 1.0, None)
     assert rc == 1 and b"vt is NULL" in lib.ti_last_error()
     assert lib.ti_attn_prefill_s8(None, None, None, None, None, 0, 64, 64, 128, 0, 0, 2, 1.0, 1.0, None) == 0

@@ -684,7 +684,7 @@ def test_fused_qk_softmax_matches_the_two_kernels_and_the_oracle():
         assert X.can_attn_qk_softmax_q(qd, buf[:, :S], md, B, H)
         assert torch.equal(X.attn_qk_softmax_q(qd, buf[:, :S], md, alpha, H), out)
     assert not X.can_attn_qk_softmax_q(qd, kd[:, :40], None, B, H)          # S not a multiple of 16
-    assert not X.can_attn_qk_softmax_q(qd[:, :, :64].contiguous(), kd[:, :, :64].contiguous(), None, B, H)
+    assert not X.can_attn_qk_softmax_q(qd[:, :, :32].contiguous(), kd[:, :, :32].contiguous(), None, B, H)   # head size 32
 
 
 def test_fused_prefill_attention_matches_the_chain():
@@ -711,7 +711,7 @@ def test_fused_prefill_attention_matches_the_chain():
         out = X.attn_prefill(qd, kd, vt, md, a_qk, a_pv, H)
         assert out.shape == (B, T, H * 128) and out.dtype == torch.int8
         assert torch.equal(out.cpu(), ref), (B, H, T, S, kind, (out.cpu() != ref).sum().item())
-    assert not X.can_attn_prefill(qd, kd[:, :432], vt[:, :, :432].contiguous(), None, B, H)   # S % 64 != 0
+    assert not X.can_attn_prefill(qd, kd[:, :440], vt[:, :, :440].contiguous(), None, B, H)   # S % 16 != 0
 
 
 def test_runs_are_deterministic():
@@ -802,3 +802,55 @@ def test_ln_q_fp16_residual_stream():
 def copy_to(module, dev):
     import copy
     return copy.deepcopy(module).to(dev)
+
+
+def _attn_masks(kind, B, T, S):
+    if kind is None:
+        return None
+    neg = torch.finfo(torch.float32).min
+    mask = torch.zeros(B, 1, T, S)
+    if kind == "causal":
+        mask += torch.zeros(T, S).masked_fill(torch.arange(S)[None, :] > torch.arange(T)[:, None] + (S - T), neg)
+    mask[0, :, :, :5] = neg      # left padding of the first batch row (adds up with causality, may overflow to -inf)
+    return mask
+
+
+def test_fused_attention_long_keys_and_head_size_64():
+    # more than 512 keys, key counts that are not multiples of 64, head size 64: the three-sweep kernel; the bytes of
+    # bmm_s8t_s8n_f32t -> attn_softmax_q (-> bmm_s8t_s8n_s8t -> head merge), from the oracle and from the device kernels
+    import torch_int._hip_ext as X
+    import torch_int._CUDA as C
+    g = torch.Generator().manual_seed(131)
+    # (batch, heads, T, S, head size, mask kind)
+    cases = [(1, 3, 2048, 2048, 128, "causal"), (2, 2, 100, 528, 128, "pad"), (1, 2, 64, 1040, 128, None),
+             (1, 2, 700, 1024, 128, "causal"), (1, 1, 17, 4096, 128, None), (2, 3, 512, 512, 64, "causal"),
+             (1, 4, 200, 208, 64, "pad"), (1, 2, 1500, 1536, 64, "causal"), (2, 2, 70, 48, 128, "causal"),
+             (1, 2, 33, 16, 64, None)]
+    for (B, H, T, S, d, kind) in cases:
+        _say(f"attn long B={B} H={H} T={T} S={S} d={d} mask={kind}")
+        q, k, v = _s8(g, B * H, T, d), _s8(g, B * H, S, d), _s8(g, B * H, S, d)
+        a_qk, a_pv = _scal(g, 2e-4, 2e-3), _scal(g, 2e-3, 2e-2)
+        mask = _attn_masks(kind, B, T, S)
+        probs_ref = orc.attn_softmax_q(orc.bmm_s8t_s8n_f32t(q, k, a_qk), mask, H)
+        ctx_ref = orc.bmm_s8t_s8t_s8t(probs_ref, v, a_pv).view(B, H, T, d).transpose(1, 2).reshape(B, T, H * d)
+        qd, kd, md = q.to(DEV), k.to(DEV), (mask.to(DEV) if mask is not None else None)
+        assert X.can_attn_qk_softmax_q(qd, kd, md, B, H)
+        probs = X.attn_qk_softmax_q(qd, kd, md, a_qk, H)
+        nbad = (probs.cpu() != probs_ref).sum().item()
+        assert nbad == 0, (B, H, T, S, d, kind, nbad)
+        assert torch.equal(probs, X.attn_softmax_q(C.bmm_s8t_s8n_f32t(qd, kd, a_qk), md, H))
+        vt = X.transpose_last2(v.to(DEV))
+        assert X.can_attn_prefill(qd, kd, vt, md, B, H)
+        ctx = X.attn_prefill(qd, kd, vt, md, a_qk, a_pv, H)
+        assert ctx.shape == (B, T, H * d)
+        nbad = (ctx.cpu() != ctx_ref).sum().item()
+        assert nbad == 0, (B, H, T, S, d, kind, nbad)
+        # keys read in place from a longer cache buffer (batch stride > S * d)
+        buf = torch.zeros(B * H, S + 48, d, dtype=torch.int8, device=DEV)
+        buf[:, :S] = kd
+        assert torch.equal(X.attn_prefill(qd, buf[:, :S], vt, md, a_qk, a_pv, H), ctx)
+    z = lambda *shape: torch.zeros(*shape, dtype=torch.int8, device=DEV)   # noqa: E731
+    assert X.can_attn_qk_softmax_q(z(2, 8, 64), z(2, 48, 64), None, 1, 2)
+    assert not X.can_attn_qk_softmax_q(z(2, 8, 64), z(2, 40, 64), None, 1, 2)      # S not a multiple of 16
+    assert not X.can_attn_qk_softmax_q(z(1, 8, 64), z(1, 4112, 64), None, 1, 1)    # more than 4096 keys
+    assert not X.can_attn_qk_softmax_q(z(2, 8, 32), z(2, 48, 32), None, 1, 2)      # head size 32

@@ -16,7 +16,7 @@ LIB_PATH = os.path.join(LIB_DIR, "libtorch_int_hip.so")
 # csrc/ti_common.h), each kind in a translation unit of its own, so that they build in parallel.
 SOURCES = [(s, [], s[:-4] + ".o") for s in
            ["api.hip", "gemm_s8.hip", "ln_q.hip", "softmax_q.hip", "permute.hip", "bmm_rowmajor.hip", "decode_attn.hip",
-            "attn_fused.hip", "diag_mfma.hip"]]
+            "attn_fused.hip", "attn_long.hip", "diag_mfma.hip"]]
 SOURCES += [("gemm_s8_kinds.hip", [f"-DTI_KIND={k}"], f"gemm_s8_kind{k}.o") for k in range(9)]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")

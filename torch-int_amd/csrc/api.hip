@@ -458,8 +458,8 @@ int ti_attn_qk_softmax_q(const int8_t* q, const int8_t* k, const float* mask, in
                                    (long long)BH, (long long)heads);
   if (BH == 0 || T == 0) return TI_OK;
   if (!attn_qk_softmax_q_supported(T, S, D))
-    return fail(TI_ERR_INVALID_ARG, "%s: unsupported shape T=%lld S=%lld head_dim=%lld (needs head_dim 128 and S a "
-                "multiple of 16 in [16, 512])", op, (long long)T, (long long)S, (long long)D);
+    return fail(TI_ERR_INVALID_ARG, "%s: unsupported shape T=%lld S=%lld head_dim=%lld (needs head_dim 64 or 128 and S "
+                "a multiple of 16 in [16, 4096])", op, (long long)T, (long long)S, (long long)D);
   if (stride_q < T * D || stride_k < S * D || stride_q % 16 != 0 || stride_k % 16 != 0)
     return fail(TI_ERR_INVALID_ARG, "%s: batch strides (%lld, %lld) must be multiples of 16 and cover one matrix", op,
                 (long long)stride_q, (long long)stride_k);
@@ -482,9 +482,9 @@ int ti_attn_prefill_s8(const int8_t* q, const int8_t* k, const int8_t* vt, const
   if (BH % heads != 0) return fail(TI_ERR_INVALID_ARG, "%s: BH = %lld is not a multiple of heads = %lld", op,
                                    (long long)BH, (long long)heads);
   if (BH == 0 || T == 0) return TI_OK;
-  if (!attn_qk_softmax_q_supported(T, S, D) || S % 64 != 0)
-    return fail(TI_ERR_INVALID_ARG, "%s: unsupported shape T=%lld S=%lld head_dim=%lld (needs head_dim 128 and S a "
-                "multiple of 64 in [64, 512])", op, (long long)T, (long long)S, (long long)D);
+  if (!attn_qk_softmax_q_supported(T, S, D))
+    return fail(TI_ERR_INVALID_ARG, "%s: unsupported shape T=%lld S=%lld head_dim=%lld (needs head_dim 64 or 128 and S "
+                "a multiple of 16 in [16, 4096])", op, (long long)T, (long long)S, (long long)D);
   if (stride_q < T * D || stride_k < S * D || stride_q % 16 != 0 || stride_k % 16 != 0)
     return fail(TI_ERR_INVALID_ARG, "%s: batch strides (%lld, %lld) must be multiples of 16 and cover one matrix", op,
                 (long long)stride_q, (long long)stride_k);

@@ -256,8 +256,19 @@ __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t*
   }
 }
 
+// attn_long.hip: any number of keys up to 4096 (a multiple of 16), head size 64 or 128, three sweeps over the keys
+bool attn_long_supported(long long T, long long S, long long D);
+int launch_attn_long(const int8_t* q, const int8_t* k, const float* mask, int8_t* probs, long long BH, long long T,
+                     long long S, long long D, long long stride_q, long long stride_k, long long heads, float alpha,
+                     const int8_t* vt, int8_t* ctx, float alpha_pv, hipStream_t stream);
+
+// shapes the single-sweep kernel of this file takes (all keys of a head in the LDS at once)
+static bool single_sweep_ok(long long T, long long S, long long D, bool pv) {
+  return T >= 1 && D == AF_D && S >= 16 && S <= AF_MAX_S && S % 16 == 0 && (!pv || S % 64 == 0);
+}
+
 bool attn_qk_softmax_q_supported(long long T, long long S, long long D) {
-  return T >= 1 && D == AF_D && S >= 16 && S <= AF_MAX_S && S % 16 == 0;
+  return single_sweep_ok(T, S, D, false) || attn_long_supported(T, S, D);
 }
 
 template <int NB, bool PV>
@@ -285,8 +296,8 @@ int launch_attn_qk_softmax_q(const int8_t* q, const int8_t* k, const float* mask
                              long long heads, float alpha, const int8_t* vt, int8_t* ctx, float alpha_pv,
                              hipStream_t stream) {
   if (BH == 0 || T == 0) return TI_OK;
-  if (!attn_qk_softmax_q_supported(T, S, D) || (vt != nullptr && S % 64 != 0))
-    return fail(TI_ERR_INVALID_ARG, "attn_qk_softmax_q: unsupported shape (T=%lld S=%lld head_dim=%lld)", T, S, D);
+  if (!single_sweep_ok(T, S, D, vt != nullptr))
+    return launch_attn_long(q, k, mask, probs, BH, T, S, D, stride_q, stride_k, heads, alpha, vt, ctx, alpha_pv, stream);
   const long long row_blocks = (T + AF_ROWS - 1) / AF_ROWS;
   if (BH * row_blocks > 0x7fffffffLL || T > 0x7fffffffLL)
     return fail(TI_ERR_INVALID_ARG, "attn_qk_softmax_q: too many row blocks (%lld)", BH * row_blocks);

@@ -1,0 +1,354 @@
+// Prefill attention for any number of keys and head sizes 64 / 128, without the fp32 score tensor in memory:
+// probs = round(127 softmax(max(alpha q.k^T + mask, lowest))) and, on request, context = s8(alpha_pv probs . V).
+// The bits are those of bmm_s8t_s8n_f32t -> attn_softmax_q -> bmm_s8t_s8n_s8t: the row maximum is taken over all
+// keys before any exponential, and the row sum adds the exponentials in the reference order (chunk c of four
+// consecutive keys belongs to partial sum c % 64, a partial sum takes its chunks in ascending order, the 64
+// partial sums meet in a xor butterfly 32 .. 1).  Because the sum needs the maximum and the probabilities need the
+// sum, the keys are swept three times, each sweep recomputing the int8 products (cheap on the matrix pipe):
+//   sweep 1  x = max(alpha acc + mask, lowest), running row maximum, and per key tile whether anything in it can
+//            have a non-zero probability (exp underflows to exactly 0 below -87);
+//   sweep 2  e = exp(x - m) over the live tiles, partial sums -> 127 / sum;
+//   sweep 3  e again, p = rint(e * 127 / sum), and either the store of p or p . V on the spot.
+// Tiles that are dead for the whole workgroup (keys above the diagonal of a causal mask) are skipped in sweeps
+// 2 and 3: they add exact zeros.
+//
+// One workgroup of four waves per (batch * head, block of 64 query rows); a wave owns 16 query rows.  Keys go
+// through the LDS in tiles of 256 (16 blocks of v_mfma_i32_16x16x64_i8 per wave): one tile is exactly one round
+// of the 64 partial sums, so lane (r, g) of a wave keeps 16 partial sums (block j of a tile = chunk 4 j + g) and
+// adds tile after tile to them.  Two workgroups share a CU; while one waits for its tile the other computes.
+#include "ti_common.h"
+#include "softmax_math.h"
+
+namespace ti {
+
+#define TI_GLOBAL_AS __attribute__((address_space(1)))
+#define TI_LDS_AS __attribute__((address_space(3)))
+
+constexpr int AL_ROWS = 64;      // query rows per workgroup
+constexpr int AL_TILE = 256;     // keys per tile
+constexpr int AL_MAX_TILES = 16; // live-tile bit mask: S <= 4096
+constexpr int AL_VPITCH = AL_TILE + 16;
+
+// 16-byte chunk c of row `row` of a panel whose rows hold D bytes sits at this chunk position
+template <int D>
+__device__ __forceinline__ int al_swz(int row, int c) {
+  return D == 128 ? (c ^ ((row >> 1) & 7)) : (c ^ ((row >> 2) & 3));
+}
+
+template <int D, bool PV>
+__global__ __launch_bounds__(256, 2) void attn_long_kernel(const int8_t* __restrict__ q, const int8_t* __restrict__ k,
+                                                           const float* __restrict__ mask, int8_t* __restrict__ probs,
+                                                           int T, int S, long long stride_q, long long stride_k,
+                                                           int heads, int row_blocks, float alpha,
+                                                           const int8_t* __restrict__ vt, int8_t* __restrict__ ctx,
+                                                           float alpha_pv) {
+  constexpr int CH = D / 16;       // 16-byte chunks per row
+  constexpr int KS = D / 64;       // MFMAs (64 bytes of head dimension each) per block
+  constexpr int RPI = 1024 / D;    // panel rows one copy instruction fills
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  char* qs_base = smem;                          // [64][D]
+  char* ks_base = smem + AL_ROWS * D;            // [256][D]
+  char* vs_base = ks_base + AL_TILE * D;         // [D][AL_VPITCH]            (PV only)
+  int* flags = reinterpret_cast<int*>(vs_base + (PV ? D * AL_VPITCH : 0));  // [4] live-tile masks of the waves
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n_bh = gridDim.x / row_blocks;
+  const long long bh = blockIdx.x % n_bh;
+  const int t0 = (row_blocks - 1 - (int)(blockIdx.x / n_bh)) * AL_ROWS;  // heaviest blocks of a causal mask first
+  const int ntiles = (S + AL_TILE - 1) / AL_TILE;
+  const int r = lane & 15, g = lane >> 4;
+
+  const int8_t* qb = q + bh * stride_q;
+  const int8_t* kb = k + bh * stride_k;
+  // ---- Q tile, once
+  for (int i = wave; i < AL_ROWS / RPI; i += 4) {
+    const int row = i * RPI + lane / CH, pos = lane % CH;
+    const int t = t0 + row < T ? t0 + row : T - 1;  // rows past the end repeat the last one; never stored
+    __builtin_amdgcn_global_load_lds((const TI_GLOBAL_AS void*)(qb + (long long)t * D + (al_swz<D>(row, pos) << 4)),
+                                     (TI_LDS_AS void*)((TI_LDS_AS char*)qs_base + i * 1024), 16, 0, 0);
+  }
+  auto load_k_tile = [&](int tile) {
+    const int k0 = tile * AL_TILE;
+    const int nkeys = S - k0 < AL_TILE ? S - k0 : AL_TILE;  // a multiple of 16
+    for (int i = wave; i < nkeys / RPI; i += 4) {
+      const int row = i * RPI + lane / CH, pos = lane % CH;
+      __builtin_amdgcn_global_load_lds(
+          (const TI_GLOBAL_AS void*)(kb + (long long)(k0 + row) * D + (al_swz<D>(row, pos) << 4)),
+          (TI_LDS_AS void*)((TI_LDS_AS char*)ks_base + i * 1024), 16, 0, 0);
+    }
+  };
+  auto load_v_tile = [&](int tile) {
+    if constexpr (PV) {
+      const int k0 = tile * AL_TILE;
+      const int nkeys = S - k0 < AL_TILE ? S - k0 : AL_TILE;
+      const int8_t* vb = vt + bh * (long long)D * S + k0;
+      for (int i = wave; i < (D * AL_VPITCH) / 1024; i += 4) {
+        const int o = i * 1024 + lane * 16;
+        const int row = o / AL_VPITCH;
+        int col = o - row * AL_VPITCH;
+        col = col < nkeys ? col : 0;  // pad bytes and columns past the last key get a copy of chunk 0: multiplied by p = 0
+        __builtin_amdgcn_global_load_lds((const TI_GLOBAL_AS void*)(vb + (long long)row * S + col),
+                                         (TI_LDS_AS void*)((TI_LDS_AS char*)vs_base + i * 1024), 16, 0, 0);
+      }
+    }
+  };
+
+  const int t = t0 + wave * 16 + r;
+  const int tc = t < T ? t : T - 1;
+  const float* mrow = mask != nullptr ? mask + (((bh / heads) * T + tc) * (long long)S) : nullptr;
+  const float lowest = -3.402823466e+38f;
+  const char* qs = qs_base + (wave * 16 + r) * D;
+  const char* ks = ks_base + r * D;
+
+  // x of one tile: acc[j][v] <- bits of max(alpha * (q . k) + mask, lowest) for block j, keys 16 j + 4 g + v
+  v4i acc[16];
+  v4i qf[KS];
+  auto tile_scores = [&](int tile, int nb) {
+    const int k0 = tile * AL_TILE;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      acc[j] = v4i{0, 0, 0, 0};
+      if (j < nb) {
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+          const v4i kf = *reinterpret_cast<const v4i*>(ks + j * 16 * D + (al_swz<D>(r, 4 * s + g) << 4));
+          acc[j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(kf, qf[s], acc[j], 0, 0, 0);
+        }
+      }
+    }
+    // mask values four blocks at a time, the next four in flight while these are used
+    v4f mk[2][4];
+    auto fetch_mask = [&](int j0, v4f (&dst)[4]) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        dst[u] = v4f{0.f, 0.f, 0.f, 0.f};
+        if (mrow != nullptr && j0 + u < nb) dst[u] = *reinterpret_cast<const v4f*>(mrow + k0 + 16 * (j0 + u) + 4 * g);
+      }
+    };
+    fetch_mask(0, mk[0]);
+#pragma unroll
+    for (int j0 = 0; j0 < 16; j0 += 4) {
+      const int cur = (j0 >> 2) & 1;
+      if (j0 + 4 < 16) fetch_mask(j0 + 4, mk[cur ^ 1]);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int j = j0 + u;
+        if (j < nb) {
+#pragma unroll
+          for (int v = 0; v < 4; ++v) {
+            float x = Epi<EPI_F32_SCALE>::apply(acc[j][v], 0.0f, alpha);
+            if (mrow != nullptr) x = x + mk[cur][u][v];
+            x = __builtin_fmaxf(x, lowest);  // NaN included
+            acc[j][v] = __float_as_int(x);
+          }
+        }
+      }
+    }
+  };
+  auto blocks_of = [&](int tile) {
+    const int left = S - tile * AL_TILE;
+    return (left < AL_TILE ? left : AL_TILE) >> 4;
+  };
+
+  // ---- sweep 1: row maximum and the largest x of every tile
+  float m = lowest;
+  float tmax[AL_MAX_TILES];
+#pragma unroll
+  for (int i = 0; i < AL_MAX_TILES; ++i) tmax[i] = lowest;
+#pragma unroll 1
+  for (int tile = 0; tile < ntiles; ++tile) {
+    __syncthreads();  // every wave is done with the previous tile
+    load_k_tile(tile);
+    asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+    if (tile == 0) {
+#pragma unroll
+      for (int s = 0; s < KS; ++s) qf[s] = *reinterpret_cast<const v4i*>(qs + (al_swz<D>(wave * 16 + r, 4 * s + g) << 4));
+    }
+    const int nb = blocks_of(tile);
+    tile_scores(tile, nb);
+    float top = lowest;
+#pragma unroll
+    for (int j = 0; j < 16; ++j)
+      if (j < nb)
+        top = __builtin_fmaxf(top, __builtin_fmaxf(__builtin_fmaxf(__int_as_float(acc[j][0]), __int_as_float(acc[j][1])),
+                                                   __builtin_fmaxf(__int_as_float(acc[j][2]), __int_as_float(acc[j][3]))));
+    m = __builtin_fmaxf(m, top);
+#pragma unroll
+    for (int i = 0; i < AL_MAX_TILES; ++i)
+      if (i == tile) tmax[i] = top;
+  }
+  {
+    float o = __shfl_xor(m, 16, 64);
+    m = m > o ? m : o;
+    o = __shfl_xor(m, 32, 64);
+    m = m > o ? m : o;
+  }
+  // tiles with something above exp's cut-off in this wave, then in the workgroup
+  unsigned live_w = 0;
+#pragma unroll
+  for (int i = 0; i < AL_MAX_TILES; ++i)
+    if (i < ntiles && __builtin_amdgcn_ballot_w64(tmax[i] - m > -87.0f) != 0) live_w |= 1u << i;
+  if (lane == 0) flags[wave] = (int)live_w;
+  __syncthreads();
+  const unsigned live_g = (unsigned)(flags[0] | flags[1] | flags[2] | flags[3]);
+
+  // ---- sweep 2: the row sum, in the reference order
+  float part[16];
+#pragma unroll
+  for (int jj = 0; jj < 16; ++jj) part[jj] = 0.0f;
+#pragma unroll 1
+  for (int tile = 0; tile < ntiles; ++tile) {
+    if (!(live_g >> tile & 1)) continue;  // uniform over the workgroup
+    __syncthreads();
+    load_k_tile(tile);
+    asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+    if (!(live_w >> tile & 1)) continue;  // uniform over the wave: every e is 0, p + 0 = p
+    const int nb = blocks_of(tile);
+    tile_scores(tile, nb);
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      if (j < nb) {
+        const float top = __builtin_fmaxf(__builtin_fmaxf(__int_as_float(acc[j][0]), __int_as_float(acc[j][1])),
+                                          __builtin_fmaxf(__int_as_float(acc[j][2]), __int_as_float(acc[j][3])));
+        if (__builtin_amdgcn_ballot_w64(top - m > -87.0f) != 0) {
+          float p = part[j];
+#pragma unroll
+          for (int v = 0; v < 4; ++v) p = p + exp_nonpos(__int_as_float(acc[j][v]) - m);
+          part[j] = p;
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int w = 8; w >= 1; w >>= 1)
+#pragma unroll
+    for (int jj = 0; jj < w; ++jj) part[jj] = part[jj] + part[jj + w];
+  float sum = part[0];
+  sum = sum + __shfl_xor(sum, 32, 64);
+  sum = sum + __shfl_xor(sum, 16, 64);
+  const float scale = 127.0f / sum;
+
+  // ---- sweep 3: probabilities, stored or multiplied with V
+  v4i o[CH];
+#pragma unroll
+  for (int c = 0; c < CH; ++c) o[c] = v4i{0, 0, 0, 0};
+  const char* vrow = vs_base + r * AL_VPITCH + 4 * g;  // V^T row (= head-dimension index) r of block c is 16 c + r
+  int8_t* prow = probs != nullptr ? probs + (bh * T + tc) * (long long)S : nullptr;
+#pragma unroll 1
+  for (int tile = 0; tile < ntiles; ++tile) {
+    const bool tile_live = live_g >> tile & 1;
+    const int nb = blocks_of(tile);
+    if (tile_live) {
+      __syncthreads();
+      load_k_tile(tile);
+      load_v_tile(tile);
+      asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+    }
+    const bool wave_live = live_w >> tile & 1;
+    if (PV && !wave_live) continue;
+    unsigned pw[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) pw[j] = 0;
+    if (wave_live) {
+      tile_scores(tile, nb);
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        if (j < nb) {
+          const float top = __builtin_fmaxf(__builtin_fmaxf(__int_as_float(acc[j][0]), __int_as_float(acc[j][1])),
+                                            __builtin_fmaxf(__int_as_float(acc[j][2]), __int_as_float(acc[j][3])));
+          if (__builtin_amdgcn_ballot_w64(top - m > -87.0f) != 0) {
+            unsigned w = 0;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+              const float pq = __builtin_rintf(exp_nonpos(__int_as_float(acc[j][v]) - m) * scale);  // in [0, 127]
+              w |= (unsigned)(int)pq << (8 * v);
+            }
+            pw[j] = w;
+          }
+        }
+      }
+    }
+    if constexpr (PV) {
+#pragma unroll
+      for (int sl = 0; sl < 4; ++sl) {
+        if (4 * sl < nb) {
+          const v4i pa = {(int)pw[4 * sl], (int)pw[4 * sl + 1], (int)pw[4 * sl + 2], (int)pw[4 * sl + 3]};
+#pragma unroll
+          for (int c = 0; c < CH; ++c) {
+            const char* src = vrow + c * 16 * AL_VPITCH + 64 * sl;
+            const v4i vf = {*reinterpret_cast<const int*>(src), *reinterpret_cast<const int*>(src + 16),
+                            *reinterpret_cast<const int*>(src + 32), *reinterpret_cast<const int*>(src + 48)};
+            o[c] = __builtin_amdgcn_mfma_i32_16x16x64_i8(vf, pa, o[c], 0, 0, 0);
+          }
+        }
+      }
+    } else {
+      // four consecutive keys per lane and block; dead tiles and blocks store their zeros
+      int* dst = reinterpret_cast<int*>(prow + tile * AL_TILE) + g;
+      if (t < T) {
+#pragma unroll
+        for (int j = 0; j < 16; ++j)
+          if (j < nb) dst[4 * j] = (int)pw[j];
+      }
+    }
+  }
+  if constexpr (PV) {
+    if (t < T) {
+      const long long b = bh / heads, h = bh - b * heads;
+      int* crow = reinterpret_cast<int*>(ctx + ((b * T + t) * heads + h) * (long long)D) + g;
+#pragma unroll
+      for (int c = 0; c < CH; ++c) {
+        unsigned w = 0;
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+          w |= (unsigned)(unsigned char)Epi<EPI_S8_SCALE>::apply(o[c][v], 0.0f, alpha_pv) << (8 * v);
+        crow[4 * c] = (int)w;
+      }
+    }
+  }
+}
+
+bool attn_long_supported(long long T, long long S, long long D) {
+  return T >= 1 && (D == 64 || D == 128) && S >= 16 && S % 16 == 0 && S <= (long long)AL_TILE * AL_MAX_TILES;
+}
+
+template <int D, bool PV>
+static int launch_al(dim3 grid, hipStream_t stream, const int8_t* q, const int8_t* k, const float* mask, int8_t* probs,
+                     int T, int S, long long stride_q, long long stride_k, int heads, int row_blocks, float alpha,
+                     const int8_t* vt, int8_t* ctx, float alpha_pv) {
+  auto kern = attn_long_kernel<D, PV>;
+  constexpr int lds = AL_ROWS * D + AL_TILE * D + (PV ? D * AL_VPITCH : 0) + 16;
+  static_assert(2 * lds <= 160 * 1024, "two workgroups per CU");
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+  if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "attn_long: LDS limit: %s", hipGetErrorString(e));
+  hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, q, k, mask, probs, T, S, stride_q, stride_k, heads, row_blocks,
+                     alpha, vt, ctx, alpha_pv);
+  e = hipGetLastError();
+  if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "attn_long launch: %s", hipGetErrorString(e));
+  return TI_OK;
+}
+
+// vt == nullptr: probabilities into probs ([BH, T, S]).  Otherwise context into ctx ([BH / heads, T, heads * D]).
+int launch_attn_long(const int8_t* q, const int8_t* k, const float* mask, int8_t* probs, long long BH, long long T,
+                     long long S, long long D, long long stride_q, long long stride_k, long long heads, float alpha,
+                     const int8_t* vt, int8_t* ctx, float alpha_pv, hipStream_t stream) {
+  if (BH == 0 || T == 0) return TI_OK;
+  if (!attn_long_supported(T, S, D))
+    return fail(TI_ERR_INVALID_ARG, "attn_long: unsupported shape (T=%lld S=%lld head_dim=%lld)", T, S, D);
+  const long long row_blocks = (T + AL_ROWS - 1) / AL_ROWS;
+  if (BH * row_blocks > 0x7fffffffLL || T > 0x7fffffffLL)
+    return fail(TI_ERR_INVALID_ARG, "attn_long: too many row blocks (%lld)", BH * row_blocks);
+  const dim3 grid((unsigned)(BH * row_blocks));
+#define TI_AL(DD, PV)                                                                                          \
+  return launch_al<DD, PV>(grid, stream, q, k, mask, probs, (int)T, (int)S, stride_q, stride_k, (int)heads,  \
+                           (int)row_blocks, alpha, vt, ctx, alpha_pv)
+  if (D == 128) {
+    if (vt == nullptr) TI_AL(128, false);
+    TI_AL(128, true);
+  }
+  if (vt == nullptr) TI_AL(64, false);
+  TI_AL(64, true);
+#undef TI_AL
+}
+
+}  // namespace ti

@@ -297,8 +297,8 @@ def kv_append(k_new, v_new, k_buf, v_buf, filled, checked=False):
 
 
 def can_attn_qk_softmax_q(q, k, mask, bsz, heads):
-    """int8 HIP q [bsz*heads, T, 128] contiguous and k [bsz*heads, S, 128] with packed rows (any batch stride that is
-    a multiple of 16), S a multiple of 16 up to 512; mask None or fp32 [bsz, 1, T, S] contiguous."""
+    """int8 HIP q [bsz*heads, T, d] contiguous and k [bsz*heads, S, d] with packed rows (any batch stride that is
+    a multiple of 16), d 64 or 128, S a multiple of 16 up to 4096; mask None or fp32 [bsz, 1, T, S] contiguous."""
     if not (_ok(q, torch.int8) and type(k) is torch.Tensor and k.dtype is torch.int8 and k.is_cuda and q.dim() == 3
             and k.dim() == 3 and q.shape[0] == k.shape[0] == bsz * heads and q.shape[2] == k.shape[2]
             and k.device == q.device and q.numel() > 0):
@@ -317,8 +317,8 @@ def attn_qk_softmax_q(q, k, mask, alpha, heads, checked=False):
     """int8 round(127 softmax(alpha q k^T + mask)) [bsz*heads, T, S] in one launch: the values of
     ``attn_softmax_q(bmm_s8t_s8n_f32t(q, k, alpha), mask, heads)`` without the fp32 scores in memory."""
     if not checked and not can_attn_qk_softmax_q(q, k, mask, q.shape[0] // heads, heads):
-        raise RuntimeError("torch_int._hip_ext.attn_qk_softmax_q: needs int8 HIP q [B*H,T,128] / k [B*H,S,128] (S a "
-                           "multiple of 16 up to 512) and an fp32 mask [B,1,T,S] or None")
+        raise RuntimeError("torch_int._hip_ext.attn_qk_softmax_q: needs int8 HIP q [B*H,T,d] / k [B*H,S,d] (d 64 or 128, "
+                           "S a multiple of 16 up to 4096) and an fp32 mask [B,1,T,S] or None")
     BH, T, d = q.shape
     S = k.shape[1]
     dev = q.device
@@ -333,8 +333,8 @@ def attn_qk_softmax_q(q, k, mask, alpha, heads, checked=False):
 
 
 def can_attn_prefill(q, k, vt, mask, bsz, heads):
-    """``can_attn_qk_softmax_q`` plus: S a multiple of 64 and vt = V transposed, int8 [bsz*heads, 128, S] contiguous."""
-    return (can_attn_qk_softmax_q(q, k, mask, bsz, heads) and k.shape[1] % 64 == 0 and _ok(vt, torch.int8)
+    """``can_attn_qk_softmax_q`` plus: vt = V transposed, int8 [bsz*heads, d, S] contiguous."""
+    return (can_attn_qk_softmax_q(q, k, mask, bsz, heads) and _ok(vt, torch.int8)
             and vt.shape == (q.shape[0], q.shape[2], k.shape[1]) and vt.device == q.device and vt.data_ptr() % 16 == 0)
 
 
@@ -343,8 +343,8 @@ def attn_prefill(q, k, vt, mask, alpha_qk, alpha_pv, heads, checked=False):
     merge_heads(bmm_s8t_s8n_s8t(attn_qk_softmax_q(q, k, mask, alpha_qk), vt, alpha_pv)), the same bits, without the
     score and probability tensors."""
     if not checked and not can_attn_prefill(q, k, vt, mask, q.shape[0] // heads, heads):
-        raise RuntimeError("torch_int._hip_ext.attn_prefill: needs int8 HIP q [B*H,T,128], k [B*H,S,128], vt [B*H,128,S] "
-                           "(S a multiple of 64 up to 512) and an fp32 mask [B,1,T,S] or None")
+        raise RuntimeError("torch_int._hip_ext.attn_prefill: needs int8 HIP q [B*H,T,d], k [B*H,S,d], vt [B*H,d,S] "
+                           "(d 64 or 128, S a multiple of 16 up to 4096) and an fp32 mask [B,1,T,S] or None")
     BH, T, d = q.shape
     S = k.shape[1]
     dev = q.device
