@@ -88,7 +88,7 @@ def build_sweep(torch, C, dev):
                     if v == "b8_o8":
                         return lambda: C.linear_a8_w8_b8_o8(x, w, b, a, be)
                     return lambda: C.linear_relu_a8_w8_b8_o8(x, w, b, a, be)
-                cases.append({"variant": v, "M": M, "N": N, "K": K, "fn": make(w), "make": make, "w": w,
+                cases.append({"variant": v, "M": M, "N": N, "K": K, "fn": make(w), "make": make, "w": w, "x": x, "b": bias[v],
                               "ops": 2.0 * M * N * K, "bytes": float(gemm_bytes(M, N, K, v))})
     return cases
 
@@ -116,13 +116,16 @@ def sustained_ms(torch, fns, window_ms=200.0, warm_launches=100):
     return start.elapsed_time(end) / iters
 
 
-def cpu_baseline(torch):
+def cpu_baseline(torch, C=None, dev=None):
     """torch CPU int32 matmul + the oracle's fp32 epilogue (the reference's integer emulation), on an M=256
-    slice of each of the sweep's three (N, K) shapes, all four variants: 10-20 s of CPU work."""
+    slice of each of the sweep's three (N, K) shapes, all four variants: 10-20 s of CPU work.  The same twelve
+    problems then run through the HIP path and every output element is compared with the CPU result (the oracle
+    as the checker): `gpu_outputs_checked` / `gpu_mismatches`."""
     from oracle import oracle as orc
     g = torch.Generator().manual_seed(0)
     M = 256
     ops = dt = 0.0
+    checked = bad = 0
     for N, K in SHAPES:
         x = torch.randint(-127, 128, (M, K), dtype=torch.int8, generator=g)
         w = torch.randint(-127, 128, (N, K), dtype=torch.int8, generator=g)
@@ -130,16 +133,50 @@ def cpu_baseline(torch):
         b32 = torch.randint(-65535, 65535, (N,), dtype=torch.int32, generator=g)
         bf = torch.randn(N, generator=g)
         t0 = time.perf_counter()
-        orc.linear_a8_w8_b32_o32(x, w, b32, acc_fn=orc.gemm_acc_torch)
-        orc.linear_a8_w8_bfp32_ofp32(x, w, bf, 0.001, 1.0, acc_fn=orc.gemm_acc_torch)
-        orc.linear_a8_w8_b8_o8(x, w, b8, 0.001, 0.01, acc_fn=orc.gemm_acc_torch)
-        orc.linear_relu_a8_w8_b8_o8(x, w, b8, 0.001, 0.01, acc_fn=orc.gemm_acc_torch)
+        refs = [orc.linear_a8_w8_b32_o32(x, w, b32, acc_fn=orc.gemm_acc_torch),
+                orc.linear_a8_w8_bfp32_ofp32(x, w, bf, 0.001, 1.0, acc_fn=orc.gemm_acc_torch),
+                orc.linear_a8_w8_b8_o8(x, w, b8, 0.001, 0.01, acc_fn=orc.gemm_acc_torch),
+                orc.linear_relu_a8_w8_b8_o8(x, w, b8, 0.001, 0.01, acc_fn=orc.gemm_acc_torch)]
         dt += time.perf_counter() - t0
         ops += 4 * 2.0 * M * N * K
+        if C is not None:
+            xd, wd = x.to(dev), w.to(dev)
+            outs = [C.linear_a8_w8_b32_o32(xd, wd, b32.to(dev)), C.linear_a8_w8_bfp32_ofp32(xd, wd, bf.to(dev), 0.001, 1.0),
+                    C.linear_a8_w8_b8_o8(xd, wd, b8.to(dev), 0.001, 0.01),
+                    C.linear_relu_a8_w8_b8_o8(xd, wd, b8.to(dev), 0.001, 0.01)]
+            for out, ref in zip(outs, refs):
+                checked += ref.numel()
+                bad += int((out.cpu() != ref).sum())
     shapes = ", ".join(f"{N}x{K}" for N, K in SHAPES)
-    return {"value": ops / dt / 1e12, "unit": "TOPS", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": f"4 variants x M={M} rows of each (N,K) in {{{shapes}}}: torch int32 matmul + fp32 epilogue, "
-                      f"{dt:.1f} s, host cpu_count={os.cpu_count()}"}
+    res = {"value": ops / dt / 1e12, "unit": "TOPS", "cores": torch.get_num_threads(), "kind": "port",
+           "sample": f"4 variants x M={M} rows of each (N,K) in {{{shapes}}}: torch int32 matmul + fp32 epilogue, "
+                     f"{dt:.1f} s, host cpu_count={os.cpu_count()}"}
+    if C is not None:
+        res["gpu_outputs_checked"] = checked
+        res["gpu_mismatches"] = bad
+    return res
+
+
+def check_timed_outputs(torch, cases):
+    """Every timed b32_o32 case (integer result: acc + bias) against an fp64 product computed by torch on the device,
+    on the first and last eight rows of the output, all columns: ties the launches that are timed to correct
+    accumulators at the timed shapes without leaving the GPU.  Returns (elements checked, mismatches)."""
+    checked = bad = 0
+    for c in cases:
+        if c["variant"] != "b32_o32":
+            continue
+        out = c["fn"]()
+        M = c["M"]
+        rows = sorted(set(range(min(M, 8))) | set(range(max(M - 8, 0), M)))
+        x, w, b = c["x"], c["w"], c["b"]
+        ref = torch.zeros((len(rows), c["N"]), dtype=torch.float64, device=out.device)
+        xs = x[rows].double()
+        for k0 in range(0, c["K"], 2560):   # fp64 is exact here; slices keep the converted weights small
+            ref += xs[:, k0:k0 + 2560] @ w[:, k0:k0 + 2560].double().t()
+        ref = (ref.round().long() + b.long()[None]).to(torch.int32)
+        checked += ref.numel()
+        bad += int((out[rows] != ref).sum())
+    return checked, bad
 
 
 def hbm_kernels(torch, C, dev):
@@ -149,10 +186,10 @@ def hbm_kernels(torch, C, dev):
     g = torch.Generator().manual_seed(1)
 
     def rot(t, total_bytes):
-        n = max(2, -(-320 * 2 ** 20 // total_bytes))
+        n = min(8, max(2, -(-320 * 2 ** 20 // total_bytes)))
         return [t] + [t.clone() for _ in range(n - 1)]
 
-    for S in (512,):
+    for S in (128, 512, 2048):
         q = torch.randint(-127, 128, (160, S, 128), dtype=torch.int8, generator=g).to(dev)
         k = torch.randint(-127, 128, (160, S, 128), dtype=torch.int8, generator=g).to(dev)
         p = torch.randint(0, 128, (160, S, S), dtype=torch.int8, generator=g).to(dev)
@@ -167,6 +204,18 @@ def hbm_kernels(torch, C, dev):
         by = 160.0 * (S * S + 128 * S + S * 128)
         out.append({"kernel": "bmm_s8t_s8n_s8t", "shape": [160, S, 128, S], "us": ms * 1e3,
                     "GBps": by / ms / 1e6, "frac": by / ms / 1e6 / PEAK_HBM_GBS})
+        # the whole attention of a prefill in one launch (no counterpart upstream; replaces the two products above, the
+        # softmax chain and the head merge): bytes = q, k, v^T, context and one pass over the causal mask
+        if S >= 512:
+            import torch_int._hip_ext as X
+            neg = torch.finfo(torch.float32).min
+            mask = torch.zeros(S, S, device=dev).masked_fill(torch.triu(torch.ones(S, S, dtype=torch.bool, device=dev), 1), neg)
+            mask = mask[None, None].expand(4, 1, S, S).contiguous()
+            ms = sustained_ms(torch, [lambda: X.attn_prefill(q, k, vt, mask, 0.002, 0.004, 40)], window_ms=60.0, warm_launches=10)
+            by = 160.0 * 4 * S * 128 + 4.0 * 4 * S * S
+            out.append({"kernel": "attn_prefill (fused, causal mask)", "shape": [160, S, S, 128], "us": ms * 1e3,
+                        "GBps": by / ms / 1e6, "frac": by / ms / 1e6 / PEAK_HBM_GBS, "bound": "valu"})
+        del p, ps, ks
     rows, H = 2048, 5120
     inp = torch.randint(-65536, 65536, (rows, H), dtype=torch.int32, generator=g).to(dev)
     res = torch.randn(rows, H, generator=g).to(dev)
@@ -176,6 +225,13 @@ def hbm_kernels(torch, C, dev):
                       window_ms=60.0)
     by = 13.0 * rows * H + 8 * H
     out.append({"kernel": "dq_add_layernorm_q", "shape": [rows, H], "us": ms * 1e3,
+                "GBps": by / ms / 1e6, "frac": by / ms / 1e6 / PEAK_HBM_GBS})
+    pairs16 = [(i, r.half()) for i, r in pairs]
+    g16, b16 = gamma.half(), beta.half()
+    ms = sustained_ms(torch, [lambda i=i, r=r: C.dq_add_layernorm_q(i, 0.01, r, g16, b16, 1e-5) for i, r in pairs16],
+                      window_ms=60.0)
+    by = 9.0 * rows * H + 4 * H
+    out.append({"kernel": "dq_add_layernorm_q (fp16 residual)", "shape": [rows, H], "us": ms * 1e3,
                 "GBps": by / ms / 1e6, "frac": by / ms / 1e6 / PEAK_HBM_GBS})
     return out
 
@@ -284,6 +340,10 @@ def main():
     }
 
     achieved = dom_ops / dom_ms / 1e9
+    n_checked, n_bad = check_timed_outputs(torch, cases)
+    result["outputs_checked"] = {"elements": n_checked, "mismatches": n_bad,
+                                 "what": "the 18 timed b32_o32 cases, first and last 8 rows, against an fp64 product on the "
+                                         "device; cpu_baseline.gpu_mismatches covers the other epilogues at M = 256"}
     result["roofline"] = {
         "bound": "mfma", "achieved": achieved, "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
         "frac": achieved / PEAK_INT8_TOPS, "traffic": FAMILIES.get(DOMINANT, {}).get("traffic"),
@@ -345,7 +405,7 @@ def main():
         result["hbm_kernels"] = hbm_kernels(torch, C, dev)
         result["decoder_layer_ms"] = decoder_layer_ms(torch, dev)
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(torch)
+        result["cpu_baseline"] = cpu_baseline(torch, C, dev)
     print(json.dumps(result), flush=True)
 
 
