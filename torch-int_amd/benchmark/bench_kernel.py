@@ -40,7 +40,7 @@ LINEAR = {
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--op", required=True, choices=list(LINEAR) + ["bmm_f32t", "bmm_s8t", "bmm_s32t", "bmm_s8t_rowmajor", "ln_q", "add_ln_q",
+    ap.add_argument("--op", required=True, choices=list(LINEAR) + ["bmm_f32t", "bmm_s8t", "bmm_s32t", "bmm_s8t_rowmajor", "ln_q", "ln_q_f16", "add_ln_q",
                                                "softmax_q", "qk_softmax_q", "attn_prefill", "decode_attn", "copy",
                                                "mfma_loop", "mfma_ceiling"])
     ap.add_argument("--shape", type=int, nargs="+", required=True)
@@ -158,6 +158,13 @@ def main():
         gamma, beta = torch.ones(H, device=dev), torch.zeros(H, device=dev)
         fn = lambda: C.dq_add_layernorm_q(inp, 0.01, res, gamma, beta, 1e-5)  # noqa: E731
         nbytes = 13.0 * rows * H + 8 * H
+    elif args.op == "ln_q_f16":
+        rows, H = args.shape
+        inp = torch.randint(-4096, 4096, (rows, H), dtype=torch.int32, device=dev, generator=g)
+        res = torch.randn(rows, H, device=dev, generator=g).half()
+        gamma, beta = torch.ones(H, device=dev).half(), torch.zeros(H, device=dev).half()
+        fn = lambda: C.dq_add_layernorm_q(inp, 0.01, res, gamma, beta, 1e-5)  # noqa: E731
+        nbytes = 9.0 * rows * H + 4 * H
     elif args.op == "mfma_loop":
         mode, steps = args.shape
         data = (torch.full((1 << 20,), 1, dtype=torch.int8, device=dev) if args.pattern == "constant"
