@@ -294,13 +294,22 @@ def main():
     marks = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in heavy]
              for _ in range(args.steps)]
 
-    def step(ev=None):
+    # A pair of event records costs the stream about 10 us (the command processor serialises on each), which is
+    # 4 % of a step if every heavy launch of every step carries one.  Each timed step therefore brackets a
+    # rotating quarter of them: launch k in the steps i with (k + i) % stride == 0, so every launch is sampled in
+    # steps / stride of the timed steps and every step carries the same share of the overhead.
+    stride = max(1, min(4, args.steps))
+
+    def step(ev=None, i=0):
         k = 0
         for c in cases:
-            if ev is not None and c["M"] >= 512:
-                ev[k][0].record()
-                c["fn"]()
-                ev[k][1].record()
+            if c["M"] >= 512:
+                if ev is not None and (k + i) % stride == 0:
+                    ev[k][0].record()
+                    c["fn"]()
+                    ev[k][1].record()
+                else:
+                    c["fn"]()
                 k += 1
             else:
                 c["fn"]()
@@ -310,16 +319,22 @@ def main():
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(args.steps):
-        step(marks[i])
+        step(marks[i], i)
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    def launch_ms(k):   # mean duration of heavy launch k over the steps that bracketed it
+        took = [marks[i][k][0].elapsed_time(marks[i][k][1]) for i in range(args.steps) if (k + i) % stride == 0]
+        return sum(took) / len(took)
+
+    per_launch = [launch_ms(k) for k in range(len(heavy))]
     bound_k = [k for k, i in enumerate(heavy) if cases[i]["ops"] / cases[i]["bytes"] >= ridge]
-    heavy_ms = sum(ev[k][0].elapsed_time(ev[k][1]) for ev in marks for k in bound_k) / max(args.steps, 1)   # per step
+    heavy_ms = sum(per_launch[k] for k in bound_k)   # per step
     heavy_ops = sum(cases[heavy[k]]["ops"] for k in bound_k)
     # the dominant kernel: the family that takes the largest share of the timed launches
     fam = {}
     for k, i in enumerate(heavy):
-        t = sum(ev[k][0].elapsed_time(ev[k][1]) for ev in marks) / max(args.steps, 1)
+        t = per_launch[k]
         f = fam.setdefault(cases[i]["kernel"], {"ms": 0.0, "ops": 0.0, "idx": []})
         f["ms"] += t
         f["ops"] += cases[i]["ops"]
@@ -352,7 +367,8 @@ def main():
                   + ", ".join(sorted({f"{cases[heavy[k]]['M']}x{cases[heavy[k]]['N']}x{cases[heavy[k]]['K']}" for k in dom})) + ")",
         "family": DOMINANT,
         "ops_per_launch": dom_ops / len(dom), "avg_launch_ms": dom_ms / len(dom), "launches_per_step": len(dom),
-        "protocol": "HIP events around each of these launches inside the timed steps",
+        "protocol": "HIP events around these launches inside the timed steps; each step brackets a rotating quarter of them "
+                    "(every launch is sampled in steps / 4 of the timed steps)",
         "all_mfma_bound_cases": {"achieved": heavy_ops / heavy_ms / 1e9, "frac": heavy_ops / heavy_ms / 1e9 / PEAK_INT8_TOPS,
                                  "launches_per_step": len(bound_k), "avg_launch_ms": heavy_ms / len(bound_k)},
         "families": {name: {"kernel": FAMILIES.get(name, {}).get("kernel", name), "launches_per_step": len(f["idx"]),
