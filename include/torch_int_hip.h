@@ -68,6 +68,12 @@ const char* ti_last_kernel(void);
 int ti_diag_mfma_loop(int mode, const int8_t* data, int64_t data_bytes, int64_t iters, int32_t* sink, void* stream);
 int64_t ti_diag_mfma_loop_ops(int64_t iters);
 
+/* Diagnostic (no counterpart in the reference): `workgroups` workgroups write 1.0f to every element of the fp32
+ * matrix out[M, N] (row-major; M a multiple of 256, N of 160), `reps` times, tile by tile with the store instructions
+ * and addresses of the 256x160 GEMM kernel's 32-bit epilogue and nothing else: a benchmark times it to learn what
+ * one CU (few workgroups) or the whole chip (one workgroup per CU) can store. */
+int ti_diag_store_loop(float* out, int64_t M, int64_t N, int workgroups, int reps, void* stream);
+
 /* ---- W8A8 linear: out[M,N] = epilogue(x[M,K] . w[N,K]^T, bias[N]) ---- */
 
 /* replaces linear_a8_w8_b32_o32 (torch_int/kernels/linear.cu:13-136;

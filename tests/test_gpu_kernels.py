@@ -743,6 +743,21 @@ def test_diag_mfma_loop_runs_and_reports_its_work():
         X.diag_mfma_loop(0, data[: 1 << 19], 200, sink)
 
 
+def test_diag_store_loop_fills_the_matrix_and_nothing_else():
+    # the store-rate diagnostic writes every element of its [M, N] matrix, for any number of workgroups, and stays
+    # inside it (guard rows before and after keep their value)
+    import torch_int._hip_ext as X
+    for (M, N, wgs, reps) in [(256, 160, 1, 1), (512, 480, 3, 2), (1024, 5120, 256, 1), (768, 320, 1000, 1)]:
+        _say(f"diag_store_loop {M}x{N} workgroups {wgs}")
+        buf = torch.full((M + 2, N), -3.0, device=DEV)
+        out = buf[1:M + 1]
+        assert X.diag_store_loop(out, wgs, reps) == M * N * 4 * reps
+        torch.cuda.synchronize()
+        assert bool((out == 1.0).all()) and bool((buf[0] == -3.0).all()) and bool((buf[M + 1] == -3.0).all())
+    with pytest.raises(RuntimeError):
+        X.diag_store_loop(torch.empty(100, 160, device=DEV), 1, 1)
+
+
 def test_ln_q_fp16_residual_stream():
     # dq_add_layernorm_q and add + LayerNormQ with fp16 residual / gamma / beta: bit-exact against the oracle's
     # restatement, and within one LSB of the chain of torch ops on the same fp16 tensors on the device

@@ -42,7 +42,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--op", required=True, choices=list(LINEAR) + ["bmm_f32t", "bmm_s8t", "bmm_s32t", "bmm_s8t_rowmajor", "ln_q", "ln_q_f16", "add_ln_q",
                                                "softmax_q", "qk_softmax_q", "attn_prefill", "decode_attn", "copy",
-                                               "mfma_loop", "mfma_ceiling"])
+                                               "mfma_loop", "mfma_ceiling", "store_loop"])
     ap.add_argument("--shape", type=int, nargs="+", required=True)
     ap.add_argument("--iters", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
@@ -172,6 +172,12 @@ def main():
         sink = torch.zeros(1, dtype=torch.int32, device=dev)
         ops = float(X.diag_mfma_loop(mode, data, steps, sink))
         fn = lambda: X.diag_mfma_loop(mode, data, steps, sink)  # noqa: E731
+    elif args.op == "store_loop":
+        # fp32 [M, N] written with the 256x160 kernel's epilogue stores by `workgroups` workgroups, `reps` times
+        M, N, workgroups, reps = args.shape
+        out = torch.empty(M, N, device=dev)
+        nbytes = float(X.diag_store_loop(out, workgroups, reps))
+        fn = lambda: X.diag_store_loop(out, workgroups, reps)  # noqa: E731
     else:  # plain device copy of a known size: reference reading for FETCH_SIZE / WRITE_SIZE
         n, = args.shape
         src = torch.empty(n, dtype=torch.uint8, device=dev).random_(generator=g)

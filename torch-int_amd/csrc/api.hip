@@ -391,6 +391,18 @@ int ti_diag_mfma_loop(int mode, const int8_t* data, int64_t data_bytes, int64_t 
   return launch_diag_mfma_loop(mode, data, iters, sink, static_cast<hipStream_t>(stream));
 }
 
+int ti_diag_store_loop(float* out, int64_t M, int64_t N, int workgroups, int reps, void* stream) {
+  g_err[0] = 0;
+  const char* op = "diag_store_loop";
+  if (M < 256 || N < 160 || M % 256 != 0 || N % 160 != 0 || M * N > (1ll << 31))
+    return fail(TI_ERR_INVALID_ARG, "%s: M must be a multiple of 256, N of 160, M * N at most 2^31 (got %lld x %lld)", op,
+                (long long)M, (long long)N);
+  if (workgroups < 1 || workgroups > 65536 || reps < 1 || reps > 65536)
+    return fail(TI_ERR_INVALID_ARG, "%s: workgroups and reps must be in [1, 65536] (got %d, %d)", op, workgroups, reps);
+  if (int rc = check_ptr(op, "out", out, 16, true)) return rc;
+  return launch_diag_store_loop(out, M, N, workgroups, reps, static_cast<hipStream_t>(stream));
+}
+
 int ti_bmm_s8t_s8n_f32t_strided(const int8_t* a, const int8_t* b, float* c, int64_t batch, int64_t M, int64_t N,
                                 int64_t K, int64_t stride_a, int64_t stride_b, float alpha, void* stream) {
   return run_gemm("bmm_s8t_s8n_f32t_strided", EPI_F32_SCALE, a, b, nullptr, 0, c, 4, batch, M, N, K, alpha, 0.0f,

@@ -116,4 +116,33 @@ int launch_diag_mfma_loop(int mode, const int8_t* data, long long iters, int* si
   return fail(TI_ERR_INVALID_ARG, "diag_mfma_loop: mode must be 0, 1 or 2 (got %d)", mode);
 }
 
+// Store-rate diagnostic: `workgroups` workgroups of 8 waves write fp32 tiles of 256 x 160 of a row-major [M, N]
+// matrix exactly as the 256x160 GEMM kernel's epilogue does (a wave owns 64 x 80, one 16-byte store per lane covers
+// 16 rows x 64 bytes), `reps` times over the tiles blockIdx.x, + gridDim.x, ...; nothing else.  Every element
+// written is 1.0f.  With few workgroups it measures what one CU can store, with one per CU the whole chip.
+__global__ __launch_bounds__(512, 2) void store_loop_kernel(float* __restrict__ out, int N, int tiles_n, int tiles,
+                                                            int reps) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave >> 1, wn = wave & 1, r = lane & 15, g = lane >> 4;
+  const v4f one = {1.0f, 1.0f, 1.0f, 1.0f};
+  for (int rep = 0; rep < reps; ++rep)
+    for (int t = blockIdx.x; t < tiles; t += gridDim.x) {
+      const int tm = t / tiles_n, tn = t - tm * tiles_n;
+      float* base = out + (size_t)(tm * 256 + wm * 64) * N + tn * 160 + wn * 80;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 5; ++j) *reinterpret_cast<v4f*>(base + (size_t)(i * 16 + r) * N + j * 16 + 4 * g) = one;
+    }
+}
+
+int launch_diag_store_loop(float* out, long long M, long long N, int workgroups, int reps, hipStream_t stream) {
+  const int tiles_n = (int)(N / 160), tiles = (int)(M / 256) * tiles_n;
+  hipLaunchKernelGGL(store_loop_kernel, dim3(workgroups), dim3(512), 0, stream, out, (int)N, tiles_n,
+                     tiles, reps);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "store loop launch: %s", hipGetErrorString(e));
+  return TI_OK;
+}
+
 }  // namespace ti

@@ -61,6 +61,8 @@ _lib.ti_diag_mfma_loop.argtypes = [ctypes.c_int, _vp, _i64, _i64, _vp, _vp]
 _lib.ti_diag_mfma_loop.restype = ctypes.c_int
 _lib.ti_diag_mfma_loop_ops.argtypes = [_i64]
 _lib.ti_diag_mfma_loop_ops.restype = _i64
+_lib.ti_diag_store_loop.argtypes = [_vp, _i64, _i64, ctypes.c_int, ctypes.c_int, _vp]
+_lib.ti_diag_store_loop.restype = ctypes.c_int
 _raw_stream = torch._C._cuda_getCurrentRawStream
 _fast = _CUDA._fast if getattr(_CUDA._fast, "kv_append", None) is not None else None
 _fast_decode_attn = getattr(_CUDA._fast, "decode_attn", None)
@@ -536,6 +538,20 @@ def diag_mfma_loop(mode, data, iters, sink):
     if rc:
         raise RuntimeError(f"torch_int._hip_ext.diag_mfma_loop: {_lib.ti_last_error().decode()} (status {rc})")
     return ops
+
+
+def diag_store_loop(out, workgroups, reps=1):
+    """Diagnostic launch: ``workgroups`` workgroups fill the fp32 HIP matrix ``out`` ([M, N] contiguous, M a multiple of
+    256, N of 160) with 1.0, ``reps`` times, using the store pattern of the 256x160 GEMM kernel's 32-bit epilogue.
+    Returns the bytes the launch writes."""
+    if not (_ok(out, torch.float32) and out.dim() == 2):
+        raise RuntimeError("torch_int._hip_ext.diag_store_loop: out must be a contiguous fp32 HIP matrix")
+    with _on(out.device):
+        rc = _lib.ti_diag_store_loop(out.data_ptr(), out.shape[0], out.shape[1], int(workgroups), int(reps),
+                                     _raw_stream(out.device.index) or None)
+    if rc:
+        raise RuntimeError(f"torch_int._hip_ext.diag_store_loop: {_lib.ti_last_error().decode()} (status {rc})")
+    return out.numel() * 4 * int(reps)
 
 
 def measure_mfma_ceiling(window_ms=250.0, iters=20000):
