@@ -106,6 +106,13 @@ __device__ __forceinline__ void quad_transpose(int (&x)[4], int lane) {
   }
 }
 
+// four int8 values (already clamped to [-128, 127], held in ints) as one dword, first value in the low byte
+__device__ __forceinline__ int pack_s8x4_ints(int a, int b, int c, int d) {
+  const unsigned lo = __builtin_amdgcn_perm((unsigned)b, (unsigned)a, 0x0c0c0400u);  // a.byte0 | b.byte0 << 8
+  const unsigned hi = __builtin_amdgcn_perm((unsigned)d, (unsigned)c, 0x0c0c0400u);
+  return (int)__builtin_amdgcn_perm(hi, lo, 0x05040100u);
+}
+
 // Applies the epilogue to a wavefront's accumulators and stores them.
 template <class Cfg>
 __device__ __forceinline__ void store_tile(v16i (&acc)[Cfg::TM][Cfg::TN], const GemmParams& p, int batch, int m0,
@@ -126,6 +133,49 @@ __device__ __forceinline__ void store_tile(v16i (&acc)[Cfg::TM][Cfg::TN], const 
     constexpr int VEC = 16 / sizeof(Out);  // outputs per 16-byte store
     const bool vec_ok = (N % VEC) == 0 && (reinterpret_cast<uintptr_t>(C) & 15) == 0;
     const bool bias_al = (reinterpret_cast<uintptr_t>(bias) & 15) == 0;
+    if constexpr (sizeof(Out) == 1 && TN == 2 && !E::kAccumulate) {
+      // Wave tiles two blocks wide whose 64 columns lie inside the matrix: a row's 64 output bytes sit in two
+      // lanes (column halves) x two blocks.  v_permlane16_swap between the two blocks' packed dwords moves
+      // block 1 of rows 0..15 into the lanes that held block 0 of rows 16..31 and the reverse, after which one
+      // store instruction writes 16 rows x 64 contiguous bytes instead of 32 rows x 32.
+      const int nw = n0 + wave_n * Cfg::WTN;
+      if (vec_ok && (!E::kHasBias || bias_al) && nw + 64 <= N) {
+        v4i braw[2] = {v4i{0, 0, 0, 0}, v4i{0, 0, 0, 0}};
+        if (E::kHasBias) {
+#pragma unroll
+          for (int j = 0; j < 2; ++j) braw[j] = *reinterpret_cast<const v4i*>(bias + nw + j * 32 + half * 16);
+        }
+        const int col = nw + ((lane >> 4) & 1) * 32 + half * 16;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+          int w[2][4];
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            BiasT bv[16];
+            __builtin_memcpy(bv, &braw[j], 16);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              int o[4];
+#pragma unroll
+              for (int k = 0; k < 4; ++k)
+                o[k] = (int)E::apply(acc[i][j][4 * q + k], E::bias_term(bv[4 * q + k], beta), alpha);
+              w[j][q] = pack_s8x4_ints(o[0], o[1], o[2], o[3]);
+            }
+          }
+          v4i lo, hi;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            auto sw = __builtin_amdgcn_permlane16_swap((unsigned)w[0][q], (unsigned)w[1][q], false, false);
+            lo[q] = (int)sw[0];  // rows 0..15 of the block row: blocks 0 | 1 by lane bit 4
+            hi[q] = (int)sw[1];  // rows 16..31
+          }
+          const int mlo = m0 + wave_m * Cfg::WTM + i * 32 + (lane & 15);
+          if (mlo < M) *reinterpret_cast<v4i*>(C + out_index(p, mlo, col)) = lo;
+          if (mlo + 16 < M) *reinterpret_cast<v4i*>(C + out_index(p, mlo + 16, col)) = hi;
+        }
+        return;
+      }
+    }
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       const int nb = n0 + wave_n * Cfg::WTN + j * 32 + half * 16;
@@ -846,13 +896,6 @@ __device__ __forceinline__ void row_transpose4(int (&x)[4]) {
   x[1] = (int)c[1];
   x[2] = (int)d[0];
   x[3] = (int)d[1];
-}
-
-// four int8 values (already clamped to [-128, 127], held in ints) as one dword, first value in the low byte
-__device__ __forceinline__ int pack_s8x4_ints(int a, int b, int c, int d) {
-  const unsigned lo = __builtin_amdgcn_perm((unsigned)b, (unsigned)a, 0x0c0c0400u);  // a.byte0 | b.byte0 << 8
-  const unsigned hi = __builtin_amdgcn_perm((unsigned)d, (unsigned)c, 0x0c0c0400u);
-  return (int)__builtin_amdgcn_perm(hi, lo, 0x05040100u);
 }
 
 // Epilogue of the 16x16-block kernels: the lane holds row (lane & 15) and four consecutive columns
