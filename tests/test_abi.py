@@ -157,3 +157,35 @@ def test_host_validation_raises_and_never_computes_on_cpu():
     with pytest.raises(RuntimeError, match="only run on a HIP"):
         C.dq_add_layernorm_q(torch.zeros(2, 8, dtype=torch.int32), 1.0, torch.zeros(2, 8), torch.ones(8),
                              torch.zeros(8), 1e-5)
+
+
+def test_split_k_choice_is_sane_at_the_opt_widths():
+    # ti_linear_workspace_bytes = splits * M * N * 4 for the split the dispatcher would take (no GPU needed: without
+    # a device the cost model prices a 256-CU part).  Pins what the design promises about it: no split for decode
+    # (M <= 16) and prefill (M > 1024) shapes or where the unsplit tiles already fill the chip, a slice count that
+    # divides K into multiples of 64, and a workspace of at most ten partial copies of the output.
+    import torch_int._CUDA as C
+    lib = ctypes.CDLL(C.LIB_PATH)
+    lib.ti_linear_workspace_bytes.restype = ctypes.c_int64
+    lib.ti_linear_workspace_bytes.argtypes = [ctypes.c_int64] * 3
+    widths = [(5120, 5120), (20480, 5120), (5120, 20480), (9216, 9216), (36864, 9216), (9216, 36864)]
+    for (N, K) in widths:
+        for M in (1, 4, 16, 1025, 2048, 8192):
+            assert lib.ti_linear_workspace_bytes(M, N, K) == 0, (M, N, K)
+        for M in (17, 64, 128, 256, 512, 1024):
+            need = lib.ti_linear_workspace_bytes(M, N, K)
+            assert need % (M * N * 4) == 0, (M, N, K, need)
+            splits = need // (M * N * 4)
+            assert splits == 0 or (2 <= splits <= 10 and (K // 64) % splits == 0), (M, N, K, splits)
+    # 512 rows of the fc1 widths make 256 tiles of 256x160 / 256x288 on their own: one launch
+    assert lib.ti_linear_workspace_bytes(512, 20480, 5120) == 0
+    assert lib.ti_linear_workspace_bytes(512, 36864, 9216) == 0
+    # few output tiles and a long K: split
+    for (M, N, K) in [(128, 5120, 5120), (512, 5120, 20480), (1024, 9216, 36864), (128, 20480, 5120)]:
+        assert lib.ti_linear_workspace_bytes(M, N, K) >= 2 * M * N * 4, (M, N, K)
+    # more slices for fewer rows at a fixed width (fewer tiles to share the chip), never fewer
+    for (N, K) in widths:
+        got = [lib.ti_linear_workspace_bytes(M, N, K) // (M * N * 4) for M in (128, 512, 1024)]
+        assert got[0] >= got[1] >= got[2], (N, K, got)
+    # OPT-125m widths are too small to be worth a second launch
+    assert lib.ti_linear_workspace_bytes(512, 768, 768) == 0
