@@ -61,7 +61,7 @@ def test_c_abi_rejects_bad_arguments_without_a_device():
     # the no-allocation linear refuses a shape whose split-K scratch exceeds its built-in buffer (before any device call)
     lib.ti_linear_a8_w8_b8_o8_noalloc.argtypes = ([ctypes.c_void_p] * 4 + [ctypes.c_int64] * 3 + [ctypes.c_float] * 2
                                                   + [ctypes.c_void_p])
-    rc = lib.ti_linear_a8_w8_b8_o8_noalloc(p, p, p, p, 512, 9216, 9216, 1.0, 1.0, None)
+    rc = lib.ti_linear_a8_w8_b8_o8_noalloc(p, p, p, p, 1024, 9216, 36864, 1.0, 1.0, None)
     assert rc == 1 and b"scratch" in lib.ti_last_error()
     # the diagnostic matrix-pipe loop validates its arguments before touching the device
     lib.ti_diag_mfma_loop.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p,

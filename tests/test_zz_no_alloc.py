@@ -82,7 +82,7 @@ def test_noalloc_linear_matches_the_workspace_entry_point_twice_in_a_row():
 def test_noalloc_linear_refuses_what_the_scratch_cannot_hold():
     import torch_int._CUDA as C
     lib = _bind(C._lib)
-    M, N, K = 512, 9216, 9216
+    M, N, K = 1024, 9216, 36864
     assert lib.ti_linear_workspace_bytes(M, N, K) > 40 * 2 ** 20
     t = torch.zeros(16, dtype=torch.int8, device=DEV)
     rc = lib.ti_linear_a8_w8_b8_o8_noalloc(t.data_ptr(), t.data_ptr(), t.data_ptr(), t.data_ptr(), M, N, K, 1.0, 1.0,

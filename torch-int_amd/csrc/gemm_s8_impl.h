@@ -1885,15 +1885,16 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmParams p, const 
 // Number of K slices for an (M,N,K) linear on this chip (1 = do not split) and the tile of the
 // raw-int32 GEMM that computes the slices.  A small cost model fitted to measurements at OPT-13B/66B
 // widths with cache-cold weights, per 64-byte K step: a 256x256 workgroup takes about 0.85 us with a CU
-// to itself, 256x160 0.55 us, 256x288 0.92 us, 128x160 0.375 us; a 128x128 workgroup 0.35 us alone and 0.70 us
+// to itself, 256x160 0.55 us, 256x288 0.92 us, 128x160 0.375 us, 128x288 0.6 us; a 128x128 workgroup 0.35 us alone and 0.70 us
 // when two share a CU; 8 us per round for pipeline fill and epilogue (4 us for 128x160, which has half the panel
-// rows to fetch and half the tile to store; at 512 rows or fewer it replaces 256x160 tiles that would need twice
+// rows to fetch and half the tile to store, 5 us for 128x288; at 512 rows or fewer they replace 256-row tiles that would need twice
 // the slices for the same number of workgroups: 512x5120x5120 31 -> 25.5 us, 128x20480x5120 38 -> 34 us,
-// 128x5120x20480 37 -> 32 us, while 512x5120x20480 stays with 256x160: 64 against 70 us); the int32 partial tiles are written
+// 128x5120x20480 37 -> 32 us, 512x9216x9216 64 -> 57 us, 128x36864x9216 101 -> 83 us, while 512x5120x20480 stays with
+// 256x160: 64 against 70 us); the int32 partial tiles are written
 // once and read once (they mostly stay in the last-level cache), plus the second launch.  The
 // unsplit candidates are in the race too, so that a shape whose 256x160 or 256x288 tiles already fill
 // the chip is left to the ordinary dispatch.
-enum SplitTile { SPLIT_128 = 0, SPLIT_256 = 1, SPLIT_256x160 = 2, SPLIT_256x288 = 3, SPLIT_128x160 = 4 };
+enum SplitTile { SPLIT_128 = 0, SPLIT_256 = 1, SPLIT_256x160 = 2, SPLIT_256x288 = 3, SPLIT_128x160 = 4, SPLIT_128x288 = 5 };
 static int choose_splits(long long M, long long N, long long K, int* tile_kind = nullptr) {
   if (tile_kind) *tile_kind = SPLIT_128;
   if (M <= 16 || M > 1024 || K % PBK != 0 || K < 1024) return 1;
@@ -1902,17 +1903,18 @@ static int choose_splits(long long M, long long N, long long K, int* tile_kind =
   int best = 1, best_kind = SPLIT_128;
   double best_t = 1e30;
   // smaller tiles first: a later candidate must be clearly faster to replace an earlier one
-  const int order[5] = {SPLIT_128, SPLIT_128x160, SPLIT_256, SPLIT_256x160, SPLIT_256x288};
-  for (int oi = 0; oi < 5; ++oi) {
+  const int order[6] = {SPLIT_128, SPLIT_128x160, SPLIT_128x288, SPLIT_256, SPLIT_256x160, SPLIT_256x288};
+  for (int oi = 0; oi < 6; ++oi) {
     const int kind = order[oi];
-    const int bm = kind == SPLIT_128 || kind == SPLIT_128x160 ? 128 : 256;
-    const int bn = kind == SPLIT_128 ? 128 : kind == SPLIT_256 ? 256 : kind == SPLIT_256x288 ? 288 : 160;
+    const bool half = kind == SPLIT_128x160 || kind == SPLIT_128x288;  // 128-row forms of the two tall tiles
+    const int bm = kind == SPLIT_128 || half ? 128 : 256;
+    const int bn = kind == SPLIT_128 ? 128 : kind == SPLIT_256 ? 256 : kind == SPLIT_256x288 || kind == SPLIT_128x288 ? 288 : 160;
     if (kind >= SPLIT_256x160 && N % bn != 0) continue;
     const double tiles = (double)((M + bm - 1) / bm) * (double)((N + bn - 1) / bn);
     for (int s = 1; s <= 16; ++s) {
       if (steps % s != 0 || steps / s < 4) continue;
       if (kind >= SPLIT_256x160 && (K / s) % QBK != 0) continue;  // these tiles step 128 bytes at a time
-      if (kind == SPLIT_128x160 && s == 1) continue;               // exists as a raw-int32 kernel only
+      if (half && s == 1) continue;                                // exist as raw-int32 kernels only
       const double wgs = tiles * s;
       double rounds, step_us, fixed_us = 8.0;
       if (kind == SPLIT_128) {
@@ -1920,13 +1922,14 @@ static int choose_splits(long long M, long long N, long long K, int* tile_kind =
         step_us = wgs <= cus ? 0.35 : 0.70;
       } else {
         rounds = (double)(long long)((wgs + cus - 1) / cus);
-        step_us = kind == SPLIT_256 ? 0.85 : kind == SPLIT_256x160 ? 0.55 : kind == SPLIT_256x288 ? 0.92 : 0.375;
-        if (kind == SPLIT_128x160) fixed_us = 4.0;  // half the panel rows to fetch first, half the tile to store
+        step_us = kind == SPLIT_256 ? 0.85 : kind == SPLIT_256x160 ? 0.55 : kind == SPLIT_256x288 ? 0.92
+                  : kind == SPLIT_128x160 ? 0.375 : 0.6;
+        if (half) fixed_us = kind == SPLIT_128x160 ? 4.0 : 5.0;  // fewer panel rows to fetch first, half the tile to store
       }
       double t = rounds * ((double)(steps / s) * step_us + fixed_us);
       // The weights come from HBM: a workgroup keeps about `ahead` K steps of its weight rows in flight, and what
       // all resident workgroups have in flight over a 2 us round trip bounds the streaming rate (5 TB/s at most).
-      const double ahead = kind == SPLIT_128 ? 4.0 : kind == SPLIT_256x160 || kind == SPLIT_128x160 ? 2.5 : 1.5;
+      const double ahead = kind == SPLIT_128 ? 4.0 : kind == SPLIT_256x160 || half ? 2.5 : 1.5;
       const double step_bytes = (double)bn * (kind == SPLIT_128 ? 64.0 : 128.0);
       const double resident = wgs < cus * (kind == SPLIT_128 ? 2 : 1) ? wgs : cus * (kind == SPLIT_128 ? 2 : 1);
       double rate = resident * ahead * step_bytes / 2.0;  // bytes per us
@@ -2016,6 +2019,7 @@ int launch_kind(const GemmParams& p, void* workspace, long long workspace_bytes,
                       : tile == SPLIT_256    ? "splitk_256x256"
                       : tile == SPLIT_256x160 ? "splitk_256x160"
                       : tile == SPLIT_128x160 ? "splitk_128x160"
+                      : tile == SPLIT_128x288 ? "splitk_128x288"
                                               : "splitk_256x288";
       GemmParams q = p;  // the K slices are the batches of one raw-int32 GEMM into the workspace
       q.K = p.K / splits;
