@@ -1902,8 +1902,9 @@ static int choose_splits(long long M, long long N, long long K, int* tile_kind =
   const long long steps = K / PBK;
   int best = 1, best_kind = SPLIT_128;
   double best_t = 1e30;
-  // smaller tiles first: a later candidate must be clearly faster to replace an earlier one
-  const int order[6] = {SPLIT_128, SPLIT_128x160, SPLIT_128x288, SPLIT_256, SPLIT_256x160, SPLIT_256x288};
+  // the 128-row forms of the tall tiles first, then by size: a later candidate must be clearly faster to replace
+  // an earlier one
+  const int order[6] = {SPLIT_128x160, SPLIT_128x288, SPLIT_128, SPLIT_256, SPLIT_256x160, SPLIT_256x288};
   for (int oi = 0; oi < 6; ++oi) {
     const int kind = order[oi];
     const bool half = kind == SPLIT_128x160 || kind == SPLIT_128x288;  // 128-row forms of the two tall tiles
@@ -1915,6 +1916,9 @@ static int choose_splits(long long M, long long N, long long K, int* tile_kind =
       if (steps % s != 0 || steps / s < 4) continue;
       if (kind >= SPLIT_256x160 && (K / s) % QBK != 0) continue;  // these tiles step 128 bytes at a time
       if (half && s == 1) continue;                                // exist as raw-int32 kernels only
+      // an unsplit candidate stands for what the ordinary dispatch would launch, which takes the 256-row tiles only
+      // when they fill most of the chip (and 128x128 tiles otherwise)
+      if (s == 1 && kind != SPLIT_128 && tiles < 0.75 * cus) continue;
       const double wgs = tiles * s;
       double rounds, step_us, fixed_us = 8.0;
       if (kind == SPLIT_128) {
@@ -1933,10 +1937,13 @@ static int choose_splits(long long M, long long N, long long K, int* tile_kind =
       const double step_bytes = (double)bn * (kind == SPLIT_128 ? 64.0 : 128.0);
       const double resident = wgs < cus * (kind == SPLIT_128 ? 2 : 1) ? wgs : cus * (kind == SPLIT_128 ? 2 : 1);
       double rate = resident * ahead * step_bytes / 2.0;  // bytes per us
-      if (rate > 5.0e6) rate = 5.0e6;
+      // 5 TB/s at most; 3.5 TB/s for the 64-byte steps of the 128x128 tiles, which ask for every line twice
+      // (128x9216x36864: 110 us against 83 us with 128x288 tiles)
+      const double cap = kind == SPLIT_128 ? 3.5e6 : 5.0e6;
+      if (rate > cap) rate = cap;
       const double t_stream = (double)N * (double)K / rate + 8.0;
       if (t < t_stream) t = t_stream;
-      if (s > 1) t += (double)(2 * s + 1) * M * N * 4.0 / 8.0e6 + 3.0;  // partials out and back in, at 8 TB/s, in us
+      if (s > 1) t += (double)(2 * s + 1) * M * N * 4.0 / 5.5e6 + 3.0;  // partials out and back in, at 5.5 TB/s, in us
       if (t < best_t * 0.97) {  // prefer fewer slices and the smaller tile unless the gain is clear
         best_t = t;
         best = s;
