@@ -213,6 +213,16 @@ int ti_add_layernorm_q(const float* x, float* residual, const float* gamma, cons
 int ti_add_layernorm_q_f16(const void* x, void* residual, const void* gamma, const void* beta, float eps,
                            int8_t* q_out, int64_t rows, int64_t H, void* stream);
 
+/* The same with an fp32 x on the fp16 stream: residual = f16(float(residual) + float(f16(x))) in place, i.e.
+ * `residual.add_(x.to(residual.dtype))` as the decoder layer adds the fp32 output of out_proj to an fp16 residual
+ * (torch_int/models/opt.py:281), then the LayerNorm-quantiser as above.  x must not be NULL. */
+int ti_add_layernorm_q_f16_xf32(const float* x, void* residual, const void* gamma, const void* beta, float eps,
+                                int8_t* q_out, int64_t rows, int64_t H, void* stream);
+
+/* residual[i] = f16(float(residual[i]) + float(f16(x[i]))) for n elements, in place: `residual.add_(x.to(residual.dtype))`
+ * of an fp32 x on an fp16 residual stream in one pass (torch_int/models/opt.py:289, the fp32 output of fc2). */
+int ti_add_f16_xf32(const float* x, void* residual, int64_t n, void* stream);
+
 /* probs[b*heads+h, t, s] = s8(rint(127 * softmax_s(max(scores[b*heads+h,t,s] + mask[b,0,t,s], -FLT_MAX))));
  * scores [batch*heads, T, S] fp32, mask [batch, 1, T, S] fp32 or NULL.
  * Replaces the mask add, clamp, softmax, *127, round and int8 cast between the two

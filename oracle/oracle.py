@@ -222,9 +222,13 @@ def dq_add_layernorm_q_f16(inp, input_scale, residual, gamma, beta, eps):
 
 
 def add_layernorm_q_f16(x, residual, gamma, beta, eps):
-    """add_layernorm_q on fp16 tensors; x may be None."""
+    """add_layernorm_q on fp16 tensors; x may be None, or fp32 (then it is rounded to fp16 before the add)."""
     if x is None:
         return _ln_f16(2, None, 1.0, residual, gamma, beta, eps)
+    if x.dtype is torch.float32:
+        x = _chk(x, torch.float32, "x")
+        assert x.shape == residual.shape
+        return _ln_f16(3, x, 1.0, residual, gamma, beta, eps)
     x = _chk(x, torch.float16, "x")
     assert x.shape == residual.shape
     return _ln_f16(1, x, 1.0, residual, gamma, beta, eps)

@@ -306,7 +306,8 @@ static inline float round_f16(float x) { return orc_f32_of_f16(orc_f16_of_f32(x)
  *      device, where it matches on every element; |in| >= 65520 becomes infinity)
  *   y = f16(fmaf((f32(r) - mean) * rstd, f32(gamma), f32(beta)))   mean / rstd from the fixed tree over f32(r)
  *   q = s8(rne(clamp(f32(y), -128, 127)))
- * mode 0: dequantise + add (`in` int32); 1: add (`in` fp16 x); 2: plain.  r_out may be NULL in mode 2. */
+ * mode 0: dequantise + add (`in` int32); 1: add (`in` fp16 x); 2: plain; 3: add of an fp32 x that is rounded to
+ * fp16 first (`residual.add_(x.to(residual.dtype))`, torch_int/models/opt.py:281).  r_out may be NULL in mode 2. */
 void orc_layernorm_q_f16(int mode, const void* in, float scale, const uint16_t* res, const uint16_t* gamma,
                          const uint16_t* beta, float eps, uint16_t* r_out, int8_t* q_out, int64_t rows, int64_t H) {
 #pragma omp parallel for schedule(static)
@@ -316,6 +317,7 @@ void orc_layernorm_q_f16(int mode, const void* in, float scale, const uint16_t* 
       float a = orc_f32_of_f16(res[row * H + i]);
       if (mode == 0) r[i] = round_f16(fmaf(scale, round_f16(f32_of_i32(((const int32_t*)in)[row * H + i])), a));
       else if (mode == 1) r[i] = round_f16(a + orc_f32_of_f16(((const uint16_t*)in)[row * H + i]));
+      else if (mode == 3) r[i] = round_f16(a + round_f16(((const float*)in)[row * H + i]));
       else r[i] = a;
     }
     float fH = (float)H;

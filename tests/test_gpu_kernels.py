@@ -814,6 +814,42 @@ def test_ln_q_fp16_residual_stream():
     q16 = copy_to(ln, DEV).half()(x16.to(DEV))
     _, ref16 = orc.add_layernorm_q_f16(None, x16, ln.weight.half(), ln.bias.half(), 1e-5)
     assert torch.equal(q16.cpu(), ref16)
+    # the decoder layer's residual update on an fp16 stream: an fp32 branch output is rounded to fp16, added in
+    # place, and the sum normalised -- one kernel; the bits of `x.add_(add.to(x.dtype))` + LayerNormQ on the device
+    for (rows, H) in [(7, 768), (64, 5120), (3, 9216), (5, 1001)]:
+        _say(f"fp16 residual += fp32 branch, LayerNormQ rows={rows} H={H}")
+        lnh = LayerNormQ(H)
+        lnh.weight, lnh.bias = (torch.randn(H, generator=g) * 20).half(), torch.randn(H, generator=g).half()
+        lnd = copy_to(lnh, DEV)
+        res, add = torch.randn(rows, H, generator=g).half(), torch.randn(rows, H, generator=g) * 2
+        r_ref, q_ref = orc.add_layernorm_q_f16(add, res, lnh.weight, lnh.bias, 1e-5)
+        rd = res.to(DEV)
+        qd = lnd(rd, add=add.to(DEV))
+        assert torch.equal(rd.cpu().view(torch.int16), r_ref.view(torch.int16)) and torch.equal(qd.cpu(), q_ref)
+        chain = res.to(DEV)
+        chain.add_(add.to(DEV).to(chain.dtype))
+        assert torch.equal(rd, chain)
+        y = torch.nn.functional.layer_norm(chain, (H,), lnd.weight, lnd.bias, 1e-5)
+        q_chain = y.round().clamp(-128, 127).to(torch.int8)
+        assert (qd.int() - q_chain.int()).abs().max() <= 1 and (qd != q_chain).float().mean() <= 0.01
+    # the same update without a LayerNorm after it (the fp32 output of fc2 added to an fp16 stream), any length
+    import torch_int._hip_ext as X
+    from torch_int.nn.linear import W8A8BFP32OFP32Linear
+    for n in (1, 7, 4096, 5 * 5120 + 3):
+        res, add = torch.randn(n, generator=g).half(), torch.randn(n, generator=g) * 2
+        rd = X.add_rounded_(res.to(DEV), add.to(DEV))
+        assert torch.equal(rd.cpu(), res.clone().add_(add.to(res.dtype)))
+        off = torch.zeros(n + 1, dtype=torch.float16, device=DEV)[1:]     # a base that is not 8-byte aligned
+        off.copy_(res)
+        assert torch.equal(X.add_rounded_(off, add.to(DEV)).cpu(), res.clone().add_(add.to(res.dtype)))
+    m = W8A8BFP32OFP32Linear(256, 320, alpha=0.003)
+    m.bias = torch.randn(1, 320, generator=g)
+    x = _s8(g, 2, 5, 256)
+    resid = torch.randn(2, 5, 320, generator=g).half()
+    ref = resid.clone().add_(orc.linear_a8_w8_bfp32_ofp32(x.view(-1, 256), m.weight, m.bias, 0.003, 1.0)
+                             .view(2, 5, 320).to(resid.dtype))
+    r = resid.to(DEV)
+    assert copy_to(m, DEV)(x.to(DEV), add_to=r) is r and torch.equal(r.cpu(), ref)
 
 
 def copy_to(module, dev):

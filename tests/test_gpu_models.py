@@ -256,6 +256,60 @@ def test_causal_lm_prefill_and_decode_on_gpu():
 
 
 @torch.no_grad()
+def test_fp16_model_runs_the_fused_kernels_and_follows_the_torch_chain():
+    # a model converted with .half() (how upstream serves its checkpoints): fp16 embeddings, residual stream,
+    # LayerNorm parameters, mask and lm_head around the int8 kernels.  The fused kernels take the fp16 stream
+    # (fp32 branch outputs rounded to fp16 on the way in, the mask read as fp32); with every fusion that touches
+    # fp16 switched off, the chain of torch ops on the device must give the same model within rounding.
+    import torch_int._hip_ext as X
+    from torch_int.models.opt import Int8OPTAttention
+    cfg = OPTConfigLite(hidden_size=256, num_hidden_layers=3, ffn_dim=1024, num_attention_heads=4, vocab_size=512,
+                        max_position_embeddings=128)
+    torch.manual_seed(0)
+    lm = Int8OPTForCausalLM(cfg)
+    g = torch.Generator().manual_seed(5)
+    for layer in lm.model.decoder.layers:
+        randomize_int8_layer(layer, g)
+    ids = torch.randint(2, 512, (2, 48), generator=g).to(DEV)
+    glm = copy.deepcopy(lm).to(DEV).half()
+    assert glm.model.decoder.layers[0].fc2.bias.dtype == torch.float32       # upstream keeps this bias in fp32
+    assert glm.model.decoder.layers[0].final_layer_norm.weight.dtype == torch.float16
+    calls = {"ln": 0, "add": 0}
+    real_ln, real_add = X.add_layernorm_q, X.add_rounded_
+
+    def count_ln(x, residual, *a, **k):
+        calls["ln"] += residual.dtype is torch.float16
+        return real_ln(x, residual, *a, **k)
+
+    def count_add(residual, x):
+        calls["add"] += 1
+        return real_add(residual, x)
+    X.add_layernorm_q, X.add_rounded_ = count_ln, count_add
+    try:
+        _say("fp16 causal LM, fused")
+        out = glm(ids, use_cache=True)
+        step = glm(ids[:, -1:], past_key_values=out.past_key_values, use_cache=True)
+    finally:
+        X.add_layernorm_q, X.add_rounded_ = real_ln, real_add
+    assert out.logits.dtype == torch.float16 and calls["ln"] == 2 * 3 * 2 and calls["add"] == 3 * 2
+    real_can = X.can_fuse_layernorm
+    X.can_fuse_layernorm = lambda x, w, b: False
+    X.add_rounded_ = lambda residual, x: residual.add_(x.to(residual.dtype))
+    Int8OPTAttention.fused_softmax = False
+    try:
+        _say("fp16 causal LM, torch chain")
+        ref = glm(ids, use_cache=True)
+    finally:
+        X.can_fuse_layernorm, X.add_rounded_ = real_can, real_add
+        Int8OPTAttention.fused_softmax = True
+    for (k1, v1), (k2, v2) in zip(out.past_key_values, ref.past_key_values):
+        for a, b in ((k1, k2), (v1, v2)):
+            assert (a.int() - b.int()).abs().max() <= 2 and (a != b).float().mean() < 2e-2
+    assert _rel_err(out.logits.float().cpu(), ref.logits.float().cpu()) <= 1e-2
+    assert torch.isfinite(step.logits).all() and step.past_key_values[0][0].shape[2] == 49
+
+
+@torch.no_grad()
 def test_side_stream_and_graph_replay_of_a_decoder_layer():
     """The launches go to torch's current stream: a layer run on a side stream, and one captured into a
     graph and replayed (with eager work and synchronisations between the replays), give the bits of the

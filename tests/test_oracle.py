@@ -379,6 +379,15 @@ def test_ln_q_f16_against_torch_ops_in_fp32(shape):
     assert (q2.int() - q_t.int()).abs().max() <= 1 and (q2 != q_t).float().mean() <= 0.01 + 1.0 / q2.numel()
     r3, q3 = orc.add_layernorm_q_f16(None, r2, gamma, beta, 1e-5)
     assert torch.equal(r3, r2) and torch.equal(q3, q2)
+    # an fp32 addend on the fp16 stream, `residual.add_(x32.to(residual.dtype))`: rounded to fp16 first, so the
+    # result is the all-fp16 form on the rounded addend -- and differs from the single rounding of res + x32
+    x32 = torch.randn(shape, generator=g) * 3 + 1e-4 * torch.randn(shape, generator=g)
+    r4, q4 = orc.add_layernorm_q_f16(x32, res, gamma, beta, 1e-5)
+    r5, q5 = orc.add_layernorm_q_f16(x32.half(), res, gamma, beta, 1e-5)
+    assert torch.equal(r4, r5) and torch.equal(q4, q5)
+    assert torch.equal(r4, res.clone().add_(x32.to(res.dtype)))          # torch's own in-place fp16 add on the CPU
+    if res.numel() >= 1000:
+        assert not torch.equal(r4, (res.float() + x32).half())
 
 
 def test_ln_q_f16_rounds_the_normalised_value_to_half_before_the_integer():

@@ -58,10 +58,15 @@ def main():
     ap.add_argument("--seq", type=int, default=512)
     ap.add_argument("--decode-steps", type=int, default=32)
     ap.add_argument("--iters", type=int, default=3)
+    ap.add_argument("--dtype", default="fp32", choices=["fp32", "fp16"],
+                    help="dtype of the embeddings, the residual stream, the LayerNorm parameters and lm_head "
+                         "(upstream serves its SmoothQuant checkpoints in fp16)")
     args = ap.parse_args()
     dev = torch.device("cuda:0")
     t0 = time.perf_counter()
     model, cfg = build(args.model, args.layers, dev)
+    if args.dtype == "fp16":
+        model = model.half()
     torch.cuda.synchronize()
     int8_bytes = sum(b.numel() for n, b in model.named_buffers() if b.dtype == torch.int8)
     build_s = time.perf_counter() - t0
@@ -106,7 +111,7 @@ def main():
     L = args.layers or L
     gemm_ops = 2.0 * tokens * L * (4 * D * D + 2 * D * F)
     print(json.dumps({
-        "model": args.model, "layers": L, "batch": args.batch, "seq": args.seq, "int8_weight_GB": int8_bytes / 1e9,
+        "model": args.model, "dtype": args.dtype, "layers": L, "batch": args.batch, "seq": args.seq, "int8_weight_GB": int8_bytes / 1e9,
         "build_s": build_s, "prefill_ms": prefill_ms, "prefill_decoder_ms": prefill_decoder_ms,
         "prefill_linear_TOPS": gemm_ops / prefill_decoder_ms / 1e9,
         "decode_steps": args.decode_steps, "decode_ms_per_token_median": steady,

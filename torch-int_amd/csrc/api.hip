@@ -361,6 +361,31 @@ int ti_add_layernorm_q_f16(const void* x, void* residual, const void* gamma, con
   return launch_add_layernorm_q_f16(x, residual, gamma, beta, eps, q_out, rows, H, static_cast<hipStream_t>(stream));
 }
 
+int ti_add_f16_xf32(const float* x, void* residual, int64_t n, void* stream) {
+  g_err[0] = 0;
+  const char* op = "add_f16_xf32";
+  if (n < 0) return fail(TI_ERR_INVALID_ARG, "%s: n must not be negative (got %lld)", op, (long long)n);
+  if (int rc = check_ptr(op, "x", x, 4, n > 0)) return rc;
+  if (int rc = check_ptr(op, "residual", residual, 2, n > 0)) return rc;
+  return launch_add_f16_xf32(x, residual, n, static_cast<hipStream_t>(stream));
+}
+
+int ti_add_layernorm_q_f16_xf32(const float* x, void* residual, const void* gamma, const void* beta, float eps,
+                                int8_t* q_out, int64_t rows, int64_t H, void* stream) {
+  g_err[0] = 0;
+  const char* op = "add_layernorm_q_f16_xf32";
+  if (rows < 0 || H < 0 || rows > 0x7fffffffLL || H > 0x7fffffffLL)
+    return fail(TI_ERR_INVALID_ARG, "%s: rows and H must be in [0, 2^31) (rows=%lld H=%lld)", op, (long long)rows,
+                (long long)H);
+  const bool nonempty = rows > 0 && H > 0;
+  if (int rc = check_ptr(op, "x", x, 4, nonempty)) return rc;
+  if (int rc = check_ptr(op, "residual", residual, 2, nonempty)) return rc;
+  if (int rc = check_ptr(op, "gamma", gamma, 2, nonempty)) return rc;
+  if (int rc = check_ptr(op, "beta", beta, 2, nonempty)) return rc;
+  if (int rc = check_ptr(op, "q_out", q_out, 1, nonempty)) return rc;
+  return launch_add_layernorm_q_f16_xf32(x, residual, gamma, beta, eps, q_out, rows, H, static_cast<hipStream_t>(stream));
+}
+
 int ti_attn_softmax_q(const float* scores, const float* mask, int8_t* probs, int64_t batch, int64_t heads, int64_t T,
                       int64_t S, void* stream) {
   g_err[0] = 0;

@@ -15,6 +15,8 @@
 //   chunk c (elements 4c..4c+3) belongs to lane c % 256; a lane adds its
 //   elements in ascending order; wavefronts combine with a xor butterfly
 //   (offsets 32..1); the four wavefront sums are added left to right.
+#include <type_traits>
+
 #include "ti_common.h"
 
 namespace ti {
@@ -67,7 +69,9 @@ __device__ __forceinline__ int pack_s8x4(float y0, float y1, float y2, float y3)
 // What is normalised: MODE_DQ_ADD  r = res + scale * float(in)   (int32 in; dq_add_layernorm_q)
 //                     MODE_ADD     r = res + x                   (fp32 x passed through `in`)
 //                     MODE_PLAIN   r = x                         (fp32 x passed through `res`; r is not stored)
-enum LnMode : int { MODE_DQ_ADD = 0, MODE_ADD = 1, MODE_PLAIN = 2 };
+//                     MODE_ADD_F32 r = res + T(x)                (fp32 x added to a stream of another type T:
+//                                                                 `residual.add_(x.to(residual.dtype))`)
+enum LnMode : int { MODE_DQ_ADD = 0, MODE_ADD = 1, MODE_PLAIN = 2, MODE_ADD_F32 = 3 };
 
 // H % 4 == 0, H <= NC * 1024, all row starts 16-byte aligned.
 // EARLY: gamma and beta are fetched together with the row instead of after the two reductions; with only
@@ -85,6 +89,7 @@ __global__ __launch_bounds__(256) void ln_q_rows_kernel(const void* __restrict__
   const int nchunks = H >> 2;
   const v4i* in4 = reinterpret_cast<const v4i*>(static_cast<const int32_t*>(in) + row * H);  // MODE_DQ_ADD
   const T* x_row = static_cast<const T*>(in) + row * H;                                        // MODE_ADD
+  const float* xf32_row = static_cast<const float*>(in) + row * H;                             // MODE_ADD_F32
   const T* res_row = res + row * H;
   T* rout_row = r_out + row * H;
   int* q4 = reinterpret_cast<int*>(q_out + row * H);
@@ -116,6 +121,10 @@ __global__ __launch_bounds__(256) void ln_q_rows_kernel(const void* __restrict__
         v4f x = load4(x_row, c);
 #pragma unroll
         for (int j = 0; j < 4; ++j) v[j] = as_stored<T>(a[j] + x[j]);
+      } else if (MODE == MODE_ADD_F32) {
+        v4f x = load4(xf32_row, c);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] = as_stored<T>(a[j] + as_stored<T>(x[j]));
       } else {
         v = a;
       }
@@ -175,6 +184,7 @@ __global__ __launch_bounds__(256) void ln_q_rows_generic_kernel(const void* __re
   const int t = threadIdx.x;
   const int32_t* x = static_cast<const int32_t*>(in) + row * H;
   const T* xf = static_cast<const T*>(in) + row * H;
+  const float* xf32 = static_cast<const float*>(in) + row * H;
   const T* a = res + row * H;
   T* ro = r_out + row * H;
   int8_t* q = q_out + row * H;
@@ -182,6 +192,7 @@ __global__ __launch_bounds__(256) void ln_q_rows_generic_kernel(const void* __re
   auto value = [&](int i) {
     if (mode == MODE_DQ_ADD) return as_stored<T>(__builtin_fmaf(scale, as_stored<T>((float)x[i]), (float)a[i]));
     if (mode == MODE_ADD) return as_stored<T>((float)a[i] + (float)xf[i]);
+    if (mode == MODE_ADD_F32) return as_stored<T>((float)a[i] + as_stored<T>(xf32[i]));
     return (float)a[i];
   };
   float s = 0.0f;
@@ -234,6 +245,10 @@ static void launch_rows(int mode, const void* in, float scale, const T* res, con
     TI_LN_LAUNCH(MODE_DQ_ADD);
   } else if (mode == MODE_ADD) {
     TI_LN_LAUNCH(MODE_ADD);
+  } else if (mode == MODE_ADD_F32) {
+    if constexpr (!std::is_same<T, float>::value) {  // for an fp32 stream this is MODE_ADD
+      TI_LN_LAUNCH(MODE_ADD_F32);
+    }
   } else {
     TI_LN_LAUNCH(MODE_PLAIN);
   }
@@ -247,7 +262,7 @@ static int launch_ln_mode(int mode, const void* in, float scale, const T* res, c
   // a chunk of four elements is one load: 16 bytes of fp32, 8 bytes of fp16 (16 bytes of the int32 input)
   constexpr uintptr_t kAlign = 4 * sizeof(T) - 1;
   auto al = [](const void* p, uintptr_t mask) { return (reinterpret_cast<uintptr_t>(p) & mask) == 0; };
-  const uintptr_t in_mask = mode == MODE_DQ_ADD ? 15 : kAlign;
+  const uintptr_t in_mask = mode == MODE_DQ_ADD || mode == MODE_ADD_F32 ? 15 : kAlign;
   const bool fast = (H % 4 == 0) && H <= 16 * 1024 && (mode == MODE_PLAIN || al(in, in_mask)) && al(res, kAlign) &&
                     al(gamma, kAlign) && al(beta, kAlign) && (mode == MODE_PLAIN || al(r_out, kAlign)) && al(q_out, 3);
   const int h = (int)H;
@@ -304,6 +319,46 @@ int launch_add_layernorm_q_f16(const void* x, void* residual, const void* gamma,
                                static_cast<const H16*>(beta), eps, nullptr, q_out, rows, H, stream);
   return launch_ln_mode<H16>(MODE_ADD, x, 1.0f, r, static_cast<const H16*>(gamma), static_cast<const H16*>(beta), eps, r,
                              q_out, rows, H, stream);
+}
+
+// residual (fp16) += fp16(x), elementwise, for an fp32 x: `residual.add_(x.to(residual.dtype))` in one pass (what the
+// decoder layer does with the fp32 output of fc2 on an fp16 stream).  Chunks of four elements; a scalar tail.
+__global__ __launch_bounds__(256) void add_f16_xf32_kernel(const float* __restrict__ x, _Float16* residual, long long n,
+                                                           bool vec) {
+  const long long c = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (c * 4 >= n) return;
+  if (vec && c * 4 + 4 <= n) {
+    const v4f a = reinterpret_cast<const v4f*>(x)[c];
+    const v4h h = reinterpret_cast<const v4h*>(residual)[c];
+    v4h o;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) o[j] = (_Float16)as_stored<_Float16>((float)h[j] + as_stored<_Float16>(a[j]));
+    reinterpret_cast<v4h*>(residual)[c] = o;
+  } else {
+    for (long long i = c * 4; i < n && i < c * 4 + 4; ++i)
+      residual[i] = (_Float16)as_stored<_Float16>((float)residual[i] + as_stored<_Float16>(x[i]));
+  }
+}
+
+int launch_add_f16_xf32(const float* x, void* residual, long long n, hipStream_t stream) {
+  if (n == 0) return TI_OK;
+  const bool vec = (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(residual) & 7) == 0;
+  const long long chunks = (n + 3) / 4;
+  hipLaunchKernelGGL(add_f16_xf32_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, stream, x,
+                     static_cast<_Float16*>(residual), n, vec);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "add_f16_xf32 launch: %s", hipGetErrorString(e));
+  return TI_OK;
+}
+
+// residual (fp16) += fp16(x) for an fp32 x, then the LayerNorm-quantiser: `residual.add_(x.to(residual.dtype))`
+// followed by LayerNormQ, as the decoder layer does with the fp32 output of out_proj on an fp16 stream.
+int launch_add_layernorm_q_f16_xf32(const float* x, void* residual, const void* gamma, const void* beta, float eps,
+                                    int8_t* q_out, long long rows, long long H, hipStream_t stream) {
+  using H16 = _Float16;
+  H16* r = static_cast<H16*>(residual);
+  return launch_ln_mode<H16>(MODE_ADD_F32, x, 1.0f, r, static_cast<const H16*>(gamma), static_cast<const H16*>(beta), eps,
+                             r, q_out, rows, H, stream);
 }
 
 }  // namespace ti

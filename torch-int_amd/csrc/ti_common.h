@@ -218,6 +218,9 @@ int launch_add_layernorm_q(const float* x, float* residual, const float* gamma, 
 int launch_dq_add_layernorm_q_f16(const int32_t* in, float scale, const void* res, const void* gamma, const void* beta,
                                   float eps, void* r_out, int8_t* q_out, long long rows, long long H,
                                   hipStream_t stream);
+int launch_add_f16_xf32(const float* x, void* residual, long long n, hipStream_t stream);
+int launch_add_layernorm_q_f16_xf32(const float* x, void* residual, const void* gamma, const void* beta, float eps,
+                                    int8_t* q_out, long long rows, long long H, hipStream_t stream);
 int launch_add_layernorm_q_f16(const void* x, void* residual, const void* gamma, const void* beta, float eps,
                                int8_t* q_out, long long rows, long long H, hipStream_t stream);
 

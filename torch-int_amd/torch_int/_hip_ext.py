@@ -25,6 +25,10 @@ _lib.ti_add_layernorm_q.argtypes = [_vp, _vp, _vp, _vp, _f32, _vp, _i64, _i64, _
 _lib.ti_add_layernorm_q.restype = ctypes.c_int
 _lib.ti_add_layernorm_q_f16.argtypes = [_vp, _vp, _vp, _vp, _f32, _vp, _i64, _i64, _vp]
 _lib.ti_add_layernorm_q_f16.restype = ctypes.c_int
+_lib.ti_add_layernorm_q_f16_xf32.argtypes = [_vp, _vp, _vp, _vp, _f32, _vp, _i64, _i64, _vp]
+_lib.ti_add_layernorm_q_f16_xf32.restype = ctypes.c_int
+_lib.ti_add_f16_xf32.argtypes = [_vp, _vp, _i64, _vp]
+_lib.ti_add_f16_xf32.restype = ctypes.c_int
 _lib.ti_attn_softmax_q.argtypes = [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]
 _lib.ti_attn_softmax_q.restype = ctypes.c_int
 _lib.ti_permute_0213_s8.argtypes = [_vp, _vp, _i64, _i64, _i64, _i64, _vp]
@@ -101,21 +105,50 @@ def can_fuse_layernorm(x, weight, bias):
             and x.dim() >= 1 and x.shape[-1] == weight.numel() == bias.numel() and x.numel() > 0)
 
 
+def can_fuse_layernorm_add(add, x):
+    """True when ``add`` can be the addend of the fused residual update of ``x``: same shape and device, contiguous,
+    and of ``x``'s dtype -- or fp32 on an fp16 stream, which the kernel rounds to fp16 first, as
+    ``x.add_(add.to(x.dtype))`` does."""
+    return (isinstance(add, torch.Tensor) and add.shape == x.shape and add.device == x.device and add.is_contiguous()
+            and (add.dtype == x.dtype or (add.dtype is torch.float32 and x.dtype is torch.float16)))
+
+
+def add_rounded_(residual, x):
+    """``residual.add_(x.to(residual.dtype))`` for an fp16 ``residual`` and an fp32 ``x`` (contiguous HIP tensors of one
+    shape) in one kernel; returns ``residual``."""
+    if not (_ok(residual, torch.float16) and _ok(x, torch.float32) and x.shape == residual.shape
+            and x.device == residual.device):
+        raise RuntimeError("torch_int._hip_ext.add_rounded_: needs a contiguous fp16 and a contiguous fp32 HIP tensor "
+                           "of one shape")
+    with _on(residual.device):
+        rc = _lib.ti_add_f16_xf32(x.data_ptr(), residual.data_ptr(), residual.numel(),
+                                  _raw_stream(residual.device.index) or None)
+    if rc:
+        raise RuntimeError(f"torch_int._hip_ext.add_rounded_: {_lib.ti_last_error().decode()} (status {rc})")
+    return residual
+
+
 def add_layernorm_q(x, residual, weight, bias, eps, checked=False):
-    """``residual += x`` in place (skipped when ``x`` is None), returns int8
+    """``residual += x`` in place (skipped when ``x`` is None; an fp32 ``x`` on an fp16 residual is rounded to fp16
+    first), returns int8
     ``clamp(round(layer_norm(residual) * weight + bias), -128, 127)``.  ``checked=True``: the caller has
     already established the conditions below (the modules do, via the ``can_*`` predicates)."""
     op = "add_layernorm_q"
     if not checked:
         if not can_fuse_layernorm(residual, weight, bias):
             raise RuntimeError(f"torch_int._hip_ext.{op}: needs contiguous HIP tensors, all fp32 or all fp16")
-        if x is not None and not (_ok(x, residual.dtype) and x.shape == residual.shape and x.device == residual.device):
-            raise RuntimeError(f"torch_int._hip_ext.{op}: x must be a contiguous tensor shaped and typed like residual")
+        if x is not None and not can_fuse_layernorm_add(x, residual):
+            raise RuntimeError(f"torch_int._hip_ext.{op}: x must be a contiguous tensor shaped like residual, of its "
+                               "dtype (or fp32 on an fp16 residual)")
     dev = residual.device
     H = residual.shape[-1]
     q = torch.empty(residual.shape, dtype=torch.int8, device=dev)
     with _on(dev):
-        if residual.dtype is torch.float16:
+        if residual.dtype is torch.float16 and x is not None and x.dtype is torch.float32:
+            rc = _lib.ti_add_layernorm_q_f16_xf32(x.data_ptr(), residual.data_ptr(), weight.data_ptr(), bias.data_ptr(),
+                                                  float(eps), q.data_ptr(), residual.numel() // H, H,
+                                                  _raw_stream(dev.index) or None)
+        elif residual.dtype is torch.float16:
             rc = _lib.ti_add_layernorm_q_f16(x.data_ptr() if x is not None else None, residual.data_ptr(),
                                              weight.data_ptr(), bias.data_ptr(), float(eps), q.data_ptr(),
                                              residual.numel() // H, H, _raw_stream(dev.index) or None)

@@ -217,6 +217,10 @@ class Int8OPTAttention(nn.Module):
         cross = key_value_states is not None
         bsz, tgt_len, _ = hidden_states.size()
         H, d = self.num_heads, self.head_dim
+        if attention_mask is not None and attention_mask.is_cuda and attention_mask.dtype in (torch.float16, torch.bfloat16):
+            # the mask of an fp16 model: it is only ever added to the fp32 scores, where type promotion turns it into
+            # these same fp32 values; the fused kernels read fp32
+            attention_mask = attention_mask.float()
 
         # Self-attention on HIP tensors takes the q/k/v projections from one of two fused forms: a single
         # grouped launch for decode-sized inputs, or projections whose stores already produce the
@@ -512,6 +516,8 @@ class Int8OPTDecoder(nn.Module):
         pos = self.embed_positions(attention_mask, past_len)
         mask = _additive_decoder_mask(attention_mask, tgt_len, past_len, inputs_embeds.dtype,
                                       inputs_embeds.device)
+        if mask.is_cuda and mask.dtype in (torch.float16, torch.bfloat16):
+            mask = mask.float()  # once here instead of once per layer (see Int8OPTAttention.forward)
         if self.project_in is not None:
             inputs_embeds = self.project_in(inputs_embeds)
         hidden = inputs_embeds + pos  # a fresh tensor: the layers update it in place

@@ -22,10 +22,10 @@ class LayerNormQ(_QuantLayerNormBase):
     def forward(self, x, add=None):
         """int8 LayerNorm of ``x``.  With ``add`` given, ``x`` is first updated in place
         (``x.add_(add)``, the residual update of the decoder layer) -- fused into the same
-        kernel when ``x`` is a contiguous fp32 HIP tensor."""
+        kernel when ``x`` is a contiguous fp32 or fp16 HIP tensor (an fp32 ``add`` on an fp16 ``x`` is rounded to
+        fp16 first, as ``x.add_(add.to(x.dtype))`` does)."""
         if _hip_ext.can_fuse_layernorm(x, self.weight, self.bias) and (
-                add is None or (add.dtype == x.dtype and add.shape == x.shape and add.device == x.device
-                                and add.is_contiguous())):
+                add is None or _hip_ext.can_fuse_layernorm_add(add, x)):
             return _hip_ext.add_layernorm_q(add, x, self.weight, self.bias, self.eps, checked=True)  # one pass, same maths
         if add is not None:
             x.add_(add.to(x.dtype))

@@ -8,7 +8,7 @@ Every class keeps upstream's constructor signature, buffer names/shapes/dtypes
 """
 import torch
 
-from .. import _CUDA
+from .. import _CUDA, _hip_ext
 from ..functional.quantization import (fake_quantize_activation_per_tensor_absmax,
                                        fake_quantize_activation_per_token_absmax,
                                        quantize_per_tensor_absmax, quantize_weight_per_channel_absmax)
@@ -167,7 +167,11 @@ class W8A8BFP32OFP32Linear(_W8A8Base):
                 and hasattr(_CUDA, "_linear_a8_w8_bfp32_ofp32_acc"))
         if not fits:
             with torch.no_grad():
-                return add_to.add_(super().forward(x).to(add_to.dtype))
+                y = super().forward(x)
+                if (add_to.dtype is torch.float16 and y.is_cuda and add_to.is_contiguous() and add_to.shape == y.shape
+                        and add_to.device == y.device):
+                    return _hip_ext.add_rounded_(add_to, y)  # the cast and the add in one pass, same bits
+                return add_to.add_(y.to(add_to.dtype))
         w, bias = self._wb()
         if bias.dtype != torch.float32:
             self.bias = bias = bias.to(torch.float32)
