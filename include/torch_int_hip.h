@@ -285,6 +285,15 @@ int ti_decode_attn_s8(const int8_t* q, const int8_t* k_new, const int8_t* v_new,
                       const float* mask, int8_t* ctx, int8_t* probs_out, int64_t BH, int64_t T, int64_t D, int64_t cap,
                       int64_t S, int64_t heads, float alpha_qk, float alpha_pv, void* stream);
 
+/* ti_decode_attn_s8 for a launch that is recorded once (HIP graph capture) and replayed while the cache grows: the
+ * number of positions after the append is read from device memory (*s_dev, T <= *s_dev <= S_max) when the kernel
+ * runs, S_max is the largest value it will ever hold (the launch is sized for it; S_max <= cap).  No mask, no
+ * probabilities out; k_new / v_new are appended at positions *s_dev - T .. *s_dev - 1.  Same arithmetic and bits as
+ * ti_decode_attn_s8 with S = *s_dev.  No counterpart in the reference (its decode step is re-issued from Python). */
+int ti_decode_attn_s8_devlen(const int8_t* q, const int8_t* k_new, const int8_t* v_new, int8_t* k_buf, int8_t* v_buf,
+                             int8_t* ctx, int64_t BH, int64_t T, int64_t D, int64_t cap, int64_t S_max,
+                             const int32_t* s_dev, int64_t heads, float alpha_qk, float alpha_pv, void* stream);
+
 /* probs[bh, t, :] = int8 round(127 * softmax(max(alpha * q[bh, t, :] . k[bh, :, :]^T + mask, most negative float)))
  * in one launch: ti_bmm_s8t_s8n_f32t followed by ti_attn_softmax_q (torch_int/models/opt.py:137-178) without the
  * fp32 score tensor in between; the same bits.  q is [BH, T, D] with stride_q elements between batches, k is

@@ -310,6 +310,44 @@ def test_fp16_model_runs_the_fused_kernels_and_follows_the_torch_chain():
 
 
 @torch.no_grad()
+@pytest.mark.parametrize("half", [False, True])
+def test_graph_decoder_replays_give_the_eager_steps(half):
+    # the decoder layers of a decode step recorded once as a HIP graph (cache length read on the device) and
+    # replayed for every new token, with the eager embedding / final LayerNorm / lm_head work between the replays:
+    # every step's logits and the caches must be those of the eager step, bit for bit
+    from torch_int.models.opt import Int8OPTGraphDecoder
+    cfg = OPTConfigLite(hidden_size=256, num_hidden_layers=3, ffn_dim=1024, num_attention_heads=4, vocab_size=512,
+                        max_position_embeddings=128)
+    torch.manual_seed(0)
+    lm = Int8OPTForCausalLM(cfg)
+    g = torch.Generator().manual_seed(11)
+    for layer in lm.model.decoder.layers:
+        randomize_int8_layer(layer, g)
+    glm = copy.deepcopy(lm).to(DEV)
+    if half:
+        glm = glm.half()
+    ids = torch.randint(2, 512, (2, 32), generator=g).to(DEV)
+    toks = torch.randint(2, 512, (2, 9), generator=g).to(DEV)
+    out = glm(ids, use_cache=True)
+    _say(f"graph decoder, half={half}: capture")
+    dec = Int8OPTGraphDecoder(glm, out.past_key_values, max_new_tokens=9)
+    past = out.past_key_values
+    for t in range(9):
+        _say(f"graph decoder step {t}")
+        eager = glm(toks[:, t:t + 1], past_key_values=past, use_cache=True)
+        past = eager.past_key_values
+        logits = dec.step(toks[:, t:t + 1])
+        assert logits.shape == eager.logits.shape and torch.equal(logits, eager.logits), t
+        for (k1, v1), (k2, v2) in zip(dec.past_key_values, past):
+            assert torch.equal(k1, k2) and torch.equal(v1, v2), t
+    assert dec.past_key_values[0][0].shape[2] == 41
+    with pytest.raises(RuntimeError, match="max_new_tokens"):
+        dec.step(toks[:, :1])
+    with pytest.raises(RuntimeError, match="exceed"):
+        Int8OPTGraphDecoder(glm, out.past_key_values, max_new_tokens=200)
+
+
+@torch.no_grad()
 def test_side_stream_and_graph_replay_of_a_decoder_layer():
     """The launches go to torch's current stream: a layer run on a side stream, and one captured into a
     graph and replayed (with eager work and synchronisations between the replays), give the bits of the

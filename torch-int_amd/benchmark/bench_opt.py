@@ -61,6 +61,9 @@ def main():
     ap.add_argument("--dtype", default="fp32", choices=["fp32", "fp16"],
                     help="dtype of the embeddings, the residual stream, the LayerNorm parameters and lm_head "
                          "(upstream serves its SmoothQuant checkpoints in fp16)")
+    ap.add_argument("--graph-decode", action="store_true",
+                    help="also time the decode steps with the decoder layers replayed from a HIP graph "
+                         "(Int8OPTGraphDecoder)")
     args = ap.parse_args()
     dev = torch.device("cuda:0")
     t0 = time.perf_counter()
@@ -104,6 +107,20 @@ def main():
             step_ms.append((time.perf_counter() - t) * 1e3)
             past = o.past_key_values
             tok = o.logits[:, -1].argmax(-1, keepdim=True)
+        graph_ms = None
+        if args.graph_decode:
+            from torch_int.models.opt import Int8OPTGraphDecoder
+            dec = Int8OPTGraphDecoder(model, out.past_key_values, max_new_tokens=args.decode_steps)
+            tok = out.logits[:, -1].argmax(-1, keepdim=True)
+            times = []
+            for _ in range(args.decode_steps):
+                torch.cuda.synchronize()
+                t = time.perf_counter()
+                logits = dec.step(tok)
+                torch.cuda.synchronize()
+                times.append((time.perf_counter() - t) * 1e3)
+                tok = logits[:, -1].argmax(-1, keepdim=True)
+            graph_ms = sorted(times)[len(times) // 2]
     finite = bool(torch.isfinite(o.logits).all())
     steady = sorted(step_ms)[len(step_ms) // 2] if step_ms else None
     tokens = args.batch * args.seq
@@ -116,6 +133,7 @@ def main():
         "prefill_linear_TOPS": gemm_ops / prefill_decoder_ms / 1e9,
         "decode_steps": args.decode_steps, "decode_ms_per_token_median": steady,
         "decode_weight_GBps": (int8_bytes / 1e9) / (steady / 1e3) if steady else None,
+        "graph_decode_ms_per_token_median": graph_ms,
         "final_src_len": int(past[0][0].shape[2]), "logits_finite": finite,
         "peak_mem_GB": torch.cuda.max_memory_allocated() / 1e9}), flush=True)
 

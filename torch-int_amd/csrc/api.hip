@@ -567,6 +567,37 @@ int ti_decode_attn_s8(const int8_t* q, const int8_t* k_new, const int8_t* v_new,
                                alpha_pv, static_cast<hipStream_t>(stream));
 }
 
+int ti_decode_attn_s8_devlen(const int8_t* q, const int8_t* k_new, const int8_t* v_new, int8_t* k_buf, int8_t* v_buf,
+                             int8_t* ctx, int64_t BH, int64_t T, int64_t D, int64_t cap, int64_t S_max,
+                             const int32_t* s_dev, int64_t heads, float alpha_qk, float alpha_pv, void* stream) {
+  g_err[0] = 0;
+  const char* op = "decode_attn_s8_devlen";
+  const int64_t lim = 0x7fffffffLL;
+  if (BH < 0 || T < 0 || D < 0 || cap < 0 || S_max < 0 || heads < 1 || BH > lim || cap > lim || heads > lim)
+    return fail(TI_ERR_INVALID_ARG, "%s: sizes must be in [0, 2^31) and heads >= 1", op);
+  if (BH % heads != 0) return fail(TI_ERR_INVALID_ARG, "%s: BH = %lld is not a multiple of heads = %lld", op,
+                                   (long long)BH, (long long)heads);
+  if (k_new == nullptr || v_new == nullptr)
+    return fail(TI_ERR_INVALID_ARG, "%s: k_new and v_new must be given", op);
+  if (S_max > cap) return fail(TI_ERR_INVALID_ARG, "%s: %lld positions do not fit a capacity of %lld", op,
+                               (long long)S_max, (long long)cap);
+  if (S_max < T) return fail(TI_ERR_INVALID_ARG, "%s: S_max = %lld counts the %lld appended positions", op,
+                             (long long)S_max, (long long)T);
+  if (BH == 0) return TI_OK;
+  if (!decode_attn_supported(T, S_max, D))
+    return fail(TI_ERR_INVALID_ARG, "%s: unsupported shape T=%lld S_max=%lld head_dim=%lld (needs 1 <= T <= 4, head_dim 64 "
+                "or 128 and scores that fit the LDS)", op, (long long)T, (long long)S_max, (long long)D);
+  if (int rc = check_ptr(op, "q", q, 16, true)) return rc;
+  if (int rc = check_ptr(op, "k_new", k_new, 16, true)) return rc;
+  if (int rc = check_ptr(op, "v_new", v_new, 16, true)) return rc;
+  if (int rc = check_ptr(op, "k_buf", k_buf, 16, true)) return rc;
+  if (int rc = check_ptr(op, "v_buf", v_buf, 16, true)) return rc;
+  if (int rc = check_ptr(op, "ctx", ctx, 1, true)) return rc;
+  if (int rc = check_ptr(op, "s_dev", s_dev, 4, true)) return rc;
+  return launch_decode_attn_s8(q, k_new, v_new, k_buf, v_buf, nullptr, ctx, nullptr, BH, T, D, cap, S_max, heads,
+                               alpha_qk, alpha_pv, static_cast<hipStream_t>(stream), s_dev);
+}
+
 int ti_transpose_last2_s8(const int8_t* src, int8_t* dst, int64_t B, int64_t R, int64_t C, void* stream) {
   g_err[0] = 0;
   const char* op = "transpose_last2_s8";

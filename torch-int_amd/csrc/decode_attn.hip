@@ -46,8 +46,11 @@ __global__ __launch_bounds__(256) void decode_attn_kernel(const int8_t* __restri
                                                           const int8_t* __restrict__ v_new, int8_t* k_buf,
                                                           int8_t* v_buf, const float* __restrict__ mask,
                                                           int8_t* __restrict__ ctx, int8_t* __restrict__ probs_out,
-                                                          int T, int S, long long cap, int heads, float alpha_qk,
-                                                          float alpha_pv) {
+                                                          int T, int S_arg, long long cap, int heads, float alpha_qk,
+                                                          float alpha_pv, const int* __restrict__ s_dev) {
+  // s_dev != nullptr: the number of positions is read from device memory (a launch recorded in a HIP graph is
+  // replayed for a cache that has grown meanwhile; S_arg is then the largest length the launch was sized for)
+  const int S = s_dev != nullptr ? s_dev[0] : S_arg;
   constexpr int LPR = D / 16;    // lanes per cache row
   constexpr int RPW = 64 / LPR;  // rows per wave per load
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -245,7 +248,9 @@ bool decode_attn_supported(long long T, long long S, long long D) {
 int launch_decode_attn_s8(const int8_t* q, const int8_t* k_new, const int8_t* v_new, int8_t* k_buf, int8_t* v_buf,
                           const float* mask, int8_t* ctx, int8_t* probs_out, long long BH, long long T, long long D,
                           long long cap, long long S, long long heads, float alpha_qk, float alpha_pv,
-                          hipStream_t stream) {
+                          hipStream_t stream, const int* s_dev) {
+  // with s_dev the kernel reads the length from device memory; S is the largest value it may find there (the LDS
+  // and the kernel variant are sized for it)
   if (BH == 0) return TI_OK;
   if (!decode_attn_supported(T, S, D))
     return fail(TI_ERR_INVALID_ARG, "decode_attn: unsupported shape (T=%lld S=%lld head_dim=%lld)", T, S, D);
@@ -256,7 +261,7 @@ int launch_decode_attn_s8(const int8_t* q, const int8_t* k_new, const int8_t* v_
   // the variant that issues all loads up front
 #define TI_DA(TQ, DD, NI)                                                                                              \
   hipLaunchKernelGGL((decode_attn_kernel<TQ, DD, NI>), grid, block, lds, stream, q, k_new, v_new, k_buf, v_buf, mask, \
-                     ctx, probs_out, (int)T, (int)S, cap, (int)heads, alpha_qk, alpha_pv)
+                     ctx, probs_out, (int)T, (int)S, cap, (int)heads, alpha_qk, alpha_pv, s_dev)
   const bool resident = T <= 2 && S <= 20 * 4 * (64 / (D / 16));
   if (D == 128) {
     if (T == 1) { if (resident) TI_DA(1, 128, 20); else TI_DA(1, 128, 0); }

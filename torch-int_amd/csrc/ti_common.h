@@ -242,7 +242,7 @@ bool decode_attn_supported(long long T, long long S, long long D);
 int launch_decode_attn_s8(const int8_t* q, const int8_t* k_new, const int8_t* v_new, int8_t* k_buf, int8_t* v_buf,
                           const float* mask, int8_t* ctx, int8_t* probs_out, long long BH, long long T, long long D,
                           long long cap, long long S, long long heads, float alpha_qk, float alpha_pv,
-                          hipStream_t stream);
+                          hipStream_t stream, const int* s_dev = nullptr);
 int launch_kv_append_s8(const int8_t* knew, const int8_t* vnew, int8_t* kbuf, int8_t* vbuf, long long BH, long long T,
                         long long D, long long cap, long long S, hipStream_t stream);
 

@@ -52,6 +52,9 @@ _lib.ti_decode_attn_supported.restype = ctypes.c_int
 _lib.ti_decode_attn_s8.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32,
                                    _f32, _vp]
 _lib.ti_decode_attn_s8.restype = ctypes.c_int
+_lib.ti_decode_attn_s8_devlen.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _f32,
+                                              _f32, _vp]
+_lib.ti_decode_attn_s8_devlen.restype = ctypes.c_int
 _lib.ti_linear_a8_w8_b8_o8_heads.argtypes = [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _f32, _f32, _i64, _i64, _vp, _i64, _vp]
 _lib.ti_linear_a8_w8_b8_o8_heads.restype = ctypes.c_int
 _pp = ctypes.POINTER(ctypes.c_void_p)
@@ -443,6 +446,29 @@ def decode_attention(q, k_new, v_new, k_buf, v_buf, filled, mask, alpha_qk, alph
     if rc:
         raise RuntimeError(f"torch_int._hip_ext.decode_attention: {_lib.ti_last_error().decode()} (status {rc})")
     return ctx, probs
+
+
+def decode_attention_devlen(q, k_new, v_new, k_buf, v_buf, length, max_length, alpha_qk, alpha_pv):
+    """``decode_attention`` without a mask for a launch that is captured into a HIP graph and replayed while the cache
+    grows: the number of positions after the append is read from ``length`` (int32 HIP tensor of one element, set
+    by the caller before every replay; T <= length <= max_length <= capacity) when the kernel runs.  Returns ctx
+    int8 [B*H, T, d]."""
+    if not (can_decode_attention(q, k_new, v_new, k_buf, v_buf, max_length - q.shape[2], None)
+            and _ok(length, torch.int32) and length.numel() == 1 and length.device == q.device):
+        raise RuntimeError("torch_int._hip_ext.decode_attention_devlen: needs contiguous int8 HIP q/k_new/v_new "
+                           "[B,H,T,d] (T <= 4, d 64 or 128), cache buffers [B,H,cap,d] with cap >= max_length, and an "
+                           "int32 HIP tensor holding the length")
+    B, H, T, d = q.shape
+    dev = q.device
+    ctx = torch.empty((B * H, T, d), dtype=torch.int8, device=dev)
+    with _on(dev):
+        rc = _lib.ti_decode_attn_s8_devlen(q.data_ptr(), k_new.data_ptr(), v_new.data_ptr(), k_buf.data_ptr(),
+                                           v_buf.data_ptr(), ctx.data_ptr(), B * H, T, d, k_buf.shape[2],
+                                           int(max_length), length.data_ptr(), H, alpha_qk, alpha_pv,
+                                           _raw_stream(dev.index) or None)
+    if rc:
+        raise RuntimeError(f"torch_int._hip_ext.decode_attention_devlen: {_lib.ti_last_error().decode()} (status {rc})")
+    return ctx
 
 
 def can_linear_group(x, weights, biases):

@@ -208,6 +208,22 @@ class Int8OPTAttention(nn.Module):
         ctx = _hip_ext.merge_heads(ctx, bsz, H, T, d)
         return self.out_proj(ctx), probs_out, present
 
+    def decode_step_devlen(self, hidden_states, k_buf, v_buf, length, max_length):
+        """Self-attention of one new token per sequence (int8 [bsz, 1, embed]) over cache buffers [bsz, heads, cap,
+        head_dim] whose length after the append is read from the int32 HIP tensor ``length`` when the kernels run
+        (``Int8OPTGraphDecoder`` records this once and replays it).  No mask, no head mask; the values of
+        ``forward`` with a cache of ``length - 1`` positions.  Returns the fp32 output of ``out_proj``."""
+        bsz, tgt_len, _ = hidden_states.shape
+        flat = self._qkv_grouped(hidden_states)
+        if flat is None or not (type(self.qk_bmm) is BMM_S8T_S8N_F32T and type(self.pv_bmm) is BMM_S8T_S8N_S8T):
+            raise RuntimeError("Int8OPTAttention.decode_step_devlen: needs the stock int8 projections and products "
+                               "on contiguous HIP tensors")
+        query4, key, value = (self._shape(t, tgt_len, bsz) for t in flat)
+        ctx = _hip_ext.decode_attention_devlen(query4, key, value, k_buf, v_buf, length, max_length,
+                                               self.qk_bmm._scalar("a"), self.pv_bmm._scalar("a"))
+        ctx = _hip_ext.merge_heads(ctx, bsz, self.num_heads, tgt_len, self.head_dim)
+        return self.out_proj(ctx)
+
     def forward(self, hidden_states: torch.Tensor, key_value_states: Optional[torch.Tensor] = None,
                 past_key_value: Optional[Tuple[torch.Tensor]] = None,
                 attention_mask: Optional[torch.Tensor] = None,
@@ -354,6 +370,20 @@ class Int8OPTDecoderLayer(nn.Module):
         q.fc1 = W8A8B8O8LinearReLU.from_float(module.fc1, fc1_input_scale, fc2_input_scale)
         q.fc2 = W8A8BFP32OFP32Linear.from_float(module.fc2, fc2_input_scale)
         return q
+
+    def decode_step_devlen(self, hidden_states, k_buf, v_buf, length, max_length):
+        """``forward`` for one new token per sequence with the cache length read on the device (see
+        ``Int8OPTAttention.decode_step_devlen``): updates ``hidden_states`` in place and appends to the cache."""
+        residual = hidden_states
+        x = self.self_attn_layer_norm(hidden_states)
+        x = self.self_attn.decode_step_devlen(x, k_buf, v_buf, length, max_length)
+        x = self.final_layer_norm(residual, add=x)
+        x = self.fc1(x)
+        if type(self.fc2) is W8A8BFP32OFP32Linear:
+            self.fc2(x, add_to=residual)
+        else:
+            residual.add_(self.fc2(x).to(residual.dtype))
+        return residual
 
     def forward(self, hidden_states: torch.Tensor, attention_mask: Optional[torch.Tensor] = None,
                 layer_head_mask: Optional[torch.Tensor] = None, output_attentions: Optional[bool] = False,
@@ -650,3 +680,90 @@ class Int8OPTForCausalLM(nn.Module):
     @staticmethod
     def _reorder_cache(past, beam_idx):
         return tuple(tuple(s.index_select(0, beam_idx) for s in layer) for layer in past)
+
+
+class Int8OPTGraphDecoder:
+    """Token-by-token decoding of an ``Int8OPTForCausalLM`` on HIP with the decoder layers of a step replayed from
+    one HIP graph (no counterpart upstream, whose ``generate`` re-issues every launch from Python).
+
+    A decode step of a small or medium model is bound by the host: seven launches per layer and the Python around
+    them.  Here the layers are recorded once, on fixed buffers: the residual stream of the new token, the key /
+    value caches (buffers with room for ``max_new_tokens`` more positions) and an int32 tensor holding the cache
+    length, which the attention kernel reads when it runs, so the same recording serves every step.  Embeddings,
+    the final LayerNorm and ``lm_head`` stay ordinary torch calls around the replay.  No padding inside the batch
+    (every sequence has the same length) and no head mask.  Values are those of ``lm(ids, past_key_values=...)``.
+
+        out = lm(prompt_ids, use_cache=True)
+        dec = Int8OPTGraphDecoder(lm, out.past_key_values, max_new_tokens=128)
+        tok = out.logits[:, -1].argmax(-1, keepdim=True)
+        for _ in range(128):
+            tok = dec.step(tok)[:, -1].argmax(-1, keepdim=True)
+    """
+
+    @torch.no_grad()
+    def __init__(self, lm, past_key_values, max_new_tokens):
+        dec = lm.model.decoder
+        k0 = past_key_values[0][0]
+        if not (k0.is_cuda and k0.dtype is torch.int8 and k0.dim() == 4 and len(past_key_values) == len(dec.layers)):
+            raise RuntimeError("Int8OPTGraphDecoder: needs the int8 HIP key/value caches of every decoder layer")
+        bsz, H, S0, d = k0.shape
+        self.lm, self.filled, self.max_length = lm, S0, S0 + int(max_new_tokens)
+        if max_new_tokens < 1 or self.max_length > dec.max_target_positions:
+            raise RuntimeError(f"Int8OPTGraphDecoder: {S0} cached + {max_new_tokens} new positions exceed the model's "
+                               f"{dec.max_target_positions}")
+        if not _hip_ext.decode_attention_shape_ok(1, self.max_length, d):
+            raise RuntimeError(f"Int8OPTGraphDecoder: the decode attention kernel does not take {self.max_length} "
+                               f"positions of head size {d}")
+        cap = -(-self.max_length // 16) * 16
+        self.caches = []
+        for k, v in past_key_values:
+            kb = torch.empty((bsz, H, cap, d), dtype=torch.int8, device=k0.device)
+            vb = torch.empty_like(kb)
+            kb[:, :, :S0].copy_(k)
+            vb[:, :, :S0].copy_(v)
+            self.caches.append((kb, vb))
+        stream_dtype = dec.embed_positions.weight.dtype
+        self.hidden = torch.zeros((bsz, 1, dec.embed_positions.weight.shape[1]), dtype=stream_dtype, device=k0.device)
+        self.length = torch.full((1,), S0 + 1, dtype=torch.int32, device=k0.device)
+        self._ones = torch.ones((bsz, self.max_length), dtype=torch.bool, device=k0.device)
+
+        def layers():
+            for layer, (kb, vb) in zip(dec.layers, self.caches):
+                layer.decode_step_devlen(self.hidden, kb, vb, self.length, self.max_length)
+        # one eager pass first: scalar caches, kernel attributes and the allocator's pools are then warm, and nothing
+        # in the recording synchronises.  It writes position S0 of the caches, which the first real step overwrites.
+        side = torch.cuda.Stream(device=k0.device)
+        side.wait_stream(torch.cuda.current_stream(k0.device))
+        with torch.cuda.stream(side):
+            layers()
+        torch.cuda.current_stream(k0.device).wait_stream(side)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            layers()
+
+    @torch.no_grad()
+    def step(self, input_ids):
+        """Logits [bsz, 1, vocab] for one new token per sequence (``input_ids`` [bsz, 1]); the caches grow by one."""
+        if self.filled >= self.max_length:
+            raise RuntimeError("Int8OPTGraphDecoder: max_new_tokens steps have been taken")
+        dec = self.lm.model.decoder
+        embeds = dec.embed_tokens(input_ids)
+        pos = dec.embed_positions(self._ones[:, :self.filled + 1], self.filled)
+        if dec.project_in is not None:
+            embeds = dec.project_in(embeds)
+        self.hidden.copy_(embeds + pos)
+        self.length.fill_(self.filled + 1)
+        self.graph.replay()
+        self.filled += 1
+        hidden = self.hidden
+        if dec.final_layer_norm is not None:
+            hidden = dec.final_layer_norm(hidden)
+        if dec.project_out is not None:
+            hidden = dec.project_out(hidden)
+        return self.lm.lm_head(hidden.to(self.lm.lm_head.weight.dtype)).contiguous()
+
+    @property
+    def past_key_values(self):
+        """The caches as ``forward`` would return them: per layer (key, value) int8 [bsz, heads, filled, head_dim]."""
+        return tuple((kb[:, :, :self.filled], vb[:, :, :self.filled]) for kb, vb in self.caches)
+
