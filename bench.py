@@ -419,6 +419,7 @@ def main():
             "protocol": "same cases, each alone: 100 warm-up launches, then >= 200 ms of back-to-back launches "
                         "between two HIP events (upstream benchmark/utils.py:81-96)"}
         result["cases"] = table
+        torch.cuda.empty_cache()   # the per-case section leaves gigabytes of split blocks in the caching allocator
         result["hbm_kernels"] = hbm_kernels(torch, C, dev)
         result["decoder_layer_ms"] = decoder_layer_ms(torch, dev)
     if not args.no_cpu_baseline:
