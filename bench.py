@@ -399,6 +399,11 @@ def main():
             if c["M"] < 2048:   # weights dominate the traffic: keep them out of the last-level cache
                 key = (c["N"], c["K"])
                 if key not in copies:
+                    # one (N, K) at a time: the copies of the previous shape go back to the device first, so that
+                    # torch's caching allocator is not left with gigabytes of split blocks (every output
+                    # allocation then costs the host about 10 us, which a 7 us launch cannot hide)
+                    copies.clear()
+                    torch.cuda.empty_cache()
                     n_copies = -(-320 * 2 ** 20 // (c["N"] * c["K"]))
                     copies[key] = [c["w"]] + [c["w"].clone() for _ in range(n_copies - 1)]
                 fns = [c["make"](w) for w in copies[key]]
