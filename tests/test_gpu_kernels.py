@@ -437,6 +437,29 @@ def test_int8_layout_kernels():
         assert out.is_contiguous() and torch.equal(out, t.transpose(1, 2).contiguous())
 
 
+def test_stream_kernel_strip_orders_and_ragged_widths():
+    # the M <= 16 streaming kernel: grids that are and are not a multiple of 8 (two strip orders), several strips
+    # per workgroup with a last partial run of 8, widths that are not a multiple of 16 or of 4 (the prefetched
+    # bias and old-output loads are clamped there), every row count class (1, <= 4, <= 16), all output kinds
+    import ctypes
+    import torch_int._CUDA as C
+    C._lib.ti_last_kernel.restype = ctypes.c_char_p
+    g = torch.Generator().manual_seed(91)
+    for (M, N, K) in [(1, 4100, 1024), (2, 4102, 2048), (16, 4099, 1024), (1, 20500, 1024), (4, 16400, 1024),
+                      (13, 8200, 2048), (16, 20480, 1024)]:
+        for variant in ("b8_o8", "relu_b8_o8", "bfp32_ofp32", "b32_o32"):
+            _say(f"stream {variant} M={M} N={N} K={K}")
+            _linear_case(C, variant, M, N, K, seed=91)
+            assert C._lib.ti_last_kernel().decode() == "stream", (M, N, K, C._lib.ti_last_kernel())
+        _say(f"stream += M={M} N={N} K={K}")
+        x, w = _s8(g, M, K), _s8(g, N, K)
+        bias, resid = torch.randn(N, generator=g), torch.randn(M, N, generator=g) * 3
+        ref = orc.linear_a8_w8_bfp32_ofp32_acc(x, w, bias, 0.003, 1.0, resid)
+        out = C._linear_a8_w8_bfp32_ofp32_acc(x.to(DEV), w.to(DEV), bias.to(DEV), 0.003, 1.0, resid.to(DEV))
+        assert _ulp_diff(out.cpu(), ref) == 0, (M, N, K)
+        assert C._lib.ti_last_kernel().decode() == "stream"
+
+
 def test_linear_accumulate_into_output():
     # inout += alpha*acc + bias in the GEMM epilogue, through every kernel family the fp32 linear can take
     import ctypes
