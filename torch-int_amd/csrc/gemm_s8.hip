@@ -27,6 +27,7 @@ const char* last_gemm_kernel() { return g_last_kernel; }
 int launch_splitk_raw(int tile, const GemmParams& q, hipStream_t stream) {
   if (tile == SPLIT_128) return launch_pipe<PipeCfg<128, 128, 2, 2, 4, EPI_S32_RAW, false>>(q, stream);
   if (tile == SPLIT_256x160) return launch_pipe16q<Pipe16QCfg<256, 160, 4, 2, EPI_S32_RAW>>(q, stream);
+  if (tile == SPLIT_128x80) return launch_pipe16q<Pipe16QCfg<128, 80, 4, 1, EPI_S32_RAW>>(q, stream);
   if (tile == SPLIT_128x160) return launch_pipe16q<Pipe16QCfg<128, 160, 4, 2, EPI_S32_RAW>>(q, stream);
   if (tile == SPLIT_128x288) return launch_pipe16q<Pipe16QCfg<128, 288, 4, 2, EPI_S32_RAW>>(q, stream);
   if (tile == SPLIT_256x288) return launch_pipe16q<Pipe16QCfg<256, 288, 4, 2, EPI_S32_RAW>>(q, stream);

@@ -1249,7 +1249,9 @@ struct Pipe16QCfg {
   static constexpr int STAGE_BYTES = (BM + BN) * QBK;
   // three stages when the LDS holds them (256x160): copies then run two to three K steps ahead of their use,
   // which covers the latency of operands that come from HBM instead of the last-level cache
-  static constexpr int STAGES = (MAX_STAGES_ >= 3 && 3 * STAGE_BYTES <= 160 * 1024) ? 3 : 2;
+  // (128x80 tiles, whose short rounds are mostly that latency when the weights are not cached, take more)
+  static constexpr int FIT_STAGES = (160 * 1024) / STAGE_BYTES;
+  static constexpr int STAGES = MAX_STAGES_ < 2 ? 2 : FIT_STAGES < 2 ? 2 : MAX_STAGES_ < FIT_STAGES ? MAX_STAGES_ : FIT_STAGES;
   static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
   static constexpr int RPW = (BM + BN) / NWAVES;  // panel rows a wave copies per step
   static constexpr int TAIL_ROWS = RPW % 8;
@@ -1995,7 +1997,16 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmParams p, const 
 // once and read once (they mostly stay in the last-level cache), plus the second launch.  The
 // unsplit candidates are in the race too, so that a shape whose 256x160 or 256x288 tiles already fill
 // the chip is left to the ordinary dispatch.
-enum SplitTile { SPLIT_128 = 0, SPLIT_256 = 1, SPLIT_256x160 = 2, SPLIT_256x288 = 3, SPLIT_128x160 = 4, SPLIT_128x288 = 5 };
+//
+// 128x80 tiles (four waves, one per SIMD; 0.27 us per 64-byte step with weights from HBM, 0.47 us when two share
+// a CU, 2.5 us per round) are the one candidate that also stands for itself unsplit: at 512 rows and N = 5120 they
+// are 256 tiles over the whole of K in ONE launch, with no partial tiles and no second launch (cache-cold
+// 512x5120x5120: 29.2 -> 24.4 us, 384x5120x5120: 27.3 -> 24.3 us, 1024x5120x5120: 42.7 -> 40.1 us; split,
+// 128x5120x5120: 19.6 -> 16.4 us), although a workgroup of this shape multiplies at half the rate of a 256x160 one
+// (its four waves read 7 fragments from the LDS per 10 MFMAs); with K = 20480 the larger tiles win
+// (512x5120x20480: 79 against 64 us).  More than three LDS stages did not help it (four to six: +1 to +3 %).
+enum SplitTile { SPLIT_128 = 0, SPLIT_256 = 1, SPLIT_256x160 = 2, SPLIT_256x288 = 3, SPLIT_128x160 = 4, SPLIT_128x288 = 5,
+                 SPLIT_128x80 = 6 };
 static int choose_splits(long long M, long long N, long long K, int* tile_kind = nullptr) {
   if (tile_kind) *tile_kind = SPLIT_128;
   if (M <= 16 || M > 1024 || K % PBK != 0 || K < 1024) return 1;
@@ -2005,12 +2016,14 @@ static int choose_splits(long long M, long long N, long long K, int* tile_kind =
   double best_t = 1e30;
   // the 128-row forms of the tall tiles first, then by size: a later candidate must be clearly faster to replace
   // an earlier one
-  const int order[6] = {SPLIT_128x160, SPLIT_128x288, SPLIT_128, SPLIT_256, SPLIT_256x160, SPLIT_256x288};
-  for (int oi = 0; oi < 6; ++oi) {
+  const int order[7] = {SPLIT_128x80, SPLIT_128x160, SPLIT_128x288, SPLIT_128, SPLIT_256, SPLIT_256x160, SPLIT_256x288};
+  for (int oi = 0; oi < 7; ++oi) {
     const int kind = order[oi];
     const bool half = kind == SPLIT_128x160 || kind == SPLIT_128x288;  // 128-row forms of the two tall tiles
-    const int bm = kind == SPLIT_128 || half ? 128 : 256;
-    const int bn = kind == SPLIT_128 ? 128 : kind == SPLIT_256 ? 256 : kind == SPLIT_256x288 || kind == SPLIT_128x288 ? 288 : 160;
+    const bool small = kind == SPLIT_128x80;
+    const int bm = kind == SPLIT_128 || half || small ? 128 : 256;
+    const int bn = small ? 80 : kind == SPLIT_128 ? 128 : kind == SPLIT_256 ? 256
+                   : kind == SPLIT_256x288 || kind == SPLIT_128x288 ? 288 : 160;
     if (kind >= SPLIT_256x160 && N % bn != 0) continue;
     const double tiles = (double)((M + bm - 1) / bm) * (double)((N + bn - 1) / bn);
     for (int s = 1; s <= 16; ++s) {
@@ -2019,12 +2032,16 @@ static int choose_splits(long long M, long long N, long long K, int* tile_kind =
       if (half && s == 1) continue;                                // exist as raw-int32 kernels only
       // an unsplit candidate stands for what the ordinary dispatch would launch, which takes the 256-row tiles only
       // when they fill most of the chip (and 128x128 tiles otherwise)
-      if (s == 1 && kind != SPLIT_128 && tiles < 0.75 * cus) continue;
+      if (s == 1 && kind != SPLIT_128 && !small && tiles < 0.75 * cus) continue;
       const double wgs = tiles * s;
       double rounds, step_us, fixed_us = 8.0;
       if (kind == SPLIT_128) {
         rounds = (double)(long long)((wgs + 2 * cus - 1) / (2 * cus));
         step_us = wgs <= cus ? 0.35 : 0.70;
+      } else if (small) {  // two fit a CU and then share it
+        rounds = wgs <= cus ? 1.0 : (double)(long long)((wgs + 2 * cus - 1) / (2 * cus));
+        step_us = wgs <= cus ? 0.27 : 0.47;
+        fixed_us = 2.5;
       } else {
         rounds = (double)(long long)((wgs + cus - 1) / cus);
         step_us = kind == SPLIT_256 ? 0.85 : kind == SPLIT_256x160 ? 0.55 : kind == SPLIT_256x288 ? 0.92
@@ -2034,7 +2051,7 @@ static int choose_splits(long long M, long long N, long long K, int* tile_kind =
       double t = rounds * ((double)(steps / s) * step_us + fixed_us);
       // The weights come from HBM: a workgroup keeps about `ahead` K steps of its weight rows in flight, and what
       // all resident workgroups have in flight over a 2 us round trip bounds the streaming rate (5 TB/s at most).
-      const double ahead = kind == SPLIT_128 ? 4.0 : kind == SPLIT_256x160 || half ? 2.5 : 1.5;
+      const double ahead = kind == SPLIT_128 ? 4.0 : kind == SPLIT_256x160 || half || small ? 2.5 : 1.5;
       const double step_bytes = (double)bn * (kind == SPLIT_128 ? 64.0 : 128.0);
       const double resident = wgs < cus * (kind == SPLIT_128 ? 2 : 1) ? wgs : cus * (kind == SPLIT_128 ? 2 : 1);
       double rate = resident * ahead * step_bytes / 2.0;  // bytes per us
@@ -2042,7 +2059,7 @@ static int choose_splits(long long M, long long N, long long K, int* tile_kind =
       // (128x9216x36864: 110 us against 83 us with 128x288 tiles)
       const double cap = kind == SPLIT_128 ? 3.5e6 : 5.0e6;
       if (rate > cap) rate = cap;
-      const double t_stream = (double)N * (double)K / rate + 8.0;
+      const double t_stream = (double)N * (double)K / rate + (small ? 4.0 : 8.0);
       if (t < t_stream) t = t_stream;
       if (s > 1) t += (double)(2 * s + 1) * M * N * 4.0 / 5.5e6 + 3.0;  // partials out and back in, at 5.5 TB/s, in us
       if (t < best_t * 0.97) {  // prefer fewer slices and the smaller tile unless the gain is clear
@@ -2121,6 +2138,10 @@ int launch_kind(const GemmParams& p, void* workspace, long long workspace_bytes,
     int tile = SPLIT_128;
     const int splits = choose_splits(p.M, p.N, p.K, &tile);
     const long long need = (long long)splits * p.M * p.N * 4;
+    if (splits == 1 && tile == SPLIT_128x80) {
+      g_last_kernel = "pipe16_128x80";
+      return launch_pipe16q<Pipe16QCfg<128, 80, 4, 1, KIND>>(p, stream);
+    }
     if (splits > 1 && workspace != nullptr && workspace_bytes >= need &&
         (reinterpret_cast<uintptr_t>(workspace) & 15) == 0) {
       g_last_kernel = tile == SPLIT_128      ? "splitk_128x128"
@@ -2128,6 +2149,7 @@ int launch_kind(const GemmParams& p, void* workspace, long long workspace_bytes,
                       : tile == SPLIT_256x160 ? "splitk_256x160"
                       : tile == SPLIT_128x160 ? "splitk_128x160"
                       : tile == SPLIT_128x288 ? "splitk_128x288"
+                      : tile == SPLIT_128x80  ? "splitk_128x80"
                                               : "splitk_256x288";
       GemmParams q = p;  // the K slices are the batches of one raw-int32 GEMM into the workspace
       q.K = p.K / splits;
