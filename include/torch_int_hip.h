@@ -59,6 +59,16 @@ int64_t ti_linear_workspace_bytes(int64_t M, int64_t N, int64_t K);
  * "skinny", "tile_*", "scalar"; "" before the first call).  Benchmarks use it to label their rows. */
 const char* ti_last_kernel(void);
 
+/* Switch (no counterpart in the reference): split-K linears whose tile is one of the 16x16-block kernel's and
+ * divides M run as ONE launch ("fusedk_*" in ti_last_kernel): the K slices of an output tile run on workgroups
+ * of one XCD and meet in its L2, the last wave to arrive adds them up and applies the epilogue; same bits as the
+ * two-launch form ("splitk_*": raw int32 slices + a reduction kernel), which everything else takes.
+ * enable = 1 / 0 turns the one-launch form on / off for the process, -1 leaves it; returns the setting before
+ * the call.  Default on, or off with the environment variable TORCH_INT_FUSED_SPLITK=0.  The form also stays off
+ * on a device whose workgroup placement is not "ids congruent mod 8 share an XCD" (probed at the first use),
+ * for more than 8 streams per device, and while a stream is being captured before the first use on its device. */
+int ti_fused_splitk(int enable);
+
 /* Diagnostic (no counterpart in the reference; computes nothing): one launch that issues the instruction mix of
  * the tiled GEMM mainloop `iters` times per wave on the first MiB of `data` (device memory, at least 1 MiB, 16-byte
  * aligned), so that a benchmark can measure what the matrix pipe of this board sustains for a given operand

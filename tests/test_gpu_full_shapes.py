@@ -85,7 +85,7 @@ def test_linear_sweep_opt13b(N, K):
             if M <= 16:
                 assert family == "stream", family
             else:
-                assert family.startswith(("pipe", "splitk", "mid")), family
+                assert family.startswith(("pipe", "splitk", "fusedk", "mid")), family
             assert out.shape == (M, N)
             got, want = out[rows.to(DEV)].cpu(), ref()
             assert got.dtype == want.dtype

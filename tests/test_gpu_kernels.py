@@ -40,6 +40,16 @@ def _ulp_diff(a, b):
     return (ai - bi).abs().max().item() if a.numel() else 0
 
 
+@pytest.fixture
+def two_launch_split_k():
+    """Split-K linears take the two-launch form (raw int32 slices + reduction kernel) even where the one-launch form
+    would run, so that the tests that walk through the kernel families still reach those kernels."""
+    import torch_int._CUDA as C
+    before = C._lib.ti_fused_splitk(0)
+    yield
+    C._lib.ti_fused_splitk(before)
+
+
 def _linear_case(C, variant, M, N, K, seed, alpha=None, beta=None):
     g = torch.Generator().manual_seed(seed)
     x, w = _s8(g, M, K), _s8(g, N, K)
@@ -105,7 +115,7 @@ def test_linear_large_tiles(variant):
         _linear_case(C, variant, M, N, K, seed=7)
 
 
-def test_every_gemm_kernel_family_is_reached_and_exact():
+def test_every_gemm_kernel_family_is_reached_and_exact(two_launch_split_k):
     # one shape per dispatch branch; the library reports which kernel family it launched
     import ctypes
     import torch_int._CUDA as C
@@ -462,7 +472,75 @@ def test_stream_kernel_strip_orders_and_ragged_widths():
         assert C._lib.ti_last_kernel().decode() == "stream"
 
 
-def test_linear_accumulate_into_output():
+def test_one_launch_split_k_is_exact_for_every_output_kind():
+    # 2 to 4 K slices on a tile of the 16x16-block kernel that divides M: the slices of a tile meet in one XCD's L2 and
+    # the wave that arrives last applies the epilogue.  Every tile shape, every epilogue, sampled rows against the
+    # oracle and all rows against the two-launch form; called three times in a row (the arrival counters must be back
+    # at zero after each call) and on a second stream (which gets counters of its own).
+    import ctypes
+    import torch_int._CUDA as C
+    import torch_int._hip_ext as X
+    lib = C._lib
+    lib.ti_last_kernel.restype = ctypes.c_char_p
+    assert lib.ti_fused_splitk(1) in (0, 1)
+    try:
+        g = torch.Generator().manual_seed(97)
+        side = torch.cuda.Stream()
+        for (M, N, K, tile) in [(256, 640, 2048, "128x80"), (256, 2880, 3584, "128x80"), (256, 3200, 7168, "128x160"),
+                                (896, 1600, 6144, "128x160"), (128, 4608, 2048, "128x288"), (128, 9216, 2048, "128x288"),
+                                (768, 3840, 9216, "256x160"), (1024, 9216, 2560, "256x288")]:
+            x, w = _s8(g, M, K), _s8(g, N, K)
+            b8, bf = _s8(g, N), torch.randn(N, generator=g)
+            b32 = torch.randint(-65535, 65535, (N,), dtype=torch.int32, generator=g)
+            resid = torch.randn(M, N, generator=g) * 3
+            alpha, beta = _scal(g, 1e-4, 1e-2), _scal(g, 1e-4, 1e-2)
+            xd, wd, b8d, bfd, b32d = x.to(DEV), w.to(DEV), b8.to(DEV), bf.to(DEV), b32.to(DEV)
+            rows = torch.arange(M) if M <= 256 else torch.cat([torch.arange(0, 64), torch.arange(M // 2 - 32, M // 2 + 32),
+                                                                torch.arange(M - 64, M)])
+            acc = orc.gemm_acc(x[rows].contiguous(), w)
+            heads_d = 128 if N % 128 == 0 else 64 if N % 64 == 0 else 32
+            runs = [
+                ("b32_o32", lambda: C.linear_a8_w8_b32_o32(xd, wd, b32d), lambda: orc.epi_b32_o32(acc, b32)),
+                ("b32_o32_scaled", lambda: C.linear_a8_w8_b32_o32_with_scaling(xd, wd, b32d, alpha, beta),
+                 lambda: orc.epi_b32_o32_scaled(acc, b32, alpha, beta)),
+                ("bfp32_ofp32", lambda: C.linear_a8_w8_bfp32_ofp32(xd, wd, bfd, alpha, 1.0),
+                 lambda: orc.epi_bfp32_ofp32(acc, bf, alpha, 1.0)),
+                ("b8_o8", lambda: C.linear_a8_w8_b8_o8(xd, wd, b8d, alpha, beta), lambda: orc.epi_b8_o8(acc, b8, alpha, beta)),
+                ("relu_b8_o8", lambda: C.linear_relu_a8_w8_b8_o8(xd, wd, b8d, alpha, beta),
+                 lambda: orc.epi_b8_o8(acc, b8, alpha, beta, relu=True)),
+                ("bfp32_ofp32 +=", lambda: C._linear_a8_w8_bfp32_ofp32_acc(xd, wd, bfd, alpha, 1.0, resid.to(DEV)),
+                 lambda: resid[rows] + orc.epi_bfp32_ofp32(acc, bf, alpha, 1.0)),
+                ("b8_o8 head-major",
+                 lambda: X.linear_a8_w8_b8_o8_heads(xd, wd, b8d, alpha, beta, 1, M, N // heads_d, heads_d)
+                 .permute(0, 2, 1, 3).reshape(M, N), lambda: orc.epi_b8_o8(acc, b8, alpha, beta)),
+            ]
+            for name, gpu, ref in runs:
+                _say(f"one-launch split-K {name} M={M} N={N} K={K}")
+                outs = [gpu() for _ in range(3)]
+                assert lib.ti_last_kernel().decode() == "fusedk_" + tile, (M, N, K, lib.ti_last_kernel())
+                with torch.cuda.stream(side):
+                    side.wait_stream(torch.cuda.current_stream())
+                    outs.append(gpu())
+                torch.cuda.current_stream().wait_stream(side)
+                lib.ti_fused_splitk(0)
+                two = gpu()
+                assert lib.ti_last_kernel().decode() == "splitk_" + tile, lib.ti_last_kernel()
+                lib.ti_fused_splitk(1)
+                want = ref()
+                for o in outs:
+                    assert torch.equal(o, two), (name, M, N, K)
+                if name == "bfp32_ofp32 +=":   # one rounding of the sum on the device, as the oracle's fused form does
+                    want = orc.linear_a8_w8_bfp32_ofp32_acc(x[rows].contiguous(), w, bf, alpha, 1.0, resid[rows].contiguous())
+                assert torch.equal(two[rows.to(DEV)].cpu(), want), (name, M, N, K)
+        # a ragged M, or more than four slices, stays with the two-launch form
+        for (M, N, K) in [(200, 640, 4096), (128, 640, 4096)]:
+            _linear_case(C, "b8_o8", M, N, K, seed=98)
+            assert lib.ti_last_kernel().decode().startswith("splitk_"), (M, N, K, lib.ti_last_kernel())
+    finally:
+        lib.ti_fused_splitk(1)
+
+
+def test_linear_accumulate_into_output(two_launch_split_k):
     # inout += alpha*acc + bias in the GEMM epilogue, through every kernel family the fp32 linear can take
     import ctypes
     import torch_int._CUDA as C
@@ -532,7 +610,7 @@ def test_bmm_rowmajor_rhs_for_decode():
     assert torch.equal(out, orc.bmm_s8t_s8t_s8t(a, b[:, 1:, :].contiguous(), 0.001))
 
 
-def test_head_major_projection_through_every_kernel_family():
+def test_head_major_projection_through_every_kernel_family(two_launch_split_k):
     # the s8 linear whose stores write [bsz, heads, seq, d]: same values as the plain linear, permuted
     import ctypes
     import torch_int._CUDA as C

@@ -62,12 +62,12 @@ def test_noalloc_linear_matches_the_workspace_entry_point_twice_in_a_row():
     # first a split-K shape that fills most of the scratch, then a smaller one that reuses its first bytes
     _say("noalloc 512x9216x9216 (split-K, 36 MiB of partial products)")
     x, w, b, out, kern = _both(lib, 512, 9216, 9216, 5, 0.0007, 0.02)
-    assert kern.startswith("splitk"), kern
+    assert kern.startswith(("splitk", "fusedk")), kern
     rows = torch.arange(0, 512, 7)
     assert torch.equal(out[rows], orc.linear_a8_w8_b8_o8(x[rows], w, b, 0.0007, 0.02, acc_fn=orc.gemm_acc_torch))
     _say("noalloc 128x640x4096 (split-K, smaller)")
     x, w, b, out, kern = _both(lib, 128, 640, 4096, 6, 0.002, 0.01)
-    assert kern.startswith("splitk"), kern
+    assert kern.startswith(("splitk", "fusedk")), kern
     assert torch.equal(out, orc.linear_a8_w8_b8_o8(x, w, b, 0.002, 0.01))
     # shapes that need no scratch go through unchanged: decode, prefill and an odd K
     for (M, N, K) in [(1, 5120, 5120), (2048, 768, 768), (33, 17, 100)]:

@@ -139,7 +139,9 @@ int ti_init(void) {
   if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
     return fail(TI_ERR_NO_DEVICE, "device %d is %s; this library holds gfx950 code only", dev, prop.gcnArchName);
   void* ptr = nullptr;  // resolve the no-allocation entry point's scratch here, outside any capture or hot loop
-  return scratch_address("ti_init", &ptr);
+  if (int rc = scratch_address("ti_init", &ptr)) return rc;
+  (void)warm_fused_split(nullptr);  // and probe the workgroup placement the one-launch split-K relies on
+  return TI_OK;
 }
 
 int64_t ti_linear_workspace_bytes(int64_t M, int64_t N, int64_t K) { return gemm_workspace_bytes(M, N, K); }
@@ -193,8 +195,13 @@ int ti_linear_a8_w8_b8_o8_noalloc(const int8_t* x, const int8_t* w, const int8_t
   if (need > 0) {
     if (int rc = scratch_address(op, &ws)) return rc;
   }
-  // the partial products are written in full before the reduction reads them: nothing to clear
-  return run_gemm(op, EPI_S8_BIAS, x, w, bias, 1, out, 1, 1, M, N, K, alpha, beta, ws, need > 0 ? need : 0, stream);
+  // the partial products are written in full before they are read: nothing to clear.  The one-launch split-K is
+  // taken only on a device where its one-time probe (which allocates) has already run, e.g. through ti_init().
+  allow_fused_split_probe(false);
+  const int rc = run_gemm(op, EPI_S8_BIAS, x, w, bias, 1, out, 1, 1, M, N, K, alpha, beta, ws, need > 0 ? need : 0,
+                          stream);
+  allow_fused_split_probe(true);
+  return rc;
 }
 
 int ti_linear_a8_w8_b8_o8_heads(const int8_t* x, const int8_t* w, const int8_t* bias, int8_t* out, int64_t M,
@@ -401,6 +408,8 @@ int ti_attn_softmax_q(const float* scores, const float* mask, int8_t* probs, int
 }
 
 const char* ti_last_kernel(void) { return last_gemm_kernel(); }
+
+int ti_fused_splitk(int enable) { return set_fused_split(enable); }
 
 int64_t ti_diag_mfma_loop_ops(int64_t iters) { return iters > 0 ? diag_mfma_loop_ops(iters) : 0; }
 

@@ -1,6 +1,9 @@
 // Host-side entry of the INT8 GEMM family: dispatch over the epilogue kinds (each kind's kernels are
 // compiled in a translation unit of their own, gemm_s8_kinds.hip with -DTI_KIND=n), the grouped q/k/v
 // launches, the split-K slice GEMM and the workspace query.
+#include <cstdlib>
+#include <mutex>
+
 #include "gemm_s8_impl.h"
 
 namespace ti {
@@ -23,6 +26,128 @@ int launch_gemm_kind_8(const GemmParams& p, void* ws, long long ws_bytes, hipStr
 
 thread_local const char* g_last_kernel = "";
 const char* last_gemm_kernel() { return g_last_kernel; }
+
+// ---------------------------------------------------------------------------
+// State of the one-launch split-K (the FUSED form of gemm_pipe16q_kernel), per device.
+//
+// Arrival counters: zero when the code object is loaded, and every launch leaves them zero (the wave that arrives
+// last puts its counter back).  Launches on one stream run one after the other, so each stream that uses the
+// fused form gets a block of counters of its own (kFusedStreams of them per device; further streams take the
+// two-launch form).
+//
+// Placement: the fused form needs all workgroups whose ids are congruent mod 8 to run on one XCD.  That is how the
+// hardware deals workgroups out (round robin over the XCDs; the XCD of workgroup 0 depends on the queue).  A probe
+// launch records the XCC id register of 256 workgroups once per device; unless it shows one XCC per residue class,
+// eight different ones, the fused form stays off.  Every fused launch checks itself as well: the workgroups of a
+// tile mark their XCC in a word of the tile, and one that finds another XCC's mark raises a flag in host memory;
+// the flag is looked at before every later launch and turns the fused form off with an error.
+static constexpr int kFusedStreams = 8;
+static constexpr int kFusedCounters = 32768;            // per stream: tiles x waves
+static constexpr int kFusedTiles = kFusedCounters / 8;  // per stream: one XCC word per tile
+static __device__ __align__(256) int g_fused_arrivals[kFusedStreams * (kFusedCounters + kFusedTiles)];
+
+__global__ void xcc_probe_kernel(unsigned* out) {
+  if (threadIdx.x == 0) out[blockIdx.x] = __builtin_amdgcn_s_getreg((3 << 11) | 20) & 0xf;  // HW_REG_XCC_ID
+}
+
+struct FusedDevice {
+  std::mutex lock;
+  int state = 0;  // 0 = not probed yet, 1 = usable, -1 = off
+  int* arrivals = nullptr;
+  int* host_words = nullptr;  // [0] = the misplacement flag, [1 .. 256] = the probe's output
+  int* host_words_dev = nullptr;
+  hipStream_t streams[kFusedStreams] = {};
+  int nstreams = 0;
+};
+static FusedDevice g_fused[64];
+
+// -1 = not decided yet: the environment variable TORCH_INT_FUSED_SPLITK=0 switches the form off
+static std::atomic<int> g_fused_on{-1};
+
+int set_fused_split(int enable) {
+  int before = g_fused_on.load(std::memory_order_relaxed);
+  if (before < 0) {
+    const char* v = getenv("TORCH_INT_FUSED_SPLITK");
+    before = !(v && v[0] == '0');
+  }
+  if (enable >= 0) g_fused_on.store(enable ? 1 : 0, std::memory_order_relaxed);
+  else g_fused_on.store(before, std::memory_order_relaxed);
+  return before;
+}
+static bool fused_enabled() { return set_fused_split(-1) != 0; }
+
+// The first use on a device allocates 1 KB of host memory and synchronises; a thread that must not allocate (the
+// entry point that promises it) clears this around its call and then only uses a device that is ready.
+static thread_local bool g_fused_may_probe = true;
+void allow_fused_split_probe(bool allow) { g_fused_may_probe = allow; }
+
+// counters < 0: only make the current device ready (the probe), on `stream`
+int fused_split_prepare(hipStream_t stream, long long counters, GemmParams& q) {
+  if (!fused_enabled() || counters > kFusedCounters) return 0;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+  FusedDevice& d = g_fused[dev];
+  std::lock_guard<std::mutex> guard(d.lock);
+  if (d.state == 0) {
+    if (!g_fused_may_probe) return 0;
+    // first use on this device: not while the stream records a graph (the probe allocates and synchronises)
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
+      (void)hipGetLastError();
+      return 0;
+    }
+    d.state = -1;
+    void* sym = nullptr;
+    if (hipGetSymbolAddress(&sym, HIP_SYMBOL(g_fused_arrivals)) != hipSuccess || sym == nullptr) return 0;
+    if (hipHostMalloc(reinterpret_cast<void**>(&d.host_words), 257 * sizeof(int), hipHostMallocMapped) != hipSuccess)
+      return 0;
+    if (hipHostGetDevicePointer(reinterpret_cast<void**>(&d.host_words_dev), d.host_words, 0) != hipSuccess)
+      return 0;
+    for (int i = 0; i < 257; ++i) d.host_words[i] = -1;
+    d.host_words[0] = 0;
+    hipLaunchKernelGGL(xcc_probe_kernel, dim3(256), dim3(64), 0, stream,
+                       reinterpret_cast<unsigned*>(d.host_words_dev + 1));
+    if (hipGetLastError() != hipSuccess || hipStreamSynchronize(stream) != hipSuccess) return 0;
+    unsigned seen = 0;
+    for (int i = 0; i < 256; ++i) {
+      const int xcc = d.host_words[1 + i];
+      if (xcc < 0 || xcc > 15 || xcc != d.host_words[1 + (i & 7)]) return 0;
+    }
+    for (int i = 0; i < 8; ++i) {
+      const unsigned xcc = (unsigned)d.host_words[1 + i];
+      if (seen & (1u << xcc)) return 0;  // two residue classes on one XCD: not the placement this needs
+      seen |= 1u << xcc;
+    }
+    d.arrivals = static_cast<int*>(sym);
+    d.state = 1;
+  }
+  if (d.state != 1) return 0;
+  if (*reinterpret_cast<volatile int*>(d.host_words) != 0) {
+    d.state = -1;  // a workgroup of an earlier fused launch ran on an unexpected XCD: its result cannot be trusted
+    return -fail(TI_ERR_LAUNCH, "an earlier one-launch split-K GEMM found a workgroup on an unexpected XCD and its "
+                                "result cannot be trusted; the form is now switched off (TORCH_INT_FUSED_SPLITK=0 "
+                                "avoids it from the start)");
+  }
+  if (counters < 0) return 1;
+  int slot = -1;
+  for (int i = 0; i < d.nstreams; ++i)
+    if (d.streams[i] == stream) slot = i;
+  if (slot < 0) {
+    if (d.nstreams == kFusedStreams) return 0;
+    slot = d.nstreams++;
+    d.streams[slot] = stream;
+  }
+  q.arrivals = d.arrivals + (long long)slot * (kFusedCounters + kFusedTiles);
+  q.xcc_seen = reinterpret_cast<unsigned*>(q.arrivals + kFusedCounters);
+  q.xcc_error = d.host_words_dev;
+  return 1;
+}
+
+int warm_fused_split(void* stream) {
+  GemmParams unused;
+  const int rc = fused_split_prepare(static_cast<hipStream_t>(stream), -1, unused);
+  return rc > 0 ? 1 : 0;
+}
 
 int launch_splitk_raw(int tile, const GemmParams& q, hipStream_t stream) {
   if (tile == SPLIT_128) return launch_pipe<PipeCfg<128, 128, 2, 2, 4, EPI_S32_RAW, false>>(q, stream);

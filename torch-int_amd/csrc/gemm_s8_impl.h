@@ -1236,9 +1236,22 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe16_kernel(GemmParams p, i
 
 // The 16x16-block kernel with K steps of 128 bytes and two LDS stages (see gemm_pipe2_kernel for the
 // stage layout and the step structure; a step here is two 64-byte slices, one MFMA deep each).
-template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int KIND_, bool GROUPED_ = false, int MAX_STAGES_ = 3>
+//
+// FUSED (split-K in one launch): the work items are (output tile, K slice) pairs, and ALL slices of a tile run on
+// workgroups of the SAME XCD (workgroup ids congruent mod 8), so that the int32 partial tiles meet in that XCD's
+// L2 and no device-scope release / acquire (which writes back and invalidates a whole L2) is needed.  Every wave
+// parks its accumulators in the workspace (16 bytes per lane and MFMA block, in register order), waits until the
+// L2 has acknowledged the stores, and counts itself on an arrival counter of (tile, wave index) with an atomic
+// that executes in the L2.  The wave that arrives last among the `splits` waves with its index adds the others'
+// accumulators to its own, applies the epilogue to its part of the tile and puts the counter back to zero.
+// Nobody waits for anybody, so there is nothing that can hang; integer sums make the result independent of
+// the order of arrival.
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int KIND_, bool GROUPED_ = false, int MAX_STAGES_ = 3,
+          bool FUSED_ = false>
 struct Pipe16QCfg {
   static constexpr int BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, KIND = KIND_;
+  static constexpr bool FUSED = FUSED_;
+  static_assert(!(FUSED_ && GROUPED_), "the fused split takes one problem");
   // GROUPED: the "batches" are the problems of a GemmGroup (same activations and shape; weight, bias,
   // output and scales per problem), so that q/k/v projections run as one persistent launch
   static constexpr bool GROUPED = GROUPED_;
@@ -1275,16 +1288,50 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe16q_kernel(GemmParams p, 
   const int M = p.M, N = p.N, K = p.K;
   const int KT = K / QBK;
   const int tiles = tiles_m * tiles_n;
-  const int first = blockIdx.x, stride = gridDim.x;
-  const int my_items = (items - first + stride - 1) / stride;
+  // Work items of this workgroup: first, first + stride, ... below `items`.  FUSED: the items of this workgroup's
+  // XCD (id mod 8; the grid is a multiple of 8) are numbered l = (tile of the XCD) * splits + slice, where the
+  // XCD's tiles are the tile ids congruent to the XCD mod 8.
+  const int xcd = blockIdx.x & 7;
+  const int first = Cfg::FUSED ? (int)(blockIdx.x >> 3) : (int)blockIdx.x;
+  const int stride = Cfg::FUSED ? (int)(gridDim.x >> 3) : (int)gridDim.x;
+  if constexpr (Cfg::FUSED) items = tiles > xcd ? ((tiles - xcd + 7) >> 3) * p.splits : 0;
+  const int my_items = items > first ? (items - first + stride - 1) / stride : 0;
+  if (my_items == 0) return;  // the same for every wave of the workgroup, before the first barrier
   const int G = my_items * KT;
+  // item -> (batch or K slice b, tile id)
+  auto decode_item = [&](int item, int& b, int& tile_id) {
+    if constexpr (Cfg::FUSED) {
+      const int t = item / p.splits;
+      b = item - t * p.splits;
+      tile_id = t * 8 + xcd;
+    } else {
+      b = item / tiles;
+      tile_id = item - b * tiles;
+    }
+  };
+  // FUSED: all workgroups of a tile must run on one XCC (the hardware deals workgroup ids out round robin, from a
+  // start that depends on the queue).  Checked, not assumed: thread 0 marks this workgroup's XCC id in the tile's
+  // word with a device-scope atomic when it takes the tile up and looks at the marks of the others when it is done.
+  unsigned xcc_bit = 0, xcc_others = 0;
+  auto mark_xcc = [&](int item) {
+    if constexpr (Cfg::FUSED) {
+      if (threadIdx.x == 0) {
+        int b, tile_id;
+        decode_item(item, b, tile_id);
+        xcc_bit = 1u << (__builtin_amdgcn_s_getreg((3 << 11) | 20) & 0xf);  // HW_REG_XCC_ID, bits 3:0
+        xcc_others = __hip_atomic_fetch_or(p.xcc_seen + tile_id, xcc_bit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+  };
+  mark_xcc(first);
 
   // ---- copy stream: copy j of this wave fills panel rows wave*RPW + 8j .. +7 of [A panel | B panel]
   const TI_GLOBAL_AS int8_t* src[COPIES];
   auto set_copy_item = [&](int item) {
-    const int b = item / tiles;
+    int b, tile_id;
+    decode_item(item, b, tile_id);
     int tile_m, tile_n;
-    tile_of_workgroup(item - b * tiles, tiles_m, tiles_n, tile_m, tile_n, p.band);
+    tile_of_workgroup(tile_id, tiles_m, tiles_n, tile_m, tile_n, p.band);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int8_t* A = Cfg::GROUPED ? p.A : p.A + (long long)b * p.strideA;
     const int8_t* B = Cfg::GROUPED ? grp.B[b] : p.B + (long long)b * p.strideB;
@@ -1419,12 +1466,57 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe16q_kernel(GemmParams p, 
     ++gs;
   };
   auto finish_item = [&]() {
-    const int b = item / tiles;
+    int b, tile_id;
+    decode_item(item, b, tile_id);
     int tile_m, tile_n;
-    tile_of_workgroup(item - b * tiles, tiles_m, tiles_n, tile_m, tile_n, p.band);
+    tile_of_workgroup(tile_id, tiles_m, tiles_n, tile_m, tile_n, p.band);
     int lane_here = lane;  // opaque copy: keeps the epilogue's address arithmetic out of the mainloop
     asm volatile("" : "+v"(lane_here));
-    if constexpr (Cfg::GROUPED) {
+    if constexpr (Cfg::FUSED) {
+      constexpr long long PER_WAVE = (long long)TM * TN * 64;  // v4i elements a wave parks per (tile, slice)
+      const int splits = p.splits;
+      v4i* parts = reinterpret_cast<v4i*>(p.parts);
+      v4i* mine = parts + (((long long)tile_id * splits + b) * Cfg::NWAVES + wave) * PER_WAVE + lane_here;
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) mine[(i * TN + j) * 64] = acc[i][j];
+      // acknowledged by the L2 (stores and loads share the counter: this also waits for the copies in flight)
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      if (threadIdx.x == 0 && (xcc_others & ~xcc_bit) != 0)  // a workgroup of this tile ran on another XCC
+        __hip_atomic_store(p.xcc_error, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      int* counter = p.arrivals + tile_id * Cfg::NWAVES + wave;
+      int earlier = 0;
+      if (lane_here == 0)
+        earlier = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      earlier = __builtin_amdgcn_readfirstlane(earlier);
+      if (earlier == splits - 1) {  // uniform over the wave
+        for (int t = 0; t < splits; ++t) {
+          if (t == b) continue;
+          const v4i* theirs = parts + (((long long)tile_id * splits + t) * Cfg::NWAVES + wave) * PER_WAVE + lane_here;
+          // two rows of blocks at a time: 2 TN loads in flight, then the adds (one statement per block would make
+          // the compiler wait for every load before it issues the next)
+          constexpr int RB = TM % 2 == 0 && TN <= 5 ? 2 : 1;
+#pragma unroll
+          for (int i0 = 0; i0 < TM; i0 += RB) {
+            v4i got[RB][TN];
+#pragma unroll
+            for (int i = 0; i < RB; ++i)
+#pragma unroll
+              for (int j = 0; j < TN; ++j) got[i][j] = theirs[((i0 + i) * TN + j) * 64];
+#pragma unroll
+            for (int i = 0; i < RB; ++i)
+#pragma unroll
+              for (int j = 0; j < TN; ++j) acc[i0 + i][j] += got[i][j];
+          }
+        }
+        if (lane_here == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        // every workgroup of the tile made its mark before its wave 0 counted itself: the last wave 0 clears the word
+        if (threadIdx.x == 0) __hip_atomic_store(p.xcc_seen + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        store_tile16<Cfg>(acc, p, 0, tile_m, tile_n, wave_m, wave_n, lane_here);
+      }
+      if (my_items > 1 && item + stride < items) mark_xcc(item + stride);
+    } else if constexpr (Cfg::GROUPED) {
       GemmParams q = p;  // problem b of the group as a one-batch problem
       q.bias = grp.bias[b];
       q.C = grp.C[b];
@@ -2079,6 +2171,33 @@ extern thread_local const char* g_last_kernel;
 // The raw-int32 GEMM over the K slices of a split-K linear (defined once, in gemm_s8.hip).
 int launch_splitk_raw(int tile, const GemmParams& q, hipStream_t stream);
 
+// Split-K inside one launch (defined once, in gemm_s8.hip): fills q.arrivals / q.xcc_of_id / q.xcc_error for a
+// launch with `counters` arrival counters on `stream` and returns 1, or returns 0 when that form cannot be used
+// here (switched off, the placement of workgroups on XCDs is not the expected one, the stream is being captured
+// before the first use, too many streams or counters) - the caller then takes the two-launch form - or minus a
+// TI_ERR_* code when an earlier fused launch reported a misplaced workgroup.
+int fused_split_prepare(hipStream_t stream, long long counters, GemmParams& q);
+
+// One launch of the FUSED form of the 16x16-block kernel: q.K is the slice length, q.splits the slice count.
+template <class Cfg>
+static int launch_fused(const GemmParams& q_in, hipStream_t stream) {
+  GemmParams q = q_in;
+  q.band = 3 * Cfg::BN <= 2 * Cfg::BM ? 4 : 8;
+  static std::atomic<unsigned long long> lds_ok{0};
+  if (int rc = allow_lds(gemm_pipe16q_kernel<Cfg>, Cfg::LDS_BYTES, lds_ok)) return rc;
+  const int tiles_m = q.M / Cfg::BM, tiles_n = q.N / Cfg::BN;  // whole tiles only (the caller checked)
+  const long long tiles = (long long)tiles_m * tiles_n;
+  // every XCD gets the same number of workgroups: enough for its tiles x slices, at most what is resident
+  const long long slots = (long long)num_cus() * ((160 * 1024) / Cfg::LDS_BYTES) / 8 * 8;
+  long long grid = ((tiles + 7) / 8) * q.splits * 8;
+  if (grid > slots) grid = slots;
+  hipLaunchKernelGGL(gemm_pipe16q_kernel<Cfg>, dim3((unsigned)grid), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, q, tiles_m,
+                     tiles_n, 0, GemmGroup{});
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "gemm launch: %s", hipGetErrorString(e));
+  return TI_OK;
+}
+
 template <int KIND>
 int launch_kind(const GemmParams& p, void* workspace, long long workspace_bytes, hipStream_t stream) {
   using Out = typename Epi<KIND>::Out;
@@ -2151,6 +2270,47 @@ int launch_kind(const GemmParams& p, void* workspace, long long workspace_bytes,
                       : tile == SPLIT_128x288 ? "splitk_128x288"
                       : tile == SPLIT_128x80  ? "splitk_128x80"
                                               : "splitk_256x288";
+      if constexpr (KIND != EPI_S32_RAW) {
+        // one launch when the tile is one of the 16x16-block kernel's and covers M in whole tiles
+        const int bm = tile == SPLIT_256x160 || tile == SPLIT_256x288 ? 256 : 128;
+        const int bn = tile == SPLIT_128x80 ? 80 : tile == SPLIT_256x160 || tile == SPLIT_128x160 ? 160 : 288;
+        const bool tall = tile == SPLIT_128x80 || tile == SPLIT_128x160 || tile == SPLIT_128x288 ||
+                          tile == SPLIT_256x160 || tile == SPLIT_256x288;
+        // up to four slices: the wave that arrives last reads the others' accumulators one slice after the other,
+        // and beyond four that tail costs more than the reduction launch it saves (measured: 2 slices -3 to -12 %,
+        // 4 slices -3 to -8 %, 7 and 8 slices +3 to +6 %)
+        if (tall && splits <= 4 && p.M % bm == 0 && p.N % bn == 0) {
+          const long long tiles = (long long)(p.M / bm) * (p.N / bn);
+          GemmParams f = p;
+          f.K = p.K / splits;
+          f.strideA = f.K;
+          f.strideB = f.K;
+          f.strideC = 0;
+          f.splits = splits;
+          f.parts = workspace;
+          const int usable = fused_split_prepare(stream, tiles * 8, f);
+          if (usable < 0) return -usable;
+          if (usable) {
+            switch (tile) {
+              case SPLIT_128x80:
+                g_last_kernel = "fusedk_128x80";
+                return launch_fused<Pipe16QCfg<128, 80, 4, 1, KIND, false, 3, true>>(f, stream);
+              case SPLIT_128x160:
+                g_last_kernel = "fusedk_128x160";
+                return launch_fused<Pipe16QCfg<128, 160, 4, 2, KIND, false, 3, true>>(f, stream);
+              case SPLIT_128x288:
+                g_last_kernel = "fusedk_128x288";
+                return launch_fused<Pipe16QCfg<128, 288, 4, 2, KIND, false, 3, true>>(f, stream);
+              case SPLIT_256x160:
+                g_last_kernel = "fusedk_256x160";
+                return launch_fused<Pipe16QCfg<256, 160, 4, 2, KIND, false, 3, true>>(f, stream);
+              default:
+                g_last_kernel = "fusedk_256x288";
+                return launch_fused<Pipe16QCfg<256, 288, 4, 2, KIND, false, 3, true>>(f, stream);
+            }
+          }
+        }
+      }
       GemmParams q = p;  // the K slices are the batches of one raw-int32 GEMM into the workspace
       q.K = p.K / splits;
       q.batch = splits;

@@ -179,6 +179,15 @@ struct GemmParams {
   int out_T = 0, out_d = 0;
   // Tile rows an XCD's run of tiles walks down before it moves to the next tile column (see tile_of_workgroup).
   int band = 8;
+  // Split-K inside one launch (the FUSED form of the 16x16-block kernel): K is the length of one slice, strideA and
+  // strideB step from slice to slice; `parts` holds splits x tiles parked accumulator tiles, `arrivals` one zeroed
+  // counter per (tile, wave), `xcc_seen` one zeroed word per tile in which the workgroups of the tile mark the XCC
+  // they run on, xcc_error = host-mapped word that is set when two of them differ.
+  int splits = 1;
+  void* parts = nullptr;
+  int* arrivals = nullptr;
+  unsigned* xcc_seen = nullptr;
+  int* xcc_error = nullptr;
 };
 
 // Offset of output element (m, n) of one batch; consecutive n stay consecutive inside a head, so vector
@@ -205,6 +214,9 @@ int launch_gemm_group_s8(const GemmParams& shape, const GemmGroup& grp, hipStrea
 int launch_gemm(int kind, const GemmParams& p, void* workspace, long long workspace_bytes,
                 hipStream_t stream);
 long long gemm_workspace_bytes(long long M, long long N, long long K);
+void allow_fused_split_probe(bool allow);  // per thread: may a GEMM call run the one-time placement probe?
+int warm_fused_split(void* stream);        // run that probe now (1 = the one-launch split-K is usable on this device)
+int set_fused_split(int enable);  // one-launch split-K on (1) / off (0) / unchanged (-1); returns the previous setting
 const char* last_gemm_kernel();  // kernel family of the calling thread's last launch_gemm ("" before the first)
 
 // ln_q.hip
