@@ -44,11 +44,11 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
 # the process: they come from rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) of this script's own sweep; commands,
 # raw counter values and the calibration against a plain copy kernel are in profiles/.
 FAMILIES = {
-    # 233 759 KiB x 2.000 fetched + 77 169 KiB written per launch, mean over its 24 launches per step (measured with
+    # 233 272 KiB x 2.000 fetched + 77 050 KiB written per launch, mean over its 24 launches per step (measured with
     # the 4 x 8 band of 256x160 tiles per XCD and 3 LDS stages: profiles/bench_py_kernel_trace.md, section 3)
-    "pipe16_256x160": {"kernel": "gemm_pipe16q_kernel<Pipe16QCfg<256,160,4,2,KIND,false,3>>", "traffic": 0.558e9},
-    # 623 058 KiB x 2.000 fetched + 424 056 KiB written per launch, mean over its 4 launches per step
-    "pipe_256x256": {"kernel": "gemm_pipe2_kernel<Pipe2Cfg<256,256,2,4,KIND,SWAP>>", "traffic": 1.710e9},
+    "pipe16_256x160": {"kernel": "gemm_pipe16q_kernel<Pipe16QCfg<256,160,4,2,KIND,false,3,false>>", "traffic": 0.557e9},
+    # 614 663 KiB x 2.000 fetched + 424 056 KiB written per launch, mean over its 4 launches per step
+    "pipe_256x256": {"kernel": "gemm_pipe2_kernel<Pipe2Cfg<256,256,2,4,KIND,SWAP>>", "traffic": 1.693e9},
 }
 SHAPES = [(5120, 5120), (20480, 5120), (5120, 20480)]   # (N, K): qkv/out_proj, fc1, fc2
 MS = [1, 16, 128, 512, 2048, 8192]
