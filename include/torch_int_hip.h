@@ -44,7 +44,10 @@ int ti_version(void);
 const char* ti_last_error(void);
 
 /* Verifies that a HIP device is present and is gfx950; returns TI_OK or
- * TI_ERR_NO_DEVICE.  Optional: every entry point works without it. */
+ * TI_ERR_NO_DEVICE.  Optional: every entry point works without it.  It also does, for the current device, the two
+ * one-time steps that the first calls would otherwise do: it resolves the address of the built-in scratch buffer
+ * of ti_linear_a8_w8_b8_o8_noalloc, and it runs the placement probe of the one-launch split-K (ti_fused_splitk;
+ * one small kernel on the null stream, 1 KB of mapped host memory, one synchronisation). */
 int ti_init(void);
 
 /* Bytes of scratch the linear entry points can use for (M,N,K) to split the K
@@ -121,7 +124,8 @@ int ti_linear_a8_w8_b8_o8(const int8_t* x, const int8_t* w, const int8_t* bias, 
  * Every call on a GPU shares that GPU's buffer: calls that may overlap in time on one GPU (different
  * streams, different threads) race and must be serialised by the caller.  The buffer needs no clearing
  * between calls (every partial product is written before it is read).  ti_init() resolves the buffer's address
- * for the current device; without it the first call on a device does. */
+ * for the current device; without it the first call on a device does.  The one-launch split-K is used only on a
+ * device where its probe has already run (ti_init() or an earlier workspace call), since the probe allocates. */
 #define TI_NOALLOC_SCRATCH_BYTES (40 * 1024 * 1024)
 int ti_linear_a8_w8_b8_o8_noalloc(const int8_t* x, const int8_t* w, const int8_t* bias, int8_t* out,
                                   int64_t M, int64_t N, int64_t K, float alpha, float beta, void* stream);
