@@ -540,6 +540,39 @@ def test_one_launch_split_k_is_exact_for_every_output_kind():
         lib.ti_fused_splitk(1)
 
 
+def test_one_launch_split_k_in_a_graph():
+    # a split-K linear captured into a HIP graph (after a warm-up on the capture stream: the first use on a device
+    # probes and is not capturable) and replayed with eager split-K launches between the replays
+    import ctypes
+    import torch_int._CUDA as C
+    lib = C._lib
+    lib.ti_last_kernel.restype = ctypes.c_char_p
+    g = torch.Generator().manual_seed(99)
+    M, N, K = 256, 2880, 3584
+    w, b = _s8(g, N, K).to(DEV), _s8(g, N).to(DEV)
+    xs = [_s8(g, M, K) for _ in range(3)]
+    refs = [orc.linear_a8_w8_b8_o8(x, w.cpu(), b.cpu(), 0.0011, 0.02) for x in xs]
+    static_x = xs[0].to(DEV)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            C.linear_a8_w8_b8_o8(static_x, w, b, 0.0011, 0.02)
+    side.synchronize()
+    assert lib.ti_last_kernel().decode() == "fusedk_128x80", lib.ti_last_kernel()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        static_out = C.linear_a8_w8_b8_o8(static_x, w, b, 0.0011, 0.02)
+    for i in (1, 2, 0, 1):
+        _say("one-launch split-K graph replay", i)
+        eager = C.linear_a8_w8_b8_o8(xs[i].to(DEV), w, b, 0.0011, 0.02)   # eager launch on the current stream
+        torch.cuda.synchronize()
+        static_x.copy_(xs[i])
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(static_out.cpu(), refs[i]) and torch.equal(eager.cpu(), refs[i]), i
+
+
 def test_linear_accumulate_into_output(two_launch_split_k):
     # inout += alpha*acc + bias in the GEMM epilogue, through every kernel family the fp32 linear can take
     import ctypes
