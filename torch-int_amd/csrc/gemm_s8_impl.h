@@ -2270,7 +2270,10 @@ int launch_kind(const GemmParams& p, void* workspace, long long workspace_bytes,
                       : tile == SPLIT_128x288 ? "splitk_128x288"
                       : tile == SPLIT_128x80  ? "splitk_128x80"
                                               : "splitk_256x288";
-      if constexpr (KIND != EPI_S32_RAW) {
+      // not for the accumulating epilogue: its reads of the old outputs, done by one workgroup per tile instead of
+      // by the whole chip in the reduction kernel, cost more than the launch saved (512x9216x36864: 288 against
+      // 178 us, 256x5120x5120: 29 against 22 us)
+      if constexpr (KIND != EPI_S32_RAW && KIND != EPI_F32_BIAS_ACC) {
         // one launch when the tile is one of the 16x16-block kernel's and covers M in whole tiles
         const int bm = tile == SPLIT_256x160 || tile == SPLIT_256x288 ? 256 : 128;
         const int bn = tile == SPLIT_128x80 ? 80 : tile == SPLIT_256x160 || tile == SPLIT_128x160 ? 160 : 288;
@@ -2279,7 +2282,8 @@ int launch_kind(const GemmParams& p, void* workspace, long long workspace_bytes,
         // up to four slices: the wave that arrives last reads the others' accumulators one slice after the other,
         // and beyond four that tail costs more than the reduction launch it saves (measured: 2 slices -3 to -12 %,
         // 4 slices -3 to -8 %, 7 and 8 slices +3 to +6 %)
-        if (tall && splits <= 4 && p.M % bm == 0 && p.N % bn == 0) {
+        // (256x288 tiles, which spill registers, with two slices only: 512x9216x36864 in four slices 181 against 179 us)
+        if (tall && splits <= (tile == SPLIT_256x288 ? 2 : 4) && p.M % bm == 0 && p.N % bn == 0) {
           const long long tiles = (long long)(p.M / bm) * (p.N / bn);
           GemmParams f = p;
           f.K = p.K / splits;
