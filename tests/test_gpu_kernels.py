@@ -543,6 +543,36 @@ def test_one_launch_split_k_is_exact_for_every_output_kind():
         lib.ti_fused_splitk(1)
 
 
+def test_one_launch_split_k_on_concurrent_streams():
+    # three streams issue split-K linears of different shapes without waiting for one another: each stream has its own
+    # workspace and its own arrival counters, so every output must equal the two-launch result
+    import ctypes
+    import torch_int._CUDA as C
+    lib = C._lib
+    lib.ti_last_kernel.restype = ctypes.c_char_p
+    g = torch.Generator().manual_seed(101)
+    cases = []
+    for (M, N, K) in [(256, 2880, 3584), (256, 640, 2048), (128, 4608, 2048), (256, 3200, 7168)]:
+        x, w, b = _s8(g, M, K).to(DEV), _s8(g, N, K).to(DEV), _s8(g, N).to(DEV)
+        before = lib.ti_fused_splitk(0)
+        try:
+            ref = C.linear_a8_w8_b8_o8(x, w, b, 0.001, 0.01)
+        finally:
+            lib.ti_fused_splitk(before)
+        cases.append((x, w, b, ref))
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream() for _ in range(3)]
+    outs = []
+    for it in range(24):
+        for si, st in enumerate(streams):
+            x, w, b, ref = cases[(it + 2 * si) % len(cases)]
+            with torch.cuda.stream(st):
+                outs.append((C.linear_a8_w8_b8_o8(x, w, b, 0.001, 0.01), ref, lib.ti_last_kernel().decode()))
+    torch.cuda.synchronize()
+    assert all(k.startswith("fusedk_") for _, _, k in outs), sorted(set(k for _, _, k in outs))
+    assert all(torch.equal(o, r) for o, r, _ in outs)
+
+
 def test_one_launch_split_k_in_a_graph():
     # a split-K linear captured into a HIP graph (after a warm-up on the capture stream: the first use on a device
     # probes and is not capturable) and replayed with eager split-K launches between the replays
