@@ -124,7 +124,7 @@ def test_every_gemm_kernel_family_is_reached_and_exact(two_launch_split_k):
               ((2000, 9216, 192), "pipe16_256x288"), ((2000, 9216, 384), "pipe16_256x288"),
               ((4096, 2816, 192), "pipe_256x256"),
               ((4096, 2816, 128), "pipe_256x256"), ((1024, 2048, 64), "pipe_128x128"),
-              ((1024, 5120, 5120), "pipe16_128x80"), ((256, 1600, 2048), "pipe16_128x80"),
+              ((512, 5120, 5120), "pipe16_128x80"), ((384, 2560, 1024), "pipe16_128x80"), ((1024, 5120, 5120), "splitk_256x160"),
               ((256, 3200, 11648), "splitk_256x160"), ((1024, 9216, 9216), "splitk_256x288"),
               ((384, 2880, 4608), "splitk_128x80"), ((128, 640, 4096), "splitk_128x80"),
               ((256, 1600, 11648), "splitk_128x160"), ((1024, 4608, 3584), "splitk_128x288"),
@@ -615,7 +615,7 @@ def test_linear_accumulate_into_output(two_launch_split_k):
     seen = set()
     for (M, N, K) in [(2048, 5120, 256), (2048, 5120, 64), (2000, 9216, 192), (2000, 9216, 128), (4096, 2816, 128),
                       (4096, 2816, 1024), (1024, 2048, 64), (1024, 5120, 5120), (1024, 4608, 3584), (256, 3072, 7744),
-                      (1024, 9216, 9216), (384, 2880, 4608), (4, 4608, 16384), (256, 3200, 11648), (256, 1600, 11648),
+                      (1024, 9216, 9216), (384, 2880, 4608), (4, 4608, 16384), (256, 3200, 11648), (256, 1600, 11648), (384, 2560, 1024),
                       (128, 640, 4096), (128, 768, 4096), (16, 5120, 3072), (3, 100, 272), (300, 200, 48), (2100, 5000, 272),
                       (70, 50, 37), (4, 64, 0)]:
         _say(f"linear += M={M} N={N} K={K}")
@@ -688,7 +688,7 @@ def test_head_major_projection_through_every_kernel_family(two_launch_split_k):
     for (B, T, H, d, K) in [(4, 512, 40, 128, 256), (4, 512, 40, 128, 192), (2, 1000, 72, 128, 192), (2, 1000, 72, 128, 256),
                             (8, 512, 22, 128, 128), (8, 512, 22, 128, 192), (2, 512, 16, 128, 64),
                             (2, 512, 40, 128, 5120), (2, 512, 36, 128, 3584), (2, 512, 72, 128, 9216), (1, 384, 90, 32, 4608),
-                            (1, 256, 24, 128, 7744), (2, 64, 5, 128, 4096), (1, 256, 25, 128, 11648), (1, 256, 25, 64, 11648), (1, 128, 6, 128, 4096), (1, 16, 40, 128, 3072), (1, 3, 5, 32, 272),
+                            (1, 256, 24, 128, 7744), (2, 64, 5, 128, 4096), (1, 256, 25, 128, 11648), (1, 256, 25, 64, 11648), (1, 384, 20, 128, 1024), (1, 128, 6, 128, 4096), (1, 16, 40, 128, 3072), (1, 3, 5, 32, 272),
                             (3, 100, 5, 48, 48), (3, 700, 39, 128, 272), (2, 35, 3, 16, 37)]:
         M, N = B * T, H * d
         _say(f"head-major linear bsz={B} seq={T} heads={H} d={d} K={K}")

@@ -2149,11 +2149,17 @@ static int choose_splits(long long M, long long N, long long K, int* tile_kind =
       double rate = resident * ahead * step_bytes / 2.0;  // bytes per us
       // 5 TB/s at most; 3.5 TB/s for the 64-byte steps of the 128x128 tiles, which ask for every line twice
       // (128x9216x36864: 110 us against 83 us with 128x288 tiles)
-      const double cap = kind == SPLIT_128 ? 3.5e6 : 5.0e6;
+      // (128x80 tiles ask for 80 scattered lines per step: 3.8 TB/s, 2.4 TB/s when two workgroups share a CU:
+      // 128x20480x5120 30 us, 256x20480x5120 48 us)
+      const double cap = kind == SPLIT_128 ? 3.5e6 : small ? (wgs <= cus ? 3.8e6 : 2.4e6) : 5.0e6;
       if (rate > cap) rate = cap;
       const double t_stream = (double)N * (double)K / rate + (small ? 4.0 : 8.0);
       if (t < t_stream) t = t_stream;
-      if (s > 1) t += (double)(2 * s + 1) * M * N * 4.0 / 5.5e6 + 3.0;  // partials out and back in, at 5.5 TB/s, in us
+      // the slices' partial tiles: written once and read once (they mostly stay in the last-level cache) plus the
+      // second launch; in the one-launch form they stay in the XCD's L2 and the reading is the last workgroup's tail
+      const bool one_launch = kind >= SPLIT_256x160 && M % bm == 0 && s <= (kind == SPLIT_256x288 ? 2 : 4);
+      if (s > 1 && one_launch) t += (double)(2 * s - 1) * M * N * 4.0 / 8.0e6 + 1.0;
+      else if (s > 1) t += (double)(2 * s + 1) * M * N * 4.0 / 5.5e6 + 3.0;  // at 5.5 TB/s, in us
       if (t < best_t * 0.97) {  // prefer fewer slices and the smaller tile unless the gain is clear
         best_t = t;
         best = s;
