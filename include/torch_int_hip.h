@@ -69,7 +69,9 @@ const char* ti_last_kernel(void);
  * enable = 1 / 0 turns the one-launch form on / off for the process, -1 leaves it; returns the setting before
  * the call.  Default on, or off with the environment variable TORCH_INT_FUSED_SPLITK=0.  The form also stays off
  * on a device whose workgroup placement is not "ids congruent mod 8 share an XCD" (probed at the first use),
- * for more than 8 streams per device, and while a stream is being captured before the first use on its device. */
+ * for more than 8 streams per device, and while a stream is being captured before the first use on its device.
+ * Each stream has arrival counters of its own; a launch recorded into a HIP graph keeps those of the stream it
+ * was recorded on, so that stream must not run other split-K linears while the graph replays on another one. */
 int ti_fused_splitk(int enable);
 
 /* Diagnostic (no counterpart in the reference; computes nothing): one launch that issues the instruction mix of
