@@ -324,6 +324,22 @@ def test_bmm_full_size_properties():
     # three full batches against the oracle
     ref = orc.bmm_s8t_s8n_s32t(q[157:].cpu(), k[157:].cpu())
     assert torch.equal(s32[157:].cpu(), ref)
+    # P.V at the same size (probabilities [160, 512, 512] x V^T [160, 128, 512]): four tiles per head and more tiles
+    # than resident workgroups, so the tiles of a head are dealt to one XCD; every head against an fp64 product on
+    # the device (exact: the sums stay far below 2^53), four heads against the oracle
+    import ctypes
+    C._lib.ti_last_kernel.restype = ctypes.c_char_p
+    _say("P.V full size")
+    prob = torch.randint(0, 128, (BH, S, S), dtype=torch.int8, generator=g).to(DEV)
+    vt = _s8(g, BH, d, S).to(DEV)
+    pv = C.bmm_s8t_s8n_s8t(prob, vt, 0.0041)
+    assert C._lib.ti_last_kernel().decode() == "pipe_128x128"
+    exact = torch.einsum("bmk,bnk->bmn", prob.double(), vt.double())
+    want = (exact.float() * 0.0041).clamp(-128, 127).round().to(torch.int8)
+    assert torch.equal(pv, want)
+    heads = [0, 53, 107, 159]
+    assert torch.equal(pv[heads].cpu(), orc.bmm_s8t_s8n_s8t(prob[heads].cpu(), vt[heads].cpu(), 0.0041))
+    assert torch.equal(C.bmm_s8t_s8n_s32t(prob, vt), exact.to(torch.int32))
 
 
 # ------------------------------------------------------------------ dq_add_layernorm_q

@@ -481,10 +481,24 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MIN_WAVES) void gemm_pipe_kernel(Gemm
 
   // ---- copy stream: copy j of this wave fills stage bytes [(wave*COPIES + j) * 1024, +1024)
   const TI_GLOBAL_AS int8_t* src[COPIES];
+  // item -> (batch, tile of the batch).  With p.group_batches (few tiles per batch, batches a multiple of 8) all
+  // tiles of a batch go to workgroups of one XCD (ids congruent mod 8), next to one another, so that the batch's
+  // B operand (V^T of a head in P.V) is fetched into one L2 instead of into as many as the batch has tiles.
+  auto decode_item = [&](int item, int& b, int& t) {
+    if (p.group_batches) {
+      const int l = item >> 3, q = l / tiles;
+      b = q * 8 + (item & 7);
+      t = l - q * tiles;
+    } else {
+      b = item / tiles;
+      t = item - b * tiles;
+    }
+  };
   auto set_copy_item = [&](int item) {
-    const int b = item / tiles;
+    int b, t;
+    decode_item(item, b, t);
     int tile_m, tile_n;
-    tile_of_workgroup(item - b * tiles, tiles_m, tiles_n, tile_m, tile_n, p.band);
+    tile_of_workgroup(t, tiles_m, tiles_n, tile_m, tile_n, p.band);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int8_t* A = p.A + (long long)b * p.strideA;
     const int8_t* B = p.B + (long long)b * p.strideB;
@@ -602,9 +616,10 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MIN_WAVES) void gemm_pipe_kernel(Gemm
     if (!LAST) interleave();
   };
   auto finish_item = [&]() {
-    const int b = item / tiles;
+    int b, t;
+    decode_item(item, b, t);
     int tile_m, tile_n;
-    tile_of_workgroup(item - b * tiles, tiles_m, tiles_n, tile_m, tile_n, p.band);
+    tile_of_workgroup(t, tiles_m, tiles_n, tile_m, tile_n, p.band);
     // opaque copy of the lane id: keeps the epilogue's address arithmetic inside the loop
     // (hoisted, it would occupy registers during the whole mainloop)
     int lane_here = lane;
@@ -2005,6 +2020,10 @@ static int launch_persistent(Kern kern, const GemmParams& p_in, hipStream_t stre
   // one resident workgroup per LDS-sized slot; a multiple of 8 keeps the XCD mapping of tile ids
   const long long slots = (long long)num_cus() * ((160 * 1024) / Cfg::LDS_BYTES);
   const int grid = (int)(items < slots ? items : slots);
+  // gemm_pipe_kernel only (the others ignore it): the tiles of a batch on one XCD when a batch has four to eight
+  // of them and there are more tiles than resident workgroups (P.V of 160 heads x 512 x 512: 19.5 -> 17.7 us; with one
+  // or two tiles per batch, or all tiles resident at once, the plain order is 4-7 % faster)
+  p.group_batches = p.batch % 8 == 0 && tiles_m * tiles_n >= 4 && tiles_m * tiles_n <= 8 && items >= slots && grid % 8 == 0;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, p, tiles_m, tiles_n, (int)items, extra...);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "gemm launch: %s", hipGetErrorString(e));

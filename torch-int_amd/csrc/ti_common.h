@@ -179,6 +179,8 @@ struct GemmParams {
   int out_T = 0, out_d = 0;
   // Tile rows an XCD's run of tiles walks down before it moves to the next tile column (see tile_of_workgroup).
   int band = 8;
+  // gemm_pipe_kernel: all tiles of a batch on one XCD (see decode_item there)
+  int group_batches = 0;
   // Split-K inside one launch (the FUSED form of the 16x16-block kernel): K is the length of one slice, strideA and
   // strideB step from slice to slice; `parts` holds splits x tiles parked accumulator tiles, `arrivals` one zeroed
   // counter per (tile, wave), `xcc_seen` one zeroed word per tile in which the workgroups of the tile mark the XCC
