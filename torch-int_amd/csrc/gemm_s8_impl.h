@@ -1319,6 +1319,10 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe16q_kernel(GemmParams p, 
       const int t = item / p.splits;
       b = item - t * p.splits;
       tile_id = t * 8 + xcd;
+    } else if (p.group_batches) {  // all tiles of a batch on one XCD, next to one another (see gemm_pipe_kernel)
+      const int l = item >> 3, q = l / tiles;
+      b = q * 8 + (item & 7);
+      tile_id = l - q * tiles;
     } else {
       b = item / tiles;
       tile_id = item - b * tiles;
@@ -2020,7 +2024,7 @@ static int launch_persistent(Kern kern, const GemmParams& p_in, hipStream_t stre
   // one resident workgroup per LDS-sized slot; a multiple of 8 keeps the XCD mapping of tile ids
   const long long slots = (long long)num_cus() * ((160 * 1024) / Cfg::LDS_BYTES);
   const int grid = (int)(items < slots ? items : slots);
-  // gemm_pipe_kernel only (the others ignore it): the tiles of a batch on one XCD when a batch has four to eight
+  // gemm_pipe_kernel and gemm_pipe16q_kernel (the others ignore it): the tiles of a batch on one XCD when a batch has four to eight
   // of them and there are more tiles than resident workgroups (P.V of 160 heads x 512 x 512: 19.5 -> 17.7 us; with one
   // or two tiles per batch, or all tiles resident at once, the plain order is 4-7 % faster)
   p.group_batches = p.batch % 8 == 0 && tiles_m * tiles_n >= 4 && tiles_m * tiles_n <= 8 && items >= slots && grid % 8 == 0;
