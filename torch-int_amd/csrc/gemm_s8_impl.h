@@ -709,10 +709,22 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe2_kernel(GemmParams p, in
   // ---- copy stream: copy j of this wave fills stage bytes [(wave*COPIES + j) * 1024, +1024)
   const bool copies_a = wave * COPIES * 8 < BM;  // this wave fills A panel rows (else B panel rows)
   const TI_GLOBAL_AS int8_t* src[COPIES];
+  // item -> (batch, tile of the batch); p.group_batches: all tiles of a batch on one XCD (see gemm_pipe_kernel)
+  auto decode_item = [&](int item, int& b, int& t) {
+    if (p.group_batches) {
+      const int l = item >> 3, q = l / tiles;
+      b = q * 8 + (item & 7);
+      t = l - q * tiles;
+    } else {
+      b = item / tiles;
+      t = item - b * tiles;
+    }
+  };
   auto set_copy_item = [&](int item) {
-    const int b = item / tiles;
+    int b, t;
+    decode_item(item, b, t);
     int tile_m, tile_n;
-    tile_of_workgroup(item - b * tiles, tiles_m, tiles_n, tile_m, tile_n, p.band);
+    tile_of_workgroup(t, tiles_m, tiles_n, tile_m, tile_n, p.band);
     const int first_row = copies_a ? tile_m * BM : tile_n * BN;  // of the panel in its operand
     const int last_row = (copies_a ? M : N) - 1;                 // edge rows re-read the last row; never stored
     const size_t ld = copies_a ? p.lda : p.ldb;
@@ -828,9 +840,10 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe2_kernel(GemmParams p, in
     if (!LAST) interleave();
   };
   auto finish_item = [&]() {
-    const int b = item / tiles;
+    int b, t;
+    decode_item(item, b, t);
     int tile_m, tile_n;
-    tile_of_workgroup(item - b * tiles, tiles_m, tiles_n, tile_m, tile_n, p.band);
+    tile_of_workgroup(t, tiles_m, tiles_n, tile_m, tile_n, p.band);
     // opaque copy of the lane id: keeps the epilogue's address arithmetic inside the loop
     int lane_here = lane;
     asm volatile("" : "+v"(lane_here));
