@@ -33,7 +33,11 @@ constexpr int AF_MAX_S = 512;
 // permutation of the 64 keys inside the slice, and the V fragments are gathered with the same permutation (four
 // 4-byte reads), so the integer sum over the slice is the same.  The context rows are written already merged:
 // ctx is [batch, T, heads * 128].
-template <int NB, bool PV>
+// SPEC: 0 = any S <= 16 * NB and a mask pointer that may be null; 1 / 2 = S == 16 * NB exactly, with / without a mask.
+// In the exact forms every "block j exists" and "there is a mask" test folds away at compile time, which leaves
+// straight-line code: the fragment reads, the matrix instructions and the mask loads of different blocks overlap
+// instead of waiting for one another block by block.
+template <int NB, bool PV, int SPEC = 0>
 __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t* __restrict__ q,
                                                                    const int8_t* __restrict__ k,
                                                                    const float* __restrict__ mask,
@@ -50,7 +54,9 @@ __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t*
   const int n_bh = gridDim.x / row_blocks;
   const long long bh = blockIdx.x % n_bh;
   const int t0 = (row_blocks - 1 - (int)(blockIdx.x / n_bh)) * AF_ROWS;
-  const int nb = S >> 4;
+  if constexpr (SPEC != 0) S = 16 * NB;
+  const int nb = SPEC != 0 ? NB : S >> 4;
+  const bool has_mask = SPEC == 1 ? true : SPEC == 2 ? false : mask != nullptr;
 
   // ---- copies: slab i = 8 rows of [Q tile (64 rows) | K panel (S rows)], 1 KiB per wave instruction
   const int8_t* qb = q + bh * stride_q;
@@ -113,7 +119,7 @@ __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t*
   // while the previous eight are consumed.
   const int t = t0 + wave * 16 + r;
   const int tc = t < T ? t : T - 1;
-  const float* mrow = mask != nullptr ? mask + (((bh / heads) * T + tc) * (long long)S) : nullptr;
+  const float* mrow = has_mask ? mask + (((bh / heads) * T + tc) * (long long)S) : nullptr;
   const float lowest = -3.402823466e+38f;
   float m = lowest;
   constexpr int MG = NB < 8 ? NB : 8;  // blocks per mask group
@@ -123,7 +129,7 @@ __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t*
     for (int u = 0; u < MG; ++u) {
       const int j = j0 + u;
       dst[u] = v4f{0.f, 0.f, 0.f, 0.f};
-      if (mrow != nullptr && j < nb) dst[u] = *reinterpret_cast<const v4f*>(mrow + 16 * j + 4 * g);
+      if (has_mask && j < nb) dst[u] = *reinterpret_cast<const v4f*>(mrow + 16 * j + 4 * g);
     }
   };
   fetch_mask(0, mk[0]);
@@ -138,7 +144,7 @@ __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t*
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
           float x = Epi<EPI_F32_SCALE>::apply(acc[j][v], 0.0f, alpha);
-          if (mrow != nullptr) x = x + mk[cur][u][v];
+          if (has_mask) x = x + mk[cur][u][v];
           x = __builtin_fmaxf(x, lowest);  // = x > lowest ? x : lowest, NaN included
           m = __builtin_fmaxf(m, x);
           acc[j][v] = __float_as_int(x);
@@ -271,11 +277,11 @@ bool attn_qk_softmax_q_supported(long long T, long long S, long long D) {
   return single_sweep_ok(T, S, D, false) || attn_long_supported(T, S, D);
 }
 
-template <int NB, bool PV>
+template <int NB, bool PV, int SPEC>
 static int launch_af(dim3 grid, size_t lds, hipStream_t stream, const int8_t* q, const int8_t* k, const float* mask,
                      int8_t* probs, int T, int S, long long stride_q, long long stride_k, int heads, int row_blocks,
                      float alpha, const int8_t* vt, int8_t* ctx, float alpha_pv) {
-  auto kern = attn_qk_softmax_q_kernel<NB, PV>;
+  auto kern = attn_qk_softmax_q_kernel<NB, PV, SPEC>;
   static unsigned long long lds_ok = 0;  // bit per device: the large dynamic LDS size has been allowed
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return fail(TI_ERR_LAUNCH, "attn_qk_softmax_q: no current device");
@@ -304,18 +310,25 @@ int launch_attn_qk_softmax_q(const int8_t* q, const int8_t* k, const float* mask
   const dim3 grid((unsigned)(BH * row_blocks));
   const size_t lds = (size_t)(AF_ROWS + S) * AF_D;
   int rc;
-#define TI_AF(NB, PV)                                                                                              \
-  rc = launch_af<NB, PV>(grid, lds, stream, q, k, mask, probs, (int)T, (int)S, stride_q, stride_k, (int)heads,    \
-                         (int)row_blocks, alpha, vt, ctx, alpha_pv)
+#define TI_AF(NB, PV, SPEC)                                                                                             \
+  rc = launch_af<NB, PV, SPEC>(grid, lds, stream, q, k, mask, probs, (int)T, (int)S, stride_q, stride_k, (int)heads,   \
+                               (int)row_blocks, alpha, vt, ctx, alpha_pv)
+#define TI_AF_NB(NB, PV)                                 \
+  do {                                                   \
+    if (S != 16 * NB) TI_AF(NB, PV, 0);                  \
+    else if (mask != nullptr) TI_AF(NB, PV, 1);          \
+    else TI_AF(NB, PV, 2);                               \
+  } while (0)
   if (vt == nullptr) {
-    if (S <= 128) TI_AF(8, false);
-    else if (S <= 256) TI_AF(16, false);
-    else TI_AF(32, false);
+    if (S <= 128) TI_AF_NB(8, false);
+    else if (S <= 256) TI_AF_NB(16, false);
+    else TI_AF_NB(32, false);
   } else {
-    if (S <= 128) TI_AF(8, true);
-    else if (S <= 256) TI_AF(16, true);
-    else TI_AF(32, true);
+    if (S <= 128) TI_AF_NB(8, true);
+    else if (S <= 256) TI_AF_NB(16, true);
+    else TI_AF_NB(32, true);
   }
+#undef TI_AF_NB
 #undef TI_AF
   if (rc) return rc;
   hipError_t e = hipGetLastError();

@@ -35,7 +35,7 @@ __device__ __forceinline__ int al_swz(int row, int c) {
   return D == 128 ? (c ^ ((row >> 1) & 7)) : (c ^ ((row >> 2) & 3));
 }
 
-template <int D, bool PV>
+template <int D, bool PV, bool MASKED>
 __global__ __launch_bounds__(256, 2) void attn_long_kernel(const int8_t* __restrict__ q, const int8_t* __restrict__ k,
                                                            const float* __restrict__ mask, int8_t* __restrict__ probs,
                                                            int T, int S, long long stride_q, long long stride_k,
@@ -95,7 +95,7 @@ __global__ __launch_bounds__(256, 2) void attn_long_kernel(const int8_t* __restr
 
   const int t = t0 + wave * 16 + r;
   const int tc = t < T ? t : T - 1;
-  const float* mrow = mask != nullptr ? mask + (((bh / heads) * T + tc) * (long long)S) : nullptr;
+  const float* mrow = MASKED ? mask + (((bh / heads) * T + tc) * (long long)S) : nullptr;
   const float lowest = -3.402823466e+38f;
   const char* qs = qs_base + (wave * 16 + r) * D;
   const char* ks = ks_base + r * D;
@@ -103,7 +103,8 @@ __global__ __launch_bounds__(256, 2) void attn_long_kernel(const int8_t* __restr
   // x of one tile: acc[j][v] <- bits of max(alpha * (q . k) + mask, lowest) for block j, keys 16 j + 4 g + v
   v4i acc[16];
   v4i qf[KS];
-  auto tile_scores = [&](int tile, int nb) {
+  auto tile_scores = [&](int tile, auto nb_) __attribute__((always_inline)) {
+    const int nb = nb_;
     const int k0 = tile * AL_TILE;
 #pragma unroll
     for (int j = 0; j < 16; ++j) {
@@ -122,7 +123,7 @@ __global__ __launch_bounds__(256, 2) void attn_long_kernel(const int8_t* __restr
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
         dst[u] = v4f{0.f, 0.f, 0.f, 0.f};
-        if (mrow != nullptr && j0 + u < nb) dst[u] = *reinterpret_cast<const v4f*>(mrow + k0 + 16 * (j0 + u) + 4 * g);
+        if (MASKED && j0 + u < nb) dst[u] = *reinterpret_cast<const v4f*>(mrow + k0 + 16 * (j0 + u) + 4 * g);
       }
     };
     fetch_mask(0, mk[0]);
@@ -137,7 +138,7 @@ __global__ __launch_bounds__(256, 2) void attn_long_kernel(const int8_t* __restr
 #pragma unroll
           for (int v = 0; v < 4; ++v) {
             float x = Epi<EPI_F32_SCALE>::apply(acc[j][v], 0.0f, alpha);
-            if (mrow != nullptr) x = x + mk[cur][u][v];
+            if (MASKED) x = x + mk[cur][u][v];
             x = __builtin_fmaxf(x, lowest);  // NaN included
             acc[j][v] = __float_as_int(x);
           }
@@ -149,6 +150,17 @@ __global__ __launch_bounds__(256, 2) void attn_long_kernel(const int8_t* __restr
     const int left = S - tile * AL_TILE;
     return (left < AL_TILE ? left : AL_TILE) >> 4;
   };
+  // The per-tile bodies below are generic lambdas run as body(nb) for the tile's number of key blocks, with the 16
+  // of a full tile as a compile-time constant: every "block j exists" test then folds away and the fragment reads,
+  // matrix instructions and mask loads of different blocks overlap instead of waiting for one another block by
+  // block.  (Inlined by force: called from two places each, the lambdas would otherwise stay functions and push
+  // the register arrays they capture by reference into scratch memory.)
+#define TI_FOR_BLOCKS_OF(tile, body)                            \
+  do {                                                          \
+    const int nb_rt = blocks_of(tile);                          \
+    if (nb_rt == 16) body(std::integral_constant<int, 16>{});   \
+    else body(nb_rt);                                           \
+  } while (0)
 
   // ---- sweep 1: row maximum and the largest x of every tile
   float m = lowest;
@@ -164,14 +176,17 @@ __global__ __launch_bounds__(256, 2) void attn_long_kernel(const int8_t* __restr
 #pragma unroll
       for (int s = 0; s < KS; ++s) qf[s] = *reinterpret_cast<const v4i*>(qs + (al_swz<D>(wave * 16 + r, 4 * s + g) << 4));
     }
-    const int nb = blocks_of(tile);
-    tile_scores(tile, nb);
     float top = lowest;
+    auto body0 = [&](auto nb_) __attribute__((always_inline)) {
+      const int nb = nb_;
+      tile_scores(tile, nb_);
 #pragma unroll
-    for (int j = 0; j < 16; ++j)
-      if (j < nb)
-        top = __builtin_fmaxf(top, __builtin_fmaxf(__builtin_fmaxf(__int_as_float(acc[j][0]), __int_as_float(acc[j][1])),
-                                                   __builtin_fmaxf(__int_as_float(acc[j][2]), __int_as_float(acc[j][3]))));
+      for (int j = 0; j < 16; ++j)
+        if (j < nb)
+          top = __builtin_fmaxf(top, __builtin_fmaxf(__builtin_fmaxf(__int_as_float(acc[j][0]), __int_as_float(acc[j][1])),
+                                                     __builtin_fmaxf(__int_as_float(acc[j][2]), __int_as_float(acc[j][3]))));
+    };
+    TI_FOR_BLOCKS_OF(tile, body0);
     m = __builtin_fmaxf(m, top);
 #pragma unroll
     for (int i = 0; i < AL_MAX_TILES; ++i)
@@ -203,21 +218,24 @@ __global__ __launch_bounds__(256, 2) void attn_long_kernel(const int8_t* __restr
     load_k_tile(tile);
     asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
     if (!(live_w >> tile & 1)) continue;  // uniform over the wave: every e is 0, p + 0 = p
-    const int nb = blocks_of(tile);
-    tile_scores(tile, nb);
+    auto body1 = [&](auto nb_) __attribute__((always_inline)) {
+      const int nb = nb_;
+      tile_scores(tile, nb_);
 #pragma unroll
-    for (int j = 0; j < 16; ++j) {
-      if (j < nb) {
-        const float top = __builtin_fmaxf(__builtin_fmaxf(__int_as_float(acc[j][0]), __int_as_float(acc[j][1])),
-                                          __builtin_fmaxf(__int_as_float(acc[j][2]), __int_as_float(acc[j][3])));
-        if (__builtin_amdgcn_ballot_w64(top - m > -87.0f) != 0) {
-          float p = part[j];
+      for (int j = 0; j < 16; ++j) {
+        if (j < nb) {
+          const float top = __builtin_fmaxf(__builtin_fmaxf(__int_as_float(acc[j][0]), __int_as_float(acc[j][1])),
+                                            __builtin_fmaxf(__int_as_float(acc[j][2]), __int_as_float(acc[j][3])));
+          if (__builtin_amdgcn_ballot_w64(top - m > -87.0f) != 0) {
+            float p = part[j];
 #pragma unroll
-          for (int v = 0; v < 4; ++v) p = p + exp_nonpos(__int_as_float(acc[j][v]) - m);
-          part[j] = p;
+            for (int v = 0; v < 4; ++v) p = p + exp_nonpos(__int_as_float(acc[j][v]) - m);
+            part[j] = p;
+          }
         }
       }
-    }
+    };
+    TI_FOR_BLOCKS_OF(tile, body1);
   }
 #pragma unroll
   for (int w = 8; w >= 1; w >>= 1)
@@ -237,7 +255,6 @@ __global__ __launch_bounds__(256, 2) void attn_long_kernel(const int8_t* __restr
 #pragma unroll 1
   for (int tile = 0; tile < ntiles; ++tile) {
     const bool tile_live = live_g >> tile & 1;
-    const int nb = blocks_of(tile);
     if (tile_live) {
       __syncthreads();
       load_k_tile(tile);
@@ -246,51 +263,55 @@ __global__ __launch_bounds__(256, 2) void attn_long_kernel(const int8_t* __restr
     }
     const bool wave_live = live_w >> tile & 1;
     if (PV && !wave_live) continue;
-    unsigned pw[16];
+    auto body2 = [&](auto nb_) __attribute__((always_inline)) {
+      const int nb = nb_;
+      unsigned pw[16];
 #pragma unroll
-    for (int j = 0; j < 16; ++j) pw[j] = 0;
-    if (wave_live) {
-      tile_scores(tile, nb);
+      for (int j = 0; j < 16; ++j) pw[j] = 0;
+      if (wave_live) {
+        tile_scores(tile, nb_);
 #pragma unroll
-      for (int j = 0; j < 16; ++j) {
-        if (j < nb) {
-          const float top = __builtin_fmaxf(__builtin_fmaxf(__int_as_float(acc[j][0]), __int_as_float(acc[j][1])),
-                                            __builtin_fmaxf(__int_as_float(acc[j][2]), __int_as_float(acc[j][3])));
-          if (__builtin_amdgcn_ballot_w64(top - m > -87.0f) != 0) {
-            unsigned w = 0;
+        for (int j = 0; j < 16; ++j) {
+          if (j < nb) {
+            const float top = __builtin_fmaxf(__builtin_fmaxf(__int_as_float(acc[j][0]), __int_as_float(acc[j][1])),
+                                              __builtin_fmaxf(__int_as_float(acc[j][2]), __int_as_float(acc[j][3])));
+            if (__builtin_amdgcn_ballot_w64(top - m > -87.0f) != 0) {
+              unsigned w = 0;
 #pragma unroll
-            for (int v = 0; v < 4; ++v) {
-              const float pq = __builtin_rintf(exp_nonpos(__int_as_float(acc[j][v]) - m) * scale);  // in [0, 127]
-              w |= (unsigned)(int)pq << (8 * v);
+              for (int v = 0; v < 4; ++v) {
+                const float pq = __builtin_rintf(exp_nonpos(__int_as_float(acc[j][v]) - m) * scale);  // in [0, 127]
+                w |= (unsigned)(int)pq << (8 * v);
+              }
+              pw[j] = w;
             }
-            pw[j] = w;
           }
         }
       }
-    }
-    if constexpr (PV) {
+      if constexpr (PV) {
 #pragma unroll
-      for (int sl = 0; sl < 4; ++sl) {
-        if (4 * sl < nb) {
-          const v4i pa = {(int)pw[4 * sl], (int)pw[4 * sl + 1], (int)pw[4 * sl + 2], (int)pw[4 * sl + 3]};
+        for (int sl = 0; sl < 4; ++sl) {
+          if (4 * sl < nb) {
+            const v4i pa = {(int)pw[4 * sl], (int)pw[4 * sl + 1], (int)pw[4 * sl + 2], (int)pw[4 * sl + 3]};
 #pragma unroll
-          for (int c = 0; c < CH; ++c) {
-            const char* src = vrow + c * 16 * AL_VPITCH + 64 * sl;
-            const v4i vf = {*reinterpret_cast<const int*>(src), *reinterpret_cast<const int*>(src + 16),
-                            *reinterpret_cast<const int*>(src + 32), *reinterpret_cast<const int*>(src + 48)};
-            o[c] = __builtin_amdgcn_mfma_i32_16x16x64_i8(vf, pa, o[c], 0, 0, 0);
+            for (int c = 0; c < CH; ++c) {
+              const char* src = vrow + c * 16 * AL_VPITCH + 64 * sl;
+              const v4i vf = {*reinterpret_cast<const int*>(src), *reinterpret_cast<const int*>(src + 16),
+                              *reinterpret_cast<const int*>(src + 32), *reinterpret_cast<const int*>(src + 48)};
+              o[c] = __builtin_amdgcn_mfma_i32_16x16x64_i8(vf, pa, o[c], 0, 0, 0);
+            }
           }
         }
-      }
-    } else {
-      // four consecutive keys per lane and block; dead tiles and blocks store their zeros
-      int* dst = reinterpret_cast<int*>(prow + tile * AL_TILE) + g;
-      if (t < T) {
+      } else {
+        // four consecutive keys per lane and block; dead tiles and blocks store their zeros
+        int* dst = reinterpret_cast<int*>(prow + tile * AL_TILE) + g;
+        if (t < T) {
 #pragma unroll
-        for (int j = 0; j < 16; ++j)
-          if (j < nb) dst[4 * j] = (int)pw[j];
+          for (int j = 0; j < 16; ++j)
+            if (j < nb) dst[4 * j] = (int)pw[j];
+        }
       }
-    }
+    };
+    TI_FOR_BLOCKS_OF(tile, body2);
   }
   if constexpr (PV) {
     if (t < T) {
@@ -312,11 +333,11 @@ bool attn_long_supported(long long T, long long S, long long D) {
   return T >= 1 && (D == 64 || D == 128) && S >= 16 && S % 16 == 0 && S <= (long long)AL_TILE * AL_MAX_TILES;
 }
 
-template <int D, bool PV>
+template <int D, bool PV, bool MASKED>
 static int launch_al(dim3 grid, hipStream_t stream, const int8_t* q, const int8_t* k, const float* mask, int8_t* probs,
                      int T, int S, long long stride_q, long long stride_k, int heads, int row_blocks, float alpha,
                      const int8_t* vt, int8_t* ctx, float alpha_pv) {
-  auto kern = attn_long_kernel<D, PV>;
+  auto kern = attn_long_kernel<D, PV, MASKED>;
   constexpr int lds = AL_ROWS * D + AL_TILE * D + (PV ? D * AL_VPITCH : 0) + 16;
   static_assert(2 * lds <= 160 * 1024, "two workgroups per CU");
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
@@ -339,9 +360,12 @@ int launch_attn_long(const int8_t* q, const int8_t* k, const float* mask, int8_t
   if (BH * row_blocks > 0x7fffffffLL || T > 0x7fffffffLL)
     return fail(TI_ERR_INVALID_ARG, "attn_long: too many row blocks (%lld)", BH * row_blocks);
   const dim3 grid((unsigned)(BH * row_blocks));
-#define TI_AL(DD, PV)                                                                                          \
-  return launch_al<DD, PV>(grid, stream, q, k, mask, probs, (int)T, (int)S, stride_q, stride_k, (int)heads,  \
-                           (int)row_blocks, alpha, vt, ctx, alpha_pv)
+#define TI_AL(DD, PV)                                                                                                 \
+  return mask != nullptr                                                                                              \
+             ? launch_al<DD, PV, true>(grid, stream, q, k, mask, probs, (int)T, (int)S, stride_q, stride_k, (int)heads,  \
+                                       (int)row_blocks, alpha, vt, ctx, alpha_pv)                                     \
+             : launch_al<DD, PV, false>(grid, stream, q, k, mask, probs, (int)T, (int)S, stride_q, stride_k, (int)heads, \
+                                        (int)row_blocks, alpha, vt, ctx, alpha_pv)
   if (D == 128) {
     if (vt == nullptr) TI_AL(128, false);
     TI_AL(128, true);
@@ -351,4 +375,5 @@ int launch_attn_long(const int8_t* q, const int8_t* k, const float* mask, int8_t
 #undef TI_AL
 }
 
+#undef TI_FOR_BLOCKS_OF
 }  // namespace ti
