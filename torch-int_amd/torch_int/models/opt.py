@@ -280,7 +280,7 @@ class Int8OPTAttention(nn.Module):
         src_len = key.size(1)
 
         # Beyond 512 keys the fused kernels sweep the keys three times and win through the key tiles a causal mask
-        # kills (160 x 2048 x 2048: 1.18 ms against 1.34 ms for the separate kernels; 1.85 ms without a mask), so
+        # kills (160 x 2048 x 2048: 0.99 ms against 1.34 ms for the separate kernels; without a mask they are slower), so
         # they are taken for a plain prefill (tgt_len == src_len) only.
         long_ok = src_len <= 512 or tgt_len == src_len
         if (self.fused_softmax and long_ok and layer_head_mask is None and not output_attentions and tgt_len > 16
