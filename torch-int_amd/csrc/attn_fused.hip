@@ -76,10 +76,28 @@ __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t*
     __builtin_amdgcn_global_load_lds((const TI_GLOBAL_AS void*)src, (TI_LDS_AS void*)((TI_LDS_AS char*)smem + i * 1024),
                                      16, 0, 0);
   }
+  // ---- mask rows: the values of eight blocks are fetched while the previous eight are consumed, the first
+  // eight together with the operand copies
+  const int r = lane & 15, g = lane >> 4;
+  const int t = t0 + wave * 16 + r;
+  const int tc = t < T ? t : T - 1;
+  const float* mrow = has_mask ? mask + (((bh / heads) * T + tc) * (long long)S) : nullptr;
+  const float lowest = -3.402823466e+38f;
+  float m = lowest;
+  constexpr int MG = NB < 8 ? NB : 8;  // blocks per mask group
+  v4f mk[2][MG];
+  auto fetch_mask = [&](int j0, v4f (&dst)[MG]) {
+#pragma unroll
+    for (int u = 0; u < MG; ++u) {
+      const int j = j0 + u;
+      dst[u] = v4f{0.f, 0.f, 0.f, 0.f};
+      if (has_mask && j < nb) dst[u] = *reinterpret_cast<const v4f*>(mrow + 16 * j + 4 * g);
+    }
+  };
+  fetch_mask(0, mk[0]);
   asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
 
   // ---- scores: acc[j] = q rows (16 of this wave) x key block j
-  const int r = lane & 15, g = lane >> 4;
   const int sw = (r >> 1) & 7;
   const char* qs = smem + (wave * 16 + r) * AF_D;
   const char* ks = smem + AF_ROWS * AF_D + r * AF_D;
@@ -103,36 +121,7 @@ __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t*
   const int pitch = S + 16;
   // V^T panel: 128 rows of pitch bytes, ending where the K panel ended (it starts inside the dead Q tile)
   char* vts = smem + (AF_ROWS + S) * AF_D - AF_D * pitch;
-  if constexpr (PV) {
-    const int8_t* vb = vt + bh * (long long)AF_D * S;
-    const int instrs = (AF_D * pitch) >> 10;  // 1 KiB each
-    for (int i = wave; i < instrs; i += 4) {
-      const int o = i * 1024 + lane * 16;
-      int row = o / pitch, col = o - row * pitch;
-      col = col < S ? col : 0;  // the 16 pad bytes of a row receive a copy of its first chunk; never read
-      __builtin_amdgcn_global_load_lds((const TI_GLOBAL_AS void*)(vb + (long long)row * S + col),
-                                       (TI_LDS_AS void*)((TI_LDS_AS char*)vts + i * 1024), 16, 0, 0);
-    }
-  }
-
-  // ---- x = max(alpha * acc + mask, lowest); row maximum.  The mask values of eight blocks are fetched
-  // while the previous eight are consumed.
-  const int t = t0 + wave * 16 + r;
-  const int tc = t < T ? t : T - 1;
-  const float* mrow = has_mask ? mask + (((bh / heads) * T + tc) * (long long)S) : nullptr;
-  const float lowest = -3.402823466e+38f;
-  float m = lowest;
-  constexpr int MG = NB < 8 ? NB : 8;  // blocks per mask group
-  v4f mk[2][MG];
-  auto fetch_mask = [&](int j0, v4f (&dst)[MG]) {
-#pragma unroll
-    for (int u = 0; u < MG; ++u) {
-      const int j = j0 + u;
-      dst[u] = v4f{0.f, 0.f, 0.f, 0.f};
-      if (has_mask && j < nb) dst[u] = *reinterpret_cast<const v4f*>(mrow + 16 * j + 4 * g);
-    }
-  };
-  fetch_mask(0, mk[0]);
+  // ---- x = max(alpha * acc + mask, lowest); row maximum
 #pragma unroll
   for (int j0 = 0; j0 < NB; j0 += MG) {
     const int cur = (j0 / MG) & 1;
@@ -158,6 +147,22 @@ __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t*
     o = __shfl_xor(m, 32, 64);
     m = m > o ? m : o;
   }
+
+  // V^T goes into the dead K panel now, after the last mask load: loads complete in issue order, so copies issued
+  // before the mask rows would have to land before the first mask value could be used.  They run under the
+  // exponentials and the quantisation and are waited for in front of P.V.
+  if constexpr (PV) {
+    const int8_t* vb = vt + bh * (long long)AF_D * S;
+    const int instrs = (AF_D * pitch) >> 10;  // 1 KiB each
+    for (int i = wave; i < instrs; i += 4) {
+      const int o = i * 1024 + lane * 16;
+      int row = o / pitch, col = o - row * pitch;
+      col = col < S ? col : 0;  // the 16 pad bytes of a row receive a copy of its first chunk; never read
+      __builtin_amdgcn_global_load_lds((const TI_GLOBAL_AS void*)(vb + (long long)row * S + col),
+                                       (TI_LDS_AS void*)((TI_LDS_AS char*)vts + i * 1024), 16, 0, 0);
+    }
+  }
+
 
   // ---- e = exp(x - m); partial sums in the reference order.  exp_nonpos returns exactly 0 below -87, so a
   // block in which no lane of the wave has anything above that (masked-out keys) skips the evaluation.
