@@ -846,7 +846,9 @@ def test_fused_qk_softmax_matches_the_two_kernels_and_the_oracle():
     neg = torch.finfo(torch.float32).min
     # (batch, heads, T, S, mask kind)
     cases = [(4, 40, 512, 512, "causal"), (2, 3, 100, 96, "pad"), (1, 4, 64, 16, None), (2, 2, 70, 272, "causal"),
-             (1, 2, 1, 512, None), (3, 1, 130, 144, "pad"), (1, 2, 300, 304, "causal")]
+             (1, 2, 1, 512, None), (3, 1, 130, 144, "pad"), (1, 2, 300, 304, "causal"),
+             # exactly 128 / 256 / 512 keys, with and without a mask: the kernels compiled for those facts
+             (2, 3, 100, 128, "pad"), (1, 2, 70, 128, None), (2, 2, 33, 256, "causal"), (1, 2, 40, 256, None)]
     for (B, H, T, S, kind) in cases:
         _say(f"qk_softmax B={B} H={H} T={T} S={S} mask={kind}")
         q, k = _s8(g, B * H, T, 128), _s8(g, B * H, S, 128)
@@ -880,7 +882,9 @@ def test_fused_prefill_attention_matches_the_chain():
     g = torch.Generator().manual_seed(97)
     neg = torch.finfo(torch.float32).min
     for (B, H, T, S, kind) in [(4, 40, 512, 512, "causal"), (2, 3, 100, 128, "pad"), (1, 4, 64, 64, None),
-                               (2, 2, 70, 256, "causal"), (1, 2, 300, 320, "causal"), (1, 1, 5, 448, None)]:
+                               (2, 2, 70, 256, "causal"), (1, 2, 300, 320, "causal"), (1, 1, 5, 448, None),
+                               # exactly 128 / 256 / 512 keys without a mask: the kernels compiled for that fact
+                               (1, 2, 80, 128, None), (1, 2, 64, 256, None), (1, 1, 100, 512, None)]:
         _say(f"attn_prefill B={B} H={H} T={T} S={S} mask={kind}")
         q, k, v = _s8(g, B * H, T, 128), _s8(g, B * H, S, 128), _s8(g, B * H, S, 128)
         a_qk, a_pv = _scal(g, 2e-4, 2e-3), _scal(g, 2e-3, 2e-2)
