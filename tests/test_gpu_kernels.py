@@ -458,11 +458,16 @@ def test_int8_layout_kernels():
         assert out.is_contiguous() and torch.equal(out, ref)
         back = X.merge_heads(out.view(B * H, T, d), B, H, T, d)
         assert back.shape == (B, T, H * d) and torch.equal(back, t)
-    for (B, R, C) in [(160, 512, 128), (8, 513, 128), (3, 70, 50), (2, 1, 128), (5, 64, 1), (1, 200, 333)]:
+    # whole 64 x 64 tiles take the 4 x 4-block kernel (the first three and the sliced, 64-byte-offset source)
+    for (B, R, C) in [(160, 512, 128), (3, 64, 64), (2, 192, 320), (8, 513, 128), (3, 70, 50), (2, 1, 128), (5, 64, 1),
+                      (1, 200, 333)]:
         _say(f"transpose_last2 B={B} R={R} C={C}")
         t = _s8(g, B, R, C).to(DEV)
         out = X.transpose_last2(t)
         assert out.is_contiguous() and torch.equal(out, t.transpose(1, 2).contiguous())
+    big = _s8(g, 5, 128, 64).to(DEV)
+    part = big[1:]   # contiguous, starts 8192 bytes into the allocation
+    assert torch.equal(X.transpose_last2(part), part.transpose(1, 2).contiguous())
 
 
 def test_stream_kernel_strip_orders_and_ragged_widths():
