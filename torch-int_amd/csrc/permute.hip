@@ -171,9 +171,52 @@ __global__ __launch_bounds__(256) void transpose_last2_tiles_kernel(const int8_t
     *reinterpret_cast<unsigned*>(dst + base + (long long)(c0 + 4 * b + k) * R + r0 + 4 * a) = o[k];
 }
 
+// The same with 128x128 tiles (R % 128 == 0, C % 128 == 0): whole 128-byte lines are read and written (eight lanes
+// fetch one row of the tile, 32 lanes store 128 contiguous bytes of an output row), four 4x4 blocks per thread.
+__global__ __launch_bounds__(256) void transpose_last2_tiles128_kernel(const int8_t* __restrict__ src,
+                                                                       int8_t* __restrict__ dst, int R, int C) {
+  __shared__ unsigned tile[128][33];
+  const long long base = (long long)blockIdx.z * R * C;
+  const int r0 = blockIdx.y * 128, c0 = blockIdx.x * 128;
+  const int t = threadIdx.x;
+  {
+    const int q = t & 7;
+    v4i v[4];
+#pragma unroll
+    for (int pass = 0; pass < 4; ++pass)
+      v[pass] = *reinterpret_cast<const v4i*>(src + base + (long long)(r0 + (t >> 3) + 32 * pass) * C + c0 + q * 16);
+#pragma unroll
+    for (int pass = 0; pass < 4; ++pass)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) tile[(t >> 3) + 32 * pass][4 * q + j] = (unsigned)v[pass][j];
+  }
+  __syncthreads();
+  const int a = t & 31;
+#pragma unroll
+  for (int pass = 0; pass < 4; ++pass) {
+    const int b = (t >> 5) + 8 * pass;
+    const unsigned w0 = tile[4 * a][b], w1 = tile[4 * a + 1][b], w2 = tile[4 * a + 2][b], w3 = tile[4 * a + 3][b];
+    const unsigned t0 = __builtin_amdgcn_perm(w1, w0, 0x05010400u), t1 = __builtin_amdgcn_perm(w1, w0, 0x07030602u);
+    const unsigned t2 = __builtin_amdgcn_perm(w3, w2, 0x05010400u), t3 = __builtin_amdgcn_perm(w3, w2, 0x07030602u);
+    const unsigned o[4] = {__builtin_amdgcn_perm(t2, t0, 0x05040100u), __builtin_amdgcn_perm(t2, t0, 0x07060302u),
+                           __builtin_amdgcn_perm(t3, t1, 0x05040100u), __builtin_amdgcn_perm(t3, t1, 0x07060302u)};
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      *reinterpret_cast<unsigned*>(dst + base + (long long)(c0 + 4 * b + k) * R + r0 + 4 * a) = o[k];
+  }
+}
+
 int launch_transpose_last2_s8(const int8_t* src, int8_t* dst, long long B, long long R, long long C,
                               hipStream_t stream) {
   if (B * R * C == 0) return TI_OK;
+  if (R % 128 == 0 && C % 128 == 0 && (reinterpret_cast<uintptr_t>(src) & 15) == 0 &&
+      (reinterpret_cast<uintptr_t>(dst) & 3) == 0) {
+    dim3 grid128((unsigned)(C / 128), (unsigned)(R / 128), (unsigned)B);
+    hipLaunchKernelGGL(transpose_last2_tiles128_kernel, grid128, dim3(256), 0, stream, src, dst, (int)R, (int)C);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "transpose launch: %s", hipGetErrorString(e));
+    return TI_OK;
+  }
   dim3 grid((unsigned)((C + 63) / 64), (unsigned)((R + 63) / 64), (unsigned)B);
   if (R % 64 == 0 && C % 64 == 0 && (reinterpret_cast<uintptr_t>(src) & 15) == 0 &&
       (reinterpret_cast<uintptr_t>(dst) & 3) == 0)
