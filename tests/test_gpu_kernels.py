@@ -458,9 +458,9 @@ def test_int8_layout_kernels():
         assert out.is_contiguous() and torch.equal(out, ref)
         back = X.merge_heads(out.view(B * H, T, d), B, H, T, d)
         assert back.shape == (B, T, H * d) and torch.equal(back, t)
-    # whole tiles take the 4 x 4-block kernels: 128 x 128 tiles (the first two), 64 x 64 tiles (the next two and the
-    # sliced source below)
-    for (B, R, C) in [(160, 512, 128), (2, 128, 384), (3, 64, 64), (2, 192, 320), (8, 513, 128), (3, 70, 50), (2, 1, 128), (5, 64, 1),
+    # R % 4 == 0 and C % 16 == 0 take the 4 x 4-block kernels: 128 x 128 tiles (the first two), 64 x 64 tiles with
+    # and without cut-off edge tiles (the next five and the sliced source below); the rest the byte-by-byte kernel
+    for (B, R, C) in [(160, 512, 128), (2, 128, 384), (3, 64, 64), (2, 192, 320), (4, 520, 128), (2, 68, 48), (3, 36, 16), (8, 513, 128), (3, 70, 50), (2, 1, 128), (5, 64, 1),
                       (1, 200, 333)]:
         _say(f"transpose_last2 B={B} R={R} C={C}")
         t = _s8(g, B, R, C).to(DEV)

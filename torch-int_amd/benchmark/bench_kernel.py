@@ -41,7 +41,7 @@ LINEAR = {
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--op", required=True, choices=list(LINEAR) + ["bmm_f32t", "bmm_s8t", "bmm_s32t", "bmm_s8t_rowmajor", "ln_q", "ln_q_f16", "add_ln_q",
-                                               "softmax_q", "qk_softmax_q", "attn_prefill", "decode_attn", "copy",
+                                               "softmax_q", "qk_softmax_q", "attn_prefill", "decode_attn", "transpose_last2", "copy",
                                                "mfma_loop", "mfma_ceiling", "store_loop"])
     ap.add_argument("--shape", type=int, nargs="+", required=True)
     ap.add_argument("--iters", type=int, default=20)
@@ -165,6 +165,16 @@ def main():
         gamma, beta = torch.ones(H, device=dev).half(), torch.zeros(H, device=dev).half()
         fn = lambda: C.dq_add_layernorm_q(inp, 0.01, res, gamma, beta, 1e-5)  # noqa: E731
         nbytes = 9.0 * rows * H + 4 * H
+    elif args.op == "transpose_last2":
+        # int8 [B, R, C] -> [B, C, R]: V -> V^T in front of P.V; --rotate sources so that none stays cached
+        B, R, C_ = args.shape
+        srcs = [s8(B, R, C_) for _ in range(max(1, args.rotate))]
+        turn = [0]
+
+        def fn():
+            turn[0] = (turn[0] + 1) % len(srcs)
+            return X.transpose_last2(srcs[turn[0]])
+        nbytes = 2.0 * B * R * C_
     elif args.op == "mfma_loop":
         mode, steps = args.shape
         data = (torch.full((1 << 20,), 1, dtype=torch.int8, device=dev) if args.pattern == "constant"

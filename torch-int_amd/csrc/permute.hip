@@ -138,7 +138,8 @@ int launch_permute_0213_s8(const int8_t* src, int8_t* dst, long long B, long lon
   return TI_OK;
 }
 
-// Whole 64x64 tiles, 16-byte aligned rows (R % 64 == 0, C % 64 == 0): a thread owns one 4x4 block of bytes.  The
+// 64x64 tiles of a matrix with R % 4 == 0 and C % 16 == 0 (edge tiles are cut off at whole 16-byte chunks of a source
+// row and whole dwords of an output row): a thread owns one 4x4 block of bytes.  The
 // tile goes into the LDS as dwords (row pitch 17 dwords); thread (a, b) reads the dwords of rows 4a .. 4a+3 at
 // dword column b, transposes the 4x4 bytes in registers with four + four v_perm_b32 and stores four dwords: bytes
 // 4a .. 4a+3 of the output rows 4b .. 4b+3.  a runs fastest over the lanes, so a wave writes 64 contiguous bytes of
@@ -152,12 +153,15 @@ __global__ __launch_bounds__(256) void transpose_last2_tiles_kernel(const int8_t
   const int t = threadIdx.x;
   {
     const int r = t >> 2, q = t & 3;
-    const v4i v = *reinterpret_cast<const v4i*>(src + base + (long long)(r0 + r) * C + c0 + q * 16);
+    if (r0 + r < R && c0 + q * 16 < C) {
+      const v4i v = *reinterpret_cast<const v4i*>(src + base + (long long)(r0 + r) * C + c0 + q * 16);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) tile[r][4 * q + j] = (unsigned)v[j];
+      for (int j = 0; j < 4; ++j) tile[r][4 * q + j] = (unsigned)v[j];
+    }
   }
   __syncthreads();
   const int a = t & 15, b = t >> 4;
+  if (r0 + 4 * a >= R || c0 + 4 * b >= C) return;  // after the only barrier
   const unsigned w0 = tile[4 * a][b], w1 = tile[4 * a + 1][b], w2 = tile[4 * a + 2][b], w3 = tile[4 * a + 3][b];
   // v_perm_b32(hi, lo, sel): result byte i = byte sel[i] of the eight bytes {lo: 0..3, hi: 4..7}
   const unsigned t0 = __builtin_amdgcn_perm(w1, w0, 0x05010400u);  // w0.0 w1.0 w0.1 w1.1
@@ -218,7 +222,7 @@ int launch_transpose_last2_s8(const int8_t* src, int8_t* dst, long long B, long 
     return TI_OK;
   }
   dim3 grid((unsigned)((C + 63) / 64), (unsigned)((R + 63) / 64), (unsigned)B);
-  if (R % 64 == 0 && C % 64 == 0 && (reinterpret_cast<uintptr_t>(src) & 15) == 0 &&
+  if (R % 4 == 0 && C % 16 == 0 && (reinterpret_cast<uintptr_t>(src) & 15) == 0 &&
       (reinterpret_cast<uintptr_t>(dst) & 3) == 0)
     hipLaunchKernelGGL(transpose_last2_tiles_kernel, grid, dim3(256), 0, stream, src, dst, (int)R, (int)C);
   else
