@@ -2383,12 +2383,18 @@ int launch_kind(const GemmParams& p, void* workspace, long long workspace_bytes,
   if (p.K % PBK == 0 && p.K >= PBK) {
     // a 256-wide tile on a narrow or short output would mostly multiply padding
     const bool wide = p.N > 128 && p.M > 128;
-    if (t256 >= 160 && wide) {
-      // 256x160 or 256x288 tiles (16x16 blocks) when the width allows it and they fill the CUs more
-      // evenly (e.g. 2048x5120: 160 tiles of 256x256 but 256 of 256x160; 2048x9216: 288 tiles of 256x256 =
-      // two rounds, but exactly 256 of 256x288).  Rates relative to the 256x256 kernel at full occupancy,
-      // measured: with 128-byte steps 0.94 (256x160, three LDS stages) and 0.95 (256x288); with 64-byte steps
-      // (K not a multiple of 128) 0.78 and 0.9.
+    if (wide) {
+      // Tiles of 256 rows: 256x256 (32x32 blocks), or 256x160 / 256x288 / 256x128 (16x16 blocks) when the width
+      // divides and they fill the CUs more evenly (2048x5120: 160 tiles of 256x256 but 256 of 256x160; 2048x9216:
+      // 288 tiles of 256x256 = two rounds, but exactly 256 of 256x288; 2048x4096: 128 of 256x256 but 256 of
+      // 256x128).  Each candidate is priced as its rate relative to the 256x256 kernel at full occupancy, measured
+      // (128-byte steps: 0.94 for 256x160 with its three LDS stages, 0.95 for 256x288, 0.93 for 256x128; 64-byte
+      // steps, K not a multiple of 128: 0.78 and 0.9), times the share of CU rounds its tiles fill.  The 128x128
+      // kernel (64-byte steps, two stages) runs at half that rate per CU, a little more with two workgroups on
+      // every CU, and takes over where few tiles of 256 rows would leave most CUs idle.
+      // Measured with this rule against the one before it, which looked at the count of 256x256 tiles only and sent
+      // everything under 160 of them to the 128x128 kernel: 1600x5120x20480 290 -> 161 us, 1600x5120x5120 76 -> 47,
+      // 2048x4096x4096 48 -> 35, 2048x4096x16384 170 -> 118, 2048x2560x2560 25 -> 20, 2048x12288x12288 285 -> 253.
       const long long cus = num_cus();
       auto fill = [&](long long tiles) { return (double)tiles / (double)(((tiles + cus - 1) / cus) * cus); };
       const long long rows256 = (p.M + 255) / 256;
@@ -2398,19 +2404,30 @@ int launch_kind(const GemmParams& p, void* workspace, long long workspace_bytes,
       const double e256 = fill(t256);
       const double e160 = p.N % 160 == 0 ? f160 * fill(rows256 * (p.N / 160) * p.batch) : 0.0;
       const double e288 = p.N % 288 == 0 ? f288 * fill(rows256 * (p.N / 288) * p.batch) : 0.0;
-      if (e160 > e256 && e160 >= e288) {
-        g_last_kernel = "pipe16_256x160";
-        if (wide_step) return launch_pipe16q<Pipe16QCfg<256, 160, 4, 2, KIND>>(p, stream);
-        return launch_pipe16<Pipe16Cfg<256, 160, 4, 2, 5, KIND>>(p, stream);
+      // (batched products keep their tuned 256x256 / 128x128 choice: they are bound by HBM, not by the matrix pipe)
+      const double e128w = wide_step && p.batch == 1 && p.N % 128 == 0 ? 0.93 * fill(rows256 * (p.N / 128)) : 0.0;
+      const double e128 = t128 >= 2 * cus ? 0.6 : t128 >= cus ? 0.47 : 0.47 * (double)t128 / (double)cus;
+      const double best = e256 > e160 ? (e256 > e288 ? (e256 > e128w ? e256 : e128w) : (e288 > e128w ? e288 : e128w))
+                                      : (e160 > e288 ? (e160 > e128w ? e160 : e128w) : (e288 > e128w ? e288 : e128w));
+      if (t256 >= 160 || (p.batch == 1 && best > e128)) {
+        if (e160 > e256 && e160 >= e288 && e160 >= e128w) {
+          g_last_kernel = "pipe16_256x160";
+          if (wide_step) return launch_pipe16q<Pipe16QCfg<256, 160, 4, 2, KIND>>(p, stream);
+          return launch_pipe16<Pipe16Cfg<256, 160, 4, 2, 5, KIND>>(p, stream);
+        }
+        if (e288 > e256 && e288 >= e128w) {
+          g_last_kernel = "pipe16_256x288";
+          if (wide_step) return launch_pipe16q<Pipe16QCfg<256, 288, 4, 2, KIND>>(p, stream);
+          return launch_pipe16<Pipe16Cfg<256, 288, 4, 2, 4, KIND>>(p, stream);
+        }
+        if (e128w > e256) {
+          g_last_kernel = "pipe16_256x128";
+          return launch_pipe16q<Pipe16QCfg<256, 128, 4, 2, KIND>>(p, stream);
+        }
+        g_last_kernel = "pipe_256x256";
+        if (p.K % QBK == 0) return launch_pipe2<Pipe2Cfg<256, 256, 2, 4, KIND, SWAP>>(p, stream);  // whole cache lines per row
+        return launch_pipe<PipeCfg<256, 256, 2, 4, 4, KIND, SWAP>>(p, stream);
       }
-      if (e288 > e256) {
-        g_last_kernel = "pipe16_256x288";
-        if (wide_step) return launch_pipe16q<Pipe16QCfg<256, 288, 4, 2, KIND>>(p, stream);
-        return launch_pipe16<Pipe16Cfg<256, 288, 4, 2, 4, KIND>>(p, stream);
-      }
-      g_last_kernel = "pipe_256x256";
-      if (p.K % QBK == 0) return launch_pipe2<Pipe2Cfg<256, 256, 2, 4, KIND, SWAP>>(p, stream);  // whole cache lines per row
-      return launch_pipe<PipeCfg<256, 256, 2, 4, 4, KIND, SWAP>>(p, stream);
     }
     // 128-wide outputs with many rows (P.V of a long prefill): 256x128 tiles, three stages of 128-byte steps
     if (p.N == 128 && p.K % QBK == 0 && p.M >= 512 && (long long)((p.M + 255) / 256) * p.batch >= 2 * num_cus()) {
