@@ -112,7 +112,7 @@ def test_linear_large_tiles(variant):
     for (M, N, K) in [(2048, 5120, 256), (2100, 5000, 272), (4096, 2560, 128), (4000, 2816, 1024), (4090, 2790, 256),
                       (2010, 5120, 384), (1990, 9216, 128), (2040, 5120, 128), (2048, 2560, 640),
                       # 256x128 tiles (widths that 160 and 288 do not divide, or fill worse), 256x160 tiles under 160 tiles of 256x256
-                      (2048, 4096, 512), (1100, 4096, 256), (1600, 5120, 640), (1290, 5120, 128)]:
+                      (2048, 4096, 2048), (1100, 4096, 2048), (1600, 5120, 2048), (1290, 5120, 2176)]:
         _say(f"linear-large {variant} M={M} N={N} K={K}")
         _linear_case(C, variant, M, N, K, seed=7)
 
@@ -126,8 +126,8 @@ def test_every_gemm_kernel_family_is_reached_and_exact(two_launch_split_k):
               ((2000, 9216, 192), "pipe16_256x288"), ((2000, 9216, 384), "pipe16_256x288"),
               ((4096, 2816, 192), "pipe_256x256"),
               ((4096, 2816, 128), "pipe_256x256"), ((1024, 2048, 64), "pipe_128x128"),
-              ((2048, 4096, 256), "pipe16_256x128"), ((1280, 5120, 256), "pipe16_256x128"), ((1600, 5120, 384), "pipe16_256x160"),
-              ((2048, 2048, 256), "pipe_128x128"), ((2048, 7168, 256), "pipe_256x256"),
+              ((2048, 4096, 2048), "pipe16_256x128"), ((1280, 5120, 2048), "pipe16_256x128"), ((1600, 5120, 2048), "pipe16_256x160"),
+              ((2048, 2048, 2048), "pipe_128x128"), ((2048, 7168, 2048), "pipe_256x256"), ((2048, 4096, 256), "pipe_128x128"),
               ((512, 5120, 5120), "pipe16_128x80"), ((384, 2560, 1024), "pipe16_128x80"), ((1024, 5120, 5120), "splitk_256x160"),
               ((256, 3200, 11648), "splitk_256x160"), ((1024, 9216, 9216), "splitk_256x288"),
               ((384, 2880, 4608), "splitk_128x80"), ((128, 640, 4096), "splitk_128x80"),
@@ -640,7 +640,7 @@ def test_linear_accumulate_into_output(two_launch_split_k):
     g = torch.Generator().manual_seed(63)
     seen = set()
     for (M, N, K) in [(2048, 5120, 256), (2048, 5120, 64), (2000, 9216, 192), (2000, 9216, 128), (4096, 2816, 128),
-                      (2048, 4096, 384),   # 256x128 tiles
+                      (2048, 4096, 2048),   # 256x128 tiles
                       (4096, 2816, 1024), (1024, 2048, 64), (1024, 5120, 5120), (1024, 4608, 3584), (256, 3072, 7744),
                       (1024, 9216, 9216), (384, 2880, 4608), (4, 4608, 16384), (256, 3200, 11648), (256, 1600, 11648), (384, 2560, 1024),
                       (128, 640, 4096), (128, 768, 4096), (16, 5120, 3072), (3, 100, 272), (300, 200, 48), (2100, 5000, 272),

@@ -2396,20 +2396,27 @@ int launch_kind(const GemmParams& p, void* workspace, long long workspace_bytes,
       // everything under 160 of them to the 128x128 kernel: 1600x5120x20480 290 -> 161 us, 1600x5120x5120 76 -> 47,
       // 2048x4096x4096 48 -> 35, 2048x4096x16384 170 -> 118, 2048x2560x2560 25 -> 20, 2048x12288x12288 285 -> 253.
       const long long cus = num_cus();
-      auto fill = [&](long long tiles) { return (double)tiles / (double)(((tiles + cus - 1) / cus) * cus); };
+      // useful outputs over the outputs the CU rounds of a tiling have room for (partial tiles and partial rounds
+      // both count as waste)
+      auto fill = [&](long long tiles, int bn) {
+        return (double)p.M * p.N * p.batch / ((double)(((tiles + cus - 1) / cus) * cus) * 256.0 * bn);
+      };
       const long long rows256 = (p.M + 255) / 256;
       const bool wide_step = p.K % QBK == 0;
       const double f160 = wide_step ? 0.94 : 0.78;
       const double f288 = wide_step ? 0.95 : 0.9;
-      const double e256 = fill(t256);
-      const double e160 = p.N % 160 == 0 ? f160 * fill(rows256 * (p.N / 160) * p.batch) : 0.0;
-      const double e288 = p.N % 288 == 0 ? f288 * fill(rows256 * (p.N / 288) * p.batch) : 0.0;
-      // (batched products keep their tuned 256x256 / 128x128 choice: they are bound by HBM, not by the matrix pipe)
-      const double e128w = wide_step && p.batch == 1 && p.N % 128 == 0 ? 0.93 * fill(rows256 * (p.N / 128)) : 0.0;
+      const double e256 = fill(t256, 256);
+      const double e160 = p.N % 160 == 0 ? f160 * fill(rows256 * (p.N / 160) * p.batch, 160) : 0.0;
+      const double e288 = p.N % 288 == 0 ? f288 * fill(rows256 * (p.N / 288) * p.batch, 288) : 0.0;
+      // The 256x128 tiles and the comparison with the 128x128 kernel are for linears with a K of some length
+      // (the rates above were measured at K >= 4096; at K = 768 the 128x128 kernel's short prologue wins); batched
+      // products keep their tuned 256x256 / 128x128 choice, they are bound by HBM, not by the matrix pipe.
+      const bool priced = p.batch == 1 && p.K >= 2048 && t128 >= 128;
+      const double e128w = priced && wide_step && p.N % 128 == 0 ? 0.93 * fill(rows256 * (p.N / 128), 128) : 0.0;
       const double e128 = t128 >= 2 * cus ? 0.6 : t128 >= cus ? 0.47 : 0.47 * (double)t128 / (double)cus;
       const double best = e256 > e160 ? (e256 > e288 ? (e256 > e128w ? e256 : e128w) : (e288 > e128w ? e288 : e128w))
                                       : (e160 > e288 ? (e160 > e128w ? e160 : e128w) : (e288 > e128w ? e288 : e128w));
-      if (t256 >= 160 || (p.batch == 1 && best > e128)) {
+      if (t256 >= 160 || (priced && best > e128)) {
         if (e160 > e256 && e160 >= e288 && e160 >= e128w) {
           g_last_kernel = "pipe16_256x160";
           if (wide_step) return launch_pipe16q<Pipe16QCfg<256, 160, 4, 2, KIND>>(p, stream);
