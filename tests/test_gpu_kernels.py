@@ -764,6 +764,8 @@ def test_grouped_prefill_linears_one_launch():
     # (bsz, seq, heads, d, K, problems, family)
     for (B, T, H, d, K, n, family) in [(4, 512, 40, 128, 256, 3, "pipe16_256x160_group"),
                                        (2, 1000, 72, 128, 128, 3, "pipe16_256x288_group"),
+                                       (4, 512, 32, 128, 256, 3, "pipe16_256x128_group"),
+                                       (1, 500, 32, 128, 384, 3, "pipe16_256x128_group"),
                                        (2, 100, 5, 128, 384, 2, "pipe16_256x160_group"),
                                        (1, 300, 9, 32, 640, 4, "pipe16_256x288_group"),
                                        (3, 171, 10, 16, 128, 3, "pipe16_256x160_group"),
@@ -784,7 +786,7 @@ def test_grouped_prefill_linears_one_launch():
         out = X.linear_a8_w8_b8_o8_group_heads(xd, wd, bd, al, be, B, T, H, d)
         if family:
             assert C._lib.ti_last_kernel().decode() == family
-        assert X.linear_group_is_one_launch(M, N, K) == (family is not None)
+        assert X.linear_group_is_one_launch(M, N, K, n) == (family is not None)
         for o, r_ in zip(out, ref):
             assert o.shape == (B, H, T, d) and o.is_contiguous()
             assert torch.equal(o.cpu(), r_.view(B, T, H, d).transpose(1, 2)), (M, N, K)

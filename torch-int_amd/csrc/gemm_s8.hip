@@ -197,15 +197,25 @@ int launch_gemm_group_s8(const GemmParams& shape, const GemmGroup& grp, hipStrea
     const long long rows256 = (shape.M + 255) / 256;
     const double e160 = shape.N % 160 == 0 ? 0.88 * fill(rows256 * (shape.N / 160) * grp.count) : 0.0;
     const double e288 = shape.N % 288 == 0 ? 0.95 * fill(rows256 * (shape.N / 288) * grp.count) : 0.0;
-    if (e160 > 0.0 || e288 > 0.0) {
+    // widths that only 128 divides (OPT-6.7B: 4096): 256x128 tiles, unless one problem at a time fills the CUs
+    // with 256x256 tiles as well (three 2048x4096x4096: 98 -> 93 us, at 512 rows 57 -> 28 us; 2048x7168x7168
+    // stays with three launches, 277 against 283 us)
+    const double e256_alone = fill(rows256 * ((shape.N + 255) / 256));
+    double e128 = shape.N % 128 == 0 ? 0.87 * fill(rows256 * (shape.N / 128) * grp.count) : 0.0;
+    if (e128 < 0.5 || e128 <= e256_alone) e128 = 0.0;
+    if (e160 > 0.0 || e288 > 0.0 || e128 > 0.0) {
       GemmParams q = shape;
       q.batch = grp.count;
-      if (e160 >= e288) {
+      if (e160 >= e288 && e160 >= e128) {
         g_last_kernel = "pipe16_256x160_group";
         return launch_pipe16q<Pipe16QCfg<256, 160, 4, 2, KIND, true>>(q, stream, grp);
       }
-      g_last_kernel = "pipe16_256x288_group";
-      return launch_pipe16q<Pipe16QCfg<256, 288, 4, 2, KIND, true>>(q, stream, grp);
+      if (e288 >= e128) {
+        g_last_kernel = "pipe16_256x288_group";
+        return launch_pipe16q<Pipe16QCfg<256, 288, 4, 2, KIND, true>>(q, stream, grp);
+      }
+      g_last_kernel = "pipe16_256x128_group";
+      return launch_pipe16q<Pipe16QCfg<256, 128, 4, 2, KIND, true>>(q, stream, grp);
     }
   }
   for (int i = 0; i < grp.count; ++i) {

@@ -515,18 +515,44 @@ def linear_a8_w8_b8_o8_group(x, weights, biases, alphas, betas, checked=False):
     return out.unbind(0)
 
 
-def linear_group_is_one_launch(M, N, K):
+_cus = []
+
+
+def _cu_count():
+    """Compute units of the current device (what the library's dispatcher counts tiles against)."""
+    if not _cus:
+        _cus.append(torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count
+                    if torch.cuda.is_available() else 256)
+    return _cus[0]
+
+
+def linear_group_is_one_launch(M, N, K, count=3):
     """Whether the library runs a group of [M,K] x [N,K] linears as ONE launch (otherwise it loops over the
     problems, without the split-K workspace that separate calls would get)."""
     if M <= 16:
         return K % 1024 == 0
-    return M > 128 and K >= 128 and K % 128 == 0 and (N % 160 == 0 or N % 288 == 0)
+    if not (M > 128 and K >= 128 and K % 128 == 0):
+        return False
+    if N % 160 == 0 or N % 288 == 0:
+        return True
+    if N % 128:
+        return False
+    # 256x128 tiles: when they fill at least half of their rounds over the CUs, and more of them than 256x256 tiles
+    # of one problem at a time would (launch_gemm_group_s8 in csrc/gemm_s8.hip decides the same way)
+    cus = _cu_count()
+    rows = (M + 255) // 256
+
+    def fill(tiles):
+        return tiles / (((tiles + cus - 1) // cus) * cus)
+    e128 = 0.87 * fill(rows * (N // 128) * count)
+    return e128 >= 0.5 and e128 > fill(rows * ((N + 255) // 256))
 
 
 def linear_a8_w8_b8_o8_group_heads(x, weights, biases, alphas, betas, bsz, seq_len, heads, head_dim, checked=False):
     """``[linear_a8_w8_b8_o8_heads(x, w, b, a, be, bsz, seq_len, heads, head_dim) for ...]`` as one call: a tuple
     of int8 [bsz, heads, seq, head_dim] outputs (views of one allocation).  The q/k/v projections of a prefill:
-    widths the 256x160 or 256x288 tiles divide run as one persistent launch over all the problems."""
+    widths the 256x160, 256x288 or (see ``linear_group_is_one_launch``) 256x128 tiles divide run as one persistent
+    launch over all the problems."""
     if not checked and not (can_linear_group(x, weights, biases)
                             and all(can_linear_heads(x, w, b, bsz, seq_len, heads, head_dim)
                                     for w, b in zip(weights, biases))):

@@ -167,7 +167,7 @@ class Int8OPTAttention(nn.Module):
         if not all(_hip_ext.can_linear_heads(x, w, b, bsz, tgt_len, H, d) for w, b in zip(weights, biases)):
             return None
         if (_hip_ext.can_linear_group(x, weights, biases)
-                and _hip_ext.linear_group_is_one_launch(x.shape[0], weights[0].shape[0], x.shape[1])):
+                and _hip_ext.linear_group_is_one_launch(x.shape[0], weights[0].shape[0], x.shape[1], len(weights))):
             # one call; widths the 16x16-block tiles divide run as a single persistent launch
             return _hip_ext.linear_a8_w8_b8_o8_group_heads(
                 x, weights, biases, [lin._scalar("a") for lin in (q, k, v)], [lin._scalar("b") for lin in (q, k, v)],
