@@ -273,6 +273,24 @@ def test_bmm_shapes():
         _bmm_case(C, B, M, N, K, seed=200 + i)
 
 
+def test_large_problems_with_an_inner_dimension_that_16_does_not_divide():
+    # the library's kernel for such shapes is one thread per output; from 2^26 products the host functions pad K
+    # with zeros and the tiled kernels run (same results: the added products are zero)
+    import ctypes
+    import torch_int._CUDA as C
+    C._lib.ti_last_kernel.restype = ctypes.c_char_p
+    for i, (B, M, N, K) in enumerate([(8, 256, 128, 1500), (3, 200, 260, 1001)]):
+        _say(f"bmm, odd K: B={B} M={M} N={N} K={K}")
+        _bmm_case(C, B, M, N, K, seed=300 + i, prob_lhs=i == 0)
+        assert C._lib.ti_last_kernel().decode() != "scalar"
+    for variant in ("b8_o8", "bfp32_ofp32"):
+        _say(f"linear, odd K: {variant}")
+        _linear_case(C, variant, 512, 640, 1001, seed=310)
+        assert C._lib.ti_last_kernel().decode() != "scalar"
+    _linear_case(C, "b8_o8", 70, 50, 37, seed=311)   # small: the one-thread-per-output kernel as it is
+    assert C._lib.ti_last_kernel().decode() == "scalar"
+
+
 def test_bmm_literal_fixture_from_upstream_tests():
     import torch_int._CUDA as C
     with open(os.path.join(GOLDEN, "bmm_literal_16x16.json")) as f:

@@ -2398,8 +2398,10 @@ int launch_kind(const GemmParams& p, void* workspace, long long workspace_bytes,
       const long long cus = num_cus();
       // useful outputs over the outputs the CU rounds of a tiling have room for (partial tiles and partial rounds
       // both count as waste)
+      // (batched products count tiles only, as they always did: they are bound by HBM, where padding costs no bytes)
       auto fill = [&](long long tiles, int bn) {
-        return (double)p.M * p.N * p.batch / ((double)(((tiles + cus - 1) / cus) * cus) * 256.0 * bn);
+        const double room = (double)(((tiles + cus - 1) / cus) * cus);
+        return p.batch == 1 ? (double)p.M * p.N / (room * 256.0 * bn) : (double)tiles / room;
       };
       const long long rows256 = (p.M + 255) / 256;
       const bool wide_step = p.K % QBK == 0;

@@ -153,6 +153,17 @@ def _workspace(dev_index, stream, nbytes):
     return ws.data_ptr(), ws.numel()
 
 
+def _pad_inner(a, b, K, macs):
+    """Operands whose inner dimension is not a multiple of 16 have no aligned rows for the tiled kernels, and the
+    library then runs a one-thread-per-output kernel (40 x 1500 x 128 x 1500: 32 ms).  From a size at which that
+    hurts, both operands are copied with K padded by zeros to a multiple of 64 first: the added products are zero,
+    the results the same (upstream rejects such shapes: "cutlass cannot implement")."""
+    if K % 16 == 0 or macs < (1 << 26):
+        return a, b, K
+    pad = -K % 64
+    return torch.nn.functional.pad(a, (0, pad)), torch.nn.functional.pad(b, (0, pad)), K + pad
+
+
 def _linear(op, kind, x, w, bias, bias_dtype, out_dtype, alpha, beta, inout=None):
     # fast accept path first; the slow path below names what is wrong
     if not (type(x) is torch.Tensor and type(w) is torch.Tensor and x.dtype is _I8 and w.dtype is _I8
@@ -184,6 +195,7 @@ def _linear(op, kind, x, w, bias, bias_dtype, out_dtype, alpha, beta, inout=None
             _fail(op, f"the tensor to add into must be a contiguous {out_dtype} tensor of {M}x{N} elements on {dev}")
     if M == 0 or N == 0:
         return out
+    x, w, K = _pad_inner(x, w, K, M * N * K)
     idx = dev.index
     switch = idx != _current_device()
     if switch:
@@ -252,6 +264,7 @@ def _bmm(op, kind, a, b, out_dtype, alpha):
     out = _empty((batch, M, N), dtype=out_dtype, device=dev)
     if out.numel() == 0:
         return out
+    a, b, K = _pad_inner(a, b, K, batch * M * N * K)
     idx = dev.index
     switch = idx != _current_device()
     if switch:
