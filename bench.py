@@ -25,6 +25,7 @@ Also reported on the same JSON line:
   decoder_layer_ms   Int8OPTDecoderLayer at OPT-13B shape (batch 4, seq 512).
 """
 import argparse
+import contextlib
 import ctypes
 import json
 import os
@@ -50,11 +51,114 @@ FAMILIES = {
     # 614 663 KiB x 2.000 fetched + 424 056 KiB written per launch, mean over its 4 launches per step
     "pipe_256x256": {"kernel": "gemm_pipe2_kernel<Pipe2Cfg<256,256,2,4,KIND,SWAP>>", "traffic": 1.693e9},
 }
+# The counter runs behind FAMILIES[*]["traffic"] were made on the kernels as this hash of their source file describes
+# them (first 16 hex digits of the SHA-256 of torch-int_amd/csrc/gemm_s8_impl.h).  When the file has changed since,
+# the bench line says so next to the figure instead of passing an old measurement off as current.
+TRAFFIC_SOURCE_SHA16 = "e6c2c36dc989644a"
+
+
+def traffic_is_current():
+    import hashlib
+    try:
+        with open(os.path.join(ROOT, "torch-int_amd", "csrc", "gemm_s8_impl.h"), "rb") as f:
+            return hashlib.sha256(f.read()).hexdigest()[:16] == TRAFFIC_SOURCE_SHA16
+    except OSError:
+        return None
+
+
 SHAPES = [(5120, 5120), (20480, 5120), (5120, 20480)]   # (N, K): qkv/out_proj, fc1, fc2
 MS = [1, 16, 128, 512, 2048, 8192]
 VARIANTS = ["b32_o32", "bfp32_ofp32", "b8_o8", "relu_b8_o8"]
 BIAS_BYTES = {"b32_o32": 4, "bfp32_ofp32": 4, "b8_o8": 1, "relu_b8_o8": 1}
 OUT_BYTES = {"b32_o32": 4, "bfp32_ofp32": 4, "b8_o8": 1, "relu_b8_o8": 1}
+
+
+class Telemetry:
+    """Shader clock and board power of the GPU while a measurement runs, read by a host thread from the amdgpu
+    driver's text files: `pp_dpm_sclk` (the line marked * is the current clock, MHz) and hwmon `power1_input`
+    (or `power1_average`; microwatts, with `power1_cap` = the board's power limit).  `with tele.window(label):`
+    samples every `period_s` for as long as the block runs and keeps mean / min / max under `label`.  Where the
+    files do not exist the record says so and nothing else changes."""
+
+    def __init__(self, period_s=0.01):
+        import glob
+        self.period_s = period_s
+        self.windows = {}
+        self.sclk_path = self.power_path = None
+        self.cap_w = None
+        for card in sorted(glob.glob("/sys/class/drm/card[0-9]*")):
+            try:
+                if open(card + "/device/vendor").read().strip() != "0x1002":
+                    continue
+            except OSError:
+                continue
+            if os.path.exists(card + "/device/pp_dpm_sclk"):
+                self.sclk_path = card + "/device/pp_dpm_sclk"
+            for hw in sorted(glob.glob(card + "/device/hwmon/hwmon*")):
+                for name in ("power1_input", "power1_average"):
+                    if self.power_path is None and os.path.exists(hw + "/" + name):
+                        self.power_path = hw + "/" + name
+                try:
+                    self.cap_w = int(open(hw + "/power1_cap").read()) / 1e6
+                except (OSError, ValueError):
+                    pass
+            break   # the first AMD card: this build runs on one GPU
+
+    def available(self):
+        return self.sclk_path is not None or self.power_path is not None
+
+    def _read(self):
+        mhz = watts = None
+        try:
+            if self.sclk_path:
+                for line in open(self.sclk_path):
+                    if "*" in line:
+                        mhz = float(line.split(":")[1].lower().replace("mhz", "").replace("*", "").strip())
+            if self.power_path:
+                watts = int(open(self.power_path).read()) / 1e6
+        except (OSError, ValueError, IndexError):
+            pass
+        return mhz, watts
+
+    def window(self, label):
+        import contextlib
+        import threading
+
+        @contextlib.contextmanager
+        def cm():
+            if not self.available():
+                yield
+                return
+            stop, samples = threading.Event(), []
+
+            def run():
+                while not stop.is_set():
+                    samples.append(self._read())
+                    stop.wait(self.period_s)
+            th = threading.Thread(target=run, daemon=True)
+            th.start()
+            try:
+                yield
+            finally:
+                stop.set()
+                th.join()
+                clk = [m for m, _ in samples if m is not None]
+                pw = [w for _, w in samples if w is not None]
+                rec = {"samples": len(samples)}
+                if clk:
+                    rec.update(sclk_mhz_mean=round(sum(clk) / len(clk), 1), sclk_mhz_min=min(clk), sclk_mhz_max=max(clk))
+                if pw:
+                    rec.update(power_w_mean=round(sum(pw) / len(pw), 1), power_w_min=round(min(pw), 1), power_w_max=round(max(pw), 1))
+                self.windows[label] = rec
+        return cm()
+
+    def report(self):
+        if not self.available():
+            return {"available": False, "note": "no amdgpu pp_dpm_sclk / hwmon power file under /sys/class/drm on this box"}
+        return {"available": True, "sclk_file": self.sclk_path, "power_file": self.power_path, "power_cap_w": self.cap_w,
+                "period_ms": self.period_s * 1e3, "windows": self.windows,
+                "note": "host-thread samples of the driver's text files during each measurement window; sclk is the "
+                        "driver's current shader clock (one figure for the whole device), power the board's input power"}
 
 
 def gemm_bytes(M, N, K, variant):
@@ -207,7 +311,7 @@ def hbm_kernels(torch, C, dev):
                     "GBps": by / ms / 1e6, "frac": by / ms / 1e6 / PEAK_HBM_GBS})
         # the whole attention of a prefill in one launch (no counterpart upstream; replaces the two products above, the
         # softmax chain and the head merge): bytes = q, k, v^T, context and one pass over the causal mask
-        if S >= 512:
+        if S >= 128:   # at S = 128 it replaces two launch-bound products of 7 us each
             import torch_int._hip_ext as X
             neg = torch.finfo(torch.float32).min
             mask = torch.zeros(S, S, device=dev).masked_fill(torch.triu(torch.ones(S, S, dtype=torch.bool, device=dev), 1), neg)
@@ -261,6 +365,51 @@ def decoder_layer_ms(torch, dev):
     return sustained_ms(torch, [lambda: layer(hidden, attention_mask=mask)], window_ms=300.0, warm_launches=20)
 
 
+def opt66b_model(torch, dev):
+    """The OPT-66B-shaped Int8OPTForCausalLM at full depth (64 layers, 65 GB of random int8 weights generated on the
+    device): decoder stack of a 512-token prefill and the per-token time of 32 decode steps, batch 1 and 4.  The
+    protocol of torch-int_amd/benchmark/bench_opt.py (upstream benchmark/bench_opt.py times the same stack)."""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location(
+        "ti_bench_opt", os.path.join(ROOT, "torch-int_amd", "benchmark", "bench_opt.py"))
+    bo = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bo)
+    model, cfg = bo.build("opt-66b", 0, dev)
+    int8_bytes = sum(b.numel() for _, b in model.named_buffers() if b.dtype == torch.int8)
+    D, H, F, L = bo.MODELS["opt-66b"]
+    out = {"model": "opt-66b", "layers": L, "int8_weight_GB": int8_bytes / 1e9, "seq": 512, "decode_steps": 32}
+    g = torch.Generator(device=dev).manual_seed(1)
+    with torch.no_grad():
+        for bsz in (4, 1):
+            ids = torch.randint(2, cfg.vocab_size, (bsz, 512), device=dev, generator=g)
+            model.model(ids, use_cache=True)   # warm-up
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            for _ in range(3):
+                model.model(ids, use_cache=True)
+            torch.cuda.synchronize()
+            stack_ms = (time.perf_counter() - t) * 1e3 / 3
+            o = model(ids, use_cache=True)
+            past, tok = o.past_key_values, o.logits[:, -1].argmax(-1, keepdim=True)
+            steps = []
+            for _ in range(32):
+                torch.cuda.synchronize()
+                t = time.perf_counter()
+                o = model(tok, past_key_values=past, use_cache=True)
+                torch.cuda.synchronize()
+                steps.append((time.perf_counter() - t) * 1e3)
+                past, tok = o.past_key_values, o.logits[:, -1].argmax(-1, keepdim=True)
+            med = sorted(steps)[len(steps) // 2]
+            ops = 2.0 * bsz * 512 * L * (4 * D * D + 2 * D * F)
+            out[f"batch{bsz}"] = {"decoder_stack_ms": stack_ms, "decoder_stack_linear_TOPS": ops / stack_ms / 1e9,
+                                  "decode_ms_per_token": med, "decode_weight_GBps": int8_bytes / 1e9 / (med / 1e3),
+                                  "logits_finite": bool(torch.isfinite(o.logits).all())}
+            del o, past
+    del model
+    torch.cuda.empty_cache()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -268,7 +417,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-ceiling", action="store_true", help="skip the matrix-pipe ceiling loops")
-    ap.add_argument("--sweep-only", action="store_true", help="skip the per-case, HBM-kernel and layer sections")
+    ap.add_argument("--sweep-only", action="store_true", help="skip the per-case, HBM-kernel, layer and model sections")
+    ap.add_argument("--no-model", action="store_true", help="skip the 64-layer OPT-66B model section")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (the path has no collectives); use --gpus 1")
@@ -314,14 +464,16 @@ def main():
             else:
                 c["fn"]()
 
+    tele = Telemetry()
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        step(marks[i], i)
-    torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    with tele.window("timed_sweep_steps"):
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            step(marks[i], i)
+        torch.cuda.synchronize()
+        ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
 
     def launch_ms(k):   # mean duration of heavy launch k over the steps that bracketed it
         took = [marks[i][k][0].elapsed_time(marks[i][k][1]) for i in range(args.steps) if (k + i) % stride == 0]
@@ -363,6 +515,8 @@ def main():
     result["roofline"] = {
         "bound": "mfma", "achieved": achieved, "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
         "frac": achieved / PEAK_INT8_TOPS, "traffic": FAMILIES.get(DOMINANT, {}).get("traffic"),
+        "traffic_source": {"counter_run_on_kernel_source_sha16": TRAFFIC_SOURCE_SHA16,
+                           "kernel_source_unchanged_since": traffic_is_current()},
         "kernel": FAMILIES.get(DOMINANT, {}).get("kernel", DOMINANT) + " (the sweep cases the library routes to it: "
                   + ", ".join(sorted({f"{cases[heavy[k]]['M']}x{cases[heavy[k]]['N']}x{cases[heavy[k]]['K']}" for k in dom})) + ")",
         "family": DOMINANT,
@@ -379,7 +533,7 @@ def main():
     if not args.no_ceiling:
         # what the matrix pipe of this board sustains on constant / random operand bytes (diagnostic loops, no GEMM)
         import torch_int._hip_ext as X
-        m = X.measure_mfma_ceiling(window_ms=250.0)
+        m = X.measure_mfma_ceiling(window_ms=250.0, window=lambda label: tele.window("ceiling_" + label))
         result["roofline"]["measured_ceiling"] = {
             "unit": "TOP/s", "constant": m["mfma_only_constant"], "random": m["mfma_only_random"],
             "lds_fed": m["lds_fed_random"], "all": m,
@@ -407,7 +561,10 @@ def main():
                     n_copies = -(-320 * 2 ** 20 // (c["N"] * c["K"]))
                     copies[key] = [c["w"]] + [c["w"].clone() for _ in range(n_copies - 1)]
                 fns = [c["make"](w) for w in copies[key]]
-            ms = sustained_ms(torch, fns, window_ms=200.0 if c["M"] >= 512 and c["kernel"] == DOMINANT or c["M"] >= 2048 else 60.0)
+            label = f"sustained_{c['variant']}_{c['M']}x{c['N']}x{c['K']}"
+            with (tele.window(label) if c["kernel"] == DOMINANT and c["M"] >= 2048 and c["variant"] in ("b8_o8", "bfp32_ofp32")
+                  else contextlib.nullcontext()):
+                ms = sustained_ms(torch, fns, window_ms=200.0 if c["M"] >= 512 and c["kernel"] == DOMINANT or c["M"] >= 2048 else 60.0)
             tops = c["ops"] / ms / 1e9
             gbs = c["bytes"] / ms / 1e6
             frac = tops / PEAK_INT8_TOPS if bound == "mfma" else gbs / PEAK_HBM_GBS
@@ -426,10 +583,18 @@ def main():
         result["cases"] = table
         torch.cuda.empty_cache()   # the per-case section leaves gigabytes of split blocks in the caching allocator
         result["hbm_kernels"] = hbm_kernels(torch, C, dev)
-        result["decoder_layer_ms"] = decoder_layer_ms(torch, dev)
+        with tele.window("decoder_layer"):
+            result["decoder_layer_ms"] = decoder_layer_ms(torch, dev)
+        if not args.no_model:
+            result["opt66b"] = opt66b_model(torch, dev)
+    # clocks and board power during the windows above: what the power-limit account of the MFMA figures rests on
+    result["roofline"]["telemetry"] = tele.report()
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(torch, C, dev)
     print(json.dumps(result), flush=True)
+    mismatches = n_bad + result.get("cpu_baseline", {}).get("gpu_mismatches", 0)
+    if mismatches:
+        sys.exit(f"bench.py: {mismatches} output elements differ from their references; the figures above are void")
 
 
 if __name__ == "__main__":

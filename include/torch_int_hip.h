@@ -52,9 +52,18 @@ int ti_init(void);
 
 /* Bytes of scratch the linear entry points can use for (M,N,K) to split the K
  * loop over workgroups when the output has too few tiles to fill the chip
- * (16 < M <= 1024 with a long K); 0 when no split is worthwhile.  Passing a
- * smaller or NULL workspace is always legal and only selects a non-split kernel. */
+ * (16 < M <= 1024 with a long K, or the last rows of a larger M: see ti_linear_row_split);
+ * 0 when no split is worthwhile.  Passing a smaller or NULL workspace is always legal and
+ * only selects a non-split kernel. */
 int64_t ti_linear_workspace_bytes(int64_t M, int64_t N, int64_t K);
+
+/* Diagnostic: the number r of rows that a linear of this shape cuts off its end and runs as a second, small
+ * problem (0 = none).  Tiled kernels pay for whole tiles of 256 rows and whole rounds of 256 CUs; when M > 1024 has
+ * a few rows (<= 128) beyond a multiple of 256 and the cost model prices "M - r rows on tiles + r rows through the
+ * split-K / streaming kernels" clearly below the whole, the library launches the two (ti_last_kernel then reads
+ * "<family>+<family>").  Same bytes out either way.  The reference's CUTLASS kernels predicate partial tiles instead
+ * (torch_int/kernels/linear.cu:35-45); prefill lengths are only padded to 16 (torch_int/models/opt.py:375-383). */
+int ti_linear_row_split(int64_t M, int64_t N, int64_t K);
 
 /* Diagnostics: the kernel family the calling thread's last linear / bmm_s8t_s8n_* call launched
  * ("pipe_256x256", "pipe16_256x160", "pipe16_256x288", "pipe16_256x128", "pipe16_128x80", "pipe_128x128",
@@ -71,9 +80,35 @@ const char* ti_last_kernel(void);
  * the call.  Default on, or off with the environment variable TORCH_INT_FUSED_SPLITK=0.  The form also stays off
  * on a device whose workgroup placement is not "ids congruent mod 8 share an XCD" (probed at the first use),
  * for more than 8 streams per device, and while a stream is being captured before the first use on its device.
- * Each stream has arrival counters of its own; a launch recorded into a HIP graph keeps those of the stream it
- * was recorded on, so that stream must not run other split-K linears while the graph replays on another one. */
+ * Each stream has arrival counters of its own (8 sets per device; a stream that has gone idle hands its set on when
+ * a ninth stream needs one).  The first split-K call on a stream runs a placement probe on it: one small kernel and
+ * ONE SYNCHRONISATION of that stream (not during a capture, where the call takes the two-launch form instead, and
+ * not from ti_linear_a8_w8_b8_o8_noalloc); ti_init() does it for the null stream.
+ * Workspace: the one-launch form needs `workspace` on a 256-byte boundary (a 16-byte aligned one takes the
+ * two-launch form).
+ * HIP graphs: a launch recorded into a graph keeps the arrival counters (and the caller's workspace) of the stream
+ * it was recorded on.  Replays of such a graph must therefore not overlap in time with other split-K linears
+ * issued on the recording stream, nor with replays of another graph recorded on that same stream.
+ * Misplacement: every one-launch GEMM checks that the workgroups of a tile ran on one XCD.  If one did not, the
+ * output of THAT call cannot be trusted although it returned TI_OK (the check runs on the device, after the call
+ * has returned): the next linear / bmm call on the device, whatever its shape, returns TI_ERR_LAUNCH once, naming
+ * the earlier call as the one to re-run, and the form switches itself off; a caller that makes no further call
+ * asks ti_fused_splitk_faulted() after it has synchronised.  No box of this pool has ever raised it. */
 int ti_fused_splitk(int enable);
+
+/* 1 when a one-launch split-K GEMM that has finished on the current device found a workgroup on an unexpected XCD
+ * (see ti_fused_splitk), else 0.  Reads one word of host memory; call it after synchronising with the launches in
+ * question.  No counterpart in the reference. */
+int ti_fused_splitk_faulted(void);
+
+/* Self-tests of the one-launch split-K's host-side bookkeeping (no GPU call, no counterpart in the reference):
+ * ti_selftest_fused_flag_action = what a GEMM call does for a device state (0 not probed, 1 usable, -1 off) and a
+ * misplacement flag: 1 go on, 0 take the two-launch form, -1 report the misplacement;
+ * ti_selftest_fused_slot = the slot of `stream` in a table of `cap` (<= 32) streams, bit i of live_mask / busy_mask
+ * saying whether slot i is registered / still has work queued; *fresh = 1 when the stream was not registered. */
+int ti_selftest_fused_flag_action(int state, int flag, int enabled, int64_t counters, int64_t max_counters);
+int ti_selftest_fused_slot(int64_t* table, uint32_t* live_mask, int cap, int64_t stream, uint32_t busy_mask,
+                           int* fresh);
 
 /* Diagnostic (no counterpart in the reference; computes nothing): one launch that issues the instruction mix of
  * the tiled GEMM mainloop `iters` times per wave on the first MiB of `data` (device memory, at least 1 MiB, 16-byte

@@ -191,3 +191,64 @@ def test_split_k_choice_is_sane_at_the_opt_widths():
         assert got[0] >= got[1] and got[0] >= got[2], (N, K, got)
     # OPT-125m widths are too small to be worth a second launch
     assert lib.ti_linear_workspace_bytes(512, 768, 768) == 0
+
+
+def test_one_launch_split_k_flag_logic():
+    # what a GEMM call does for a device state (0 not probed / 1 usable / -1 off) and a misplacement flag:
+    # 1 = go on with the one-launch form, 0 = two-launch form, -1 = report the misplacement
+    import torch_int._CUDA as C
+    lib = ctypes.CDLL(C.LIB_PATH)
+    act = lib.ti_selftest_fused_flag_action
+    act.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int64]
+    assert act(1, 0, 1, 100, 32768) == 1          # usable, nothing flagged
+    assert act(0, 0, 1, 100, 32768) == 1          # first use: the probe decides
+    assert act(1, 0, 0, 100, 32768) == 0          # switched off by the caller
+    assert act(-1, 0, 1, 100, 32768) == 0         # the probe said no
+    assert act(1, 0, 1, 32769, 32768) == 0        # more counters than a stream owns
+    # a flagged misplacement is reported whatever else holds, also when the form is switched off meanwhile or the
+    # call would not have used it
+    assert act(1, 1, 1, 100, 32768) == -1
+    assert act(1, 1, 0, 100, 32768) == -1
+    assert act(1, 1, 1, 1 << 40, 32768) == -1
+    assert act(-1, 1, 1, 100, 32768) == -1        # the caller then sees state -1 and reports nothing twice
+    # without a device there is nothing to report
+    lib.ti_fused_splitk_faulted.restype = ctypes.c_int
+    assert lib.ti_fused_splitk_faulted() == 0
+
+
+def test_one_launch_split_k_stream_slots_are_recycled():
+    # eight sets of arrival counters per device: a stream keeps its set, a new stream takes a vacant one, then the
+    # set of a stream that has gone idle; with every stream busy it gets none (two-launch form)
+    import torch_int._CUDA as C
+    lib = ctypes.CDLL(C.LIB_PATH)
+    fn = lib.ti_selftest_fused_slot
+    fn.argtypes = [ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_uint32), ctypes.c_int, ctypes.c_int64,
+                   ctypes.c_uint32, ctypes.POINTER(ctypes.c_int)]
+    table, live, fresh = (ctypes.c_int64 * 8)(), ctypes.c_uint32(0), ctypes.c_int(0)
+
+    def slot(stream, busy):
+        s = fn(table, ctypes.byref(live), 8, stream, busy, ctypes.byref(fresh))
+        return s, fresh.value
+    # the null stream (handle 0) is a stream like any other: it must not match an empty slot
+    assert slot(0, 0) == (0, 1) and live.value == 1
+    assert slot(0, 0) == (0, 0)
+    for i in range(1, 8):
+        assert slot(1000 + i, 0xFF) == (i, 1)
+    assert live.value == 0xFF
+    assert slot(1003, 0xFF) == (3, 0)                     # known stream: its own slot, busy or not
+    assert slot(2000, 0xFF) == (-1, 1)                    # ninth stream, all busy
+    assert slot(2000, 0xFF & ~(1 << 5)) == (5, 1)         # slot 5's stream is idle: handed on
+    assert table[5] == 2000 and slot(2000, 0xFF) == (5, 0)
+    assert slot(1005, 0xFF) == (-1, 1)                    # the stream that lost its slot is a new one now
+    live.value &= ~(1 << 2)                               # a slot given back (probe refused the stream)
+    assert slot(3000, 0xFF) == (2, 1)
+
+
+def test_graph_decoder_refuses_steps_beyond_its_buffers():
+    # Int8OPTGraphDecoder.step guards the device-side cache length: after max_new_tokens steps it raises before
+    # anything is launched (the recorded attention kernel also clamps the length it reads)
+    from torch_int.models.opt import Int8OPTGraphDecoder
+    dec = object.__new__(Int8OPTGraphDecoder)
+    dec.filled, dec.max_length = 40, 40
+    with pytest.raises(RuntimeError, match="max_new_tokens"):
+        dec.step(torch.zeros(1, 1, dtype=torch.long))

@@ -41,6 +41,49 @@ def _sample_rows(M, n=64):
     return torch.cat([torch.arange(0, n), torch.arange(mid, mid + n), torch.arange(M - n, M)])
 
 
+# ------------------------------------------------------------------ all-tile references computed on the device
+
+def _acc_on_device(xd, wd):
+    """x . w^T as int64 through an fp64 product on the device: exact, since every partial sum stays below 2^53.
+    A route that shares nothing with the kernels under test (no int8 matrix instruction, no tiling of theirs)."""
+    return (xd.double() @ wd.double().t()).round().long()
+
+
+def _fma32_on_device(alpha, a32, bt32):
+    """fp32 fma(alpha, a, bt), correctly rounded, from fp64 arithmetic: alpha * a is exact in fp64 (24 x 24 bits); the
+    fp64 sum with bt is rounded to odd (its rounding error from the two-sum identity decides), after which the
+    rounding to fp32 cannot double-round."""
+    p = a32.double() * float(torch.tensor(alpha, dtype=torch.float32))
+    b = bt32.double()
+    r = p + b
+    bb = r - p
+    e = (p - (r - bb)) + (b - bb)                      # exact error of the fp64 sum
+    even = (r.view(torch.int64) & 1) == 0
+    toward = torch.where(e > 0, torch.full_like(r, float("inf")), torch.full_like(r, float("-inf")))
+    r = torch.where((e != 0) & even, torch.nextafter(r, toward), r)
+    return r.float()
+
+
+def _check_every_tile(name, out, xd, wd, bias_d, alpha, beta, chunk=2048):
+    """The whole output against references built on the device from the exact accumulators, row chunk by row chunk:
+    every tile of every kernel family is covered, not only the rows the host oracle can afford."""
+    M = xd.shape[0]
+    for r0 in range(0, M, chunk):
+        acc = _acc_on_device(xd[r0:r0 + chunk], wd)
+        got = out[r0:r0 + chunk]
+        if name == "b32_o32":
+            want = (acc + bias_d.long()).to(torch.int32)   # wraps like the kernel's 32-bit add
+        else:
+            bt = (torch.tensor(beta, dtype=torch.float32, device=acc.device) * bias_d.float())
+            t = _fma32_on_device(alpha, acc.float(), bt.expand_as(acc))
+            if name.startswith("bfp32_ofp32"):
+                want = t
+            else:
+                want = t.round().clamp(0 if name == "relu_b8_o8" else -128, 127).to(torch.int8)
+        nbad = (got != want).sum().item()
+        assert nbad == 0, f"{name}: {nbad} outputs of rows {r0}..{r0 + got.shape[0] - 1} differ from the device-side reference"
+
+
 # ------------------------------------------------------------------ the OPT-13B linear sweep
 
 SWEEP_SHAPES = [(5120, 5120), (20480, 5120), (5120, 20480)]   # (N, K): q/k/v/out_proj, fc1, fc2
@@ -93,6 +136,12 @@ def test_linear_sweep_opt13b(N, K):
             assert nbad == 0, f"{name} {M}x{N}x{K} ({family}): {nbad} of {want.numel()} sampled outputs differ"
             if name == "relu_b8_o8":
                 assert int(out.min()) >= 0
+            if M >= 512:
+                # every tile, not only the sampled rows (the sampled rows tie this reference to the host oracle:
+                # both must equal the kernel's output there)
+                a, b = {"b32_o32": (1.0, 1.0), "bfp32_ofp32 beta=1": (scal["bfp32_ofp32"][0], 1.0)}.get(name) or scal[name]
+                bias_d = b32d if name == "b32_o32" else bfd if name.startswith("bfp32") else b8d
+                _check_every_tile(name, out, xd, wd, bias_d, a, b)
         del xd
 
 
@@ -350,3 +399,111 @@ def test_decoder_layer_opt66b_shape_prefill_and_decode(bsz):
         for name, a, kw, live, res in tap.calls:
             _check_call(name, a, kw, live, res, sample)
     _say("  decode launches seen:", sorted(seen))
+
+
+# ------------------------------------------------------------------ the whole OPT-66B-shaped model
+
+def _bench_opt():
+    import importlib.util
+    import os
+    path = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "torch-int_amd", "benchmark",
+                        "bench_opt.py")
+    spec = importlib.util.spec_from_file_location("ti_bench_opt", path)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
+@torch.no_grad()
+def test_opt66b_causal_lm_at_full_depth():
+    """Int8OPTForCausalLM at the OPT-66B configuration, all 64 layers resident (65 GB of int8 weights generated on
+    the device, vocabulary 50272): batch 4 x 512 prefill + 32 single-token steps, as upstream's tests/test_opt.py:46-58
+    runs its model end to end.
+      * layers 0, 31 and 63: every kernel launch of the prefill and of decode steps 1, 16 and 32 against the oracle
+        on the operands it received;
+      * the same prompt twice gives the same logits and caches, bit for bit;
+      * a 513-token prefill (padded to 528: 2112 rows, tiles with a ragged edge, the three-sweep attention kernel)
+        and the 512-token prefill followed by one decode step (streaming linears, one-launch decode attention) give
+        the same last hidden state for token 513, bit for bit: every fused form claims the bits of the operator
+        chain, and this is where two different sets of them meet."""
+    bo = _bench_opt()
+    dev = torch.device(DEV)
+    _say("OPT-66B, 64 layers: weights")
+    model, cfg = bo.build("opt-66b", 0, dev, seed=3)
+    layers = model.model.decoder.layers
+    assert len(layers) == 64 and cfg.vocab_size == 50272
+    g = torch.Generator().manual_seed(660)
+    bsz, T = 4, 512
+    ids513 = torch.randint(2, cfg.vocab_size, (bsz, T + 1), generator=g).to(dev)
+    ids = ids513[:, :T].contiguous()
+    sample = lambda BH: sorted({0, BH // 3, BH - 1})   # noqa: E731
+    tapped = (0, 31, 63)
+    static = [b for i in tapped for b in layers[i].buffers()]
+    tap = _Tap(static)
+
+    def with_taps(fn):
+        """Runs fn() with the launches of the tapped layers recorded (hooks switch the recorder on and off)."""
+        ctx, hooks = {}, []
+        for i in tapped:
+            def pre(_m, _a, _k=None, i=i):
+                ctx[i] = tap.on()
+                ctx[i].__enter__()
+
+            def post(_m, _a, _o, i=i):
+                ctx.pop(i).__exit__(None, None, None)
+            hooks.append(layers[i].register_forward_pre_hook(pre))
+            hooks.append(layers[i].register_forward_hook(post))
+        try:
+            tap.calls.clear()
+            return fn()
+        finally:
+            for h in hooks:
+                h.remove()
+
+    _say("  prefill 4 x 512, layers 0 / 31 / 63 tapped")
+    out = with_taps(lambda: model(ids, use_cache=True))
+    names = [c[0] for c in tap.calls]
+    assert names.count("attn_prefill") == 3 and names.count("linear_a8_w8_b8_o8_group_heads") == 3, names
+    for name, a, kw, live, res in tap.calls:
+        _check_call(name, a, kw, live, res, sample)
+    assert out.logits.shape == (bsz, T, cfg.vocab_size) and torch.isfinite(out.logits).all()
+    assert len(out.past_key_values) == 64 and out.past_key_values[63][0].shape == (bsz, 72, T, 128)
+    logits_last = out.logits[:, -1].clone()
+    k63 = out.past_key_values[63][0].clone()
+
+    _say("  the same prompt again")
+    again = model(ids, use_cache=True)
+    assert torch.equal(again.logits, out.logits)
+    assert torch.equal(again.past_key_values[63][0], k63) and torch.equal(again.past_key_values[31][1], out.past_key_values[31][1])
+    del again
+
+    _say("  513-token prefill against 512 + one decode step")
+    hid_full = model.model(ids513).last_hidden_state.clone()          # [4, 513, 9216], after the final LayerNorm
+    hid_512 = model.model(ids).last_hidden_state
+    # the first 512 positions of the longer prefill repeat the shorter one (causal: they cannot see token 513)
+    assert torch.equal(hid_full[:, :T], hid_512)
+    step = model.model(ids513[:, T:], past_key_values=out.past_key_values, use_cache=True)
+    assert step.past_key_values[0][0].shape[2] == T + 1
+    assert torch.equal(step.last_hidden_state[:, -1], hid_full[:, -1]), "prefill and decode paths differ in the last hidden state"
+    # (logits are a torch fp32 GEMM outside this library whose summation order depends on the row count, so the
+    # comparison stops at the hidden state that feeds it)
+    del hid_full, hid_512, step
+
+    _say("  32 decode steps")
+    past = out.past_key_values
+    tok = logits_last.argmax(-1, keepdim=True)
+    for s in range(32):
+        if s + 1 in (1, 16, 32):
+            o = with_taps(lambda: model(tok, past_key_values=past, use_cache=True))
+            names = [c[0] for c in tap.calls]
+            assert names.count("decode_attention") == 3 and names.count("linear_a8_w8_b8_o8_group") == 3, names
+            for name, a, kw, live, res in tap.calls:
+                _check_call(name, a, kw, live, res, sample)
+        else:
+            o = model(tok, past_key_values=past, use_cache=True)
+        past = o.past_key_values
+        assert past[0][0].shape[2] == T + s + 1 and torch.isfinite(o.logits).all()
+        tok = o.logits[:, -1].argmax(-1, keepdim=True)
+    _say("  peak memory %.1f GB" % (torch.cuda.max_memory_allocated() / 1e9))
+    del model, out, past
+    torch.cuda.empty_cache()

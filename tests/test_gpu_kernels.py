@@ -283,10 +283,24 @@ def test_large_problems_with_an_inner_dimension_that_16_does_not_divide():
         _say(f"bmm, odd K: B={B} M={M} N={N} K={K}")
         _bmm_case(C, B, M, N, K, seed=300 + i, prob_lhs=i == 0)
         assert C._lib.ti_last_kernel().decode() != "scalar"
-    for variant in ("b8_o8", "bfp32_ofp32"):
+    for variant in ("b8_o8", "bfp32_ofp32", "b32_o32", "relu_b8_o8"):
         _say(f"linear, odd K: {variant}")
         _linear_case(C, variant, 512, 640, 1001, seed=310)
         assert C._lib.ti_last_kernel().decode() != "scalar"
+    # the zero-padded copy of a weight is made once per weight tensor and version: a second call reuses it, a weight
+    # changed in place gets a new one
+    g = torch.Generator().manual_seed(312)
+    x, w, b = _s8(g, 512, 1001), _s8(g, 640, 1001), _s8(g, 640)
+    xd, wd, bd = x.to(DEV), w.to(DEV), b.to(DEV)
+    for _ in range(2):
+        assert torch.equal(C.linear_a8_w8_b8_o8(xd, wd, bd, 0.001, 0.01).cpu(), orc.linear_a8_w8_b8_o8(x, w, b, 0.001, 0.01))
+    assert id(wd) in C._padded
+    w2 = _s8(g, 640, 1001)
+    wd.copy_(w2)
+    assert torch.equal(C.linear_a8_w8_b8_o8(xd, wd, bd, 0.001, 0.01).cpu(), orc.linear_a8_w8_b8_o8(x, w2, b, 0.001, 0.01))
+    key = id(wd)
+    del wd
+    assert key not in C._padded
     _linear_case(C, "b8_o8", 70, 50, 37, seed=311)   # small: the one-thread-per-output kernel as it is
     assert C._lib.ti_last_kernel().decode() == "scalar"
 
@@ -648,6 +662,62 @@ def test_one_launch_split_k_in_a_graph():
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(static_out.cpu(), refs[i]) and torch.equal(eager.cpu(), refs[i]), i
+
+
+def test_one_launch_split_k_needs_a_256_byte_aligned_workspace():
+    # through the C ABI: the waves park and read back 1 KiB regions of the workspace, which must not share a 128-byte
+    # line with a neighbour's; a workspace that is only 16-byte aligned takes the two-launch form, same bytes
+    import ctypes
+    import torch_int._CUDA as C
+    lib = C._lib
+    lib.ti_last_kernel.restype = ctypes.c_char_p
+    g = torch.Generator().manual_seed(103)
+    M, N, K = 256, 2880, 3584
+    x, w, b = _s8(g, M, K).to(DEV), _s8(g, N, K).to(DEV), _s8(g, N).to(DEV)
+    need = lib.ti_linear_workspace_bytes(M, N, K)
+    assert need > 0
+    ws = torch.empty(need + 512, dtype=torch.uint8, device=DEV)
+    base = (ws.data_ptr() + 255) // 256 * 256
+    outs, kernels = [], []
+    for off in (0, 16, 128, 256):
+        _say(f"one-launch split-K, workspace offset {off}")
+        out = torch.empty((M, N), dtype=torch.int8, device=DEV)
+        rc = lib.ti_linear_a8_w8_b8_o8(x.data_ptr(), w.data_ptr(), b.data_ptr(), out.data_ptr(), M, N, K, 0.0013, 0.02,
+                                       base + off, need, torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, lib.ti_last_error()
+        kernels.append(lib.ti_last_kernel().decode())
+        outs.append(out.cpu())
+    assert kernels[0].startswith("fusedk_") and kernels[3].startswith("fusedk_"), kernels
+    assert kernels[1].startswith("splitk_") and kernels[2].startswith("splitk_"), kernels
+    ref = orc.linear_a8_w8_b8_o8(x.cpu(), w.cpu(), b.cpu(), 0.0013, 0.02)
+    for o in outs:
+        assert torch.equal(o, ref)
+    assert lib.ti_fused_splitk_faulted() == 0
+
+
+def test_one_launch_split_k_hands_counter_sets_on_to_new_streams():
+    # more streams than the eight sets of arrival counters a device has: a stream that has gone idle hands its set
+    # on, so every one of twelve streams used one after the other still gets the one-launch form, with exact results
+    import ctypes
+    import torch_int._CUDA as C
+    lib = C._lib
+    lib.ti_last_kernel.restype = ctypes.c_char_p
+    g = torch.Generator().manual_seed(105)
+    M, N, K = 256, 640, 2048
+    x, w, b = _s8(g, M, K).to(DEV), _s8(g, N, K).to(DEV), _s8(g, N).to(DEV)
+    ref = orc.linear_a8_w8_b8_o8(x.cpu(), w.cpu(), b.cpu(), 0.001, 0.01)
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream() for _ in range(12)]
+    for i, st in enumerate(streams):
+        _say("one-launch split-K on stream", i)
+        with torch.cuda.stream(st):
+            out = C.linear_a8_w8_b8_o8(x, w, b, 0.001, 0.01)
+            out2 = C.linear_a8_w8_b8_o8(x, w, b, 0.001, 0.01)
+        kern = lib.ti_last_kernel().decode()
+        st.synchronize()
+        assert kern.startswith("fusedk_"), (i, kern)
+        assert torch.equal(out.cpu(), ref) and torch.equal(out2.cpu(), ref), i
+    assert lib.ti_fused_splitk_faulted() == 0
 
 
 def test_linear_accumulate_into_output(two_launch_split_k):

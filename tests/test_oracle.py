@@ -118,6 +118,57 @@ def test_fp32_epilogue_is_one_fma_of_separately_rounded_bias_term():
     assert n_differs_from_unfused > 0
 
 
+def _rint_half_even(fr):
+    fl = fr.numerator // fr.denominator
+    rem = fr - fl
+    if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and fl % 2 == 1):
+        fl += 1
+    return fl
+
+
+@pytest.mark.parametrize("which", ["b8_o8", "relu_b8_o8", "b32_o32_scaled"])
+def test_integer_output_epilogues_are_one_fma_then_one_rint(which):
+    """The s8, ReLU-s8 and scaled-s32 epilogues against exact rationals: t = fp32(alpha * f32(acc) + fp32(beta * bias))
+    with ONE rounding of the sum (an fma), then round-half-even and the clamp.  The cases are searched for, not drawn:
+    only inputs on which a separately rounded product followed by an add would produce a different integer are kept,
+    so an oracle that slipped to mul + add fails every one of them."""
+    a32, b32 = np.float32(0.0037), np.float32(0.83)
+    if which == "b32_o32_scaled":
+        rng = np.random.default_rng(5)
+        acc = rng.integers(-2 ** 31, 2 ** 31, 400000).astype(np.int64)
+        bias = rng.integers(-2 ** 20, 2 ** 20, acc.size).astype(np.int64)
+    else:  # every accumulator whose scaled value lands in the int8 range, against a spread of int8 bias values
+        acc = np.repeat(np.arange(-36000, 36001, dtype=np.int64), 128)
+        bias = np.tile(np.arange(-127, 128, 2, dtype=np.int64)[:128], acc.size // 128)
+    accf = acc.astype(np.float32)                        # int32 -> fp32, round to nearest even
+    bt = (b32 * bias.astype(np.float32)).astype(np.float32)      # the separately rounded bias term
+    fused = (accf.astype(np.float64) * np.float64(a32) + bt.astype(np.float64)).astype(np.float32)
+    unfused = ((a32 * accf).astype(np.float32) + bt).astype(np.float32)
+    tell = np.nonzero(np.rint(fused.astype(np.float64)) != np.rint(unfused.astype(np.float64)))[0]
+    assert tell.size >= 20, tell.size            # the search found inputs that tell the two forms apart
+    tell = tell[:300]
+    acc_t = torch.from_numpy(acc[tell].astype(np.int32)).view(1, -1)
+    if which == "b32_o32_scaled":
+        out = orc.epi_b32_o32_scaled(acc_t, torch.from_numpy(bias[tell].astype(np.int32)), float(a32), float(b32))[0]
+    else:
+        out = orc.epi_b8_o8(acc_t, torch.from_numpy(bias[tell].astype(np.int8)), float(a32), float(b32),
+                            relu=which == "relu_b8_o8")[0]
+    n_unfused_differs = 0
+    for j, i in enumerate(tell):
+        bb = Fraction(float(bt[i]))
+        t = Fraction(_round_to_f32(Fraction(float(a32)) * Fraction(float(accf[i])) + bb))   # the one rounding of the fma
+        if which == "b32_o32_scaled":
+            want = max(min(_rint_half_even(t), 2 ** 31 - 1), -2 ** 31)
+            other = max(min(int(np.rint(np.float64(unfused[i]))), 2 ** 31 - 1), -2 ** 31)
+        else:
+            lo = 0 if which == "relu_b8_o8" else -128
+            want = max(min(_rint_half_even(t), 127), lo)
+            other = max(min(int(np.rint(np.float64(unfused[i]))), 127), lo)
+        assert out[j].item() == want, (which, int(acc[i]), int(bias[i]))
+        n_unfused_differs += int(other != want)
+    assert n_unfused_differs > 0
+
+
 def test_int_to_float_conversion_rounds_to_nearest_even():
     acc = torch.tensor([2 ** 24 + 1, 2 ** 24 + 3, -(2 ** 24 + 1), 2 ** 31 - 1, -2 ** 31], dtype=torch.int32)
     out = orc.epi_f32t(acc, 1.0)

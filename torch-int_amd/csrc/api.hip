@@ -145,6 +145,7 @@ int ti_init(void) {
 }
 
 int64_t ti_linear_workspace_bytes(int64_t M, int64_t N, int64_t K) { return gemm_workspace_bytes(M, N, K); }
+int ti_linear_row_split(int64_t M, int64_t N, int64_t K) { return gemm_row_split(M, N, K); }
 
 int ti_linear_a8_w8_b32_o32(const int8_t* x, const int8_t* w, const int32_t* bias, int32_t* out, int64_t M,
                             int64_t N, int64_t K, void* ws, int64_t ws_bytes, void* stream) {
@@ -410,6 +411,16 @@ int ti_attn_softmax_q(const float* scores, const float* mask, int8_t* probs, int
 const char* ti_last_kernel(void) { return last_gemm_kernel(); }
 
 int ti_fused_splitk(int enable) { return set_fused_split(enable); }
+int ti_fused_splitk_faulted(void) { return fused_split_faulted(); }
+int ti_selftest_fused_flag_action(int state, int flag, int enabled, int64_t counters, int64_t max_counters) {
+  return fused_flag_action(state, flag, enabled != 0, counters, max_counters);
+}
+int ti_selftest_fused_slot(int64_t* table, uint32_t* live_mask, int cap, int64_t stream, uint32_t busy_mask,
+                           int* fresh) {
+  static_assert(sizeof(long long) == sizeof(int64_t) && sizeof(unsigned) == sizeof(uint32_t), "plain forwards");
+  return fused_slot_for_test(reinterpret_cast<long long*>(table), reinterpret_cast<unsigned*>(live_mask), cap, stream,
+                             busy_mask, fresh);
+}
 
 int64_t ti_diag_mfma_loop_ops(int64_t iters) { return iters > 0 ? diag_mfma_loop_ops(iters) : 0; }
 

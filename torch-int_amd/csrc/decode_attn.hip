@@ -50,7 +50,14 @@ __global__ __launch_bounds__(256) void decode_attn_kernel(const int8_t* __restri
                                                           float alpha_pv, const int* __restrict__ s_dev) {
   // s_dev != nullptr: the number of positions is read from device memory (a launch recorded in a HIP graph is
   // replayed for a cache that has grown meanwhile; S_arg is then the largest length the launch was sized for)
-  const int S = s_dev != nullptr ? s_dev[0] : S_arg;
+  // (clamped to the contract T <= length <= S_arg: the host cannot check a value it never sees, and a length
+  // outside that range would index past the LDS score rows and the cache buffers)
+  int S = S_arg;
+  if (s_dev != nullptr) {
+    S = s_dev[0];
+    S = S < T ? T : S;
+    S = S > S_arg ? S_arg : S;
+  }
   constexpr int LPR = D / 16;    // lanes per cache row
   constexpr int RPW = 64 / LPR;  // rows per wave per load
   extern __shared__ __attribute__((aligned(16))) char smem[];

@@ -9,6 +9,10 @@
 namespace ti {
 
 long long gemm_workspace_bytes(long long M, long long N, long long K) {
+  if (M > 1024) {  // the rows beyond the last multiple of 256 as a small problem of their own (row_split_rows)
+    long long need = 0;
+    return row_split_rows(M, N, K, &need) > 0 ? need : 0;
+  }
   const int s = choose_splits(M, N, K);
   return s > 1 ? (long long)s * M * N * 4 : 0;
 }
@@ -23,6 +27,8 @@ int launch_gemm_kind_5(const GemmParams& p, void* ws, long long ws_bytes, hipStr
 int launch_gemm_kind_6(const GemmParams& p, void* ws, long long ws_bytes, hipStream_t stream);
 int launch_gemm_kind_7(const GemmParams& p, void* ws, long long ws_bytes, hipStream_t stream);
 int launch_gemm_kind_8(const GemmParams& p, void* ws, long long ws_bytes, hipStream_t stream);
+
+int gemm_row_split(long long M, long long N, long long K) { return row_split_rows(M, N, K); }
 
 thread_local const char* g_last_kernel = "";
 const char* last_gemm_kernel() { return g_last_kernel; }
@@ -57,7 +63,8 @@ struct FusedDevice {
   int* host_words = nullptr;  // [0] = the misplacement flag, [1 .. 256] = the probe's output
   int* host_words_dev = nullptr;
   hipStream_t streams[kFusedStreams] = {};
-  int nstreams = 0;
+  bool live[kFusedStreams] = {};
+  bool pinned[kFusedStreams] = {};  // a launch with this slot's counters was recorded into a graph: never handed on
 };
 static FusedDevice g_fused[64];
 
@@ -81,61 +88,171 @@ static bool fused_enabled() { return set_fused_split(-1) != 0; }
 static thread_local bool g_fused_may_probe = true;
 void allow_fused_split_probe(bool allow) { g_fused_may_probe = allow; }
 
-// counters < 0: only make the current device ready (the probe), on `stream`
-int fused_split_prepare(hipStream_t stream, long long counters, GemmParams& q) {
-  if (!fused_enabled() || counters > kFusedCounters) return 0;
+// Runs the placement probe on `stream` (which must not be capturing) and waits for it: true when the 256 probe
+// workgroups show one XCC per residue class of the workgroup id mod 8, eight different ones.
+static bool probe_placement(FusedDevice& d, hipStream_t stream) {
+  for (int i = 0; i < 256; ++i) d.host_words[1 + i] = -1;
+  hipLaunchKernelGGL(xcc_probe_kernel, dim3(256), dim3(64), 0, stream, reinterpret_cast<unsigned*>(d.host_words_dev + 1));
+  if (hipGetLastError() != hipSuccess || hipStreamSynchronize(stream) != hipSuccess) return false;
+  unsigned seen = 0;
+  for (int i = 0; i < 256; ++i) {
+    const int xcc = d.host_words[1 + i];
+    if (xcc < 0 || xcc > 15 || xcc != d.host_words[1 + (i & 7)]) return false;
+  }
+  for (int i = 0; i < 8; ++i) {
+    const unsigned xcc = (unsigned)d.host_words[1 + i];
+    if (seen & (1u << xcc)) return false;  // two residue classes on one XCD: not the placement this needs
+    seen |= 1u << xcc;
+  }
+  return true;
+}
+
+static bool is_capturing(hipStream_t stream) {
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &capturing) != hipSuccess) {
+    (void)hipGetLastError();
+    return true;  // unknown: treat as capturing (no probe, no registration)
+  }
+  return capturing != hipStreamCaptureStatusNone;
+}
+
+// 1 when a one-launch split-K GEMM on the current device has found a workgroup on an unexpected XCD (the output of
+// that call cannot be trusted), 0 otherwise.  Reads one word of host memory; meaningful once the launches in
+// question have finished.
+int fused_split_faulted() {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
   FusedDevice& d = g_fused[dev];
   std::lock_guard<std::mutex> guard(d.lock);
+  return d.host_words != nullptr && *reinterpret_cast<volatile int*>(d.host_words) != 0 ? 1 : 0;
+}
+
+// Decision logic of the fused form's bookkeeping, free of HIP calls so that it can be tested on the CPU.
+// `flag` is the misplacement word, `state` the device state (0 not probed, 1 usable, -1 off).  Returns the action:
+//   0 = take the two-launch form, 1 = go on (probe / slot lookup), -1 = report the misplacement and switch off.
+int fused_flag_action(int state, int flag, bool enabled, long long counters, long long max_counters) {
+  if (flag != 0 && state != 0) return -1;  // reported by whichever GEMM call comes next, fused or not
+  if (!enabled || counters > max_counters) return 0;
+  if (state < 0) return 0;
+  return 1;
+}
+
+// Slot of `stream` among the `cap` slots of a device (`live[i]` = slot i holds a registered stream, `busy(i)` =
+// that stream still has work queued): the stream's own slot, else a vacant one, else the first whose stream is
+// idle (its counters are zero again: every launch leaves them zero), else -1.  `fresh` is set when the stream was
+// not registered before.  Free of HIP calls so that it can be tested on the CPU.
+template <class Busy>
+static int pick_stream_slot(hipStream_t* streams, bool* live, int cap, hipStream_t stream, Busy busy, bool& fresh) {
+  fresh = false;
+  for (int i = 0; i < cap; ++i)
+    if (live[i] && streams[i] == stream) return i;
+  fresh = true;
+  int slot = -1;
+  for (int i = 0; i < cap && slot < 0; ++i)
+    if (!live[i]) slot = i;
+  for (int i = 0; i < cap && slot < 0; ++i)
+    if (!busy(i)) slot = i;
+  if (slot >= 0) {
+    streams[slot] = stream;
+    live[slot] = true;
+  }
+  return slot;
+}
+
+// CPU-testable face of pick_stream_slot: streams are plain integers, bit i of live_mask / busy_mask describes
+// slot i; returns the slot and updates table / live_mask.
+int fused_slot_for_test(long long* table, unsigned* live_mask, int cap, long long stream, unsigned busy_mask,
+                        int* fresh) {
+  hipStream_t tmp[32];
+  bool live[32];
+  if (cap > 32) cap = 32;
+  for (int i = 0; i < cap; ++i) {
+    tmp[i] = reinterpret_cast<hipStream_t>(table[i]);
+    live[i] = (*live_mask >> i) & 1u;
+  }
+  bool f = false;
+  const int slot = pick_stream_slot(tmp, live, cap, reinterpret_cast<hipStream_t>(stream),
+                                    [&](int i) { return ((busy_mask >> i) & 1u) != 0; }, f);
+  *live_mask = 0;
+  for (int i = 0; i < cap; ++i) {
+    table[i] = reinterpret_cast<long long>(tmp[i]);
+    if (live[i]) *live_mask |= 1u << i;
+  }
+  *fresh = f ? 1 : 0;
+  return slot;
+}
+
+static const char* kMisplacedMsg =
+    "an earlier one-launch split-K GEMM on this device found a workgroup on an unexpected XCD and its result cannot "
+    "be trusted (re-run it); the form is now switched off (TORCH_INT_FUSED_SPLITK=0 avoids it from the start)";
+
+// Reports (once) a misplacement that an earlier fused launch on the current device flagged: TI_OK or TI_ERR_LAUNCH.
+// Called at the start of every GEMM launch, whatever kernel it will take.
+int fused_split_check() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return TI_OK;
+  FusedDevice& d = g_fused[dev];
+  if (d.host_words == nullptr) return TI_OK;  // never used here (written under the lock, before any fused launch)
+  std::lock_guard<std::mutex> guard(d.lock);
+  if (d.state == 1 && *reinterpret_cast<volatile int*>(d.host_words) != 0) {
+    d.state = -1;
+    return fail(TI_ERR_LAUNCH, "%s", kMisplacedMsg);
+  }
+  return TI_OK;
+}
+
+// counters == 0: only make the current device and `stream` ready (the probe)
+int fused_split_prepare(hipStream_t stream, long long counters, GemmParams& q) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+  FusedDevice& d = g_fused[dev];
+  std::lock_guard<std::mutex> guard(d.lock);
+  const int flag = d.host_words != nullptr ? *reinterpret_cast<volatile int*>(d.host_words) : 0;
+  const int action = fused_flag_action(d.state, flag, fused_enabled(), counters, kFusedCounters);
+  if (action < 0) {
+    if (d.state == 1) {
+      d.state = -1;
+      return -fail(TI_ERR_LAUNCH, "%s", kMisplacedMsg);
+    }
+    return 0;  // already reported
+  }
+  if (action == 0) return 0;
+  bool probed_now = false;  // the device's first probe ran on `stream` just now and vouches for it
   if (d.state == 0) {
     if (!g_fused_may_probe) return 0;
     // first use on this device: not while the stream records a graph (the probe allocates and synchronises)
-    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(stream, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
-      (void)hipGetLastError();
-      return 0;
-    }
+    if (is_capturing(stream)) return 0;
     d.state = -1;
     void* sym = nullptr;
     if (hipGetSymbolAddress(&sym, HIP_SYMBOL(g_fused_arrivals)) != hipSuccess || sym == nullptr) return 0;
-    if (hipHostMalloc(reinterpret_cast<void**>(&d.host_words), 257 * sizeof(int), hipHostMallocMapped) != hipSuccess)
+    if (hipHostMalloc(reinterpret_cast<void**>(&d.host_words), 257 * sizeof(int), hipHostMallocMapped) != hipSuccess) {
+      d.host_words = nullptr;
       return 0;
+    }
+    d.host_words[0] = 0;
     if (hipHostGetDevicePointer(reinterpret_cast<void**>(&d.host_words_dev), d.host_words, 0) != hipSuccess)
       return 0;
-    for (int i = 0; i < 257; ++i) d.host_words[i] = -1;
-    d.host_words[0] = 0;
-    hipLaunchKernelGGL(xcc_probe_kernel, dim3(256), dim3(64), 0, stream,
-                       reinterpret_cast<unsigned*>(d.host_words_dev + 1));
-    if (hipGetLastError() != hipSuccess || hipStreamSynchronize(stream) != hipSuccess) return 0;
-    unsigned seen = 0;
-    for (int i = 0; i < 256; ++i) {
-      const int xcc = d.host_words[1 + i];
-      if (xcc < 0 || xcc > 15 || xcc != d.host_words[1 + (i & 7)]) return 0;
-    }
-    for (int i = 0; i < 8; ++i) {
-      const unsigned xcc = (unsigned)d.host_words[1 + i];
-      if (seen & (1u << xcc)) return 0;  // two residue classes on one XCD: not the placement this needs
-      seen |= 1u << xcc;
-    }
+    if (!probe_placement(d, stream)) return 0;
     d.arrivals = static_cast<int*>(sym);
     d.state = 1;
+    probed_now = true;
   }
-  if (d.state != 1) return 0;
-  if (*reinterpret_cast<volatile int*>(d.host_words) != 0) {
-    d.state = -1;  // a workgroup of an earlier fused launch ran on an unexpected XCD: its result cannot be trusted
-    return -fail(TI_ERR_LAUNCH, "an earlier one-launch split-K GEMM found a workgroup on an unexpected XCD and its "
-                                "result cannot be trusted; the form is now switched off (TORCH_INT_FUSED_SPLITK=0 "
-                                "avoids it from the start)");
-  }
-  if (counters < 0) return 1;
-  int slot = -1;
-  for (int i = 0; i < d.nstreams; ++i)
-    if (d.streams[i] == stream) slot = i;
-  if (slot < 0) {
-    if (d.nstreams == kFusedStreams) return 0;
-    slot = d.nstreams++;
-    d.streams[slot] = stream;
+  bool fresh = false;
+  const int slot = pick_stream_slot(d.streams, d.live, kFusedStreams, stream,
+                                    [&](int i) { return d.pinned[i] || hipStreamQuery(d.streams[i]) == hipErrorNotReady; },
+                                    fresh);
+  (void)hipGetLastError();  // a query of a destroyed stream leaves an error behind; the slot counts as idle
+  if (slot < 0) return 0;
+  if (fresh && !probed_now) {
+    // a stream seen for the first time: the XCD on which its workgroup 0 starts may differ, and a stream made with
+    // a CU mask may not deal workgroups out this way at all, so the probe runs on it once (it synchronises the
+    // stream, so not during a capture or from a caller that must not wait: the slot is given back then)
+    if (!g_fused_may_probe || is_capturing(stream) || !probe_placement(d, stream)) {
+      d.live[slot] = false;
+      return 0;
+    }
+  } else if (!d.pinned[slot] && is_capturing(stream)) {
+    d.pinned[slot] = true;  // the recording keeps these counters for as long as the graph lives
   }
   q.arrivals = d.arrivals + (long long)slot * (kFusedCounters + kFusedTiles);
   q.xcc_seen = reinterpret_cast<unsigned*>(q.arrivals + kFusedCounters);
@@ -145,7 +262,7 @@ int fused_split_prepare(hipStream_t stream, long long counters, GemmParams& q) {
 
 int warm_fused_split(void* stream) {
   GemmParams unused;
-  const int rc = fused_split_prepare(static_cast<hipStream_t>(stream), -1, unused);
+  const int rc = fused_split_prepare(static_cast<hipStream_t>(stream), 0, unused);
   return rc > 0 ? 1 : 0;
 }
 
@@ -232,6 +349,7 @@ int launch_gemm_group_s8(const GemmParams& shape, const GemmGroup& grp, hipStrea
 
 int launch_gemm(int kind, const GemmParams& p, void* ws, long long ws_bytes, hipStream_t stream) {
   if (p.M == 0 || p.N == 0 || p.batch == 0) return TI_OK;
+  if (int rc = fused_split_check()) return rc;
   switch (kind) {
     case EPI_S32_BIAS: return launch_gemm_kind_0(p, ws, ws_bytes, stream);
     case EPI_S32_SCALED: return launch_gemm_kind_1(p, ws, ws_bytes, stream);

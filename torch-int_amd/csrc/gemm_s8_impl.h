@@ -19,6 +19,7 @@
 //     of a half-wave store 128 contiguous bytes of 32-bit results.
 #pragma once
 #include <atomic>
+#include <cstdio>
 #include <cstdlib>
 #include <type_traits>
 #include "ti_common.h"
@@ -2135,8 +2136,9 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmParams p, const 
 // (512x5120x20480: 79 against 64 us).  More than three LDS stages did not help it (four to six: +1 to +3 %).
 enum SplitTile { SPLIT_128 = 0, SPLIT_256 = 1, SPLIT_256x160 = 2, SPLIT_256x288 = 3, SPLIT_128x160 = 4, SPLIT_128x288 = 5,
                  SPLIT_128x80 = 6 };
-static int choose_splits(long long M, long long N, long long K, int* tile_kind = nullptr) {
+static int choose_splits(long long M, long long N, long long K, int* tile_kind = nullptr, double* time_us = nullptr) {
   if (tile_kind) *tile_kind = SPLIT_128;
+  if (time_us) *time_us = -1.0;  // no estimate
   if (M <= 16 || M > 1024 || K % PBK != 0 || K < 1024) return 1;
   const double cus = num_cus();
   const long long steps = K / PBK;
@@ -2204,6 +2206,7 @@ static int choose_splits(long long M, long long N, long long K, int* tile_kind =
     }
   }
   if (tile_kind) *tile_kind = best_kind;
+  if (time_us && best_t < 1e29) *time_us = best_t;
   return best;
 }
 
@@ -2238,6 +2241,83 @@ static int launch_fused(const GemmParams& q_in, hipStream_t stream) {
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "gemm launch: %s", hipGetErrorString(e));
   return TI_OK;
+}
+
+// Tiles of 256 rows for a linear or batched product with M, N > 128: 256x256 (32x32 blocks), or 256x160 /
+// 256x288 / 256x128 (16x16 blocks) when the width divides and they fill the CUs more evenly (2048x5120: 160 tiles
+// of 256x256 but 256 of 256x160; 2048x9216: 288 tiles of 256x256 = two rounds, but exactly 256 of 256x288;
+// 2048x4096: 128 of 256x256 but 256 of 256x128).  Each candidate is priced as its rate relative to the 256x256
+// kernel at full occupancy, measured (128-byte steps: 0.94 for 256x160 with its three LDS stages, 0.95 for 256x288,
+// 0.93 for 256x128; 64-byte steps, K not a multiple of 128: 0.78 and 0.9), times the share of CU rounds its tiles
+// fill (useful outputs over the outputs the rounds of a tiling have room for: partial tiles and partial rounds both
+// count as waste; batched products count tiles only, they are bound by HBM, where padding costs no bytes).  The
+// 128x128 kernel (64-byte steps, two stages) runs at half that rate per CU, a little more with two workgroups on
+// every CU, and takes over where few tiles of 256 rows would leave most CUs idle.
+enum WideTile { WIDE_NONE = 0, WIDE_256x160, WIDE_256x288, WIDE_256x128, WIDE_256x256 };
+struct WidePick {
+  int tile;       // WideTile; WIDE_NONE = leave it to the 128x128 / small-tile kernels
+  double eff;     // efficiency of the choice relative to the 256x256 kernel on a full chip (0 for WIDE_NONE)
+};
+static WidePick pick_wide(long long M, long long N, long long K, long long batch) {
+  const long long cus = num_cus();
+  const long long t256 = ((M + 255) / 256) * ((N + 255) / 256) * batch;
+  const long long t128 = ((M + 127) / 128) * ((N + 127) / 128) * batch;
+  auto fill = [&](long long tiles, int bn) {
+    const double room = (double)(((tiles + cus - 1) / cus) * cus);
+    return batch == 1 ? (double)M * N / (room * 256.0 * bn) : (double)tiles / room;
+  };
+  const long long rows256 = (M + 255) / 256;
+  const bool wide_step = K % QBK == 0;
+  const double f160 = wide_step ? 0.94 : 0.78;
+  const double f288 = wide_step ? 0.95 : 0.9;
+  const double e256 = fill(t256, 256);
+  const double e160 = N % 160 == 0 ? f160 * fill(rows256 * (N / 160) * batch, 160) : 0.0;
+  const double e288 = N % 288 == 0 ? f288 * fill(rows256 * (N / 288) * batch, 288) : 0.0;
+  // The 256x128 tiles and the comparison with the 128x128 kernel are for linears with a K of some length
+  // (the rates above were measured at K >= 4096; at K = 768 the 128x128 kernel's short prologue wins); batched
+  // products keep their tuned 256x256 / 128x128 choice, they are bound by HBM, not by the matrix pipe.
+  const bool priced = batch == 1 && K >= 2048 && t128 >= 128;
+  const double e128w = priced && wide_step && N % 128 == 0 ? 0.93 * fill(rows256 * (N / 128), 128) : 0.0;
+  const double e128 = t128 >= 2 * cus ? 0.6 : t128 >= cus ? 0.47 : 0.47 * (double)t128 / (double)cus;
+  const double best = e256 > e160 ? (e256 > e288 ? (e256 > e128w ? e256 : e128w) : (e288 > e128w ? e288 : e128w))
+                                  : (e160 > e288 ? (e160 > e128w ? e160 : e128w) : (e288 > e128w ? e288 : e128w));
+  if (!(t256 >= 160 || (priced && best > e128))) return WidePick{WIDE_NONE, 0.0};
+  if (e160 > e256 && e160 >= e288 && e160 >= e128w) return WidePick{WIDE_256x160, e160};
+  if (e288 > e256 && e288 >= e128w) return WidePick{WIDE_256x288, e288};
+  if (e128w > e256) return WidePick{WIDE_256x128, e128w};
+  return WidePick{WIDE_256x256, e256};
+}
+
+// Rows to cut off the end of a linear with many rows and run as a second, small problem (0 = none).
+// A tiled GEMM pays for whole tiles and whole rounds of 256 CUs: 2112 rows (a 4 x 528-token prefill; prefill lengths
+// are padded to 16, not to 256) are nine row tiles where 2048 rows are eight, 288 tiles of 256x160 instead of 256 - a
+// second round for 64 rows.  When the rows beyond the last multiple of 256 are few, the first M - r rows run on the
+// tiling that suits them and the r rows left over as a problem of their own through the split-K forms, if the cost
+// model prices the pair clearly below the whole.  Times in us: a tiling of efficiency e takes M N K / e at the 256x256
+// kernel's rate (0.85 us per 64-byte step and 256 tiles) plus 8 us of fill and epilogue; the small problem is priced
+// by choose_splits (its workspace must have been given), rows <= 16 as weight streaming at 4.5 TB/s.
+static int row_split_rows(long long M, long long N, long long K, long long* rest_ws_bytes = nullptr) {
+  if (rest_ws_bytes) *rest_ws_bytes = 0;
+  const long long r = M % 256;
+  if (M <= 1024 || r == 0 || r > 128 || N <= 128 || K % QBK != 0 || K < 1024) return 0;
+  const WidePick whole = pick_wide(M, N, K, 1), main = pick_wide(M - r, N, K, 1);
+  if (whole.tile == WIDE_NONE || main.tile == WIDE_NONE) return 0;
+  auto tiled_us = [&](long long rows, double eff) {
+    return (double)rows * (double)N * (double)(K / 64) * 0.85 / (65536.0 * (double)num_cus() * eff) + 8.0;
+  };
+  double rest_us = 0.0;
+  long long need = 0;
+  if (r <= 16) {
+    rest_us = (double)N * (double)K / 4.5e6 + 4.0;
+  } else {
+    int tile = 0;
+    const int splits = choose_splits(r, N, K, &tile, &rest_us);
+    if (rest_us < 0.0) return 0;
+    need = splits > 1 ? (long long)splits * r * N * 4 : 0;
+  }
+  if (tiled_us(M - r, main.eff) + rest_us + 3.0 >= 0.95 * tiled_us(M, whole.eff)) return 0;
+  if (rest_ws_bytes) *rest_ws_bytes = need;
+  return (int)r;
 }
 
 template <int KIND>
@@ -2295,6 +2375,27 @@ int launch_kind(const GemmParams& p, void* workspace, long long workspace_bytes,
     if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "gemm launch: %s", hipGetErrorString(e));
     return TI_OK;
   }
+  if (p.batch == 1 && p.lda == p.K && p.ldb == p.K && p.M > 1024) {
+    // many rows, a few of them beyond the last multiple of 256: two problems (see row_split_rows)
+    long long need = 0;
+    const int r = row_split_rows(p.M, p.N, p.K, &need);
+    if (r > 0 && (need == 0 || (workspace != nullptr && workspace_bytes >= need))) {
+      GemmParams head = p;
+      head.M = p.M - r;
+      if (int rc = launch_kind<KIND>(head, workspace, workspace_bytes, stream)) return rc;
+      static thread_local char label[96];
+      const int used = snprintf(label, sizeof(label), "%s+", g_last_kernel);
+      GemmParams rest = p;
+      rest.M = r;
+      rest.A = p.A + (long long)head.M * p.lda;
+      if (p.out_d == 0) rest.C = static_cast<Out*>(p.C) + (long long)head.M * p.N;
+      else rest.m_base = p.m_base + head.M;
+      if (int rc = launch_kind<KIND>(rest, workspace, workspace_bytes, stream)) return rc;
+      if (used > 0 && used < (int)sizeof(label)) snprintf(label + used, sizeof(label) - used, "%s", g_last_kernel);
+      g_last_kernel = label;
+      return TI_OK;
+    }
+  }
   if (p.batch == 1 && p.lda == p.K && p.ldb == p.K) {
     int tile = SPLIT_128;
     const int splits = choose_splits(p.M, p.N, p.K, &tile);
@@ -2325,7 +2426,10 @@ int launch_kind(const GemmParams& p, void* workspace, long long workspace_bytes,
         // and beyond four that tail costs more than the reduction launch it saves (measured: 2 slices -3 to -12 %,
         // 4 slices -3 to -8 %, 7 and 8 slices +3 to +6 %)
         // (256x288 tiles, which spill registers, with two slices only: 512x9216x36864 in four slices 181 against 179 us)
-        if (tall && splits <= (tile == SPLIT_256x288 ? 2 : 4) && p.M % bm == 0 && p.N % bn == 0) {
+        // (a workspace on a 256-byte boundary only: the 1 KiB regions the waves park and read back must not share a
+        // 128-byte line with a neighbour's, or a line fetched for one region could be reused, stale, for the next)
+        if (tall && splits <= (tile == SPLIT_256x288 ? 2 : 4) && p.M % bm == 0 && p.N % bn == 0 &&
+            (reinterpret_cast<uintptr_t>(workspace) & 255) == 0) {
           const long long tiles = (long long)(p.M / bm) * (p.N / bn);
           GemmParams f = p;
           f.K = p.K / splits;
@@ -2384,58 +2488,29 @@ int launch_kind(const GemmParams& p, void* workspace, long long workspace_bytes,
     // a 256-wide tile on a narrow or short output would mostly multiply padding
     const bool wide = p.N > 128 && p.M > 128;
     if (wide) {
-      // Tiles of 256 rows: 256x256 (32x32 blocks), or 256x160 / 256x288 / 256x128 (16x16 blocks) when the width
-      // divides and they fill the CUs more evenly (2048x5120: 160 tiles of 256x256 but 256 of 256x160; 2048x9216:
-      // 288 tiles of 256x256 = two rounds, but exactly 256 of 256x288; 2048x4096: 128 of 256x256 but 256 of
-      // 256x128).  Each candidate is priced as its rate relative to the 256x256 kernel at full occupancy, measured
-      // (128-byte steps: 0.94 for 256x160 with its three LDS stages, 0.95 for 256x288, 0.93 for 256x128; 64-byte
-      // steps, K not a multiple of 128: 0.78 and 0.9), times the share of CU rounds its tiles fill.  The 128x128
-      // kernel (64-byte steps, two stages) runs at half that rate per CU, a little more with two workgroups on
-      // every CU, and takes over where few tiles of 256 rows would leave most CUs idle.
-      // Measured with this rule against the one before it, which looked at the count of 256x256 tiles only and sent
-      // everything under 160 of them to the 128x128 kernel: 1600x5120x20480 290 -> 161 us, 1600x5120x5120 76 -> 47,
-      // 2048x4096x4096 48 -> 35, 2048x4096x16384 170 -> 118, 2048x2560x2560 25 -> 20, 2048x12288x12288 285 -> 253.
-      const long long cus = num_cus();
-      // useful outputs over the outputs the CU rounds of a tiling have room for (partial tiles and partial rounds
-      // both count as waste)
-      // (batched products count tiles only, as they always did: they are bound by HBM, where padding costs no bytes)
-      auto fill = [&](long long tiles, int bn) {
-        const double room = (double)(((tiles + cus - 1) / cus) * cus);
-        return p.batch == 1 ? (double)p.M * p.N / (room * 256.0 * bn) : (double)tiles / room;
-      };
-      const long long rows256 = (p.M + 255) / 256;
+      // Measured with pick_wide's rule against the one before it, which looked at the count of 256x256 tiles only and
+      // sent everything under 160 of them to the 128x128 kernel: 1600x5120x20480 290 -> 161 us, 1600x5120x5120
+      // 76 -> 47, 2048x4096x4096 48 -> 35, 2048x4096x16384 170 -> 118, 2048x2560x2560 25 -> 20, 2048x12288x12288
+      // 285 -> 253.
       const bool wide_step = p.K % QBK == 0;
-      const double f160 = wide_step ? 0.94 : 0.78;
-      const double f288 = wide_step ? 0.95 : 0.9;
-      const double e256 = fill(t256, 256);
-      const double e160 = p.N % 160 == 0 ? f160 * fill(rows256 * (p.N / 160) * p.batch, 160) : 0.0;
-      const double e288 = p.N % 288 == 0 ? f288 * fill(rows256 * (p.N / 288) * p.batch, 288) : 0.0;
-      // The 256x128 tiles and the comparison with the 128x128 kernel are for linears with a K of some length
-      // (the rates above were measured at K >= 4096; at K = 768 the 128x128 kernel's short prologue wins); batched
-      // products keep their tuned 256x256 / 128x128 choice, they are bound by HBM, not by the matrix pipe.
-      const bool priced = p.batch == 1 && p.K >= 2048 && t128 >= 128;
-      const double e128w = priced && wide_step && p.N % 128 == 0 ? 0.93 * fill(rows256 * (p.N / 128), 128) : 0.0;
-      const double e128 = t128 >= 2 * cus ? 0.6 : t128 >= cus ? 0.47 : 0.47 * (double)t128 / (double)cus;
-      const double best = e256 > e160 ? (e256 > e288 ? (e256 > e128w ? e256 : e128w) : (e288 > e128w ? e288 : e128w))
-                                      : (e160 > e288 ? (e160 > e128w ? e160 : e128w) : (e288 > e128w ? e288 : e128w));
-      if (t256 >= 160 || (priced && best > e128)) {
-        if (e160 > e256 && e160 >= e288 && e160 >= e128w) {
+      switch (pick_wide(p.M, p.N, p.K, p.batch).tile) {
+        case WIDE_256x160:
           g_last_kernel = "pipe16_256x160";
           if (wide_step) return launch_pipe16q<Pipe16QCfg<256, 160, 4, 2, KIND>>(p, stream);
           return launch_pipe16<Pipe16Cfg<256, 160, 4, 2, 5, KIND>>(p, stream);
-        }
-        if (e288 > e256 && e288 >= e128w) {
+        case WIDE_256x288:
           g_last_kernel = "pipe16_256x288";
           if (wide_step) return launch_pipe16q<Pipe16QCfg<256, 288, 4, 2, KIND>>(p, stream);
           return launch_pipe16<Pipe16Cfg<256, 288, 4, 2, 4, KIND>>(p, stream);
-        }
-        if (e128w > e256) {
+        case WIDE_256x128:
           g_last_kernel = "pipe16_256x128";
           return launch_pipe16q<Pipe16QCfg<256, 128, 4, 2, KIND>>(p, stream);
-        }
-        g_last_kernel = "pipe_256x256";
-        if (p.K % QBK == 0) return launch_pipe2<Pipe2Cfg<256, 256, 2, 4, KIND, SWAP>>(p, stream);  // whole cache lines per row
-        return launch_pipe<PipeCfg<256, 256, 2, 4, 4, KIND, SWAP>>(p, stream);
+        case WIDE_256x256:
+          g_last_kernel = "pipe_256x256";
+          if (wide_step) return launch_pipe2<Pipe2Cfg<256, 256, 2, 4, KIND, SWAP>>(p, stream);  // whole cache lines per row
+          return launch_pipe<PipeCfg<256, 256, 2, 4, 4, KIND, SWAP>>(p, stream);
+        default:
+          break;
       }
     }
     // 128-wide outputs with many rows (P.V of a long prefill): 256x128 tiles, three stages of 128-byte steps

@@ -177,6 +177,9 @@ struct GemmParams {
   // stored as element [b][h][t][dd] of a packed [M/out_T, N/out_d, out_T, out_d] tensor -- the layout the
   // attention products want, written by the projection itself.  0 = plain row-major [M, N].  8-bit outputs only.
   int out_T = 0, out_d = 0;
+  // Head-major output of a problem that is the last rows of a larger one: row m of this problem is row m + m_base
+  // of the whole (plain row-major output needs no such field: C points at the first row).
+  int m_base = 0;
   // Tile rows an XCD's run of tiles walks down before it moves to the next tile column (see tile_of_workgroup).
   int band = 8;
   // gemm_pipe_kernel: all tiles of a batch on one XCD (see decode_item there)
@@ -196,6 +199,7 @@ struct GemmParams {
 // stores of VEC columns starting at a multiple of VEC are unaffected when out_d % VEC == 0.
 __device__ __forceinline__ long long out_index(const GemmParams& p, int m, int n) {
   if (p.out_d == 0) return (long long)m * p.N + n;
+  m += p.m_base;
   const int b = m / p.out_T, t = m - b * p.out_T;
   const int h = n / p.out_d, dd = n - h * p.out_d;
   return (((long long)b * (p.N / p.out_d) + h) * p.out_T + t) * p.out_d + dd;
@@ -216,8 +220,12 @@ int launch_gemm_group_s8(const GemmParams& shape, const GemmGroup& grp, hipStrea
 int launch_gemm(int kind, const GemmParams& p, void* workspace, long long workspace_bytes,
                 hipStream_t stream);
 long long gemm_workspace_bytes(long long M, long long N, long long K);
+int gemm_row_split(long long M, long long N, long long K);  // rows a linear cuts off its end and runs as a second problem
 void allow_fused_split_probe(bool allow);  // per thread: may a GEMM call run the one-time placement probe?
 int warm_fused_split(void* stream);        // run that probe now (1 = the one-launch split-K is usable on this device)
+int fused_split_faulted();                 // 1 = a one-launch split-K on the current device flagged a misplaced workgroup
+int fused_flag_action(int state, int flag, bool enabled, long long counters, long long max_counters);
+int fused_slot_for_test(long long* table, unsigned* live_mask, int cap, long long stream, unsigned busy_mask, int* fresh);
 int set_fused_split(int enable);  // one-launch split-K on (1) / off (0) / unchanged (-1); returns the previous setting
 const char* last_gemm_kernel();  // kernel family of the calling thread's last launch_gemm ("" before the first)
 

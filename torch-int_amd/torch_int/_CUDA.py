@@ -11,6 +11,7 @@ library or a missing GPU raise instead of silently computing elsewhere.
 """
 import ctypes
 import os
+import weakref
 
 import torch
 
@@ -153,7 +154,7 @@ def _workspace(dev_index, stream, nbytes):
     return ws.data_ptr(), ws.numel()
 
 
-def _pad_inner(a, b, K, macs):
+def _pad_inner(a, b, K, macs, weight=False):
     """Operands whose inner dimension is not a multiple of 16 have no aligned rows for the tiled kernels, and the
     library then runs a one-thread-per-output kernel (40 x 1500 x 128 x 1500: 32 ms).  From a size at which that
     hurts, both operands are copied with K padded by zeros to a multiple of 64 first: the added products are zero,
@@ -161,7 +162,24 @@ def _pad_inner(a, b, K, macs):
     if K % 16 == 0 or macs < (1 << 26):
         return a, b, K
     pad = -K % 64
-    return torch.nn.functional.pad(a, (0, pad)), torch.nn.functional.pad(b, (0, pad)), K + pad
+    return torch.nn.functional.pad(a, (0, pad)), _padded_weight(b, pad) if weight else torch.nn.functional.pad(b, (0, pad)), K + pad
+
+
+_padded = {}  # id(weight) -> (weak reference, version counter, padded copy)
+
+
+def _padded_weight(w, pad):
+    """The zero-padded copy of a linear's weight, made once per weight tensor and version (a module calls with the
+    same tensor object every time) instead of once per forward.  Entries go when their tensor does."""
+    key = id(w)
+    hit = _padded.get(key)
+    if hit is not None and hit[0]() is w and hit[1] == w._version and hit[2].shape[1] == w.shape[1] + pad:
+        return hit[2]
+    if len(_padded) >= 256:
+        _padded.clear()
+    padded = torch.nn.functional.pad(w, (0, pad))
+    _padded[key] = (weakref.ref(w, lambda _r, k=key: _padded.pop(k, None)), w._version, padded)
+    return padded
 
 
 def _linear(op, kind, x, w, bias, bias_dtype, out_dtype, alpha, beta, inout=None):
@@ -195,7 +213,7 @@ def _linear(op, kind, x, w, bias, bias_dtype, out_dtype, alpha, beta, inout=None
             _fail(op, f"the tensor to add into must be a contiguous {out_dtype} tensor of {M}x{N} elements on {dev}")
     if M == 0 or N == 0:
         return out
-    x, w, K = _pad_inner(x, w, K, M * N * K)
+    x, w, K = _pad_inner(x, w, K, M * N * K, weight=True)
     idx = dev.index
     switch = idx != _current_device()
     if switch:
@@ -204,7 +222,7 @@ def _linear(op, kind, x, w, bias, bias_dtype, out_dtype, alpha, beta, inout=None
     try:
         stream = _raw_stream(idx)
         # split-K scratch is only ever wanted for mid-sized M (see choose_splits in csrc/gemm_s8.hip)
-        ws_ptr, ws_bytes = _workspace(idx, stream, _ws_bytes(M, N, K)) if 16 < M <= 1024 else (0, 0)
+        ws_ptr, ws_bytes = _workspace(idx, stream, _ws_bytes(M, N, K)) if M > 16 else (0, 0)
         if _fast is not None:
             rc = _fast.linear(kind, x.data_ptr(), w.data_ptr(), bias.data_ptr(), out.data_ptr(), M, N, K,
                               alpha, beta, ws_ptr, ws_bytes, stream)

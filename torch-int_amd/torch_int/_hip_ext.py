@@ -598,7 +598,7 @@ def linear_a8_w8_b8_o8_heads(x, w, bias, alpha, beta, bsz, seq_len, heads, head_
     idx = x.device.index
     with _on(x.device):
         stream = _raw_stream(idx)
-        ws_ptr, ws_bytes = _CUDA._workspace(idx, stream, _CUDA._ws_bytes(M, N, K)) if 16 < M <= 1024 else (0, 0)
+        ws_ptr, ws_bytes = _CUDA._workspace(idx, stream, _CUDA._ws_bytes(M, N, K)) if M > 16 else (0, 0)
         rc = _lib.ti_linear_a8_w8_b8_o8_heads(x.data_ptr(), w.data_ptr(), bias.data_ptr(), out.data_ptr(), M, N, K,
                                               float(alpha), float(beta), seq_len, head_dim, ws_ptr or None, ws_bytes,
                                               stream or None)
@@ -639,11 +639,13 @@ def diag_store_loop(out, workgroups, reps=1):
     return out.numel() * 4 * int(reps)
 
 
-def measure_mfma_ceiling(window_ms=250.0, iters=20000):
+def measure_mfma_ceiling(window_ms=250.0, iters=20000, window=None):
     """What the int8 matrix pipe of the current device sustains, in TOP/s, for the three loop modes of
     ``diag_mfma_loop`` on constant and on uniformly random operand bytes: back-to-back launches between two HIP
     events for at least ``window_ms`` per figure (after the same again as warm-up, so the clocks have settled under
-    the board's power limit)."""
+    the board's power limit).  ``window(label)``, when given, returns a context manager that is entered around the
+    timed window of each figure (a benchmark samples clocks and board power there)."""
+    import contextlib
     dev = torch.device("cuda", torch.cuda.current_device())
     sink = torch.zeros(1, dtype=torch.int32, device=dev)
     patterns = {"constant": torch.full((1 << 20,), 1, dtype=torch.int8, device=dev),
@@ -658,10 +660,11 @@ def measure_mfma_ceiling(window_ms=250.0, iters=20000):
             torch.cuda.synchronize()
             n = max(2, int(window_ms / max(start.elapsed_time(end), 1e-3)) + 1)
             for timed in (False, True):
-                start.record()
-                for _ in range(n):
-                    diag_mfma_loop(mode, data, iters, sink)
-                end.record()
-                torch.cuda.synchronize()
+                with (window(f"{label}_{pname}") if timed and window is not None else contextlib.nullcontext()):
+                    start.record()
+                    for _ in range(n):
+                        diag_mfma_loop(mode, data, iters, sink)
+                    end.record()
+                    torch.cuda.synchronize()
             out[f"{label}_{pname}"] = ops * n / start.elapsed_time(end) / 1e9
     return out

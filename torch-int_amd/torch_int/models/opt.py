@@ -737,8 +737,10 @@ class Int8OPTGraphDecoder:
         with torch.cuda.stream(side):
             layers()
         torch.cuda.current_stream(k0.device).wait_stream(side)
+        # recorded on the stream of the eager pass: the library's per-stream state (split-K workspace and arrival
+        # counters, placement probe) is then ready, and nothing in the recording has to fall back or synchronise
         self.graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(self.graph):
+        with torch.cuda.graph(self.graph, stream=side):
             layers()
 
     @torch.no_grad()
