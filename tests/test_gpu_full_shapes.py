@@ -145,6 +145,66 @@ def test_linear_sweep_opt13b(N, K):
         del xd
 
 
+# ------------------------------------------------------------------ row counts that are not multiples of the tile
+
+@pytest.mark.parametrize("M,N,K", [(2112, 5120, 20480), (2176, 5120, 5120), (2050, 5120, 5120), (2064, 5120, 5120),
+                                   (4160, 4096, 8192), (2112, 5120, 5120), (1600, 5120, 5120)])
+def test_linear_with_rows_beyond_a_multiple_of_256(M, N, K):
+    """Prefill lengths are padded to 16, not to the tile height (upstream models/opt.py:375-383), so M = 4 x 528 = 2112
+    rows is an everyday shape.  Where the cost model says so the library runs the rows beyond the last multiple of 256
+    as a second, small problem (ti_linear_row_split); every epilogue kind, every output element against the
+    device-side reference and the last rows - the ones that travel separately - against the host oracle as well."""
+    import torch_int._CUDA as C
+    import torch_int._hip_ext as X
+    lib = C._lib
+    lib.ti_last_kernel.restype = ctypes.c_char_p
+    lib.ti_linear_row_split.argtypes = [ctypes.c_int64] * 3
+    r = lib.ti_linear_row_split(M, N, K)
+    g = torch.Generator().manual_seed(M + N + K)
+    x, w = _s8(g, M, K), _s8(g, N, K)
+    b32 = torch.randint(-65535, 65535, (N,), dtype=torch.int32, generator=g)
+    bf, b8 = torch.randn(N, generator=g), _s8(g, N)
+    xd, wd, b32d, bfd, b8d = x.to(DEV), w.to(DEV), b32.to(DEV), bf.to(DEV), b8.to(DEV)
+    al, be = _scal(g, 1e-4, 1e-2), _scal(g, 1e-4, 1e-2)
+    tail = torch.arange(M - 136, M)
+    acc_tail = orc.gemm_acc(x[tail].contiguous(), w)
+    resid = torch.randn(M, N, generator=g) * 3
+    hb = 4 if M % 4 == 0 else 2      # "batch" of the head-major form: hb sequences of T rows
+    T = M // hb
+    hd = 128
+    runs = [
+        ("b32_o32", lambda: C.linear_a8_w8_b32_o32(xd, wd, b32d), (1.0, 1.0), b32d, lambda: orc.epi_b32_o32(acc_tail, b32)),
+        ("bfp32_ofp32", lambda: C.linear_a8_w8_bfp32_ofp32(xd, wd, bfd, al, 1.0), (al, 1.0), bfd,
+         lambda: orc.epi_bfp32_ofp32(acc_tail, bf, al, 1.0)),
+        ("b8_o8", lambda: C.linear_a8_w8_b8_o8(xd, wd, b8d, al, be), (al, be), b8d, lambda: orc.epi_b8_o8(acc_tail, b8, al, be)),
+        ("relu_b8_o8", lambda: C.linear_relu_a8_w8_b8_o8(xd, wd, b8d, al, be), (al, be), b8d,
+         lambda: orc.epi_b8_o8(acc_tail, b8, al, be, relu=True)),
+        ("b8_o8 head-major", lambda: X.linear_a8_w8_b8_o8_heads(xd, wd, b8d, al, be, hb, T, N // hd, hd)
+         .permute(0, 2, 1, 3).reshape(M, N), (al, be), b8d, lambda: orc.epi_b8_o8(acc_tail, b8, al, be)),
+    ]
+    for name, gpu, (a, b), bias_d, ref in runs:
+        out = gpu()
+        family = lib.ti_last_kernel().decode()
+        _say(f"ragged rows {name} M={M} N={N} K={K} split={r} -> {family}")
+        assert ("+" in family) == (r > 0), (family, r)
+        _check_every_tile(name.split()[0], out, xd, wd, bias_d, a, b)
+        assert torch.equal(out[tail.to(DEV)].cpu(), ref()), name
+    # the accumulating kind: inout += alpha * acc + bias, one fp32 add after the linear's own rounding
+    inout = resid.to(DEV)
+    out = C._linear_a8_w8_bfp32_ofp32_acc(xd, wd, bfd, al, 1.0, inout)
+    family = lib.ti_last_kernel().decode()
+    _say(f"ragged rows += M={M} N={N} K={K} -> {family}")
+    assert ("+" in family) == (r > 0), (family, r)
+    fresh = C.linear_a8_w8_bfp32_ofp32(xd, wd, bfd, al, 1.0)     # checked in full above
+    assert torch.equal(out, resid.to(DEV) + fresh)
+    # without a workspace the call still works (whole problem on tiles, or a split whose rest needs none)
+    out8 = torch.empty((M, N), dtype=torch.int8, device=DEV)
+    rc = lib.ti_linear_a8_w8_b8_o8(xd.data_ptr(), wd.data_ptr(), b8d.data_ptr(), out8.data_ptr(), M, N, K, al, be, None, 0,
+                                   torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, lib.ti_last_error()
+    assert torch.equal(out8, C.linear_a8_w8_b8_o8(xd, wd, b8d, al, be))
+
+
 # ------------------------------------------------------------------ attention products, batch*heads = 160
 
 @pytest.mark.parametrize("S", [128, 2048])

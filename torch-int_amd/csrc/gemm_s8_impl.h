@@ -2298,6 +2298,11 @@ static WidePick pick_wide(long long M, long long N, long long K, long long batch
 // by choose_splits (its workspace must have been given), rows <= 16 as weight streaming at 4.5 TB/s.
 static int row_split_rows(long long M, long long N, long long K, long long* rest_ws_bytes = nullptr) {
   if (rest_ws_bytes) *rest_ws_bytes = 0;
+  static const bool enabled = [] {  // TORCH_INT_ROW_SPLIT=0 keeps every linear in one piece
+    const char* v = getenv("TORCH_INT_ROW_SPLIT");
+    return !(v && v[0] == '0');
+  }();
+  if (!enabled) return 0;
   const long long r = M % 256;
   if (M <= 1024 || r == 0 || r > 128 || N <= 128 || K % QBK != 0 || K < 1024) return 0;
   const WidePick whole = pick_wide(M, N, K, 1), main = pick_wide(M - r, N, K, 1);
