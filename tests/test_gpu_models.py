@@ -413,3 +413,35 @@ def test_fused_softmax_switch_restores_the_torch_chain():
     assert (p_f - p_p).abs().max() <= 1 and (p_f != p_p).float().mean() < 5e-3
     assert torch.equal(fused[2][0], plain[2][0]) and torch.equal(fused[2][1], plain[2][1])   # K / V: before the softmax
     assert _rel_err(fused[0], plain[0]) < 2e-2
+
+
+@torch.no_grad()
+@pytest.mark.parametrize("D,H", [(640, 8), (192, 4), (2560, 32)])
+def test_prefill_attention_with_a_head_size_the_fused_kernel_pads(D, H):
+    """Head sizes that are multiples of 16 other than 64 / 128 (OPT-2.7B: 2560 / 32 = 80) take the one-launch prefill
+    attention on zero-padded q, k and V^T.  Same bits as the operator chain (Q.K^T, softmax-quantiser, P.V, head merge),
+    which a call that wants the probabilities back still runs."""
+    import torch_int._hip_ext as X
+    g = torch.Generator().manual_seed(D + H)
+    layer = randomize_int8_layer(Int8OPTDecoderLayer(D, H, 2 * D), g).to(DEV)
+    B, T = 2, 112
+    hidden = torch.randn(B, T, D, generator=g).to(DEV)
+    mask = causal_mask(B, T, T).to(DEV)
+    mask[1, :, :, :5] = torch.finfo(torch.float32).min   # left padding on one sequence
+    calls = []
+    real = X.attn_prefill
+
+    def counted(*a, **kw):
+        calls.append(a[0].shape)
+        return real(*a, **kw)
+    X.attn_prefill = counted
+    try:
+        fused = layer(hidden.clone(), attention_mask=mask, use_cache=True)
+        assert len(calls) == 1 and calls[0][2] in (64, 128) and calls[0][2] > D // H, calls
+        chain = layer(hidden.clone(), attention_mask=mask, use_cache=True, output_attentions=True)
+        assert len(calls) == 1   # the second call went down the operator chain
+    finally:
+        X.attn_prefill = real
+    assert torch.equal(fused[0], chain[0])
+    assert torch.equal(fused[-1][0], chain[-1][0]) and torch.equal(fused[-1][1], chain[-1][1])
+    assert chain[1].shape == (B, H, T, T)
