@@ -272,6 +272,7 @@ int launch_splitk_raw(int tile, const GemmParams& q, hipStream_t stream) {
   if (tile == SPLIT_128x80) return launch_pipe16q<Pipe16QCfg<128, 80, 4, 1, EPI_S32_RAW>>(q, stream);
   if (tile == SPLIT_128x160) return launch_pipe16q<Pipe16QCfg<128, 160, 4, 2, EPI_S32_RAW>>(q, stream);
   if (tile == SPLIT_128x288) return launch_pipe16q<Pipe16QCfg<128, 288, 4, 2, EPI_S32_RAW>>(q, stream);
+  if (tile == SPLIT_128x192) return launch_pipe16q<Pipe16QCfg<128, 192, 4, 2, EPI_S32_RAW>>(q, stream);
   if (tile == SPLIT_256x288) return launch_pipe16q<Pipe16QCfg<256, 288, 4, 2, EPI_S32_RAW>>(q, stream);
   if (q.K % QBK == 0) return launch_pipe2<Pipe2Cfg<256, 256, 2, 4, EPI_S32_RAW, false>>(q, stream);
   return launch_pipe<PipeCfg<256, 256, 2, 4, 4, EPI_S32_RAW, false>>(q, stream);

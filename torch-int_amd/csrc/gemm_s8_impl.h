@@ -2135,7 +2135,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmParams p, const 
 // (its four waves read 7 fragments from the LDS per 10 MFMAs); with K = 20480 the larger tiles win
 // (512x5120x20480: 79 against 64 us).  More than three LDS stages did not help it (four to six: +1 to +3 %).
 enum SplitTile { SPLIT_128 = 0, SPLIT_256 = 1, SPLIT_256x160 = 2, SPLIT_256x288 = 3, SPLIT_128x160 = 4, SPLIT_128x288 = 5,
-                 SPLIT_128x80 = 6 };
+                 SPLIT_128x80 = 6, SPLIT_128x192 = 7 };
 static int choose_splits(long long M, long long N, long long K, int* tile_kind = nullptr, double* time_us = nullptr) {
   if (tile_kind) *tile_kind = SPLIT_128;
   if (time_us) *time_us = -1.0;  // no estimate
@@ -2146,15 +2146,21 @@ static int choose_splits(long long M, long long N, long long K, int* tile_kind =
   double best_t = 1e30;
   // the 128-row forms of the tall tiles first, then by size: a later candidate must be clearly faster to replace
   // an earlier one
-  const int order[7] = {SPLIT_128x80, SPLIT_128x160, SPLIT_128x288, SPLIT_128, SPLIT_256, SPLIT_256x160, SPLIT_256x288};
-  for (int oi = 0; oi < 7; ++oi) {
+  // (128x192 tiles: widths that 192 divides but neither 160 nor 288 nor 80 does - 12288 and 49152, the GPT-3-sized
+  // layers of upstream's scripts/bench_linear_kernels.sh - had only the 128x128 and 256x256 tiles of the 64-byte-step
+  // and 32x32-block kernels to split over; 512 x 12288 outputs are exactly 256 tiles of 128x192 and run unsplit)
+  const int order[8] = {SPLIT_128x80, SPLIT_128x160, SPLIT_128x192, SPLIT_128x288, SPLIT_128, SPLIT_256, SPLIT_256x160,
+                        SPLIT_256x288};
+  for (int oi = 0; oi < 8; ++oi) {
     const int kind = order[oi];
+    const bool wide192 = kind == SPLIT_128x192;
     const bool half = kind == SPLIT_128x160 || kind == SPLIT_128x288;  // 128-row forms of the two tall tiles
     const bool small = kind == SPLIT_128x80;
-    const int bm = kind == SPLIT_128 || half || small ? 128 : 256;
-    const int bn = small ? 80 : kind == SPLIT_128 ? 128 : kind == SPLIT_256 ? 256
+    const int bm = kind == SPLIT_128 || half || small || wide192 ? 128 : 256;
+    const int bn = small ? 80 : wide192 ? 192 : kind == SPLIT_128 ? 128 : kind == SPLIT_256 ? 256
                    : kind == SPLIT_256x288 || kind == SPLIT_128x288 ? 288 : 160;
     if (kind >= SPLIT_256x160 && N % bn != 0) continue;
+    if (wide192 && (N % 160 == 0 || N % 288 == 0)) continue;  // those widths keep their tuned tiles
     const double tiles = (double)((M + bm - 1) / bm) * (double)((N + bn - 1) / bn);
     for (int s = 1; s <= 16; ++s) {
       if (steps % s != 0 || steps / s < 4) continue;
@@ -2163,6 +2169,7 @@ static int choose_splits(long long M, long long N, long long K, int* tile_kind =
       // an unsplit candidate stands for what the ordinary dispatch would launch, which takes the 256-row tiles only
       // when they fill most of the chip (and 128x128 tiles otherwise)
       if (s == 1 && kind != SPLIT_128 && !small && tiles < 0.75 * cus) continue;
+      if (s == 1 && wide192 && tiles > cus) continue;  // more than a round: the 256-row tilings of the ordinary dispatch
       const double wgs = tiles * s;
       double rounds, step_us, fixed_us = 8.0;
       if (kind == SPLIT_128) {
@@ -2175,13 +2182,14 @@ static int choose_splits(long long M, long long N, long long K, int* tile_kind =
       } else {
         rounds = (double)(long long)((wgs + cus - 1) / cus);
         step_us = kind == SPLIT_256 ? 0.85 : kind == SPLIT_256x160 ? 0.55 : kind == SPLIT_256x288 ? 0.92
-                  : kind == SPLIT_128x160 ? 0.375 : 0.6;
+                  : kind == SPLIT_128x160 ? 0.375 : wide192 ? 0.41 : 0.6;
         if (half) fixed_us = kind == SPLIT_128x160 ? 4.0 : 5.0;  // fewer panel rows to fetch first, half the tile to store
+        if (wide192) fixed_us = 4.5;
       }
       double t = rounds * ((double)(steps / s) * step_us + fixed_us);
       // The weights come from HBM: a workgroup keeps about `ahead` K steps of its weight rows in flight, and what
       // all resident workgroups have in flight over a 2 us round trip bounds the streaming rate (5 TB/s at most).
-      const double ahead = kind == SPLIT_128 ? 4.0 : kind == SPLIT_256x160 || half || small ? 2.5 : 1.5;
+      const double ahead = kind == SPLIT_128 ? 4.0 : kind == SPLIT_256x160 || half || small || wide192 ? 2.5 : 1.5;
       const double step_bytes = (double)bn * (kind == SPLIT_128 ? 64.0 : 128.0);
       const double resident = wgs < cus * (kind == SPLIT_128 ? 2 : 1) ? wgs : cus * (kind == SPLIT_128 ? 2 : 1);
       double rate = resident * ahead * step_bytes / 2.0;  // bytes per us
@@ -2409,6 +2417,10 @@ int launch_kind(const GemmParams& p, void* workspace, long long workspace_bytes,
       g_last_kernel = "pipe16_128x80";
       return launch_pipe16q<Pipe16QCfg<128, 80, 4, 1, KIND>>(p, stream);
     }
+    if (splits == 1 && tile == SPLIT_128x192) {
+      g_last_kernel = "pipe16_128x192";
+      return launch_pipe16q<Pipe16QCfg<128, 192, 4, 2, KIND>>(p, stream);
+    }
     if (splits > 1 && workspace != nullptr && workspace_bytes >= need &&
         (reinterpret_cast<uintptr_t>(workspace) & 15) == 0) {
       g_last_kernel = tile == SPLIT_128      ? "splitk_128x128"
@@ -2417,6 +2429,7 @@ int launch_kind(const GemmParams& p, void* workspace, long long workspace_bytes,
                       : tile == SPLIT_128x160 ? "splitk_128x160"
                       : tile == SPLIT_128x288 ? "splitk_128x288"
                       : tile == SPLIT_128x80  ? "splitk_128x80"
+                      : tile == SPLIT_128x192 ? "splitk_128x192"
                                               : "splitk_256x288";
       // not for the accumulating epilogue: its reads of the old outputs, done by one workgroup per tile instead of
       // by the whole chip in the reduction kernel, cost more than the launch saved (512x9216x36864: 288 against
@@ -2424,9 +2437,10 @@ int launch_kind(const GemmParams& p, void* workspace, long long workspace_bytes,
       if constexpr (KIND != EPI_S32_RAW && KIND != EPI_F32_BIAS_ACC) {
         // one launch when the tile is one of the 16x16-block kernel's and covers M in whole tiles
         const int bm = tile == SPLIT_256x160 || tile == SPLIT_256x288 ? 256 : 128;
-        const int bn = tile == SPLIT_128x80 ? 80 : tile == SPLIT_256x160 || tile == SPLIT_128x160 ? 160 : 288;
+        const int bn = tile == SPLIT_128x80 ? 80 : tile == SPLIT_128x192 ? 192
+                       : tile == SPLIT_256x160 || tile == SPLIT_128x160 ? 160 : 288;
         const bool tall = tile == SPLIT_128x80 || tile == SPLIT_128x160 || tile == SPLIT_128x288 ||
-                          tile == SPLIT_256x160 || tile == SPLIT_256x288;
+                          tile == SPLIT_256x160 || tile == SPLIT_256x288 || tile == SPLIT_128x192;
         // up to four slices: the wave that arrives last reads the others' accumulators one slice after the other,
         // and beyond four that tail costs more than the reduction launch it saves (measured: 2 slices -3 to -12 %,
         // 4 slices -3 to -8 %, 7 and 8 slices +3 to +6 %)
@@ -2453,6 +2467,9 @@ int launch_kind(const GemmParams& p, void* workspace, long long workspace_bytes,
               case SPLIT_128x160:
                 g_last_kernel = "fusedk_128x160";
                 return launch_fused<Pipe16QCfg<128, 160, 4, 2, KIND, false, 3, true>>(f, stream);
+              case SPLIT_128x192:
+                g_last_kernel = "fusedk_128x192";
+                return launch_fused<Pipe16QCfg<128, 192, 4, 2, KIND, false, 3, true>>(f, stream);
               case SPLIT_128x288:
                 g_last_kernel = "fusedk_128x288";
                 return launch_fused<Pipe16QCfg<128, 288, 4, 2, KIND, false, 3, true>>(f, stream);
