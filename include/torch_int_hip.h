@@ -220,6 +220,21 @@ int ti_bmm_s8t_s8n_s8t(const int8_t* a, const int8_t* b, int8_t* c,
 int ti_bmm_s8t_s8n_s32t(const int8_t* a, const int8_t* b, int32_t* c,
                         int64_t batch, int64_t M, int64_t N, int64_t K, void* stream);
 
+/* The three batched products with a split-K workspace (no counterpart in the reference, whose GemmBatched takes
+ * none): same arguments, same bytes out as ti_bmm_s8t_s8n_*.  When the problems together have too few output tiles
+ * to fill the chip and the inner dimension is long - upstream's own benchmark/bench_bmm.py:9-15 multiplies
+ * [batch, seq, 12288] operands, batch 1..16 - K is cut into slices that run side by side (raw int32 partial
+ * products in `workspace`, then one reduction launch; a single problem takes the linears' forms, the one-launch one
+ * included).  ti_bmm_workspace_bytes = bytes that lets the library do so for a shape (0 = it would not split;
+ * attention-shaped products, K = head size, never do); a smaller or NULL workspace only selects the unsplit kernels. */
+int64_t ti_bmm_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K);
+int ti_bmm_s8t_s8n_f32t_ws(const int8_t* a, const int8_t* b, float* c, int64_t batch, int64_t M, int64_t N, int64_t K,
+                           float alpha, void* workspace, int64_t workspace_bytes, void* stream);
+int ti_bmm_s8t_s8n_s8t_ws(const int8_t* a, const int8_t* b, int8_t* c, int64_t batch, int64_t M, int64_t N, int64_t K,
+                          float alpha, void* workspace, int64_t workspace_bytes, void* stream);
+int ti_bmm_s8t_s8n_s32t_ws(const int8_t* a, const int8_t* b, int32_t* c, int64_t batch, int64_t M, int64_t N, int64_t K,
+                           void* workspace, int64_t workspace_bytes, void* stream);
+
 /* ---- fused dequantise + residual add + LayerNorm + quantise ---- */
 
 /* replaces dq_add_layernorm_q (torch_int/kernels/fused.cu:5-25; include/fused.h:6-14):

@@ -274,6 +274,34 @@ def test_bmm_shapes():
         _bmm_case(C, B, M, N, K, seed=200 + i)
 
 
+def test_bmm_split_k_over_a_long_inner_dimension():
+    # upstream's benchmark/bench_bmm.py multiplies [batch, seq, 12288] operands: few output tiles, a long K.  The
+    # library then cuts K into slices (all problems' slices in one raw-int32 launch + one reduction; a single problem
+    # takes the linears' forms); same bits as the oracle for all three output kinds, ragged shapes included
+    import ctypes
+    import torch_int._CUDA as C
+    lib = C._lib
+    lib.ti_last_kernel.restype = ctypes.c_char_p
+    for i, (B, M, N, K) in enumerate([(4, 256, 256, 12288), (16, 256, 256, 4096), (8, 512, 512, 2048), (3, 200, 260, 4096),
+                                      (1, 512, 512, 12288), (1, 256, 256, 12288), (2, 100, 128, 6144), (5, 64, 384, 8192)]):
+        _say(f"bmm, long K: B={B} M={M} N={N} K={K}")
+        split = lib.ti_bmm_workspace_bytes(B, M, N, K) > 0
+        assert split or i == 2, (B, M, N, K)      # (8 x 512 x 512 x 2048 fills the chip without)
+        _bmm_case(C, B, M, N, K, seed=400 + i)
+        assert lib.ti_last_kernel().decode().startswith(("splitk_", "fusedk_")) == split, (B, M, N, K, lib.ti_last_kernel())
+    # attention-shaped products never split, and a call without the workspace still works
+    assert lib.ti_bmm_workspace_bytes(160, 512, 512, 128) == 0 and lib.ti_bmm_workspace_bytes(160, 512, 128, 512) == 0
+    g = torch.Generator().manual_seed(409)
+    a, b = _s8(g, 4, 256, 4096), _s8(g, 4, 256, 4096)
+    out = torch.empty((4, 256, 256), dtype=torch.int8, device=DEV)
+    ad, bd = a.to(DEV), b.to(DEV)
+    rc = lib.ti_bmm_s8t_s8n_s8t(ad.data_ptr(), bd.data_ptr(), out.data_ptr(), 4, 256, 256, 4096, 0.002,
+                                torch.cuda.current_stream().cuda_stream)
+    assert rc == 0 and not lib.ti_last_kernel().decode().startswith("splitk_")
+    assert torch.equal(out, C.bmm_s8t_s8n_s8t(ad, bd, 0.002))
+    assert lib.ti_last_kernel().decode().startswith("splitk_")
+
+
 def test_large_problems_with_an_inner_dimension_that_16_does_not_divide():
     # the library's kernel for such shapes is one thread per output; from 2^26 products the host functions pad K
     # with zeros and the tiled kernels run (same results: the added products are zero)

@@ -298,6 +298,29 @@ int ti_bmm_s8t_s8n_s32t(const int8_t* a, const int8_t* b, int32_t* c, int64_t ba
                   0, stream);
 }
 
+int64_t ti_bmm_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K) {
+  if (batch <= 0 || M <= 0 || N <= 0 || K <= 0) return 0;
+  return bmm_workspace_bytes(batch, M, N, K);
+}
+
+int ti_bmm_s8t_s8n_f32t_ws(const int8_t* a, const int8_t* b, float* c, int64_t batch, int64_t M, int64_t N, int64_t K,
+                           float alpha, void* ws, int64_t ws_bytes, void* stream) {
+  return run_gemm("bmm_s8t_s8n_f32t", EPI_F32_SCALE, a, b, nullptr, 0, c, 4, batch, M, N, K, alpha, 0.0f, ws, ws_bytes,
+                  stream);
+}
+
+int ti_bmm_s8t_s8n_s8t_ws(const int8_t* a, const int8_t* b, int8_t* c, int64_t batch, int64_t M, int64_t N, int64_t K,
+                          float alpha, void* ws, int64_t ws_bytes, void* stream) {
+  return run_gemm("bmm_s8t_s8n_s8t", EPI_S8_SCALE, a, b, nullptr, 0, c, 1, batch, M, N, K, alpha, 0.0f, ws, ws_bytes,
+                  stream);
+}
+
+int ti_bmm_s8t_s8n_s32t_ws(const int8_t* a, const int8_t* b, int32_t* c, int64_t batch, int64_t M, int64_t N, int64_t K,
+                           void* ws, int64_t ws_bytes, void* stream) {
+  return run_gemm("bmm_s8t_s8n_s32t", EPI_S32_RAW, a, b, nullptr, 0, c, 4, batch, M, N, K, 1.0f, 0.0f, ws, ws_bytes,
+                  stream);
+}
+
 int ti_dq_add_layernorm_q(const int32_t* input, float input_scale, const float* residual, const float* gamma,
                           const float* beta, float eps, float* r_out, int8_t* q_out, int64_t rows, int64_t H,
                           void* stream) {

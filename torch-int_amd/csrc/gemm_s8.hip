@@ -30,6 +30,12 @@ int launch_gemm_kind_8(const GemmParams& p, void* ws, long long ws_bytes, hipStr
 
 int gemm_row_split(long long M, long long N, long long K) { return row_split_rows(M, N, K); }
 
+long long bmm_workspace_bytes(long long batch, long long M, long long N, long long K) {
+  if (batch == 1) return gemm_workspace_bytes(M, N, K);  // one problem: the linears' split-K forms
+  const int s = batched_splits(batch, M, N, K);
+  return s > 1 ? (long long)s * batch * M * N * 4 : 0;
+}
+
 thread_local const char* g_last_kernel = "";
 const char* last_gemm_kernel() { return g_last_kernel; }
 

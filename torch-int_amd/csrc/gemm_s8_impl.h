@@ -501,8 +501,8 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MIN_WAVES) void gemm_pipe_kernel(Gemm
     int tile_m, tile_n;
     tile_of_workgroup(t, tiles_m, tiles_n, tile_m, tile_n, p.band);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
-    const int8_t* A = p.A + (long long)b * p.strideA;
-    const int8_t* B = p.B + (long long)b * p.strideB;
+    const int8_t* A = a_of_batch(p, b);
+    const int8_t* B = b_of_batch(p, b);
 #pragma unroll
     for (int j = 0; j < COPIES; ++j) {
       const int slab = wave * COPIES + j;        // 16-row slab inside [A panel | B panel]
@@ -729,7 +729,7 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe2_kernel(GemmParams p, in
     const int first_row = copies_a ? tile_m * BM : tile_n * BN;  // of the panel in its operand
     const int last_row = (copies_a ? M : N) - 1;                 // edge rows re-read the last row; never stored
     const size_t ld = copies_a ? p.lda : p.ldb;
-    const int8_t* origin = copies_a ? p.A + (long long)b * p.strideA : p.B + (long long)b * p.strideB;
+    const int8_t* origin = copies_a ? a_of_batch(p, b) : b_of_batch(p, b);
 #pragma unroll
     for (int j = 0; j < COPIES; ++j) {
       const int prow = (wave * COPIES + j) * 8 + (lane >> 3) - (copies_a ? 0 : BM);  // row inside the panel
@@ -1104,8 +1104,8 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe16_kernel(GemmParams p, i
     int tile_m, tile_n;
     tile_of_workgroup(item - b * tiles, tiles_m, tiles_n, tile_m, tile_n, p.band);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
-    const int8_t* A = p.A + (long long)b * p.strideA;
-    const int8_t* B = p.B + (long long)b * p.strideB;
+    const int8_t* A = a_of_batch(p, b);
+    const int8_t* B = b_of_batch(p, b);
 #pragma unroll
     for (int j = 0; j < COPIES; ++j) {
       int prow = wave * Cfg::RPW + j * 16 + (lane >> 2);
@@ -1366,8 +1366,8 @@ __global__ __launch_bounds__(Cfg::NT, 2) void gemm_pipe16q_kernel(GemmParams p, 
     int tile_m, tile_n;
     tile_of_workgroup(tile_id, tiles_m, tiles_n, tile_m, tile_n, p.band);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
-    const int8_t* A = Cfg::GROUPED ? p.A : p.A + (long long)b * p.strideA;
-    const int8_t* B = Cfg::GROUPED ? grp.B[b] : p.B + (long long)b * p.strideB;
+    const int8_t* A = Cfg::GROUPED ? p.A : a_of_batch(p, b);
+    const int8_t* B = Cfg::GROUPED ? grp.B[b] : b_of_batch(p, b);
 #pragma unroll
     for (int j = 0; j < COPIES; ++j) {
       int prow = wave * Cfg::RPW + j * 8 + (lane >> 3);
@@ -2080,7 +2080,9 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmParams p, const 
   const long long i0 = ((long long)blockIdx.x * 256 + threadIdx.x) * 4;
   if (i0 >= total) return;
   const BiasT* bias = reinterpret_cast<const BiasT*>(p.bias);
-  Out* C = reinterpret_cast<Out*>(p.C);
+  // blockIdx.y = problem of a batched product: its slices follow one another in the workspace
+  ws += (long long)blockIdx.y * splits * total;
+  Out* C = reinterpret_cast<Out*>(p.C) + (long long)blockIdx.y * p.strideC;
   if ((p.N & 3) == 0 && (reinterpret_cast<uintptr_t>(C) & 15) == 0) {  // four consecutive columns of one row
     v4i acc = *reinterpret_cast<const v4i*>(ws + i0);
     for (int s = 1; s < splits; ++s) acc += *reinterpret_cast<const v4i*>(ws + (long long)s * total + i0);
@@ -2136,7 +2138,11 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmParams p, const 
 // (512x5120x20480: 79 against 64 us).  More than three LDS stages did not help it (four to six: +1 to +3 %).
 enum SplitTile { SPLIT_128 = 0, SPLIT_256 = 1, SPLIT_256x160 = 2, SPLIT_256x288 = 3, SPLIT_128x160 = 4, SPLIT_128x288 = 5,
                  SPLIT_128x80 = 6, SPLIT_128x192 = 7 };
-static int choose_splits(long long M, long long N, long long K, int* tile_kind = nullptr, double* time_us = nullptr) {
+// `batch` > 1: a batched product (A and B per batch); every tile count, byte count and the streaming floor scale with
+// it, the one-launch form is not available, and the tile shapes are those that exist for every epilogue of the
+// raw-int32 kernels.
+static int choose_splits(long long M, long long N, long long K, int* tile_kind = nullptr, double* time_us = nullptr,
+                         long long batch = 1) {
   if (tile_kind) *tile_kind = SPLIT_128;
   if (time_us) *time_us = -1.0;  // no estimate
   if (M <= 16 || M > 1024 || K % PBK != 0 || K < 1024) return 1;
@@ -2161,11 +2167,12 @@ static int choose_splits(long long M, long long N, long long K, int* tile_kind =
                    : kind == SPLIT_256x288 || kind == SPLIT_128x288 ? 288 : 160;
     if (kind >= SPLIT_256x160 && N % bn != 0) continue;
     if (wide192 && (N % 160 == 0 || N % 288 == 0)) continue;  // those widths keep their tuned tiles
-    const double tiles = (double)((M + bm - 1) / bm) * (double)((N + bn - 1) / bn);
+    const double tiles = (double)((M + bm - 1) / bm) * (double)((N + bn - 1) / bn) * (double)batch;
     for (int s = 1; s <= 16; ++s) {
       if (steps % s != 0 || steps / s < 4) continue;
       if (kind >= SPLIT_256x160 && (K / s) % QBK != 0) continue;  // these tiles step 128 bytes at a time
       if (half && s == 1) continue;                                // exist as raw-int32 kernels only
+      if (batch > 1 && s == 1 && (small || wide192)) continue;       // unsplit batched products keep their dispatch
       // an unsplit candidate stands for what the ordinary dispatch would launch, which takes the 256-row tiles only
       // when they fill most of the chip (and 128x128 tiles otherwise)
       if (s == 1 && kind != SPLIT_128 && !small && tiles < 0.75 * cus) continue;
@@ -2199,13 +2206,13 @@ static int choose_splits(long long M, long long N, long long K, int* tile_kind =
       // 128x20480x5120 30 us, 256x20480x5120 48 us)
       const double cap = kind == SPLIT_128 ? 3.5e6 : small ? (wgs <= cus ? 3.8e6 : 2.4e6) : 5.0e6;
       if (rate > cap) rate = cap;
-      const double t_stream = (double)N * (double)K / rate + (small ? 4.0 : 8.0);
+      const double t_stream = (double)batch * (double)N * (double)K / rate + (small ? 4.0 : 8.0);
       if (t < t_stream) t = t_stream;
       // the slices' partial tiles: written once and read once (they mostly stay in the last-level cache) plus the
       // second launch; in the one-launch form they stay in the XCD's L2 and the reading is the last workgroup's tail
-      const bool one_launch = kind >= SPLIT_256x160 && M % bm == 0 && s <= (kind == SPLIT_256x288 ? 2 : 4);
+      const bool one_launch = batch == 1 && kind >= SPLIT_256x160 && M % bm == 0 && s <= (kind == SPLIT_256x288 ? 2 : 4);
       if (s > 1 && one_launch) t += (double)(2 * s - 1) * M * N * 4.0 / 8.0e6 + 1.0;
-      else if (s > 1) t += (double)(2 * s + 1) * M * N * 4.0 / 5.5e6 + 3.0;  // at 5.5 TB/s, in us
+      else if (s > 1) t += (double)batch * (double)(2 * s + 1) * M * N * 4.0 / 5.5e6 + 3.0;  // at 5.5 TB/s, in us
       if (t < best_t * 0.97) {  // prefer fewer slices and the smaller tile unless the gain is clear
         best_t = t;
         best = s;
@@ -2284,8 +2291,10 @@ static WidePick pick_wide(long long M, long long N, long long K, long long batch
   // The 256x128 tiles and the comparison with the 128x128 kernel are for linears with a K of some length
   // (the rates above were measured at K >= 4096; at K = 768 the 128x128 kernel's short prologue wins); batched
   // products keep their tuned 256x256 / 128x128 choice, they are bound by HBM, not by the matrix pipe.
-  const bool priced = batch == 1 && K >= 2048 && t128 >= 128;
-  const double e128w = priced && wide_step && N % 128 == 0 ? 0.93 * fill(rows256 * (N / 128), 128) : 0.0;
+  // (a batched product with an inner dimension that long is a stack of linears, not an attention product, and is
+  // priced like them: 8 x 1024 x 1024 x 12288 makes 256 tiles of 256x128 where it made 128 of 256x256)
+  const bool priced = K >= 2048 && t128 >= 128;
+  const double e128w = priced && wide_step && N % 128 == 0 ? 0.93 * fill(rows256 * (N / 128) * batch, 128) : 0.0;
   const double e128 = t128 >= 2 * cus ? 0.6 : t128 >= cus ? 0.47 : 0.47 * (double)t128 / (double)cus;
   const double best = e256 > e160 ? (e256 > e288 ? (e256 > e128w ? e256 : e128w) : (e288 > e128w ? e288 : e128w))
                                   : (e160 > e288 ? (e160 > e128w ? e160 : e128w) : (e288 > e128w ? e288 : e128w));
@@ -2294,6 +2303,17 @@ static WidePick pick_wide(long long M, long long N, long long K, long long batch
   if (e288 > e256 && e288 >= e128w) return WidePick{WIDE_256x288, e288};
   if (e128w > e256) return WidePick{WIDE_256x128, e128w};
   return WidePick{WIDE_256x256, e256};
+}
+
+// K slices for a batched product (1 = none): only where the problems together have too few 128x128 tiles to fill
+// the chip twice and the inner dimension is long; attention-shaped products (K = head size, or many heads) keep
+// their own dispatch.
+static int batched_splits(long long batch, long long M, long long N, long long K, int* tile_kind = nullptr) {
+  if (tile_kind) *tile_kind = SPLIT_128;
+  if (batch <= 1 || M <= 16 || M > 1024 || N <= 16 || K < 2048 || K % PBK != 0) return 1;
+  const long long t128 = ((M + 127) / 128) * ((N + 127) / 128) * batch;
+  if (t128 >= 2 * (long long)num_cus()) return 1;
+  return choose_splits(M, N, K, tile_kind, nullptr, batch);
 }
 
 // Rows to cut off the end of a linear with many rows and run as a second, small problem (0 = none).
@@ -2387,6 +2407,41 @@ int launch_kind(const GemmParams& p, void* workspace, long long workspace_bytes,
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "gemm launch: %s", hipGetErrorString(e));
     return TI_OK;
+  }
+  if (p.batch > 1 && p.batch <= 65535 && p.lda == p.K && p.ldb == p.K && p.out_d == 0 && workspace != nullptr &&
+      (reinterpret_cast<uintptr_t>(workspace) & 15) == 0) {
+    // A batched product with few output tiles and a long inner dimension (upstream's benchmark/bench_bmm.py multiplies
+    // [batch, seq, 12288] operands): K slices as for the linears, the slices of all problems being the batches of one
+    // raw-int32 launch, then one reduction launch.
+    int tile = SPLIT_128;
+    const int splits = batched_splits(p.batch, p.M, p.N, p.K, &tile);
+    const long long need = (long long)splits * p.batch * p.M * p.N * 4;
+    if (splits > 1 && workspace_bytes >= need) {
+      g_last_kernel = tile == SPLIT_128      ? "splitk_128x128"
+                      : tile == SPLIT_256    ? "splitk_256x256"
+                      : tile == SPLIT_256x160 ? "splitk_256x160"
+                      : tile == SPLIT_128x160 ? "splitk_128x160"
+                      : tile == SPLIT_128x288 ? "splitk_128x288"
+                      : tile == SPLIT_128x80  ? "splitk_128x80"
+                      : tile == SPLIT_128x192 ? "splitk_128x192"
+                                              : "splitk_256x288";
+      GemmParams q = p;
+      q.K = p.K / splits;
+      q.kslices = splits;
+      q.strideAk = q.K;
+      q.strideBk = q.K;
+      q.batch = p.batch * splits;
+      q.strideC = (long long)p.M * p.N;
+      q.C = workspace;
+      q.bias = nullptr;
+      if (int rc = launch_splitk_raw(tile, q, stream)) return rc;
+      const long long quads = ((long long)p.M * p.N + 3) / 4;
+      hipLaunchKernelGGL(splitk_reduce_kernel<KIND>, dim3((unsigned)((quads + 255) / 256), (unsigned)p.batch), dim3(256), 0,
+                         stream, p, static_cast<const int*>(workspace), splits);
+      hipError_t e = hipGetLastError();
+      if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "split-K reduce launch: %s", hipGetErrorString(e));
+      return TI_OK;
+    }
   }
   if (p.batch == 1 && p.lda == p.K && p.ldb == p.K && p.M > 1024) {
     // many rows, a few of them beyond the last multiple of 256: two problems (see row_split_rows)

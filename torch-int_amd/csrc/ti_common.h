@@ -189,11 +189,31 @@ struct GemmParams {
   // counter per (tile, wave), `xcc_seen` one zeroed word per tile in which the workgroups of the tile mark the XCC
   // they run on, xcc_error = host-mapped word that is set when two of them differ.
   int splits = 1;
+  // Split-K of a batched product (the pipelined kernels): batch index b of the launch is (problem b / kslices,
+  // K slice b % kslices); problems are strideA / strideB apart, slices strideAk / strideBk (K is one slice's length).
+  int kslices = 1;
+  long long strideAk = 0, strideBk = 0;
   void* parts = nullptr;
   int* arrivals = nullptr;
   unsigned* xcc_seen = nullptr;
   int* xcc_error = nullptr;
 };
+
+// First byte of the A / B operand of batch index b of a launch.
+__device__ __forceinline__ const int8_t* a_of_batch(const GemmParams& p, int b) {
+  if (p.kslices > 1) {
+    const int bb = b / p.kslices;
+    return p.A + (long long)bb * p.strideA + (long long)(b - bb * p.kslices) * p.strideAk;
+  }
+  return p.A + (long long)b * p.strideA;
+}
+__device__ __forceinline__ const int8_t* b_of_batch(const GemmParams& p, int b) {
+  if (p.kslices > 1) {
+    const int bb = b / p.kslices;
+    return p.B + (long long)bb * p.strideB + (long long)(b - bb * p.kslices) * p.strideBk;
+  }
+  return p.B + (long long)b * p.strideB;
+}
 
 // Offset of output element (m, n) of one batch; consecutive n stay consecutive inside a head, so vector
 // stores of VEC columns starting at a multiple of VEC are unaffected when out_d % VEC == 0.
@@ -220,7 +240,8 @@ int launch_gemm_group_s8(const GemmParams& shape, const GemmGroup& grp, hipStrea
 int launch_gemm(int kind, const GemmParams& p, void* workspace, long long workspace_bytes,
                 hipStream_t stream);
 long long gemm_workspace_bytes(long long M, long long N, long long K);
-int gemm_row_split(long long M, long long N, long long K);  // rows a linear cuts off its end and runs as a second problem
+int gemm_row_split(long long M, long long N, long long K);
+long long bmm_workspace_bytes(long long batch, long long M, long long N, long long K);  // split-K scratch of a batched product  // rows a linear cuts off its end and runs as a second problem
 void allow_fused_split_probe(bool allow);  // per thread: may a GEMM call run the one-time placement probe?
 int warm_fused_split(void* stream);        // run that probe now (1 = the one-launch split-K is usable on this device)
 int fused_split_faulted();                 // 1 = a one-launch split-K on the current device flagged a misplaced workgroup

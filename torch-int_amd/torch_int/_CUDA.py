@@ -44,6 +44,9 @@ _SIGNATURES = {
     "ti_bmm_s8t_s8n_f32t": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _f32, _vp],
     "ti_bmm_s8t_s8n_s8t": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _f32, _vp],
     "ti_bmm_s8t_s8n_s32t": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],
+    "ti_bmm_s8t_s8n_f32t_ws": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _f32, _vp, _i64, _vp],
+    "ti_bmm_s8t_s8n_s8t_ws": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _f32, _vp, _i64, _vp],
+    "ti_bmm_s8t_s8n_s32t_ws": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _i64, _vp],
     "ti_dq_add_layernorm_q": [_vp, _f32, _vp, _vp, _vp, _f32, _vp, _vp, _i64, _i64, _vp],
     "ti_dq_add_layernorm_q_f16": [_vp, _f32, _vp, _vp, _vp, _f32, _vp, _vp, _i64, _i64, _vp],
 }
@@ -64,6 +67,8 @@ def _load_library():
     lib.ti_init.restype = _int
     lib.ti_linear_workspace_bytes.argtypes = [_i64, _i64, _i64]
     lib.ti_linear_workspace_bytes.restype = _i64
+    lib.ti_bmm_workspace_bytes.argtypes = [_i64, _i64, _i64, _i64]
+    lib.ti_bmm_workspace_bytes.restype = _i64
     return lib
 
 
@@ -103,6 +108,8 @@ _LINEAR_CTYPES = {_K_B32: _lib.ti_linear_a8_w8_b32_o32, _K_B32S: _lib.ti_linear_
                   _K_RELU: _lib.ti_linear_relu_a8_w8_b8_o8, _K_F32_ACC: _lib.ti_linear_a8_w8_bfp32_ofp32_acc}
 _BMM_CTYPES = {_K_BMM_F32: _lib.ti_bmm_s8t_s8n_f32t, _K_BMM_S8: _lib.ti_bmm_s8t_s8n_s8t,
                _K_BMM_S32: _lib.ti_bmm_s8t_s8n_s32t}
+_BMM_WS_CTYPES = {_K_BMM_F32: _lib.ti_bmm_s8t_s8n_f32t_ws, _K_BMM_S8: _lib.ti_bmm_s8t_s8n_s8t_ws,
+                  _K_BMM_S32: _lib.ti_bmm_s8t_s8n_s32t_ws}
 
 
 def _fail(op, msg):
@@ -138,6 +145,17 @@ def _ws_bytes(M, N, K):
     n = _ws_need.get(key)
     if n is None:
         n = _ws_need[key] = int(_lib.ti_linear_workspace_bytes(M, N, K))
+    return n
+
+
+_bmm_ws_need = {}  # (batch, M, N, K) -> bytes of workspace the library can use for that batched product
+
+
+def _bmm_ws_bytes(batch, M, N, K):
+    key = (batch, M, N, K)
+    n = _bmm_ws_need.get(key)
+    if n is None:
+        n = _bmm_ws_need[key] = int(_lib.ti_bmm_workspace_bytes(batch, M, N, K))
     return n
 
 
@@ -290,7 +308,14 @@ def _bmm(op, kind, a, b, out_dtype, alpha):
         torch.cuda.set_device(idx)
     try:
         stream = _raw_stream(idx)
-        if _fast is not None:
+        # few output tiles and a long inner dimension (never an attention product): split-K with a workspace
+        need = _bmm_ws_bytes(batch, M, N, K) if K >= 1024 and M > 16 else 0
+        if need:
+            ws_ptr, ws_bytes = _workspace(idx, stream, need)
+            scal = () if kind == _K_BMM_S32 else (alpha,)
+            rc = _BMM_WS_CTYPES[kind](a.data_ptr(), b.data_ptr(), out.data_ptr(), batch, M, N, K, *scal, ws_ptr, ws_bytes,
+                                      stream or None)
+        elif _fast is not None:
             rc = _fast.bmm(kind, a.data_ptr(), b.data_ptr(), out.data_ptr(), batch, M, N, K, alpha, stream)
         else:
             scal = () if kind == _K_BMM_S32 else (alpha,)
