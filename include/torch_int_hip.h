@@ -374,6 +374,24 @@ int ti_attn_qk_softmax_q(const int8_t* q, const int8_t* k, const float* mask, in
                          int64_t S, int64_t D, int64_t stride_q, int64_t stride_k, int64_t heads, float alpha,
                          void* stream);
 
+/* Classes of an additive attention mask, an optional accelerator for the two prefill entry points above (no
+ * counterpart in the reference).  classes[b][i][j] describes the mask values of batch b, query rows 64 i .. 64 i + 63,
+ * keys 256 j .. 256 j + 255: 1 = all of them are +-0 (the kernels then do not read them), 2 = all of them are one
+ * and the same value, -1e30 or below (the row-maximum sweep of the long-prefill kernel then takes that value instead
+ * of loading keys and multiplying), 0 = anything else.  ti_attn_mask_classes fills the array (one read of the mask;
+ * ti_attn_mask_classes_bytes = its size, 0 when the shape takes none), once per mask: every head and every layer that
+ * adds the same mask shares it.  The _mc entry points are ti_attn_qk_softmax_q / ti_attn_prefill_s8 with that
+ * array (NULL = none); the bits of the results do not depend on it.  Under a causal mask only the tiles on the
+ * diagonal are class 0, which removes most of the mask traffic and half of the first sweep. */
+int64_t ti_attn_mask_classes_bytes(int64_t batch, int64_t T, int64_t S);
+int ti_attn_mask_classes(const float* mask, uint8_t* classes, int64_t batch, int64_t T, int64_t S, void* stream);
+int ti_attn_qk_softmax_q_mc(const int8_t* q, const int8_t* k, const float* mask, const uint8_t* mask_classes,
+                            int8_t* probs, int64_t BH, int64_t T, int64_t S, int64_t D, int64_t stride_q,
+                            int64_t stride_k, int64_t heads, float alpha, void* stream);
+int ti_attn_prefill_s8_mc(const int8_t* q, const int8_t* k, const int8_t* vt, const float* mask,
+                          const uint8_t* mask_classes, int8_t* ctx, int64_t BH, int64_t T, int64_t S, int64_t D,
+                          int64_t stride_q, int64_t stride_k, int64_t heads, float alpha_qk, float alpha_pv, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1227,3 +1227,71 @@ def test_fused_attention_long_keys_and_head_size_64():
     assert not X.can_attn_qk_softmax_q(z(2, 8, 64), z(2, 40, 64), None, 1, 2)      # S not a multiple of 16
     assert not X.can_attn_qk_softmax_q(z(1, 8, 64), z(1, 4112, 64), None, 1, 1)    # more than 4096 keys
     assert not X.can_attn_qk_softmax_q(z(2, 8, 32), z(2, 48, 32), None, 1, 2)      # head size 32
+
+
+def test_attention_mask_classes():
+    # the class array of a mask (per batch, 64 query rows, 256 keys: mixed / all zero / all one masked value) against
+    # a plain restatement, and the long-prefill kernel with and without it on masks built to sit on the class
+    # boundaries: same bytes either way, and those of the oracle
+    import ctypes
+    import torch_int._CUDA as C
+    import torch_int._hip_ext as X
+    lib = C._lib
+    neg = torch.finfo(torch.float32).min
+    B, H, T, S, d = 3, 2, 200, 784, 128            # 4 row blocks (the last one 8 rows), 4 key tiles (the last one 16 keys)
+    g = torch.Generator().manual_seed(141)
+    mask = torch.zeros(B, 1, T, S)
+    mask[0, 0, :64, 256:512] = neg                  # uniform
+    mask[0, 0, :64, 512:768] = -1e30                # uniform, exactly on the bound
+    mask[0, 0, 64:128, 0:256] = -9.9e29             # uniform but above the bound: mixed
+    mask[0, 0, 64:128, 256:512] = neg
+    mask[0, 0, 100, 300] = -3e38                    # one value differs: mixed
+    mask[0, 0, 128:192, 0:256] = -0.0               # negative zero counts as zero
+    mask[0, 0, 128:192, 256:512] = torch.randn(64, 256, generator=g)
+    mask[0, 0, 192:, 768:] = neg                    # ragged corner, uniform
+    mask[1, 0] = neg                                # everything masked: every row is a uniform distribution
+    mask[1, 0, 70:, :300] = 0.0
+    mask[2, 0] = torch.zeros(T, S).masked_fill(torch.arange(S)[None, :] > torch.arange(T)[:, None] + (S - T), neg)
+    mask[2, 0, :, :7] = neg                         # left padding on top of causality
+    n = lib.ti_attn_mask_classes_bytes(B, T, S)
+    assert n == B * 4 * 4
+    md = mask.to(DEV)
+    cls = X.mask_classes(md)
+    assert cls is not None and cls.numel() == n and X.mask_classes(md) is cls          # cached per mask tensor
+    want = torch.zeros(B, 4, 4, dtype=torch.uint8)
+    for b in range(B):
+        for i in range(4):
+            for j in range(4):
+                blk = mask[b, 0, 64 * i:64 * i + 64, 256 * j:256 * j + 256]
+                if (blk == 0).all():
+                    want[b, i, j] = 1
+                elif (blk.view(torch.int32) == blk.view(torch.int32).flatten()[0]).all() and blk.flatten()[0] <= -1e30:
+                    want[b, i, j] = 2
+    assert torch.equal(cls.cpu().view(B, 4, 4), want), (cls.cpu().view(B, 4, 4), want)
+    assert want[0, 0].tolist() == [1, 2, 2, 1] and want[0, 1].tolist() == [0, 0, 1, 1] and want[0, 2].tolist() == [1, 0, 1, 1]
+    assert want[0, 3, 3] == 2 and want[1, 0].tolist() == [2, 2, 2, 2] and want[1, 1].tolist() == [0, 0, 2, 2]
+    md[0, 0, 0, 0] = 1.0                            # an in-place change makes a new class array
+    assert X.mask_classes(md) is not cls and X.mask_classes(md)[0] == 0
+    md[0, 0, 0, 0] = 0.0
+    cls = X.mask_classes(md)
+
+    q, k, v = _s8(g, B * H, T, d), _s8(g, B * H, S, d), _s8(g, B * H, S, d)
+    a_qk, a_pv = 0.0007, 0.011
+    probs_ref = orc.attn_softmax_q(orc.bmm_s8t_s8n_f32t(q, k, a_qk), mask, H)
+    ctx_ref = orc.bmm_s8t_s8t_s8t(probs_ref, v, a_pv).view(B, H, T, d).transpose(1, 2).reshape(B, T, H * d)
+    qd, kd = q.to(DEV), k.to(DEV)
+    vt = X.transpose_last2(v.to(DEV))
+    stream = torch.cuda.current_stream().cuda_stream
+    for classes in (None, cls.data_ptr()):
+        _say("attention with mask classes:", classes is not None)
+        probs = torch.empty((B * H, T, S), dtype=torch.int8, device=DEV)
+        rc = lib.ti_attn_qk_softmax_q_mc(qd.data_ptr(), kd.data_ptr(), md.data_ptr(), classes, probs.data_ptr(), B * H, T, S, d,
+                                         T * d, S * d, H, a_qk, stream)
+        assert rc == 0, lib.ti_last_error()
+        assert (probs.cpu() != probs_ref).sum().item() == 0
+        ctx = torch.empty((B, T, H * d), dtype=torch.int8, device=DEV)
+        rc = lib.ti_attn_prefill_s8_mc(qd.data_ptr(), kd.data_ptr(), vt.data_ptr(), md.data_ptr(), classes, ctx.data_ptr(),
+                                       B * H, T, S, d, T * d, S * d, H, a_qk, a_pv, stream)
+        assert rc == 0, lib.ti_last_error()
+        assert (ctx.cpu() != ctx_ref).sum().item() == 0
+    assert probs_ref[2:4].max() > 0 and (probs_ref[2, 0] == probs_ref[2, 0, 0]).all()   # batch 1, row 0: all keys alike

@@ -526,9 +526,27 @@ int ti_attn_qk_softmax_q_supported(int64_t T, int64_t S, int64_t D) {
   return attn_qk_softmax_q_supported(T, S, D) ? 1 : 0;
 }
 
+int64_t ti_attn_mask_classes_bytes(int64_t batch, int64_t T, int64_t S) { return attn_mask_classes_bytes(batch, T, S); }
+
+int ti_attn_mask_classes(const float* mask, uint8_t* classes, int64_t batch, int64_t T, int64_t S, void* stream) {
+  g_err[0] = 0;
+  const char* op = "attn_mask_classes";
+  if (batch < 0 || T < 0 || S < 0) return fail(TI_ERR_INVALID_ARG, "%s: negative size", op);
+  if (batch == 0 || T == 0) return TI_OK;
+  if (int rc = check_ptr(op, "mask", mask, 16, true)) return rc;
+  if (int rc = check_ptr(op, "classes", classes, 1, true)) return rc;
+  return launch_attn_mask_classes(mask, classes, batch, T, S, static_cast<hipStream_t>(stream));
+}
+
 int ti_attn_qk_softmax_q(const int8_t* q, const int8_t* k, const float* mask, int8_t* probs, int64_t BH, int64_t T,
                          int64_t S, int64_t D, int64_t stride_q, int64_t stride_k, int64_t heads, float alpha,
                          void* stream) {
+  return ti_attn_qk_softmax_q_mc(q, k, mask, nullptr, probs, BH, T, S, D, stride_q, stride_k, heads, alpha, stream);
+}
+
+int ti_attn_qk_softmax_q_mc(const int8_t* q, const int8_t* k, const float* mask, const uint8_t* mask_classes,
+                            int8_t* probs, int64_t BH, int64_t T, int64_t S, int64_t D, int64_t stride_q,
+                            int64_t stride_k, int64_t heads, float alpha, void* stream) {
   g_err[0] = 0;
   const char* op = "attn_qk_softmax_q";
   const int64_t lim = 0x7fffffffLL;
@@ -548,12 +566,19 @@ int ti_attn_qk_softmax_q(const int8_t* q, const int8_t* k, const float* mask, in
   if (int rc = check_ptr(op, "mask", mask, 16, mask != nullptr)) return rc;
   if (int rc = check_ptr(op, "probs", probs, 16, true)) return rc;
   return launch_attn_qk_softmax_q(q, k, mask, probs, BH, T, S, D, stride_q, stride_k, heads, alpha, nullptr, nullptr,
-                                  0.0f, static_cast<hipStream_t>(stream));
+                                  0.0f, static_cast<hipStream_t>(stream), mask_classes);
 }
 
 int ti_attn_prefill_s8(const int8_t* q, const int8_t* k, const int8_t* vt, const float* mask, int8_t* ctx, int64_t BH,
                        int64_t T, int64_t S, int64_t D, int64_t stride_q, int64_t stride_k, int64_t heads,
                        float alpha_qk, float alpha_pv, void* stream) {
+  return ti_attn_prefill_s8_mc(q, k, vt, mask, nullptr, ctx, BH, T, S, D, stride_q, stride_k, heads, alpha_qk, alpha_pv,
+                               stream);
+}
+
+int ti_attn_prefill_s8_mc(const int8_t* q, const int8_t* k, const int8_t* vt, const float* mask,
+                          const uint8_t* mask_classes, int8_t* ctx, int64_t BH, int64_t T, int64_t S, int64_t D,
+                          int64_t stride_q, int64_t stride_k, int64_t heads, float alpha_qk, float alpha_pv, void* stream) {
   g_err[0] = 0;
   const char* op = "attn_prefill_s8";
   const int64_t lim = 0x7fffffffLL;
@@ -574,7 +599,7 @@ int ti_attn_prefill_s8(const int8_t* q, const int8_t* k, const int8_t* vt, const
   if (int rc = check_ptr(op, "mask", mask, 16, mask != nullptr)) return rc;
   if (int rc = check_ptr(op, "ctx", ctx, 4, true)) return rc;
   return launch_attn_qk_softmax_q(q, k, mask, nullptr, BH, T, S, D, stride_q, stride_k, heads, alpha_qk, vt, ctx,
-                                  alpha_pv, static_cast<hipStream_t>(stream));
+                                  alpha_pv, static_cast<hipStream_t>(stream), mask_classes);
 }
 
 int ti_decode_attn_supported(int64_t T, int64_t S, int64_t D) { return decode_attn_supported(T, S, D) ? 1 : 0; }

@@ -271,7 +271,7 @@ __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t*
 bool attn_long_supported(long long T, long long S, long long D);
 int launch_attn_long(const int8_t* q, const int8_t* k, const float* mask, int8_t* probs, long long BH, long long T,
                      long long S, long long D, long long stride_q, long long stride_k, long long heads, float alpha,
-                     const int8_t* vt, int8_t* ctx, float alpha_pv, hipStream_t stream);
+                     const int8_t* vt, int8_t* ctx, float alpha_pv, hipStream_t stream, const unsigned char* cls);
 
 // shapes the single-sweep kernel of this file takes (all keys of a head in the LDS at once)
 static bool single_sweep_ok(long long T, long long S, long long D, bool pv) {
@@ -305,10 +305,11 @@ static int launch_af(dim3 grid, size_t lds, hipStream_t stream, const int8_t* q,
 int launch_attn_qk_softmax_q(const int8_t* q, const int8_t* k, const float* mask, int8_t* probs, long long BH,
                              long long T, long long S, long long D, long long stride_q, long long stride_k,
                              long long heads, float alpha, const int8_t* vt, int8_t* ctx, float alpha_pv,
-                             hipStream_t stream) {
+                             hipStream_t stream, const unsigned char* mask_classes) {
   if (BH == 0 || T == 0) return TI_OK;
   if (!single_sweep_ok(T, S, D, vt != nullptr))
-    return launch_attn_long(q, k, mask, probs, BH, T, S, D, stride_q, stride_k, heads, alpha, vt, ctx, alpha_pv, stream);
+    return launch_attn_long(q, k, mask, probs, BH, T, S, D, stride_q, stride_k, heads, alpha, vt, ctx, alpha_pv, stream,
+                            mask_classes);
   const long long row_blocks = (T + AF_ROWS - 1) / AF_ROWS;
   if (BH * row_blocks > 0x7fffffffLL || T > 0x7fffffffLL)
     return fail(TI_ERR_INVALID_ARG, "attn_qk_softmax_q: too many row blocks (%lld)", BH * row_blocks);

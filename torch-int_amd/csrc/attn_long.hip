@@ -8,7 +8,8 @@
 //   sweep 1  x = max(alpha acc + mask, lowest), running row maximum, and per key tile whether anything in it can
 //            have a non-zero probability (exp underflows to exactly 0 below -87);
 //   sweep 2  e = exp(x - m) over the live tiles, partial sums -> 127 / sum;
-//   sweep 3  e again, p = rint(e * 127 / sum), and either the store of p or p . V on the spot.
+//   sweep 3  e again (only in blocks of keys where some probability can round to more than 0), p = rint(e * 127 / sum),
+//            and either the store of p or p . V on the spot.
 // Tiles that are dead for the whole workgroup (keys above the diagonal of a causal mask) are skipped in sweeps
 // 2 and 3: they add exact zeros.
 //
@@ -35,13 +36,46 @@ __device__ __forceinline__ int al_swz(int row, int c) {
   return D == 128 ? (c ^ ((row >> 1) & 7)) : (c ^ ((row >> 2) & 3));
 }
 
+// Classes of the additive mask, one per (batch, block of 64 query rows, tile of 256 keys), made once per mask by
+// mask_classes_kernel and shared by every head and layer that uses the mask: MIXED = read the mask values; ZERO =
+// every value is +-0 (adding it changes nothing: the mask is not read); UNIFORM = every value is the same number,
+// -1e30 or below (x = alpha acc + v is then v itself for any |alpha acc| < 1e12, since half an ulp of v is above
+// 3e22: the first sweep takes its maximum from one mask value and neither loads the keys nor multiplies).  Under a
+// causal mask only the tiles on the diagonal are MIXED.
+constexpr int MC_MIXED = 0, MC_ZERO = 1, MC_UNIFORM = 2;
+
+__global__ __launch_bounds__(256) void mask_classes_kernel(const float* __restrict__ mask, unsigned char* __restrict__ cls,
+                                                           int T, int S, int row_blocks, int ntiles) {
+  const int tile = blockIdx.x % ntiles;
+  const int rb = (blockIdx.x / ntiles) % row_blocks;
+  const long long b = blockIdx.x / (ntiles * row_blocks);
+  const int t0 = rb * AL_ROWS, k0 = tile * AL_TILE;
+  const int rows = T - t0 < AL_ROWS ? T - t0 : AL_ROWS;
+  const int quads = (S - k0 < AL_TILE ? S - k0 : AL_TILE) >> 2;  // S is a multiple of 16
+  const float* base = mask + (b * T + t0) * (long long)S + k0;
+  const int first = __float_as_int(base[0]);
+  bool zero = true, same = true;
+  for (int i = threadIdx.x; i < rows * quads; i += 256) {
+    const int row = i / quads, qd = i - row * quads;
+    const v4f v = *reinterpret_cast<const v4f*>(base + (long long)row * S + 4 * qd);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      zero = zero && v[e] == 0.0f;
+      same = same && __float_as_int(v[e]) == first;
+    }
+  }
+  const int all_zero = __syncthreads_and(zero), all_same = __syncthreads_and(same);
+  if (threadIdx.x == 0)
+    cls[blockIdx.x] = all_zero ? MC_ZERO : (all_same && __int_as_float(first) <= -1e30f) ? MC_UNIFORM : MC_MIXED;
+}
+
 template <int D, bool PV, bool MASKED>
 __global__ __launch_bounds__(256, 2) void attn_long_kernel(const int8_t* __restrict__ q, const int8_t* __restrict__ k,
                                                            const float* __restrict__ mask, int8_t* __restrict__ probs,
                                                            int T, int S, long long stride_q, long long stride_k,
                                                            int heads, int row_blocks, float alpha,
                                                            const int8_t* __restrict__ vt, int8_t* __restrict__ ctx,
-                                                           float alpha_pv) {
+                                                           float alpha_pv, const unsigned char* __restrict__ cls) {
   constexpr int CH = D / 16;       // 16-byte chunks per row
   constexpr int KS = D / 64;       // MFMAs (64 bytes of head dimension each) per block
   constexpr int RPI = 1024 / D;    // panel rows one copy instruction fills
@@ -57,6 +91,9 @@ __global__ __launch_bounds__(256, 2) void attn_long_kernel(const int8_t* __restr
   const int t0 = (row_blocks - 1 - (int)(blockIdx.x / n_bh)) * AL_ROWS;  // heaviest blocks of a causal mask first
   const int ntiles = (S + AL_TILE - 1) / AL_TILE;
   const int r = lane & 15, g = lane >> 4;
+  // mask classes of this workgroup's row block (nullptr: every tile MIXED)
+  const unsigned char* cls_row = MASKED && cls != nullptr ? cls + ((bh / heads) * row_blocks + t0 / AL_ROWS) * ntiles : nullptr;
+  auto tile_class = [&](int tile) { return cls_row != nullptr ? (int)cls_row[tile] : MC_MIXED; };
 
   const int8_t* qb = q + bh * stride_q;
   const int8_t* kb = k + bh * stride_k;
@@ -103,7 +140,7 @@ __global__ __launch_bounds__(256, 2) void attn_long_kernel(const int8_t* __restr
   // x of one tile: acc[j][v] <- bits of max(alpha * (q . k) + mask, lowest) for block j, keys 16 j + 4 g + v
   v4i acc[16];
   v4i qf[KS];
-  auto tile_scores = [&](int tile, auto nb_) __attribute__((always_inline)) {
+  auto tile_scores = [&](int tile, auto nb_, bool use_mask) __attribute__((always_inline)) {
     const int nb = nb_;
     const int k0 = tile * AL_TILE;
 #pragma unroll
@@ -123,7 +160,7 @@ __global__ __launch_bounds__(256, 2) void attn_long_kernel(const int8_t* __restr
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
         dst[u] = v4f{0.f, 0.f, 0.f, 0.f};
-        if (MASKED && j0 + u < nb) dst[u] = *reinterpret_cast<const v4f*>(mrow + k0 + 16 * (j0 + u) + 4 * g);
+        if (MASKED && use_mask && j0 + u < nb) dst[u] = *reinterpret_cast<const v4f*>(mrow + k0 + 16 * (j0 + u) + 4 * g);
       }
     };
     fetch_mask(0, mk[0]);
@@ -138,7 +175,7 @@ __global__ __launch_bounds__(256, 2) void attn_long_kernel(const int8_t* __restr
 #pragma unroll
           for (int v = 0; v < 4; ++v) {
             float x = Epi<EPI_F32_SCALE>::apply(acc[j][v], 0.0f, alpha);
-            if (MASKED) x = x + mk[cur][u][v];
+            if (MASKED && use_mask) x = x + mk[cur][u][v];
             x = __builtin_fmaxf(x, lowest);  // NaN included
             acc[j][v] = __float_as_int(x);
           }
@@ -167,19 +204,33 @@ __global__ __launch_bounds__(256, 2) void attn_long_kernel(const int8_t* __restr
   float tmax[AL_MAX_TILES];
 #pragma unroll
   for (int i = 0; i < AL_MAX_TILES; ++i) tmax[i] = lowest;
+  bool have_q = false;  // the query fragments are read after the first wait that covers the copy of the Q tile
+  auto read_q = [&]() {
+    if (!have_q) {
+#pragma unroll
+      for (int s = 0; s < KS; ++s) qf[s] = *reinterpret_cast<const v4i*>(qs + (al_swz<D>(wave * 16 + r, 4 * s + g) << 4));
+      have_q = true;
+    }
+  };
 #pragma unroll 1
   for (int tile = 0; tile < ntiles; ++tile) {
+    const int mc = tile_class(tile);
+    if (MASKED && mc == MC_UNIFORM) {  // every x of the tile is this one mask value (uniform over the workgroup)
+      const float v = __builtin_fmaxf(mrow[tile * AL_TILE], lowest);
+      m = __builtin_fmaxf(m, v);
+#pragma unroll
+      for (int i = 0; i < AL_MAX_TILES; ++i)
+        if (i == tile) tmax[i] = v;
+      continue;
+    }
     __syncthreads();  // every wave is done with the previous tile
     load_k_tile(tile);
     asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
-    if (tile == 0) {
-#pragma unroll
-      for (int s = 0; s < KS; ++s) qf[s] = *reinterpret_cast<const v4i*>(qs + (al_swz<D>(wave * 16 + r, 4 * s + g) << 4));
-    }
+    read_q();
     float top = lowest;
     auto body0 = [&](auto nb_) __attribute__((always_inline)) {
       const int nb = nb_;
-      tile_scores(tile, nb_);
+      tile_scores(tile, nb_, mc != MC_ZERO);
 #pragma unroll
       for (int j = 0; j < 16; ++j)
         if (j < nb)
@@ -217,10 +268,12 @@ __global__ __launch_bounds__(256, 2) void attn_long_kernel(const int8_t* __restr
     __syncthreads();
     load_k_tile(tile);
     asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+    read_q();
     if (!(live_w >> tile & 1)) continue;  // uniform over the wave: every e is 0, p + 0 = p
+    const bool use_mask = tile_class(tile) != MC_ZERO;
     auto body1 = [&](auto nb_) __attribute__((always_inline)) {
       const int nb = nb_;
-      tile_scores(tile, nb_);
+      tile_scores(tile, nb_, use_mask);
 #pragma unroll
       for (int j = 0; j < 16; ++j) {
         if (j < nb) {
@@ -245,6 +298,12 @@ __global__ __launch_bounds__(256, 2) void attn_long_kernel(const int8_t* __restr
   sum = sum + __shfl_xor(sum, 32, 64);
   sum = sum + __shfl_xor(sum, 16, 64);
   const float scale = 127.0f / sum;
+  // Sweep 3 needs an exponential only where the probability can be non-zero: p = rint(e * scale) is 0 whenever
+  // e * scale < 0.5.  With x - m <= ln(0.45 / scale) - 0.02 the exponential is below 0.442 / scale (its error is
+  // parts per million, the logarithm's as well), the product below 0.45, the rounded value 0: skipping such values
+  // changes no bit.  The row maximum itself contributes e = 1, so sum >= 1, scale <= 127 and the bound is at most
+  // -5.6: in a peaked row nearly every block of sixteen keys falls under it for all sixteen rows of the wave.
+  const float skip_below = __builtin_fmaxf(__logf(0.45f / scale) - 0.02f, -87.0f);
 
   // ---- sweep 3: probabilities, stored or multiplied with V
   v4i o[CH];
@@ -260,22 +319,24 @@ __global__ __launch_bounds__(256, 2) void attn_long_kernel(const int8_t* __restr
       load_k_tile(tile);
       load_v_tile(tile);
       asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+      read_q();
     }
     const bool wave_live = live_w >> tile & 1;
     if (PV && !wave_live) continue;
+    const bool use_mask = tile_class(tile) != MC_ZERO;
     auto body2 = [&](auto nb_) __attribute__((always_inline)) {
       const int nb = nb_;
       unsigned pw[16];
 #pragma unroll
       for (int j = 0; j < 16; ++j) pw[j] = 0;
       if (wave_live) {
-        tile_scores(tile, nb_);
+        tile_scores(tile, nb_, use_mask);
 #pragma unroll
         for (int j = 0; j < 16; ++j) {
           if (j < nb) {
             const float top = __builtin_fmaxf(__builtin_fmaxf(__int_as_float(acc[j][0]), __int_as_float(acc[j][1])),
                                               __builtin_fmaxf(__int_as_float(acc[j][2]), __int_as_float(acc[j][3])));
-            if (__builtin_amdgcn_ballot_w64(top - m > -87.0f) != 0) {
+            if (__builtin_amdgcn_ballot_w64(top - m > skip_below) != 0) {
               unsigned w = 0;
 #pragma unroll
               for (int v = 0; v < 4; ++v) {
@@ -290,7 +351,10 @@ __global__ __launch_bounds__(256, 2) void attn_long_kernel(const int8_t* __restr
       if constexpr (PV) {
 #pragma unroll
         for (int sl = 0; sl < 4; ++sl) {
-          if (4 * sl < nb) {
+          // (a slice of 64 keys whose probabilities are zero in all sixteen rows of the wave adds nothing: its V^T
+          // fragments are not even read)
+          if (4 * sl < nb &&
+              __builtin_amdgcn_ballot_w64((pw[4 * sl] | pw[4 * sl + 1] | pw[4 * sl + 2] | pw[4 * sl + 3]) != 0) != 0) {
             const v4i pa = {(int)pw[4 * sl], (int)pw[4 * sl + 1], (int)pw[4 * sl + 2], (int)pw[4 * sl + 3]};
 #pragma unroll
             for (int c = 0; c < CH; ++c) {
@@ -336,14 +400,14 @@ bool attn_long_supported(long long T, long long S, long long D) {
 template <int D, bool PV, bool MASKED>
 static int launch_al(dim3 grid, hipStream_t stream, const int8_t* q, const int8_t* k, const float* mask, int8_t* probs,
                      int T, int S, long long stride_q, long long stride_k, int heads, int row_blocks, float alpha,
-                     const int8_t* vt, int8_t* ctx, float alpha_pv) {
+                     const int8_t* vt, int8_t* ctx, float alpha_pv, const unsigned char* cls) {
   auto kern = attn_long_kernel<D, PV, MASKED>;
   constexpr int lds = AL_ROWS * D + AL_TILE * D + (PV ? D * AL_VPITCH : 0) + 16;
   static_assert(2 * lds <= 160 * 1024, "two workgroups per CU");
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
   if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "attn_long: LDS limit: %s", hipGetErrorString(e));
   hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, q, k, mask, probs, T, S, stride_q, stride_k, heads, row_blocks,
-                     alpha, vt, ctx, alpha_pv);
+                     alpha, vt, ctx, alpha_pv, cls);
   e = hipGetLastError();
   if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "attn_long launch: %s", hipGetErrorString(e));
   return TI_OK;
@@ -352,8 +416,10 @@ static int launch_al(dim3 grid, hipStream_t stream, const int8_t* q, const int8_
 // vt == nullptr: probabilities into probs ([BH, T, S]).  Otherwise context into ctx ([BH / heads, T, heads * D]).
 int launch_attn_long(const int8_t* q, const int8_t* k, const float* mask, int8_t* probs, long long BH, long long T,
                      long long S, long long D, long long stride_q, long long stride_k, long long heads, float alpha,
-                     const int8_t* vt, int8_t* ctx, float alpha_pv, hipStream_t stream) {
+                     const int8_t* vt, int8_t* ctx, float alpha_pv, hipStream_t stream, const unsigned char* cls) {
   if (BH == 0 || T == 0) return TI_OK;
+  // the UNIFORM class stands for "adding alpha acc to the mask value leaves the mask value": not for absurd scales
+  if (mask == nullptr || !(alpha >= -1e12f && alpha <= 1e12f)) cls = nullptr;
   if (!attn_long_supported(T, S, D))
     return fail(TI_ERR_INVALID_ARG, "attn_long: unsupported shape (T=%lld S=%lld head_dim=%lld)", T, S, D);
   const long long row_blocks = (T + AL_ROWS - 1) / AL_ROWS;
@@ -363,9 +429,9 @@ int launch_attn_long(const int8_t* q, const int8_t* k, const float* mask, int8_t
 #define TI_AL(DD, PV)                                                                                                 \
   return mask != nullptr                                                                                              \
              ? launch_al<DD, PV, true>(grid, stream, q, k, mask, probs, (int)T, (int)S, stride_q, stride_k, (int)heads,  \
-                                       (int)row_blocks, alpha, vt, ctx, alpha_pv)                                     \
+                                       (int)row_blocks, alpha, vt, ctx, alpha_pv, cls)                                \
              : launch_al<DD, PV, false>(grid, stream, q, k, mask, probs, (int)T, (int)S, stride_q, stride_k, (int)heads, \
-                                        (int)row_blocks, alpha, vt, ctx, alpha_pv)
+                                        (int)row_blocks, alpha, vt, ctx, alpha_pv, nullptr)
   if (D == 128) {
     if (vt == nullptr) TI_AL(128, false);
     TI_AL(128, true);
@@ -373,6 +439,23 @@ int launch_attn_long(const int8_t* q, const int8_t* k, const float* mask, int8_t
   if (vt == nullptr) TI_AL(64, false);
   TI_AL(64, true);
 #undef TI_AL
+}
+
+// Bytes of the class array of a mask [batch, 1, T, S] (0: the shape takes no classes), and the launch that fills it.
+long long attn_mask_classes_bytes(long long batch, long long T, long long S) {
+  if (batch <= 0 || T <= 0 || S < 16 || S % 16 != 0 || S > (long long)AL_TILE * AL_MAX_TILES) return 0;
+  return batch * ((T + AL_ROWS - 1) / AL_ROWS) * ((S + AL_TILE - 1) / AL_TILE);
+}
+int launch_attn_mask_classes(const float* mask, unsigned char* cls, long long batch, long long T, long long S,
+                             hipStream_t stream) {
+  const long long n = attn_mask_classes_bytes(batch, T, S);
+  if (n == 0) return fail(TI_ERR_INVALID_ARG, "attn_mask_classes: unsupported shape (batch=%lld T=%lld S=%lld)", batch, T, S);
+  if (n > 0x7fffffffLL) return fail(TI_ERR_INVALID_ARG, "attn_mask_classes: too many blocks (%lld)", n);
+  hipLaunchKernelGGL(mask_classes_kernel, dim3((unsigned)n), dim3(256), 0, stream, mask, cls, (int)T, (int)S,
+                     (int)((T + AL_ROWS - 1) / AL_ROWS), (int)((S + AL_TILE - 1) / AL_TILE));
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "attn_mask_classes launch: %s", hipGetErrorString(e));
+  return TI_OK;
 }
 
 #undef TI_FOR_BLOCKS_OF

@@ -280,6 +280,9 @@ bool attn_qk_softmax_q_supported(long long T, long long S, long long D);
 int launch_attn_qk_softmax_q(const int8_t* q, const int8_t* k, const float* mask, int8_t* probs, long long BH,
                              long long T, long long S, long long D, long long stride_q, long long stride_k,
                              long long heads, float alpha, const int8_t* vt, int8_t* ctx, float alpha_pv,
+                             hipStream_t stream, const unsigned char* mask_classes = nullptr);
+long long attn_mask_classes_bytes(long long batch, long long T, long long S);
+int launch_attn_mask_classes(const float* mask, unsigned char* cls, long long batch, long long T, long long S,
                              hipStream_t stream);
 bool decode_attn_supported(long long T, long long S, long long D);
 int launch_decode_attn_s8(const int8_t* q, const int8_t* k_new, const int8_t* v_new, int8_t* k_buf, int8_t* v_buf,

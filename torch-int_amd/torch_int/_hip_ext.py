@@ -47,6 +47,14 @@ _lib.ti_attn_qk_softmax_q.argtypes = [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64
 _lib.ti_attn_qk_softmax_q.restype = ctypes.c_int
 _lib.ti_attn_prefill_s8.argtypes = [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _f32, _vp]
 _lib.ti_attn_prefill_s8.restype = ctypes.c_int
+_lib.ti_attn_qk_softmax_q_mc.argtypes = [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _vp]
+_lib.ti_attn_qk_softmax_q_mc.restype = ctypes.c_int
+_lib.ti_attn_prefill_s8_mc.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _f32, _vp]
+_lib.ti_attn_prefill_s8_mc.restype = ctypes.c_int
+_lib.ti_attn_mask_classes_bytes.argtypes = [_i64, _i64, _i64]
+_lib.ti_attn_mask_classes_bytes.restype = _i64
+_lib.ti_attn_mask_classes.argtypes = [_vp, _vp, _i64, _i64, _i64, _vp]
+_lib.ti_attn_mask_classes.restype = ctypes.c_int
 _lib.ti_decode_attn_supported.argtypes = [_i64, _i64, _i64]
 _lib.ti_decode_attn_supported.restype = ctypes.c_int
 _lib.ti_decode_attn_s8.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32,
@@ -351,6 +359,41 @@ def can_attn_qk_softmax_q(q, k, mask, bsz, heads):
                             and mask.data_ptr() % 16 == 0)
 
 
+_mask_classes_cache = {}  # id(mask) -> (weak reference, version counter, classes tensor)
+
+
+def mask_classes(mask):
+    """The class array of an additive fp32 mask [bsz, 1, T, S] for the long-prefill attention kernel (which tiles of
+    64 rows x 256 keys are all zero / all one masked value / mixed), or None when the shape takes none.  Made once per
+    mask tensor and version: every head and every layer of a forward pass adds the same mask."""
+    import weakref
+    key = id(mask)
+    hit = _mask_classes_cache.get(key)
+    if hit is not None and hit[0]() is mask and hit[1] == mask._version:
+        return hit[2]
+    bsz, _, T, S = mask.shape
+    n = _lib.ti_attn_mask_classes_bytes(bsz, T, S)
+    if n <= 0:
+        return None
+    cls = torch.empty(n, dtype=torch.uint8, device=mask.device)
+    with _on(mask.device):
+        rc = _lib.ti_attn_mask_classes(mask.data_ptr(), cls.data_ptr(), bsz, T, S, _raw_stream(mask.device.index) or None)
+    if rc:
+        raise RuntimeError(f"torch_int._hip_ext.mask_classes: {_lib.ti_last_error().decode()} (status {rc})")
+    if len(_mask_classes_cache) >= 64:
+        _mask_classes_cache.clear()
+    _mask_classes_cache[key] = (weakref.ref(mask, lambda _r, k=key: _mask_classes_cache.pop(k, None)), mask._version, cls)
+    return cls
+
+
+def _classes_ptr(mask, S):
+    """Pointer to the mask's class array where the kernel that will run reads one (more than 512 keys), else None."""
+    if mask is None or S <= 512:
+        return None
+    cls = mask_classes(mask)
+    return cls.data_ptr() if cls is not None else None
+
+
 def attn_qk_softmax_q(q, k, mask, alpha, heads, checked=False):
     """int8 round(127 softmax(alpha q k^T + mask)) [bsz*heads, T, S] in one launch: the values of
     ``attn_softmax_q(bmm_s8t_s8n_f32t(q, k, alpha), mask, heads)`` without the fp32 scores in memory."""
@@ -362,9 +405,9 @@ def attn_qk_softmax_q(q, k, mask, alpha, heads, checked=False):
     dev = q.device
     probs = torch.empty((BH, T, S), dtype=torch.int8, device=dev)
     with _on(dev):
-        rc = _lib.ti_attn_qk_softmax_q(q.data_ptr(), k.data_ptr(), mask.data_ptr() if mask is not None else None,
-                                       probs.data_ptr(), BH, T, S, d, T * d, k.stride(0), heads, alpha,
-                                       _raw_stream(dev.index) or None)
+        rc = _lib.ti_attn_qk_softmax_q_mc(q.data_ptr(), k.data_ptr(), mask.data_ptr() if mask is not None else None,
+                                          _classes_ptr(mask, S), probs.data_ptr(), BH, T, S, d, T * d, k.stride(0), heads,
+                                          alpha, _raw_stream(dev.index) or None)
     if rc:
         raise RuntimeError(f"torch_int._hip_ext.attn_qk_softmax_q: {_lib.ti_last_error().decode()} (status {rc})")
     return probs
@@ -388,9 +431,10 @@ def attn_prefill(q, k, vt, mask, alpha_qk, alpha_pv, heads, checked=False):
     dev = q.device
     ctx = torch.empty((BH // heads, T, heads * d), dtype=torch.int8, device=dev)
     with _on(dev):
-        rc = _lib.ti_attn_prefill_s8(q.data_ptr(), k.data_ptr(), vt.data_ptr(),
-                                     mask.data_ptr() if mask is not None else None, ctx.data_ptr(), BH, T, S, d, T * d,
-                                     k.stride(0), heads, alpha_qk, alpha_pv, _raw_stream(dev.index) or None)
+        rc = _lib.ti_attn_prefill_s8_mc(q.data_ptr(), k.data_ptr(), vt.data_ptr(),
+                                        mask.data_ptr() if mask is not None else None, _classes_ptr(mask, S),
+                                        ctx.data_ptr(), BH, T, S, d, T * d, k.stride(0), heads, alpha_qk, alpha_pv,
+                                        _raw_stream(dev.index) or None)
     if rc:
         raise RuntimeError(f"torch_int._hip_ext.attn_prefill: {_lib.ti_last_error().decode()} (status {rc})")
     return ctx
