@@ -54,7 +54,7 @@ FAMILIES = {
 # The counter runs behind FAMILIES[*]["traffic"] were made on the kernels as this hash of their source file describes
 # them (first 16 hex digits of the SHA-256 of torch-int_amd/csrc/gemm_s8_impl.h).  When the file has changed since,
 # the bench line says so next to the figure instead of passing an old measurement off as current.
-TRAFFIC_SOURCE_SHA16 = "e6c2c36dc989644a"
+TRAFFIC_SOURCE_SHA16 = "69043ebc0ef2aa5e"
 
 
 def traffic_is_current():
