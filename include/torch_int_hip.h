@@ -66,7 +66,7 @@ int64_t ti_linear_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int ti_linear_row_split(int64_t M, int64_t N, int64_t K);
 
 /* Diagnostics: the kernel family the calling thread's last linear / bmm_s8t_s8n_* call launched
- * ("pipe_256x256", "pipe16_256x160", "pipe16_256x288", "pipe16_256x128", "pipe16_128x80", "pipe16_128x192", "pipe_128x128",
+ * ("pipe_256x256", "pipe16_256x160", "pipe16_256x288", "pipe16_256x128", "pipe16_128x80", "pipe16_128x192", "pipe16_256x192", "pipe_128x128",
  * "splitk_<tile>" and "fusedk_<tile>" for the two- and one-launch split-K forms, "stream", "skinny", "tile_*",
  * "scalar"; grouped launches add "_group": "stream_group", "pipe16_256x160_group", "pipe16_256x288_group",
  * "pipe16_256x128_group"; "<family>+<family>" when the last rows ran as a second problem, see ti_linear_row_split;
@@ -126,6 +126,15 @@ int64_t ti_diag_mfma_loop_ops(int64_t iters);
  * and addresses of the 256x160 GEMM kernel's 32-bit epilogue and nothing else: a benchmark times it to learn what
  * one CU (few workgroups) or the whole chip (one workgroup per CU) can store. */
 int ti_diag_store_loop(float* out, int64_t M, int64_t N, int workgroups, int reps, void* stream);
+
+/* Diagnostic (no counterpart in the reference; computes nothing): one workgroup of eight waves per CU fetches, `iters`
+ * times, 48 KiB (a 256x160 tile's share of one 128-byte K step) as row pieces of 128 contiguous bytes from rows 5120
+ * bytes apart in the first 2 MiB of `data` (device memory, at least 2 MiB, 16-byte aligned; shared by all workgroups,
+ * so it is served by the L2), two steps in flight.  mode 0: global->LDS copies; 1: 16-byte loads into registers.  A
+ * benchmark times it to learn what the copy path alone delivers per CU.  `sink` as for ti_diag_mfma_loop.
+ * ti_diag_copy_loop_bytes(iters) = bytes one such launch fetches on the current device. */
+int ti_diag_copy_loop(int mode, const int8_t* data, int64_t data_bytes, int64_t iters, int32_t* sink, void* stream);
+int64_t ti_diag_copy_loop_bytes(int64_t iters);
 
 /* ---- W8A8 linear: out[M,N] = epilogue(x[M,K] . w[N,K]^T, bias[N]) ---- */
 

@@ -135,6 +135,7 @@ def test_every_gemm_kernel_family_is_reached_and_exact(two_launch_split_k):
               ((768, 3072, 11648), "splitk_256x256"), ((256, 3072, 7744), "splitk_256x256"),  # 128- and 64-byte steps
               ((128, 1024, 4096), "splitk_128x128"), ((256, 2048, 11648), "splitk_128x128"),
               ((512, 3072, 1024), "splitk_128x192"), ((128, 768, 4096), "splitk_128x192"), ((512, 12288, 2048), "pipe16_128x192"),
+              ((1024, 12288, 1024), "pipe16_256x192"), ((256, 49152, 1024), "pipe16_256x192"),
               ((16, 5120, 3072), "stream"), ((3, 4608, 16384), "stream"), ((3, 100, 272), "skinny"), ((300, 200, 48), "tile_64x64"),
               ((2100, 5000, 272), "tile_256x256"), ((1024, 2048, 80), "tile_128x128"), ((70, 50, 37), "scalar")]
     for (M, N, K), family in expect:
@@ -761,7 +762,7 @@ def test_linear_accumulate_into_output(two_launch_split_k):
                       (2048, 4096, 2048),   # 256x128 tiles
                       (4096, 2816, 1024), (1024, 2048, 64), (1024, 5120, 5120), (1024, 4608, 3584), (256, 3072, 7744),
                       (1024, 9216, 9216), (384, 2880, 4608), (4, 4608, 16384), (256, 3200, 11648), (256, 1600, 11648), (384, 2560, 1024),
-                      (128, 640, 4096), (128, 768, 4096), (128, 1024, 4096), (512, 12288, 2048), (16, 5120, 3072), (3, 100, 272), (300, 200, 48), (2100, 5000, 272),
+                      (128, 640, 4096), (128, 768, 4096), (128, 1024, 4096), (512, 12288, 2048), (1024, 12288, 1024), (16, 5120, 3072), (3, 100, 272), (300, 200, 48), (2100, 5000, 272),
                       (70, 50, 37), (4, 64, 0)]:
         _say(f"linear += M={M} N={N} K={K}")
         x, w = _s8(g, M, K), _s8(g, N, K)
@@ -773,7 +774,7 @@ def test_linear_accumulate_into_output(two_launch_split_k):
         assert out.data_ptr() == inout.data_ptr()
         assert _ulp_diff(out.cpu(), ref) == 0, (M, N, K)
         seen.add(C._lib.ti_last_kernel().decode())
-    assert {"pipe16_256x160", "pipe16_256x288", "pipe16_256x128", "pipe16_128x80", "pipe16_128x192", "pipe_256x256", "pipe_128x128", "splitk_256x256", "splitk_256x160",
+    assert {"pipe16_256x160", "pipe16_256x288", "pipe16_256x128", "pipe16_128x80", "pipe16_128x192", "pipe16_256x192", "pipe_256x256", "pipe_128x128", "splitk_256x256", "splitk_256x160",
             "splitk_256x288", "splitk_128x160", "splitk_128x288", "splitk_128x80", "splitk_128x192", "splitk_128x128", "stream", "skinny", "tile_64x64", "tile_256x256", "scalar"} <= seen, seen
     # the module route: W8A8BFP32OFP32Linear(x, add_to=residual)
     from torch_int.nn.linear import W8A8BFP32OFP32Linear
@@ -833,7 +834,7 @@ def test_head_major_projection_through_every_kernel_family(two_launch_split_k):
     for (B, T, H, d, K) in [(4, 512, 40, 128, 256), (4, 512, 40, 128, 192), (2, 1000, 72, 128, 192), (2, 1000, 72, 128, 256),
                             (8, 512, 22, 128, 128), (8, 512, 22, 128, 192), (2, 512, 16, 128, 64),
                             (2, 512, 40, 128, 5120), (2, 512, 36, 128, 3584), (2, 512, 72, 128, 9216), (1, 384, 90, 32, 4608),
-                            (1, 256, 24, 128, 7744), (2, 64, 5, 128, 4096), (1, 256, 25, 128, 11648), (1, 256, 25, 64, 11648), (1, 384, 20, 128, 1024), (1, 128, 6, 128, 4096), (1, 128, 8, 128, 4096), (4, 128, 96, 128, 2048), (1, 16, 40, 128, 3072), (1, 3, 5, 32, 272),
+                            (1, 256, 24, 128, 7744), (2, 64, 5, 128, 4096), (1, 256, 25, 128, 11648), (1, 256, 25, 64, 11648), (1, 384, 20, 128, 1024), (1, 128, 6, 128, 4096), (1, 128, 8, 128, 4096), (4, 128, 96, 128, 2048), (2, 512, 96, 128, 1024), (1, 16, 40, 128, 3072), (1, 3, 5, 32, 272),
                             (3, 100, 5, 48, 48), (3, 700, 39, 128, 272), (2, 35, 3, 16, 37)]:
         M, N = B * T, H * d
         _say(f"head-major linear bsz={B} seq={T} heads={H} d={d} K={K}")
@@ -844,7 +845,7 @@ def test_head_major_projection_through_every_kernel_family(two_launch_split_k):
         assert out.shape == (B, H, T, d) and out.is_contiguous()
         assert torch.equal(out.cpu(), ref), (B, T, H, d, K)
         seen.add(C._lib.ti_last_kernel().decode())
-    assert {"pipe16_256x160", "pipe16_256x288", "pipe16_128x80", "pipe16_128x192", "pipe_256x256", "pipe_128x128", "splitk_256x256", "splitk_256x160",
+    assert {"pipe16_256x160", "pipe16_256x288", "pipe16_128x80", "pipe16_128x192", "pipe16_256x192", "pipe_256x256", "pipe_128x128", "splitk_256x256", "splitk_256x160",
             "splitk_256x288", "splitk_128x160", "splitk_128x288", "splitk_128x80", "splitk_128x192", "splitk_128x128", "stream", "skinny", "tile_64x64", "tile_256x256", "scalar"} <= seen, seen
     with pytest.raises(RuntimeError):
         X.linear_a8_w8_b8_o8_heads(x.to(DEV), w.to(DEV), b.to(DEV), alpha, beta, 2, 35, 6, 8)   # d not a multiple of 16

@@ -12,6 +12,7 @@ Examples
   python torch-int_amd/benchmark/bench_kernel.py --op mfma_loop --shape 2 20000 --pattern random --iters 200
       # matrix-pipe ceiling: mode (0 MFMA only, 1 + LDS reads, 2 + LDS-DMA copies and barrier), steps per wave
   python torch-int_amd/benchmark/bench_kernel.py --op mfma_ceiling --shape 250    # all six figures, 250 ms windows
+  python torch-int_amd/benchmark/bench_kernel.py --op copy_loop --shape 0 4000     # L2 -> CU copy rate: mode (0 into LDS, 1 into registers), steps
   rocprofv3 --kernel-trace --stats --output-format csv -d out -- python3 .../bench_kernel.py --op ...
 
 Prints one JSON line: mean microseconds per call (HIP events on the launch stream), algorithmic
@@ -42,7 +43,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--op", required=True, choices=list(LINEAR) + ["bmm_f32t", "bmm_s8t", "bmm_s32t", "bmm_s8t_rowmajor", "ln_q", "ln_q_f16", "add_ln_q",
                                                "softmax_q", "qk_softmax_q", "attn_prefill", "decode_attn", "transpose_last2", "copy",
-                                               "mfma_loop", "mfma_ceiling", "store_loop"])
+                                               "mfma_loop", "mfma_ceiling", "store_loop", "copy_loop"])
     ap.add_argument("--shape", type=int, nargs="+", required=True)
     ap.add_argument("--iters", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
@@ -188,6 +189,12 @@ def main():
         out = torch.empty(M, N, device=dev)
         nbytes = float(X.diag_store_loop(out, workgroups, reps))
         fn = lambda: X.diag_store_loop(out, workgroups, reps)  # noqa: E731
+    elif args.op == "copy_loop":
+        # every CU fetches 48 KiB per step from an L2-resident 2 MiB with the mainloop's access pattern, nothing else
+        mode, steps = args.shape
+        data, sink = s8(2 << 20), torch.zeros(1, dtype=torch.int32, device=dev)
+        nbytes = float(X.diag_copy_loop(mode, data, steps, sink))
+        fn = lambda: X.diag_copy_loop(mode, data, steps, sink)  # noqa: E731
     else:  # plain device copy of a known size: reference reading for FETCH_SIZE / WRITE_SIZE
         n, = args.shape
         src = torch.empty(n, dtype=torch.uint8, device=dev).random_(generator=g)

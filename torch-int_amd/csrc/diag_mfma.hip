@@ -145,4 +145,58 @@ int launch_diag_store_loop(float* out, long long M, long long N, int workgroups,
   return TI_OK;
 }
 
+// Copy-rate diagnostic: what one CU moves from the L2 with the GEMM mainloop's access pattern and nothing else.  One
+// workgroup of 8 waves per CU; per step a wave fetches six row pieces of 128 contiguous bytes per 8-lane group (48 KiB
+// per workgroup and step, a 256x160 tile's K step) from rows 5120 bytes apart, two steps in flight; the 2 MiB source is
+// shared by all workgroups and stays in the L2.
+//   mode 0  global->LDS copies (global_load_lds_dwordx4) into three rotating LDS stages
+//   mode 1  16-byte loads into registers, folded with xor
+static constexpr int kCopyPieces = 6, kCopyPitch = 5120;
+template <int MODE>
+__global__ __launch_bounds__(512) void copy_loop_kernel(const int8_t* __restrict__ data, int iters, int* sink) {
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const char* src[kCopyPieces];
+#pragma unroll
+  for (int j = 0; j < kCopyPieces; ++j)
+    src[j] = reinterpret_cast<const char*>(data) + (size_t)((wave * kCopyPieces + j) * 8 + lane / 8) * kCopyPitch +
+             (lane % 8) * 16;
+  v4i acc = {0, 0, 0, 0};
+  int koff = 0;
+  for (int it = 0; it < iters; ++it) {
+    if (MODE == 0) {
+      TI_LDS_AS char* dst = (TI_LDS_AS char*)smem + (it % 3) * (8 * kCopyPieces * 1024) + wave * kCopyPieces * 1024;
+#pragma unroll
+      for (int j = 0; j < kCopyPieces; ++j)
+        __builtin_amdgcn_global_load_lds((const TI_GLOBAL_AS void*)(src[j] + koff), (TI_LDS_AS void*)(dst + j * 1024),
+                                         16, 0, 0);
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kCopyPieces) : "memory");
+    } else {
+      v4i v[kCopyPieces];
+#pragma unroll
+      for (int j = 0; j < kCopyPieces; ++j) v[j] = *reinterpret_cast<const v4i*>(src[j] + koff);
+#pragma unroll
+      for (int j = 0; j < kCopyPieces; ++j) acc ^= v[j];
+    }
+    koff = koff + 256 > kCopyPitch ? 0 : koff + 128;
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  if (acc[0] + acc[1] + acc[2] + acc[3] == 0x12345678 || (iters < 0 && smem[threadIdx.x] == 77)) sink[0] = 1;
+}
+
+long long diag_copy_loop_bytes(long long iters) { return (long long)diag_grid() * 8 * kCopyPieces * 1024 * iters; }
+
+int launch_diag_copy_loop(int mode, const int8_t* data, long long iters, int* sink, hipStream_t stream) {
+  if (mode != 0 && mode != 1) return fail(TI_ERR_INVALID_ARG, "diag_copy_loop: mode must be 0 or 1 (got %d)", mode);
+  const int lds = mode == 0 ? 3 * 8 * kCopyPieces * 1024 : 0;
+  auto kern = mode == 0 ? copy_loop_kernel<0> : copy_loop_kernel<1>;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     3 * 8 * kCopyPieces * 1024);
+  if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+  hipLaunchKernelGGL(kern, dim3(diag_grid()), dim3(512), lds, stream, data, (int)iters, sink);
+  e = hipGetLastError();
+  if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "copy loop launch: %s", hipGetErrorString(e));
+  return TI_OK;
+}
+
 }  // namespace ti

@@ -2137,7 +2137,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmParams p, const 
 // (its four waves read 7 fragments from the LDS per 10 MFMAs); with K = 20480 the larger tiles win
 // (512x5120x20480: 79 against 64 us).  More than three LDS stages did not help it (four to six: +1 to +3 %).
 enum SplitTile { SPLIT_128 = 0, SPLIT_256 = 1, SPLIT_256x160 = 2, SPLIT_256x288 = 3, SPLIT_128x160 = 4, SPLIT_128x288 = 5,
-                 SPLIT_128x80 = 6, SPLIT_128x192 = 7 };
+                 SPLIT_128x80 = 6, SPLIT_128x192 = 7, SPLIT_256x192 = 8 };
 // `batch` > 1: a batched product (A and B per batch); every tile count, byte count and the streaming floor scale with
 // it, the one-launch form is not available, and the tile shapes are those that exist for every epilogue of the
 // raw-int32 kernels.
@@ -2155,28 +2155,33 @@ static int choose_splits(long long M, long long N, long long K, int* tile_kind =
   // (128x192 tiles: widths that 192 divides but neither 160 nor 288 nor 80 does - 12288 and 49152, the GPT-3-sized
   // layers of upstream's scripts/bench_linear_kernels.sh - had only the 128x128 and 256x256 tiles of the 64-byte-step
   // and 32x32-block kernels to split over; 512 x 12288 outputs are exactly 256 tiles of 128x192 and run unsplit)
-  const int order[8] = {SPLIT_128x80, SPLIT_128x160, SPLIT_128x192, SPLIT_128x288, SPLIT_128, SPLIT_256, SPLIT_256x160,
-                        SPLIT_256x288};
-  for (int oi = 0; oi < 8; ++oi) {
+  // (256x192 tiles, unsplit only: 256 x 49152 or 1024 x 12288 outputs are exactly 256 of them.  Their two LDS stages
+  // leave weights that come from HBM one step of cover, and the split forms lost to the 128x192 tiles: 512 x 12288 x
+  // 49152 in two slices 319 against 309 us, 512 x 49152 x 12288 331 against 290 us for 256x128 tiles)
+  const int order[9] = {SPLIT_128x80, SPLIT_128x160, SPLIT_128x192, SPLIT_128x288, SPLIT_128, SPLIT_256, SPLIT_256x160,
+                        SPLIT_256x192, SPLIT_256x288};
+  for (int oi = 0; oi < 9; ++oi) {
     const int kind = order[oi];
     const bool wide192 = kind == SPLIT_128x192;
+    const bool tall192 = kind == SPLIT_256x192;
     const bool half = kind == SPLIT_128x160 || kind == SPLIT_128x288;  // 128-row forms of the two tall tiles
     const bool small = kind == SPLIT_128x80;
     const int bm = kind == SPLIT_128 || half || small || wide192 ? 128 : 256;
-    const int bn = small ? 80 : wide192 ? 192 : kind == SPLIT_128 ? 128 : kind == SPLIT_256 ? 256
+    const int bn = small ? 80 : wide192 || tall192 ? 192 : kind == SPLIT_128 ? 128 : kind == SPLIT_256 ? 256
                    : kind == SPLIT_256x288 || kind == SPLIT_128x288 ? 288 : 160;
     if (kind >= SPLIT_256x160 && N % bn != 0) continue;
-    if (wide192 && (N % 160 == 0 || N % 288 == 0)) continue;  // those widths keep their tuned tiles
+    if ((wide192 || tall192) && (N % 160 == 0 || N % 288 == 0)) continue;  // those widths keep their tuned tiles
     const double tiles = (double)((M + bm - 1) / bm) * (double)((N + bn - 1) / bn) * (double)batch;
     for (int s = 1; s <= 16; ++s) {
       if (steps % s != 0 || steps / s < 4) continue;
       if (kind >= SPLIT_256x160 && (K / s) % QBK != 0) continue;  // these tiles step 128 bytes at a time
       if (half && s == 1) continue;                                // exist as raw-int32 kernels only
-      if (batch > 1 && s == 1 && (small || wide192)) continue;       // unsplit batched products keep their dispatch
+      if (tall192 && s > 1) continue;
+      if (batch > 1 && s == 1 && (small || wide192 || tall192)) continue;  // unsplit batched products keep their dispatch
       // an unsplit candidate stands for what the ordinary dispatch would launch, which takes the 256-row tiles only
       // when they fill most of the chip (and 128x128 tiles otherwise)
       if (s == 1 && kind != SPLIT_128 && !small && tiles < 0.75 * cus) continue;
-      if (s == 1 && wide192 && tiles > cus) continue;  // more than a round: the 256-row tilings of the ordinary dispatch
+      if (s == 1 && (wide192 || tall192) && tiles > cus) continue;  // more than a round: left to the ordinary dispatch
       const double wgs = tiles * s;
       double rounds, step_us, fixed_us = 8.0;
       if (kind == SPLIT_128) {
@@ -2189,7 +2194,7 @@ static int choose_splits(long long M, long long N, long long K, int* tile_kind =
       } else {
         rounds = (double)(long long)((wgs + cus - 1) / cus);
         step_us = kind == SPLIT_256 ? 0.85 : kind == SPLIT_256x160 ? 0.55 : kind == SPLIT_256x288 ? 0.92
-                  : kind == SPLIT_128x160 ? 0.375 : wide192 ? 0.41 : 0.6;
+                  : kind == SPLIT_128x160 ? 0.375 : wide192 ? 0.41 : tall192 ? 0.66 : 0.6;
         if (half) fixed_us = kind == SPLIT_128x160 ? 4.0 : 5.0;  // fewer panel rows to fetch first, half the tile to store
         if (wide192) fixed_us = 4.5;
       }
@@ -2268,7 +2273,7 @@ static int launch_fused(const GemmParams& q_in, hipStream_t stream) {
 // count as waste; batched products count tiles only, they are bound by HBM, where padding costs no bytes).  The
 // 128x128 kernel (64-byte steps, two stages) runs at half that rate per CU, a little more with two workgroups on
 // every CU, and takes over where few tiles of 256 rows would leave most CUs idle.
-enum WideTile { WIDE_NONE = 0, WIDE_256x160, WIDE_256x288, WIDE_256x128, WIDE_256x256 };
+enum WideTile { WIDE_NONE = 0, WIDE_256x160, WIDE_256x288, WIDE_256x128, WIDE_256x256, WIDE_256x192 };
 struct WidePick {
   int tile;       // WideTile; WIDE_NONE = leave it to the 128x128 / small-tile kernels
   double eff;     // efficiency of the choice relative to the 256x256 kernel on a full chip (0 for WIDE_NONE)
@@ -2285,6 +2290,7 @@ static WidePick pick_wide(long long M, long long N, long long K, long long batch
   const bool wide_step = K % QBK == 0;
   const double f160 = wide_step ? 0.94 : 0.78;
   const double f288 = wide_step ? 0.95 : 0.9;
+  const double F192 = 0.90;
   const double e256 = fill(t256, 256);
   const double e160 = N % 160 == 0 ? f160 * fill(rows256 * (N / 160) * batch, 160) : 0.0;
   const double e288 = N % 288 == 0 ? f288 * fill(rows256 * (N / 288) * batch, 288) : 0.0;
@@ -2296,9 +2302,15 @@ static WidePick pick_wide(long long M, long long N, long long K, long long batch
   const bool priced = K >= 2048 && t128 >= 128;
   const double e128w = priced && wide_step && N % 128 == 0 ? 0.93 * fill(rows256 * (N / 128) * batch, 128) : 0.0;
   const double e128 = t128 >= 2 * cus ? 0.6 : t128 >= cus ? 0.47 : 0.47 * (double)t128 / (double)cus;
-  const double best = e256 > e160 ? (e256 > e288 ? (e256 > e128w ? e256 : e128w) : (e288 > e128w ? e288 : e128w))
+  // 256x192 (two LDS stages) for the widths that 192 divides but 160 and 288 do not (12288, 49152: 512 x 49152
+  // outputs are 512 tiles, two full rounds, where 256x256 tiles make 384, a round and a half)
+  const double e192 = priced && wide_step && N % 192 == 0 && N % 160 != 0 && N % 288 != 0
+                          ? F192 * fill(rows256 * (N / 192) * batch, 192) : 0.0;
+  const double best_other = e256 > e160 ? (e256 > e288 ? (e256 > e128w ? e256 : e128w) : (e288 > e128w ? e288 : e128w))
                                   : (e160 > e288 ? (e160 > e128w ? e160 : e128w) : (e288 > e128w ? e288 : e128w));
+  const double best = best_other > e192 ? best_other : e192;
   if (!(t256 >= 160 || (priced && best > e128))) return WidePick{WIDE_NONE, 0.0};
+  if (e192 > best_other * 1.03) return WidePick{WIDE_256x192, e192};
   if (e160 > e256 && e160 >= e288 && e160 >= e128w) return WidePick{WIDE_256x160, e160};
   if (e288 > e256 && e288 >= e128w) return WidePick{WIDE_256x288, e288};
   if (e128w > e256) return WidePick{WIDE_256x128, e128w};
@@ -2476,6 +2488,10 @@ int launch_kind(const GemmParams& p, void* workspace, long long workspace_bytes,
       g_last_kernel = "pipe16_128x192";
       return launch_pipe16q<Pipe16QCfg<128, 192, 4, 2, KIND>>(p, stream);
     }
+    if (splits == 1 && tile == SPLIT_256x192) {
+      g_last_kernel = "pipe16_256x192";
+      return launch_pipe16q<Pipe16QCfg<256, 192, 4, 2, KIND>>(p, stream);
+    }
     if (splits > 1 && workspace != nullptr && workspace_bytes >= need &&
         (reinterpret_cast<uintptr_t>(workspace) & 15) == 0) {
       g_last_kernel = tile == SPLIT_128      ? "splitk_128x128"
@@ -2582,6 +2598,9 @@ int launch_kind(const GemmParams& p, void* workspace, long long workspace_bytes,
         case WIDE_256x128:
           g_last_kernel = "pipe16_256x128";
           return launch_pipe16q<Pipe16QCfg<256, 128, 4, 2, KIND>>(p, stream);
+        case WIDE_256x192:
+          g_last_kernel = "pipe16_256x192";
+          return launch_pipe16q<Pipe16QCfg<256, 192, 4, 2, KIND>>(p, stream);
         case WIDE_256x256:
           g_last_kernel = "pipe_256x256";
           if (wide_step) return launch_pipe2<Pipe2Cfg<256, 256, 2, 4, KIND, SWAP>>(p, stream);  // whole cache lines per row

@@ -78,6 +78,10 @@ _lib.ti_diag_mfma_loop_ops.argtypes = [_i64]
 _lib.ti_diag_mfma_loop_ops.restype = _i64
 _lib.ti_diag_store_loop.argtypes = [_vp, _i64, _i64, ctypes.c_int, ctypes.c_int, _vp]
 _lib.ti_diag_store_loop.restype = ctypes.c_int
+_lib.ti_diag_copy_loop.argtypes = [ctypes.c_int, _vp, _i64, _i64, _vp, _vp]
+_lib.ti_diag_copy_loop.restype = ctypes.c_int
+_lib.ti_diag_copy_loop_bytes.argtypes = [_i64]
+_lib.ti_diag_copy_loop_bytes.restype = _i64
 _raw_stream = torch._C._cuda_getCurrentRawStream
 _fast = _CUDA._fast if getattr(_CUDA._fast, "kv_append", None) is not None else None
 _fast_decode_attn = getattr(_CUDA._fast, "decode_attn", None)
@@ -681,6 +685,23 @@ def diag_store_loop(out, workgroups, reps=1):
     if rc:
         raise RuntimeError(f"torch_int._hip_ext.diag_store_loop: {_lib.ti_last_error().decode()} (status {rc})")
     return out.numel() * 4 * int(reps)
+
+
+def diag_copy_loop(mode, data, iters, sink):
+    """Diagnostic launch (computes nothing): every CU fetches 48 KiB per step, ``iters`` steps, from the first 2 MiB of
+    ``data`` (one-byte HIP tensor) with the GEMM mainloop's access pattern; mode 0 = global->LDS copies, 1 = loads into
+    registers.  Returns the bytes the launch fetches."""
+    if not (isinstance(data, torch.Tensor) and data.is_cuda and data.is_contiguous() and data.element_size() == 1):
+        raise RuntimeError("torch_int._hip_ext.diag_copy_loop: data must be a contiguous one-byte HIP tensor")
+    if not (_ok(sink, torch.int32) and sink.numel() >= 1 and sink.device == data.device):
+        raise RuntimeError("torch_int._hip_ext.diag_copy_loop: sink must be an int32 HIP tensor on the same device")
+    with _on(data.device):
+        rc = _lib.ti_diag_copy_loop(int(mode), data.data_ptr(), data.numel(), int(iters), sink.data_ptr(),
+                                    _raw_stream(data.device.index) or None)
+        nbytes = int(_lib.ti_diag_copy_loop_bytes(int(iters)))
+    if rc:
+        raise RuntimeError(f"torch_int._hip_ext.diag_copy_loop: {_lib.ti_last_error().decode()} (status {rc})")
+    return nbytes
 
 
 def measure_mfma_ceiling(window_ms=250.0, iters=20000, window=None):
