@@ -54,7 +54,7 @@ FAMILIES = {
 # The counter runs behind FAMILIES[*]["traffic"] were made on the kernels as this hash of their source file describes
 # them (first 16 hex digits of the SHA-256 of torch-int_amd/csrc/gemm_s8_impl.h).  When the file has changed since,
 # the bench line says so next to the figure instead of passing an old measurement off as current.
-TRAFFIC_SOURCE_SHA16 = "69043ebc0ef2aa5e"
+TRAFFIC_SOURCE_SHA16 = "8f1091d02dca5b89"
 
 
 def traffic_is_current():
@@ -538,9 +538,13 @@ def main():
             "unit": "TOP/s", "constant": m["mfma_only_constant"], "random": m["mfma_only_random"],
             "lds_fed": m["lds_fed_random"], "all": m,
             "frac_of_lds_fed": achieved / m["lds_fed_random"],
+            "step_mix": m["step_mix_256x160_random"], "frac_of_step_mix": achieved / m["step_mix_256x160_random"],
             "note": "back-to-back launches of ti_diag_mfma_loop over 250 ms windows: v_mfma_i32_32x32x32_i8 only "
                     "(constant / random operand bytes), and with LDS fragment reads, global->LDS copies and a barrier "
-                    "per step on random bytes (lds_fed); the published peak stays the denominator of frac"}
+                    "per step on random bytes (lds_fed); step_mix = ti_diag_mix_loop, the instructions of one K step of "
+                    "the 256x160 tile and nothing else (40 v_mfma_i32_16x16x64_i8, 18 fragment reads, 7 copies and a "
+                    "barrier per wave) on random bytes: the rate no kernel with this mainloop can exceed on this board; "
+                    "the published peak stays the denominator of frac"}
     if not args.sweep_only:
         # per-case launch durations, upstream's protocol; HBM-bound cases rotate weight copies (> 256 MB in total)
         table = []

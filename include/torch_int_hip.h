@@ -136,6 +136,17 @@ int ti_diag_store_loop(float* out, int64_t M, int64_t N, int workgroups, int rep
 int ti_diag_copy_loop(int mode, const int8_t* data, int64_t data_bytes, int64_t iters, int32_t* sink, void* stream);
 int64_t ti_diag_copy_loop_bytes(int64_t iters);
 
+/* Diagnostic (no counterpart in the reference; computes nothing): one workgroup per CU issues, `iters` times, the
+ * instructions a wave of the 16x16-block GEMM kernels issues per 128-byte K step and nothing else, on operands that
+ * change every step.  shape 0 = the 256x160 tile (8 waves, each 40 v_mfma_i32_16x16x64_i8, 18 ds_read_b128, 7 1-KiB
+ * global->LDS copies), shape 1 = the 128x80 tile (4 waves, each 20 / 14 / 7).  parts is a bit set: 1 MFMAs, 2 fragment
+ * reads, 4 copies and their wait, 8 workgroup barrier.  `data`: at least 3 MiB of device memory, 16-byte aligned (fill
+ * it with random bytes); `sink` as for ti_diag_mfma_loop.  The time per step of parts = 15 is the floor of that
+ * kernel's K step on the board; ti_diag_mix_loop_ops(shape, iters) = integer operations of a launch with bit 1 set. */
+int ti_diag_mix_loop(int shape, int parts, const int8_t* data, int64_t data_bytes, int64_t iters, int32_t* sink,
+                     void* stream);
+int64_t ti_diag_mix_loop_ops(int shape, int64_t iters);
+
 /* ---- W8A8 linear: out[M,N] = epilogue(x[M,K] . w[N,K]^T, bias[N]) ---- */
 
 /* replaces linear_a8_w8_b32_o32 (torch_int/kernels/linear.cu:13-136;

@@ -13,6 +13,8 @@ Examples
       # matrix-pipe ceiling: mode (0 MFMA only, 1 + LDS reads, 2 + LDS-DMA copies and barrier), steps per wave
   python torch-int_amd/benchmark/bench_kernel.py --op mfma_ceiling --shape 250    # all six figures, 250 ms windows
   python torch-int_amd/benchmark/bench_kernel.py --op copy_loop --shape 0 4000     # L2 -> CU copy rate: mode (0 into LDS, 1 into registers), steps
+  python torch-int_amd/benchmark/bench_kernel.py --op mix_loop --shape 0 15 20000   # floor of a K step: tile (0 256x160, 1 128x80), parts
+      # (bit set: 1 MFMAs, 2 fragment reads, 4 copies, 8 barrier), steps; us / steps = time per K step
   rocprofv3 --kernel-trace --stats --output-format csv -d out -- python3 .../bench_kernel.py --op ...
 
 Prints one JSON line: mean microseconds per call (HIP events on the launch stream), algorithmic
@@ -43,7 +45,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--op", required=True, choices=list(LINEAR) + ["bmm_f32t", "bmm_s8t", "bmm_s32t", "bmm_s8t_rowmajor", "ln_q", "ln_q_f16", "add_ln_q",
                                                "softmax_q", "qk_softmax_q", "attn_prefill", "decode_attn", "transpose_last2", "copy",
-                                               "mfma_loop", "mfma_ceiling", "store_loop", "copy_loop"])
+                                               "mfma_loop", "mfma_ceiling", "store_loop", "copy_loop", "mix_loop"])
     ap.add_argument("--shape", type=int, nargs="+", required=True)
     ap.add_argument("--iters", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
@@ -189,6 +191,13 @@ def main():
         out = torch.empty(M, N, device=dev)
         nbytes = float(X.diag_store_loop(out, workgroups, reps))
         fn = lambda: X.diag_store_loop(out, workgroups, reps)  # noqa: E731
+    elif args.op == "mix_loop":
+        # the instruction mix of one K step of the 256x160 (shape 0) or 128x80 (shape 1) tile, parts as a bit set
+        shape, parts, steps = args.shape
+        data = (torch.full((3 << 20,), 1, dtype=torch.int8, device=dev) if args.pattern == "constant" else s8(3 << 20))
+        sink = torch.zeros(1, dtype=torch.int32, device=dev)
+        ops = float(X.diag_mix_loop(shape, parts, data, steps, sink)) if parts & 1 else 0.0
+        fn = lambda: X.diag_mix_loop(shape, parts, data, steps, sink)  # noqa: E731
     elif args.op == "copy_loop":
         # every CU fetches 48 KiB per step from an L2-resident 2 MiB with the mainloop's access pattern, nothing else
         mode, steps = args.shape

@@ -485,6 +485,21 @@ int ti_diag_copy_loop(int mode, const int8_t* data, int64_t data_bytes, int64_t 
   return launch_diag_copy_loop(mode, data, iters, sink, static_cast<hipStream_t>(stream));
 }
 
+int64_t ti_diag_mix_loop_ops(int shape, int64_t iters) { return iters > 0 ? diag_mix_loop_ops(shape, iters) : 0; }
+
+int ti_diag_mix_loop(int shape, int parts, const int8_t* data, int64_t data_bytes, int64_t iters, int32_t* sink,
+                     void* stream) {
+  g_err[0] = 0;
+  const char* op = "diag_mix_loop";
+  if (iters < 1 || iters > (1 << 30))
+    return fail(TI_ERR_INVALID_ARG, "%s: iters must be in [1, 2^30] (got %lld)", op, (long long)iters);
+  if (data_bytes < (3 << 20))
+    return fail(TI_ERR_INVALID_ARG, "%s: data must hold at least 3 MiB (got %lld bytes)", op, (long long)data_bytes);
+  if (int rc = check_ptr(op, "data", data, 16, true)) return rc;
+  if (int rc = check_ptr(op, "sink", sink, 4, true)) return rc;
+  return launch_diag_mix_loop(shape, parts, data, iters, sink, static_cast<hipStream_t>(stream));
+}
+
 int ti_bmm_s8t_s8n_f32t_strided(const int8_t* a, const int8_t* b, float* c, int64_t batch, int64_t M, int64_t N,
                                 int64_t K, int64_t stride_a, int64_t stride_b, float alpha, void* stream) {
   return run_gemm("bmm_s8t_s8n_f32t_strided", EPI_F32_SCALE, a, b, nullptr, 0, c, 4, batch, M, N, K, alpha, 0.0f,

@@ -199,4 +199,87 @@ int launch_diag_copy_loop(int mode, const int8_t* data, long long iters, int* si
   return TI_OK;
 }
 
+// Instruction-mix diagnostic for the 16x16-block GEMM kernels: one workgroup per CU runs `iters` K steps of nothing
+// but the instructions a wave of the real kernel issues per step, on operands that change every step (the LDS
+// region the fragment reads fetch is filled from `data`), with no dependence on what the copies deliver:
+//   shape 0  the 256x160 tile: 8 waves, each 40 v_mfma_i32_16x16x64_i8, 18 ds_read_b128, 7 global->LDS copies of 1 KiB
+//   shape 1  the 128x80 tile:  4 waves, each 20 MFMAs, 14 reads, 7 copies
+// `parts` is a bit set: 1 the MFMAs, 2 the fragment reads, 4 the copies (L2-resident source, two steps in flight) and
+// their wait, 8 the workgroup barrier.  The time of parts = 15 is the floor of the kernel's K step on this board.
+template <int WAVES, int NM, int NR, int NC, int PARTS>
+__global__ __launch_bounds__(WAVES * 64) void mix_loop_kernel(const int8_t* __restrict__ data, int iters, int* sink) {
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const char* g = reinterpret_cast<const char*>(data);
+  for (int i = threadIdx.x; i < 2048; i += WAVES * 64)
+    *reinterpret_cast<v4i*>(smem + i * 16) = *reinterpret_cast<const v4i*>(g + (size_t)i * 16);
+  __syncthreads();
+  const char* src = g + (size_t)(blockIdx.x % 8) * 262144 + (size_t)wave * 8 * kCopyPitch + (lane >> 3) * kCopyPitch +
+                    (lane & 7) * 16;
+  v4i acc[10], f[14];
+#pragma unroll
+  for (int i = 0; i < 10; ++i) acc[i] = v4i{0, 0, 0, 0};
+#pragma unroll
+  for (int i = 0; i < 14; ++i) f[i] = v4i{lane, i, wave, 1};
+  const int rd = lane * 16 + (wave & 3) * 8192;
+  int koff = 0;
+  for (int it = 0; it < iters; ++it) {
+    if (PARTS & 4) {
+      TI_LDS_AS char* dst = (TI_LDS_AS char*)smem + 32768 + (it & 1) * (WAVES * NC * 1024) + wave * NC * 1024;
+#pragma unroll
+      for (int j = 0; j < NC; ++j)
+        __builtin_amdgcn_global_load_lds((const TI_GLOBAL_AS void*)(src + koff + j * 8 * kCopyPitch),
+                                         (TI_LDS_AS void*)(dst + j * 1024), 16, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < NM; ++i) {
+      if (PARTS & 1)
+        asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+v"(acc[i % 10]) : "v"(f[i % 7]), "v"(f[7 + i % 7]));
+      if ((PARTS & 2) && i < NR)
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(f[i % 14]) : "v"(rd), "n"((i % 8) * 1024));
+    }
+    if (PARTS & 4) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NC) : "memory");  // two steps in flight, as the kernel
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    if (PARTS & 8) asm volatile("s_barrier" ::: "memory");
+    koff = (koff + 128) & 4095;
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  int s = 0;
+#pragma unroll
+  for (int i = 0; i < 10; ++i) s += acc[i][0] + acc[i][3];
+#pragma unroll
+  for (int i = 0; i < 14; ++i) s += f[i][1];
+  if (s == 0x12345678) sink[0] = 1;
+}
+
+long long diag_mix_loop_ops(int shape, long long iters) {
+  return (long long)diag_grid() * (shape == 0 ? 8 * 40 : 4 * 20) * iters * 32768;
+}
+
+template <int WAVES, int NM, int NR, int NC, int PARTS>
+static int launch_mix(const int8_t* data, int iters, int* sink, hipStream_t stream) {
+  auto kern = mix_loop_kernel<WAVES, NM, NR, NC, PARTS>;
+  constexpr int lds = 32768 + 2 * WAVES * NC * 1024;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+  if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+  hipLaunchKernelGGL(kern, dim3(diag_grid()), dim3(WAVES * 64), lds, stream, data, iters, sink);
+  e = hipGetLastError();
+  if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "mix loop launch: %s", hipGetErrorString(e));
+  return TI_OK;
+}
+
+int launch_diag_mix_loop(int shape, int parts, const int8_t* data, long long iters, int* sink, hipStream_t stream) {
+#define TI_MIX(P)                                                                                 \
+  case P:                                                                                         \
+    return shape == 0 ? launch_mix<8, 40, 18, 7, P>(data, (int)iters, sink, stream)               \
+                      : launch_mix<4, 20, 14, 7, P>(data, (int)iters, sink, stream)
+  if (shape != 0 && shape != 1) return fail(TI_ERR_INVALID_ARG, "diag_mix_loop: shape must be 0 or 1 (got %d)", shape);
+  switch (parts) {
+    TI_MIX(1); TI_MIX(2); TI_MIX(3); TI_MIX(4); TI_MIX(5); TI_MIX(6); TI_MIX(7); TI_MIX(8);
+    TI_MIX(9); TI_MIX(10); TI_MIX(11); TI_MIX(12); TI_MIX(13); TI_MIX(14); TI_MIX(15);
+  }
+#undef TI_MIX
+  return fail(TI_ERR_INVALID_ARG, "diag_mix_loop: parts must be in [1, 15] (got %d)", parts);
+}
+
 }  // namespace ti

@@ -298,6 +298,8 @@ long long diag_mfma_loop_ops(long long iters);
 int launch_diag_store_loop(float* out, long long M, long long N, int workgroups, int reps, hipStream_t stream);
 int launch_diag_copy_loop(int mode, const int8_t* data, long long iters, int* sink, hipStream_t stream);
 long long diag_copy_loop_bytes(long long iters);
+int launch_diag_mix_loop(int shape, int parts, const int8_t* data, long long iters, int* sink, hipStream_t stream);
+long long diag_mix_loop_ops(int shape, long long iters);
 
 // bmm_rowmajor.hip
 int launch_bmm_s8t_s8t_s8t(const int8_t* a, const int8_t* b, int8_t* c, long long batch, long long M, long long N,

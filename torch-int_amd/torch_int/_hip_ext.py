@@ -82,6 +82,10 @@ _lib.ti_diag_copy_loop.argtypes = [ctypes.c_int, _vp, _i64, _i64, _vp, _vp]
 _lib.ti_diag_copy_loop.restype = ctypes.c_int
 _lib.ti_diag_copy_loop_bytes.argtypes = [_i64]
 _lib.ti_diag_copy_loop_bytes.restype = _i64
+_lib.ti_diag_mix_loop.argtypes = [ctypes.c_int, ctypes.c_int, _vp, _i64, _i64, _vp, _vp]
+_lib.ti_diag_mix_loop.restype = ctypes.c_int
+_lib.ti_diag_mix_loop_ops.argtypes = [ctypes.c_int, _i64]
+_lib.ti_diag_mix_loop_ops.restype = _i64
 _raw_stream = torch._C._cuda_getCurrentRawStream
 _fast = _CUDA._fast if getattr(_CUDA._fast, "kv_append", None) is not None else None
 _fast_decode_attn = getattr(_CUDA._fast, "decode_attn", None)
@@ -704,9 +708,27 @@ def diag_copy_loop(mode, data, iters, sink):
     return nbytes
 
 
+def diag_mix_loop(shape, parts, data, iters, sink):
+    """Diagnostic launch (computes nothing): ``iters`` K steps of the instruction mix of the 256x160 (``shape`` 0) or
+    128x80 (``shape`` 1) GEMM tile; ``parts`` bit set: 1 MFMAs, 2 LDS fragment reads, 4 global->LDS copies, 8 barrier.
+    ``data``: one-byte HIP tensor of at least 3 MiB.  Returns the integer operations of the MFMAs of one launch."""
+    if not (isinstance(data, torch.Tensor) and data.is_cuda and data.is_contiguous() and data.element_size() == 1):
+        raise RuntimeError("torch_int._hip_ext.diag_mix_loop: data must be a contiguous one-byte HIP tensor")
+    if not (_ok(sink, torch.int32) and sink.numel() >= 1 and sink.device == data.device):
+        raise RuntimeError("torch_int._hip_ext.diag_mix_loop: sink must be an int32 HIP tensor on the same device")
+    with _on(data.device):
+        rc = _lib.ti_diag_mix_loop(int(shape), int(parts), data.data_ptr(), data.numel(), int(iters), sink.data_ptr(),
+                                   _raw_stream(data.device.index) or None)
+        ops = int(_lib.ti_diag_mix_loop_ops(int(shape), int(iters)))
+    if rc:
+        raise RuntimeError(f"torch_int._hip_ext.diag_mix_loop: {_lib.ti_last_error().decode()} (status {rc})")
+    return ops
+
+
 def measure_mfma_ceiling(window_ms=250.0, iters=20000, window=None):
     """What the int8 matrix pipe of the current device sustains, in TOP/s, for the three loop modes of
-    ``diag_mfma_loop`` on constant and on uniformly random operand bytes: back-to-back launches between two HIP
+    ``diag_mfma_loop`` and for the K step of the 256x160 GEMM tile as a bare instruction mix (``diag_mix_loop``), each
+    on constant and on uniformly random operand bytes: back-to-back launches between two HIP
     events for at least ``window_ms`` per figure (after the same again as warm-up, so the clocks have settled under
     the board's power limit).  ``window(label)``, when given, returns a context manager that is entered around the
     timed window of each figure (a benchmark samples clocks and board power there)."""
@@ -732,4 +754,22 @@ def measure_mfma_ceiling(window_ms=250.0, iters=20000, window=None):
                     end.record()
                     torch.cuda.synchronize()
             out[f"{label}_{pname}"] = ops * n / start.elapsed_time(end) / 1e9
+    # the K step of the 256x160 GEMM tile as a bare instruction mix (16x16x64 MFMAs, fragment reads, copies, barrier)
+    big = {"constant": torch.full((3 << 20,), 1, dtype=torch.int8, device=dev),
+           "random": torch.randint(-127, 128, (3 << 20,), dtype=torch.int8, device=dev)}
+    for pname, data in big.items():
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        ops = diag_mix_loop(0, 15, data, iters, sink)
+        end.record()
+        torch.cuda.synchronize()
+        n = max(2, int(window_ms / max(start.elapsed_time(end), 1e-3)) + 1)
+        for timed in (False, True):
+            with (window(f"step_mix_256x160_{pname}") if timed and window is not None else contextlib.nullcontext()):
+                start.record()
+                for _ in range(n):
+                    diag_mix_loop(0, 15, data, iters, sink)
+                end.record()
+                torch.cuda.synchronize()
+        out[f"step_mix_256x160_{pname}"] = ops * n / start.elapsed_time(end) / 1e9
     return out
