@@ -72,6 +72,14 @@ def test_c_abi_rejects_bad_arguments_without_a_device():
                                        ctypes.c_void_p]
     assert lib.ti_diag_store_loop(p, 256, 100, 1, 1, None) == 1 and b"multiple of 256" in lib.ti_last_error()
     assert lib.ti_diag_store_loop(p, 256, 160, 0, 1, None) == 1 and b"workgroups" in lib.ti_last_error()
+    lib.ti_diag_copy_loop.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p,
+                                      ctypes.c_void_p]
+    assert lib.ti_diag_copy_loop(0, p, 1 << 20, 10, p, None) == 1 and b"2 MiB" in lib.ti_last_error()
+    assert lib.ti_diag_copy_loop(0, p, 2 << 20, 0, p, None) == 1 and b"iters" in lib.ti_last_error()
+    lib.ti_diag_mix_loop.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64,
+                                     ctypes.c_void_p, ctypes.c_void_p]
+    assert lib.ti_diag_mix_loop(0, 15, p, 2 << 20, 10, p, None) == 1 and b"3 MiB" in lib.ti_last_error()
+    assert lib.ti_diag_mix_loop(0, 15, p, 3 << 20, 0, p, None) == 1 and b"iters" in lib.ti_last_error()
     # beyond the 32-bit tiling limits
     rc = lib.ti_linear_a8_w8_b32_o32(p, p, p, p, 1 << 20, 4, 1 << 20, None, 0, None)
     assert rc == 1 and b"limits" in lib.ti_last_error()

@@ -1066,6 +1066,28 @@ def test_diag_mfma_loop_runs_and_reports_its_work():
         X.diag_mfma_loop(0, data[: 1 << 19], 200, sink)
 
 
+def test_diag_copy_and_mix_loops_run_and_report_their_work():
+    # the copy-rate and instruction-mix diagnostics: every form launches, exits and counts its bytes / operations
+    import torch_int._hip_ext as X
+    data = torch.randint(-127, 128, (3 << 20,), dtype=torch.int8, device=DEV)
+    sink = torch.zeros(1, dtype=torch.int32, device=DEV)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    for mode in (0, 1):
+        _say(f"diag_copy_loop mode {mode}")
+        assert X.diag_copy_loop(mode, data, 50, sink) == cus * 48 * 1024 * 50
+        torch.cuda.synchronize()
+    for shape, per_cu in ((0, 8 * 40), (1, 4 * 20)):
+        for parts in range(1, 16):
+            _say(f"diag_mix_loop shape {shape} parts {parts}")
+            assert X.diag_mix_loop(shape, parts, data, 50, sink) == cus * per_cu * 50 * 32768
+        torch.cuda.synchronize()
+    assert int(sink.item()) == 0
+    for bad in (lambda: X.diag_copy_loop(2, data, 50, sink), lambda: X.diag_mix_loop(2, 15, data, 50, sink),
+                lambda: X.diag_mix_loop(0, 16, data, 50, sink), lambda: X.diag_mix_loop(0, 15, data[: 1 << 20], 50, sink)):
+        with pytest.raises(RuntimeError):
+            bad()
+
+
 def test_diag_store_loop_fills_the_matrix_and_nothing_else():
     # the store-rate diagnostic writes every element of its [M, N] matrix, for any number of workgroups, and stays
     # inside it (guard rows before and after keep their value)
