@@ -11,7 +11,11 @@ namespace ti {
 long long gemm_workspace_bytes(long long M, long long N, long long K) {
   if (M > 1024) {  // the rows beyond the last multiple of 256 as a small problem of their own (row_split_rows)
     long long need = 0;
-    return row_split_rows(M, N, K, &need) > 0 ? need : 0;
+    const int r = row_split_rows(M, N, K, &need);
+    if (r <= 0) return 0;
+    // the first rows are a problem of their own too: at exactly 1024 of them they may split K themselves
+    const long long head = M - r <= 1024 ? gemm_workspace_bytes(M - r, N, K) : 0;
+    return head > need ? head : need;
   }
   const int s = choose_splits(M, N, K);
   return s > 1 ? (long long)s * M * N * 4 : 0;
