@@ -21,7 +21,8 @@ from torch_int.models.opt import Int8OPTForCausalLM, OPTConfigLite  # noqa: E402
 
 # hidden, heads, ffn, layers (facebook/opt-* configurations; vocab 50272, 2048 positions)
 MODELS = {
-    "opt-125m": (768, 12, 3072, 12), "opt-1.3b": (2048, 32, 8192, 24), "opt-6.7b": (4096, 32, 16384, 32),
+    "opt-125m": (768, 12, 3072, 12), "opt-1.3b": (2048, 32, 8192, 24), "opt-2.7b": (2560, 32, 10240, 32),
+    "opt-6.7b": (4096, 32, 16384, 32),
     "opt-13b": (5120, 40, 20480, 40), "opt-30b": (7168, 56, 28672, 48), "opt-66b": (9216, 72, 36864, 64),
 }
 
