@@ -355,7 +355,7 @@ int ti_kv_append_s8(const int8_t* k_new, const int8_t* v_new, int8_t* k_buf, int
  * same bits, without the score and probability tensors.  vt is V transposed, [BH, D, S] packed (what
  * ti_transpose_last2_s8 makes, as upstream's `value_states.transpose(1,2).contiguous()`); ctx is [BH/heads, T,
  * heads*D] packed.  Limits: D = 64 or 128, S a multiple of 16 in [16, 4096] (ti_attn_qk_softmax_q_supported).  Up to
- * 512 keys (a multiple of 64) at D = 128 all keys of a head sit in the LDS and are swept once; other shapes sweep
+ * 512 keys (a multiple of 64) all keys of a head sit in the LDS and are swept once; other shapes sweep
  * the keys three times in tiles of 256 (row maximum, row sum, probabilities): the same bits either way. */
 int ti_attn_prefill_s8(const int8_t* q, const int8_t* k, const int8_t* vt, const float* mask, int8_t* ctx, int64_t BH,
                        int64_t T, int64_t S, int64_t D, int64_t stride_q, int64_t stride_k, int64_t heads,

@@ -1013,12 +1013,14 @@ def test_fused_prefill_attention_matches_the_chain():
     import torch_int._hip_ext as X
     g = torch.Generator().manual_seed(97)
     neg = torch.finfo(torch.float32).min
-    for (B, H, T, S, kind) in [(4, 40, 512, 512, "causal"), (2, 3, 100, 128, "pad"), (1, 4, 64, 64, None),
-                               (2, 2, 70, 256, "causal"), (1, 2, 300, 320, "causal"), (1, 1, 5, 448, None),
-                               # exactly 128 / 256 / 512 keys without a mask: the kernels compiled for that fact
-                               (1, 2, 80, 128, None), (1, 2, 64, 256, None), (1, 1, 100, 512, None)]:
-        _say(f"attn_prefill B={B} H={H} T={T} S={S} mask={kind}")
-        q, k, v = _s8(g, B * H, T, 128), _s8(g, B * H, S, 128), _s8(g, B * H, S, 128)
+    shapes = [(4, 40, 512, 512, "causal"), (2, 3, 100, 128, "pad"), (1, 4, 64, 64, None),
+              (2, 2, 70, 256, "causal"), (1, 2, 300, 320, "causal"), (1, 1, 5, 448, None),
+              # exactly 128 / 256 / 512 keys without a mask: the kernels compiled for that fact
+              (1, 2, 80, 128, None), (1, 2, 64, 256, None), (1, 1, 100, 512, None)]
+    # head size 128, and 64 (OPT-125m ... 1.3B) on the same kernel's 64-byte-row form
+    for (B, H, T, S, kind, d) in [sh + (128,) for sh in shapes] + [sh + (64,) for sh in [(4, 12, 512, 512, "causal")] + shapes[1:]]:
+        _say(f"attn_prefill B={B} H={H} T={T} S={S} mask={kind} d={d}")
+        q, k, v = _s8(g, B * H, T, d), _s8(g, B * H, S, d), _s8(g, B * H, S, d)
         a_qk, a_pv = _scal(g, 2e-4, 2e-3), _scal(g, 2e-3, 2e-2)
         mask = None
         if kind is not None:
@@ -1027,13 +1029,15 @@ def test_fused_prefill_attention_matches_the_chain():
                 mask += torch.zeros(T, S).masked_fill(torch.arange(S)[None, :] > torch.arange(T)[:, None] + (S - T), neg)
             mask[0, :, :, :5] = neg
         probs = orc.attn_softmax_q(orc.bmm_s8t_s8n_f32t(q, k, a_qk), mask, H)
-        ref = orc.bmm_s8t_s8t_s8t(probs, v, a_pv).view(B, H, T, 128).transpose(1, 2).reshape(B, T, H * 128)
+        ref = orc.bmm_s8t_s8t_s8t(probs, v, a_pv).view(B, H, T, d).transpose(1, 2).reshape(B, T, H * d)
         qd, kd, md = q.to(DEV), k.to(DEV), (mask.to(DEV) if mask is not None else None)
         vt = X.transpose_last2(v.to(DEV))
         assert X.can_attn_prefill(qd, kd, vt, md, B, H)
         out = X.attn_prefill(qd, kd, vt, md, a_qk, a_pv, H)
-        assert out.shape == (B, T, H * 128) and out.dtype == torch.int8
-        assert torch.equal(out.cpu(), ref), (B, H, T, S, kind, (out.cpu() != ref).sum().item())
+        assert out.shape == (B, T, H * d) and out.dtype == torch.int8
+        assert torch.equal(out.cpu(), ref), (B, H, T, S, kind, d, (out.cpu() != ref).sum().item())
+        # the probabilities alone (the form that stores them instead of multiplying on)
+        assert torch.equal(X.attn_qk_softmax_q(qd, kd, md, a_qk, H).cpu(), probs), (B, H, T, S, kind, d)
     assert not X.can_attn_prefill(qd, kd[:, :440], vt[:, :, :440].contiguous(), None, B, H)   # S % 16 != 0
 
 

@@ -1,11 +1,12 @@
 // Q.K^T fused with the mask, the softmax and the int8 quantisation of the probabilities, for prefill with
-// up to 512 key positions and head size 128: probs = round(127 softmax(max(alpha q.k^T + mask, lowest))).
+// up to 512 key positions and head size 128 or 64: probs = round(127 softmax(max(alpha q.k^T + mask, lowest))).
 // The fp32 scores (4 bytes per query-key pair written and read again by the two-kernel form) never leave
 // the registers.  Arithmetic and summation order are those of attn_softmax_q on the scores of
 // bmm_s8t_s8n_f32t, so the bytes are the same.
 //
 // One workgroup of four waves per (batch * head, block of 64 query rows).  The 64 query rows and all S key
-// rows are copied to LDS once (128-byte rows, chunk c of row r at position c ^ ((r >> 1) & 7)).  A wave owns
+// rows are copied to LDS once (head size 128: 128-byte rows, chunk c of row r at position c ^ ((r >> 1) & 7); head
+// size 64: 64-byte rows as they are - the 16 rows a fragment read touches are one contiguous KiB).  A wave owns
 // 16 query rows and all S keys: S/16 blocks of v_mfma_i32_16x16x64_i8 (keys as the row operand), after which
 // lane (r, g) = (lane & 15, lane >> 4) holds, for block j, the scores of query row r and keys 16j + 4g .. +3.
 // A score row is therefore spread over four lanes, each holding whole chunks of four consecutive keys, which is
@@ -22,7 +23,7 @@ namespace ti {
 #define TI_LDS_AS __attribute__((address_space(3)))
 
 constexpr int AF_ROWS = 64;   // query rows per workgroup
-constexpr int AF_D = 128;     // head size
+constexpr int AF_D = 128;     // largest head size (sizes the LDS limit)
 constexpr int AF_MAX_S = 512;
 
 // NB = key blocks of 16 the registers are sized for (S <= 16 * NB).
@@ -37,7 +38,7 @@ constexpr int AF_MAX_S = 512;
 // In the exact forms every "block j exists" and "there is a mask" test folds away at compile time, which leaves
 // straight-line code: the fragment reads, the matrix instructions and the mask loads of different blocks overlap
 // instead of waiting for one another block by block.
-template <int NB, bool PV, int SPEC = 0>
+template <int NB, bool PV, int SPEC = 0, int D = 128>
 __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t* __restrict__ q,
                                                                    const int8_t* __restrict__ k,
                                                                    const float* __restrict__ mask,
@@ -61,17 +62,21 @@ __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t*
   // ---- copies: slab i = 8 rows of [Q tile (64 rows) | K panel (S rows)], 1 KiB per wave instruction
   const int8_t* qb = q + bh * stride_q;
   const int8_t* kb = k + bh * stride_k;
-  const int slabs = (AF_ROWS + S) >> 3;
+  static_assert(D == 64 || D == 128, "head size");
+  constexpr int CPR = D / 16;        // 16-byte chunks per row
+  constexpr int RPS = 64 / CPR;      // rows per 1 KiB slab
+  constexpr int SWZ = D == 128 ? 7 : 0;
+  const int slabs = (AF_ROWS + S) / RPS;
   for (int i = wave; i < slabs; i += 4) {
-    const int row = i * 8 + (lane >> 3);  // row of the stacked panels
-    const int pos = lane & 7;
+    const int row = i * RPS + lane / CPR;  // row of the stacked panels
+    const int pos = lane % CPR;
     const int8_t* src;
     if (row < AF_ROWS) {
       const int t = t0 + row < T ? t0 + row : T - 1;  // rows past the end repeat the last one; never stored
-      src = qb + (long long)t * AF_D + ((pos ^ ((row >> 1) & 7)) << 4);
+      src = qb + (long long)t * D + ((pos ^ ((row >> 1) & SWZ)) << 4);
     } else {
       const int kr = row - AF_ROWS;
-      src = kb + (long long)kr * AF_D + ((pos ^ ((kr >> 1) & 7)) << 4);
+      src = kb + (long long)kr * D + ((pos ^ ((kr >> 1) & SWZ)) << 4);
     }
     __builtin_amdgcn_global_load_lds((const TI_GLOBAL_AS void*)src, (TI_LDS_AS void*)((TI_LDS_AS char*)smem + i * 1024),
                                      16, 0, 0);
@@ -98,20 +103,21 @@ __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t*
   asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
 
   // ---- scores: acc[j] = q rows (16 of this wave) x key block j
-  const int sw = (r >> 1) & 7;
-  const char* qs = smem + (wave * 16 + r) * AF_D;
-  const char* ks = smem + AF_ROWS * AF_D + r * AF_D;
-  v4i qf[2];
+  const int sw = (r >> 1) & SWZ;
+  const char* qs = smem + (wave * 16 + r) * D;
+  const char* ks = smem + AF_ROWS * D + r * D;
+  constexpr int KS = D / 64;  // 64-byte slices of the head dimension = MFMAs per block
+  v4i qf[KS];
 #pragma unroll
-  for (int s = 0; s < 2; ++s) qf[s] = *reinterpret_cast<const v4i*>(qs + (((4 * s + g) ^ sw) << 4));
+  for (int s = 0; s < KS; ++s) qf[s] = *reinterpret_cast<const v4i*>(qs + (((4 * s + g) ^ sw) << 4));
   v4i acc[NB];
 #pragma unroll
   for (int j = 0; j < NB; ++j) {
     acc[j] = v4i{0, 0, 0, 0};
     if (j < nb) {
 #pragma unroll
-      for (int s = 0; s < 2; ++s) {
-        const v4i kf = *reinterpret_cast<const v4i*>(ks + j * 16 * AF_D + (((4 * s + g) ^ sw) << 4));
+      for (int s = 0; s < KS; ++s) {
+        const v4i kf = *reinterpret_cast<const v4i*>(ks + j * 16 * D + (((4 * s + g) ^ sw) << 4));
         acc[j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(kf, qf[s], acc[j], 0, 0, 0);
       }
     }
@@ -119,8 +125,8 @@ __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t*
 
   __syncthreads();  // all waves have read their fragments: the K panel may be overwritten (see the stores below)
   const int pitch = S + 16;
-  // V^T panel: 128 rows of pitch bytes, ending where the K panel ended (it starts inside the dead Q tile)
-  char* vts = smem + (AF_ROWS + S) * AF_D - AF_D * pitch;
+  // V^T panel: D rows of pitch bytes, ending where the K panel ended (it starts inside the dead Q tile)
+  char* vts = smem + (AF_ROWS + S) * D - D * pitch;
   // ---- x = max(alpha * acc + mask, lowest); row maximum
 #pragma unroll
   for (int j0 = 0; j0 < NB; j0 += MG) {
@@ -152,8 +158,8 @@ __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t*
   // before the mask rows would have to land before the first mask value could be used.  They run under the
   // exponentials and the quantisation and are waited for in front of P.V.
   if constexpr (PV) {
-    const int8_t* vb = vt + bh * (long long)AF_D * S;
-    const int instrs = (AF_D * pitch) >> 10;  // 1 KiB each
+    const int8_t* vb = vt + bh * (long long)D * S;
+    const int instrs = (D * pitch) >> 10;  // 1 KiB each
     for (int i = wave; i < instrs; i += 4) {
       const int o = i * 1024 + lane * 16;
       int row = o / pitch, col = o - row * pitch;
@@ -219,7 +225,9 @@ __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t*
   if constexpr (!PV) {
     // staged through the part of the K panel this wave may reuse (every wave is past the barrier above, so
     // nobody reads the panel any more) and written out as whole rows, 16 bytes per lane
-    char* stage = smem + AF_ROWS * AF_D + wave * 16 * pitch;
+    // (with 64-byte rows the four waves' 64 rows of pitch bytes are a little more than the K panel: they start in the
+    // Q tile, whose fragments every wave holds in registers since before the barrier)
+    char* stage = smem + (D == 128 ? AF_ROWS * D : 0) + wave * 16 * pitch;
 #pragma unroll
     for (int j = 0; j < NB; ++j)
       if (j < nb) *reinterpret_cast<unsigned*>(stage + r * pitch + 16 * j + 4 * g) = pw[j];
@@ -235,16 +243,16 @@ __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t*
   } else {
     // ---- context = P . V: all V^T copies of the workgroup must have landed
     asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
-    v4i o[AF_D / 16];
+    v4i o[D / 16];
 #pragma unroll
-    for (int c = 0; c < AF_D / 16; ++c) o[c] = v4i{0, 0, 0, 0};
+    for (int c = 0; c < D / 16; ++c) o[c] = v4i{0, 0, 0, 0};
     const char* vrow = vts + r * pitch + 4 * g;  // V^T row (= head-dim index) r of block c is 16c + r
 #pragma unroll
     for (int sl = 0; sl < NB / 4; ++sl) {
       if (4 * sl < nb) {
         const v4i pa = {(int)pw[4 * sl], (int)pw[4 * sl + 1], (int)pw[4 * sl + 2], (int)pw[4 * sl + 3]};
 #pragma unroll
-        for (int c = 0; c < AF_D / 16; ++c) {
+        for (int c = 0; c < D / 16; ++c) {
           const char* src = vrow + c * 16 * pitch + 64 * sl;
           const v4i vf = {*reinterpret_cast<const int*>(src), *reinterpret_cast<const int*>(src + 16),
                           *reinterpret_cast<const int*>(src + 32), *reinterpret_cast<const int*>(src + 48)};
@@ -254,9 +262,9 @@ __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t*
     }
     if (t < T) {
       const long long b = bh / heads, h = bh - b * heads;
-      int* crow = reinterpret_cast<int*>(ctx + ((b * T + t) * heads + h) * (long long)AF_D) + g;
+      int* crow = reinterpret_cast<int*>(ctx + ((b * T + t) * heads + h) * (long long)D) + g;
 #pragma unroll
-      for (int c = 0; c < AF_D / 16; ++c) {
+      for (int c = 0; c < D / 16; ++c) {
         unsigned w = 0;
 #pragma unroll
         for (int v = 0; v < 4; ++v)
@@ -275,18 +283,18 @@ int launch_attn_long(const int8_t* q, const int8_t* k, const float* mask, int8_t
 
 // shapes the single-sweep kernel of this file takes (all keys of a head in the LDS at once)
 static bool single_sweep_ok(long long T, long long S, long long D, bool pv) {
-  return T >= 1 && D == AF_D && S >= 16 && S <= AF_MAX_S && S % 16 == 0 && (!pv || S % 64 == 0);
+  return T >= 1 && (D == 128 || D == 64) && S >= 16 && S <= AF_MAX_S && S % 16 == 0 && (!pv || S % 64 == 0);
 }
 
 bool attn_qk_softmax_q_supported(long long T, long long S, long long D) {
   return single_sweep_ok(T, S, D, false) || attn_long_supported(T, S, D);
 }
 
-template <int NB, bool PV, int SPEC>
+template <int NB, bool PV, int SPEC, int D>
 static int launch_af(dim3 grid, size_t lds, hipStream_t stream, const int8_t* q, const int8_t* k, const float* mask,
                      int8_t* probs, int T, int S, long long stride_q, long long stride_k, int heads, int row_blocks,
                      float alpha, const int8_t* vt, int8_t* ctx, float alpha_pv) {
-  auto kern = attn_qk_softmax_q_kernel<NB, PV, SPEC>;
+  auto kern = attn_qk_softmax_q_kernel<NB, PV, SPEC, D>;
   static unsigned long long lds_ok = 0;  // bit per device: the large dynamic LDS size has been allowed
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return fail(TI_ERR_LAUNCH, "attn_qk_softmax_q: no current device");
@@ -314,11 +322,13 @@ int launch_attn_qk_softmax_q(const int8_t* q, const int8_t* k, const float* mask
   if (BH * row_blocks > 0x7fffffffLL || T > 0x7fffffffLL)
     return fail(TI_ERR_INVALID_ARG, "attn_qk_softmax_q: too many row blocks (%lld)", BH * row_blocks);
   const dim3 grid((unsigned)(BH * row_blocks));
-  const size_t lds = (size_t)(AF_ROWS + S) * AF_D;
+  const size_t lds = (size_t)(AF_ROWS + S) * D;
   int rc;
-#define TI_AF(NB, PV, SPEC)                                                                                             \
-  rc = launch_af<NB, PV, SPEC>(grid, lds, stream, q, k, mask, probs, (int)T, (int)S, stride_q, stride_k, (int)heads,   \
-                               (int)row_blocks, alpha, vt, ctx, alpha_pv)
+#define TI_AF(NB, PV, SPEC)                                                                                            \
+  rc = D == 128 ? launch_af<NB, PV, SPEC, 128>(grid, lds, stream, q, k, mask, probs, (int)T, (int)S, stride_q, stride_k, \
+                                               (int)heads, (int)row_blocks, alpha, vt, ctx, alpha_pv)                  \
+                : launch_af<NB, PV, SPEC, 64>(grid, lds, stream, q, k, mask, probs, (int)T, (int)S, stride_q, stride_k,  \
+                                              (int)heads, (int)row_blocks, alpha, vt, ctx, alpha_pv)
 #define TI_AF_NB(NB, PV)                                 \
   do {                                                   \
     if (S != 16 * NB) TI_AF(NB, PV, 0);                  \
