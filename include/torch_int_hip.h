@@ -218,6 +218,13 @@ int ti_linear_a8_w8_b8_o8_group_heads(const int8_t* x, const int8_t* const* w, c
                                       int8_t* const* out, const float* alpha, const float* beta, int64_t count,
                                       int64_t M, int64_t N, int64_t K, int64_t T, int64_t head_dim, void* stream);
 
+/* Diagnostic (no counterpart in the reference): 1 when a group call of `count` problems of that shape runs as ONE
+ * launch on the current device (the streaming kernel for M <= 16 with K % 1024 == 0; a persistent tiled launch when
+ * the 256x160, 256x288 or 256x128 tiles divide N, K % 128 == 0, M > 128, and the cost model does not price the
+ * problems' own one-round tilings below it), 0 when it loops over the problems - without the split-K workspace that
+ * separate ti_linear_a8_w8_b8_o8 calls could be given, so a caller that holds one does better with those. */
+int ti_linear_group_is_one_launch(int64_t M, int64_t N, int64_t K, int count);
+
 /* replaces linear_relu_a8_w8_b8_o8 (linear.cu:476-625; linear.h:28-33):
  * out = s8(rint(min(max(alpha*acc + beta*bias, 0), 127))). */
 int ti_linear_relu_a8_w8_b8_o8(const int8_t* x, const int8_t* w, const int8_t* bias, int8_t* out,

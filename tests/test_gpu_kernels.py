@@ -888,6 +888,8 @@ def test_grouped_prefill_linears_one_launch():
                                        (2, 100, 5, 128, 384, 2, "pipe16_256x160_group"),
                                        (1, 300, 9, 32, 640, 4, "pipe16_256x288_group"),
                                        (3, 171, 10, 16, 128, 3, "pipe16_256x160_group"),
+                                       # 512 x 12288: each problem is one round of 128x192 tiles and runs by itself
+                                       (1, 512, 96, 128, 2048, 3, None),
                                        (2, 100, 6, 128, 128, 3, None), (2, 60, 5, 128, 128, 3, None),
                                        (2, 100, 5, 128, 192, 3, None)]:
         M, N = B * T, H * d
@@ -900,6 +902,8 @@ def test_grouped_prefill_linears_one_launch():
         out = X.linear_a8_w8_b8_o8_group(xd, wd, bd, al, be)
         if family:
             assert C._lib.ti_last_kernel().decode() == family
+        elif N == 12288:
+            assert C._lib.ti_last_kernel().decode() == "pipe16_128x192"
         for o, r_ in zip(out, ref):
             assert torch.equal(o.cpu(), r_), (M, N, K)
         out = X.linear_a8_w8_b8_o8_group_heads(xd, wd, bd, al, be, B, T, H, d)

@@ -146,6 +146,9 @@ int ti_init(void) {
 
 int64_t ti_linear_workspace_bytes(int64_t M, int64_t N, int64_t K) { return gemm_workspace_bytes(M, N, K); }
 int ti_linear_row_split(int64_t M, int64_t N, int64_t K) { return gemm_row_split(M, N, K); }
+int ti_linear_group_is_one_launch(int64_t M, int64_t N, int64_t K, int count) {
+  return M > 0 && N > 0 && K > 0 && count > 0 ? gemm_group_is_one_launch(M, N, K, count) : 0;
+}
 
 int ti_linear_a8_w8_b32_o32(const int8_t* x, const int8_t* w, const int32_t* bias, int32_t* out, int64_t M,
                             int64_t N, int64_t K, void* ws, int64_t ws_bytes, void* stream) {

@@ -288,6 +288,47 @@ int launch_splitk_raw(int tile, const GemmParams& q, hipStream_t stream) {
   return launch_pipe<PipeCfg<256, 256, 2, 4, 4, EPI_S32_RAW, false>>(q, stream);
 }
 
+// Tile width of the one persistent launch that runs a group of `count` [M,K] x [N,K] s8 linears at prefill sizes
+// (160, 288 or 128), or 0 when the problems run one after the other.
+static int group_prefill_tile(long long M, long long N, long long K, int count) {
+  if (!(M > 128 && K % QBK == 0 && K >= QBK && count > 1)) return 0;
+  const long long cus = num_cus();
+  auto fill = [&](long long tiles) { return (double)tiles / (double)(((tiles + cus - 1) / cus) * cus); };
+  const long long rows256 = (M + 255) / 256;
+  const double e160 = N % 160 == 0 ? 0.88 * fill(rows256 * (N / 160) * count) : 0.0;
+  const double e288 = N % 288 == 0 ? 0.95 * fill(rows256 * (N / 288) * count) : 0.0;
+  // widths that only 128 divides (OPT-6.7B: 4096): 256x128 tiles, unless one problem at a time fills the CUs
+  // with 256x256 tiles as well (three 2048x4096x4096: 98 -> 93 us, at 512 rows 57 -> 28 us; 2048x7168x7168
+  // stays with three launches, 277 against 283 us)
+  const double e256_alone = fill(rows256 * ((N + 255) / 256));
+  double e128 = N % 128 == 0 ? 0.87 * fill(rows256 * (N / 128) * count) : 0.0;
+  if (e128 < 0.5 || e128 <= e256_alone) e128 = 0.0;
+  const double e = e160 > e288 ? (e160 > e128 ? e160 : e128) : (e288 > e128 ? e288 : e128);
+  if (e <= 0.0) return 0;
+  // Up to 1024 rows a problem may have a one-round tiling of its own that needs no workspace (128x80, 128x192 or
+  // 256x192 tiles over the whole of K): when the cost model prices the problems one after the other below the
+  // grouped launch, they run that way (three 512x12288x12288: 260 us grouped on 256x128 tiles, 250 us apart;
+  // three 512x5120x5120 stay grouped).  Times as row_split_rows prices a tiling.
+  if (M <= 1024) {
+    int tile = 0;
+    double t_one = -1.0;
+    const int splits = choose_splits(M, N, K, &tile, &t_one);
+    if (splits == 1 && t_one > 0.0 && (tile == SPLIT_128x80 || tile == SPLIT_128x192 || tile == SPLIT_256x192)) {
+      const double t_group = (double)count * M * N * (double)(K / 64) * 0.85 / (65536.0 * (double)cus * e) + 8.0;
+      if ((double)count * t_one < t_group) return 0;
+    }
+  }
+  return e160 >= e288 && e160 >= e128 ? 160 : e288 >= e128 ? 288 : 128;
+}
+
+// Whether a group call of that shape is ONE launch (the streaming kernel at decode sizes, a tiled kernel at prefill
+// sizes) rather than a loop over the problems; a caller that holds a split-K workspace does better with separate
+// calls in the second case.
+int gemm_group_is_one_launch(long long M, long long N, long long K, int count) {
+  if (M <= 16) return K % SBK == 0 ? 1 : 0;
+  return group_prefill_tile(M, N, K, count) != 0 ? 1 : 0;
+}
+
 // q/k/v-style group of s8 linears.  Decode shapes (M <= 16, K % 1024 == 0, enough strips) take one launch
 // of the streaming kernel over all the weights; anything else runs problem by problem.
 int launch_gemm_group_s8(const GemmParams& shape, const GemmGroup& grp, hipStream_t stream) {
@@ -316,29 +357,18 @@ int launch_gemm_group_s8(const GemmParams& shape, const GemmGroup& grp, hipStrea
     if (shape.M <= 4) return launch(gemm_stream_kernel<KIND, 4, 2, true>, 20, 3);
     return launch(gemm_stream_kernel<KIND, 16, 2, true>, 32, 2);
   }
-  // Prefill shapes whose width the 256x160 or 256x288 tiles divide: the problems are the batches of one
+  // Prefill shapes whose width the 256x160, 256x288 or 256x128 tiles divide: the problems are the batches of one
   // persistent launch, so the pipeline fill and the epilogue of one projection overlap the next one's work.
-  if (ptr_ok && shape.M > 128 && shape.K % QBK == 0 && shape.K >= QBK && grp.count > 1 && shape.lda == shape.K &&
-      shape.ldb == shape.K) {
-    const long long cus = num_cus();
-    auto fill = [&](long long tiles) { return (double)tiles / (double)(((tiles + cus - 1) / cus) * cus); };
-    const long long rows256 = (shape.M + 255) / 256;
-    const double e160 = shape.N % 160 == 0 ? 0.88 * fill(rows256 * (shape.N / 160) * grp.count) : 0.0;
-    const double e288 = shape.N % 288 == 0 ? 0.95 * fill(rows256 * (shape.N / 288) * grp.count) : 0.0;
-    // widths that only 128 divides (OPT-6.7B: 4096): 256x128 tiles, unless one problem at a time fills the CUs
-    // with 256x256 tiles as well (three 2048x4096x4096: 98 -> 93 us, at 512 rows 57 -> 28 us; 2048x7168x7168
-    // stays with three launches, 277 against 283 us)
-    const double e256_alone = fill(rows256 * ((shape.N + 255) / 256));
-    double e128 = shape.N % 128 == 0 ? 0.87 * fill(rows256 * (shape.N / 128) * grp.count) : 0.0;
-    if (e128 < 0.5 || e128 <= e256_alone) e128 = 0.0;
-    if (e160 > 0.0 || e288 > 0.0 || e128 > 0.0) {
+  if (ptr_ok && shape.lda == shape.K && shape.ldb == shape.K) {
+    const int tile = group_prefill_tile(shape.M, shape.N, shape.K, grp.count);
+    if (tile != 0) {
       GemmParams q = shape;
       q.batch = grp.count;
-      if (e160 >= e288 && e160 >= e128) {
+      if (tile == 160) {
         g_last_kernel = "pipe16_256x160_group";
         return launch_pipe16q<Pipe16QCfg<256, 160, 4, 2, KIND, true>>(q, stream, grp);
       }
-      if (e288 >= e128) {
+      if (tile == 288) {
         g_last_kernel = "pipe16_256x288_group";
         return launch_pipe16q<Pipe16QCfg<256, 288, 4, 2, KIND, true>>(q, stream, grp);
       }

@@ -240,6 +240,7 @@ int launch_gemm_group_s8(const GemmParams& shape, const GemmGroup& grp, hipStrea
 int launch_gemm(int kind, const GemmParams& p, void* workspace, long long workspace_bytes,
                 hipStream_t stream);
 long long gemm_workspace_bytes(long long M, long long N, long long K);
+int gemm_group_is_one_launch(long long M, long long N, long long K, int count);
 int gemm_row_split(long long M, long long N, long long K);
 long long bmm_workspace_bytes(long long batch, long long M, long long N, long long K);  // split-K scratch of a batched product  // rows a linear cuts off its end and runs as a second problem
 void allow_fused_split_probe(bool allow);  // per thread: may a GEMM call run the one-time placement probe?

@@ -78,6 +78,9 @@ _lib.ti_diag_mfma_loop_ops.argtypes = [_i64]
 _lib.ti_diag_mfma_loop_ops.restype = _i64
 _lib.ti_diag_store_loop.argtypes = [_vp, _i64, _i64, ctypes.c_int, ctypes.c_int, _vp]
 _lib.ti_diag_store_loop.restype = ctypes.c_int
+_lib.ti_linear_group_is_one_launch.argtypes = [_i64, _i64, _i64, ctypes.c_int]
+_lib.ti_linear_group_is_one_launch.restype = ctypes.c_int
+_group_one_launch = {}
 _lib.ti_diag_copy_loop.argtypes = [ctypes.c_int, _vp, _i64, _i64, _vp, _vp]
 _lib.ti_diag_copy_loop.restype = ctypes.c_int
 _lib.ti_diag_copy_loop_bytes.argtypes = [_i64]
@@ -567,37 +570,15 @@ def linear_a8_w8_b8_o8_group(x, weights, biases, alphas, betas, checked=False):
     return out.unbind(0)
 
 
-_cus = []
-
-
-def _cu_count():
-    """Compute units of the current device (what the library's dispatcher counts tiles against)."""
-    if not _cus:
-        _cus.append(torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count
-                    if torch.cuda.is_available() else 256)
-    return _cus[0]
-
-
 def linear_group_is_one_launch(M, N, K, count=3):
     """Whether the library runs a group of [M,K] x [N,K] linears as ONE launch (otherwise it loops over the
-    problems, without the split-K workspace that separate calls would get)."""
-    if M <= 16:
-        return K % 1024 == 0
-    if not (M > 128 and K >= 128 and K % 128 == 0):
-        return False
-    if N % 160 == 0 or N % 288 == 0:
-        return True
-    if N % 128:
-        return False
-    # 256x128 tiles: when they fill at least half of their rounds over the CUs, and more of them than 256x256 tiles
-    # of one problem at a time would (launch_gemm_group_s8 in csrc/gemm_s8.hip decides the same way)
-    cus = _cu_count()
-    rows = (M + 255) // 256
-
-    def fill(tiles):
-        return tiles / (((tiles + cus - 1) // cus) * cus)
-    e128 = 0.87 * fill(rows * (N // 128) * count)
-    return e128 >= 0.5 and e128 > fill(rows * ((N + 255) // 256))
+    problems, without the split-K workspace that separate calls would get).  The library's own decision
+    (``ti_linear_group_is_one_launch``), cached per shape."""
+    key = (int(M), int(N), int(K), int(count))
+    hit = _group_one_launch.get(key)
+    if hit is None:
+        hit = _group_one_launch[key] = bool(_lib.ti_linear_group_is_one_launch(*key))
+    return hit
 
 
 def linear_a8_w8_b8_o8_group_heads(x, weights, biases, alphas, betas, bsz, seq_len, heads, head_dim, checked=False):
