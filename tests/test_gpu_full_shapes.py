@@ -147,6 +147,62 @@ def test_linear_sweep_opt13b(N, K):
 
 # ------------------------------------------------------------------ row counts that are not multiples of the tile
 
+@pytest.mark.parametrize("seed", [5, 6])
+def test_linear_random_shapes_every_epilogue(seed):
+    """400 seeded random (M, N, K) per seed over the widths of OPT-125m ... 66B and GPT-3 (768 ... 49152), row counts
+    from one decoded token to ragged prefills (1 ... 4224, multiples of 256 and not), inner dimensions that 128, 64 or
+    only 16 divide: all six linear epilogues, every output element against the device-side exact references
+    (_acc_on_device, _fma32_on_device).  Whatever kernel family, split or row cut the dispatcher picks for a shape
+    nobody listed by hand, the bits must be these."""
+    import random
+    import torch_int._CUDA as C
+    C._lib.ti_last_kernel.restype = ctypes.c_char_p
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    rnd = random.Random(seed)
+    widths = [768, 3072, 12288, 5120, 2560, 640, 1600, 2880, 4608, 9216, 3200, 1000, 4096, 7168, 2048, 20480, 49152,
+              192, 384, 960]
+    inner = [1024, 2048, 3584, 5120, 4096, 7168, 640, 1040, 12288, 768, 3072, 9216, 128, 256, 16384]
+
+    def s8(*shape):
+        return torch.randint(-127, 128, shape, dtype=torch.int8, device=DEV, generator=g)
+    seen = set()
+    for it in range(400):
+        mode = it % 5
+        M = (rnd.choice([1, 2, 3, 4, 7, 16]) if mode == 0 else
+             rnd.choice([17, 64, 100, 128, 200, 256, 384, 512, 640, 896, 1024]) if mode == 1 else
+             rnd.choice([1025, 1040, 1088, 1152, 1600, 2050, 2112, 2176, 3000, 4096, 4224]) if mode == 2 else
+             rnd.choice([2048, 2304, 8192]) if mode == 3 else rnd.randrange(17, 1400))
+        N, K = rnd.choice(widths), rnd.choice(inner)
+        if mode == 4:
+            K = rnd.choice([16 * rnd.randrange(1, 80), 64 * rnd.randrange(1, 40), 128 * rnd.randrange(1, 40)])
+        if M * N > 40e6 or N * K > 700e6 or M * K > 200e6:
+            continue
+        _say(f"random linear {it}: M={M} N={N} K={K}")
+        x, w, b8 = s8(M, K), s8(N, K), s8(N)
+        bf = torch.randn(N, device=DEV, generator=g)
+        b32 = torch.randint(-65535, 65535, (N,), dtype=torch.int32, device=DEV, generator=g)
+        al, be = rnd.uniform(1e-4, 1e-2), rnd.uniform(1e-4, 1e-2)
+        acc = _acc_on_device(x, w)
+        beta32 = torch.tensor(be, dtype=torch.float32, device=DEV)
+        t8 = _fma32_on_device(al, acc.float(), (beta32 * b8.float()).expand_as(acc))
+        tf = _fma32_on_device(al, acc.float(), bf.expand_as(acc))
+        ts = _fma32_on_device(al, acc.float(), (beta32 * b32.float()).expand_as(acc))
+        assert torch.equal(C.linear_a8_w8_b32_o32(x, w, b32), (acc + b32.long()).to(torch.int32)), (M, N, K)
+        out8 = C.linear_a8_w8_b8_o8(x, w, b8, al, be)
+        family = C._lib.ti_last_kernel().decode()
+        seen.add(family)
+        assert torch.equal(out8, t8.round().clamp(-128, 127).to(torch.int8)), (M, N, K, family)
+        assert torch.equal(C.linear_relu_a8_w8_b8_o8(x, w, b8, al, be), t8.round().clamp(0, 127).to(torch.int8)), (M, N, K)
+        assert torch.equal(C.linear_a8_w8_bfp32_ofp32(x, w, bf, al, 1.0), tf), (M, N, K, family)
+        inout = torch.randn(M, N, device=DEV, generator=g)
+        want = inout + tf
+        C._linear_a8_w8_bfp32_ofp32_acc(x, w, bf, al, 1.0, inout)
+        assert torch.equal(inout, want), (M, N, K, family)
+        scaled = ts.round().clamp(-2.0 ** 31, 2.0 ** 31 - 1).to(torch.int64).clamp(-2 ** 31, 2 ** 31 - 1).to(torch.int32)
+        assert torch.equal(C.linear_a8_w8_b32_o32_with_scaling(x, w, b32, al, be), scaled), (M, N, K)
+    assert len(seen) >= 15, seen   # the sweep does reach most of the dispatcher
+
+
 @pytest.mark.parametrize("M,N,K", [(2112, 5120, 20480), (2176, 5120, 5120), (2050, 5120, 5120), (2064, 5120, 5120),
                                    (4160, 4096, 8192), (2112, 5120, 5120), (1600, 5120, 5120)])
 def test_linear_with_rows_beyond_a_multiple_of_256(M, N, K):

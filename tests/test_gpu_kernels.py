@@ -1260,6 +1260,49 @@ def test_fused_attention_long_keys_and_head_size_64():
     assert not X.can_attn_qk_softmax_q(z(2, 8, 32), z(2, 48, 32), None, 1, 2)      # head size 32
 
 
+@pytest.mark.parametrize("seed", [3, 4])
+def test_fused_attention_random_shapes_against_the_operator_chain(seed):
+    # 250 seeded random (batch, heads, T, S, head size, mask) per seed through ti_attn_qk_softmax_q and
+    # ti_attn_prefill_s8 - single sweep or three, head size 64 or 128, ragged T, causal / padded / fully masked rows /
+    # no mask - against the chain of the separate device kernels (each of which the tests above pin to the oracle)
+    import random
+    import torch_int._CUDA as C
+    import torch_int._hip_ext as X
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    rnd = random.Random(seed + 2)
+    neg = torch.finfo(torch.float32).min
+    ran = 0
+    for it in range(250):
+        D = rnd.choice([128, 64, 64])
+        B, H = rnd.choice([1, 2, 3]), rnd.choice([1, 2, 5, 8, 33])
+        S = (16 * rnd.randrange(1, 70) if it % 3 == 1 else 16 * rnd.randrange(1, 33) if it % 3 == 2 else
+             rnd.choice([64, 128, 256, 512, 1024, 2048]))
+        T = S if it % 2 == 0 else rnd.randrange(17, min(S, 700) + 1) if S > 17 else S
+        kind = rnd.choice(["causal", "pad", None, "rows_masked"])
+        _say(f"random attention {it}: B={B} H={H} T={T} S={S} d={D} mask={kind}")
+        q, k, v = (torch.randint(-127, 128, (B * H, n, D), dtype=torch.int8, device=DEV, generator=g) for n in (T, S, S))
+        a_qk, a_pv = rnd.uniform(2e-4, 2e-3), rnd.uniform(2e-3, 2e-2)
+        mask = None
+        if kind is not None:
+            mask = torch.zeros(B, 1, T, S, device=DEV)
+            if kind == "causal":
+                mask.masked_fill_(torch.triu(torch.ones(T, S, dtype=torch.bool, device=DEV), S - T + 1), neg)
+            elif kind == "pad":
+                mask[:, :, :, : rnd.randrange(0, max(1, S // 3))] = neg
+            else:
+                mask[:, :, : max(1, T // 4), :] = neg      # fully masked rows: uniform probabilities
+        if not X.can_attn_qk_softmax_q(q, k, mask, B, H):
+            continue
+        ran += 1
+        want = X.attn_softmax_q(C.bmm_s8t_s8n_f32t(q, k, a_qk), mask, H)
+        assert torch.equal(X.attn_qk_softmax_q(q, k, mask, a_qk, H), want), (B, H, T, S, D, kind)
+        vt = X.transpose_last2(v)
+        if X.can_attn_prefill(q, k, vt, mask, B, H):
+            ctx = X.merge_heads(C.bmm_s8t_s8n_s8t(want, vt, a_pv), B, H, T, D)
+            assert torch.equal(X.attn_prefill(q, k, vt, mask, a_qk, a_pv, H), ctx), (B, H, T, S, D, kind)
+    assert ran >= 200, ran
+
+
 def test_attention_mask_classes():
     # the class array of a mask (per batch, 64 query rows, 256 keys: mixed / all zero / all one masked value) against
     # a plain restatement, and the long-prefill kernel with and without it on masks built to sit on the class
