@@ -557,6 +557,7 @@ int ti_kv_append_s8(const int8_t* k_new, const int8_t* v_new, int8_t* k_buf, int
 int ti_attn_qk_softmax_q_supported(int64_t T, int64_t S, int64_t D) {
   return attn_qk_softmax_q_supported(T, S, D) ? 1 : 0;
 }
+int ti_attn_prefill_supported(int64_t T, int64_t S, int64_t D) { return attn_prefill_supported(T, S, D) ? 1 : 0; }
 
 int64_t ti_attn_mask_classes_bytes(int64_t batch, int64_t T, int64_t S) { return attn_mask_classes_bytes(batch, T, S); }
 
@@ -588,8 +589,9 @@ int ti_attn_qk_softmax_q_mc(const int8_t* q, const int8_t* k, const float* mask,
                                    (long long)BH, (long long)heads);
   if (BH == 0 || T == 0) return TI_OK;
   if (!attn_qk_softmax_q_supported(T, S, D))
-    return fail(TI_ERR_INVALID_ARG, "%s: unsupported shape T=%lld S=%lld head_dim=%lld (needs head_dim 64 or 128 and S "
-                "a multiple of 16 in [16, 4096])", op, (long long)T, (long long)S, (long long)D);
+    return fail(TI_ERR_INVALID_ARG, "%s: unsupported shape T=%lld S=%lld head_dim=%lld (needs S a multiple of 16 in "
+                "[16, 4096] and head_dim 64 or 128, or any multiple of 16 up to 128 with at most 512 keys)", op,
+                (long long)T, (long long)S, (long long)D);
   if (stride_q < T * D || stride_k < S * D || stride_q % 16 != 0 || stride_k % 16 != 0)
     return fail(TI_ERR_INVALID_ARG, "%s: batch strides (%lld, %lld) must be multiples of 16 and cover one matrix", op,
                 (long long)stride_q, (long long)stride_k);
@@ -619,9 +621,10 @@ int ti_attn_prefill_s8_mc(const int8_t* q, const int8_t* k, const int8_t* vt, co
   if (BH % heads != 0) return fail(TI_ERR_INVALID_ARG, "%s: BH = %lld is not a multiple of heads = %lld", op,
                                    (long long)BH, (long long)heads);
   if (BH == 0 || T == 0) return TI_OK;
-  if (!attn_qk_softmax_q_supported(T, S, D))
-    return fail(TI_ERR_INVALID_ARG, "%s: unsupported shape T=%lld S=%lld head_dim=%lld (needs head_dim 64 or 128 and S "
-                "a multiple of 16 in [16, 4096])", op, (long long)T, (long long)S, (long long)D);
+  if (!attn_prefill_supported(T, S, D))
+    return fail(TI_ERR_INVALID_ARG, "%s: unsupported shape T=%lld S=%lld head_dim=%lld (needs S a multiple of 16 in "
+                "[16, 4096] and head_dim 64 or 128, or any multiple of 16 up to 128 with at most 512 keys, a multiple of 64)",
+                op, (long long)T, (long long)S, (long long)D);
   if (stride_q < T * D || stride_k < S * D || stride_q % 16 != 0 || stride_k % 16 != 0)
     return fail(TI_ERR_INVALID_ARG, "%s: batch strides (%lld, %lld) must be multiples of 16 and cover one matrix", op,
                 (long long)stride_q, (long long)stride_k);

@@ -1,5 +1,6 @@
 // Q.K^T fused with the mask, the softmax and the int8 quantisation of the probabilities, for prefill with
-// up to 512 key positions and head size 128 or 64: probs = round(127 softmax(max(alpha q.k^T + mask, lowest))).
+// up to 512 key positions and head sizes up to 128 (any multiple of 16; the LDS rows are 64 or 128 bytes, zero-filled
+// beyond the head size, so OPT-2.7B's 80 needs no padded copies of q, k and V^T): probs = round(127 softmax(max(alpha q.k^T + mask, lowest))).
 // The fp32 scores (4 bytes per query-key pair written and read again by the two-kernel form) never leave
 // the registers.  Arithmetic and summation order are those of attn_softmax_q on the scores of
 // bmm_s8t_s8n_f32t, so the bytes are the same.
@@ -46,7 +47,8 @@ __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t*
                                                                    long long stride_q, long long stride_k, int heads,
                                                                    int row_blocks, float alpha,
                                                                    const int8_t* __restrict__ vt,
-                                                                   int8_t* __restrict__ ctx, float alpha_pv) {
+                                                                   int8_t* __restrict__ ctx, float alpha_pv, int dr) {
+  // dr = the head size of q, k, vt and ctx in memory (a multiple of 16, D / 2 < dr <= D); D = the LDS row size
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -66,20 +68,27 @@ __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t*
   constexpr int CPR = D / 16;        // 16-byte chunks per row
   constexpr int RPS = 64 / CPR;      // rows per 1 KiB slab
   constexpr int SWZ = D == 128 ? 7 : 0;
+  const int nc = dr >> 4;  // 16-byte chunks of a row in memory; LDS chunks beyond them hold zeros
   const int slabs = (AF_ROWS + S) / RPS;
   for (int i = wave; i < slabs; i += 4) {
     const int row = i * RPS + lane / CPR;  // row of the stacked panels
     const int pos = lane % CPR;
     const int8_t* src;
+    int chunk;
     if (row < AF_ROWS) {
       const int t = t0 + row < T ? t0 + row : T - 1;  // rows past the end repeat the last one; never stored
-      src = qb + (long long)t * D + ((pos ^ ((row >> 1) & SWZ)) << 4);
+      chunk = pos ^ ((row >> 1) & SWZ);
+      src = qb + (long long)t * dr + (chunk << 4);
     } else {
       const int kr = row - AF_ROWS;
-      src = kb + (long long)kr * D + ((pos ^ ((kr >> 1) & SWZ)) << 4);
+      chunk = pos ^ ((kr >> 1) & SWZ);
+      src = kb + (long long)kr * dr + (chunk << 4);
     }
-    __builtin_amdgcn_global_load_lds((const TI_GLOBAL_AS void*)src, (TI_LDS_AS void*)((TI_LDS_AS char*)smem + i * 1024),
-                                     16, 0, 0);
+    if (chunk < nc)
+      __builtin_amdgcn_global_load_lds((const TI_GLOBAL_AS void*)src,
+                                       (TI_LDS_AS void*)((TI_LDS_AS char*)smem + i * 1024), 16, 0, 0);
+    else
+      *reinterpret_cast<v4i*>(smem + i * 1024 + lane * 16) = v4i{0, 0, 0, 0};
   }
   // ---- mask rows: the values of eight blocks are fetched while the previous eight are consumed, the first
   // eight together with the operand copies
@@ -100,7 +109,7 @@ __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t*
     }
   };
   fetch_mask(0, mk[0]);
-  asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
 
   // ---- scores: acc[j] = q rows (16 of this wave) x key block j
   const int sw = (r >> 1) & SWZ;
@@ -158,14 +167,15 @@ __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t*
   // before the mask rows would have to land before the first mask value could be used.  They run under the
   // exponentials and the quantisation and are waited for in front of P.V.
   if constexpr (PV) {
-    const int8_t* vb = vt + bh * (long long)D * S;
-    const int instrs = (D * pitch) >> 10;  // 1 KiB each
+    const int8_t* vb = vt + bh * (long long)dr * S;
+    const int instrs = (dr * pitch + 1023) >> 10;  // 1 KiB each; rows dr .. D-1 of the panel are never read
     for (int i = wave; i < instrs; i += 4) {
       const int o = i * 1024 + lane * 16;
       int row = o / pitch, col = o - row * pitch;
       col = col < S ? col : 0;  // the 16 pad bytes of a row receive a copy of its first chunk; never read
-      __builtin_amdgcn_global_load_lds((const TI_GLOBAL_AS void*)(vb + (long long)row * S + col),
-                                       (TI_LDS_AS void*)((TI_LDS_AS char*)vts + i * 1024), 16, 0, 0);
+      if (row < dr)
+        __builtin_amdgcn_global_load_lds((const TI_GLOBAL_AS void*)(vb + (long long)row * S + col),
+                                         (TI_LDS_AS void*)((TI_LDS_AS char*)vts + i * 1024), 16, 0, 0);
     }
   }
 
@@ -251,6 +261,8 @@ __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t*
     for (int sl = 0; sl < NB / 4; ++sl) {
       if (4 * sl < nb) {
         const v4i pa = {(int)pw[4 * sl], (int)pw[4 * sl + 1], (int)pw[4 * sl + 2], (int)pw[4 * sl + 3]};
+        // (blocks c >= nc multiply rows of the panel that no copy filled: whatever the LDS holds there; their
+        // results are not stored.  A test on c here cost the 256-key forms their register allocation.)
 #pragma unroll
         for (int c = 0; c < D / 16; ++c) {
           const char* src = vrow + c * 16 * pitch + 64 * sl;
@@ -262,14 +274,14 @@ __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t*
     }
     if (t < T) {
       const long long b = bh / heads, h = bh - b * heads;
-      int* crow = reinterpret_cast<int*>(ctx + ((b * T + t) * heads + h) * (long long)D) + g;
+      int* crow = reinterpret_cast<int*>(ctx + ((b * T + t) * heads + h) * (long long)dr) + g;
 #pragma unroll
       for (int c = 0; c < D / 16; ++c) {
         unsigned w = 0;
 #pragma unroll
         for (int v = 0; v < 4; ++v)
           w |= (unsigned)(unsigned char)Epi<EPI_S8_SCALE>::apply(o[c][v], 0.0f, alpha_pv) << (8 * v);
-        crow[4 * c] = (int)w;
+        if (c < nc) crow[4 * c] = (int)w;
       }
     }
   }
@@ -283,17 +295,23 @@ int launch_attn_long(const int8_t* q, const int8_t* k, const float* mask, int8_t
 
 // shapes the single-sweep kernel of this file takes (all keys of a head in the LDS at once)
 static bool single_sweep_ok(long long T, long long S, long long D, bool pv) {
-  return T >= 1 && (D == 128 || D == 64) && S >= 16 && S <= AF_MAX_S && S % 16 == 0 && (!pv || S % 64 == 0);
+  return T >= 1 && D >= 16 && D <= 128 && D % 16 == 0 && S >= 16 && S <= AF_MAX_S && S % 16 == 0 &&
+         (!pv || S % 64 == 0);
 }
 
 bool attn_qk_softmax_q_supported(long long T, long long S, long long D) {
   return single_sweep_ok(T, S, D, false) || attn_long_supported(T, S, D);
 }
 
+// the form that multiplies on with V^T: the single sweep needs whole slices of 64 keys
+bool attn_prefill_supported(long long T, long long S, long long D) {
+  return single_sweep_ok(T, S, D, true) || attn_long_supported(T, S, D);
+}
+
 template <int NB, bool PV, int SPEC, int D>
 static int launch_af(dim3 grid, size_t lds, hipStream_t stream, const int8_t* q, const int8_t* k, const float* mask,
                      int8_t* probs, int T, int S, long long stride_q, long long stride_k, int heads, int row_blocks,
-                     float alpha, const int8_t* vt, int8_t* ctx, float alpha_pv) {
+                     float alpha, const int8_t* vt, int8_t* ctx, float alpha_pv, int dr) {
   auto kern = attn_qk_softmax_q_kernel<NB, PV, SPEC, D>;
   static unsigned long long lds_ok = 0;  // bit per device: the large dynamic LDS size has been allowed
   int dev = 0;
@@ -305,7 +323,7 @@ static int launch_af(dim3 grid, size_t lds, hipStream_t stream, const int8_t* q,
     lds_ok |= 1ull << dev;
   }
   hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, q, k, mask, probs, T, S, stride_q, stride_k, heads, row_blocks,
-                     alpha, vt, ctx, alpha_pv);
+                     alpha, vt, ctx, alpha_pv, dr);
   return TI_OK;
 }
 
@@ -322,13 +340,15 @@ int launch_attn_qk_softmax_q(const int8_t* q, const int8_t* k, const float* mask
   if (BH * row_blocks > 0x7fffffffLL || T > 0x7fffffffLL)
     return fail(TI_ERR_INVALID_ARG, "attn_qk_softmax_q: too many row blocks (%lld)", BH * row_blocks);
   const dim3 grid((unsigned)(BH * row_blocks));
-  const size_t lds = (size_t)(AF_ROWS + S) * D;
+  const int row_bytes = D <= 64 ? 64 : 128;  // LDS row size = the kernel's template head size
+  const size_t lds = (size_t)(AF_ROWS + S) * row_bytes;
   int rc;
 #define TI_AF(NB, PV, SPEC)                                                                                            \
-  rc = D == 128 ? launch_af<NB, PV, SPEC, 128>(grid, lds, stream, q, k, mask, probs, (int)T, (int)S, stride_q, stride_k, \
-                                               (int)heads, (int)row_blocks, alpha, vt, ctx, alpha_pv)                  \
-                : launch_af<NB, PV, SPEC, 64>(grid, lds, stream, q, k, mask, probs, (int)T, (int)S, stride_q, stride_k,  \
-                                              (int)heads, (int)row_blocks, alpha, vt, ctx, alpha_pv)
+  rc = row_bytes == 128                                                                                                \
+           ? launch_af<NB, PV, SPEC, 128>(grid, lds, stream, q, k, mask, probs, (int)T, (int)S, stride_q, stride_k,      \
+                                          (int)heads, (int)row_blocks, alpha, vt, ctx, alpha_pv, (int)D)               \
+           : launch_af<NB, PV, SPEC, 64>(grid, lds, stream, q, k, mask, probs, (int)T, (int)S, stride_q, stride_k,       \
+                                         (int)heads, (int)row_blocks, alpha, vt, ctx, alpha_pv, (int)D)
 #define TI_AF_NB(NB, PV)                                 \
   do {                                                   \
     if (S != 16 * NB) TI_AF(NB, PV, 0);                  \

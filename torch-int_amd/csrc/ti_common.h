@@ -278,6 +278,7 @@ int launch_permute_0213_s8(const int8_t* src, int8_t* dst, long long B, long lon
 int launch_transpose_last2_s8(const int8_t* src, int8_t* dst, long long B, long long R, long long C,
                               hipStream_t stream);
 bool attn_qk_softmax_q_supported(long long T, long long S, long long D);
+bool attn_prefill_supported(long long T, long long S, long long D);
 int launch_attn_qk_softmax_q(const int8_t* q, const int8_t* k, const float* mask, int8_t* probs, long long BH,
                              long long T, long long S, long long D, long long stride_q, long long stride_k,
                              long long heads, float alpha, const int8_t* vt, int8_t* ctx, float alpha_pv,

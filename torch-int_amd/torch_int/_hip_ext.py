@@ -43,6 +43,8 @@ _lib.ti_kv_append_s8.argtypes = [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i6
 _lib.ti_kv_append_s8.restype = ctypes.c_int
 _lib.ti_attn_qk_softmax_q_supported.argtypes = [_i64, _i64, _i64]
 _lib.ti_attn_qk_softmax_q_supported.restype = ctypes.c_int
+_lib.ti_attn_prefill_supported.argtypes = [_i64, _i64, _i64]
+_lib.ti_attn_prefill_supported.restype = ctypes.c_int
 _lib.ti_attn_qk_softmax_q.argtypes = [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _vp]
 _lib.ti_attn_qk_softmax_q.restype = ctypes.c_int
 _lib.ti_attn_prefill_s8.argtypes = [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _f32, _vp]
@@ -355,7 +357,8 @@ def kv_append(k_new, v_new, k_buf, v_buf, filled, checked=False):
 
 def can_attn_qk_softmax_q(q, k, mask, bsz, heads):
     """int8 HIP q [bsz*heads, T, d] contiguous and k [bsz*heads, S, d] with packed rows (any batch stride that is
-    a multiple of 16), d 64 or 128, S a multiple of 16 up to 4096; mask None or fp32 [bsz, 1, T, S] contiguous."""
+    a multiple of 16), d 64 or 128 and S a multiple of 16 up to 4096, or d any multiple of 16 up to 128 and S up to 512;
+    mask None or fp32 [bsz, 1, T, S] contiguous."""
     if not (_ok(q, torch.int8) and type(k) is torch.Tensor and k.dtype is torch.int8 and k.is_cuda and q.dim() == 3
             and k.dim() == 3 and q.shape[0] == k.shape[0] == bsz * heads and q.shape[2] == k.shape[2]
             and k.device == q.device and q.numel() > 0):
@@ -425,9 +428,16 @@ def attn_qk_softmax_q(q, k, mask, alpha, heads, checked=False):
 
 
 def can_attn_prefill(q, k, vt, mask, bsz, heads):
-    """``can_attn_qk_softmax_q`` plus: vt = V transposed, int8 [bsz*heads, d, S] contiguous."""
+    """``can_attn_qk_softmax_q`` plus: vt = V transposed, int8 [bsz*heads, d, S] contiguous, and a shape the form
+    that multiplies on with V takes (``ti_attn_prefill_supported``)."""
     return (can_attn_qk_softmax_q(q, k, mask, bsz, heads) and _ok(vt, torch.int8)
-            and vt.shape == (q.shape[0], q.shape[2], k.shape[1]) and vt.device == q.device and vt.data_ptr() % 16 == 0)
+            and vt.shape == (q.shape[0], q.shape[2], k.shape[1]) and vt.device == q.device and vt.data_ptr() % 16 == 0
+            and bool(_lib.ti_attn_prefill_supported(q.shape[1], k.shape[1], q.shape[2])))
+
+
+def attn_prefill_shape_ok(T, S, d):
+    """Whether ``attn_prefill`` takes T query rows over S keys at head size d (cheap: before V is transposed)."""
+    return bool(_lib.ti_attn_prefill_supported(int(T), int(S), int(d)))
 
 
 def attn_prefill(q, k, vt, mask, alpha_qk, alpha_pv, heads, checked=False):

@@ -303,19 +303,21 @@ class Int8OPTAttention(nn.Module):
         # they are taken for a plain prefill (tgt_len == src_len) only.
         long_ok = src_len <= 512 or tgt_len == src_len
         if (self.fused_softmax and long_ok and layer_head_mask is None and not output_attentions and tgt_len > 16
-                and d % 16 == 0 and d < 128 and d != 64 and query.is_cuda
-                and type(self.qk_bmm) is BMM_S8T_S8N_F32T and type(self.pv_bmm) is BMM_S8T_S8N_S8T):
-            ctx = self._prefill_padded_heads(query, key, value, attention_mask, bsz, tgt_len)
-            if ctx is not None:
-                return self.out_proj(ctx), None, present
-        if (self.fused_softmax and long_ok and layer_head_mask is None and not output_attentions and tgt_len > 16
                 and type(self.qk_bmm) is BMM_S8T_S8N_F32T and type(self.pv_bmm) is BMM_S8T_S8N_S8T
-                and _hip_ext.can_attn_qk_softmax_q(query, key, attention_mask, bsz, H) and value.is_cuda):
+                and _hip_ext.can_attn_qk_softmax_q(query, key, attention_mask, bsz, H) and value.is_cuda
+                and _hip_ext.attn_prefill_shape_ok(tgt_len, src_len, d)):
             # the whole attention (Q.K^T, softmax-quant, P.V, head merge) in one kernel on V transposed
             vt = _hip_ext.transpose_last2(value.contiguous())
             if _hip_ext.can_attn_prefill(query, key, vt, attention_mask, bsz, H):
                 ctx = _hip_ext.attn_prefill(query, key, vt, attention_mask, self.qk_bmm._scalar("a"),
                                             self.pv_bmm._scalar("a"), H, checked=True)
+                return self.out_proj(ctx), None, present
+        if (self.fused_softmax and long_ok and layer_head_mask is None and not output_attentions and tgt_len > 16
+                and d % 16 == 0 and d < 128 and d != 64 and query.is_cuda
+                and type(self.qk_bmm) is BMM_S8T_S8N_F32T and type(self.pv_bmm) is BMM_S8T_S8N_S8T):
+            # a head size that the kernel taking this many keys has no form of (OPT-2.7B: 80 beyond 512 keys)
+            ctx = self._prefill_padded_heads(query, key, value, attention_mask, bsz, tgt_len)
+            if ctx is not None:
                 return self.out_proj(ctx), None, present
         probs_q = None
         if (self.fused_softmax and long_ok and layer_head_mask is None and tgt_len > 16
