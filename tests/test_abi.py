@@ -269,3 +269,24 @@ def test_graph_decoder_refuses_steps_beyond_its_buffers():
     dec.filled, dec.max_length = 40, 40
     with pytest.raises(RuntimeError, match="max_new_tokens"):
         dec.step(torch.zeros(1, 1, dtype=torch.long))
+
+
+def test_only_the_256x288_gemm_tiles_spill_registers():
+    """The build writes every kernel's register and scratch use (the compiler's own figures) next to the library.
+    A kernel that spills still gives the right bits, several times slower, so parity tests cannot see it: only the
+    256x288 GEMM tiles, whose 144 accumulator registers per lane leave too few for the operands, are allowed to
+    (they are priced with that cost), and every pipelined GEMM and fused attention kernel must fit two waves per
+    SIMD (256 registers per lane), which their launch bounds and tilings assume."""
+    import json
+    import torch_int._CUDA as C
+    path = os.path.join(os.path.dirname(C.LIB_PATH), "kernel_resources.json")
+    if not os.path.exists(path) or os.path.getmtime(path) + 60 < os.path.getmtime(C.LIB_PATH):
+        pytest.skip("no kernel_resources.json from the build of this library")
+    kernels = json.load(open(path))["kernels"]
+    assert len(kernels) > 300
+    spilling = sorted(k for k, v in kernels.items() if v.get("scratch_bytes_per_lane", 0) > 0)
+    unexpected = [k for k in spilling if "ILi256ELi288E" not in k]
+    assert not unexpected, unexpected
+    for k, v in kernels.items():
+        if "gemm_pipe" in k or "attn_qk_softmax_q_kernel" in k or "attn_long_kernel" in k:
+            assert v["occupancy_waves_per_simd"] >= 2 and v["vgprs"] + v.get("agprs", 0) <= 256, (k, v)

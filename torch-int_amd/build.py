@@ -41,6 +41,29 @@ def build_fastcall(verbose=True):
     return out
 
 
+def write_kernel_resources(remarks):
+    """The compiler's per-kernel resource remarks as torch_int/lib/kernel_resources.json: registers, scratch bytes per
+    lane (register spills) and occupancy of every kernel in the library.  A kernel that starts to spill after an edit
+    still computes the right bits, only several times slower; tests/test_abi.py reads this file."""
+    import json
+    import re
+    kernels, name = {}, None
+    for ln in remarks:
+        m = re.search(r"remark: (?:[^:]*:\d+:\d+: )?(.*?) \[-Rpass-analysis", ln)
+        text = m.group(1).strip() if m else ln
+        if text.startswith("Function Name:"):
+            name = text.split(":", 1)[1].strip()
+            kernels[name] = {}
+        elif name is not None:
+            for key, label in (("vgprs", "VGPRs:"), ("agprs", "AGPRs:"), ("scratch_bytes_per_lane", "ScratchSize [bytes/lane]:"),
+                               ("occupancy_waves_per_simd", "Occupancy [waves/SIMD]:"), ("lds_bytes_per_block", "LDS Size [bytes/block]:")):
+                if text.startswith(label):
+                    kernels[name][key] = int(text.split(":", 1)[1].strip())
+    with open(os.path.join(LIB_DIR, "kernel_resources.json"), "w") as f:
+        json.dump({"kernels": kernels}, f, indent=0, sort_keys=True)
+    return kernels
+
+
 def build(verbose=True, extra_flags=()):
     """Compiles every source to an object file (in parallel: the files are independent) and links them."""
     from concurrent.futures import ThreadPoolExecutor
@@ -51,14 +74,24 @@ def build(verbose=True, extra_flags=()):
     def compile_one(item):
         src, defines, name = item
         obj = os.path.join(obj_dir, name)
-        cmd = [HIPCC, *FLAGS, *defines, *extra_flags, "-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = [HIPCC, *FLAGS, "-Rpass-analysis=kernel-resource-usage", *defines, *extra_flags, "-c",
+               os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
-        subprocess.check_call(cmd)
-        return obj
+        done = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
+        remarks = [ln for ln in done.stderr.splitlines() if "[-Rpass-analysis=kernel-resource-usage]" in ln]
+        rest = [ln for ln in done.stderr.splitlines() if "[-Rpass-analysis=kernel-resource-usage]" not in ln]
+        if verbose or done.returncode:
+            sys.stdout.write(done.stdout)
+            sys.stderr.write("\n".join(rest) + ("\n" if rest else ""))
+        if done.returncode:
+            raise subprocess.CalledProcessError(done.returncode, cmd)
+        return obj, remarks
 
     with ThreadPoolExecutor(max_workers=min(len(SOURCES), os.cpu_count() or 4, 16)) as pool:
-        objs = list(pool.map(compile_one, SOURCES))
+        results = list(pool.map(compile_one, SOURCES))
+    objs = [obj for obj, _ in results]
+    write_kernel_resources([ln for _, remarks in results for ln in remarks])
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH, *objs]
     if verbose:
         print(" ".join(cmd), flush=True)
