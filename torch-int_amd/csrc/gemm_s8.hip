@@ -342,8 +342,8 @@ int launch_gemm_group_s8(const GemmParams& shape, const GemmGroup& grp, hipStrea
   if (aligned && shape.M <= 16 && strips >= 256) {
     g_last_kernel = "stream_group";
     const int cus = num_cus();
-    auto launch = [&](auto kern, int rows, int per_cu) -> int {
-      const int lds = 2 * rows * SBK + S_RED;
+    auto launch = [&](auto kern, int stages, int rows, int per_cu) -> int {
+      const int lds = stages * rows * SBK + S_RED;
       static std::atomic<unsigned long long> lds_ok{0};
       if (int rc = allow_lds(kern, lds, lds_ok)) return rc;
       const long long slots = (long long)cus * per_cu;
@@ -353,9 +353,13 @@ int launch_gemm_group_s8(const GemmParams& shape, const GemmGroup& grp, hipStrea
       if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "gemm launch: %s", hipGetErrorString(e));
       return TI_OK;
     };
-    if (shape.M == 1) return launch(gemm_stream_kernel<KIND, 1, 2, true>, 17, 4);
-    if (shape.M <= 4) return launch(gemm_stream_kernel<KIND, 4, 2, true>, 20, 3);
-    return launch(gemm_stream_kernel<KIND, 16, 2, true>, 32, 2);
+    const bool deep = stream_deep_pipeline(shape.M, strips, cus);
+    if (shape.M == 1)
+      return deep ? launch(gemm_stream_kernel<KIND, 1, 3, true>, 3, 17, 2)
+                  : launch(gemm_stream_kernel<KIND, 1, 2, true>, 2, 17, 3);
+    if (shape.M <= 4) return launch(gemm_stream_kernel<KIND, 4, 2, true>, 2, 20, 3);
+    return deep ? launch(gemm_stream_kernel<KIND, 16, 3, true>, 3, 32, 1)
+                : launch(gemm_stream_kernel<KIND, 16, 2, true>, 2, 32, 2);
   }
   // Prefill shapes whose width the 256x160, 256x288 or 256x128 tiles divide: the problems are the batches of one
   // persistent launch, so the pipeline fill and the epilogue of one projection overlap the next one's work.

@@ -2374,6 +2374,22 @@ static int row_split_rows(long long M, long long N, long long K, long long* rest
   return (int)r;
 }
 
+// Stages and resident workgroups of the streaming kernel.  One row: three stages of 17 KiB with two workgroups per
+// CU read cold weights 3-6 % faster than two stages with three or four (1x20480x5120 20.1 -> 19.0 us, 1x36864x9216
+// 54.2 -> 52.3 us) -- unless the strips then fall into rounds that leave CUs idle (576 strips on 512 workgroups:
+// 62.5 against 58.3 us), where two stages with three workgroups (768) stay.  Five to sixteen rows: two stages of
+// 32 KiB with two workgroups per CU, except where one workgroup per CU with three stages quantises much better
+// (16x9216x36864, 576 strips: 86.9 -> 75.0 us).  Two to four rows keep two stages and three workgroups.
+static inline bool stream_deep_pipeline(int M, long long strips, int cus) {
+  auto waste = [&](long long slots) {  // work of the fullest workgroup slot over the mean
+    if (strips <= slots) return 1.0;
+    return (double)((strips + slots - 1) / slots * slots) / (double)strips;
+  };
+  if (M == 1) return waste(2LL * cus) <= 1.15 * waste(3LL * cus);
+  if (M > 4) return waste(2LL * cus) >= 1.3 * waste(1LL * cus);
+  return false;
+}
+
 template <int KIND>
 int launch_kind(const GemmParams& p, void* workspace, long long workspace_bytes, hipStream_t stream) {
   using Out = typename Epi<KIND>::Out;
@@ -2395,8 +2411,6 @@ int launch_kind(const GemmParams& p, void* workspace, long long workspace_bytes,
     const long long strips = (long long)spb * p.batch;
     if (strips > 0x7fffffffLL) return fail(TI_ERR_INVALID_ARG, "too many output strips (%lld)", strips);
     const int cus = num_cus();
-    // Stage depth beyond two did not raise the measured bandwidth (5.2-5.4 TB/s at N=20480), so two
-    // stages and as many resident workgroups as the LDS allows.
     auto launch = [&](auto kern, int stages, int rows, int per_cu) -> int {
       const int lds = stages * rows * SBK + S_RED;
       static std::atomic<unsigned long long> lds_ok{0};  // one mask per kernel instantiation (the lambda is generic)
@@ -2408,9 +2422,10 @@ int launch_kind(const GemmParams& p, void* workspace, long long workspace_bytes,
       if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "gemm launch: %s", hipGetErrorString(e));
       return TI_OK;
     };
-    if (p.M == 1) return launch(gemm_stream_kernel<KIND, 1, 2>, 2, 17, 4);
+    const bool deep = stream_deep_pipeline(p.M, strips, cus);
+    if (p.M == 1) return deep ? launch(gemm_stream_kernel<KIND, 1, 3>, 3, 17, 2) : launch(gemm_stream_kernel<KIND, 1, 2>, 2, 17, 3);
     if (p.M <= 4) return launch(gemm_stream_kernel<KIND, 4, 2>, 2, 20, 3);
-    return launch(gemm_stream_kernel<KIND, 16, 2>, 2, 32, 2);
+    return deep ? launch(gemm_stream_kernel<KIND, 16, 3>, 3, 32, 1) : launch(gemm_stream_kernel<KIND, 16, 2>, 2, 32, 2);
   }
   if (p.M <= 16) {
     g_last_kernel = "skinny";
