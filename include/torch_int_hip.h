@@ -136,6 +136,14 @@ int ti_diag_store_loop(float* out, int64_t M, int64_t N, int workgroups, int rep
 int ti_diag_copy_loop(int mode, const int8_t* data, int64_t data_bytes, int64_t iters, int32_t* sink, void* stream);
 int64_t ti_diag_copy_loop_bytes(int64_t iters);
 
+/* Diagnostic (no counterpart in the reference; computes nothing): one pass over an int8 matrix data[N][K] (N a multiple
+ * of 16, K of 1024, 16-byte aligned device memory of N*K bytes) with the loads alone, to learn what a kernel that reads
+ * its weights once can reach.  mode 0: flat 4 KiB pieces per workgroup, four loads in flight per lane; 1: the same,
+ * non-temporal; 2: the copy pipeline of the M <= 16 streaming GEMM without its arithmetic (strips of 16 rows, 1 KiB per
+ * row and global->LDS copy, three stages, one wait and barrier per block, two workgroups per CU, non-temporal copies);
+ * 3: mode 2 with the default cache policy.  `sink` as for ti_diag_mfma_loop. */
+int ti_diag_read_loop(int mode, const int8_t* data, int64_t N, int64_t K, int32_t* sink, void* stream);
+
 /* Diagnostic (no counterpart in the reference; computes nothing): one workgroup per CU issues, `iters` times, the
  * instructions a wave of the 16x16-block GEMM kernels issues per 128-byte K step and nothing else, on operands that
  * change every step.  shape 0 = the 256x160 tile (8 waves, each 40 v_mfma_i32_16x16x64_i8, 18 ds_read_b128, 7 1-KiB

@@ -80,6 +80,11 @@ def test_c_abi_rejects_bad_arguments_without_a_device():
                                      ctypes.c_void_p, ctypes.c_void_p]
     assert lib.ti_diag_mix_loop(0, 15, p, 2 << 20, 10, p, None) == 1 and b"3 MiB" in lib.ti_last_error()
     assert lib.ti_diag_mix_loop(0, 15, p, 3 << 20, 0, p, None) == 1 and b"iters" in lib.ti_last_error()
+    lib.ti_diag_read_loop.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p,
+                                      ctypes.c_void_p]
+    assert lib.ti_diag_read_loop(4, p, 16, 1024, p, None) == 1 and b"mode" in lib.ti_last_error()
+    assert lib.ti_diag_read_loop(2, p, 24, 1024, p, None) == 1 and b"multiple of 16" in lib.ti_last_error()
+    assert lib.ti_diag_read_loop(2, p, 16, 1000, p, None) == 1 and b"multiple of 1024" in lib.ti_last_error()
     # beyond the 32-bit tiling limits
     rc = lib.ti_linear_a8_w8_b32_o32(p, p, p, p, 1 << 20, 4, 1 << 20, None, 0, None)
     assert rc == 1 and b"limits" in lib.ti_last_error()

@@ -1095,6 +1095,15 @@ def test_diag_copy_and_mix_loops_run_and_report_their_work():
             _say(f"diag_mix_loop shape {shape} parts {parts}")
             assert X.diag_mix_loop(shape, parts, data, 50, sink) == cus * per_cu * 50 * 32768
         torch.cuda.synchronize()
+    # the read-rate diagnostic: every mode launches and exits, for fewer strips than workgroups and for more
+    for (N, K) in [(16, 1024), (64, 3072), (9216, 2048), (20480, 1024)]:
+        mat = torch.randint(-127, 128, (N, K), dtype=torch.int8, device=DEV)
+        for mode in range(4):
+            _say(f"diag_read_loop mode {mode} {N}x{K}")
+            assert X.diag_read_loop(mode, mat, sink) == N * K
+        torch.cuda.synchronize()
+    with pytest.raises(RuntimeError):
+        X.diag_read_loop(2, torch.zeros(24, 1024, dtype=torch.int8, device=DEV), sink)
     assert int(sink.item()) == 0
     for bad in (lambda: X.diag_copy_loop(2, data, 50, sink), lambda: X.diag_mix_loop(2, 15, data, 50, sink),
                 lambda: X.diag_mix_loop(0, 16, data, 50, sink), lambda: X.diag_mix_loop(0, 15, data[: 1 << 20], 50, sink)):

@@ -15,6 +15,8 @@ Examples
   python torch-int_amd/benchmark/bench_kernel.py --op copy_loop --shape 0 4000     # L2 -> CU copy rate: mode (0 into LDS, 1 into registers), steps
   python torch-int_amd/benchmark/bench_kernel.py --op mix_loop --shape 0 15 20000   # floor of a K step: tile (0 256x160, 1 128x80), parts
       # (bit set: 1 MFMAs, 2 fragment reads, 4 copies, 8 barrier), steps; us / steps = time per K step
+  python torch-int_amd/benchmark/bench_kernel.py --op read_loop --shape 2 20480 5120 --rotate 13   # read rate of a weight matrix:
+      # mode (0 flat, 1 flat non-temporal, 2 the streaming GEMM's copies alone, 3 those with the default cache policy), N, K
   rocprofv3 --kernel-trace --stats --output-format csv -d out -- python3 .../bench_kernel.py --op ...
 
 Prints one JSON line: mean microseconds per call (HIP events on the launch stream), algorithmic
@@ -45,7 +47,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--op", required=True, choices=list(LINEAR) + ["bmm_f32t", "bmm_s8t", "bmm_s32t", "bmm_s8t_rowmajor", "ln_q", "ln_q_f16", "add_ln_q",
                                                "softmax_q", "qk_softmax_q", "attn_prefill", "decode_attn", "transpose_last2", "copy",
-                                               "mfma_loop", "mfma_ceiling", "store_loop", "copy_loop", "mix_loop"])
+                                               "mfma_loop", "mfma_ceiling", "store_loop", "copy_loop", "mix_loop", "read_loop"])
     ap.add_argument("--shape", type=int, nargs="+", required=True)
     ap.add_argument("--iters", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
@@ -204,6 +206,16 @@ def main():
         data, sink = s8(2 << 20), torch.zeros(1, dtype=torch.int32, device=dev)
         nbytes = float(X.diag_copy_loop(mode, data, steps, sink))
         fn = lambda: X.diag_copy_loop(mode, data, steps, sink)  # noqa: E731
+    elif args.op == "read_loop":
+        # one read-only pass over an int8 [N, K] matrix; --rotate copies so that none stays in the last-level cache
+        mode, N, K = args.shape
+        mats, sink = [s8(N, K) for _ in range(max(1, args.rotate))], torch.zeros(1, dtype=torch.int32, device=dev)
+        nbytes = float(N) * K
+        state = {"i": 0}
+
+        def fn():
+            state["i"] += 1
+            X.diag_read_loop(mode, mats[state["i"] % len(mats)], sink)
     else:  # plain device copy of a known size: reference reading for FETCH_SIZE / WRITE_SIZE
         n, = args.shape
         src = torch.empty(n, dtype=torch.uint8, device=dev).random_(generator=g)

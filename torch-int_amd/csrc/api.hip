@@ -488,6 +488,14 @@ int ti_diag_copy_loop(int mode, const int8_t* data, int64_t data_bytes, int64_t 
   return launch_diag_copy_loop(mode, data, iters, sink, static_cast<hipStream_t>(stream));
 }
 
+int ti_diag_read_loop(int mode, const int8_t* data, int64_t N, int64_t K, int32_t* sink, void* stream) {
+  g_err[0] = 0;
+  const char* op = "diag_read_loop";
+  if (int rc = check_ptr(op, "data", data, 16, true)) return rc;
+  if (int rc = check_ptr(op, "sink", sink, 4, true)) return rc;
+  return launch_diag_read_loop(mode, data, N, K, sink, static_cast<hipStream_t>(stream));
+}
+
 int64_t ti_diag_mix_loop_ops(int shape, int64_t iters) { return iters > 0 ? diag_mix_loop_ops(shape, iters) : 0; }
 
 int ti_diag_mix_loop(int shape, int parts, const int8_t* data, int64_t data_bytes, int64_t iters, int32_t* sink,

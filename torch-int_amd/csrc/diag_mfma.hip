@@ -184,6 +184,102 @@ __global__ __launch_bounds__(512) void copy_loop_kernel(const int8_t* __restrict
   if (acc[0] + acc[1] + acc[2] + acc[3] == 0x12345678 || (iters < 0 && smem[threadIdx.x] == 77)) sink[0] = 1;
 }
 
+// Read-rate diagnostic: one pass over a weight matrix [N][K] of int8 with nothing but the loads, for the ceilings of
+// the HBM-bound kernels (the streaming GEMM above all).
+//   mode 0  flat: every workgroup reads 4 KiB pieces (256 lanes x 16 bytes), four in flight per lane, grid-stride
+//   mode 1  the same with non-temporal loads
+//   mode 2  the streaming GEMM's copy pipeline without its arithmetic: a workgroup of four waves owns strips of 16
+//           rows and walks K in blocks of 1 KiB per row (one global->LDS copy instruction per row and block, waves
+//           1..3 copy), three LDS stages, one wait and one barrier per block, non-temporal copies
+//   mode 3  mode 2 with the default cache policy
+template <bool NT>
+__global__ __launch_bounds__(256) void read_flat_kernel(const v4i* __restrict__ src, long long n16, int* sink) {
+  v4i acc = {0, 0, 0, 0};
+  const long long stride = (long long)gridDim.x * 1024;
+  for (long long i = (long long)blockIdx.x * 1024 + threadIdx.x; i < n16; i += stride) {
+    v4i v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const v4i* a = src + i + u * 256;
+      v[u] = i + u * 256 < n16 ? (NT ? __builtin_nontemporal_load(a) : *a) : v4i{0, 0, 0, 0};
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) acc ^= v[u];
+  }
+  if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x12345678) sink[0] = 1;
+}
+
+template <int AUX>
+__global__ __launch_bounds__(256) void read_strips_kernel(const char* __restrict__ w, int N, int K, int* sink) {
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  constexpr int S = 3, STAGE = 16 * 1024, NCOPY = 6;  // 3 copying waves x 6 row copies >= 16 rows
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int strips = N / 16, KB = K / 1024;
+  int my = 0;
+  for (int s = blockIdx.x; s < strips; s += gridDim.x) ++my;
+  if (my == 0) return;  // the same for every wave of the workgroup, before the first barrier
+  const int G = my * KB;
+  const int cw = wave > 0 ? wave - 1 : 0;
+  int c_s = blockIdx.x, c_kb = 0, c_g = 0, live = 1;
+  auto issue = [&]() {
+    TI_LDS_AS char* dst = (TI_LDS_AS char*)smem + (c_g % S) * STAGE;
+    const char* base = w + (size_t)c_s * 16 * K + (size_t)c_kb * 1024 + lane * 16;
+#pragma unroll
+    for (int i = 0; i < NCOPY; ++i) {
+      int q = cw + 3 * i;
+      q = q < 16 ? q : 15;
+      __builtin_amdgcn_global_load_lds((const TI_GLOBAL_AS void*)(base + (size_t)q * K), (TI_LDS_AS void*)(dst + q * 1024),
+                                       16, 0, AUX);
+    }
+    c_kb += live;
+    ++c_g;
+    if (live && c_kb == KB) {  // past the last strip the final block is copied again: the wait count never changes
+      if (c_g < G) {
+        c_kb = 0;
+        c_s += gridDim.x;
+      } else {
+        live = 0;
+        c_kb = KB - 1;
+      }
+    }
+  };
+  if (wave > 0)
+    for (int i = 0; i < S - 1; ++i) issue();
+  int acc = 0;
+  for (int g = 0; g < G; ++g) {
+    if (wave > 0) asm volatile("s_waitcnt vmcnt(%0)" ::"n"((S - 2) * NCOPY) : "memory");
+    asm volatile("s_barrier" ::: "memory");
+    if (wave > 0) issue();
+    acc ^= *reinterpret_cast<const int*>(smem + (g % S) * STAGE + threadIdx.x * 4);
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  if (acc == 0x12345678) sink[0] = 1;
+}
+
+int launch_diag_read_loop(int mode, const int8_t* data, long long N, long long K, int* sink, hipStream_t stream) {
+  if (mode < 0 || mode > 3) return fail(TI_ERR_INVALID_ARG, "diag_read_loop: mode must be 0 ... 3 (got %d)", mode);
+  if (N < 16 || N % 16 != 0 || K < 1024 || K % 1024 != 0 || N > (1 << 24) || K > (1 << 24))
+    return fail(TI_ERR_INVALID_ARG, "diag_read_loop: N must be a multiple of 16 and K a multiple of 1024 (got %lld, %lld)",
+                N, K);
+  const int cus = diag_grid();
+  if (mode <= 1) {
+    auto kern = mode == 0 ? read_flat_kernel<false> : read_flat_kernel<true>;
+    hipLaunchKernelGGL(kern, dim3(cus * 4), dim3(256), 0, stream, reinterpret_cast<const v4i*>(data), N * K / 16, sink);
+  } else {
+    auto kern = mode == 2 ? read_strips_kernel<2> : read_strips_kernel<0>;
+    const int lds = 3 * 16 * 1024 + 29 * 1024;  // padded to 77 KiB: two workgroups per CU, as the GEMM kernel has
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    const long long strips = N / 16, slots = 2LL * cus;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(strips < slots ? strips : slots)), dim3(256), lds, stream,
+                       reinterpret_cast<const char*>(data), (int)N, (int)K, sink);
+  }
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "read loop launch: %s", hipGetErrorString(e));
+  return TI_OK;
+}
+
 long long diag_copy_loop_bytes(long long iters) { return (long long)diag_grid() * 8 * kCopyPieces * 1024 * iters; }
 
 int launch_diag_copy_loop(int mode, const int8_t* data, long long iters, int* sink, hipStream_t stream) {

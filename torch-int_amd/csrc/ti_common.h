@@ -298,6 +298,7 @@ int launch_kv_append_s8(const int8_t* knew, const int8_t* vnew, int8_t* kbuf, in
 int launch_diag_mfma_loop(int mode, const int8_t* data, long long iters, int* sink, hipStream_t stream);
 long long diag_mfma_loop_ops(long long iters);
 int launch_diag_store_loop(float* out, long long M, long long N, int workgroups, int reps, hipStream_t stream);
+int launch_diag_read_loop(int mode, const int8_t* data, long long N, long long K, int* sink, hipStream_t stream);
 int launch_diag_copy_loop(int mode, const int8_t* data, long long iters, int* sink, hipStream_t stream);
 long long diag_copy_loop_bytes(long long iters);
 int launch_diag_mix_loop(int shape, int parts, const int8_t* data, long long iters, int* sink, hipStream_t stream);

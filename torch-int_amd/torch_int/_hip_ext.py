@@ -85,6 +85,8 @@ _lib.ti_linear_group_is_one_launch.restype = ctypes.c_int
 _group_one_launch = {}
 _lib.ti_diag_copy_loop.argtypes = [ctypes.c_int, _vp, _i64, _i64, _vp, _vp]
 _lib.ti_diag_copy_loop.restype = ctypes.c_int
+_lib.ti_diag_read_loop.argtypes = [ctypes.c_int, _vp, _i64, _i64, _vp, _vp]
+_lib.ti_diag_read_loop.restype = ctypes.c_int
 _lib.ti_diag_copy_loop_bytes.argtypes = [_i64]
 _lib.ti_diag_copy_loop_bytes.restype = _i64
 _lib.ti_diag_mix_loop.argtypes = [ctypes.c_int, ctypes.c_int, _vp, _i64, _i64, _vp, _vp]
@@ -680,6 +682,22 @@ def diag_store_loop(out, workgroups, reps=1):
     if rc:
         raise RuntimeError(f"torch_int._hip_ext.diag_store_loop: {_lib.ti_last_error().decode()} (status {rc})")
     return out.numel() * 4 * int(reps)
+
+
+def diag_read_loop(mode, data, sink):
+    """One read-only pass over the int8 matrix ``data`` [N, K] (``ti_diag_read_loop``): mode 0 flat, 1 flat
+    non-temporal, 2 the streaming GEMM's copy pipeline (non-temporal), 3 the same with the default cache policy.
+    Returns the bytes read."""
+    if not (_ok(data, torch.int8) and data.dim() == 2):
+        raise RuntimeError("torch_int._hip_ext.diag_read_loop: data must be a contiguous int8 HIP matrix")
+    if not (_ok(sink, torch.int32) and sink.device == data.device and sink.numel() >= 1):
+        raise RuntimeError("torch_int._hip_ext.diag_read_loop: sink must be an int32 HIP tensor on the same device")
+    with _on(data.device):
+        rc = _lib.ti_diag_read_loop(int(mode), data.data_ptr(), data.shape[0], data.shape[1], sink.data_ptr(),
+                                    _raw_stream(data.device.index) or None)
+    if rc:
+        raise RuntimeError(f"torch_int._hip_ext.diag_read_loop: {_lib.ti_last_error().decode()} (status {rc})")
+    return data.numel()
 
 
 def diag_copy_loop(mode, data, iters, sink):
