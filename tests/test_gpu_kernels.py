@@ -560,6 +560,32 @@ def test_stream_kernel_strip_orders_and_ragged_widths():
         assert C._lib.ti_last_kernel().decode() == "stream"
 
 
+def test_stream_kernel_on_the_view_with_rows_cut_into_parts():
+    # one or two rows of activations against few, long weight rows (fc2 of a decode step): the streaming kernel
+    # multiplies the view with every row cut into four (two) parts and its epilogue adds the parts of each output.
+    # Every output kind, widths with a last partial run of strips, the shapes next to the rule's limits.
+    import ctypes
+    import torch_int._CUDA as C
+    C._lib.ti_last_kernel.restype = ctypes.c_char_p
+    g = torch.Generator().manual_seed(92)
+    for (M, N, K, kern) in [(1, 5120, 20480, "stream_parts"), (1, 4096, 8192, "stream_parts"), (1, 9232, 12288, "stream_parts"),
+                            (2, 5120, 20480, "stream_parts"), (2, 4112, 10240, "stream_parts"), (1, 16384, 8192, "stream_parts"),
+                            (1, 5120, 10240, "stream"), (2, 5120, 7168, "stream"), (3, 5120, 20480, "stream"),
+                            (1, 4104, 8192, "stream"), (1, 16400, 8192, "stream"), (1, 4096, 16384, "stream"),
+                            (2, 4096, 8192, "stream")]:
+        for variant in VARIANTS:
+            _say(f"stream view {variant} M={M} N={N} K={K}")
+            _linear_case(C, variant, M, N, K, seed=92)
+            assert C._lib.ti_last_kernel().decode() == kern, (M, N, K, C._lib.ti_last_kernel())
+        _say(f"stream view += M={M} N={N} K={K}")
+        x, w = _s8(g, M, K), _s8(g, N, K)
+        bias, resid = torch.randn(N, generator=g), torch.randn(M, N, generator=g) * 3
+        ref = orc.linear_a8_w8_bfp32_ofp32_acc(x, w, bias, 0.003, 1.0, resid)
+        out = C._linear_a8_w8_bfp32_ofp32_acc(x.to(DEV), w.to(DEV), bias.to(DEV), 0.003, 1.0, resid.to(DEV))
+        assert _ulp_diff(out.cpu(), ref) == 0, (M, N, K)
+        assert C._lib.ti_last_kernel().decode() == kern
+
+
 def test_one_launch_split_k_is_exact_for_every_output_kind():
     # 2 to 4 K slices on a tile of the 16x16-block kernel that divides M: the slices of a tile meet in one XCD's L2 and
     # the wave that arrives last applies the epilogue.  Every tile shape, every epilogue, sampled rows against the

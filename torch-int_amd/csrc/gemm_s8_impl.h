@@ -1771,9 +1771,15 @@ static constexpr int S_RED = 3 * 256 * 4;  // partial tiles of waves 1..3
 // MX = activation rows staged per block (1, 4 or 16 >= M); S = LDS stages.
 // GROUPED: the "batches" are the problems of a GemmGroup (same activations and shape; weight, bias,
 // output and scales per problem) instead of slices of one strided tensor.
-template <int KIND, int MX, int S, bool GROUPED = false>
+// PARTS = 2 or 4 (one batch, plain row-major output): the launch multiplies the VIEW of the problem in which every
+// row of the activations and of the weights is cut into PARTS rows of K / PARTS bytes -- p holds the view: M, N
+// and PARTS times the real ones, K, lda, ldb a PARTS-th -- and the epilogue adds the PARTS entries of the product
+// of the views that belong to one output, out[m][n] = sum_f C'[n PARTS + f][m PARTS + f].  A weight matrix with few,
+// long rows (fc2 of a decode step) then has PARTS times the strips, of rows a PARTS-th as far apart.
+template <int KIND, int MX, int S, bool GROUPED = false, int PARTS = 1>
 __global__ __launch_bounds__(256) void gemm_stream_kernel(GemmParams p, int strips_per_batch, int strips,
                                                           GemmGroup grp) {
+  static_assert(PARTS == 1 || ((PARTS == 2 || PARTS == 4) && !GROUPED), "views of two or four parts, one problem");
   constexpr int ROWS = 16 + MX;              // row copies per block
   constexpr int COPIES = (ROWS + 2) / 3;     // per copying wave (1..3); indices past ROWS repeat the last row copy
   constexpr int STAGE = ROWS * SBK;
@@ -1873,6 +1879,22 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(GemmParams p, int stri
   typename EpiT::Bias bias_pre[4];
   typename EpiT::Out old_pre[4];
   auto fetch_epilogue_operands = [&](int strip_) {
+    if constexpr (PARTS > 1) {
+      // lane (r, g) of the view's tile ends up with the real outputs (m = r / PARTS, n = n_first .. + 4 / PARTS - 1)
+      const int n_real = N / PARTS, m_real = M / PARTS;
+      const int n_first = strip_ * (16 / PARTS) + g * (4 / PARTS);
+      const int m = r / PARTS < m_real ? r / PARTS : m_real - 1;
+      const typename EpiT::Bias* bias = reinterpret_cast<const typename EpiT::Bias*>(p.bias);
+      const typename EpiT::Out* C = reinterpret_cast<const typename EpiT::Out*>(p.C);
+#pragma unroll
+      for (int v = 0; v < 4 / PARTS; ++v) {
+        const int n = n_first + v < n_real ? n_first + v : n_real - 1;
+        if constexpr (EpiT::kHasBias) bias_pre[v] = bias[n];
+        else bias_pre[v] = typename EpiT::Bias(0);
+        if constexpr (EpiT::kAccumulate) old_pre[v] = C[(size_t)m * n_real + n];
+      }
+      return;
+    }
     const int b = strip_ / strips_per_batch;
     const int nb = (strip_ - b * strips_per_batch) * 16 + 4 * g;
     const typename EpiT::Bias* bias = reinterpret_cast<const typename EpiT::Bias*>(GROUPED ? grp.bias[b] : p.bias);
@@ -1930,6 +1952,37 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(GemmParams p, int stri
         for (int w = 0; w < 3; ++w)
 #pragma unroll
           for (int v = 0; v < 4; ++v) acc[v] += red[w * 256 + v * 64 + lane];
+        if constexpr (PARTS > 1) {
+          // entry (n' = 4g + v, m' = r) of the view's tile belongs to output (n' / PARTS, m' / PARTS) when
+          // n' % PARTS == m' % PARTS: each lane picks its own, the PARTS lanes of an output add up
+          using E = Epi<KIND>;
+          using Out = typename E::Out;
+          const int n_real = N / PARTS, m_real = M / PARTS;
+          const int f = r & (PARTS - 1);
+          int d[4 / PARTS];
+          if constexpr (PARTS == 4) {
+            d[0] = f == 0 ? acc[0] : f == 1 ? acc[1] : f == 2 ? acc[2] : acc[3];
+          } else {
+            d[0] = f == 0 ? acc[0] : acc[1];
+            d[1] = f == 0 ? acc[2] : acc[3];
+          }
+#pragma unroll
+          for (int v = 0; v < 4 / PARTS; ++v) {
+            d[v] += __shfl_xor(d[v], 1, 64);
+            if constexpr (PARTS == 4) d[v] += __shfl_xor(d[v], 2, 64);
+          }
+          const int m = r / PARTS;
+          const int n_first = strip * (16 / PARTS) + g * (4 / PARTS);
+          Out* C = reinterpret_cast<Out*>(p.C);
+#pragma unroll
+          for (int v = 0; v < 4 / PARTS; ++v) {
+            Out o = E::apply(d[v], E::bias_term(bias_pre[v], p.beta), p.alpha);
+            if constexpr (E::kAccumulate) o = old_pre[v] + o;
+            if (f == 0 && m < m_real && n_first + v < n_real) C[(size_t)m * n_real + n_first + v] = o;
+          }
+          acc = v4i{0, 0, 0, 0};
+          continue;
+        }
         const int b = strip / strips_per_batch;
         if (GROUPED) {
           GemmParams q = p;  // problem b of the group as a one-batch problem
@@ -2422,6 +2475,38 @@ int launch_kind(const GemmParams& p, void* workspace, long long workspace_bytes,
       if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "gemm launch: %s", hipGetErrorString(e));
       return TI_OK;
     };
+    // Few, long weight rows (fc2 of a decode step: 1x5120x20480, 1x9216x36864): the view of the problem in which
+    // every row is cut into four (two rows of activations: two) parts has that many times the strips, and its rows
+    // lie a part instead of a whole row apart, which spreads the 16 rows of a strip over the memory channels
+    // (a multiple of 4 KiB between them does not): 1x5120x20480 22.4 -> 19.6 us, 1x9216x36864 58.5 -> 52.2 us,
+    // 2x5120x20480 23.9 -> 20.1 us.
+    const int parts = p.batch == 1 && p.out_d == 0 && p.m_base == 0 && p.lda == p.K && p.ldb == p.K && p.N % 16 == 0 &&
+                              p.K >= 8192 && spb <= 4 * cus
+                          ? (p.M == 1 && p.K % 4096 == 0 && p.K % 16384 != 0       ? 4
+                             : p.M == 2 && p.K % 2048 == 0 && p.K % 8192 != 0 ? 2
+                                                                              : 1)
+                          : 1;  // not when the parts are again a multiple of 4 KiB apart (1x4096x16384: 13.5 -> 15.1 us)
+    if (parts > 1) {
+      g_last_kernel = "stream_parts";
+      GemmParams q = p;
+      q.M = p.M * parts;
+      q.N = p.N * parts;
+      q.K = q.lda = q.ldb = p.K / parts;
+      const int view_strips = q.N / 16;
+      auto launch_view = [&](auto kern) -> int {
+        const int lds = 2 * 20 * SBK + S_RED;
+        static std::atomic<unsigned long long> lds_ok{0};
+        if (int rc = allow_lds(kern, lds, lds_ok)) return rc;
+        const long long slots = 3LL * cus;
+        hipLaunchKernelGGL(kern, dim3((unsigned)(view_strips < slots ? view_strips : slots)), dim3(256), lds, stream, q,
+                           view_strips, view_strips, GemmGroup{});
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "gemm launch: %s", hipGetErrorString(e));
+        return TI_OK;
+      };
+      return parts == 4 ? launch_view(gemm_stream_kernel<KIND, 4, 2, false, 4>)
+                        : launch_view(gemm_stream_kernel<KIND, 4, 2, false, 2>);
+    }
     const bool deep = stream_deep_pipeline(p.M, strips, cus);
     if (p.M == 1) return deep ? launch(gemm_stream_kernel<KIND, 1, 3>, 3, 17, 2) : launch(gemm_stream_kernel<KIND, 1, 2>, 2, 17, 3);
     if (p.M <= 4) return launch(gemm_stream_kernel<KIND, 4, 2>, 2, 20, 3);
