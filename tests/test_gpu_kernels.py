@@ -550,28 +550,30 @@ def test_stream_kernel_strip_orders_and_ragged_widths():
         for variant in ("b8_o8", "relu_b8_o8", "bfp32_ofp32", "b32_o32"):
             _say(f"stream {variant} M={M} N={N} K={K}")
             _linear_case(C, variant, M, N, K, seed=91)
-            assert C._lib.ti_last_kernel().decode() == "stream", (M, N, K, C._lib.ti_last_kernel())
+            assert C._lib.ti_last_kernel().decode() == ("gemv" if M == 1 else "stream"), (M, N, K, C._lib.ti_last_kernel())
         _say(f"stream += M={M} N={N} K={K}")
         x, w = _s8(g, M, K), _s8(g, N, K)
         bias, resid = torch.randn(N, generator=g), torch.randn(M, N, generator=g) * 3
         ref = orc.linear_a8_w8_bfp32_ofp32_acc(x, w, bias, 0.003, 1.0, resid)
         out = C._linear_a8_w8_bfp32_ofp32_acc(x.to(DEV), w.to(DEV), bias.to(DEV), 0.003, 1.0, resid.to(DEV))
         assert _ulp_diff(out.cpu(), ref) == 0, (M, N, K)
-        assert C._lib.ti_last_kernel().decode() == "stream"
+        assert C._lib.ti_last_kernel().decode() == ("gemv" if M == 1 else "stream")
 
 
 def test_stream_kernel_on_the_view_with_rows_cut_into_parts():
     # one or two rows of activations against few, long weight rows (fc2 of a decode step): the streaming kernel
     # multiplies the view with every row cut into four (two) parts and its epilogue adds the parts of each output.
-    # Every output kind, widths with a last partial run of strips, the shapes next to the rule's limits.
+    # One row otherwise runs on the flat-reading dot-product kernel.  Every output kind, widths with a last partial
+    # run of strips or of rows, the shapes next to the rules' limits.
     import ctypes
     import torch_int._CUDA as C
     C._lib.ti_last_kernel.restype = ctypes.c_char_p
     g = torch.Generator().manual_seed(92)
-    for (M, N, K, kern) in [(1, 5120, 20480, "stream_parts"), (1, 4096, 8192, "stream_parts"), (1, 9232, 12288, "stream_parts"),
-                            (2, 5120, 20480, "stream_parts"), (2, 4112, 10240, "stream_parts"), (1, 16384, 8192, "stream_parts"),
-                            (1, 5120, 10240, "stream"), (2, 5120, 7168, "stream"), (3, 5120, 20480, "stream"),
-                            (1, 4104, 8192, "stream"), (1, 16400, 8192, "stream"), (1, 4096, 16384, "stream"),
+    for (M, N, K, kern) in [(1, 4096, 28672, "stream_parts"), (1, 9216, 36864, "stream_parts"), (1, 4096, 53248, "stream_parts"),
+                            (2, 5120, 20480, "stream_parts"), (2, 4112, 10240, "stream_parts"), (2, 16384, 10240, "stream_parts"),
+                            (1, 5120, 20480, "gemv"), (1, 4096, 8192, "gemv"), (1, 9232, 12288, "gemv"), (1, 4099, 1024, "gemv"),
+                            (1, 4096, 32768, "gemv"), (1, 4097, 49152, "gemv"), (1, 20481, 2048, "gemv"),
+                            (1, 4104, 53248, "stream"), (2, 5120, 7168, "stream"), (3, 5120, 20480, "stream"),
                             (2, 4096, 8192, "stream")]:
         for variant in VARIANTS:
             _say(f"stream view {variant} M={M} N={N} K={K}")
@@ -883,7 +885,8 @@ def test_grouped_qkv_linear():
     import torch_int._hip_ext as X
     C._lib.ti_last_kernel.restype = ctypes.c_char_p
     g = torch.Generator().manual_seed(29)
-    for (M, N, K, n, family) in [(4, 5120, 5120, 3, "stream_group"), (1, 2048, 1024, 3, "stream_group"),
+    for (M, N, K, n, family) in [(4, 5120, 5120, 3, "stream_group"), (1, 2048, 1024, 3, "gemv_group"),
+                                 (1, 5120, 5120, 3, "gemv_group"), (1, 4098, 2048, 2, "gemv_group"),
                                  (16, 1536, 2048, 4, "stream_group"), (9, 4100, 3072, 2, "stream_group"),
                                  (4, 640, 1024, 3, None), (40, 512, 256, 3, None), (3, 100, 272, 1, None)]:
         _say(f"grouped linear M={M} N={N} K={K} n={n}")

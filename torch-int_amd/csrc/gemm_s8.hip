@@ -339,6 +339,10 @@ int launch_gemm_group_s8(const GemmParams& shape, const GemmGroup& grp, hipStrea
   const bool aligned = ptr_ok && (shape.K % SBK == 0) && shape.K > 0;
   const int spb = (shape.N + 15) / 16;
   const long long strips = (long long)spb * grp.count;
+  if (aligned && gemv_takes(shape) && strips >= 256) {
+    g_last_kernel = "gemv_group";
+    return launch_gemv<KIND, true>(shape, grp, grp.count, stream);
+  }
   if (aligned && shape.M <= 16 && strips >= 256) {
     g_last_kernel = "stream_group";
     const int cus = num_cus();

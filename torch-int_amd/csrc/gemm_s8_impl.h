@@ -2006,6 +2006,80 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(GemmParams p, int stri
   __builtin_amdgcn_s_waitcnt(0x0F70);  // trailing filler copies must land before the LDS is released
 }
 
+// ---------------------------------------------------------------------------
+// One row of activations (a decode step at batch 1) against W[N][K], K % 1024 == 0: dot products on the vector
+// ALUs (v_dot4_i32_i8) instead of the matrix cores, whose 16x16 tiles would be fifteen sixteenths padding here
+// and, worse, force the weights to be read as strips of 16 rows.  A wave owns one weight row at a time and reads it
+// flat: every load instruction fetches 1 KiB of consecutive bytes (64 lanes x 16), non-temporal, eight in flight
+// per wave -- the access shape with which a read-only pass reaches 6.5-6.9 TB/s on this chip, where strips of 16
+// rows reach 5.9-6.7 and less when the rows lie a multiple of 4 KiB apart.  The activation row lives in the LDS;
+// lane l multiplies its 16 weight bytes of a block with bytes 16 l .. 16 l + 15 of the same block of x.  At the end
+// of a row the 64 lanes add up (integer sums: the bits are those of every other kernel) and lane 0 applies the
+// epilogue.  A workgroup is four waves on four consecutive rows; blockIdx.y = problem of a GemmGroup.
+// 1x20480x5120 19.5 -> 18.2 us, 1x5120x5120 8.2 -> 6.4, 1x9216x9216 17.7 -> 16.0, 1x36864x9216 52.6 -> 50.3.
+static constexpr int GEMV_LOADS = 8;
+template <int KIND, bool GROUPED>
+__global__ __launch_bounds__(256) void gemm_gemv_kernel(GemmParams p, GemmGroup grp) {
+  using E = Epi<KIND>;
+  using Out = typename E::Out;
+  using BiasT = typename E::Bias;
+  extern __shared__ __attribute__((aligned(16))) char xs[];  // [K]
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int N = p.N, K = p.K, KB = K >> 10;
+  const int prob = GROUPED ? blockIdx.y : 0;
+  const int n = blockIdx.x * 4 + wave;
+  const int nc = n < N ? n : N - 1;  // a wave past the last row repeats it and stores nothing
+  const int8_t* B = GROUPED ? grp.B[prob] : p.B;
+  const char* row = reinterpret_cast<const char*>(B) + (size_t)nc * p.ldb + lane * 16;
+  // the first weight loads fly while the activation row is staged
+  v4i w[GEMV_LOADS];
+#pragma unroll
+  for (int u = 0; u < GEMV_LOADS; ++u)
+    w[u] = u < KB ? __builtin_nontemporal_load(reinterpret_cast<const v4i*>(row + (size_t)u * 1024)) : v4i{0, 0, 0, 0};
+  // the epilogue's memory operands as well (lane 0 uses them)
+  const BiasT* bias = reinterpret_cast<const BiasT*>(GROUPED ? grp.bias[prob] : p.bias);
+  Out* C = reinterpret_cast<Out*>(GROUPED ? grp.C[prob] : p.C);
+  Out* dst = C + out_index(p, 0, nc);
+  BiasT bv = BiasT(0);
+  if constexpr (E::kHasBias) bv = bias[nc];
+  Out old = Out(0);
+  if constexpr (E::kAccumulate) old = *dst;
+  for (int i = threadIdx.x * 16; i < K; i += 256 * 16)
+    *reinterpret_cast<v4i*>(xs + i) = *reinterpret_cast<const v4i*>(reinterpret_cast<const char*>(p.A) + i);
+  __syncthreads();
+  int acc = 0;
+  for (int b0 = 0; b0 < KB; b0 += GEMV_LOADS) {
+    v4i cur[GEMV_LOADS];
+#pragma unroll
+    for (int u = 0; u < GEMV_LOADS; ++u) cur[u] = w[u];
+    if (b0 + GEMV_LOADS < KB) {
+#pragma unroll
+      for (int u = 0; u < GEMV_LOADS; ++u)
+        w[u] = b0 + GEMV_LOADS + u < KB
+                   ? __builtin_nontemporal_load(reinterpret_cast<const v4i*>(row + (size_t)(b0 + GEMV_LOADS + u) * 1024))
+                   : v4i{0, 0, 0, 0};
+    }
+#pragma unroll
+    for (int u = 0; u < GEMV_LOADS; ++u) {
+      if (b0 + u < KB) {
+        const v4i xv = *reinterpret_cast<const v4i*>(xs + (b0 + u) * 1024 + lane * 16);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc = __builtin_amdgcn_sdot4(cur[u][j], xv[j], acc, false);
+      }
+    }
+  }
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) acc += __shfl_xor(acc, off, 64);
+  if (lane == 0 && n < N) {
+    const float alpha = GROUPED ? grp.alpha[prob] : p.alpha;
+    const float beta = GROUPED ? grp.beta[prob] : p.beta;
+    Out o = E::apply(acc, E::bias_term(bv, beta), alpha);
+    if constexpr (E::kAccumulate) o = old + o;
+    *dst = o;
+  }
+}
+
 // waves per workgroup for the skinny kernel: enough waves to cover HBM latency, at
 // least one 256-byte block of K per wave
 static int skinny_waves(const GemmParams& p) {
@@ -2427,6 +2501,21 @@ static int row_split_rows(long long M, long long N, long long K, long long* rest
   return (int)r;
 }
 
+template <int KIND, bool GROUPED>
+static int launch_gemv(const GemmParams& p, const GemmGroup& grp, int problems, hipStream_t stream) {
+  static std::atomic<unsigned long long> lds_ok{0};
+  if (int rc = allow_lds(gemm_gemv_kernel<KIND, GROUPED>, 48 * 1024, lds_ok)) return rc;
+  hipLaunchKernelGGL((gemm_gemv_kernel<KIND, GROUPED>), dim3((unsigned)((p.N + 3) / 4), (unsigned)problems), dim3(256),
+                     (size_t)p.K, stream, p, grp);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "gemm launch: %s", hipGetErrorString(e));
+  return TI_OK;
+}
+// the shapes the kernel takes: one row, one batch, whole KiB blocks, a row of x that the LDS holds thrice over
+static inline bool gemv_takes(const GemmParams& p) {
+  return p.M == 1 && p.batch == 1 && p.K % 1024 == 0 && p.K <= 48 * 1024 && p.lda == p.K;
+}
+
 // Stages and resident workgroups of the streaming kernel.  One row: three stages of 17 KiB with two workgroups per
 // CU read cold weights 3-6 % faster than two stages with three or four (1x20480x5120 20.1 -> 19.0 us, 1x36864x9216
 // 54.2 -> 52.3 us) -- unless the strips then fall into rounds that leave CUs idle (576 strips on 512 workgroups:
@@ -2486,6 +2575,12 @@ int launch_kind(const GemmParams& p, void* workspace, long long workspace_bytes,
                              : p.M == 2 && p.K % 2048 == 0 && p.K % 8192 != 0 ? 2
                                                                               : 1)
                           : 1;  // not when the parts are again a multiple of 4 KiB apart (1x4096x16384: 13.5 -> 15.1 us)
+    // one row of activations: the flat-reading dot-product kernel, except against the few very long rows where the
+    // view with rows cut into parts is ahead (1x9216x36864: 52.2 against 54.6 us; 1x5120x20480: 19.6 against 18.5)
+    if (gemv_takes(p) && !(parts > 1 && p.K > 24 * 1024)) {
+      g_last_kernel = "gemv";
+      return launch_gemv<KIND, false>(p, GemmGroup{}, 1, stream);
+    }
     if (parts > 1) {
       g_last_kernel = "stream_parts";
       GemmParams q = p;
