@@ -67,8 +67,9 @@ int ti_linear_row_split(int64_t M, int64_t N, int64_t K);
 
 /* Diagnostics: the kernel family the calling thread's last linear / bmm_s8t_s8n_* call launched
  * ("pipe_256x256", "pipe16_256x160", "pipe16_256x288", "pipe16_256x128", "pipe16_128x80", "pipe16_128x192", "pipe16_256x192", "pipe_128x128",
- * "splitk_<tile>" and "fusedk_<tile>" for the two- and one-launch split-K forms, "stream", "skinny", "tile_*",
- * "scalar"; grouped launches add "_group": "stream_group", "pipe16_256x160_group", "pipe16_256x288_group",
+ * "splitk_<tile>" and "fusedk_<tile>" for the two- and one-launch split-K forms, "stream", "stream_parts" (the streaming
+ * kernel on the view with rows cut into parts), "gemv" (one row of activations), "skinny", "tile_*",
+ * "scalar"; grouped launches add "_group": "stream_group", "gemv_group", "pipe16_256x160_group", "pipe16_256x288_group",
  * "pipe16_256x128_group"; "<family>+<family>" when the last rows ran as a second problem, see ti_linear_row_split;
  * "" before the first call).  Benchmarks use it to label their rows. */
 const char* ti_last_kernel(void);
