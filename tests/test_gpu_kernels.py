@@ -863,6 +863,7 @@ def test_head_major_projection_through_every_kernel_family(two_launch_split_k):
                             (8, 512, 22, 128, 128), (8, 512, 22, 128, 192), (2, 512, 16, 128, 64),
                             (2, 512, 40, 128, 5120), (2, 512, 36, 128, 3584), (2, 512, 72, 128, 9216), (1, 384, 90, 32, 4608),
                             (1, 256, 24, 128, 7744), (2, 64, 5, 128, 4096), (1, 256, 25, 128, 11648), (1, 256, 25, 64, 11648), (1, 384, 20, 128, 1024), (1, 128, 6, 128, 4096), (1, 128, 8, 128, 4096), (4, 128, 96, 128, 2048), (2, 512, 96, 128, 1024), (1, 16, 40, 128, 3072), (1, 3, 5, 32, 272),
+                            (1, 1, 40, 128, 5120), (1, 1, 40, 128, 20480), (2, 1, 40, 128, 20480), (1, 4, 40, 128, 2048),  # decode rows
                             (3, 100, 5, 48, 48), (3, 700, 39, 128, 272), (2, 35, 3, 16, 37)]:
         M, N = B * T, H * d
         _say(f"head-major linear bsz={B} seq={T} heads={H} d={d} K={K}")
@@ -874,7 +875,7 @@ def test_head_major_projection_through_every_kernel_family(two_launch_split_k):
         assert torch.equal(out.cpu(), ref), (B, T, H, d, K)
         seen.add(C._lib.ti_last_kernel().decode())
     assert {"pipe16_256x160", "pipe16_256x288", "pipe16_128x80", "pipe16_128x192", "pipe16_256x192", "pipe_256x256", "pipe_128x128", "splitk_256x256", "splitk_256x160",
-            "splitk_256x288", "splitk_128x160", "splitk_128x288", "splitk_128x80", "splitk_128x192", "splitk_128x128", "stream", "skinny", "tile_64x64", "tile_256x256", "scalar"} <= seen, seen
+            "splitk_256x288", "splitk_128x160", "splitk_128x288", "splitk_128x80", "splitk_128x192", "splitk_128x128", "stream", "gemv", "skinny", "tile_64x64", "tile_256x256", "scalar"} <= seen, seen
     with pytest.raises(RuntimeError):
         X.linear_a8_w8_b8_o8_heads(x.to(DEV), w.to(DEV), b.to(DEV), alpha, beta, 2, 35, 6, 8)   # d not a multiple of 16
 
