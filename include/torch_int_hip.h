@@ -385,8 +385,8 @@ int ti_attn_prefill_s8(const int8_t* q, const int8_t* k, const int8_t* vt, const
  * them), then ctx[bh, t, :] = s8(alpha_pv * sum_s p[t, s] * v[s, :]) with p = round(127 * softmax(max(alpha_qk *
  * q.k^T + mask, FLT_MIN_NEG))) -- the same arithmetic, bit for bit, as ti_bmm_s8t_s8n_f32t, ti_attn_softmax_q and
  * ti_bmm_s8t_s8t_s8t chained.  mask is fp32 [BH/heads, 1, T, S] or NULL; probs_out ([BH, T, S] int8) receives the
- * quantised probabilities when not NULL.  Limits: 1 <= T <= 4, D = 64 or 128, and the scores of one (batch, head)
- * must fit the LDS: ti_decode_attn_supported(T, S, D) says whether a shape is accepted. */
+ * quantised probabilities when not NULL.  Limits: 1 <= T <= 4, D a multiple of 16 up to 128 (OPT-2.7B: 80), and the scores of one
+ * (batch, head) must fit the LDS: ti_decode_attn_supported(T, S, D) says whether a shape is accepted. */
 int ti_decode_attn_supported(int64_t T, int64_t S, int64_t D);
 int ti_decode_attn_s8(const int8_t* q, const int8_t* k_new, const int8_t* v_new, int8_t* k_buf, int8_t* v_buf,
                       const float* mask, int8_t* ctx, int8_t* probs_out, int64_t BH, int64_t T, int64_t D, int64_t cap,

@@ -104,7 +104,9 @@ def test_c_abi_rejects_bad_arguments_without_a_device():
     lib.ti_decode_attn_s8.argtypes = [ctypes.c_void_p] * 8 + [i64] * 6 + [ctypes.c_float] * 2 + [ctypes.c_void_p]
     lib.ti_decode_attn_supported.argtypes = [i64] * 3
     assert lib.ti_decode_attn_supported(1, 2048, 128) == 1 and lib.ti_decode_attn_supported(4, 2048, 128) == 1
-    assert lib.ti_decode_attn_supported(5, 16, 128) == 0 and lib.ti_decode_attn_supported(1, 16, 96) == 0
+    assert lib.ti_decode_attn_supported(5, 16, 128) == 0 and lib.ti_decode_attn_supported(1, 16, 96) == 1
+    assert lib.ti_decode_attn_supported(1, 544, 80) == 1 and lib.ti_decode_attn_supported(1, 16, 40) == 0
+    assert lib.ti_decode_attn_supported(1, 16, 144) == 0 and lib.ti_decode_attn_supported(1, 16, 0) == 0
     assert lib.ti_decode_attn_supported(4, 1 << 20, 128) == 0 and lib.ti_decode_attn_supported(1, 0, 128) == 0
     rc = lib.ti_decode_attn_s8(p, p, p, p, p, None, p, None, 4, 5, 128, 64, 32, 2, 1.0, 1.0, None)
     assert rc == 1 and b"unsupported shape" in lib.ti_last_error()

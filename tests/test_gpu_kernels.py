@@ -970,7 +970,10 @@ def test_decode_attention_matches_the_separate_kernels_and_the_oracle():
     # (batch, heads, cap, d, filled, T, masked)
     cases = [(4, 72, 656, 128, 543, 1, True), (1, 40, 2064, 128, 2047, 1, False), (2, 12, 96, 64, 70, 1, True),
              (2, 5, 48, 128, 0, 1, False), (2, 3, 600, 128, 513, 4, True), (1, 2, 80, 64, 61, 3, False),
-             (3, 2, 40, 128, 7, 2, True)]
+             (3, 2, 40, 128, 7, 2, True),
+             # head sizes between the two lane layouts (OPT-2.7B: 80): rows of their own length in memory
+             (2, 32, 560, 80, 543, 1, True), (1, 3, 700, 80, 650, 1, False), (2, 4, 96, 96, 30, 4, True),
+             (1, 5, 64, 48, 17, 2, True), (2, 2, 48, 16, 5, 1, False), (1, 2, 128, 112, 100, 3, True), (1, 3, 80, 32, 0, 1, False)]
     for (B, H, cap, d, S0, T, masked) in cases:
         _say(f"decode_attn B={B} H={H} cap={cap} d={d} filled={S0} T={T} mask={masked}")
         S = S0 + T
@@ -1001,7 +1004,7 @@ def test_decode_attention_matches_the_separate_kernels_and_the_oracle():
         ctx2, none = X.decode_attention(*args, a_qk, a_pv)   # same cache rows again, no probabilities wanted
         assert none is None and torch.equal(ctx2, ctx)
     assert not X.can_decode_attention(args[0], args[1], args[2], kd, vd, cap, None)        # no room
-    assert not X.can_decode_attention(args[0][:, :, :, :32].contiguous(), args[1], args[2], kd, vd, 0, None)
+    assert not X.can_decode_attention(args[0][:, :, :, :16].contiguous(), args[1], args[2], kd, vd, 0, None)   # q narrower than the cache rows
 
 
 def test_fused_qk_softmax_matches_the_two_kernels_and_the_oracle():

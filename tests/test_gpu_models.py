@@ -310,13 +310,13 @@ def test_fp16_model_runs_the_fused_kernels_and_follows_the_torch_chain():
 
 
 @torch.no_grad()
-@pytest.mark.parametrize("half", [False, True])
-def test_graph_decoder_replays_give_the_eager_steps(half):
+@pytest.mark.parametrize("half,hidden,heads", [(False, 256, 4), (True, 256, 4), (False, 320, 4)])   # head sizes 64 and 80
+def test_graph_decoder_replays_give_the_eager_steps(half, hidden, heads):
     # the decoder layers of a decode step recorded once as a HIP graph (cache length read on the device) and
     # replayed for every new token, with the eager embedding / final LayerNorm / lm_head work between the replays:
     # every step's logits and the caches must be those of the eager step, bit for bit
     from torch_int.models.opt import Int8OPTGraphDecoder
-    cfg = OPTConfigLite(hidden_size=256, num_hidden_layers=3, ffn_dim=1024, num_attention_heads=4, vocab_size=512,
+    cfg = OPTConfigLite(hidden_size=hidden, num_hidden_layers=3, ffn_dim=1024, num_attention_heads=heads, vocab_size=512,
                         max_position_embeddings=128)
     torch.manual_seed(0)
     lm = Int8OPTForCausalLM(cfg)

@@ -665,8 +665,8 @@ int ti_decode_attn_s8(const int8_t* q, const int8_t* k_new, const int8_t* v_new,
     return fail(TI_ERR_INVALID_ARG, "%s: S = %lld counts the %lld appended positions", op, (long long)S, (long long)T);
   if (BH == 0) return TI_OK;
   if (!decode_attn_supported(T, S, D))
-    return fail(TI_ERR_INVALID_ARG, "%s: unsupported shape T=%lld S=%lld head_dim=%lld (needs 1 <= T <= 4, head_dim 64 or "
-                "128, S >= 1 and scores that fit the LDS)", op, (long long)T, (long long)S, (long long)D);
+    return fail(TI_ERR_INVALID_ARG, "%s: unsupported shape T=%lld S=%lld head_dim=%lld (needs 1 <= T <= 4, head_dim a multiple of 16 up "
+                "to 128, S >= 1 and scores that fit the LDS)", op, (long long)T, (long long)S, (long long)D);
   if (int rc = check_ptr(op, "q", q, 16, true)) return rc;
   if (int rc = check_ptr(op, "k_new", k_new, 16, k_new != nullptr)) return rc;
   if (int rc = check_ptr(op, "v_new", v_new, 16, v_new != nullptr)) return rc;
@@ -696,8 +696,8 @@ int ti_decode_attn_s8_devlen(const int8_t* q, const int8_t* k_new, const int8_t*
                              (long long)S_max, (long long)T);
   if (BH == 0) return TI_OK;
   if (!decode_attn_supported(T, S_max, D))
-    return fail(TI_ERR_INVALID_ARG, "%s: unsupported shape T=%lld S_max=%lld head_dim=%lld (needs 1 <= T <= 4, head_dim 64 "
-                "or 128 and scores that fit the LDS)", op, (long long)T, (long long)S_max, (long long)D);
+    return fail(TI_ERR_INVALID_ARG, "%s: unsupported shape T=%lld S_max=%lld head_dim=%lld (needs 1 <= T <= 4, head_dim a multiple of 16 "
+                "up to 128 and scores that fit the LDS)", op, (long long)T, (long long)S_max, (long long)D);
   if (int rc = check_ptr(op, "q", q, 16, true)) return rc;
   if (int rc = check_ptr(op, "k_new", k_new, 16, true)) return rc;
   if (int rc = check_ptr(op, "v_new", v_new, 16, true)) return rc;

@@ -47,7 +47,9 @@ __global__ __launch_bounds__(256) void decode_attn_kernel(const int8_t* __restri
                                                           int8_t* v_buf, const float* __restrict__ mask,
                                                           int8_t* __restrict__ ctx, int8_t* __restrict__ probs_out,
                                                           int T, int S_arg, long long cap, int heads, float alpha_qk,
-                                                          float alpha_pv, const int* __restrict__ s_dev) {
+                                                          float alpha_pv, const int* __restrict__ s_dev, int dr) {
+  // dr = the head size in memory, a multiple of 16 up to D (64 or 128, the lanes a cache row is spread over):
+  // rows of q, the caches and ctx are dr bytes long; the lanes beyond a row hold zeros and store nothing
   // s_dev != nullptr: the number of positions is read from device memory (a launch recorded in a HIP graph is
   // replayed for a cache that has grown meanwhile; S_arg is then the largest length the launch was sized for)
   // (clamped to the contract T <= length <= S_arg: the host cannot check a value it never sees, and a length
@@ -68,18 +70,19 @@ __global__ __launch_bounds__(256) void decode_attn_kernel(const int8_t* __restri
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int rs = lane / LPR, cs = lane % LPR;
+  const bool in_row = cs * 16 < dr;
   const long long bh = blockIdx.x;
   const int S_old = k_new != nullptr ? S - T : S;  // rows below come from the cache, the rest from k_new / v_new
-  int8_t* kb = k_buf + bh * cap * D;
-  int8_t* vb = v_buf + bh * cap * D;
-  const int8_t* kn = k_new != nullptr ? k_new + bh * T * D : nullptr;
-  const int8_t* vn = v_new != nullptr ? v_new + bh * T * D : nullptr;
+  int8_t* kb = k_buf + bh * cap * dr;
+  int8_t* vb = v_buf + bh * cap * dr;
+  const int8_t* kn = k_new != nullptr ? k_new + bh * T * dr : nullptr;
+  const int8_t* vn = v_new != nullptr ? v_new + bh * T * dr : nullptr;
 
   // ---- phase 1: scores[t][s] = alpha_qk * (q[t] . k[s]); new key rows go into the cache on the way
   v4i qr[TQ];
 #pragma unroll
   for (int t = 0; t < TQ; ++t)
-    qr[t] = t < T ? *reinterpret_cast<const v4i*>(q + (bh * T + t) * D + cs * 16) : v4i{0, 0, 0, 0};
+    qr[t] = t < T && in_row ? *reinterpret_cast<const v4i*>(q + (bh * T + t) * dr + cs * 16) : v4i{0, 0, 0, 0};
   constexpr int U = NI > 0 ? NI : 4;  // row groups in flight per wave
   // Rows past the end re-read the last row (their products are never used), so the loads need no branches;
   // rows that come from k_new / v_new are also written into the cache.
@@ -88,14 +91,14 @@ __global__ __launch_bounds__(256) void decode_attn_kernel(const int8_t* __restri
     for (int u = 0; u < U; ++u) {
       int s = base + u * 4 * RPW + rs;
       s = s < S ? s : S - 1;
-      const int8_t* src = s < S_old ? buf + (long long)s * D : fresh + (long long)(s - S_old) * D;
-      dst[u] = *reinterpret_cast<const v4i*>(src + cs * 16);
+      const int8_t* src = s < S_old ? buf + (long long)s * dr : fresh + (long long)(s - S_old) * dr;
+      dst[u] = in_row ? *reinterpret_cast<const v4i*>(src + cs * 16) : v4i{0, 0, 0, 0};
     }
     if (S_old < S) {
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int s = base + u * 4 * RPW + rs;
-        if (s >= S_old && s < S) *reinterpret_cast<v4i*>(buf + (long long)s * D + cs * 16) = dst[u];
+        if (s >= S_old && s < S && in_row) *reinterpret_cast<v4i*>(buf + (long long)s * dr + cs * 16) = dst[u];
       }
     }
   };
@@ -243,13 +246,19 @@ __global__ __launch_bounds__(256) void decode_attn_kernel(const int8_t* __restri
   }
   __syncthreads();
   for (int idx = tid; idx < T * D; idx += 256) {
-    const int sum = red[idx] + red[T * D + idx] + red[2 * T * D + idx] + red[3 * T * D + idx];
-    ctx[bh * T * D + idx] = Epi<EPI_S8_SCALE>::apply(sum, 0.0f, alpha_pv);
+    const int t = idx / D, c = idx - t * D;
+    if (c < dr) {
+      const int sum = red[idx] + red[T * D + idx] + red[2 * T * D + idx] + red[3 * T * D + idx];
+      ctx[(bh * T + t) * dr + c] = Epi<EPI_S8_SCALE>::apply(sum, 0.0f, alpha_pv);
+    }
   }
 }
 
+// D = the head size in memory: any multiple of 16 up to 128 (sizes up to 64 run on four lanes per cache row, the
+// others on eight)
 bool decode_attn_supported(long long T, long long S, long long D) {
-  return T >= 1 && T <= DA_MAX_T && S >= 1 && (D == 64 || D == 128) && decode_attn_lds(T, S, D) <= DA_LDS_LIMIT;
+  return T >= 1 && T <= DA_MAX_T && S >= 1 && D >= 16 && D <= 128 && D % 16 == 0 &&
+         decode_attn_lds(T, S, D <= 64 ? 64 : 128) <= DA_LDS_LIMIT;
 }
 
 int launch_decode_attn_s8(const int8_t* q, const int8_t* k_new, const int8_t* v_new, int8_t* k_buf, int8_t* v_buf,
@@ -263,14 +272,15 @@ int launch_decode_attn_s8(const int8_t* q, const int8_t* k_new, const int8_t* v_
     return fail(TI_ERR_INVALID_ARG, "decode_attn: unsupported shape (T=%lld S=%lld head_dim=%lld)", T, S, D);
   if (BH > 0x7fffffffLL) return fail(TI_ERR_INVALID_ARG, "decode_attn: too many (batch, head) pairs (%lld)", BH);
   const dim3 grid((unsigned)BH), block(256);
-  const size_t lds = (size_t)decode_attn_lds(T, S, D);
+  const int lanes_d = D <= 64 ? 64 : 128;  // the kernel variant: bytes of a cache row that its lanes cover
+  const size_t lds = (size_t)decode_attn_lds(T, S, lanes_d);
   // caches of at most 20 row groups per lane (640 positions at head size 128) with one or two query rows take
   // the variant that issues all loads up front
 #define TI_DA(TQ, DD, NI)                                                                                              \
   hipLaunchKernelGGL((decode_attn_kernel<TQ, DD, NI>), grid, block, lds, stream, q, k_new, v_new, k_buf, v_buf, mask, \
-                     ctx, probs_out, (int)T, (int)S, cap, (int)heads, alpha_qk, alpha_pv, s_dev)
-  const bool resident = T <= 2 && S <= 20 * 4 * (64 / (D / 16));
-  if (D == 128) {
+                     ctx, probs_out, (int)T, (int)S, cap, (int)heads, alpha_qk, alpha_pv, s_dev, (int)D)
+  const bool resident = T <= 2 && S <= 20 * 4 * (64 / (lanes_d / 16));
+  if (lanes_d == 128) {
     if (T == 1) { if (resident) TI_DA(1, 128, 20); else TI_DA(1, 128, 0); }
     else if (T == 2) { if (resident) TI_DA(2, 128, 20); else TI_DA(2, 128, 0); }
     else TI_DA(4, 128, 0);

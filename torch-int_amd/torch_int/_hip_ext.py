@@ -469,7 +469,7 @@ def decode_attention_shape_ok(T, S, d):
 
 
 def can_decode_attention(q, k_new, v_new, k_buf, v_buf, filled, mask):
-    """int8 HIP tensors on one device: q / k_new / v_new [B, H, T, d] contiguous with 1 <= T <= 4 and d 64 or 128,
+    """int8 HIP tensors on one device: q / k_new / v_new [B, H, T, d] contiguous with 1 <= T <= 4 and d a multiple of 16 up to 128,
     cache buffers [B, H, cap, d] contiguous holding ``filled`` positions with room for T more; mask None or fp32
     [B, 1, T, filled + T] contiguous; and scores that fit the LDS."""
     if not (_ok(q, torch.int8) and q.dim() == 4 and can_kv_append(k_new, v_new, k_buf, v_buf)
@@ -492,7 +492,7 @@ def decode_attention(q, k_new, v_new, k_buf, v_buf, filled, mask, alpha_qk, alph
     Q.K^T, softmax and P.V kernels return."""
     if not checked and not can_decode_attention(q, k_new, v_new, k_buf, v_buf, filled, mask):
         raise RuntimeError("torch_int._hip_ext.decode_attention: needs contiguous int8 HIP q/k_new/v_new [B,H,T,d] "
-                           "(T <= 4, d 64 or 128), cache buffers [B,H,cap,d] with room, and an fp32 mask [B,1,T,S] or None")
+                           "(T <= 4, d a multiple of 16 up to 128), cache buffers [B,H,cap,d] with room, and an fp32 mask [B,1,T,S] or None")
     B, H, T, d = q.shape
     S = filled + T
     dev = q.device
@@ -523,7 +523,7 @@ def decode_attention_devlen(q, k_new, v_new, k_buf, v_buf, length, max_length, a
     if not (can_decode_attention(q, k_new, v_new, k_buf, v_buf, max_length - q.shape[2], None)
             and _ok(length, torch.int32) and length.numel() == 1 and length.device == q.device):
         raise RuntimeError("torch_int._hip_ext.decode_attention_devlen: needs contiguous int8 HIP q/k_new/v_new "
-                           "[B,H,T,d] (T <= 4, d 64 or 128), cache buffers [B,H,cap,d] with cap >= max_length, and an "
+                           "[B,H,T,d] (T <= 4, d a multiple of 16 up to 128), cache buffers [B,H,cap,d] with cap >= max_length, and an "
                            "int32 HIP tensor holding the length")
     B, H, T, d = q.shape
     dev = q.device
