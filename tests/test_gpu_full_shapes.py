@@ -203,6 +203,64 @@ def test_linear_random_shapes_every_epilogue(seed):
     assert len(seen) >= 15, seen   # the sweep does reach most of the dispatcher
 
 
+@pytest.mark.parametrize("seed", [7, 8])
+def test_decode_linear_random_shapes_every_epilogue(seed):
+    """250 seeded random decode shapes per seed: 1 to 16 rows of activations against weight matrices of the OPT and
+    GPT-3 widths, inner dimensions that 1024 divides (the dot-product kernel, the streaming kernel with its stage /
+    workgroup choices, the view with rows cut into parts) and a few that it does not (the skinny kernel); the six
+    linear epilogues and the grouped q/k/v call, every output element against the device-side exact references."""
+    import random
+    import torch_int._CUDA as C
+    import torch_int._hip_ext as X
+    C._lib.ti_last_kernel.restype = ctypes.c_char_p
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    rnd = random.Random(seed)
+    widths = [4096, 4100, 5120, 9216, 12288, 16384, 20480, 4112, 8200, 2048, 50272, 7168, 27648, 4099, 36864]
+    inner = [1024, 2048, 3072, 4096, 5120, 7168, 8192, 9216, 10240, 12288, 16384, 20480, 28672, 36864, 49152, 53248,
+             2560, 768]
+
+    def s8(*shape):
+        return torch.randint(-127, 128, shape, dtype=torch.int8, device=DEV, generator=g)
+
+    def epi8(acc, bias, al, be):
+        t = _fma32_on_device(al, acc.float(), (torch.tensor(be, dtype=torch.float32, device=DEV) * bias.float()).expand_as(acc))
+        return t
+    seen = set()
+    for it in range(250):
+        M, N, K = rnd.choice([1, 1, 1, 2, 2, 3, 4, 5, 8, 13, 16]), rnd.choice(widths), rnd.choice(inner)
+        if N * K > 900e6:
+            continue
+        _say(f"random decode linear {it}: M={M} N={N} K={K}")
+        x, w, b8 = s8(M, K), s8(N, K), s8(N)
+        bf = torch.randn(N, device=DEV, generator=g)
+        b32 = torch.randint(-65535, 65535, (N,), dtype=torch.int32, device=DEV, generator=g)
+        al, be = rnd.uniform(1e-4, 1e-2), rnd.uniform(1e-4, 1e-2)
+        acc = _acc_on_device(x, w)
+        t8 = epi8(acc, b8, al, be)
+        tf = _fma32_on_device(al, acc.float(), bf.expand_as(acc))
+        ts = epi8(acc, b32, al, be)
+        assert torch.equal(C.linear_a8_w8_b32_o32(x, w, b32), (acc + b32.long()).to(torch.int32)), (M, N, K)
+        family = C._lib.ti_last_kernel().decode()
+        seen.add(family)
+        assert torch.equal(C.linear_a8_w8_b8_o8(x, w, b8, al, be), t8.round().clamp(-128, 127).to(torch.int8)), (M, N, K, family)
+        assert torch.equal(C.linear_relu_a8_w8_b8_o8(x, w, b8, al, be), t8.round().clamp(0, 127).to(torch.int8)), (M, N, K)
+        assert torch.equal(C.linear_a8_w8_bfp32_ofp32(x, w, bf, al, 1.0), tf), (M, N, K, family)
+        inout = torch.randn(M, N, device=DEV, generator=g)
+        want = inout + tf
+        C._linear_a8_w8_bfp32_ofp32_acc(x, w, bf, al, 1.0, inout)
+        assert torch.equal(inout, want), (M, N, K, family)
+        scaled = ts.round().clamp(-2.0 ** 31, 2.0 ** 31 - 1).to(torch.int64).clamp(-2 ** 31, 2 ** 31 - 1).to(torch.int32)
+        assert torch.equal(C.linear_a8_w8_b32_o32_with_scaling(x, w, b32, al, be), scaled), (M, N, K)
+        ws, bs = [w, s8(N, K), s8(N, K)], [b8, s8(N), s8(N)]
+        als, bes = [al, al * 0.7, al * 1.3], [be, be * 0.5, be * 2]
+        outs = X.linear_a8_w8_b8_o8_group(x, ws, bs, als, bes)
+        seen.add(C._lib.ti_last_kernel().decode())
+        for wi, bi, ai, bei, o in zip(ws, bs, als, bes, outs):
+            ti = epi8(_acc_on_device(x, wi), bi, ai, bei)
+            assert torch.equal(o, ti.round().clamp(-128, 127).to(torch.int8)), (M, N, K, "group")
+    assert {"gemv", "gemv_group", "stream", "stream_group", "stream_parts", "skinny"} <= seen, seen
+
+
 @pytest.mark.parametrize("M,N,K", [(2112, 5120, 20480), (2176, 5120, 5120), (2050, 5120, 5120), (2064, 5120, 5120),
                                    (4160, 4096, 8192), (2112, 5120, 5120), (1600, 5120, 5120)])
 def test_linear_with_rows_beyond_a_multiple_of_256(M, N, K):
