@@ -370,8 +370,8 @@ int ti_kv_append_s8(const int8_t* k_new, const int8_t* v_new, int8_t* k_buf, int
  * ti_bmm_s8t_s8n_f32t, ti_attn_softmax_q, ti_bmm_s8t_s8n_s8t and the head merge `transpose(1,2).reshape(...)`,
  * same bits, without the score and probability tensors.  vt is V transposed, [BH, D, S] packed (what
  * ti_transpose_last2_s8 makes, as upstream's `value_states.transpose(1,2).contiguous()`); ctx is [BH/heads, T,
- * heads*D] packed.  Limits (ti_attn_prefill_supported): S a multiple of 16 in [16, 4096] and D = 64 or 128; or S a
- * multiple of 64 up to 512 and D any multiple of 16 up to 128 (OPT-2.7B: 80).  Up to 512 keys (a multiple of 64) all keys
+ * heads*D] packed.  Limits (ti_attn_prefill_supported): S a multiple of 16 in [16, 4096] and D a multiple of 16 up to
+ * 128 (OPT-2.7B: 80; rows keep their own length in memory).  Up to 512 keys (a multiple of 64) all keys
  * of a head sit in the LDS and are swept once; other shapes sweep the keys three times in tiles of 256 (row maximum, row
  * sum, probabilities): the same bits either way. */
 int ti_attn_prefill_supported(int64_t T, int64_t S, int64_t D);
@@ -405,7 +405,7 @@ int ti_decode_attn_s8_devlen(const int8_t* q, const int8_t* k_new, const int8_t*
  * in one launch: ti_bmm_s8t_s8n_f32t followed by ti_attn_softmax_q (torch_int/models/opt.py:137-178) without the
  * fp32 score tensor in between; the same bits.  q is [BH, T, D] with stride_q elements between batches, k is
  * [BH, S, D] with stride_k, rows packed; mask fp32 [BH/heads, 1, T, S] or NULL; probs [BH, T, S] packed.
- * Limits: S a multiple of 16 in [16, 4096] and D = 64 or 128, or S up to 512 and D any multiple of 16 up to 128:
+ * Limits: S a multiple of 16 in [16, 4096] and D a multiple of 16 up to 128:
  * ti_attn_qk_softmax_q_supported(T, S, D) says whether a shape is accepted. */
 int ti_attn_qk_softmax_q_supported(int64_t T, int64_t S, int64_t D);
 int ti_attn_qk_softmax_q(const int8_t* q, const int8_t* k, const float* mask, int8_t* probs, int64_t BH, int64_t T,

@@ -126,13 +126,14 @@ def test_c_abi_rejects_bad_arguments_without_a_device():
     assert lib.ti_attn_qk_softmax_q_supported(512, 528, 128) == 1 and lib.ti_attn_qk_softmax_q_supported(512, 40, 128) == 0
     assert lib.ti_attn_qk_softmax_q_supported(512, 512, 64) == 1 and lib.ti_attn_qk_softmax_q_supported(2048, 4096, 64) == 1
     assert lib.ti_attn_qk_softmax_q_supported(512, 4112, 128) == 0 and lib.ti_attn_qk_softmax_q_supported(512, 512, 96) == 1
-    # other head sizes (multiples of 16 up to 128) only where all keys of a head are swept once: up to 512 of them
-    assert lib.ti_attn_qk_softmax_q_supported(512, 528, 96) == 0 and lib.ti_attn_qk_softmax_q_supported(512, 512, 144) == 0
+    # every head size that is a multiple of 16 up to 128, in the single-sweep and the three-sweep kernel alike
+    assert lib.ti_attn_qk_softmax_q_supported(512, 528, 96) == 1 and lib.ti_attn_qk_softmax_q_supported(512, 512, 144) == 0
     assert lib.ti_attn_qk_softmax_q_supported(512, 512, 72) == 0 and lib.ti_attn_qk_softmax_q_supported(64, 48, 16) == 1
     lib.ti_attn_prefill_supported.argtypes = [i64] * 3
     assert lib.ti_attn_prefill_supported(512, 512, 80) == 1 and lib.ti_attn_prefill_supported(512, 448, 80) == 1
-    assert lib.ti_attn_prefill_supported(512, 400, 80) == 0 and lib.ti_attn_prefill_supported(512, 400, 64) == 1
-    assert lib.ti_attn_prefill_supported(512, 1024, 80) == 0 and lib.ti_attn_prefill_supported(512, 1024, 128) == 1
+    assert lib.ti_attn_prefill_supported(512, 400, 80) == 1 and lib.ti_attn_prefill_supported(512, 400, 64) == 1
+    assert lib.ti_attn_prefill_supported(512, 1024, 80) == 1 and lib.ti_attn_prefill_supported(512, 1024, 128) == 1
+    assert lib.ti_attn_prefill_supported(512, 4112, 80) == 0 and lib.ti_attn_prefill_supported(512, 1024, 8) == 0
     rc = lib.ti_attn_qk_softmax_q(p, p, None, p, 4, 64, 520, 128, 64 * 128, 520 * 128, 2, 1.0, None)
     assert rc == 1 and b"unsupported shape" in lib.ti_last_error()
     rc = lib.ti_attn_qk_softmax_q(p, p, None, p, 4, 64, 64, 128, 64 * 128, 63 * 128, 2, 1.0, None)
@@ -143,8 +144,8 @@ def test_c_abi_rejects_bad_arguments_without_a_device():
     lib.ti_attn_prefill_s8.argtypes = [ctypes.c_void_p] * 5 + [i64] * 7 + [ctypes.c_float] * 2 + [ctypes.c_void_p]
     rc = lib.ti_attn_prefill_s8(p, p, p, None, p, 4, 64, 72, 128, 64 * 128, 72 * 128, 2, 1.0, 1.0, None)
     assert rc == 1 and b"multiple of 16" in lib.ti_last_error()
-    rc = lib.ti_attn_prefill_s8(p, p, p, None, p, 4, 64, 80, 80, 64 * 80, 80 * 80, 2, 1.0, 1.0, None)
-    assert rc == 1 and b"unsupported shape" in lib.ti_last_error()   # head size 80 with a key count 64 does not divide
+    rc = lib.ti_attn_prefill_s8(p, p, p, None, p, 4, 64, 80, 72, 64 * 72, 80 * 72, 2, 1.0, 1.0, None)
+    assert rc == 1 and b"unsupported shape" in lib.ti_last_error()   # head size 72 is not a multiple of 16
     rc = lib.ti_attn_prefill_s8(p, p, None, None, p, 4, 64, 64, 128, 64 * 128, 64 * 128, 2, 1.0, 1.0, None)
     assert rc == 1 and b"vt is NULL" in lib.ti_last_error()
     assert lib.ti_attn_prefill_s8(None, None, None, None, None, 0, 64, 64, 128, 0, 0, 2, 1.0, 1.0, None) == 0

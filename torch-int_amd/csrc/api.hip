@@ -598,7 +598,7 @@ int ti_attn_qk_softmax_q_mc(const int8_t* q, const int8_t* k, const float* mask,
   if (BH == 0 || T == 0) return TI_OK;
   if (!attn_qk_softmax_q_supported(T, S, D))
     return fail(TI_ERR_INVALID_ARG, "%s: unsupported shape T=%lld S=%lld head_dim=%lld (needs S a multiple of 16 in "
-                "[16, 4096] and head_dim 64 or 128, or any multiple of 16 up to 128 with at most 512 keys)", op,
+                "[16, 4096] and head_dim a multiple of 16 up to 128)", op,
                 (long long)T, (long long)S, (long long)D);
   if (stride_q < T * D || stride_k < S * D || stride_q % 16 != 0 || stride_k % 16 != 0)
     return fail(TI_ERR_INVALID_ARG, "%s: batch strides (%lld, %lld) must be multiples of 16 and cover one matrix", op,
@@ -631,7 +631,7 @@ int ti_attn_prefill_s8_mc(const int8_t* q, const int8_t* k, const int8_t* vt, co
   if (BH == 0 || T == 0) return TI_OK;
   if (!attn_prefill_supported(T, S, D))
     return fail(TI_ERR_INVALID_ARG, "%s: unsupported shape T=%lld S=%lld head_dim=%lld (needs S a multiple of 16 in "
-                "[16, 4096] and head_dim 64 or 128, or any multiple of 16 up to 128 with at most 512 keys, a multiple of 64)",
+                "[16, 4096] and head_dim a multiple of 16 up to 128)",
                 op, (long long)T, (long long)S, (long long)D);
   if (stride_q < T * D || stride_k < S * D || stride_q % 16 != 0 || stride_k % 16 != 0)
     return fail(TI_ERR_INVALID_ARG, "%s: batch strides (%lld, %lld) must be multiples of 16 and cover one matrix", op,

@@ -75,7 +75,10 @@ __global__ __launch_bounds__(256, 2) void attn_long_kernel(const int8_t* __restr
                                                            int T, int S, long long stride_q, long long stride_k,
                                                            int heads, int row_blocks, float alpha,
                                                            const int8_t* __restrict__ vt, int8_t* __restrict__ ctx,
-                                                           float alpha_pv, const unsigned char* __restrict__ cls) {
+                                                           float alpha_pv, const unsigned char* __restrict__ cls, int dr) {
+  // dr = the head size in memory, a multiple of 16 up to D (the LDS row size, 64 or 128): rows of q, k and the
+  // context are dr bytes long, V^T has dr rows; the chunks of an LDS row beyond dr hold zeros, which add nothing to
+  // the integer products, and the context blocks beyond dr are computed on whatever the LDS holds and not stored.
   constexpr int CH = D / 16;       // 16-byte chunks per row
   constexpr int KS = D / 64;       // MFMAs (64 bytes of head dimension each) per block
   constexpr int RPI = 1024 / D;    // panel rows one copy instruction fills
@@ -101,31 +104,39 @@ __global__ __launch_bounds__(256, 2) void attn_long_kernel(const int8_t* __restr
   for (int i = wave; i < AL_ROWS / RPI; i += 4) {
     const int row = i * RPI + lane / CH, pos = lane % CH;
     const int t = t0 + row < T ? t0 + row : T - 1;  // rows past the end repeat the last one; never stored
-    __builtin_amdgcn_global_load_lds((const TI_GLOBAL_AS void*)(qb + (long long)t * D + (al_swz<D>(row, pos) << 4)),
-                                     (TI_LDS_AS void*)((TI_LDS_AS char*)qs_base + i * 1024), 16, 0, 0);
+    const int chunk = al_swz<D>(row, pos);
+    if (chunk * 16 < dr)
+      __builtin_amdgcn_global_load_lds((const TI_GLOBAL_AS void*)(qb + (long long)t * dr + (chunk << 4)),
+                                       (TI_LDS_AS void*)((TI_LDS_AS char*)qs_base + i * 1024), 16, 0, 0);
+    else
+      *reinterpret_cast<v4i*>(qs_base + i * 1024 + lane * 16) = v4i{0, 0, 0, 0};
   }
   auto load_k_tile = [&](int tile) {
     const int k0 = tile * AL_TILE;
     const int nkeys = S - k0 < AL_TILE ? S - k0 : AL_TILE;  // a multiple of 16
     for (int i = wave; i < nkeys / RPI; i += 4) {
       const int row = i * RPI + lane / CH, pos = lane % CH;
-      __builtin_amdgcn_global_load_lds(
-          (const TI_GLOBAL_AS void*)(kb + (long long)(k0 + row) * D + (al_swz<D>(row, pos) << 4)),
-          (TI_LDS_AS void*)((TI_LDS_AS char*)ks_base + i * 1024), 16, 0, 0);
+      const int chunk = al_swz<D>(row, pos);
+      if (chunk * 16 < dr)
+        __builtin_amdgcn_global_load_lds((const TI_GLOBAL_AS void*)(kb + (long long)(k0 + row) * dr + (chunk << 4)),
+                                         (TI_LDS_AS void*)((TI_LDS_AS char*)ks_base + i * 1024), 16, 0, 0);
+      else
+        *reinterpret_cast<v4i*>(ks_base + i * 1024 + lane * 16) = v4i{0, 0, 0, 0};
     }
   };
   auto load_v_tile = [&](int tile) {
     if constexpr (PV) {
       const int k0 = tile * AL_TILE;
       const int nkeys = S - k0 < AL_TILE ? S - k0 : AL_TILE;
-      const int8_t* vb = vt + bh * (long long)D * S + k0;
+      const int8_t* vb = vt + bh * (long long)dr * S + k0;
       for (int i = wave; i < (D * AL_VPITCH) / 1024; i += 4) {
         const int o = i * 1024 + lane * 16;
         const int row = o / AL_VPITCH;
         int col = o - row * AL_VPITCH;
         col = col < nkeys ? col : 0;  // pad bytes and columns past the last key get a copy of chunk 0: multiplied by p = 0
-        __builtin_amdgcn_global_load_lds((const TI_GLOBAL_AS void*)(vb + (long long)row * S + col),
-                                         (TI_LDS_AS void*)((TI_LDS_AS char*)vs_base + i * 1024), 16, 0, 0);
+        if (row < dr)  // rows of V^T beyond the head size stay as they are: their context blocks are not stored
+          __builtin_amdgcn_global_load_lds((const TI_GLOBAL_AS void*)(vb + (long long)row * S + col),
+                                           (TI_LDS_AS void*)((TI_LDS_AS char*)vs_base + i * 1024), 16, 0, 0);
       }
     }
   };
@@ -380,34 +391,35 @@ __global__ __launch_bounds__(256, 2) void attn_long_kernel(const int8_t* __restr
   if constexpr (PV) {
     if (t < T) {
       const long long b = bh / heads, h = bh - b * heads;
-      int* crow = reinterpret_cast<int*>(ctx + ((b * T + t) * heads + h) * (long long)D) + g;
+      int* crow = reinterpret_cast<int*>(ctx + ((b * T + t) * heads + h) * (long long)dr) + g;
 #pragma unroll
       for (int c = 0; c < CH; ++c) {
         unsigned w = 0;
 #pragma unroll
         for (int v = 0; v < 4; ++v)
           w |= (unsigned)(unsigned char)Epi<EPI_S8_SCALE>::apply(o[c][v], 0.0f, alpha_pv) << (8 * v);
-        crow[4 * c] = (int)w;
+        if (16 * c < dr) crow[4 * c] = (int)w;
       }
     }
   }
 }
 
+// D = the head size in memory: any multiple of 16 up to 128 (LDS rows of 64 bytes up to 64, of 128 beyond)
 bool attn_long_supported(long long T, long long S, long long D) {
-  return T >= 1 && (D == 64 || D == 128) && S >= 16 && S % 16 == 0 && S <= (long long)AL_TILE * AL_MAX_TILES;
+  return T >= 1 && D >= 16 && D <= 128 && D % 16 == 0 && S >= 16 && S % 16 == 0 && S <= (long long)AL_TILE * AL_MAX_TILES;
 }
 
 template <int D, bool PV, bool MASKED>
 static int launch_al(dim3 grid, hipStream_t stream, const int8_t* q, const int8_t* k, const float* mask, int8_t* probs,
                      int T, int S, long long stride_q, long long stride_k, int heads, int row_blocks, float alpha,
-                     const int8_t* vt, int8_t* ctx, float alpha_pv, const unsigned char* cls) {
+                     const int8_t* vt, int8_t* ctx, float alpha_pv, const unsigned char* cls, int dr) {
   auto kern = attn_long_kernel<D, PV, MASKED>;
   constexpr int lds = AL_ROWS * D + AL_TILE * D + (PV ? D * AL_VPITCH : 0) + 16;
   static_assert(2 * lds <= 160 * 1024, "two workgroups per CU");
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
   if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "attn_long: LDS limit: %s", hipGetErrorString(e));
   hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, q, k, mask, probs, T, S, stride_q, stride_k, heads, row_blocks,
-                     alpha, vt, ctx, alpha_pv, cls);
+                     alpha, vt, ctx, alpha_pv, cls, dr);
   e = hipGetLastError();
   if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "attn_long launch: %s", hipGetErrorString(e));
   return TI_OK;
@@ -429,10 +441,10 @@ int launch_attn_long(const int8_t* q, const int8_t* k, const float* mask, int8_t
 #define TI_AL(DD, PV)                                                                                                 \
   return mask != nullptr                                                                                              \
              ? launch_al<DD, PV, true>(grid, stream, q, k, mask, probs, (int)T, (int)S, stride_q, stride_k, (int)heads,  \
-                                       (int)row_blocks, alpha, vt, ctx, alpha_pv, cls)                                \
+                                       (int)row_blocks, alpha, vt, ctx, alpha_pv, cls, (int)D)                       \
              : launch_al<DD, PV, false>(grid, stream, q, k, mask, probs, (int)T, (int)S, stride_q, stride_k, (int)heads, \
-                                        (int)row_blocks, alpha, vt, ctx, alpha_pv, nullptr)
-  if (D == 128) {
+                                        (int)row_blocks, alpha, vt, ctx, alpha_pv, nullptr, (int)D)
+  if (D > 64) {
     if (vt == nullptr) TI_AL(128, false);
     TI_AL(128, true);
   }

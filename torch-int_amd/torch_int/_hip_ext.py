@@ -359,7 +359,7 @@ def kv_append(k_new, v_new, k_buf, v_buf, filled, checked=False):
 
 def can_attn_qk_softmax_q(q, k, mask, bsz, heads):
     """int8 HIP q [bsz*heads, T, d] contiguous and k [bsz*heads, S, d] with packed rows (any batch stride that is
-    a multiple of 16), d 64 or 128 and S a multiple of 16 up to 4096, or d any multiple of 16 up to 128 and S up to 512;
+    a multiple of 16), d a multiple of 16 up to 128 and S a multiple of 16 up to 4096;
     mask None or fp32 [bsz, 1, T, S] contiguous."""
     if not (_ok(q, torch.int8) and type(k) is torch.Tensor and k.dtype is torch.int8 and k.is_cuda and q.dim() == 3
             and k.dim() == 3 and q.shape[0] == k.shape[0] == bsz * heads and q.shape[2] == k.shape[2]
@@ -414,7 +414,7 @@ def attn_qk_softmax_q(q, k, mask, alpha, heads, checked=False):
     """int8 round(127 softmax(alpha q k^T + mask)) [bsz*heads, T, S] in one launch: the values of
     ``attn_softmax_q(bmm_s8t_s8n_f32t(q, k, alpha), mask, heads)`` without the fp32 scores in memory."""
     if not checked and not can_attn_qk_softmax_q(q, k, mask, q.shape[0] // heads, heads):
-        raise RuntimeError("torch_int._hip_ext.attn_qk_softmax_q: needs int8 HIP q [B*H,T,d] / k [B*H,S,d] (d 64 or 128, "
+        raise RuntimeError("torch_int._hip_ext.attn_qk_softmax_q: needs int8 HIP q [B*H,T,d] / k [B*H,S,d] (d a multiple of 16 up to 128, "
                            "S a multiple of 16 up to 4096) and an fp32 mask [B,1,T,S] or None")
     BH, T, d = q.shape
     S = k.shape[1]
@@ -448,7 +448,7 @@ def attn_prefill(q, k, vt, mask, alpha_qk, alpha_pv, heads, checked=False):
     score and probability tensors."""
     if not checked and not can_attn_prefill(q, k, vt, mask, q.shape[0] // heads, heads):
         raise RuntimeError("torch_int._hip_ext.attn_prefill: needs int8 HIP q [B*H,T,d], k [B*H,S,d], vt [B*H,d,S] "
-                           "(d 64 or 128, S a multiple of 16 up to 4096) and an fp32 mask [B,1,T,S] or None")
+                           "(d a multiple of 16 up to 128, S a multiple of 16 up to 4096) and an fp32 mask [B,1,T,S] or None")
     BH, T, d = q.shape
     S = k.shape[1]
     dev = q.device

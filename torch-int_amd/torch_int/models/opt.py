@@ -208,25 +208,6 @@ class Int8OPTAttention(nn.Module):
         ctx = _hip_ext.merge_heads(ctx, bsz, H, T, d)
         return self.out_proj(ctx), probs_out, present
 
-    def _prefill_padded_heads(self, query, key, value, attention_mask, bsz, tgt_len):
-        """The one-launch prefill attention for a head size the kernel has no form of (OPT-2.7B: 80): q, k and V^T
-        are padded with zeros to the next size it has (64 or 128).  The added dimensions contribute zero to every
-        q.k product and give context columns that are exactly zero and are cut off again, so the int8 result is the
-        one of the unpadded operator chain; three small copies instead of the fp32 score tensor.  None when the
-        shapes or tensors do not qualify."""
-        H, d = self.num_heads, self.head_dim
-        dp = 64 if d < 64 else 128
-        pad = nn.functional.pad
-        qp, kp = pad(query, (0, dp - d)), pad(key, (0, dp - d))
-        if not _hip_ext.can_attn_qk_softmax_q(qp, kp, attention_mask, bsz, H):
-            return None
-        vt = pad(_hip_ext.transpose_last2(value.contiguous()), (0, 0, 0, dp - d))   # [bsz*H, dp, src]
-        if not _hip_ext.can_attn_prefill(qp, kp, vt, attention_mask, bsz, H):
-            return None
-        ctx = _hip_ext.attn_prefill(qp, kp, vt, attention_mask, self.qk_bmm._scalar("a"), self.pv_bmm._scalar("a"), H,
-                                    checked=True)                                      # [bsz, tgt, H * dp]
-        return ctx.view(bsz, tgt_len, H, dp)[..., :d].reshape(bsz, tgt_len, H * d)
-
     def decode_step_devlen(self, hidden_states, k_buf, v_buf, length, max_length):
         """Self-attention of one new token per sequence (int8 [bsz, 1, embed]) over cache buffers [bsz, heads, cap,
         head_dim] whose length after the append is read from the int32 HIP tensor ``length`` when the kernels run
@@ -311,13 +292,6 @@ class Int8OPTAttention(nn.Module):
             if _hip_ext.can_attn_prefill(query, key, vt, attention_mask, bsz, H):
                 ctx = _hip_ext.attn_prefill(query, key, vt, attention_mask, self.qk_bmm._scalar("a"),
                                             self.pv_bmm._scalar("a"), H, checked=True)
-                return self.out_proj(ctx), None, present
-        if (self.fused_softmax and long_ok and layer_head_mask is None and not output_attentions and tgt_len > 16
-                and d % 16 == 0 and d < 128 and d != 64 and query.is_cuda
-                and type(self.qk_bmm) is BMM_S8T_S8N_F32T and type(self.pv_bmm) is BMM_S8T_S8N_S8T):
-            # a head size that the kernel taking this many keys has no form of (OPT-2.7B: 80 beyond 512 keys)
-            ctx = self._prefill_padded_heads(query, key, value, attention_mask, bsz, tgt_len)
-            if ctx is not None:
                 return self.out_proj(ctx), None, present
         probs_q = None
         if (self.fused_softmax and long_ok and layer_head_mask is None and tgt_len > 16
