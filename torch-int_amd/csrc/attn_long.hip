@@ -69,13 +69,15 @@ __global__ __launch_bounds__(256) void mask_classes_kernel(const float* __restri
     cls[blockIdx.x] = all_zero ? MC_ZERO : (all_same && __int_as_float(first) <= -1e30f) ? MC_UNIFORM : MC_MIXED;
 }
 
-template <int D, bool PV, bool MASKED>
+// PART: the head size in memory (dr) is smaller than the LDS row size D; the forms for dr == D carry none of its tests.
+template <int D, bool PV, bool MASKED, bool PART>
 __global__ __launch_bounds__(256, 2) void attn_long_kernel(const int8_t* __restrict__ q, const int8_t* __restrict__ k,
                                                            const float* __restrict__ mask, int8_t* __restrict__ probs,
                                                            int T, int S, long long stride_q, long long stride_k,
                                                            int heads, int row_blocks, float alpha,
                                                            const int8_t* __restrict__ vt, int8_t* __restrict__ ctx,
-                                                           float alpha_pv, const unsigned char* __restrict__ cls, int dr) {
+                                                           float alpha_pv, const unsigned char* __restrict__ cls, int dr_arg) {
+  const int dr = PART ? dr_arg : D;
   // dr = the head size in memory, a multiple of 16 up to D (the LDS row size, 64 or 128): rows of q, k and the
   // context are dr bytes long, V^T has dr rows; the chunks of an LDS row beyond dr hold zeros, which add nothing to
   // the integer products, and the context blocks beyond dr are computed on whatever the LDS holds and not stored.
@@ -105,7 +107,7 @@ __global__ __launch_bounds__(256, 2) void attn_long_kernel(const int8_t* __restr
     const int row = i * RPI + lane / CH, pos = lane % CH;
     const int t = t0 + row < T ? t0 + row : T - 1;  // rows past the end repeat the last one; never stored
     const int chunk = al_swz<D>(row, pos);
-    if (chunk * 16 < dr)
+    if (!PART || chunk * 16 < dr)
       __builtin_amdgcn_global_load_lds((const TI_GLOBAL_AS void*)(qb + (long long)t * dr + (chunk << 4)),
                                        (TI_LDS_AS void*)((TI_LDS_AS char*)qs_base + i * 1024), 16, 0, 0);
     else
@@ -117,7 +119,7 @@ __global__ __launch_bounds__(256, 2) void attn_long_kernel(const int8_t* __restr
     for (int i = wave; i < nkeys / RPI; i += 4) {
       const int row = i * RPI + lane / CH, pos = lane % CH;
       const int chunk = al_swz<D>(row, pos);
-      if (chunk * 16 < dr)
+      if (!PART || chunk * 16 < dr)
         __builtin_amdgcn_global_load_lds((const TI_GLOBAL_AS void*)(kb + (long long)(k0 + row) * dr + (chunk << 4)),
                                          (TI_LDS_AS void*)((TI_LDS_AS char*)ks_base + i * 1024), 16, 0, 0);
       else
@@ -134,7 +136,7 @@ __global__ __launch_bounds__(256, 2) void attn_long_kernel(const int8_t* __restr
         const int row = o / AL_VPITCH;
         int col = o - row * AL_VPITCH;
         col = col < nkeys ? col : 0;  // pad bytes and columns past the last key get a copy of chunk 0: multiplied by p = 0
-        if (row < dr)  // rows of V^T beyond the head size stay as they are: their context blocks are not stored
+        if (!PART || row < dr)  // rows of V^T beyond the head size stay as they are: their context blocks are not stored
           __builtin_amdgcn_global_load_lds((const TI_GLOBAL_AS void*)(vb + (long long)row * S + col),
                                            (TI_LDS_AS void*)((TI_LDS_AS char*)vs_base + i * 1024), 16, 0, 0);
       }
@@ -203,6 +205,12 @@ __global__ __launch_bounds__(256, 2) void attn_long_kernel(const int8_t* __restr
   // matrix instructions and mask loads of different blocks overlap instead of waiting for one another block by
   // block.  (Inlined by force: called from two places each, the lambdas would otherwise stay functions and push
   // the register arrays they capture by reference into scratch memory.)
+  // the tile's copies have landed (and, PART, the zeros this wave wrote beside them); then the workgroup meets
+#define TI_AL_TILE_READY()                                                                         \
+  do {                                                                                             \
+    if constexpr (PART) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");   \
+    else asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");                             \
+  } while (0)
 #define TI_FOR_BLOCKS_OF(tile, body)                            \
   do {                                                          \
     const int nb_rt = blocks_of(tile);                          \
@@ -236,7 +244,7 @@ __global__ __launch_bounds__(256, 2) void attn_long_kernel(const int8_t* __restr
     }
     __syncthreads();  // every wave is done with the previous tile
     load_k_tile(tile);
-    asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+    TI_AL_TILE_READY();
     read_q();
     float top = lowest;
     auto body0 = [&](auto nb_) __attribute__((always_inline)) {
@@ -278,7 +286,7 @@ __global__ __launch_bounds__(256, 2) void attn_long_kernel(const int8_t* __restr
     if (!(live_g >> tile & 1)) continue;  // uniform over the workgroup
     __syncthreads();
     load_k_tile(tile);
-    asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+    TI_AL_TILE_READY();
     read_q();
     if (!(live_w >> tile & 1)) continue;  // uniform over the wave: every e is 0, p + 0 = p
     const bool use_mask = tile_class(tile) != MC_ZERO;
@@ -329,7 +337,7 @@ __global__ __launch_bounds__(256, 2) void attn_long_kernel(const int8_t* __restr
       __syncthreads();
       load_k_tile(tile);
       load_v_tile(tile);
-      asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+      TI_AL_TILE_READY();
       read_q();
     }
     const bool wave_live = live_w >> tile & 1;
@@ -398,7 +406,7 @@ __global__ __launch_bounds__(256, 2) void attn_long_kernel(const int8_t* __restr
 #pragma unroll
         for (int v = 0; v < 4; ++v)
           w |= (unsigned)(unsigned char)Epi<EPI_S8_SCALE>::apply(o[c][v], 0.0f, alpha_pv) << (8 * v);
-        if (16 * c < dr) crow[4 * c] = (int)w;
+        if (!PART || 16 * c < dr) crow[4 * c] = (int)w;
       }
     }
   }
@@ -409,11 +417,11 @@ bool attn_long_supported(long long T, long long S, long long D) {
   return T >= 1 && D >= 16 && D <= 128 && D % 16 == 0 && S >= 16 && S % 16 == 0 && S <= (long long)AL_TILE * AL_MAX_TILES;
 }
 
-template <int D, bool PV, bool MASKED>
+template <int D, bool PV, bool MASKED, bool PART>
 static int launch_al(dim3 grid, hipStream_t stream, const int8_t* q, const int8_t* k, const float* mask, int8_t* probs,
                      int T, int S, long long stride_q, long long stride_k, int heads, int row_blocks, float alpha,
                      const int8_t* vt, int8_t* ctx, float alpha_pv, const unsigned char* cls, int dr) {
-  auto kern = attn_long_kernel<D, PV, MASKED>;
+  auto kern = attn_long_kernel<D, PV, MASKED, PART>;
   constexpr int lds = AL_ROWS * D + AL_TILE * D + (PV ? D * AL_VPITCH : 0) + 16;
   static_assert(2 * lds <= 160 * 1024, "two workgroups per CU");
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
@@ -438,19 +446,26 @@ int launch_attn_long(const int8_t* q, const int8_t* k, const float* mask, int8_t
   if (BH * row_blocks > 0x7fffffffLL || T > 0x7fffffffLL)
     return fail(TI_ERR_INVALID_ARG, "attn_long: too many row blocks (%lld)", BH * row_blocks);
   const dim3 grid((unsigned)(BH * row_blocks));
-#define TI_AL(DD, PV)                                                                                                 \
-  return mask != nullptr                                                                                              \
-             ? launch_al<DD, PV, true>(grid, stream, q, k, mask, probs, (int)T, (int)S, stride_q, stride_k, (int)heads,  \
-                                       (int)row_blocks, alpha, vt, ctx, alpha_pv, cls, (int)D)                       \
-             : launch_al<DD, PV, false>(grid, stream, q, k, mask, probs, (int)T, (int)S, stride_q, stride_k, (int)heads, \
-                                        (int)row_blocks, alpha, vt, ctx, alpha_pv, nullptr, (int)D)
-  if (D > 64) {
-    if (vt == nullptr) TI_AL(128, false);
-    TI_AL(128, true);
+#define TI_AL_ARGS(c) \
+  grid, stream, q, k, mask, probs, (int)T, (int)S, stride_q, stride_k, (int)heads, (int)row_blocks, alpha, vt, ctx, alpha_pv, c, (int)D
+#define TI_AL(DD, PV, PART) \
+  return mask != nullptr ? launch_al<DD, PV, true, PART>(TI_AL_ARGS(cls)) : launch_al<DD, PV, false, PART>(TI_AL_ARGS(nullptr))
+  if (D == 128) {
+    if (vt == nullptr) TI_AL(128, false, false);
+    TI_AL(128, true, false);
   }
-  if (vt == nullptr) TI_AL(64, false);
-  TI_AL(64, true);
+  if (D > 64) {
+    if (vt == nullptr) TI_AL(128, false, true);
+    TI_AL(128, true, true);
+  }
+  if (D == 64) {
+    if (vt == nullptr) TI_AL(64, false, false);
+    TI_AL(64, true, false);
+  }
+  if (vt == nullptr) TI_AL(64, false, true);
+  TI_AL(64, true, true);
 #undef TI_AL
+#undef TI_AL_ARGS
 }
 
 // Bytes of the class array of a mask [batch, 1, T, S] (0: the shape takes no classes), and the launch that fills it.
@@ -471,4 +486,5 @@ int launch_attn_mask_classes(const float* mask, unsigned char* cls, long long ba
 }
 
 #undef TI_FOR_BLOCKS_OF
+#undef TI_AL_TILE_READY
 }  // namespace ti

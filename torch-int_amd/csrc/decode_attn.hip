@@ -41,13 +41,16 @@ __host__ __device__ inline long long decode_attn_lds(long long T, long long S, l
 // NI > 0: the whole cache of the (batch, head) is at most NI row groups per lane and all of its loads are
 // issued up front (keys and values, 16 bytes each per lane), so the kernel waits for memory once.
 // NI == 0: any length, four row groups in flight at a time.
-template <int TQ, int D, int NI>
+// PART: the head size in memory is smaller than D, the bytes of a cache row that the lanes cover; the forms for
+// head sizes 64 and 128 carry none of its tests.
+template <int TQ, int D, int NI, bool PART>
 __global__ __launch_bounds__(256) void decode_attn_kernel(const int8_t* __restrict__ q, const int8_t* __restrict__ k_new,
                                                           const int8_t* __restrict__ v_new, int8_t* k_buf,
                                                           int8_t* v_buf, const float* __restrict__ mask,
                                                           int8_t* __restrict__ ctx, int8_t* __restrict__ probs_out,
                                                           int T, int S_arg, long long cap, int heads, float alpha_qk,
-                                                          float alpha_pv, const int* __restrict__ s_dev, int dr) {
+                                                          float alpha_pv, const int* __restrict__ s_dev, int dr_arg) {
+  const int dr = PART ? dr_arg : D;
   // dr = the head size in memory, a multiple of 16 up to D (64 or 128, the lanes a cache row is spread over):
   // rows of q, the caches and ctx are dr bytes long; the lanes beyond a row hold zeros and store nothing
   // s_dev != nullptr: the number of positions is read from device memory (a launch recorded in a HIP graph is
@@ -70,7 +73,7 @@ __global__ __launch_bounds__(256) void decode_attn_kernel(const int8_t* __restri
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int rs = lane / LPR, cs = lane % LPR;
-  const bool in_row = cs * 16 < dr;
+  const bool in_row = !PART || cs * 16 < dr;
   const long long bh = blockIdx.x;
   const int S_old = k_new != nullptr ? S - T : S;  // rows below come from the cache, the rest from k_new / v_new
   int8_t* kb = k_buf + bh * cap * dr;
@@ -247,7 +250,7 @@ __global__ __launch_bounds__(256) void decode_attn_kernel(const int8_t* __restri
   __syncthreads();
   for (int idx = tid; idx < T * D; idx += 256) {
     const int t = idx / D, c = idx - t * D;
-    if (c < dr) {
+    if (!PART || c < dr) {
       const int sum = red[idx] + red[T * D + idx] + red[2 * T * D + idx] + red[3 * T * D + idx];
       ctx[(bh * T + t) * dr + c] = Epi<EPI_S8_SCALE>::apply(sum, 0.0f, alpha_pv);
     }
@@ -277,8 +280,14 @@ int launch_decode_attn_s8(const int8_t* q, const int8_t* k_new, const int8_t* v_
   // caches of at most 20 row groups per lane (640 positions at head size 128) with one or two query rows take
   // the variant that issues all loads up front
 #define TI_DA(TQ, DD, NI)                                                                                              \
-  hipLaunchKernelGGL((decode_attn_kernel<TQ, DD, NI>), grid, block, lds, stream, q, k_new, v_new, k_buf, v_buf, mask, \
-                     ctx, probs_out, (int)T, (int)S, cap, (int)heads, alpha_qk, alpha_pv, s_dev, (int)D)
+  do {                                                                                                                 \
+    if (D == DD)                                                                                                       \
+      hipLaunchKernelGGL((decode_attn_kernel<TQ, DD, NI, false>), grid, block, lds, stream, q, k_new, v_new, k_buf,    \
+                         v_buf, mask, ctx, probs_out, (int)T, (int)S, cap, (int)heads, alpha_qk, alpha_pv, s_dev, (int)D); \
+    else                                                                                                               \
+      hipLaunchKernelGGL((decode_attn_kernel<TQ, DD, NI, true>), grid, block, lds, stream, q, k_new, v_new, k_buf,     \
+                         v_buf, mask, ctx, probs_out, (int)T, (int)S, cap, (int)heads, alpha_qk, alpha_pv, s_dev, (int)D); \
+  } while (0)
   const bool resident = T <= 2 && S <= 20 * 4 * (64 / (lanes_d / 16));
   if (lanes_d == 128) {
     if (T == 1) { if (resident) TI_DA(1, 128, 20); else TI_DA(1, 128, 0); }
