@@ -371,7 +371,7 @@ int ti_kv_append_s8(const int8_t* k_new, const int8_t* v_new, int8_t* k_buf, int
  * same bits, without the score and probability tensors.  vt is V transposed, [BH, D, S] packed (what
  * ti_transpose_last2_s8 makes, as upstream's `value_states.transpose(1,2).contiguous()`); ctx is [BH/heads, T,
  * heads*D] packed.  Limits (ti_attn_prefill_supported): S a multiple of 16 in [16, 4096] and D a multiple of 16 up to
- * 128 (OPT-2.7B: 80; rows keep their own length in memory).  Up to 512 keys (a multiple of 64) all keys
+ * 128 (OPT-2.7B: 80; rows keep their own length in memory).  Up to 576 keys all keys
  * of a head sit in the LDS and are swept once; other shapes sweep the keys three times in tiles of 256 (row maximum, row
  * sum, probabilities): the same bits either way. */
 int ti_attn_prefill_supported(int64_t T, int64_t S, int64_t D);

@@ -1053,11 +1053,15 @@ def test_fused_prefill_attention_matches_the_chain():
     shapes = [(4, 40, 512, 512, "causal"), (2, 3, 100, 128, "pad"), (1, 4, 64, 64, None),
               (2, 2, 70, 256, "causal"), (1, 2, 300, 320, "causal"), (1, 1, 5, 448, None),
               # exactly 128 / 256 / 512 keys without a mask: the kernels compiled for that fact
-              (1, 2, 80, 128, None), (1, 2, 64, 256, None), (1, 1, 100, 512, None)]
+              (1, 2, 80, 128, None), (1, 2, 64, 256, None), (1, 1, 100, 512, None),
+              # 513 to 576 keys: still one sweep (36 blocks of 16 keys in the registers), 576 exactly with / without a mask;
+              # key counts that 64 does not divide multiply on with V through a last slice that is partly zeros
+              (1, 3, 528, 528, "causal"), (2, 2, 64, 544, "pad"), (1, 2, 576, 576, "causal"), (1, 2, 100, 576, None),
+              (1, 2, 130, 560, None), (1, 2, 90, 400, "causal"), (1, 2, 64, 16, None), (1, 1, 70, 208, "pad")]
     # head size 128, and 64 (OPT-125m ... 1.3B) on the same kernel's 64-byte-row form
     others = [(2, 32, 512, 512, "causal", 80), (2, 3, 100, 128, "pad", 80), (1, 2, 300, 320, "causal", 96),
               (1, 1, 5, 448, None, 112), (1, 2, 64, 256, None, 48), (2, 2, 70, 256, "causal", 32), (1, 4, 64, 64, None, 16),
-              # the three-sweep kernel (more than 512 keys, or a key count that 64 does not divide) at those head sizes
+              # the three-sweep kernel (more than 576 keys) and single sweeps with a partly filled last slice at those head sizes
               (2, 32, 1024, 1024, "causal", 80), (1, 3, 200, 784, "pad", 80), (2, 2, 100, 400, "causal", 96),
               (1, 2, 528, 528, "causal", 112), (1, 2, 70, 1040, None, 48), (1, 3, 600, 2048, "causal", 32), (1, 2, 40, 560, "pad", 16)]
     for (B, H, T, S, kind, d) in ([sh + (128,) for sh in shapes] + [sh + (64,) for sh in [(4, 12, 512, 512, "causal")] + shapes[1:]]
@@ -1083,7 +1087,7 @@ def test_fused_prefill_attention_matches_the_chain():
         assert torch.equal(X.attn_qk_softmax_q(qd, kd, md, a_qk, H).cpu(), probs), (B, H, T, S, kind, d)
     z = lambda *shape: torch.zeros(*shape, dtype=torch.int8, device=DEV)   # noqa: E731
     assert not X.can_attn_prefill(z(2, 64, 128), z(2, 440, 128), z(2, 128, 440), None, 1, 2)   # S % 16 != 0
-    assert X.can_attn_prefill(z(2, 64, 80), z(2, 400, 80), z(2, 80, 400), None, 1, 2)          # head size 80, S % 64 != 0: three sweeps
+    assert X.can_attn_prefill(z(2, 64, 80), z(2, 400, 80), z(2, 80, 400), None, 1, 2)          # head size 80, S % 64 != 0
     assert not X.can_attn_prefill(z(2, 64, 72), z(2, 400, 72), z(2, 72, 400), None, 1, 2)      # head size 72
 
 
@@ -1271,7 +1275,7 @@ def _attn_masks(kind, B, T, S):
 
 
 def test_fused_attention_long_keys_and_head_size_64():
-    # more than 512 keys, key counts that are not multiples of 64, head size 64: the three-sweep kernel; the bytes of
+    # more than 576 keys (three sweeps), key counts that are not multiples of 64, head size 64; the bytes of
     # bmm_s8t_s8n_f32t -> attn_softmax_q (-> bmm_s8t_s8n_s8t -> head merge), from the oracle and from the device kernels
     import torch_int._hip_ext as X
     import torch_int._CUDA as C

@@ -1,5 +1,5 @@
 // Q.K^T fused with the mask, the softmax and the int8 quantisation of the probabilities, for prefill with
-// up to 512 key positions and head sizes up to 128 (any multiple of 16; the LDS rows are 64 or 128 bytes, zero-filled
+// up to 576 key positions and head sizes up to 128 (any multiple of 16; the LDS rows are 64 or 128 bytes, zero-filled
 // beyond the head size, so OPT-2.7B's 80 needs no padded copies of q, k and V^T): probs = round(127 softmax(max(alpha q.k^T + mask, lowest))).
 // The fp32 scores (4 bytes per query-key pair written and read again by the two-kernel form) never leave
 // the registers.  Arithmetic and summation order are those of attn_softmax_q on the scores of
@@ -25,21 +25,26 @@ namespace ti {
 
 constexpr int AF_ROWS = 64;   // query rows per workgroup
 constexpr int AF_D = 128;     // largest head size (sizes the LDS limit)
-constexpr int AF_MAX_S = 512;
+constexpr int AF_MAX_S = 576;  // (64 + 576) rows of 128 bytes = 80 KiB: two workgroups per CU
 
-// NB = key blocks of 16 the registers are sized for (S <= 16 * NB).
-// PV: instead of storing the probabilities, multiply them with V right away (S a multiple of 64): vt is V
-// transposed, [batch*heads, 128, S]; it is copied into the LDS the K panel occupied while the softmax runs
-// (row pitch S + 16 against bank conflicts).  The probabilities of a 64-key slice sit in a lane as four dwords
+// NB = key blocks of 16 the registers are sized for, a multiple of 4: 16 * (NB - 3) <= S <= 16 * NB.  All but the
+// last three blocks exist whatever S is, so every test on them folds away at compile time, which leaves straight-line
+// code: the fragment reads, the matrix instructions and the mask loads of different blocks overlap instead of waiting
+// for one another block by block.  The last three are multiplied and evaluated like the others (on whatever the LDS
+// holds beyond the K panel) and, where S ends before them, their scores are replaced by -infinity: they then take no
+// part in the row maximum, their exponentials are exact zeros that are never added (a block without a live value is
+// skipped), and their probabilities are zeros that meet whatever the V^T panel holds beyond S.
+// PV: instead of storing the probabilities, multiply them with V right away: vt is V transposed,
+// [batch*heads, head size, S]; it is copied into the LDS the K panel occupied while the softmax runs (row pitch =
+// S rounded up to whole slices of 64 keys, + 16 against bank conflicts; the bytes of a row beyond S are whatever the
+// LDS held and meet probabilities that are zero).  The probabilities of a 64-key slice sit in a lane as four dwords
 // (keys 16i + 4g .. +3, i = 0..3); used as they are for the 16 operand bytes of lane (r, g), they fix a
 // permutation of the 64 keys inside the slice, and the V fragments are gathered with the same permutation (four
 // 4-byte reads), so the integer sum over the slice is the same.  The context rows are written already merged:
 // ctx is [batch, T, heads * 128].
-// SPEC: 0 = any S <= 16 * NB and a mask pointer that may be null; 1 / 2 = S == 16 * NB exactly, with / without a mask.
-// In the exact forms every "block j exists" and "there is a mask" test folds away at compile time, which leaves
-// straight-line code: the fragment reads, the matrix instructions and the mask loads of different blocks overlap
-// instead of waiting for one another block by block.
-template <int NB, bool PV, int SPEC = 0, int D = 128>
+// SPEC: 1 / 2 = with / without a mask.  PAD = false: S == 16 * NB, the last three blocks exist like the others (the
+// forms for 128, 256, 512 ... keys are 2 to 4 % faster without the three tests).
+template <int NB, bool PV, int SPEC, int D = 128, bool PAD = true>
 __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t* __restrict__ q,
                                                                    const int8_t* __restrict__ k,
                                                                    const float* __restrict__ mask,
@@ -57,9 +62,10 @@ __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t*
   const int n_bh = gridDim.x / row_blocks;
   const long long bh = blockIdx.x % n_bh;
   const int t0 = (row_blocks - 1 - (int)(blockIdx.x / n_bh)) * AF_ROWS;
-  if constexpr (SPEC != 0) S = 16 * NB;
-  const int nb = SPEC != 0 ? NB : S >> 4;
-  const bool has_mask = SPEC == 1 ? true : SPEC == 2 ? false : mask != nullptr;
+  static_assert(NB % 4 == 0 && (SPEC == 1 || SPEC == 2), "forms");
+  const int nb = S >> 4;
+  constexpr bool has_mask = SPEC == 1;
+  auto exists = [&](int j) { return !PAD || j < NB - 3 || j < nb; };  // block j holds keys (j < NB)
 
   // ---- copies: slab i = 8 rows of [Q tile (64 rows) | K panel (S rows)], 1 KiB per wave instruction
   const int8_t* qb = q + bh * stride_q;
@@ -98,14 +104,15 @@ __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t*
   const float* mrow = has_mask ? mask + (((bh / heads) * T + tc) * (long long)S) : nullptr;
   const float lowest = -3.402823466e+38f;
   float m = lowest;
-  constexpr int MG = NB < 8 ? NB : 8;  // blocks per mask group
+  constexpr int MG = NB < 8 || NB > 32 ? 4 : 8;  // blocks per mask group (36 blocks: the registers hold no more)
   v4f mk[2][MG];
   auto fetch_mask = [&](int j0, v4f (&dst)[MG]) {
 #pragma unroll
     for (int u = 0; u < MG; ++u) {
       const int j = j0 + u;
       dst[u] = v4f{0.f, 0.f, 0.f, 0.f};
-      if (has_mask && j < nb) dst[u] = *reinterpret_cast<const v4f*>(mrow + 16 * j + 4 * g);
+      // (a block beyond S reads the values of block 0 instead - no branch; its scores are replaced below)
+      if (has_mask && j < NB) dst[u] = *reinterpret_cast<const v4f*>(mrow + (exists(j) ? 16 * j : 0) + 4 * g);
     }
   };
   fetch_mask(0, mk[0]);
@@ -123,17 +130,15 @@ __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t*
 #pragma unroll
   for (int j = 0; j < NB; ++j) {
     acc[j] = v4i{0, 0, 0, 0};
-    if (j < nb) {
 #pragma unroll
-      for (int s = 0; s < KS; ++s) {
-        const v4i kf = *reinterpret_cast<const v4i*>(ks + j * 16 * D + (((4 * s + g) ^ sw) << 4));
-        acc[j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(kf, qf[s], acc[j], 0, 0, 0);
-      }
+    for (int s = 0; s < KS; ++s) {
+      const v4i kf = *reinterpret_cast<const v4i*>(ks + j * 16 * D + (((4 * s + g) ^ sw) << 4));
+      acc[j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(kf, qf[s], acc[j], 0, 0, 0);
     }
   }
 
   __syncthreads();  // all waves have read their fragments: the K panel may be overwritten (see the stores below)
-  const int pitch = S + 16;
+  const int pitch = 16 * NB + 16;
   // V^T panel: D rows of pitch bytes, ending where the K panel ended (it starts inside the dead Q tile)
   char* vts = smem + (AF_ROWS + S) * D - D * pitch;
   // ---- x = max(alpha * acc + mask, lowest); row maximum
@@ -144,12 +149,14 @@ __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t*
 #pragma unroll
     for (int u = 0; u < MG; ++u) {
       const int j = j0 + u;
-      if (j < nb) {
+      if (j < NB) {
+        const bool real = exists(j);
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
           float x = Epi<EPI_F32_SCALE>::apply(acc[j][v], 0.0f, alpha);
           if (has_mask) x = x + mk[cur][u][v];
           x = __builtin_fmaxf(x, lowest);  // = x > lowest ? x : lowest, NaN included
+          if (PAD && j >= NB - 3) x = real ? x : -__builtin_inff();
           m = __builtin_fmaxf(m, x);
           acc[j][v] = __float_as_int(x);
         }
@@ -182,19 +189,19 @@ __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t*
 
   // ---- e = exp(x - m); partial sums in the reference order.  exp_nonpos returns exactly 0 below -87, so a
   // block in which no lane of the wave has anything above that (masked-out keys) skips the evaluation.
-  unsigned live = 0;  // bit j: block j has non-zero probabilities somewhere in the wave
+  unsigned long long live = 0;  // bit j: block j has non-zero probabilities somewhere in the wave
   float part[16];
 #pragma unroll
   for (int jj = 0; jj < 16; ++jj) {
     float p = 0.0f;
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
+    for (int h = 0; h < (NB + 15) / 16; ++h) {
       const int j = jj + 16 * h;
-      if (j < NB && j < nb) {
+      if (j < NB) {
         const float top = __builtin_fmaxf(__builtin_fmaxf(__int_as_float(acc[j][0]), __int_as_float(acc[j][1])),
                                           __builtin_fmaxf(__int_as_float(acc[j][2]), __int_as_float(acc[j][3])));
         if (__builtin_amdgcn_ballot_w64(top - m > -87.0f) != 0) {
-          live |= 1u << j;
+          live |= 1ull << j;
 #pragma unroll
           for (int v = 0; v < 4; ++v) {
             const float e = exp_nonpos(__int_as_float(acc[j][v]) - m);
@@ -223,7 +230,7 @@ __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t*
 #pragma unroll
   for (int j = 0; j < NB; ++j) {
     unsigned w = 0;
-    if (j < nb && (live >> j & 1)) {
+    if (live >> j & 1) {
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
         const float pq = __builtin_rintf(__int_as_float(acc[j][v]) * scale);  // in [0, 127]
@@ -240,7 +247,7 @@ __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t*
     char* stage = smem + (D == 128 ? AF_ROWS * D : 0) + wave * 16 * pitch;
 #pragma unroll
     for (int j = 0; j < NB; ++j)
-      if (j < nb) *reinterpret_cast<unsigned*>(stage + r * pitch + 16 * j + 4 * g) = pw[j];
+      *reinterpret_cast<unsigned*>(stage + r * pitch + 16 * j + 4 * g) = pw[j];
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the wave's own LDS writes are done; its reads below follow
     const int cpr = S >> 4;                              // 16-byte chunks per row
     int8_t* pbase = probs + (bh * T + t0 + wave * 16) * (long long)S;
@@ -259,7 +266,7 @@ __global__ __launch_bounds__(256, 2) void attn_qk_softmax_q_kernel(const int8_t*
     const char* vrow = vts + r * pitch + 4 * g;  // V^T row (= head-dim index) r of block c is 16c + r
 #pragma unroll
     for (int sl = 0; sl < NB / 4; ++sl) {
-      if (4 * sl < nb) {
+      {
         const v4i pa = {(int)pw[4 * sl], (int)pw[4 * sl + 1], (int)pw[4 * sl + 2], (int)pw[4 * sl + 3]};
         // (blocks c >= nc multiply rows of the panel that no copy filled: whatever the LDS holds there; their
         // results are not stored.  A test on c here cost the 256-key forms their register allocation.)
@@ -295,24 +302,24 @@ int launch_attn_long(const int8_t* q, const int8_t* k, const float* mask, int8_t
 
 // shapes the single-sweep kernel of this file takes (all keys of a head in the LDS at once)
 static bool single_sweep_ok(long long T, long long S, long long D, bool pv) {
-  return T >= 1 && D >= 16 && D <= 128 && D % 16 == 0 && S >= 16 && S <= AF_MAX_S && S % 16 == 0 &&
-         (!pv || S % 64 == 0);
+  (void)pv;  // with or without the product with V
+  return T >= 1 && D >= 16 && D <= 128 && D % 16 == 0 && S >= 16 && S <= AF_MAX_S && S % 16 == 0;
 }
 
 bool attn_qk_softmax_q_supported(long long T, long long S, long long D) {
   return single_sweep_ok(T, S, D, false) || attn_long_supported(T, S, D);
 }
 
-// the form that multiplies on with V^T: the single sweep needs whole slices of 64 keys
+// the form that multiplies on with V^T
 bool attn_prefill_supported(long long T, long long S, long long D) {
   return single_sweep_ok(T, S, D, true) || attn_long_supported(T, S, D);
 }
 
-template <int NB, bool PV, int SPEC, int D>
+template <int NB, bool PV, int SPEC, int D, bool PAD>
 static int launch_af(dim3 grid, size_t lds, hipStream_t stream, const int8_t* q, const int8_t* k, const float* mask,
                      int8_t* probs, int T, int S, long long stride_q, long long stride_k, int heads, int row_blocks,
                      float alpha, const int8_t* vt, int8_t* ctx, float alpha_pv, int dr) {
-  auto kern = attn_qk_softmax_q_kernel<NB, PV, SPEC, D>;
+  auto kern = attn_qk_softmax_q_kernel<NB, PV, SPEC, D, PAD>;
   static unsigned long long lds_ok = 0;  // bit per device: the large dynamic LDS size has been allowed
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return fail(TI_ERR_LAUNCH, "attn_qk_softmax_q: no current device");
@@ -327,7 +334,7 @@ static int launch_af(dim3 grid, size_t lds, hipStream_t stream, const int8_t* q,
   return TI_OK;
 }
 
-// vt == nullptr: probabilities into probs.  Otherwise context into ctx ([batch, T, heads*128]); needs S % 64 == 0.
+// vt == nullptr: probabilities into probs.  Otherwise context into ctx ([batch, T, heads * head size]).
 int launch_attn_qk_softmax_q(const int8_t* q, const int8_t* k, const float* mask, int8_t* probs, long long BH,
                              long long T, long long S, long long D, long long stride_q, long long stride_k,
                              long long heads, float alpha, const int8_t* vt, int8_t* ctx, float alpha_pv,
@@ -341,31 +348,43 @@ int launch_attn_qk_softmax_q(const int8_t* q, const int8_t* k, const float* mask
     return fail(TI_ERR_INVALID_ARG, "attn_qk_softmax_q: too many row blocks (%lld)", BH * row_blocks);
   const dim3 grid((unsigned)(BH * row_blocks));
   const int row_bytes = D <= 64 ? 64 : 128;  // LDS row size = the kernel's template head size
-  const size_t lds = (size_t)(AF_ROWS + S) * row_bytes;
+  const int nb4 = (int)((S + 63) / 64);        // the form: NB = 4 * nb4 blocks of 16 keys
+  const size_t lds = (size_t)(AF_ROWS + 64 * nb4) * row_bytes;  // the blocks beyond S are read (and not used)
   int rc;
-#define TI_AF(NB, PV, SPEC)                                                                                            \
-  rc = row_bytes == 128                                                                                                \
-           ? launch_af<NB, PV, SPEC, 128>(grid, lds, stream, q, k, mask, probs, (int)T, (int)S, stride_q, stride_k,      \
-                                          (int)heads, (int)row_blocks, alpha, vt, ctx, alpha_pv, (int)D)               \
-           : launch_af<NB, PV, SPEC, 64>(grid, lds, stream, q, k, mask, probs, (int)T, (int)S, stride_q, stride_k,       \
-                                         (int)heads, (int)row_blocks, alpha, vt, ctx, alpha_pv, (int)D)
-#define TI_AF_NB(NB, PV)                                 \
-  do {                                                   \
-    if (S != 16 * NB) TI_AF(NB, PV, 0);                  \
-    else if (mask != nullptr) TI_AF(NB, PV, 1);          \
-    else TI_AF(NB, PV, 2);                               \
-  } while (0)
-  if (vt == nullptr) {
-    if (S <= 128) TI_AF_NB(8, false);
-    else if (S <= 256) TI_AF_NB(16, false);
-    else TI_AF_NB(32, false);
-  } else {
-    if (S <= 128) TI_AF_NB(8, true);
-    else if (S <= 256) TI_AF_NB(16, true);
-    else TI_AF_NB(32, true);
+#define TI_AF_ARGS                                                                                                   \
+  (grid, lds, stream, q, k, mask, probs, (int)T, (int)S, stride_q, stride_k, (int)heads, (int)row_blocks, alpha, vt, ctx, \
+   alpha_pv, (int)D)
+#define TI_AF(NB, PV, SPEC)                                                                      \
+  rc = row_bytes == 128 ? (S == 16 * NB ? launch_af<NB, PV, SPEC, 128, false> TI_AF_ARGS         \
+                                        : launch_af<NB, PV, SPEC, 128, true> TI_AF_ARGS)         \
+                        : (S == 16 * NB ? launch_af<NB, PV, SPEC, 64, false> TI_AF_ARGS          \
+                                        : launch_af<NB, PV, SPEC, 64, true> TI_AF_ARGS)
+#define TI_AF_NB(NB)                                  \
+  case NB / 4:                                        \
+    if (vt == nullptr) {                              \
+      if (mask != nullptr) TI_AF(NB, false, 1);       \
+      else TI_AF(NB, false, 2);                       \
+    } else {                                          \
+      if (mask != nullptr) TI_AF(NB, true, 1);        \
+      else TI_AF(NB, true, 2);                        \
+    }                                                 \
+    break
+  switch (nb4) {
+    TI_AF_NB(4);
+    TI_AF_NB(8);
+    TI_AF_NB(12);
+    TI_AF_NB(16);
+    TI_AF_NB(20);
+    TI_AF_NB(24);
+    TI_AF_NB(28);
+    TI_AF_NB(32);
+    TI_AF_NB(36);
+    default:
+      return fail(TI_ERR_INVALID_ARG, "attn_qk_softmax_q: %lld keys", S);
   }
 #undef TI_AF_NB
 #undef TI_AF
+#undef TI_AF_ARGS
   if (rc) return rc;
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(TI_ERR_LAUNCH, "attn_qk_softmax_q launch: %s", hipGetErrorString(e));

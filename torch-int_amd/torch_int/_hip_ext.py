@@ -403,8 +403,8 @@ def mask_classes(mask):
 
 
 def _classes_ptr(mask, S):
-    """Pointer to the mask's class array where the kernel that will run reads one (more than 512 keys), else None."""
-    if mask is None or S <= 512:
+    """Pointer to the mask's class array where the kernel that will run reads one (more than 576 keys), else None."""
+    if mask is None or S <= 576:
         return None
     cls = mask_classes(mask)
     return cls.data_ptr() if cls is not None else None

@@ -279,10 +279,10 @@ class Int8OPTAttention(nn.Module):
         value = value.view(bsz * H, -1, d) if value.is_contiguous() else value.reshape(bsz * H, value.shape[2], d)
         src_len = key.size(1)
 
-        # Beyond 512 keys the fused kernels sweep the keys three times and win through the key tiles a causal mask
+        # Beyond 576 keys the fused kernels sweep the keys three times and win through the key tiles a causal mask
         # kills (160 x 2048 x 2048: 0.99 ms against 1.34 ms for the separate kernels; without a mask they are slower), so
         # they are taken for a plain prefill (tgt_len == src_len) only.
-        long_ok = src_len <= 512 or tgt_len == src_len
+        long_ok = src_len <= 576 or tgt_len == src_len
         if (self.fused_softmax and long_ok and layer_head_mask is None and not output_attentions and tgt_len > 16
                 and type(self.qk_bmm) is BMM_S8T_S8N_F32T and type(self.pv_bmm) is BMM_S8T_S8N_S8T
                 and _hip_ext.can_attn_qk_softmax_q(query, key, attention_mask, bsz, H) and value.is_cuda
