@@ -12,6 +12,7 @@ each model is built once, and a row runs 3 warm-up forwards and then enough of t
   python torch-int_amd/benchmark/bench_opt_grid.py --models opt-30b opt-66b --batches 1 4 --seqs 512
 """
 import argparse
+import gc
 import json
 import os
 import sys
@@ -67,6 +68,7 @@ def main():
                                   "linear_TOPS": round(ops / ms / 1e9, 1), "tokens_per_s": round(tokens / ms * 1e3),
                                   "int8_weight_GB": round(weights_gb, 2)}), flush=True)
         del model, stack
+        gc.collect()  # the modules hold reference cycles: without this the next model's peak includes this one's weights
         torch.cuda.empty_cache()
 
 
