@@ -416,16 +416,18 @@ def test_fused_softmax_switch_restores_the_torch_chain():
 
 
 @torch.no_grad()
-@pytest.mark.parametrize("D,H", [(640, 8), (192, 4), (2560, 32)])
-def test_prefill_attention_at_head_sizes_between_the_lane_layouts(D, H):
+@pytest.mark.parametrize("D,H,T", [(640, 8, 112), (192, 4, 112), (2560, 32, 112), (256, 4, 528), (512, 4, 544),
+                                   (320, 4, 592)])
+def test_prefill_attention_at_head_sizes_between_the_lane_layouts(D, H, T):
     """Head sizes that are multiples of 16 other than 64 / 128 (OPT-2.7B: 2560 / 32 = 80) take the one-launch prefill
-    attention on q, k and V^T as they are (112 keys: the three-sweep kernel; its LDS rows are zero-filled beyond the
-    head size).  Same bits as the operator chain (Q.K^T, softmax-quantiser, P.V, head merge), which a call that wants
-    the probabilities back still runs."""
+    attention on q, k and V^T as they are (the LDS rows are zero-filled beyond the head size), and so do key counts that
+    64 does not divide (112: a last slice of keys that is partly padding) and those between 513 and 576 (still one
+    sweep; 592: three).  Same bits as the operator chain (Q.K^T, softmax-quantiser, P.V, head merge), which a call that
+    wants the probabilities back still runs."""
     import torch_int._hip_ext as X
     g = torch.Generator().manual_seed(D + H)
     layer = randomize_int8_layer(Int8OPTDecoderLayer(D, H, 2 * D), g).to(DEV)
-    B, T = 2, 112
+    B = 2
     hidden = torch.randn(B, T, D, generator=g).to(DEV)
     mask = causal_mask(B, T, T).to(DEV)
     mask[1, :, :, :5] = torch.finfo(torch.float32).min   # left padding on one sequence
