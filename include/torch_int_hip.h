@@ -430,6 +430,41 @@ int ti_attn_prefill_s8_mc(const int8_t* q, const int8_t* k, const int8_t* vt, co
                           const uint8_t* mask_classes, int8_t* ctx, int64_t BH, int64_t T, int64_t S, int64_t D,
                           int64_t stride_q, int64_t stride_k, int64_t heads, float alpha_qk, float alpha_pv, void* stream);
 
+/* One decode step of one decoder layer (torch_int/models/opt.py:202-299, Int8OPTDecoderLayer.forward, with one new token
+ * per sequence and a KV cache) from one call: LayerNormQ, the q/k/v projections, the cache append and the attention,
+ * out_proj, the residual update fused with the second LayerNormQ, fc1 (ReLU) and fc2 added into the residual
+ * stream.  Each step is the entry point above that the modules call for it (ti_add_layernorm_q[_f16[_xf32]],
+ * ti_linear_a8_w8_b8_o8_group, ti_decode_attn_s8, ti_linear_a8_w8_bfp32_ofp32[_acc], ti_linear_relu_a8_w8_b8_o8,
+ * ti_add_f16_xf32), with the same arguments: the values are theirs; what the call saves is the host time of eight
+ * trips through the caller's language.  hidden is the residual stream [B, 1, embed] (fp32, or fp16 with half = 1: then
+ * the LayerNorm parameters are fp16 too), updated in place; mask fp32 [B, 1, 1, S] or NULL; k_buf / v_buf the cache
+ * buffers [B, heads, cap, head_dim] holding S - 1 positions, S after the call; scratch: device memory of
+ * ti_opt_decoder_layer_decode_scratch_bytes(B, embed, ffn) bytes on a 256-byte boundary (the layers of a model can
+ * share it: calls on one stream run one after the other).  B <= 16. */
+typedef struct TiOptDecodeLayer {
+  int64_t embed, heads, head_dim, ffn;
+  int32_t half;                 /* 1: residual stream and LayerNorm parameters are fp16 */
+  float ln1_eps, ln2_eps;
+  const void *ln1_gamma, *ln1_beta, *ln2_gamma, *ln2_beta;
+  const int8_t *wq, *wk, *wv;   /* [embed, embed] */
+  const int8_t *bq, *bk, *bv;   /* [embed] */
+  float alpha_q, alpha_k, alpha_v, beta_q, beta_k, beta_v;
+  float alpha_qk, alpha_pv;     /* scales of the two attention products */
+  const int8_t* wo;             /* out_proj [embed, embed], fp32 bias, beta = 1 */
+  const float* bo;
+  float alpha_o;
+  const int8_t* w1;             /* fc1 [ffn, embed], int8 bias */
+  const int8_t* b1;
+  float alpha_1, beta_1;
+  const int8_t* w2;             /* fc2 [embed, ffn], fp32 bias, beta = 1 */
+  const float* b2;
+  float alpha_2;
+} TiOptDecodeLayer;
+int64_t ti_opt_decoder_layer_decode_scratch_bytes(int64_t B, int64_t embed, int64_t ffn);
+int ti_opt_decoder_layer_decode(const TiOptDecodeLayer* layer, void* hidden, const float* mask, int8_t* k_buf,
+                                int8_t* v_buf, int64_t B, int64_t cap, int64_t S, void* scratch, int64_t scratch_bytes,
+                                void* stream);
+
 #ifdef __cplusplus
 }
 #endif

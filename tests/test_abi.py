@@ -160,6 +160,27 @@ def test_c_abi_rejects_bad_arguments_without_a_device():
     rc = lib.ti_linear_a8_w8_b8_o8_group_heads(p, None, ptrs, ptrs, scal, scal, 3, 8, 32, 16, 4, 16, None)
     assert rc == 1 and b"NULL" in lib.ti_last_error()
     assert lib.ti_linear_a8_w8_b8_o8_group_heads(p, ptrs, ptrs, ptrs, scal, scal, 0, 8, 32, 16, 4, 16, None) == 0
+    # one decoder layer's decode step from one call: layer description, batch limit, scratch size
+    import torch_int._hip_ext as X
+    st = X.OptDecodeLayer()
+    st.embed, st.heads, st.head_dim, st.ffn = 256, 4, 64, 1024
+    need = lib.ti_opt_decoder_layer_decode_scratch_bytes(4, 256, 1024)
+    assert need == 5 * 1024 + 4096 + 4096 and lib.ti_opt_decoder_layer_decode_scratch_bytes(0, 256, 1024) == 0
+    big = ctypes.create_string_buffer(512)
+    pa = (ctypes.addressof(big) + 255) // 256 * 256
+    assert lib.ti_opt_decoder_layer_decode(None, p, None, p, p, 4, 64, 10, pa, need, None) == 1
+    assert b"no layer" in lib.ti_last_error()
+    assert lib.ti_opt_decoder_layer_decode(ctypes.addressof(st), p, None, p, p, 17, 64, 10, pa, need, None) == 1
+    assert b"0 to 16" in lib.ti_last_error()
+    assert lib.ti_opt_decoder_layer_decode(ctypes.addressof(st), p, None, p, p, 4, 64, 10, pa, need - 1, None) == 1
+    assert b"scratch" in lib.ti_last_error()
+    assert lib.ti_opt_decoder_layer_decode(ctypes.addressof(st), None, None, p, p, 4, 64, 10, pa, need, None) == 1
+    assert b"NULL" in lib.ti_last_error()
+    st.head_dim = 80
+    assert lib.ti_opt_decoder_layer_decode(ctypes.addressof(st), p, None, p, p, 4, 64, 10, pa, need, None) == 1
+    assert b"heads * head_dim" in lib.ti_last_error()
+    st.head_dim = 64
+    assert lib.ti_opt_decoder_layer_decode(ctypes.addressof(st), None, None, None, None, 0, 64, 10, None, 0, None) == 0
     # empty problems succeed without touching pointers or a device
     assert lib.ti_linear_a8_w8_b8_o8(None, None, None, None, 0, 16, 16, 1.0, 1.0, None, 0, None) == 0
     assert lib.ti_dq_add_layernorm_q(None, 1.0, None, None, None, 1e-5, None, None, 0, 128, None) == 0

@@ -417,9 +417,14 @@ class _Tap:
             wrap(C, n)
         for n in self.X_NAMES:
             wrap(X, n)
+        # a decode step normally issues a layer's kernels from one C call; the tap is there to see them one by one
+        from torch_int.models.opt import Int8OPTDecoderLayer
+        one_call = Int8OPTDecoderLayer.decode_in_one_call
+        Int8OPTDecoderLayer.decode_in_one_call = False
         try:
             yield self
         finally:
+            Int8OPTDecoderLayer.decode_in_one_call = one_call
             for mod, name, fn in saved:
                 setattr(mod, name, fn)
 
@@ -560,10 +565,16 @@ def test_decoder_layer_opt66b_shape_prefill_and_decode(bsz):
         m = torch.zeros(bsz, 1, 1, src)
         if bsz > 1:
             m[1, :, :, :7] = torch.finfo(torch.float32).min   # one batch row with left padding
+        if step in (0, 15, 31):
+            # the same step issued from one C call (what an untapped layer does), on copies of the state
+            past_copy = tuple(t.clone() for t in past)
+            one = layer(x.clone(), attention_mask=m.to(DEV), use_cache=True, past_key_value=past_copy)
         with tap.on():
             out = layer(x, attention_mask=m.to(DEV), use_cache=True, past_key_value=past)
         new = out[1]
         assert new[0].shape == (bsz, H, src, D // H) and new[0].data_ptr() == (past[0].data_ptr() if step else new[0].data_ptr())
+        if step in (0, 15, 31):
+            assert torch.equal(one[0], out[0]) and torch.equal(one[1][0], new[0]) and torch.equal(one[1][1], new[1]), step
         past = new
         names = [c[0] for c in tap.calls]
         if step in (0, 31):

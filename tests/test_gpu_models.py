@@ -274,8 +274,12 @@ def test_fp16_model_runs_the_fused_kernels_and_follows_the_torch_chain():
     glm = copy.deepcopy(lm).to(DEV).half()
     assert glm.model.decoder.layers[0].fc2.bias.dtype == torch.float32       # upstream keeps this bias in fp32
     assert glm.model.decoder.layers[0].final_layer_norm.weight.dtype == torch.float16
-    calls = {"ln": 0, "add": 0}
-    real_ln, real_add = X.add_layernorm_q, X.add_rounded_
+    calls = {"ln": 0, "add": 0, "one": 0}
+    real_ln, real_add, real_one = X.add_layernorm_q, X.add_rounded_, X.opt_layer_decode
+
+    def count_one(plan, hidden, *a, **k):
+        calls["one"] += plan.half and hidden.dtype is torch.float16
+        return real_one(plan, hidden, *a, **k)
 
     def count_ln(x, residual, *a, **k):
         calls["ln"] += residual.dtype is torch.float16
@@ -284,14 +288,16 @@ def test_fp16_model_runs_the_fused_kernels_and_follows_the_torch_chain():
     def count_add(residual, x):
         calls["add"] += 1
         return real_add(residual, x)
-    X.add_layernorm_q, X.add_rounded_ = count_ln, count_add
+    X.add_layernorm_q, X.add_rounded_, X.opt_layer_decode = count_ln, count_add, count_one
     try:
         _say("fp16 causal LM, fused")
         out = glm(ids, use_cache=True)
         step = glm(ids[:, -1:], past_key_values=out.past_key_values, use_cache=True)
     finally:
-        X.add_layernorm_q, X.add_rounded_ = real_ln, real_add
-    assert out.logits.dtype == torch.float16 and calls["ln"] == 2 * 3 * 2 and calls["add"] == 3 * 2
+        X.add_layernorm_q, X.add_rounded_, X.opt_layer_decode = real_ln, real_add, real_one
+    # the prefill goes through the modules (two LayerNorm-quantisers and one rounded add per layer), the decode step
+    # through one call per layer that issues the same fp16 kernels
+    assert out.logits.dtype == torch.float16 and calls["ln"] == 2 * 3 and calls["add"] == 3 and calls["one"] == 3, calls
     real_can = X.can_fuse_layernorm
     X.can_fuse_layernorm = lambda x, w, b: False
     X.add_rounded_ = lambda residual, x: residual.add_(x.to(residual.dtype))
@@ -448,3 +454,68 @@ def test_prefill_attention_at_head_sizes_between_the_lane_layouts(D, H, T):
     assert torch.equal(fused[0], chain[0])
     assert torch.equal(fused[-1][0], chain[-1][0]) and torch.equal(fused[-1][1], chain[-1][1])
     assert chain[1].shape == (B, H, T, T)
+
+
+@torch.no_grad()
+@pytest.mark.parametrize("half", [False, True])
+@pytest.mark.parametrize("D,H,bsz", [(256, 4, 1), (320, 4, 3), (512, 4, 16)])
+def test_decode_step_from_one_call_gives_the_modules_values(D, H, bsz, half):
+    """One new token per sequence over a KV cache: the layer issues its kernels from one C call
+    (ti_opt_decoder_layer_decode).  Residual stream and cache, step after step (the cache outgrows its buffer on the
+    way), bit for bit those of the same layer going through its modules; a hook on a sub-module switches the one
+    call off."""
+    g = torch.Generator().manual_seed(7 * D + bsz)
+    layer = randomize_int8_layer(Int8OPTDecoderLayer(D, H, 3 * D), g).to(DEV)
+    if half:
+        layer = layer.half()
+    dt = torch.float16 if half else torch.float32
+    T0 = 40
+    hidden = torch.randn(bsz, T0, D, generator=g).to(DEV).to(dt)
+    mask = causal_mask(bsz, T0, T0).to(DEV)
+    if bsz > 1:
+        mask[1, :, :, :3] = torch.finfo(torch.float32).min     # left padding on one sequence
+    out = layer(hidden.clone(), attention_mask=mask.to(dt) if half else mask, use_cache=True)
+    caches = {True: out[-1], False: tuple(t.clone() for t in out[-1])}
+    assert type(layer).decode_in_one_call is True
+    seen = []
+    real = _hip_ext_mod().opt_layer_decode
+
+    def counted(*a, **kw):
+        seen.append(a[-1])
+        return real(*a, **kw)
+    _hip_ext_mod().opt_layer_decode = counted
+    try:
+        for step in range(90):
+            S = T0 + step + 1
+            x = torch.randn(bsz, 1, D, generator=g).to(DEV).to(dt)
+            m = torch.zeros(bsz, 1, 1, S, device=DEV)
+            if bsz > 1:
+                m[1, :, :, :3] = torch.finfo(torch.float32).min
+            if step % 3 == 2:
+                m = None                                          # no mask at all
+            elif half:
+                m = m.to(dt)
+            res = {}
+            for one_call in (True, False):
+                layer.decode_in_one_call = one_call
+                res[one_call] = layer(x.clone(), attention_mask=m, past_key_value=caches[one_call], use_cache=True)
+                caches[one_call] = res[one_call][-1]
+            assert torch.equal(res[True][0], res[False][0]), (step, (res[True][0] != res[False][0]).sum().item())
+            for a, b in zip(caches[True], caches[False]):
+                assert a.shape == b.shape == (bsz, H, S, D // H) and torch.equal(a, b), step
+        assert seen == list(range(T0 + 1, T0 + 91)), seen          # every step of the first variant took the one call
+        layer.decode_in_one_call = True
+        handle = layer.fc1.register_forward_hook(lambda mod, inp, out: None)
+        n = len(seen)
+        layer(x.clone(), attention_mask=None, past_key_value=caches[True], use_cache=True)
+        handle.remove()
+        assert len(seen) == n                                        # the hook saw fc1 being called instead
+    finally:
+        _hip_ext_mod().opt_layer_decode = real
+        layer.decode_in_one_call = True
+        del layer.decode_in_one_call
+
+
+def _hip_ext_mod():
+    import torch_int._hip_ext as X
+    return X

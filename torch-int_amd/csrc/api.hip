@@ -721,4 +721,76 @@ int ti_transpose_last2_s8(const int8_t* src, int8_t* dst, int64_t B, int64_t R, 
   return launch_transpose_last2_s8(src, dst, B, R, C, static_cast<hipStream_t>(stream));
 }
 
+// One decoder layer of a decode step: the seven (fp16 stream: eight) calls an Int8OPTDecoderLayer makes for one new
+// token per sequence, issued from one C call.  Each step IS the public entry point the Python modules call, with
+// the arguments they pass, so the values are theirs.
+int64_t ti_opt_decoder_layer_decode_scratch_bytes(int64_t B, int64_t embed, int64_t ffn) {
+  if (B <= 0 || embed <= 0 || ffn <= 0) return 0;
+  auto up = [](int64_t n) { return (n + 255) / 256 * 256; };
+  return 5 * up(B * embed) + up(4 * B * embed) + up(B * ffn);
+}
+
+int ti_opt_decoder_layer_decode(const TiOptDecodeLayer* L, void* hidden, const float* mask, int8_t* k_buf, int8_t* v_buf,
+                                int64_t B, int64_t cap, int64_t S, void* scratch, int64_t scratch_bytes, void* stream) {
+  g_err[0] = 0;
+  const char* op = "opt_decoder_layer_decode";
+  if (L == nullptr) return fail(TI_ERR_INVALID_ARG, "%s: no layer description", op);
+  const int64_t E = L->embed, H = L->heads, d = L->head_dim, F = L->ffn;
+  if (E <= 0 || H <= 0 || d <= 0 || F <= 0 || H * d != E)
+    return fail(TI_ERR_INVALID_ARG, "%s: needs embed = heads * head_dim > 0 and ffn > 0 (got %lld, %lld x %lld, %lld)", op,
+                (long long)E, (long long)H, (long long)d, (long long)F);
+  if (B < 0 || B > 16) return fail(TI_ERR_INVALID_ARG, "%s: 0 to 16 sequences, one new token each (got %lld)", op, (long long)B);
+  if (B == 0) return TI_OK;
+  if (int rc = check_ptr(op, "hidden", hidden, L->half ? 2 : 4, true)) return rc;
+  if (int rc = check_ptr(op, "scratch", scratch, 256, true)) return rc;
+  if (scratch_bytes < ti_opt_decoder_layer_decode_scratch_bytes(B, E, F))
+    return fail(TI_ERR_INVALID_ARG, "%s: scratch of %lld bytes, needs %lld", op, (long long)scratch_bytes,
+                (long long)ti_opt_decoder_layer_decode_scratch_bytes(B, E, F));
+  auto up = [](int64_t n) { return (n + 255) / 256 * 256; };
+  char* at = static_cast<char*>(scratch);
+  auto take = [&](int64_t bytes) {
+    char* r = at;
+    at += up(bytes);
+    return r;
+  };
+  int8_t* x = reinterpret_cast<int8_t*>(take(B * E));      // LayerNorm-quantised input of the projections, then of fc1
+  int8_t* q = reinterpret_cast<int8_t*>(take(B * E));
+  int8_t* k = reinterpret_cast<int8_t*>(take(B * E));
+  int8_t* v = reinterpret_cast<int8_t*>(take(B * E));
+  int8_t* ctx = reinterpret_cast<int8_t*>(take(B * E));
+  float* f32 = reinterpret_cast<float*>(take(4 * B * E));   // output of out_proj, then (fp16 stream) of fc2
+  int8_t* h = reinterpret_cast<int8_t*>(take(B * F));
+  int rc;
+  // self_attn_layer_norm
+  rc = L->half ? ti_add_layernorm_q_f16(nullptr, hidden, L->ln1_gamma, L->ln1_beta, L->ln1_eps, x, B, E, stream)
+               : ti_add_layernorm_q(nullptr, static_cast<float*>(hidden), static_cast<const float*>(L->ln1_gamma),
+                                    static_cast<const float*>(L->ln1_beta), L->ln1_eps, x, B, E, stream);
+  if (rc) return rc;
+  // q, k, v projections
+  const int8_t* w3[3] = {L->wq, L->wk, L->wv};
+  const int8_t* b3[3] = {L->bq, L->bk, L->bv};
+  int8_t* o3[3] = {q, k, v};
+  const float a3[3] = {L->alpha_q, L->alpha_k, L->alpha_v};
+  const float be3[3] = {L->beta_q, L->beta_k, L->beta_v};
+  if ((rc = ti_linear_a8_w8_b8_o8_group(x, w3, b3, o3, a3, be3, 3, B, E, E, stream))) return rc;
+  // cache append + attention; [B, 1, E] rows are [B * heads, 1, head_dim] as they lie
+  if ((rc = ti_decode_attn_s8(q, k, v, k_buf, v_buf, mask, ctx, nullptr, B * H, 1, d, cap, S, H, L->alpha_qk, L->alpha_pv,
+                              stream)))
+    return rc;
+  // out_proj, then the residual update fused with final_layer_norm
+  if ((rc = ti_linear_a8_w8_bfp32_ofp32(ctx, L->wo, L->bo, f32, B, E, E, L->alpha_o, 1.0f, nullptr, 0, stream))) return rc;
+  rc = L->half ? ti_add_layernorm_q_f16_xf32(f32, hidden, L->ln2_gamma, L->ln2_beta, L->ln2_eps, x, B, E, stream)
+               : ti_add_layernorm_q(f32, static_cast<float*>(hidden), static_cast<const float*>(L->ln2_gamma),
+                                    static_cast<const float*>(L->ln2_beta), L->ln2_eps, x, B, E, stream);
+  if (rc) return rc;
+  // fc1 (ReLU), fc2 added into the residual stream
+  if ((rc = ti_linear_relu_a8_w8_b8_o8(x, L->w1, L->b1, h, B, F, E, L->alpha_1, L->beta_1, nullptr, 0, stream))) return rc;
+  if (L->half) {
+    if ((rc = ti_linear_a8_w8_bfp32_ofp32(h, L->w2, L->b2, f32, B, E, F, L->alpha_2, 1.0f, nullptr, 0, stream))) return rc;
+    return ti_add_f16_xf32(f32, hidden, B * E, stream);
+  }
+  return ti_linear_a8_w8_bfp32_ofp32_acc(h, L->w2, L->b2, static_cast<float*>(hidden), B, E, F, L->alpha_2, 1.0f, nullptr, 0,
+                                         stream);
+}
+
 }  // extern "C"

@@ -196,6 +196,24 @@ static PyObject* fc_decode_attn(PyObject* self, PyObject* const* a, Py_ssize_t n
                                            (float)apv, st));
 }
 
+/* opt_layer_decode(layer, hidden, mask, k_buf, v_buf, B, cap, S, scratch, scratch_bytes, stream) -> status;
+ * layer = address of a TiOptDecodeLayer that the caller keeps alive */
+static PyObject* fc_opt_layer_decode(PyObject* self, PyObject* const* a, Py_ssize_t n) {
+  (void)self;
+  if (n != 11) {
+    PyErr_SetString(PyExc_TypeError, "opt_layer_decode expects 11 arguments");
+    return NULL;
+  }
+  void *layer = as_ptr(a[0]), *hidden = as_ptr(a[1]), *mask = as_ptr(a[2]), *kb = as_ptr(a[3]), *vb = as_ptr(a[4]);
+  int64_t B = as_i64(a[5]), cap = as_i64(a[6]), S = as_i64(a[7]);
+  void* scratch = as_ptr(a[8]);
+  int64_t sb = as_i64(a[9]);
+  void* st = as_ptr(a[10]);
+  if (PyErr_Occurred()) return NULL;
+  return PyLong_FromLong(ti_opt_decoder_layer_decode((const TiOptDecodeLayer*)layer, hidden, (const float*)mask, kb, vb, B,
+                                                     cap, S, scratch, sb, st));
+}
+
 static PyObject* fc_last_error(PyObject* self, PyObject* noargs) {
   (void)self;
   (void)noargs;
@@ -213,6 +231,7 @@ static PyMethodDef methods[] = {
     {"linear_group3", (PyCFunction)(void (*)(void))fc_linear_group3, METH_FASTCALL, "forward to ti_linear_a8_w8_b8_o8_group"},
     {"kv_append", (PyCFunction)(void (*)(void))fc_kv_append, METH_FASTCALL, "forward to ti_kv_append_s8"},
     {"decode_attn", (PyCFunction)(void (*)(void))fc_decode_attn, METH_FASTCALL, "forward to ti_decode_attn_s8"},
+    {"opt_layer_decode", (PyCFunction)(void (*)(void))fc_opt_layer_decode, METH_FASTCALL, "forward to ti_opt_decoder_layer_decode"},
     {"last_error", fc_last_error, METH_NOARGS, "ti_last_error()"},
     {NULL, NULL, 0, NULL}};
 

@@ -93,7 +93,24 @@ _lib.ti_diag_mix_loop.argtypes = [ctypes.c_int, ctypes.c_int, _vp, _i64, _i64, _
 _lib.ti_diag_mix_loop.restype = ctypes.c_int
 _lib.ti_diag_mix_loop_ops.argtypes = [ctypes.c_int, _i64]
 _lib.ti_diag_mix_loop_ops.restype = _i64
+
+
+class OptDecodeLayer(ctypes.Structure):
+    """``TiOptDecodeLayer`` of include/torch_int_hip.h: what one decoder layer's decode step reads."""
+    _fields_ = ([(n, _i64) for n in ("embed", "heads", "head_dim", "ffn")]
+                + [("half", ctypes.c_int32), ("ln1_eps", _f32), ("ln2_eps", _f32)]
+                + [(n, _vp) for n in ("ln1_gamma", "ln1_beta", "ln2_gamma", "ln2_beta", "wq", "wk", "wv", "bq", "bk", "bv")]
+                + [(n, _f32) for n in ("alpha_q", "alpha_k", "alpha_v", "beta_q", "beta_k", "beta_v", "alpha_qk", "alpha_pv")]
+                + [("wo", _vp), ("bo", _vp), ("alpha_o", _f32), ("w1", _vp), ("b1", _vp), ("alpha_1", _f32), ("beta_1", _f32),
+                   ("w2", _vp), ("b2", _vp), ("alpha_2", _f32)])
+
+
+_lib.ti_opt_decoder_layer_decode_scratch_bytes.argtypes = [_i64, _i64, _i64]
+_lib.ti_opt_decoder_layer_decode_scratch_bytes.restype = _i64
+_lib.ti_opt_decoder_layer_decode.argtypes = [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _i64, _vp]
+_lib.ti_opt_decoder_layer_decode.restype = ctypes.c_int
 _raw_stream = torch._C._cuda_getCurrentRawStream
+_fast_opt_layer_decode = getattr(_CUDA._fast, "opt_layer_decode", None)
 _fast = _CUDA._fast if getattr(_CUDA._fast, "kv_append", None) is not None else None
 _fast_decode_attn = getattr(_CUDA._fast, "decode_attn", None)
 _fast_group3 = getattr(_CUDA._fast, "linear_group3", None)
@@ -513,6 +530,55 @@ def decode_attention(q, k_new, v_new, k_buf, v_buf, filled, mask, alpha_qk, alph
     if rc:
         raise RuntimeError(f"torch_int._hip_ext.decode_attention: {_lib.ti_last_error().decode()} (status {rc})")
     return ctx, probs
+
+
+_decode_attn_ok = {}
+
+
+def decode_attention_shape_ok_cached(T, S, d):
+    """``decode_attention_shape_ok`` remembered per shape (a decode loop asks once per layer and step)."""
+    key = (T, S, d)
+    ok = _decode_attn_ok.get(key)
+    if ok is None:
+        if len(_decode_attn_ok) > 65536:
+            _decode_attn_ok.clear()
+        ok = _decode_attn_ok[key] = bool(_lib.ti_decode_attn_supported(T, S, d))
+    return ok
+
+
+_decode_scratch = {}
+
+
+def opt_layer_decode(plan, hidden, mask, k_buf, v_buf, S):
+    """One decode step of one decoder layer from one C call (``ti_opt_decoder_layer_decode``): ``hidden`` [B, 1, embed]
+    (fp32, or fp16 when the plan says half) is updated in place, the new key and value rows are appended to the cache
+    buffers, which hold S - 1 positions before the call.  ``plan`` carries ``addr`` (the address of an ``OptDecodeLayer``
+    that the caller filled from tensors it keeps alive), ``embed`` and ``ffn``; the caller has checked shapes, dtypes,
+    devices and contiguity (the decoder layer does).  The scratch memory is one buffer per device, stream and size,
+    shared by every layer."""
+    dev = hidden.device
+    B = hidden.shape[0]
+    with _on(dev):
+        stream = _raw_stream(dev.index)
+        key = (dev.index, stream, B, plan.embed, plan.ffn)
+        scratch = _decode_scratch.get(key)
+        if scratch is None:
+            if len(_decode_scratch) >= 64:
+                _decode_scratch.clear()
+            n = _lib.ti_opt_decoder_layer_decode_scratch_bytes(B, plan.embed, plan.ffn)
+            scratch = _decode_scratch[key] = torch.empty(n, dtype=torch.uint8, device=dev)
+        if _fast_opt_layer_decode is not None:
+            rc = _fast_opt_layer_decode(plan.addr, hidden.data_ptr(),
+                                        mask.data_ptr() if mask is not None else 0, k_buf.data_ptr(), v_buf.data_ptr(),
+                                        B, k_buf.shape[2], S, scratch.data_ptr(), scratch.numel(), stream)
+        else:
+            rc = _lib.ti_opt_decoder_layer_decode(plan.addr, hidden.data_ptr(),
+                                                  mask.data_ptr() if mask is not None else None, k_buf.data_ptr(),
+                                                  v_buf.data_ptr(), B, k_buf.shape[2], S, scratch.data_ptr(),
+                                                  scratch.numel(), stream or None)
+    if rc:
+        raise RuntimeError(f"torch_int._hip_ext.opt_layer_decode: {_lib.ti_last_error().decode()} (status {rc})")
+    return hidden
 
 
 def decode_attention_devlen(q, k_new, v_new, k_buf, v_buf, length, max_length, alpha_qk, alpha_pv):

@@ -8,6 +8,7 @@ mask, final LayerNorm, fp ``lm_head``) instead of borrowing methods from a
 particular ``transformers`` release; any object with OPTConfig's field names
 works as ``config``.
 """
+import ctypes
 from dataclasses import dataclass
 from typing import List, Optional, Tuple
 
@@ -37,6 +38,16 @@ def _kv_room(past, new):
     if (kv is not None and kv.filled == S and S + T <= kv.buf.shape[2] and past.data_ptr() == kv.buf.data_ptr()
             and past.stride() == kv.buf.stride() and past.shape[:2] == new.shape[:2] and past.shape[3] == new.shape[3]
             and past.dtype == new.dtype and past.device == new.device):
+        return kv
+    return None
+
+
+def _kv_room_for(past, T):
+    """``_kv_room`` for T new positions that will be written by a kernel (there is no tensor to compare with)."""
+    kv = getattr(past, "_ti_kv", None)
+    S = past.shape[2]
+    if (kv is not None and kv.filled == S and S + T <= kv.buf.shape[2] and past.data_ptr() == kv.buf.data_ptr()
+            and past.stride() == kv.buf.stride()):
         return kv
     return None
 
@@ -345,6 +356,87 @@ class Int8OPTAttention(nn.Module):
         return self.out_proj(ctx), probs_out, present
 
 
+class _DecodePlan:
+    """``Int8OPTDecoderLayer`` flattened into the structure ``ti_opt_decoder_layer_decode`` reads, plus what it was
+    built from: (dict that holds the tensor, its name, the tensor, its version) for every buffer, so that a replaced
+    or rewritten buffer is noticed."""
+    __slots__ = ("ok", "half", "device", "struct", "addr", "sources", "modules", "embed", "heads", "head_dim", "ffn")
+
+    @staticmethod
+    def build(layer, half, device):
+        plan = _DecodePlan()
+        plan.ok, plan.half, plan.device, plan.sources = False, half, device, []
+        at = layer.self_attn
+        plan.modules = (at, at.q_proj, at.k_proj, at.v_proj, at.out_proj, at.qk_bmm, at.pv_bmm, layer.fc1, layer.fc2,
+                        layer.self_attn_layer_norm, layer.final_layer_norm)
+        stock = (type(at.q_proj) is W8A8B8O8Linear and type(at.k_proj) is W8A8B8O8Linear
+                 and type(at.v_proj) is W8A8B8O8Linear and type(at.out_proj) is W8A8BFP32OFP32Linear
+                 and type(layer.fc1) is W8A8B8O8LinearReLU and type(layer.fc2) is W8A8BFP32OFP32Linear
+                 and type(at.qk_bmm) is BMM_S8T_S8N_F32T and type(at.pv_bmm) is BMM_S8T_S8N_S8T
+                 and type(layer.self_attn_layer_norm) is LayerNormQ and type(layer.final_layer_norm) is LayerNormQ)
+        if not stock:
+            return plan
+        E, H, d, F = at.embed_dim, at.num_heads, at.head_dim, layer.fc1.out_features
+        fdt = torch.float16 if half else torch.float32
+
+        def tensor(mod, name, dtype, numel):
+            holder = mod._buffers if mod._buffers.get(name) is not None else mod._parameters
+            t = holder.get(name)
+            if not (isinstance(t, torch.Tensor) and t.device == device and t.dtype is dtype and t.is_contiguous()
+                    and t.numel() == numel and t.data_ptr() % 16 == 0):
+                raise _NotStock
+            plan.sources.append((holder, name, t, t._version))
+            return t.data_ptr()
+
+        def scalar(mod, name):
+            value = mod._scalar(name)
+            t = mod._buffers.get(name)
+            if isinstance(t, torch.Tensor):
+                plan.sources.append((mod._buffers, name, t, t._version))
+            else:
+                raise _NotStock   # a scale that is not a registered buffer cannot be watched
+            return value
+
+        try:
+            for lin in (at.out_proj, layer.fc2):   # their fp32 bias may still be in the dtype a cast left (see _run)
+                _, bias = lin._wb()
+                if bias.dtype is not torch.float32:
+                    lin.bias = bias.to(torch.float32)
+            st = _hip_ext.OptDecodeLayer()
+            st.embed, st.heads, st.head_dim, st.ffn, st.half = E, H, d, F, int(half)
+            ln1, ln2 = layer.self_attn_layer_norm, layer.final_layer_norm
+            st.ln1_eps, st.ln2_eps = float(ln1.eps), float(ln2.eps)
+            st.ln1_gamma, st.ln1_beta = tensor(ln1, "weight", fdt, E), tensor(ln1, "bias", fdt, E)
+            st.ln2_gamma, st.ln2_beta = tensor(ln2, "weight", fdt, E), tensor(ln2, "bias", fdt, E)
+            st.wq, st.wk, st.wv = (tensor(m, "weight", torch.int8, E * E) for m in (at.q_proj, at.k_proj, at.v_proj))
+            st.bq, st.bk, st.bv = (tensor(m, "bias", torch.int8, E) for m in (at.q_proj, at.k_proj, at.v_proj))
+            st.alpha_q, st.alpha_k, st.alpha_v = (scalar(m, "a") for m in (at.q_proj, at.k_proj, at.v_proj))
+            st.beta_q, st.beta_k, st.beta_v = (scalar(m, "b") for m in (at.q_proj, at.k_proj, at.v_proj))
+            st.alpha_qk, st.alpha_pv = scalar(at.qk_bmm, "a"), scalar(at.pv_bmm, "a")
+            st.wo, st.bo = tensor(at.out_proj, "weight", torch.int8, E * E), tensor(at.out_proj, "bias", torch.float32, E)
+            st.alpha_o = scalar(at.out_proj, "a")
+            st.w1, st.b1 = tensor(layer.fc1, "weight", torch.int8, F * E), tensor(layer.fc1, "bias", torch.int8, F)
+            st.alpha_1, st.beta_1 = scalar(layer.fc1, "a"), scalar(layer.fc1, "b")
+            st.w2, st.b2 = tensor(layer.fc2, "weight", torch.int8, E * F), tensor(layer.fc2, "bias", torch.float32, E)
+            st.alpha_2 = scalar(layer.fc2, "a")
+        except _NotStock:
+            return plan
+        if H * d != E or at.q_proj.in_features != E or layer.fc2.in_features != F:
+            return plan
+        plan.struct, plan.addr = st, ctypes.addressof(st)
+        plan.embed, plan.heads, plan.head_dim, plan.ffn = E, H, d, F
+        plan.ok = True
+        return plan
+
+
+class _NotStock(Exception):
+    pass
+
+
+_GLOBAL_FORWARD_HOOKS = torch.nn.modules.module._global_forward_hooks
+_GLOBAL_FORWARD_PRE_HOOKS = torch.nn.modules.module._global_forward_pre_hooks
+
+
 class Int8OPTDecoderLayer(nn.Module):
     """Pre-LN OPT block on an fp residual stream: LayerNormQ -> int8 attention -> add ->
     LayerNormQ -> fc1 (ReLU, int8) -> fc2 (fp32) -> add.  The input tensor is updated in
@@ -372,6 +464,76 @@ class Int8OPTDecoderLayer(nn.Module):
         q.fc2 = W8A8BFP32OFP32Linear.from_float(module.fc2, fc2_input_scale)
         return q
 
+    #: one new token per sequence with a KV cache: the layer's kernels are issued from one C call
+    #: (``ti_opt_decoder_layer_decode``: the same entry points with the same arguments, so the same values) instead of
+    #: one Python call per module; set to False to go through the modules
+    decode_in_one_call = True
+
+    def _decode_plan(self, half, device):
+        """The layer as ``ti_opt_decoder_layer_decode`` reads it, built once and rebuilt when a tensor it was built from
+        has been replaced or written to; None when the layer is not the stock int8 block on ``device``."""
+        plan = self.__dict__.get("_ti_decode_plan")
+        if plan is not None and plan.half == half and plan.device == device:
+            for holder, name, tensor, version in plan.sources:
+                if holder.get(name) is not tensor or tensor._version != version:
+                    plan = None
+                    break
+        else:
+            plan = None
+        if plan is None:
+            plan = self.__dict__["_ti_decode_plan"] = _DecodePlan.build(self, half, device)
+        if not plan.ok or _GLOBAL_FORWARD_HOOKS or _GLOBAL_FORWARD_PRE_HOOKS:
+            return None
+        for mod in plan.modules:   # a hook on a sub-module wants to see that module's call
+            if mod._forward_hooks or mod._forward_pre_hooks:
+                return None
+        return plan
+
+    def _decode_in_one_call(self, hidden_states, attention_mask, past_key_value, use_cache):
+        """``forward`` for one new token per sequence over a KV cache, or None when the tensors do not qualify."""
+        hs = hidden_states
+        dtype = hs.dtype
+        if not (hs.is_cuda and hs.is_contiguous() and hs.shape[0] <= 16
+                and (dtype is torch.float32 or dtype is torch.float16)):
+            return None
+        past_k, past_v = past_key_value
+        bsz = hs.shape[0]
+        if not (past_k.dim() == 4 and past_v.shape == past_k.shape and past_k.dtype is torch.int8
+                and past_v.dtype is torch.int8 and past_k.device == hs.device and past_v.device == hs.device
+                and past_k.shape[0] == bsz):
+            return None
+        plan = self._decode_plan(dtype is torch.float16, hs.device)
+        if plan is None or past_k.shape[1] != plan.heads or past_k.shape[3] != plan.head_dim or hs.shape[2] != plan.embed:
+            return None
+        S = past_k.shape[2] + 1
+        if not _hip_ext.decode_attention_shape_ok_cached(1, S, plan.head_dim):
+            return None
+        mask = attention_mask
+        if mask is not None:
+            if not mask.is_cuda:
+                return None
+            if mask.dtype is torch.float16 or mask.dtype is torch.bfloat16:
+                # the mask of an fp16 model is only ever added to fp32 scores (see Int8OPTAttention.forward); converted
+                # once per mask tensor, not once per layer
+                m32 = getattr(mask, "_ti_f32", None)
+                if m32 is None or m32[0] != mask._version:
+                    m32 = (mask._version, mask.float())
+                    mask._ti_f32 = m32
+                mask = m32[1]
+            if not (mask.dtype is torch.float32 and mask.is_contiguous() and mask.shape == (bsz, 1, 1, S)
+                    and mask.device == hs.device):
+                return None
+        kk = _kv_room_for(past_k, 1) or _kv_fresh(past_k, 1)
+        vv = _kv_room_for(past_v, 1) or _kv_fresh(past_v, 1)
+        if kk.buf.data_ptr() % 16 or vv.buf.data_ptr() % 16 or not (kk.buf.is_contiguous() and vv.buf.is_contiguous()
+                                                                    and kk.buf.shape == vv.buf.shape):
+            return None
+        _hip_ext.opt_layer_decode(plan, hs, mask, kk.buf, vv.buf, S)
+        kk.filled = vv.filled = S
+        if use_cache:
+            return hs, (_kv_view(kk, S), _kv_view(vv, S))
+        return (hs,)
+
     def decode_step_devlen(self, hidden_states, k_buf, v_buf, length, max_length):
         """``forward`` for one new token per sequence with the cache length read on the device (see
         ``Int8OPTAttention.decode_step_devlen``): updates ``hidden_states`` in place and appends to the cache."""
@@ -390,6 +552,12 @@ class Int8OPTDecoderLayer(nn.Module):
                 layer_head_mask: Optional[torch.Tensor] = None, output_attentions: Optional[bool] = False,
                 use_cache: Optional[bool] = False, past_key_value: Optional[Tuple[torch.Tensor]] = None):
         """hidden_states: fp [batch, time, embed_dim] residual stream -> tuple starting with it."""
+        if (past_key_value is not None and self.decode_in_one_call and hidden_states.dim() == 3
+                and hidden_states.shape[1] == 1 and layer_head_mask is None and not output_attentions
+                and self.self_attn.kv_cache_in_place and self.self_attn.fused_softmax):
+            out = self._decode_in_one_call(hidden_states, attention_mask, past_key_value, use_cache)
+            if out is not None:
+                return out
         residual = hidden_states
         x = self.self_attn_layer_norm(hidden_states)
         x, attn_weights, present = self.self_attn(
