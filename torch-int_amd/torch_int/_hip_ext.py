@@ -566,7 +566,9 @@ def opt_layer_decode(plan, hidden, mask, k_buf, v_buf, S):
             if len(_decode_scratch) >= 64:
                 _decode_scratch.clear()
             n = _lib.ti_opt_decoder_layer_decode_scratch_bytes(B, plan.embed, plan.ffn)
-            scratch = _decode_scratch[key] = torch.empty(n, dtype=torch.uint8, device=dev)
+            scratch = torch.empty(n, dtype=torch.uint8, device=dev)
+            if not torch.cuda.is_current_stream_capturing():   # memory from a capture's pool belongs to that graph
+                _decode_scratch[key] = scratch
         if _fast_opt_layer_decode is not None:
             rc = _fast_opt_layer_decode(plan.addr, hidden.data_ptr(),
                                         mask.data_ptr() if mask is not None else 0, k_buf.data_ptr(), v_buf.data_ptr(),
