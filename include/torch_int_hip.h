@@ -465,6 +465,23 @@ int ti_opt_decoder_layer_decode(const TiOptDecodeLayer* layer, void* hidden, con
                                 int8_t* v_buf, int64_t B, int64_t cap, int64_t S, void* scratch, int64_t scratch_bytes,
                                 void* stream);
 
+/* The same for a prefill (Int8OPTDecoderLayer.forward, torch_int/models/opt.py:202-299, on T > 16 tokens per sequence
+ * without a cache): LayerNormQ, the q/k/v projections stored head-major (one grouped launch where
+ * ti_linear_group_is_one_launch says so, else three calls with the workspace), V transposed, the one-launch prefill
+ * attention with the head merge (ti_attn_prefill_s8_mc), out_proj, the residual update fused with the second
+ * LayerNormQ, fc1 (ReLU), fc2 added into the residual stream -- the entry points and arguments of the module path, so
+ * its values.  hidden [B, T, embed] is updated in place; mask fp32 [B, 1, T, T] or NULL, mask_classes its class array
+ * (ti_attn_mask_classes) or NULL; k_out / v_out receive the key and value rows [B, heads, T, head_dim] (the cache the
+ * decode steps continue).  T a multiple of 16 that ti_attn_prefill_supported(T, T, head_dim) accepts, B * T <= 4096
+ * (larger prefills are bound by their kernels, not by the host).  scratch:
+ * ti_opt_decoder_layer_prefill_scratch_bytes(B * T, embed, ffn) bytes on a 256-byte boundary; workspace: the split-K
+ * workspace of the linears (ti_linear_workspace_bytes of the largest of them, or NULL). */
+int64_t ti_opt_decoder_layer_prefill_scratch_bytes(int64_t rows, int64_t embed, int64_t ffn);
+int ti_opt_decoder_layer_prefill(const TiOptDecodeLayer* layer, void* hidden, const float* mask,
+                                 const uint8_t* mask_classes, int8_t* k_out, int8_t* v_out, int64_t B, int64_t T,
+                                 void* scratch, int64_t scratch_bytes, void* workspace, int64_t workspace_bytes,
+                                 void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -181,6 +181,22 @@ def test_c_abi_rejects_bad_arguments_without_a_device():
     assert b"heads * head_dim" in lib.ti_last_error()
     st.head_dim = 64
     assert lib.ti_opt_decoder_layer_decode(ctypes.addressof(st), None, None, None, None, 0, 64, 10, None, 0, None) == 0
+    # ... and a short prefill: token limit, key counts the attention takes, scratch size
+    need = lib.ti_opt_decoder_layer_prefill_scratch_bytes(64, 256, 1024)
+    assert need == 4 * 64 * 256 + 4 * 64 * 256 + 64 * 1024
+    adr = ctypes.addressof(st)
+    p16 = (ctypes.addressof(big) + 15) // 16 * 16
+    # (arguments that pass: the first step then refuses the description's missing LayerNorm parameters, before any device call)
+    assert lib.ti_opt_decoder_layer_prefill(adr, p, None, None, p16, p16, 2, 32, pa, need, None, 0, None) == 1
+    assert b"gamma is NULL" in lib.ti_last_error()
+    assert lib.ti_opt_decoder_layer_prefill(adr, p, None, None, p16, p16, 8, 1024, pa, need, None, 0, None) == 1
+    assert b"4096 tokens" in lib.ti_last_error()
+    assert lib.ti_opt_decoder_layer_prefill(adr, p, None, None, p16, p16, 2, 40, pa, need, None, 0, None) == 1
+    assert b"multiple of 16" in lib.ti_last_error()
+    assert lib.ti_opt_decoder_layer_prefill(adr, p, None, None, p16, p16, 2, 32, pa, need - 1, None, 0, None) == 1
+    assert b"scratch" in lib.ti_last_error()
+    assert lib.ti_opt_decoder_layer_prefill(None, p, None, None, p16, p16, 2, 32, pa, need, None, 0, None) == 1
+    assert lib.ti_opt_decoder_layer_prefill(adr, None, None, None, None, None, 0, 32, None, 0, None, 0, None) == 0
     # empty problems succeed without touching pointers or a device
     assert lib.ti_linear_a8_w8_b8_o8(None, None, None, None, 0, 16, 16, 1.0, 1.0, None, 0, None) == 0
     assert lib.ti_dq_add_layernorm_q(None, 1.0, None, None, None, 1e-5, None, None, 0, 128, None) == 0

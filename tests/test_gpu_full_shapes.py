@@ -417,14 +417,14 @@ class _Tap:
             wrap(C, n)
         for n in self.X_NAMES:
             wrap(X, n)
-        # a decode step normally issues a layer's kernels from one C call; the tap is there to see them one by one
+        # a layer normally issues the kernels of a decode step or a short prefill from one C call; the tap is there to see them one by one
         from torch_int.models.opt import Int8OPTDecoderLayer
-        one_call = Int8OPTDecoderLayer.decode_in_one_call
-        Int8OPTDecoderLayer.decode_in_one_call = False
+        one_call = Int8OPTDecoderLayer.decode_in_one_call, Int8OPTDecoderLayer.prefill_in_one_call
+        Int8OPTDecoderLayer.decode_in_one_call = Int8OPTDecoderLayer.prefill_in_one_call = False
         try:
             yield self
         finally:
-            Int8OPTDecoderLayer.decode_in_one_call = one_call
+            Int8OPTDecoderLayer.decode_in_one_call, Int8OPTDecoderLayer.prefill_in_one_call = one_call
             for mod, name, fn in saved:
                 setattr(mod, name, fn)
 

@@ -274,12 +274,16 @@ def test_fp16_model_runs_the_fused_kernels_and_follows_the_torch_chain():
     glm = copy.deepcopy(lm).to(DEV).half()
     assert glm.model.decoder.layers[0].fc2.bias.dtype == torch.float32       # upstream keeps this bias in fp32
     assert glm.model.decoder.layers[0].final_layer_norm.weight.dtype == torch.float16
-    calls = {"ln": 0, "add": 0, "one": 0}
-    real_ln, real_add, real_one = X.add_layernorm_q, X.add_rounded_, X.opt_layer_decode
+    calls = {"ln": 0, "add": 0, "one": 0, "pre": 0}
+    real_ln, real_add, real_one, real_pre = X.add_layernorm_q, X.add_rounded_, X.opt_layer_decode, X.opt_layer_prefill
 
     def count_one(plan, hidden, *a, **k):
         calls["one"] += plan.half and hidden.dtype is torch.float16
         return real_one(plan, hidden, *a, **k)
+
+    def count_pre(plan, hidden, *a, **k):
+        calls["pre"] += plan.half and hidden.dtype is torch.float16
+        return real_pre(plan, hidden, *a, **k)
 
     def count_ln(x, residual, *a, **k):
         calls["ln"] += residual.dtype is torch.float16
@@ -288,16 +292,24 @@ def test_fp16_model_runs_the_fused_kernels_and_follows_the_torch_chain():
     def count_add(residual, x):
         calls["add"] += 1
         return real_add(residual, x)
-    X.add_layernorm_q, X.add_rounded_, X.opt_layer_decode = count_ln, count_add, count_one
+    X.add_layernorm_q, X.add_rounded_, X.opt_layer_decode, X.opt_layer_prefill = count_ln, count_add, count_one, count_pre
+    Layer = type(glm.model.decoder.layers[0])
     try:
         _say("fp16 causal LM, fused")
         out = glm(ids, use_cache=True)
         step = glm(ids[:, -1:], past_key_values=out.past_key_values, use_cache=True)
+        # prefill and decode step each went through one call per layer that issues the fp16 kernels
+        assert out.logits.dtype == torch.float16 and calls == {"ln": 0, "add": 0, "one": 3, "pre": 3}, calls
+        # through the modules: two LayerNorm-quantisers and one rounded add per layer and forward, on the fp16 stream,
+        # and the same logits bit for bit
+        Layer.prefill_in_one_call = Layer.decode_in_one_call = False
+        out_m = glm(ids, use_cache=True)
+        step_m = glm(ids[:, -1:], past_key_values=out_m.past_key_values, use_cache=True)
+        assert calls == {"ln": 2 * 3 * 2, "add": 3 * 2, "one": 3, "pre": 3}, calls
+        assert torch.equal(out.logits, out_m.logits) and torch.equal(step.logits, step_m.logits)
     finally:
-        X.add_layernorm_q, X.add_rounded_, X.opt_layer_decode = real_ln, real_add, real_one
-    # the prefill goes through the modules (two LayerNorm-quantisers and one rounded add per layer), the decode step
-    # through one call per layer that issues the same fp16 kernels
-    assert out.logits.dtype == torch.float16 and calls["ln"] == 2 * 3 and calls["add"] == 3 and calls["one"] == 3, calls
+        X.add_layernorm_q, X.add_rounded_, X.opt_layer_decode, X.opt_layer_prefill = real_ln, real_add, real_one, real_pre
+        Layer.prefill_in_one_call = Layer.decode_in_one_call = True
     real_can = X.can_fuse_layernorm
     X.can_fuse_layernorm = lambda x, w, b: False
     X.add_rounded_ = lambda residual, x: residual.add_(x.to(residual.dtype))
@@ -433,6 +445,7 @@ def test_prefill_attention_at_head_sizes_between_the_lane_layouts(D, H, T):
     import torch_int._hip_ext as X
     g = torch.Generator().manual_seed(D + H)
     layer = randomize_int8_layer(Int8OPTDecoderLayer(D, H, 2 * D), g).to(DEV)
+    layer.prefill_in_one_call = False   # through the modules: this test counts their calls (the one-call form has its own)
     B = 2
     hidden = torch.randn(B, T, D, generator=g).to(DEV)
     mask = causal_mask(B, T, T).to(DEV)
@@ -519,3 +532,58 @@ def test_decode_step_from_one_call_gives_the_modules_values(D, H, bsz, half):
 def _hip_ext_mod():
     import torch_int._hip_ext as X
     return X
+
+
+@torch.no_grad()
+@pytest.mark.parametrize("half", [False, True])
+@pytest.mark.parametrize("D,H,bsz,T", [(256, 4, 2, 48), (320, 4, 3, 112), (512, 4, 1, 528), (256, 4, 2, 592),
+                                       (1024, 8, 4, 512), (256, 2, 1, 32), (5120, 40, 1, 128)])
+def test_prefill_from_one_call_gives_the_modules_values(D, H, bsz, T, half):
+    """A prefill of up to 4096 tokens: the layer issues its kernels from one C call (ti_opt_decoder_layer_prefill).
+    Residual stream and key / value rows bit for bit those of the same layer going through its modules: grouped or
+    separate head-major projections (with the split-K workspace), single-sweep and three-sweep attention with mask
+    classes, head sizes 64 / 80 / 128, causal and padded masks and none, fp32 and fp16 streams."""
+    X = _hip_ext_mod()
+    g = torch.Generator().manual_seed(3 * D + T)
+    layer = randomize_int8_layer(Int8OPTDecoderLayer(D, H, 4 * D), g).to(DEV)
+    if half:
+        layer = layer.half()
+    dt = torch.float16 if half else torch.float32
+    hidden = torch.randn(bsz, T, D, generator=g).to(DEV).to(dt)
+    seen = []
+    real = X.opt_layer_prefill
+
+    def counted(*a, **kw):
+        seen.append(a[1].shape)
+        return real(*a, **kw)
+    X.opt_layer_prefill = counted
+    try:
+        for kind in ("causal", "pad", None):
+            mask = None
+            if kind is not None:
+                mask = causal_mask(bsz, T, T).to(DEV)
+                if kind == "pad":
+                    mask[bsz - 1, :, :, :5] = torch.finfo(torch.float32).min
+                if half:
+                    mask = mask.to(dt)
+            res = {}
+            for one_call in (True, False):
+                layer.prefill_in_one_call = one_call
+                res[one_call] = layer(hidden.clone(), attention_mask=mask, use_cache=True)
+            assert torch.equal(res[True][0], res[False][0]), (kind, (res[True][0] != res[False][0]).sum().item())
+            for a, b in zip(res[True][1], res[False][1]):
+                assert a.shape == b.shape == (bsz, H, T, D // H) and torch.equal(a, b), kind
+            # and a decode step continues from either cache alike
+            x = torch.randn(bsz, 1, D, generator=g).to(DEV).to(dt)
+            nxt = [layer(x.clone(), past_key_value=res[oc][1], use_cache=True)[0] for oc in (True, False)]
+            assert torch.equal(nxt[0], nxt[1]), kind
+        assert len(seen) == 3, seen
+        layer.prefill_in_one_call = True
+        handle = layer.self_attn.out_proj.register_forward_pre_hook(lambda mod, inp: None)
+        layer(hidden.clone(), attention_mask=None, use_cache=True)
+        handle.remove()
+        assert len(seen) == 3                                        # the hook saw out_proj being called instead
+    finally:
+        X.opt_layer_prefill = real
+        if "prefill_in_one_call" in layer.__dict__:
+            del layer.prefill_in_one_call

@@ -793,4 +793,95 @@ int ti_opt_decoder_layer_decode(const TiOptDecodeLayer* L, void* hidden, const f
                                          stream);
 }
 
+// One decoder layer of a prefill (no cache yet): the launches an Int8OPTDecoderLayer makes for T > 16 tokens per
+// sequence when its attention takes the one-launch prefill kernel, issued from one C call through the public entry
+// points, with the arguments the modules pass.
+int64_t ti_opt_decoder_layer_prefill_scratch_bytes(int64_t rows, int64_t embed, int64_t ffn) {
+  if (rows <= 0 || embed <= 0 || ffn <= 0) return 0;
+  auto up = [](int64_t n) { return (n + 255) / 256 * 256; };
+  return 4 * up(rows * embed) + up(4 * rows * embed) + up(rows * ffn);
+}
+
+int ti_opt_decoder_layer_prefill(const TiOptDecodeLayer* L, void* hidden, const float* mask, const uint8_t* mask_classes,
+                                 int8_t* k_out, int8_t* v_out, int64_t B, int64_t T, void* scratch, int64_t scratch_bytes,
+                                 void* workspace, int64_t workspace_bytes, void* stream) {
+  g_err[0] = 0;
+  const char* op = "opt_decoder_layer_prefill";
+  if (L == nullptr) return fail(TI_ERR_INVALID_ARG, "%s: no layer description", op);
+  const int64_t E = L->embed, H = L->heads, d = L->head_dim, F = L->ffn;
+  if (E <= 0 || H <= 0 || d <= 0 || F <= 0 || H * d != E)
+    return fail(TI_ERR_INVALID_ARG, "%s: needs embed = heads * head_dim > 0 and ffn > 0 (got %lld, %lld x %lld, %lld)", op,
+                (long long)E, (long long)H, (long long)d, (long long)F);
+  if (B < 0 || T < 0 || B > 65535 || T > 4096) return fail(TI_ERR_INVALID_ARG, "%s: needs 0 <= B <= 65535, 0 <= T <= 4096", op);
+  const int64_t M = B * T;
+  if (M == 0) return TI_OK;
+  if (M > 4096) return fail(TI_ERR_INVALID_ARG, "%s: up to 4096 tokens in all (got %lld x %lld)", op, (long long)B, (long long)T);
+  if (!attn_prefill_supported(T, T, d))
+    return fail(TI_ERR_INVALID_ARG, "%s: %lld tokens per sequence at head size %lld: needs a multiple of 16 up to 4096 and a "
+                "head size that is a multiple of 16 up to 128", op, (long long)T, (long long)d);
+  if (int rc = check_ptr(op, "hidden", hidden, L->half ? 2 : 4, true)) return rc;
+  if (int rc = check_ptr(op, "k_out", k_out, 16, true)) return rc;
+  if (int rc = check_ptr(op, "v_out", v_out, 16, true)) return rc;
+  if (int rc = check_ptr(op, "scratch", scratch, 256, true)) return rc;
+  if (scratch_bytes < ti_opt_decoder_layer_prefill_scratch_bytes(M, E, F))
+    return fail(TI_ERR_INVALID_ARG, "%s: scratch of %lld bytes, needs %lld", op, (long long)scratch_bytes,
+                (long long)ti_opt_decoder_layer_prefill_scratch_bytes(M, E, F));
+  auto up = [](int64_t n) { return (n + 255) / 256 * 256; };
+  char* at = static_cast<char*>(scratch);
+  auto take = [&](int64_t bytes) {
+    char* r = at;
+    at += up(bytes);
+    return r;
+  };
+  int8_t* x = reinterpret_cast<int8_t*>(take(M * E));     // LayerNorm-quantised input of the projections, then of fc1
+  int8_t* q = reinterpret_cast<int8_t*>(take(M * E));     // [B, heads, T, head_dim]
+  int8_t* vt = reinterpret_cast<int8_t*>(take(M * E));    // [B * heads, head_dim, T]
+  int8_t* ctx = reinterpret_cast<int8_t*>(take(M * E));   // [B, T, embed]
+  float* f32 = reinterpret_cast<float*>(take(4 * M * E)); // output of out_proj, then (fp16 stream) of fc2
+  int8_t* h = reinterpret_cast<int8_t*>(take(M * F));
+  int rc;
+  rc = L->half ? ti_add_layernorm_q_f16(nullptr, hidden, L->ln1_gamma, L->ln1_beta, L->ln1_eps, x, M, E, stream)
+               : ti_add_layernorm_q(nullptr, static_cast<float*>(hidden), static_cast<const float*>(L->ln1_gamma),
+                                    static_cast<const float*>(L->ln1_beta), L->ln1_eps, x, M, E, stream);
+  if (rc) return rc;
+  // q, k, v stored head-major by the projections themselves: one grouped launch where the library has one, else one
+  // call per projection with the split-K workspace (the choice the attention module makes)
+  const int8_t* w3[3] = {L->wq, L->wk, L->wv};
+  const int8_t* b3[3] = {L->bq, L->bk, L->bv};
+  int8_t* o3[3] = {q, k_out, v_out};
+  const float a3[3] = {L->alpha_q, L->alpha_k, L->alpha_v};
+  const float be3[3] = {L->beta_q, L->beta_k, L->beta_v};
+  if (ti_linear_group_is_one_launch(M, E, E, 3)) {
+    if ((rc = ti_linear_a8_w8_b8_o8_group_heads(x, w3, b3, o3, a3, be3, 3, M, E, E, T, d, stream))) return rc;
+  } else {
+    for (int i = 0; i < 3; ++i)
+      if ((rc = ti_linear_a8_w8_b8_o8_heads(x, w3[i], b3[i], o3[i], M, E, E, a3[i], be3[i], T, d, workspace,
+                                             workspace_bytes, stream)))
+        return rc;
+  }
+  // V transposed, then the whole attention with the head merge
+  if ((rc = ti_transpose_last2_s8(v_out, vt, B * H, T, d, stream))) return rc;
+  if ((rc = ti_attn_prefill_s8_mc(q, k_out, vt, mask, mask_classes, ctx, B * H, T, T, d, T * d, T * d, H, L->alpha_qk,
+                                  L->alpha_pv, stream)))
+    return rc;
+  if ((rc = ti_linear_a8_w8_bfp32_ofp32(ctx, L->wo, L->bo, f32, M, E, E, L->alpha_o, 1.0f, workspace, workspace_bytes,
+                                        stream)))
+    return rc;
+  rc = L->half ? ti_add_layernorm_q_f16_xf32(f32, hidden, L->ln2_gamma, L->ln2_beta, L->ln2_eps, x, M, E, stream)
+               : ti_add_layernorm_q(f32, static_cast<float*>(hidden), static_cast<const float*>(L->ln2_gamma),
+                                    static_cast<const float*>(L->ln2_beta), L->ln2_eps, x, M, E, stream);
+  if (rc) return rc;
+  if ((rc = ti_linear_relu_a8_w8_b8_o8(x, L->w1, L->b1, h, M, F, E, L->alpha_1, L->beta_1, workspace, workspace_bytes,
+                                       stream)))
+    return rc;
+  if (L->half) {
+    if ((rc = ti_linear_a8_w8_bfp32_ofp32(h, L->w2, L->b2, f32, M, E, F, L->alpha_2, 1.0f, workspace, workspace_bytes,
+                                          stream)))
+      return rc;
+    return ti_add_f16_xf32(f32, hidden, M * E, stream);
+  }
+  return ti_linear_a8_w8_bfp32_ofp32_acc(h, L->w2, L->b2, static_cast<float*>(hidden), M, E, F, L->alpha_2, 1.0f, workspace,
+                                         workspace_bytes, stream);
+}
+
 }  // extern "C"

@@ -214,6 +214,26 @@ static PyObject* fc_opt_layer_decode(PyObject* self, PyObject* const* a, Py_ssiz
                                                      cap, S, scratch, sb, st));
 }
 
+/* opt_layer_prefill(layer, hidden, mask, classes, k_out, v_out, B, T, scratch, scratch_bytes, ws, ws_bytes, stream) -> status */
+static PyObject* fc_opt_layer_prefill(PyObject* self, PyObject* const* a, Py_ssize_t n) {
+  (void)self;
+  if (n != 13) {
+    PyErr_SetString(PyExc_TypeError, "opt_layer_prefill expects 13 arguments");
+    return NULL;
+  }
+  void *layer = as_ptr(a[0]), *hidden = as_ptr(a[1]), *mask = as_ptr(a[2]), *cls = as_ptr(a[3]);
+  void *ko = as_ptr(a[4]), *vo = as_ptr(a[5]);
+  int64_t B = as_i64(a[6]), T = as_i64(a[7]);
+  void* scratch = as_ptr(a[8]);
+  int64_t sb = as_i64(a[9]);
+  void* ws = as_ptr(a[10]);
+  int64_t wsb = as_i64(a[11]);
+  void* st = as_ptr(a[12]);
+  if (PyErr_Occurred()) return NULL;
+  return PyLong_FromLong(ti_opt_decoder_layer_prefill((const TiOptDecodeLayer*)layer, hidden, (const float*)mask,
+                                                      (const uint8_t*)cls, ko, vo, B, T, scratch, sb, ws, wsb, st));
+}
+
 static PyObject* fc_last_error(PyObject* self, PyObject* noargs) {
   (void)self;
   (void)noargs;
@@ -232,6 +252,7 @@ static PyMethodDef methods[] = {
     {"kv_append", (PyCFunction)(void (*)(void))fc_kv_append, METH_FASTCALL, "forward to ti_kv_append_s8"},
     {"decode_attn", (PyCFunction)(void (*)(void))fc_decode_attn, METH_FASTCALL, "forward to ti_decode_attn_s8"},
     {"opt_layer_decode", (PyCFunction)(void (*)(void))fc_opt_layer_decode, METH_FASTCALL, "forward to ti_opt_decoder_layer_decode"},
+    {"opt_layer_prefill", (PyCFunction)(void (*)(void))fc_opt_layer_prefill, METH_FASTCALL, "forward to ti_opt_decoder_layer_prefill"},
     {"last_error", fc_last_error, METH_NOARGS, "ti_last_error()"},
     {NULL, NULL, 0, NULL}};
 

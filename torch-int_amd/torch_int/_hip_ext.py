@@ -109,8 +109,13 @@ _lib.ti_opt_decoder_layer_decode_scratch_bytes.argtypes = [_i64, _i64, _i64]
 _lib.ti_opt_decoder_layer_decode_scratch_bytes.restype = _i64
 _lib.ti_opt_decoder_layer_decode.argtypes = [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _i64, _vp]
 _lib.ti_opt_decoder_layer_decode.restype = ctypes.c_int
+_lib.ti_opt_decoder_layer_prefill_scratch_bytes.argtypes = [_i64, _i64, _i64]
+_lib.ti_opt_decoder_layer_prefill_scratch_bytes.restype = _i64
+_lib.ti_opt_decoder_layer_prefill.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp, _i64, _vp, _i64, _vp]
+_lib.ti_opt_decoder_layer_prefill.restype = ctypes.c_int
 _raw_stream = torch._C._cuda_getCurrentRawStream
 _fast_opt_layer_decode = getattr(_CUDA._fast, "opt_layer_decode", None)
+_fast_opt_layer_prefill = getattr(_CUDA._fast, "opt_layer_prefill", None)
 _fast = _CUDA._fast if getattr(_CUDA._fast, "kv_append", None) is not None else None
 _fast_decode_attn = getattr(_CUDA._fast, "decode_attn", None)
 _fast_group3 = getattr(_CUDA._fast, "linear_group3", None)
@@ -546,7 +551,38 @@ def decode_attention_shape_ok_cached(T, S, d):
     return ok
 
 
-_decode_scratch = {}
+_attn_prefill_ok = {}
+
+
+def attn_prefill_shape_ok_cached(T, S, d):
+    """``attn_prefill_shape_ok`` remembered per shape."""
+    key = (T, S, d)
+    ok = _attn_prefill_ok.get(key)
+    if ok is None:
+        if len(_attn_prefill_ok) > 65536:
+            _attn_prefill_ok.clear()
+        ok = _attn_prefill_ok[key] = bool(_lib.ti_attn_prefill_supported(T, S, d))
+    return ok
+
+
+_layer_scratch = {}   # (device, stream) -> uint8 tensor: the intermediate tensors of a layer issued from one C call
+
+
+def _scratch_for(dev, stream, nbytes):
+    """One buffer per device and stream, grown on demand and shared by every layer (calls on one stream run one
+    after the other).  Memory allocated while the stream is capturing belongs to that graph's pool and is not kept."""
+    key = (dev.index, stream)
+    buf = _layer_scratch.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(int(nbytes), dtype=torch.uint8, device=dev)
+        if not torch.cuda.is_current_stream_capturing():
+            if len(_layer_scratch) >= 64:
+                _layer_scratch.clear()
+            _layer_scratch[key] = buf
+    return buf
+
+
+_layer_scratch_need = {}
 
 
 def opt_layer_decode(plan, hidden, mask, k_buf, v_buf, S):
@@ -560,15 +596,11 @@ def opt_layer_decode(plan, hidden, mask, k_buf, v_buf, S):
     B = hidden.shape[0]
     with _on(dev):
         stream = _raw_stream(dev.index)
-        key = (dev.index, stream, B, plan.embed, plan.ffn)
-        scratch = _decode_scratch.get(key)
-        if scratch is None:
-            if len(_decode_scratch) >= 64:
-                _decode_scratch.clear()
-            n = _lib.ti_opt_decoder_layer_decode_scratch_bytes(B, plan.embed, plan.ffn)
-            scratch = torch.empty(n, dtype=torch.uint8, device=dev)
-            if not torch.cuda.is_current_stream_capturing():   # memory from a capture's pool belongs to that graph
-                _decode_scratch[key] = scratch
+        key = (0, B, plan.embed, plan.ffn)
+        need = _layer_scratch_need.get(key)
+        if need is None:
+            need = _layer_scratch_need[key] = _lib.ti_opt_decoder_layer_decode_scratch_bytes(B, plan.embed, plan.ffn)
+        scratch = _scratch_for(dev, stream, need)
         if _fast_opt_layer_decode is not None:
             rc = _fast_opt_layer_decode(plan.addr, hidden.data_ptr(),
                                         mask.data_ptr() if mask is not None else 0, k_buf.data_ptr(), v_buf.data_ptr(),
@@ -580,6 +612,40 @@ def opt_layer_decode(plan, hidden, mask, k_buf, v_buf, S):
                                                   scratch.numel(), stream or None)
     if rc:
         raise RuntimeError(f"torch_int._hip_ext.opt_layer_decode: {_lib.ti_last_error().decode()} (status {rc})")
+    return hidden
+
+
+def opt_layer_prefill(plan, hidden, mask, k_out, v_out):
+    """A prefill through one decoder layer from one C call (``ti_opt_decoder_layer_prefill``): ``hidden`` [B, T, embed]
+    is updated in place, ``k_out`` / ``v_out`` (int8 [B, heads, T, head_dim], contiguous) receive the layer's key and
+    value rows.  ``plan`` as for ``opt_layer_decode``; the caller has checked shapes, dtypes, devices and contiguity."""
+    dev = hidden.device
+    B, T = hidden.shape[0], hidden.shape[1]
+    M, E, F = B * T, plan.embed, plan.ffn
+    with _on(dev):
+        stream = _raw_stream(dev.index)
+        key = (1, M, E, F)
+        need = _layer_scratch_need.get(key)
+        if need is None:
+            if len(_layer_scratch_need) > 4096:
+                _layer_scratch_need.clear()
+            need = _layer_scratch_need[key] = (
+                _lib.ti_opt_decoder_layer_prefill_scratch_bytes(M, E, F),
+                max(_CUDA._ws_bytes(M, E, E), _CUDA._ws_bytes(M, F, E), _CUDA._ws_bytes(M, E, F)))
+        scratch = _scratch_for(dev, stream, need[0])
+        ws_ptr, ws_bytes = _CUDA._workspace(dev.index, stream, need[1])
+        cls = _classes_ptr(mask, T) if mask is not None else None
+        if _fast_opt_layer_prefill is not None:
+            rc = _fast_opt_layer_prefill(plan.addr, hidden.data_ptr(), mask.data_ptr() if mask is not None else 0,
+                                         cls or 0, k_out.data_ptr(), v_out.data_ptr(), B, T, scratch.data_ptr(),
+                                         scratch.numel(), ws_ptr, ws_bytes, stream)
+        else:
+            rc = _lib.ti_opt_decoder_layer_prefill(plan.addr, hidden.data_ptr(),
+                                                   mask.data_ptr() if mask is not None else None, cls, k_out.data_ptr(),
+                                                   v_out.data_ptr(), B, T, scratch.data_ptr(), scratch.numel(),
+                                                   ws_ptr or None, ws_bytes, stream or None)
+    if rc:
+        raise RuntimeError(f"torch_int._hip_ext.opt_layer_prefill: {_lib.ti_last_error().decode()} (status {rc})")
     return hidden
 
 

@@ -433,6 +433,23 @@ class _NotStock(Exception):
     pass
 
 
+def _mask_as_fp32(mask):
+    """The additive mask as the fused kernels read it: fp32 on the device (None when it is neither that nor an fp16 /
+    bf16 HIP tensor).  The mask of an fp16 model is only ever added to fp32 scores (see ``Int8OPTAttention.forward``);
+    it is converted once per mask tensor and version, not once per layer."""
+    if not mask.is_cuda:
+        return None
+    if mask.dtype is torch.float32:
+        return mask
+    if mask.dtype is torch.float16 or mask.dtype is torch.bfloat16:
+        m32 = getattr(mask, "_ti_f32", None)
+        if m32 is None or m32[0] != mask._version:
+            m32 = (mask._version, mask.float())
+            mask._ti_f32 = m32
+        return m32[1]
+    return None
+
+
 _GLOBAL_FORWARD_HOOKS = torch.nn.modules.module._global_forward_hooks
 _GLOBAL_FORWARD_PRE_HOOKS = torch.nn.modules.module._global_forward_pre_hooks
 
@@ -510,18 +527,8 @@ class Int8OPTDecoderLayer(nn.Module):
             return None
         mask = attention_mask
         if mask is not None:
-            if not mask.is_cuda:
-                return None
-            if mask.dtype is torch.float16 or mask.dtype is torch.bfloat16:
-                # the mask of an fp16 model is only ever added to fp32 scores (see Int8OPTAttention.forward); converted
-                # once per mask tensor, not once per layer
-                m32 = getattr(mask, "_ti_f32", None)
-                if m32 is None or m32[0] != mask._version:
-                    m32 = (mask._version, mask.float())
-                    mask._ti_f32 = m32
-                mask = m32[1]
-            if not (mask.dtype is torch.float32 and mask.is_contiguous() and mask.shape == (bsz, 1, 1, S)
-                    and mask.device == hs.device):
+            mask = _mask_as_fp32(mask)
+            if not (mask is not None and mask.is_contiguous() and mask.shape == (bsz, 1, 1, S) and mask.device == hs.device):
                 return None
         kk = _kv_room_for(past_k, 1) or _kv_fresh(past_k, 1)
         vv = _kv_room_for(past_v, 1) or _kv_fresh(past_v, 1)
@@ -532,6 +539,34 @@ class Int8OPTDecoderLayer(nn.Module):
         kk.filled = vv.filled = S
         if use_cache:
             return hs, (_kv_view(kk, S), _kv_view(vv, S))
+        return (hs,)
+
+    #: a prefill of up to 4096 tokens in all (more than 16 per sequence, a multiple of 16): likewise one C call
+    #: (``ti_opt_decoder_layer_prefill``); at those sizes a layer's kernels take less time than eight trips through Python
+    prefill_in_one_call = True
+
+    def _prefill_in_one_call(self, hidden_states, attention_mask, use_cache):
+        """``forward`` without a cache on T > 16 tokens per sequence, or None when the tensors do not qualify."""
+        hs = hidden_states
+        dtype = hs.dtype
+        bsz, T = hs.shape[0], hs.shape[1]
+        if not (hs.is_cuda and hs.is_contiguous() and T % 16 == 0 and 0 < bsz * T <= 4096
+                and (dtype is torch.float32 or dtype is torch.float16)):
+            return None
+        plan = self._decode_plan(dtype is torch.float16, hs.device)
+        if plan is None or hs.shape[2] != plan.embed or not _hip_ext.attn_prefill_shape_ok_cached(T, T, plan.head_dim):
+            return None
+        mask = attention_mask
+        if mask is not None:
+            mask = _mask_as_fp32(mask)
+            if not (mask is not None and mask.is_contiguous() and mask.shape == (bsz, 1, T, T) and mask.device == hs.device
+                    and mask.data_ptr() % 16 == 0):
+                return None
+        key = torch.empty((bsz, plan.heads, T, plan.head_dim), dtype=torch.int8, device=hs.device)
+        value = torch.empty((bsz, plan.heads, T, plan.head_dim), dtype=torch.int8, device=hs.device)
+        _hip_ext.opt_layer_prefill(plan, hs, mask, key, value)
+        if use_cache:
+            return hs, (key, value)
         return (hs,)
 
     def decode_step_devlen(self, hidden_states, k_buf, v_buf, length, max_length):
@@ -556,6 +591,12 @@ class Int8OPTDecoderLayer(nn.Module):
                 and hidden_states.shape[1] == 1 and layer_head_mask is None and not output_attentions
                 and self.self_attn.kv_cache_in_place and self.self_attn.fused_softmax):
             out = self._decode_in_one_call(hidden_states, attention_mask, past_key_value, use_cache)
+            if out is not None:
+                return out
+        elif (past_key_value is None and self.prefill_in_one_call and hidden_states.dim() == 3
+                and 16 < hidden_states.shape[1] and layer_head_mask is None and not output_attentions
+                and self.self_attn.fused_softmax):
+            out = self._prefill_in_one_call(hidden_states, attention_mask, use_cache)
             if out is not None:
                 return out
         residual = hidden_states
